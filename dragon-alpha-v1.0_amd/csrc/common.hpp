@@ -1,0 +1,81 @@
+// Shared declarations of the gfx950 conv kernels: launch-argument structs, exact integer
+// division by launch-time constants, and the host-side launcher prototypes called by the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace alpha {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// Unsigned division by a run-time constant d >= 1 for dividends n < 2^31:
+// q = (mulhi(n, mul) + n) >> shift, exact for every such n (round-up method with a 33-bit
+// multiplier whose top bit is the "+ n").
+struct FastDiv {
+    uint32_t mul, shift, d;
+};
+
+inline FastDiv make_fastdiv(uint32_t d)
+{
+    FastDiv f;
+    f.d = d;
+    uint32_t s = 0;
+    while ((1ull << s) < d) s++;
+    f.shift = s;
+    f.mul = (uint32_t)(((1ull << 32) * ((1ull << s) - d)) / d + 1);
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
+{
+    return (__umulhi(n, f.mul) + n) >> f.shift;
+}
+
+// One launch of the generic implicit-GEMM "gather convolution":
+//   O[o_off + n*o_sn + i*o_sh + j*o_sw + co] =
+//       sum_{th<TH, tw<TW, c<AC}  A[n, i*sh - ph + th, j*sw - pw + tw, c] * B[b_off + th*b_sth + tw*b_stw + c*b_sc + co*b_sn]
+// for n < N, i < OHt, j < OWt, co < CO, taps outside [0,AH)x[0,AW) contributing zero.
+// GEMM view: M = N*OHt*OWt rows (pixels), CO columns, K = TH*TW*AC ordered (th, tw, c).
+// Forward, stride-1 backward-data, 1x1 and each phase of kernel-split backward-data are all
+// instances (see conv_api.hip). Exactly one of b_sc, b_sn is 1 (which operand axis is contiguous).
+struct GatherConvArgs {
+    const float *A;
+    const float *B;
+    float *O;
+    int M, K, CO;
+    int AH, AW, AC;
+    int sh, sw, ph, pw;
+    int a_sn;                       // AH*AW*AC
+    int o_off, o_sn, o_sh, o_sw;    // output strides, elements
+    int b_off, b_sth, b_stw, b_sc, b_sn;
+    FastDiv d_AC, d_TW, d_OWt, d_OHWt;
+};
+
+hipError_t launch_gather_conv(hipStream_t stream, const GatherConvArgs &a, int TH, int TW, int OHt, int OWt, int N);
+
+// Backward-filter implicit GEMM with split-K over k = (n, oh, ow):
+//   dst_z[oc, fh, fw, ic] = sum_{k in slice z} deltaY[k, oc] * X[n, oh*sh - ph + fh, ow*sw - pw + fw, ic]
+// slice z = [z*GK_slice, (z+1)*GK_slice), the last one running to GK; dst_0 = deltaW,
+// dst_z = deltaW_buf + (z-1)*sizeW.
+struct DeltaWArgs {
+    const float *X;
+    const float *dY;
+    float *dW;
+    float *dW_buf;
+    int IH, IW, IC, OH, OW, OC, FW;
+    int sh, sw, ph, pw;
+    int GM;        // FH*FW*IC   (columns)
+    int GK, GK_slice, GZ;
+    FastDiv d_IC, d_FW, d_OW, d_OHW;
+};
+
+hipError_t launch_deltaW(hipStream_t stream, const DeltaWArgs &a);
+
+// Re-layout / reduction helpers.
+hipError_t launch_kernel_remode(hipStream_t s, const float *W, float *CW, int FH, int FW, int OC, int IC);
+hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, int FW, float *CW,
+                            int mCFH, int mCFW, int OC, int IC, int sh, int sw);
+hipError_t launch_buf_summary(hipStream_t s, const float *buf, float *dW, int part, int sizeW);
+
+}  // namespace alpha

@@ -1,0 +1,397 @@
+// C ABI of the conv3D hot path (declared in include/alpha_conv.h): argument checks and the mapping
+// of every reference entry point onto the gfx950 kernels. Everything is enqueued on streams[0];
+// nothing is allocated, freed or synchronised here.
+#include "../../include/alpha_conv.h"
+#include "common.hpp"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+using namespace alpha;
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_status(hipError_t e, const char *what)
+{
+    if (e == hipSuccess) return 0;
+    return fail((int)e, "%s: %s", what, hipGetErrorString(e));
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline hipStream_t stream0(const int64_t *streams) { return reinterpret_cast<hipStream_t>((intptr_t)streams[0]); }
+
+#define CHECK_STREAMS()                                                                    \
+    do {                                                                                   \
+        if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", __func__); \
+    } while (0)
+
+#define CHECK_PTR(p)                                                                                        \
+    do {                                                                                                    \
+        if ((p) == nullptr || !aligned16(p)) return fail(ALPHA_CONV_EINVAL, "%s: %s is null or not 16-byte aligned", __func__, #p); \
+    } while (0)
+
+int check_dims(const char *fn, int N, int IC, int OC, int IH, int IW, int OH, int OW, int FH, int FW, int sh, int sw, int ph, int pw)
+{
+    if (N < 1 || IC < 4 || OC < 4 || IH < 1 || IW < 1 || OH < 1 || OW < 1 || FH < 1 || FW < 1 || sh < 1 || sw < 1 || ph < 0 || pw < 0)
+        return fail(ALPHA_CONV_EINVAL, "%s: non-positive dimension", fn);
+    if ((IC & 3) || (OC & 3)) return fail(ALPHA_CONV_EINVAL, "%s: IC and OC must be multiples of 4 (got %d, %d)", fn, IC, OC);
+    if ((long)N * IH * IW * IC >= (1L << 31) || (long)N * OH * OW * OC >= (1L << 31) || (long)OC * FH * FW * IC >= (1L << 31))
+        return fail(ALPHA_CONV_EINVAL, "%s: tensor exceeds 2^31 elements", fn);
+    return 0;
+}
+
+enum FilterLayout { FILTER_W, FILTER_CW };
+
+// Forward: Y = conv(X, filter). FILTER_W reads W[OC,FH,FW,IC]; FILTER_CW reads CW[FH,FW,IC,OC].
+int forward(const char *fn, const int64_t *streams, int length,
+            const float *X, int IH, int IW, const float *F, FilterLayout layout, int FH, int FW,
+            float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
+    if (!X || !F || !Y || !aligned16(X) || !aligned16(F) || !aligned16(Y))
+        return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
+    if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
+
+    GatherConvArgs a{};
+    a.A = X; a.B = F; a.O = Y;
+    a.CO = OC;
+    a.AH = IH; a.AW = IW; a.AC = IC;
+    a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
+    a.o_off = 0; a.o_sn = OH * OW * OC; a.o_sh = OW * OC; a.o_sw = OC;
+    a.b_off = 0;
+    if (layout == FILTER_CW) {
+        a.b_sth = FW * IC * OC; a.b_stw = IC * OC; a.b_sc = OC; a.b_sn = 1;
+    } else {
+        a.b_sth = FW * IC; a.b_stw = IC; a.b_sc = 1; a.b_sn = FH * FW * IC;
+    }
+    return hip_status(launch_gather_conv(stream0(streams), a, FH, FW, OH, OW, N), fn);
+}
+
+// Backward-data, stride 1, reading W[OC,FH,FW,IC] in place rotated by 180 degrees:
+// deltaX[n,ih,iw,ic] = sum_{t_h,t_w,oc} deltaY[n, ih - (FH-1-ph) + t_h, iw - (FW-1-pw) + t_w, oc] * W[oc, FH-1-t_h, FW-1-t_w, ic]
+int deltaX_s1(const char *fn, const int64_t *streams, int length,
+              const float *dY, int OH, int OW, const float *W, int FH, int FW,
+              float *dX, int IH, int IW, int N, int IC, int OC, int ph, int pw)
+{
+    if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
+    if (!dY || !W || !dX || !aligned16(dY) || !aligned16(W) || !aligned16(dX))
+        return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
+    if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, 1, 1, ph, pw)) return e;
+    if (FH - 1 - ph < 0 || FW - 1 - pw < 0) return fail(ALPHA_CONV_EINVAL, "%s: padding larger than FH-1", fn);
+
+    GatherConvArgs a{};
+    a.A = dY; a.B = W; a.O = dX;
+    a.CO = IC;
+    a.AH = OH; a.AW = OW; a.AC = OC;
+    a.sh = 1; a.sw = 1; a.ph = FH - 1 - ph; a.pw = FW - 1 - pw;
+    a.o_off = 0; a.o_sn = IH * IW * IC; a.o_sh = IW * IC; a.o_sw = IC;
+    a.b_off = ((FH - 1) * FW + (FW - 1)) * IC;
+    a.b_sth = -FW * IC; a.b_stw = -IC; a.b_sc = FH * FW * IC; a.b_sn = 1;
+    return hip_status(launch_gather_conv(stream0(streams), a, FH, FW, IH, IW, N), fn);
+}
+
+// Backward-data for any stride as sh*sw dense sub-problems ("kernel split"): phase (y, x) owns the
+// taps fh = y (mod sh), fw = x (mod sw) and produces the deltaX sub-lattice ih = ihs (mod sh),
+// iw = iws (mod sw). from_CW: filter taken from the v2 kernel-split layout; otherwise from W in place.
+int deltaX_phases(const char *fn, const int64_t *streams, int length,
+                  const float *dY, int OH, int OW, const float *F, bool from_CW, int FH, int FW,
+                  float *dX, int IH, int IW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
+    if (!dY || !F || !dX || !aligned16(dY) || !aligned16(F) || !aligned16(dX))
+        return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
+    if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
+
+    const int mCFH = (FH + sh - 1) / sh, mCFW = (FW + sw - 1) / sw;
+    const int CWstride = mCFH * mCFW * OC * IC;
+    hipStream_t s = stream0(streams);
+    for (int y = 0; y < sh; y++)
+        for (int x = 0; x < sw; x++) {
+            const int CFH = (FH - y + sh - 1) / sh, CFW = (FW - x + sw - 1) / sw;
+            const int phy = ph - y, pwx = pw - x;
+            const int ihs = -phy + (phy > 0 ? (phy + sh - 1) / sh * sh : 0);
+            const int iws = -pwx + (pwx > 0 ? (pwx + sw - 1) / sw * sw : 0);
+            const int OHt = IH > ihs ? (IH - ihs + sh - 1) / sh : 0;
+            const int OWt = IW > iws ? (IW - iws + sw - 1) / sw : 0;
+            if (OHt == 0 || OWt == 0) continue;
+
+            GatherConvArgs a{};
+            a.A = dY; a.B = F; a.O = dX;
+            a.CO = IC;
+            a.AH = OH; a.AW = OW; a.AC = OC;
+            a.sh = 1; a.sw = 1;
+            a.ph = (CFH - 1) - (ihs + phy) / sh;
+            a.pw = (CFW - 1) - (iws + pwx) / sw;
+            a.o_off = (ihs * IW + iws) * IC; a.o_sn = IH * IW * IC; a.o_sh = sh * IW * IC; a.o_sw = sw * IC;
+            if (from_CW) {
+                a.b_off = (y * sw + x) * CWstride;
+                a.b_sth = CFW * OC * IC; a.b_stw = OC * IC; a.b_sc = IC; a.b_sn = 1;
+            } else {
+                a.b_off = ((y + (CFH - 1) * sh) * FW + (x + (CFW - 1) * sw)) * IC;
+                a.b_sth = -sh * FW * IC; a.b_stw = -sw * IC; a.b_sc = FH * FW * IC; a.b_sn = 1;
+            }
+            const int th = CFH > 0 && CFW > 0 ? CFH : 0, tw = CFH > 0 && CFW > 0 ? CFW : 0;
+            if (th == 0) a.b_off = 0;
+            if (int e = hip_status(launch_gather_conv(s, a, th, tw, OHt, OWt, N), fn)) return e;
+        }
+    return 0;
+}
+
+int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
+           const float *X, int IH, int IW, const float *dY, int OH, int OW,
+           float *dW, float *dW_buf, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
+    if (!X || !dY || !dW || !aligned16(X) || !aligned16(dY) || !aligned16(dW))
+        return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
+    if (GridZ < 1) return fail(ALPHA_CONV_EINVAL, "%s: GridZ must be >= 1", fn);
+    if (GridZ > 1 && (!dW_buf || !aligned16(dW_buf))) return fail(ALPHA_CONV_EINVAL, "%s: deltaW_buf is null or misaligned", fn);
+    if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
+
+    DeltaWArgs a{};
+    a.X = X; a.dY = dY; a.dW = dW; a.dW_buf = dW_buf;
+    a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC; a.FW = FW;
+    a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
+    a.GM = FH * FW * IC;
+    a.GK = N * OH * OW;
+    a.GZ = GridZ;
+    a.GK_slice = (a.GK / GridZ) >> 3 << 3;
+    return hip_status(launch_deltaW(stream0(streams), a), fn);
+}
+
+}  // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+const char *alpha_conv_version(void) { return "alpha-conv-hip gfx950 0.1"; }
+const char *alpha_conv_last_error(void) { return g_err; }
+
+static int g_fwd_algo = -1;
+int alpha_conv_get_fwd_algo(void)
+{
+    if (g_fwd_algo < 0) {
+        const char *e = getenv("ALPHA_HIP_CONV_ALGO");
+        int v = 0;
+        if (e && !strcmp(e, "igemm")) v = 1;
+        else if (e && !strcmp(e, "winograd")) v = 2;
+        g_fwd_algo = v;
+    }
+    return g_fwd_algo;
+}
+int alpha_conv_set_fwd_algo(int algo)
+{
+    if (algo < 0 || algo > 2) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0, 1 or 2");
+    g_fwd_algo = algo;
+    return 0;
+}
+
+// ---- forward -------------------------------------------------------------------------------
+int alpha_conv3D(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, int FH, int FW,
+                 float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    return forward(__func__, streams, length, X, IH, IW, W, FILTER_W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_conv3D_texture(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, int FH, int FW,
+                         float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    return forward(__func__, streams, length, X, IH, IW, W, FILTER_W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_conv3DV2(int useTexture, const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, int FH, int FW,
+                   float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    (void)useTexture;
+    return forward(__func__, streams, length, X, IH, IW, W, FILTER_W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_conv3D_np(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, int FH, int FW,
+                    float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw)
+{
+    return forward(__func__, streams, length, X, IH, IW, W, FILTER_W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, 0, 0);
+}
+int alpha_conv3D_W1(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, float *Y,
+                    int N, int IC, int OC)
+{
+    return forward(__func__, streams, length, X, IH, IW, W, FILTER_W, 1, 1, Y, IH, IW, N, IC, OC, 1, 1, 0, 0);
+}
+int alpha_kernel_remode(int64_t stream, const float *W, float *CW, int FH, int FW, int OC, int IC)
+{
+    CHECK_PTR(W);
+    CHECK_PTR(CW);
+    if (FH < 1 || FW < 1 || OC < 4 || IC < 4 || (OC & 3) || (IC & 3))
+        return fail(ALPHA_CONV_EINVAL, "%s: bad filter dims", __func__);
+    return hip_status(launch_kernel_remode(reinterpret_cast<hipStream_t>((intptr_t)stream), W, CW, FH, FW, OC, IC), __func__);
+}
+int alpha_conv3D_GemmR(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, const float *CW,
+                       int FH, int FW, float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    (void)W;
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_conv3D_GemmR_texture(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, const float *CW,
+                               int FH, int FW, float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    (void)W;
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_conv3D_GemmV2R(int useTexture, const int64_t *streams, int length, const float *X, int IH, int IW, const float *W,
+                         const float *CW, int FH, int FW, float *Y, int OH, int OW, int N, int IC, int OC,
+                         int sh, int sw, int ph, int pw)
+{
+    (void)useTexture;
+    (void)W;
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_conv3D_GemmR_W1(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, const float *CW,
+                          float *Y, int N, int IC, int OC)
+{
+    (void)W;
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, 1, 1, Y, IH, IW, N, IC, OC, 1, 1, 0, 0);
+}
+
+// ---- backward-data ---------------------------------------------------------------------------
+int alpha_dconv3D_deltaX_s1(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *W, int FH, int FW,
+                            float *deltaX, int IH, int IW, int N, int IC, int OC, int ph, int pw)
+{
+    return deltaX_s1(__func__, streams, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+}
+int alpha_dconv3D_deltaX_s1_texture(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *W,
+                                    int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC, int ph, int pw)
+{
+    return deltaX_s1(__func__, streams, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+}
+int alpha_dconv3D_deltaX_V2_s1(int useTexture, const int64_t *streams, int length, const float *deltaY, int OH, int OW,
+                               const float *W, int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC, int ph, int pw)
+{
+    (void)useTexture;
+    return deltaX_s1(__func__, streams, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+}
+int alpha_dconv3D_deltaX_W1(const int64_t *streams, int length, const float *deltaY, const float *W, float *deltaX,
+                            int IH, int IW, int N, int IC, int OC)
+{
+    return deltaX_s1(__func__, streams, length, deltaY, IH, IW, W, 1, 1, deltaX, IH, IW, N, IC, OC, 0, 0);
+}
+int alpha_ks_remode(int64_t stream, const float *W, int FH, int FW, float *CW, int CFH, int CFW, int OC, int IC, int sh, int sw)
+{
+    CHECK_PTR(W);
+    CHECK_PTR(CW);
+    if (FH < 1 || FW < 1 || OC < 4 || IC < 4 || (OC & 3) || (IC & 3) || sh < 1 || sw < 1 || CFH != (FH + sh - 1) / sh || CFW != (FW + sw - 1) / sw)
+        return fail(ALPHA_CONV_EINVAL, "%s: bad filter dims", __func__);
+    return hip_status(launch_ks_remode(reinterpret_cast<hipStream_t>((intptr_t)stream), 1, W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw), __func__);
+}
+int alpha_ks_remodev2(int64_t stream, const float *W, int FH, int FW, float *CW, int CFH, int CFW, int OC, int IC, int sh, int sw)
+{
+    CHECK_PTR(W);
+    CHECK_PTR(CW);
+    if (FH < 1 || FW < 1 || OC < 4 || IC < 4 || (OC & 3) || (IC & 3) || sh < 1 || sw < 1 || CFH != (FH + sh - 1) / sh || CFW != (FW + sw - 1) / sw)
+        return fail(ALPHA_CONV_EINVAL, "%s: bad filter dims", __func__);
+    return hip_status(launch_ks_remode(reinterpret_cast<hipStream_t>((intptr_t)stream), 2, W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw), __func__);
+}
+int alpha_dconv3D_deltaX_kernelSplit(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *CW,
+                                     int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC,
+                                     int sh, int sw, int ph, int pw)
+{
+    return deltaX_phases(__func__, streams, length, deltaY, OH, OW, CW, true, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_dconv3D_deltaX_ksImsR(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *CW,
+                                int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC,
+                                int sh, int sw, int ph, int pw)
+{
+    return deltaX_phases(__func__, streams, length, deltaY, OH, OW, CW, true, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_dconv3D_deltaX_ksImsR_texture(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *CW,
+                                        int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC,
+                                        int sh, int sw, int ph, int pw)
+{
+    return deltaX_phases(__func__, streams, length, deltaY, OH, OW, CW, true, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_dconv3D_deltaX_ksIms2R(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *CW,
+                                 int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC, int ph, int pw)
+{
+    return deltaX_phases(__func__, streams, length, deltaY, OH, OW, CW, true, FH, FW, deltaX, IH, IW, N, IC, OC, 2, 2, ph, pw);
+}
+int alpha_dconv3D_deltaX_ksIms2R_texture(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *CW,
+                                         int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC, int ph, int pw)
+{
+    return deltaX_phases(__func__, streams, length, deltaY, OH, OW, CW, true, FH, FW, deltaX, IH, IW, N, IC, OC, 2, 2, ph, pw);
+}
+int alpha_dconv3D_deltaX_ksV2_Ims2R(int useTexture, const int64_t *streams, int length, const float *deltaY, int OH, int OW,
+                                    const float *CW, int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC,
+                                    int ph, int pw)
+{
+    (void)useTexture;
+    return deltaX_phases(__func__, streams, length, deltaY, OH, OW, CW, true, FH, FW, deltaX, IH, IW, N, IC, OC, 2, 2, ph, pw);
+}
+int alpha_dconv3D_deltaX_crossAdd(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *W,
+                                  int FH, int FW, float *deltaX, int IH, int IW, int N, int IC, int OC,
+                                  int sh, int sw, int ph, int pw)
+{
+    return deltaX_phases(__func__, streams, length, deltaY, OH, OW, W, false, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
+}
+
+// ---- backward-filter ----------------------------------------------------------------------------
+int alpha_dconv3D_deltaW(const int64_t *streams, int length, const float *X, int IH, int IW, const float *deltaY, int OH, int OW,
+                         float *deltaW, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    return deltaW_impl(__func__, streams, length, 1, X, IH, IW, deltaY, OH, OW, deltaW, nullptr, FH, FW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_dconv3D_deltaW_W1(const int64_t *streams, int length, const float *X, int IH, int IW, const float *deltaY,
+                            float *deltaW, int N, int IC, int OC)
+{
+    return deltaW_impl(__func__, streams, length, 1, X, IH, IW, deltaY, IH, IW, deltaW, nullptr, 1, 1, N, IC, OC, 1, 1, 0, 0);
+}
+int alpha_buf_summary(int64_t stream, const float *deltaW_buf, float *deltaW, int part, int sizeW)
+{
+    CHECK_PTR(deltaW);
+    if (part < 0 || sizeW < 1) return fail(ALPHA_CONV_EINVAL, "%s: bad part/sizeW", __func__);
+    if (part == 0) return 0;
+    CHECK_PTR(deltaW_buf);
+    return hip_status(launch_buf_summary(reinterpret_cast<hipStream_t>((intptr_t)stream), deltaW_buf, deltaW, part, sizeW), __func__);
+}
+int alpha_dconv3D_deltaW_GemmSK(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
+                                const float *deltaY, int OH, int OW, float *deltaW, float *deltaW_buf, int FH, int FW,
+                                int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    return deltaW_impl(__func__, streams, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_dconv3D_deltaW_GemmV2SK(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
+                                  const float *deltaY, int OH, int OW, float *deltaW, float *deltaW_buf, int FH, int FW,
+                                  int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    return deltaW_impl(__func__, streams, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw);
+}
+int alpha_dconv3D_deltaW_GemmSK_W1(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
+                                   const float *deltaY, float *deltaW, float *deltaW_buf, int N, int IC, int OC)
+{
+    return deltaW_impl(__func__, streams, length, GridZ, X, IH, IW, deltaY, IH, IW, deltaW, deltaW_buf, 1, 1, N, IC, OC, 1, 1, 0, 0);
+}
+
+// ---- Winograd (filled in by winograd.hip once built) ------------------------------------------
+long alpha_winograd_filter_size(int IC, int OC) { return 16L * IC * OC; }
+int alpha_winograd_filter_transform(int64_t stream, const float *W, float *U, int IC, int OC)
+{
+    (void)stream; (void)W; (void)U; (void)IC; (void)OC;
+    return fail(ALPHA_CONV_EINVAL, "%s: not available in this build", __func__);
+}
+int alpha_conv3D_winograd(const int64_t *streams, int length, const float *X, int IH, int IW, const float *U, float *Y,
+                          int OH, int OW, int N, int IC, int OC, int ph, int pw)
+{
+    (void)streams; (void)length; (void)X; (void)IH; (void)IW; (void)U; (void)Y; (void)OH; (void)OW; (void)N; (void)IC; (void)OC; (void)ph; (void)pw;
+    return fail(ALPHA_CONV_EINVAL, "%s: not available in this build", __func__);
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

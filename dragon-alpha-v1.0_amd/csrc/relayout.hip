@@ -1,0 +1,144 @@
+// Filter re-layouts and the split-K partial-buffer summation. All are pure HBM-bandwidth
+// kernels: 128-bit accesses, lanes along the contiguous axis of whichever side can be.
+#include "common.hpp"
+
+namespace alpha {
+
+// W[OC][K] -> CW[K][OC] with K = FH*FW*IC: a matrix transpose through a padded 64x64 LDS tile so
+// that both the read (along K) and the write (along OC) are coalesced.
+__global__ __launch_bounds__(256) void kernel_remode_kernel(const float *__restrict__ W, float *__restrict__ CW,
+                                                            int OC, int K)
+{
+    __shared__ float tile[64][65];
+    const int k0 = blockIdx.x * 64, oc0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;  // 16 x 16
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int oc = oc0 + ty + 16 * r, k = k0 + tx * 4;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (oc < OC && k < K) v = *reinterpret_cast<const float4 *>(W + (size_t)oc * K + k);  // K % 4 == 0
+        tile[ty + 16 * r][tx * 4 + 0] = v.x;
+        tile[ty + 16 * r][tx * 4 + 1] = v.y;
+        tile[ty + 16 * r][tx * 4 + 2] = v.z;
+        tile[ty + 16 * r][tx * 4 + 3] = v.w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int k = k0 + ty + 16 * r, oc = oc0 + tx * 4;
+        if (k < K && oc < OC) {  // OC % 4 == 0
+            float4 v;
+            v.x = tile[tx * 4 + 0][ty + 16 * r];
+            v.y = tile[tx * 4 + 1][ty + 16 * r];
+            v.z = tile[tx * 4 + 2][ty + 16 * r];
+            v.w = tile[tx * 4 + 3][ty + 16 * r];
+            *reinterpret_cast<float4 *>(CW + (size_t)k * OC + oc) = v;
+        }
+    }
+}
+
+hipError_t launch_kernel_remode(hipStream_t s, const float *W, float *CW, int FH, int FW, int OC, int IC)
+{
+    const int K = FH * FW * IC;
+    if (K <= 0 || OC <= 0) return hipSuccess;
+    dim3 grid((K + 63) / 64, (OC + 63) / 64);
+    hipLaunchKernelGGL(kernel_remode_kernel, grid, dim3(256), 0, s, W, CW, OC, K);
+    return hipGetLastError();
+}
+
+// Kernel-split filter layouts for strided backward-data. Phase (y, x) holds the taps
+// fh = y + (CFH_y-1-fhr)*sh, fw = x + (CFW_x-1-fwr)*sw packed from the start of its block of
+// OC*mCFH*mCFW*IC floats; V2 orders a block [fhr][fwr][oc][ic], V1 orders it [oc][fhr][fwr][ic].
+template <bool V2>
+__global__ __launch_bounds__(256) void ks_remode_kernel(const float *__restrict__ W, int FH, int FW,
+                                                        float *__restrict__ CW, int mCFH, int mCFW,
+                                                        int OC, int IC, int sh, int sw)
+{
+    const int by = blockIdx.y;
+    const int y = by / sw, x = by - y * sw;
+    const int CFH = (FH - y + sh - 1) / sh, CFW = (FW - x + sw - 1) / sw;
+    float *blk = CW + (size_t)by * OC * mCFH * mCFW * IC;
+    const int n4 = (OC * CFH * CFW * IC) >> 2;
+    const int IC4 = IC >> 2;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += gridDim.x * blockDim.x) {
+        int r = i;
+        const int ic = (r % IC4) * 4;
+        r /= IC4;
+        int oc, fhr, fwr;
+        if (V2) {
+            oc = r % OC; r /= OC;
+            fwr = r % CFW; fhr = r / CFW;
+        } else {
+            fwr = r % CFW; r /= CFW;
+            fhr = r % CFH; oc = r / CFH;
+        }
+        const int fh = y + (CFH - 1 - fhr) * sh, fw = x + (CFW - 1 - fwr) * sw;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (fh < FH && fw < FW) v = *reinterpret_cast<const float4 *>(W + (((size_t)oc * FH + fh) * FW + fw) * IC + ic);
+        *reinterpret_cast<float4 *>(blk + (size_t)i * 4) = v;
+    }
+}
+
+hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, int FW, float *CW,
+                            int mCFH, int mCFW, int OC, int IC, int sh, int sw)
+{
+    const int n4 = (OC * mCFH * mCFW * IC) >> 2;
+    if (n4 <= 0 || sh <= 0 || sw <= 0) return hipSuccess;
+    int bx = (n4 + 255) / 256;
+    if (bx > 4096) bx = 4096;
+    dim3 grid(bx, sh * sw);
+    if (version == 2)
+        hipLaunchKernelGGL(ks_remode_kernel<true>, grid, dim3(256), 0, s, W, FH, FW, CW, mCFH, mCFW, OC, IC, sh, sw);
+    else
+        hipLaunchKernelGGL(ks_remode_kernel<false>, grid, dim3(256), 0, s, W, FH, FW, CW, mCFH, mCFW, OC, IC, sh, sw);
+    return hipGetLastError();
+}
+
+// deltaW += sum_{p < part} deltaW_buf[p], summed in the fixed order p = 0, 1, ... with fp32 Kahan
+// compensation; one thread owns four consecutive elements for the whole sum.
+__global__ __launch_bounds__(256) void buf_summary_kernel(const float *__restrict__ buf, float *__restrict__ dW,
+                                                          int part, int sizeW)
+{
+    const int n4 = sizeW >> 2;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += gridDim.x * blockDim.x) {
+        float4 dw = *reinterpret_cast<const float4 *>(dW + (size_t)i * 4);
+        float4 c = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int p = 0; p < part; p++) {
+            float4 b = *reinterpret_cast<const float4 *>(buf + (size_t)p * sizeW + (size_t)i * 4);
+            b.x -= c.x; b.y -= c.y; b.z -= c.z; b.w -= c.w;
+            float4 s;
+            s.x = dw.x + b.x; s.y = dw.y + b.y; s.z = dw.z + b.z; s.w = dw.w + b.w;
+            c.x = (s.x - dw.x) - b.x;
+            c.y = (s.y - dw.y) - b.y;
+            c.z = (s.z - dw.z) - b.z;
+            c.w = (s.w - dw.w) - b.w;
+            dw = s;
+        }
+        *reinterpret_cast<float4 *>(dW + (size_t)i * 4) = dw;
+    }
+    // sizeW is a multiple of 4 on this path (IC % 4 == 0); a ragged tail is summed scalar-wise.
+    const int tail = sizeW & 3;
+    if (tail && blockIdx.x == 0 && threadIdx.x < tail) {
+        const int i = (n4 << 2) + threadIdx.x;
+        float dw = dW[i], c = 0.f;
+        for (int p = 0; p < part; p++) {
+            float b = buf[(size_t)p * sizeW + i] - c;
+            float s = dw + b;
+            c = (s - dw) - b;
+            dw = s;
+        }
+        dW[i] = dw;
+    }
+}
+
+hipError_t launch_buf_summary(hipStream_t s, const float *buf, float *dW, int part, int sizeW)
+{
+    if (sizeW <= 0 || part <= 0) return hipSuccess;
+    int bx = ((sizeW >> 2) + 255) / 256;
+    if (bx < 1) bx = 1;
+    if (bx > 8192) bx = 8192;
+    hipLaunchKernelGGL(buf_summary_kernel, dim3(bx), dim3(256), 0, s, buf, dW, part, sizeW);
+    return hipGetLastError();
+}
+
+}  // namespace alpha

@@ -1,0 +1,261 @@
+"""ctypes mirror of the reference's JNI native classes over the C ABI (include/alpha_conv.h).
+
+Class and method names, argument order and meaning follow
+  src/alpha_src/z/dragon/engine/cuda/impl/math/Cuda_conv3D.java           (natives at :240-766)
+  src/alpha_src/z/dragon/engine/cuda/impl/math/Cuda_dconv3D_deltaX.java   (natives at :311-980)
+  src/alpha_src/z/dragon/engine/cuda/impl/math/Cuda_dconv3D_deltaW.java   (natives at :243-472)
+Addresses are plain integers (device pointers / hipStream_t handles), exactly like the jlong
+arguments of the Java side. Where the Java natives return void and throw on error, these raise
+AlphaConvError.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_NAME = "libalpha_conv_hip.so"
+_lib = None
+
+_I = ctypes.c_int
+_L = ctypes.c_int64
+_P = ctypes.c_void_p
+_S = ctypes.POINTER(ctypes.c_int64)
+
+# signature strings: S = stream array, i = int, p = device pointer, l = int64 handle
+_SIGS = {
+    "alpha_conv3D": "sipiipiipiiiiiiiii",
+    "alpha_conv3D_texture": "sipiipiipiiiiiiiii",
+    "alpha_conv3DV2": "isipiipiipiiiiiiiii",
+    "alpha_conv3D_np": "sipiipiipiiiiiii",
+    "alpha_conv3D_W1": "sipiippiii",
+    "alpha_kernel_remode": "lppiiii",
+    "alpha_conv3D_GemmR": "sipiippiipiiiiiiiii",
+    "alpha_conv3D_GemmR_texture": "sipiippiipiiiiiiiii",
+    "alpha_conv3D_GemmV2R": "isipiippiipiiiiiiiii",
+    "alpha_conv3D_GemmR_W1": "sipiipppiii",
+    "alpha_dconv3D_deltaX_s1": "sipiipiipiiiiiii",
+    "alpha_dconv3D_deltaX_s1_texture": "sipiipiipiiiiiii",
+    "alpha_dconv3D_deltaX_V2_s1": "isipiipiipiiiiiii",
+    "alpha_dconv3D_deltaX_W1": "sipppiiiii",
+    "alpha_ks_remode": "lpiipiiiiii",
+    "alpha_ks_remodev2": "lpiipiiiiii",
+    "alpha_dconv3D_deltaX_kernelSplit": "sipiipiipiiiiiiiii",
+    "alpha_dconv3D_deltaX_ksImsR": "sipiipiipiiiiiiiii",
+    "alpha_dconv3D_deltaX_ksImsR_texture": "sipiipiipiiiiiiiii",
+    "alpha_dconv3D_deltaX_ksIms2R": "sipiipiipiiiiiii",
+    "alpha_dconv3D_deltaX_ksIms2R_texture": "sipiipiipiiiiiii",
+    "alpha_dconv3D_deltaX_ksV2_Ims2R": "isipiipiipiiiiiii",
+    "alpha_dconv3D_deltaX_crossAdd": "sipiipiipiiiiiiiii",
+    "alpha_dconv3D_deltaW": "sipiipiipiiiiiiiii",
+    "alpha_dconv3D_deltaW_W1": "sipiippiii",
+    "alpha_buf_summary": "lppii",
+    "alpha_dconv3D_deltaW_GemmSK": "siipiipiippiiiiiiiii",
+    "alpha_dconv3D_deltaW_GemmV2SK": "siipiipiippiiiiiiiii",
+    "alpha_dconv3D_deltaW_GemmSK_W1": "siipiipppiii",
+    "alpha_winograd_filter_transform": "lppii",
+    "alpha_conv3D_winograd": "sipiippiiiiiii",
+}
+_CT = {"s": _S, "i": _I, "p": _P, "l": _L}
+
+
+class AlphaConvError(RuntimeError):
+    """Raised where the Java natives would throw CudaException."""
+
+
+def lib_path():
+    return os.path.join(_HERE, _LIB_NAME)
+
+
+def exported_symbols():
+    """Names the C ABI must export (every function include/alpha_conv.h declares)."""
+    return sorted(list(_SIGS) + ["alpha_conv_version", "alpha_conv_last_error", "alpha_conv_set_fwd_algo",
+                                 "alpha_conv_get_fwd_algo", "alpha_winograd_filter_size"])
+
+
+def lib():
+    """Loads the HIP library; raises if it has not been built (there is no fallback path)."""
+    global _lib
+    if _lib is None:
+        path = lib_path()
+        if not os.path.exists(path):
+            raise AlphaConvError("%s is not built: run `python %s`" % (path, os.path.join(_HERE, "build.py")))
+        L = ctypes.CDLL(path)
+        for name, sig in _SIGS.items():
+            fn = getattr(L, name)
+            fn.argtypes = [_CT[c] for c in sig]
+            fn.restype = _I
+        L.alpha_conv_version.restype = ctypes.c_char_p
+        L.alpha_conv_last_error.restype = ctypes.c_char_p
+        L.alpha_conv_set_fwd_algo.argtypes = [_I]
+        L.alpha_conv_get_fwd_algo.restype = _I
+        L.alpha_winograd_filter_size.argtypes = [_I, _I]
+        L.alpha_winograd_filter_size.restype = ctypes.c_long
+        _lib = L
+    return _lib
+
+
+def _call(name, *args):
+    L = lib()
+    sig = _SIGS[name]
+    conv = []
+    keep = []
+    it = iter(args)
+    for c in sig:
+        a = next(it)
+        if c == "s":
+            arr = (ctypes.c_int64 * max(1, len(a)))(*a)
+            keep.append(arr)
+            conv.append(arr)
+        elif c == "p":
+            conv.append(ctypes.c_void_p(int(a)))
+        elif c == "l":
+            conv.append(ctypes.c_int64(int(a)))
+        else:
+            conv.append(int(a))
+    rc = getattr(L, name)(*conv)
+    if rc != 0:
+        raise AlphaConvError("%s failed (%d): %s" % (name, rc, L.alpha_conv_last_error().decode()))
+
+
+class Cuda_conv3D:
+    """Forward natives (Cuda_conv3D.java)."""
+
+    @staticmethod
+    def outputTensorDim(IH, IW, FH, FW, N, OC, sh, sw, ph, pw):
+        return [N, (IH + (ph << 1) - FH) // sh + 1, (IW + (pw << 1) - FW) // sw + 1, OC]
+
+    @staticmethod
+    def conv3D(streamArray, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D", streamArray, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_texture(streamArray, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D_texture", streamArray, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3DV2(useTexture, streamArray, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3DV2", useTexture, streamArray, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_np(streamArray, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw):
+        _call("alpha_conv3D_np", streamArray, length, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw)
+
+    @staticmethod
+    def conv3D_W1(streamArray, length, X, IH, IW, W, Y, N, IC, OC):
+        _call("alpha_conv3D_W1", streamArray, length, X, IH, IW, W, Y, N, IC, OC)
+
+    @staticmethod
+    def kernel_remode(stream, W, CW, FH, FW, OC, IC):
+        _call("alpha_kernel_remode", stream, W, CW, FH, FW, OC, IC)
+
+    @staticmethod
+    def conv3D_GemmR(streamArray, length, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D_GemmR", streamArray, length, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_GemmR_texture(streamArray, length, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D_GemmR_texture", streamArray, length, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_GemmV2R(useTexture, streamArray, length, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D_GemmV2R", useTexture, streamArray, length, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_GemmR_W1(streamArray, length, X, IH, IW, W, CW, Y, N, IC, OC):
+        _call("alpha_conv3D_GemmR_W1", streamArray, length, X, IH, IW, W, CW, Y, N, IC, OC)
+
+    # additional algorithm of this build (no Java counterpart)
+    @staticmethod
+    def winograd_filter_size(IC, OC):
+        return int(lib().alpha_winograd_filter_size(IC, OC))
+
+    @staticmethod
+    def winograd_filter_transform(stream, W, U, IC, OC):
+        _call("alpha_winograd_filter_transform", stream, W, U, IC, OC)
+
+    @staticmethod
+    def conv3D_winograd(streamArray, length, X, IH, IW, U, Y, OH, OW, N, IC, OC, ph, pw):
+        _call("alpha_conv3D_winograd", streamArray, length, X, IH, IW, U, Y, OH, OW, N, IC, OC, ph, pw)
+
+
+class Cuda_dconv3D_deltaX:
+    """Backward-data natives (Cuda_dconv3D_deltaX.java)."""
+
+    @staticmethod
+    def dconv3D_deltaX_s1(streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):
+        _call("alpha_dconv3D_deltaX_s1", streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_s1_texture(streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):
+        _call("alpha_dconv3D_deltaX_s1_texture", streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_V2_s1(useTexture, streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):
+        _call("alpha_dconv3D_deltaX_V2_s1", useTexture, streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_W1(streamArray, length, deltaY, W, deltaX, IH, IW, N, IC, OC):
+        _call("alpha_dconv3D_deltaX_W1", streamArray, length, deltaY, W, deltaX, IH, IW, N, IC, OC)
+
+    @staticmethod
+    def ks_remode(stream, W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw):
+        _call("alpha_ks_remode", stream, W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw)
+
+    @staticmethod
+    def ks_remodev2(stream, W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw):
+        _call("alpha_ks_remodev2", stream, W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw)
+
+    @staticmethod
+    def dconv3D_deltaX_kernelSplit(streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaX_kernelSplit", streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_ksImsR(streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaX_ksImsR", streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_ksImsR_texture(streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaX_ksImsR_texture", streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_ksIms2R(streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):
+        _call("alpha_dconv3D_deltaX_ksIms2R", streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_ksIms2R_texture(streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):
+        _call("alpha_dconv3D_deltaX_ksIms2R_texture", streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_ksV2_Ims2R(useTexture, streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):
+        _call("alpha_dconv3D_deltaX_ksV2_Ims2R", useTexture, streamArray, length, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_crossAdd(streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaX_crossAdd", streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw)
+
+
+class Cuda_dconv3D_deltaW:
+    """Backward-filter natives (Cuda_dconv3D_deltaW.java)."""
+
+    @staticmethod
+    def dconv3D_deltaW(streamArray, length, X, IH, IW, deltaY, OH, OW, deltaW, FH, FW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaW", streamArray, length, X, IH, IW, deltaY, OH, OW, deltaW, FH, FW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaW_W1(streamArray, length, X, IH, IW, deltaY, deltaW, N, IC, OC):
+        _call("alpha_dconv3D_deltaW_W1", streamArray, length, X, IH, IW, deltaY, deltaW, N, IC, OC)
+
+    @staticmethod
+    def buf_summary(stream, deltaW_buf, deltaW, part, sizeW):
+        _call("alpha_buf_summary", stream, deltaW_buf, deltaW, part, sizeW)
+
+    @staticmethod
+    def dconv3D_deltaW_GemmSK(streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaW_GemmSK", streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaW_GemmV2SK(streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaW_GemmV2SK", streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaW_GemmSK_W1(streamArray, length, GridZ, X, IH, IW, deltaY, deltaW, deltaW_buf, N, IC, OC):
+        _call("alpha_dconv3D_deltaW_GemmSK_W1", streamArray, length, GridZ, X, IH, IW, deltaY, deltaW, deltaW_buf, N, IC, OC)

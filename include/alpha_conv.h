@@ -1,0 +1,266 @@
+/*
+ * alpha_conv.h — C ABI of the MI355X (gfx950) replacement for Dragon-Alpha's cu32 conv3D hot path.
+ *
+ * One entry point per JNI native method of the reference classes
+ *   z.dragon.engine.cuda.impl.math.Cuda_conv3D          (10 methods)
+ *   z.dragon.engine.cuda.impl.math.Cuda_dconv3D_deltaX  (13 methods)
+ *   z.dragon.engine.cuda.impl.math.Cuda_dconv3D_deltaW  ( 6 methods)
+ * with the same argument order and meaning as the reference's native implementations
+ * (cited per function as <project>/A.cu:<line>, where
+ *   conv = src/cu32_src/Cuda_conv3D/Cuda_conv3D,
+ *   dX   = src/cu32_src/Cuda_dconv3D_deltaX/Cuda_dconv3D_deltaX,
+ *   dW   = src/cu32_src/Cuda_dconv3D_deltaW/Cuda_dconv3D_deltaW).
+ * The JNI shim (csrc/jni_shim.cpp) exports the exact Java_z_dragon_..._<method> symbols and
+ * forwards to these functions after copying the stream handles out of the jlongArray.
+ *
+ * Conventions (identical to the reference):
+ *   - fp32 everywhere. X[N,IH,IW,IC], W[OC,FH,FW,IC], Y[N,OH,OW,OC], dense row-major (NHWC).
+ *   - N, IC and OC are multiples of 4 (the engine pads them); pad channels hold zeros.
+ *   - OH = (IH + 2*ph - FH)/sh + 1, OW likewise.
+ *   - All pointers are DEVICE pointers, borrowed for the duration of the enqueued work. Nothing
+ *     is allocated or freed; scratch (CW, deltaW_buf) is supplied by the caller.
+ *   - `streams` is an array of `length` stream handles (hipStream_t cast to int64, exactly what
+ *     the Java side holds as jlong). Work is only ENQUEUED; the caller observes completion with
+ *     events on those streams. This implementation enqueues everything on streams[0].
+ *   - Outputs are overwritten (no alpha/beta, no bias).
+ *   - `texture` variants and `useTexture` flags are performance hints in the reference; here they
+ *     select nothing (same kernels, same results).
+ *
+ * Return value: 0 on success, otherwise a hipError_t value (or ALPHA_CONV_EINVAL for arguments
+ * the kernels cannot serve). alpha_conv_last_error() returns a thread-local message.
+ */
+#ifndef ALPHA_CONV_H
+#define ALPHA_CONV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ALPHA_CONV_EINVAL 10001
+
+/* ---- library ---------------------------------------------------------------------------- */
+const char *alpha_conv_version(void);
+const char *alpha_conv_last_error(void);
+
+/* Forward algorithm used inside the forward entries when the layer is 3x3, stride 1:
+ * 0 = auto, 1 = implicit GEMM only, 2 = Winograd F(2x2,3x3) where eligible.
+ * Also read once from the environment variable ALPHA_HIP_CONV_ALGO = auto|igemm|winograd.
+ * No counterpart in the reference (its Winograd experiments are compiled out, conv/conv3D.cuh:39-44). */
+int alpha_conv_set_fwd_algo(int algo);
+int alpha_conv_get_fwd_algo(void);
+
+/* ---- Cuda_conv3D: forward ------------------------------------------------------------------ */
+
+/* conv/A.cu:14   Java: Cuda_conv3D.conv3D */
+int alpha_conv3D(const int64_t *streams, int length,
+                 const float *X, int IH, int IW,
+                 const float *W, int FH, int FW,
+                 float *Y, int OH, int OW,
+                 int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* conv/A.cu:38   Java: Cuda_conv3D.conv3D_texture */
+int alpha_conv3D_texture(const int64_t *streams, int length,
+                         const float *X, int IH, int IW,
+                         const float *W, int FH, int FW,
+                         float *Y, int OH, int OW,
+                         int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* conv/A.cu:64   Java: Cuda_conv3D.conv3DV2 */
+int alpha_conv3DV2(int useTexture, const int64_t *streams, int length,
+                   const float *X, int IH, int IW,
+                   const float *W, int FH, int FW,
+                   float *Y, int OH, int OW,
+                   int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* conv/A.cu:89   Java: Cuda_conv3D.conv3D_np  (ph = pw = 0) */
+int alpha_conv3D_np(const int64_t *streams, int length,
+                    const float *X, int IH, int IW,
+                    const float *W, int FH, int FW,
+                    float *Y, int OH, int OW,
+                    int N, int IC, int OC, int sh, int sw);
+
+/* conv/A.cu:112  Java: Cuda_conv3D.conv3D_W1  (1x1 filter, stride 1, pad 0) */
+int alpha_conv3D_W1(const int64_t *streams, int length,
+                    const float *X, int IH, int IW,
+                    const float *W, float *Y,
+                    int N, int IC, int OC);
+
+/* conv/A.cu:137  Java: Cuda_conv3D.kernel_remode   W[OC,FH,FW,IC] -> CW[FH,FW,IC,OC] */
+int alpha_kernel_remode(int64_t stream, const float *W, float *CW, int FH, int FW, int OC, int IC);
+
+/* conv/A.cu:149  Java: Cuda_conv3D.conv3D_GemmR   (CW = remoded filter; W kept for signature parity) */
+int alpha_conv3D_GemmR(const int64_t *streams, int length,
+                       const float *X, int IH, int IW,
+                       const float *W, const float *CW, int FH, int FW,
+                       float *Y, int OH, int OW,
+                       int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* conv/A.cu:174  Java: Cuda_conv3D.conv3D_GemmR_texture */
+int alpha_conv3D_GemmR_texture(const int64_t *streams, int length,
+                               const float *X, int IH, int IW,
+                               const float *W, const float *CW, int FH, int FW,
+                               float *Y, int OH, int OW,
+                               int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* conv/A.cu:201  Java: Cuda_conv3D.conv3D_GemmV2R */
+int alpha_conv3D_GemmV2R(int useTexture, const int64_t *streams, int length,
+                         const float *X, int IH, int IW,
+                         const float *W, const float *CW, int FH, int FW,
+                         float *Y, int OH, int OW,
+                         int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* conv/A.cu:227  Java: Cuda_conv3D.conv3D_GemmR_W1 */
+int alpha_conv3D_GemmR_W1(const int64_t *streams, int length,
+                          const float *X, int IH, int IW,
+                          const float *W, const float *CW, float *Y,
+                          int N, int IC, int OC);
+
+/* ---- Cuda_dconv3D_deltaX: backward-data ------------------------------------------------------ */
+
+/* dX/A.cu:14   Java: Cuda_dconv3D_deltaX.dconv3D_deltaX_s1  (stride 1) */
+int alpha_dconv3D_deltaX_s1(const int64_t *streams, int length,
+                            const float *deltaY, int OH, int OW,
+                            const float *W, int FH, int FW,
+                            float *deltaX, int IH, int IW,
+                            int N, int IC, int OC, int ph, int pw);
+
+/* dX/A.cu:38   Java: dconv3D_deltaX_s1_texture */
+int alpha_dconv3D_deltaX_s1_texture(const int64_t *streams, int length,
+                                    const float *deltaY, int OH, int OW,
+                                    const float *W, int FH, int FW,
+                                    float *deltaX, int IH, int IW,
+                                    int N, int IC, int OC, int ph, int pw);
+
+/* dX/A.cu:64   Java: dconv3D_deltaX_V2_s1 */
+int alpha_dconv3D_deltaX_V2_s1(int useTexture, const int64_t *streams, int length,
+                               const float *deltaY, int OH, int OW,
+                               const float *W, int FH, int FW,
+                               float *deltaX, int IH, int IW,
+                               int N, int IC, int OC, int ph, int pw);
+
+/* dX/A.cu:88   Java: dconv3D_deltaX_W1  (1x1, stride 1, pad 0) */
+int alpha_dconv3D_deltaX_W1(const int64_t *streams, int length,
+                            const float *deltaY, const float *W,
+                            float *deltaX, int IH, int IW,
+                            int N, int IC, int OC);
+
+/* dX/A.cu:115  Java: ks_remode   W -> CW[sh*sw][OC][CFH][CFW][IC]  (layout v1; CFH = ceil(FH/sh)) */
+int alpha_ks_remode(int64_t stream, const float *W, int FH, int FW,
+                    float *CW, int CFH, int CFW, int OC, int IC, int sh, int sw);
+
+/* dX/A.cu:128  Java: ks_remodev2 W -> CW[sh*sw][CFH][CFW][OC][IC]  (layout v2, the one consumed below) */
+int alpha_ks_remodev2(int64_t stream, const float *W, int FH, int FW,
+                      float *CW, int CFH, int CFW, int OC, int IC, int sh, int sw);
+
+/* dX/A.cu:141  Java: dconv3D_deltaX_kernelSplit  (any stride; CW in layout v2) */
+int alpha_dconv3D_deltaX_kernelSplit(const int64_t *streams, int length,
+                                     const float *deltaY, int OH, int OW,
+                                     const float *CW, int FH, int FW,
+                                     float *deltaX, int IH, int IW,
+                                     int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* dX/A.cu:166  Java: dconv3D_deltaX_ksImsR  (IH % sh == 0, IW % sw == 0) */
+int alpha_dconv3D_deltaX_ksImsR(const int64_t *streams, int length,
+                                const float *deltaY, int OH, int OW,
+                                const float *CW, int FH, int FW,
+                                float *deltaX, int IH, int IW,
+                                int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* dX/A.cu:191  Java: dconv3D_deltaX_ksImsR_texture */
+int alpha_dconv3D_deltaX_ksImsR_texture(const int64_t *streams, int length,
+                                        const float *deltaY, int OH, int OW,
+                                        const float *CW, int FH, int FW,
+                                        float *deltaX, int IH, int IW,
+                                        int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* dX/A.cu:218  Java: dconv3D_deltaX_ksIms2R  (sh = sw = 2, IH and IW even) */
+int alpha_dconv3D_deltaX_ksIms2R(const int64_t *streams, int length,
+                                 const float *deltaY, int OH, int OW,
+                                 const float *CW, int FH, int FW,
+                                 float *deltaX, int IH, int IW,
+                                 int N, int IC, int OC, int ph, int pw);
+
+/* dX/A.cu:243  Java: dconv3D_deltaX_ksIms2R_texture */
+int alpha_dconv3D_deltaX_ksIms2R_texture(const int64_t *streams, int length,
+                                         const float *deltaY, int OH, int OW,
+                                         const float *CW, int FH, int FW,
+                                         float *deltaX, int IH, int IW,
+                                         int N, int IC, int OC, int ph, int pw);
+
+/* dX/A.cu:270  Java: dconv3D_deltaX_ksV2_Ims2R */
+int alpha_dconv3D_deltaX_ksV2_Ims2R(int useTexture, const int64_t *streams, int length,
+                                    const float *deltaY, int OH, int OW,
+                                    const float *CW, int FH, int FW,
+                                    float *deltaX, int IH, int IW,
+                                    int N, int IC, int OC, int ph, int pw);
+
+/* dX/A.cu:300  Java: dconv3D_deltaX_crossAdd  (small IC; reads W, not CW).
+ * The reference zero-fills deltaX and scatters with atomicAdd (summation order varies from run
+ * to run). This implementation gathers instead: same mathematical result, no atomics, no
+ * memset, bit-reproducible. */
+int alpha_dconv3D_deltaX_crossAdd(const int64_t *streams, int length,
+                                  const float *deltaY, int OH, int OW,
+                                  const float *W, int FH, int FW,
+                                  float *deltaX, int IH, int IW,
+                                  int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* ---- Cuda_dconv3D_deltaW: backward-filter ---------------------------------------------------- */
+
+/* dW/A.cu:16   Java: Cuda_dconv3D_deltaW.dconv3D_deltaW  (single pass over GK = N*OH*OW) */
+int alpha_dconv3D_deltaW(const int64_t *streams, int length,
+                         const float *X, int IH, int IW,
+                         const float *deltaY, int OH, int OW,
+                         float *deltaW, int FH, int FW,
+                         int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* dW/A.cu:39   Java: dconv3D_deltaW_W1  (1x1, stride 1, pad 0) */
+int alpha_dconv3D_deltaW_W1(const int64_t *streams, int length,
+                            const float *X, int IH, int IW,
+                            const float *deltaY, float *deltaW,
+                            int N, int IC, int OC);
+
+/* dW/A.cu:66   Java: buf_summary   deltaW += sum_{p<part} deltaW_buf[p], fixed order, fp32 Kahan */
+int alpha_buf_summary(int64_t stream, const float *deltaW_buf, float *deltaW, int part, int sizeW);
+
+/* dW/A.cu:79   Java: dconv3D_deltaW_GemmSK.  Split-K: GK_slice = (GK/GridZ) >> 3 << 3; slice 0 is
+ * written to deltaW, slice z >= 1 to deltaW_buf[z-1] (sizeW floats each); the last slice takes the
+ * remainder. The caller sums with alpha_buf_summary(part = GridZ-1). No atomics: bit-reproducible. */
+int alpha_dconv3D_deltaW_GemmSK(const int64_t *streams, int length, int GridZ,
+                                const float *X, int IH, int IW,
+                                const float *deltaY, int OH, int OW,
+                                float *deltaW, float *deltaW_buf, int FH, int FW,
+                                int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* dW/A.cu:106  Java: dconv3D_deltaW_GemmV2SK  (same contract as GemmSK) */
+int alpha_dconv3D_deltaW_GemmV2SK(const int64_t *streams, int length, int GridZ,
+                                  const float *X, int IH, int IW,
+                                  const float *deltaY, int OH, int OW,
+                                  float *deltaW, float *deltaW_buf, int FH, int FW,
+                                  int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
+/* dW/A.cu:132  Java: dconv3D_deltaW_GemmSK_W1  (1x1 split-K) */
+int alpha_dconv3D_deltaW_GemmSK_W1(const int64_t *streams, int length, int GridZ,
+                                   const float *X, int IH, int IW,
+                                   const float *deltaY, float *deltaW, float *deltaW_buf,
+                                   int N, int IC, int OC);
+
+/* ---- this build's additional forward algorithm ------------------------------------------- */
+
+/* Winograd F(2x2,3x3) forward for FH = FW = 3, stride 1. No counterpart among the reference's
+ * JNI methods. U is scratch of alpha_winograd_filter_size(IC, OC) floats supplied by the caller
+ * (the transformed filter, 16 * IC * OC); alpha_winograd_filter_transform fills it from
+ * W[OC,3,3,IC]; alpha_conv3D_winograd then consumes it. */
+long alpha_winograd_filter_size(int IC, int OC);
+int alpha_winograd_filter_transform(int64_t stream, const float *W, float *U, int IC, int OC);
+int alpha_conv3D_winograd(const int64_t *streams, int length,
+                          const float *X, int IH, int IW,
+                          const float *U,
+                          float *Y, int OH, int OW,
+                          int N, int IC, int OC, int ph, int pw);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ALPHA_CONV_H */

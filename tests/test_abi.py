@@ -1,0 +1,57 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads and exports every symbol that
+include/alpha_conv.h declares, the JNI symbols of the three reference classes are present, and
+argument validation rejects bad calls without touching a GPU."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from util import ROOT, load_package
+
+pkg = load_package()
+
+
+def _header_functions():
+    hdr = open(os.path.join(ROOT, "include", "alpha_conv.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    return sorted(set(re.findall(r"\b(alpha_\w+)\s*\(", hdr)))
+
+
+def _exported():
+    out = subprocess.check_output(["nm", "-D", "--defined-only", pkg.lib_path()], text=True)
+    return {l.split()[-1] for l in out.splitlines() if " T " in l}
+
+
+def test_library_is_built_and_loads():
+    assert os.path.exists(pkg.lib_path()), "run __graft_entry__.build() first"
+    assert pkg.lib().alpha_conv_version().decode().startswith("alpha-conv-hip")
+
+
+def test_every_declared_symbol_is_exported():
+    declared = _header_functions()
+    assert len(declared) >= 35
+    exported = _exported()
+    missing = [f for f in declared if f not in exported]
+    assert not missing, missing
+    assert sorted(pkg.exported_symbols()) == declared  # the ctypes mirror binds exactly the header
+
+
+def test_argument_validation_without_gpu():
+    L = pkg.lib()
+    one = (ctypes.c_int64 * 1)(0)
+    p = ctypes.c_void_p(256)
+    # IC not a multiple of 4
+    rc = L.alpha_conv3D(one, 1, p, 8, 8, p, 3, 3, p, 8, 8, 4, 6, 8, 1, 1, 1, 1)
+    assert rc == 10001 and b"multiples of 4" in L.alpha_conv_last_error()
+    # empty stream array
+    rc = L.alpha_conv3D(one, 0, p, 8, 8, p, 3, 3, p, 8, 8, 4, 4, 8, 1, 1, 1, 1)
+    assert rc == 10001 and b"stream" in L.alpha_conv_last_error()
+    # null / misaligned pointer
+    rc = L.alpha_conv3D(one, 1, ctypes.c_void_p(4), 8, 8, p, 3, 3, p, 8, 8, 4, 4, 8, 1, 1, 1, 1)
+    assert rc == 10001
+    rc = L.alpha_dconv3D_deltaW_GemmSK(one, 1, 4, p, 8, 8, p, 8, 8, p, None, 3, 3, 4, 4, 8, 1, 1, 1, 1)
+    assert rc == 10001 and b"deltaW_buf" in L.alpha_conv_last_error()
+    with pytest.raises(pkg.AlphaConvError):
+        pkg.Cuda_conv3D.kernel_remode(0, 0, 0, 3, 3, 8, 4)

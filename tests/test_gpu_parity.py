@@ -1,0 +1,344 @@
+"""GPU parity tests: every C-ABI entry of the conv3D hot path against the CPU oracle.
+
+Bar (stated per test): max relative error 1e-4 with an absolute floor of 1e-5 near zero, measured
+against the fp64 oracle (ratio err/allowed <= 1), plus the reference's own pass criterion
+(Vector.samePercentRelative, thresholds of experiments/test_cuda/Cuda_conv3D_test.java:86-97,
+Cuda_dconv3D_dX_test.java:93-100, Cuda_dconv3D_dW_test.java:98-105). Index-only work (filter
+re-layouts) and the Kahan buffer summation must be bit-exact.
+"""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from util import Dev, he_normal, load_package, normal, out_dim, uniform
+
+pytestmark = pytest.mark.gpu
+
+pkg = load_package()
+C3 = pkg.Cuda_conv3D
+DX = pkg.Cuda_dconv3D_deltaX
+DW = pkg.Cuda_dconv3D_deltaW
+
+REL, ABS = 1e-4, 1e-5
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return Dev()
+
+
+def check(got, want64, what, sp_thr=1e-5, sp_min=0.999):
+    ratio = O.max_err_ratio(got, want64, REL, ABS)
+    assert ratio <= 1.0, "%s: err/allowed = %.3f (rel %g, abs floor %g)" % (what, ratio, REL, ABS)
+    sp = O.samePercentRelative(want64.astype(np.float32), got, sp_thr)
+    assert sp >= sp_min, "%s: samePercentRelative(%g) = %.5f < %g" % (what, sp_thr, sp, sp_min)
+
+
+# ----------------------------------------------------------------------------------------------
+# forward
+# ----------------------------------------------------------------------------------------------
+FWD_SHAPES = [
+    # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw
+    (4, 32, 32, 4, 64, 3, 3, 1, 1, 1, 1),      # BASELINE config 1 (IC=3 stored as 4)
+    (8, 33, 33, 64, 128, 4, 4, 1, 1, 1, 1),    # the reference's logged shape (Cuda_conv3D.java:185)
+    (4, 32, 32, 64, 252, 3, 3, 2, 2, 1, 1),    # ragged OC (Cuda_conv3D.java:191)
+    (4, 16, 16, 128, 128, 3, 3, 1, 1, 1, 1),
+    (4, 8, 8, 256, 256, 3, 3, 1, 1, 1, 1),
+    (4, 7, 7, 512, 512, 3, 3, 1, 1, 1, 1),
+    (4, 30, 30, 4, 64, 7, 7, 2, 2, 3, 3),      # stem-like
+    (4, 14, 14, 64, 128, 3, 3, 2, 2, 1, 1),
+    (4, 14, 14, 64, 128, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2 through the general entry
+    (4, 9, 11, 12, 20, 5, 5, 2, 2, 2, 2),
+    (4, 10, 9, 8, 36, 2, 2, 1, 1, 0, 0),
+    (4, 9, 9, 4, 4, 3, 2, 3, 2, 0, 1),
+    (4, 5, 5, 4, 8, 3, 3, 1, 1, 2, 2),
+    (4, 13, 13, 20, 132, 3, 3, 1, 1, 1, 1),
+]
+
+
+def _run_fwd(dev, entry, X, W, sh, sw, ph, pw):
+    N, IH, IW, IC = X.shape
+    OC, FH, FW, _ = W.shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    dXd, dWd = dev.put(X), dev.put(W)
+    Y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    S, L = dev.streams, 1
+    x, w, y = dXd.data_ptr(), dWd.data_ptr(), Y.data_ptr()
+    if entry in ("conv3D", "conv3D_texture"):
+        getattr(C3, entry)(S, L, x, IH, IW, w, FH, FW, y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+    elif entry == "conv3DV2":
+        C3.conv3DV2(True, S, L, x, IH, IW, w, FH, FW, y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+    elif entry == "conv3D_np":
+        assert ph == 0 and pw == 0
+        C3.conv3D_np(S, L, x, IH, IW, w, FH, FW, y, OH, OW, N, IC, OC, sh, sw)
+    elif entry == "conv3D_W1":
+        C3.conv3D_W1(S, L, x, IH, IW, w, y, N, IC, OC)
+    else:
+        CW = dev.empty(FH, FW, IC, OC, fill=float("nan"))
+        C3.kernel_remode(dev.stream, w, CW.data_ptr(), FH, FW, OC, IC)
+        cw = CW.data_ptr()
+        if entry in ("conv3D_GemmR", "conv3D_GemmR_texture"):
+            getattr(C3, entry)(S, L, x, IH, IW, w, cw, FH, FW, y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+        elif entry == "conv3D_GemmV2R":
+            C3.conv3D_GemmV2R(False, S, L, x, IH, IW, w, cw, FH, FW, y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+        elif entry == "conv3D_GemmR_W1":
+            C3.conv3D_GemmR_W1(S, L, x, IH, IW, w, cw, y, N, IC, OC)
+        else:
+            raise AssertionError(entry)
+    return dev.get(Y)
+
+
+@pytest.mark.parametrize("shape", FWD_SHAPES)
+@pytest.mark.parametrize("entry", ["conv3D", "conv3D_GemmR"])
+def test_forward_general_entries(dev, shape, entry):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
+    X = uniform((N, IH, IW, IC), 1001)
+    W = he_normal(OC, FH, FW, IC, 1002)
+    want = O.conv3D_f64(X, W, sh, sw, ph, pw)
+    check(_run_fwd(dev, entry, X, W, sh, sw, ph, pw), want, "%s %s" % (entry, shape))
+
+
+@pytest.mark.parametrize("entry", ["conv3D_texture", "conv3DV2", "conv3D_GemmR_texture", "conv3D_GemmV2R"])
+def test_forward_hint_variants_give_same_result(dev, entry):
+    shape = (8, 12, 12, 32, 96, 3, 3, 1, 1, 1, 1)
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
+    X, W = normal((N, IH, IW, IC), 1003), he_normal(OC, FH, FW, IC, 1004)
+    check(_run_fwd(dev, entry, X, W, sh, sw, ph, pw), O.conv3D_f64(X, W, sh, sw, ph, pw), entry)
+
+
+def test_forward_np_and_w1_entries(dev):
+    X, W = normal((4, 11, 10, 16), 1005), he_normal(40, 3, 3, 16, 1006)
+    check(_run_fwd(dev, "conv3D_np", X, W, 2, 1, 0, 0), O.conv3D_f64(X, W, 2, 1, 0, 0), "conv3D_np")
+    X, W = normal((4, 14, 14, 256), 1007), he_normal(1024, 1, 1, 256, 1008)
+    want = O.conv3D_f64(X, W, 1, 1, 0, 0)
+    check(_run_fwd(dev, "conv3D_W1", X, W, 1, 1, 0, 0), want, "conv3D_W1")
+    check(_run_fwd(dev, "conv3D_GemmR_W1", X, W, 1, 1, 0, 0), want, "conv3D_GemmR_W1")
+
+
+def test_forward_oc_sweep_covers_every_ragged_width(dev):
+    # the reference's "for OC from 1 to 128: correct" sweep (Cuda_conv3D_test.java:155-156), in steps of 4
+    X = uniform((4, 9, 9, 8), 1009)
+    for OC in range(4, 136, 4):
+        W = he_normal(OC, 3, 3, 8, 1010 + OC)
+        want = O.conv3D_f64(X, W, 1, 1, 1, 1)
+        check(_run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, 1, 1), want, "GemmR OC=%d" % OC)
+        check(_run_fwd(dev, "conv3D", X, W, 1, 1, 1, 1), want, "conv3D OC=%d" % OC)
+
+
+def test_forward_exact_small_integers(dev):
+    # all-ones tensors: every partial sum is a small integer, so the result must be bit-exact
+    X, W = np.ones((4, 7, 6, 8), np.float32), np.ones((12, 3, 3, 8), np.float32)
+    want = O.conv3D_naive(X, W, 1, 1, 1, 1)
+    assert np.array_equal(_run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, 1, 1), want)
+    assert np.array_equal(_run_fwd(dev, "conv3D", X, W, 1, 1, 1, 1), want)
+
+
+def test_kernel_remode_bit_exact(dev):
+    for (OC, FH, FW, IC) in [(64, 3, 3, 64), (8, 1, 1, 4), (252, 4, 4, 12), (4, 7, 7, 4), (132, 3, 5, 20)]:
+        W = uniform((OC, FH, FW, IC), 1011)
+        CW = dev.empty(FH, FW, IC, OC, fill=float("nan"))
+        C3.kernel_remode(dev.stream, dev.put(W).data_ptr(), CW.data_ptr(), FH, FW, OC, IC)
+        assert np.array_equal(dev.get(CW), O.kernel_remode(W))
+
+
+# ----------------------------------------------------------------------------------------------
+# backward-data
+# ----------------------------------------------------------------------------------------------
+DX_S1_SHAPES = [
+    (4, 32, 32, 64, 64, 3, 3, 1, 1),     # N, IH, IW, IC, OC, FH, FW, ph, pw
+    (4, 31, 31, 128, 32, 4, 4, 1, 1),    # Cuda_dconv3D_deltaX.java:259 (OH=31-ish)
+    (4, 16, 16, 256, 64, 3, 3, 1, 1),
+    (4, 8, 8, 256, 256, 3, 3, 1, 1),
+    (4, 9, 10, 12, 20, 5, 5, 2, 2),
+    (4, 9, 9, 8, 8, 3, 3, 0, 0),
+    (4, 7, 9, 4, 36, 3, 2, 2, 1),
+    (4, 12, 12, 132, 44, 3, 3, 1, 1),
+]
+
+
+@pytest.mark.parametrize("shape", DX_S1_SHAPES)
+def test_deltaX_s1_entries(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, ph, pw = shape
+    OH, OW = out_dim(IH, IW, FH, FW, 1, 1, ph, pw)
+    dY, W = normal((N, OH, OW, OC), 2001), he_normal(OC, FH, FW, IC, 2002)
+    want = O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw)
+    dy, w = dev.put(dY), dev.put(W)
+    for entry in ("dconv3D_deltaX_s1", "dconv3D_deltaX_s1_texture", "dconv3D_deltaX_V2_s1"):
+        dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+        args = (dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC, ph, pw)
+        if entry == "dconv3D_deltaX_V2_s1":
+            DX.dconv3D_deltaX_V2_s1(True, *args)
+        else:
+            getattr(DX, entry)(*args)
+        check(dev.get(dXo), want, "%s %s" % (entry, shape), sp_thr=1e-4)
+
+
+def test_deltaX_W1(dev):
+    for (N, IH, IW, IC, OC) in [(4, 14, 14, 256, 64), (4, 9, 7, 64, 256), (4, 5, 5, 12, 20)]:
+        dY, W = normal((N, IH, IW, OC), 2003), he_normal(OC, 1, 1, IC, 2004)
+        dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+        DX.dconv3D_deltaX_W1(dev.streams, 1, dev.put(dY).data_ptr(), dev.put(W).data_ptr(), dXo.data_ptr(), IH, IW, N, IC, OC)
+        check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, 0, 0), "deltaX_W1", sp_thr=1e-4)
+
+
+KS_SHAPES = [
+    # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw
+    (4, 16, 16, 64, 128, 3, 3, 2, 2, 1, 1),
+    (4, 32, 32, 64, 32, 4, 4, 2, 2, 1, 1),
+    (4, 14, 14, 32, 64, 1, 1, 2, 2, 0, 0),
+    (4, 16, 12, 16, 24, 5, 5, 2, 2, 2, 2),
+    (4, 12, 12, 20, 16, 7, 7, 2, 2, 3, 3),
+    (4, 12, 9, 16, 16, 3, 3, 3, 3, 1, 1),     # Ims: IH % sh == 0
+    (4, 13, 11, 16, 16, 5, 4, 3, 2, 2, 1),    # general kernel split (IH % sh != 0)
+    (4, 9, 9, 12, 8, 2, 2, 2, 2, 0, 0),       # odd IH with stride 2
+]
+
+
+@pytest.mark.parametrize("shape", KS_SHAPES)
+def test_deltaX_kernel_split_family(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    dY, W = normal((N, OH, OW, OC), 2005), he_normal(OC, FH, FW, IC, 2006)
+    want = O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw)
+    CFH, CFW = O.ks_dims(FH, FW, sh, sw)
+    dy, w = dev.put(dY), dev.put(W)
+    CW = dev.empty(sh * sw * OC * CFH * CFW * IC, fill=0.0)
+    DX.ks_remodev2(dev.stream, w.data_ptr(), FH, FW, CW.data_ptr(), CFH, CFW, OC, IC, sh, sw)
+    assert np.array_equal(dev.get(CW), O.ks_remodev2(W, sh, sw)), "ks_remodev2 layout"
+    CW1 = dev.empty(sh * sw * OC * CFH * CFW * IC, fill=0.0)
+    DX.ks_remode(dev.stream, w.data_ptr(), FH, FW, CW1.data_ptr(), CFH, CFW, OC, IC, sh, sw)
+    assert np.array_equal(dev.get(CW1), O.ks_remode(W, sh, sw)), "ks_remode layout"
+
+    entries = ["dconv3D_deltaX_kernelSplit"]
+    if IH % sh == 0 and IW % sw == 0:
+        entries += ["dconv3D_deltaX_ksImsR", "dconv3D_deltaX_ksImsR_texture"]
+    if sh == 2 and sw == 2 and IH % 2 == 0 and IW % 2 == 0:
+        entries += ["dconv3D_deltaX_ksIms2R", "dconv3D_deltaX_ksIms2R_texture", "dconv3D_deltaX_ksV2_Ims2R"]
+    for entry in entries:
+        dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+        base = (dev.streams, 1, dy.data_ptr(), OH, OW, CW.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC)
+        if entry == "dconv3D_deltaX_ksV2_Ims2R":
+            DX.dconv3D_deltaX_ksV2_Ims2R(False, *base, ph, pw)
+        elif "Ims2R" in entry:
+            getattr(DX, entry)(*base, ph, pw)
+        else:
+            getattr(DX, entry)(*base, sh, sw, ph, pw)
+        check(dev.get(dXo), want, "%s %s" % (entry, shape), sp_thr=1e-4)
+
+
+@pytest.mark.parametrize("shape", [
+    (4, 16, 16, 4, 64, 7, 7, 2, 2, 3, 3),      # stem backward (IC = 3 stored as 4)
+    (4, 12, 12, 8, 32, 3, 3, 1, 1, 1, 1),
+    (4, 12, 12, 16, 32, 4, 4, 2, 2, 1, 1),
+    (4, 11, 13, 8, 12, 3, 3, 3, 2, 1, 0),
+])
+def test_deltaX_crossAdd_is_deterministic_gather(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    dY, W = normal((N, OH, OW, OC), 2007), he_normal(OC, FH, FW, IC, 2008)
+    dy, w = dev.put(dY), dev.put(W)
+    outs = []
+    for _ in range(2):
+        dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+        DX.dconv3D_deltaX_crossAdd(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW,
+                                   N, IC, OC, sh, sw, ph, pw)
+        outs.append(dev.get(dXo))
+    check(outs[0], O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw), "crossAdd %s" % (shape,), sp_thr=1e-4)
+    assert np.array_equal(outs[0], outs[1])
+
+
+# ----------------------------------------------------------------------------------------------
+# backward-filter
+# ----------------------------------------------------------------------------------------------
+DW_SHAPES = [
+    # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw
+    (4, 32, 32, 64, 64, 3, 3, 1, 1, 1, 1),
+    (4, 32, 32, 64, 256, 4, 4, 2, 2, 1, 1),    # Cuda_dconv3D_deltaW.java:327
+    (8, 8, 8, 256, 256, 3, 3, 1, 1, 1, 1),
+    (4, 16, 16, 4, 64, 7, 7, 2, 2, 3, 3),
+    (4, 13, 11, 12, 20, 5, 3, 2, 1, 2, 1),
+    (4, 9, 9, 132, 36, 3, 3, 1, 1, 1, 1),
+]
+
+
+def _sum_partials(dev, dWo, buf, GridZ):
+    DW.buf_summary(dev.stream, buf.data_ptr(), dWo.data_ptr(), GridZ - 1, dWo.numel())
+    return dev.get(dWo)
+
+
+@pytest.mark.parametrize("shape", DW_SHAPES)
+def test_deltaW_entries(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    X, dY = normal((N, IH, IW, IC), 3001), normal((N, OH, OW, OC), 3002)
+    want = O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw)
+    x, dy = dev.put(X), dev.put(dY)
+    dWo = dev.empty(OC, FH, FW, IC, fill=float("nan"))
+    DW.dconv3D_deltaW(dev.streams, 1, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
+    check(dev.get(dWo), want, "dconv3D_deltaW %s" % (shape,), sp_min=1.0)
+    sizeW = OC * FH * FW * IC
+    for entry in ("dconv3D_deltaW_GemmSK", "dconv3D_deltaW_GemmV2SK"):
+        for GridZ in (2, 5, 16):
+            dWo = dev.empty(OC, FH, FW, IC, fill=float("nan"))
+            buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+            getattr(DW, entry)(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
+                               FH, FW, N, IC, OC, sh, sw, ph, pw)
+            check(_sum_partials(dev, dWo, buf, GridZ), want, "%s GridZ=%d %s" % (entry, GridZ, shape), sp_min=1.0)
+
+
+def test_deltaW_split_k_slices_follow_the_reference_partition(dev):
+    # slice z must hold exactly k in [z*GK_slice, ...) with GK_slice = (GK/GZ)>>3<<3, the last slice the rest
+    N, IH, IW, IC, OC, F_, s, p = 4, 9, 9, 8, 8, 3, 1, 1
+    OH, OW = out_dim(IH, IW, F_, F_, s, s, p, p)
+    X, dY = normal((N, IH, IW, IC), 3003), normal((N, OH, OW, OC), 3004)
+    x, dy = dev.put(X), dev.put(dY)
+    GridZ, sizeW = 5, OC * F_ * F_ * IC
+    dWo = dev.empty(OC, F_, F_, IC, fill=float("nan"))
+    buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+    DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
+                             F_, F_, N, IC, OC, s, s, p, p)
+    parts = [dev.get(dWo)] + [b.reshape(OC, F_, F_, IC) for b in dev.get(buf)]
+    for z in range(GridZ):
+        check(parts[z], O.deltaW_slice_f64(X, dY, F_, F_, s, s, p, p, GridZ, z), "slice %d" % z, sp_min=0.99)
+
+
+def test_deltaW_W1_entries(dev):
+    for (N, IH, IW, IC, OC) in [(4, 14, 14, 256, 64), (4, 12, 12, 64, 256), (4, 7, 9, 12, 20)]:
+        X, dY = normal((N, IH, IW, IC), 3005), normal((N, IH, IW, OC), 3006)
+        want = O.deltaW_f64(X, dY, 1, 1, 1, 1, 0, 0)
+        x, dy = dev.put(X), dev.put(dY)
+        dWo = dev.empty(OC, 1, 1, IC, fill=float("nan"))
+        DW.dconv3D_deltaW_W1(dev.streams, 1, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), N, IC, OC)
+        check(dev.get(dWo), want, "deltaW_W1", sp_min=1.0)
+        GridZ = 3
+        dWo = dev.empty(OC, 1, 1, IC, fill=float("nan"))
+        buf = dev.empty(GridZ - 1, OC * IC, fill=float("nan"))
+        DW.dconv3D_deltaW_GemmSK_W1(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), buf.data_ptr(), N, IC, OC)
+        check(_sum_partials(dev, dWo, buf, GridZ), want, "deltaW_GemmSK_W1", sp_min=1.0)
+
+
+def test_buf_summary_bit_exact_kahan(dev):
+    r = np.random.Generator(np.random.PCG64(3007))
+    for part, sizeW in [(1, 64), (15, 36864), (127, 2308), (3, 8)]:
+        buf = (r.standard_normal((part, sizeW)) * 10.0 ** r.integers(-3, 4, (part, sizeW))).astype(np.float32)
+        dw = r.standard_normal(sizeW).astype(np.float32)
+        d = dev.put(dw)
+        DW.buf_summary(dev.stream, dev.put(buf).data_ptr(), d.data_ptr(), part, sizeW)
+        assert np.array_equal(dev.get(d), O.buf_summary(buf, dw)), (part, sizeW)
+
+
+def test_deltaW_bit_reproducible_run_to_run(dev):
+    # BASELINE config 5 requirement at reduced N: identical bits for identical (shape, GridZ)
+    N, IH, IW, IC, OC = 4, 56, 56, 64, 64
+    X, dY = normal((N, IH, IW, IC), 3008), normal((N, IH, IW, OC), 3009)
+    x, dy = dev.put(X), dev.put(dY)
+    GridZ, sizeW = 16, OC * 9 * IC
+    outs = []
+    for _ in range(3):
+        dWo = dev.empty(OC, 3, 3, IC, fill=float("nan"))
+        buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+        DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), IH, IW, dWo.data_ptr(), buf.data_ptr(),
+                                 3, 3, N, IC, OC, 1, 1, 1, 1)
+        outs.append(_sum_partials(dev, dWo, buf, GridZ))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    check(outs[0], O.deltaW_f64(X, dY, 3, 3, 1, 1, 1, 1), "config-5b dW (N=4)", sp_min=1.0)
