@@ -10,6 +10,7 @@ AlphaConvError.
 """
 import ctypes
 import os
+import sys
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_NAME = "libalpha_conv_hip.so"
@@ -71,6 +72,26 @@ def exported_symbols():
                                  "alpha_conv_get_fwd_algo", "alpha_winograd_filter_size"])
 
 
+def _preload_hip_runtime():
+    """A process must hold exactly ONE HIP runtime. PyTorch wheels bundle their own libamdhip64.so
+    (same SONAME as /opt/rocm's, different file); a second copy in the process finds no device.
+    When torch is installed, map its copy first so that this library's NEEDED libamdhip64.so.7
+    binds to it; a later `import torch` then re-uses the same file. Without torch the loader
+    takes the system runtime as usual."""
+    import importlib.util
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.origin:
+        return
+    cand = os.path.join(os.path.dirname(spec.origin), "lib", "libamdhip64.so")
+    if os.path.exists(cand):
+        ctypes.CDLL(cand, mode=ctypes.RTLD_GLOBAL)
+
+
 def lib():
     """Loads the HIP library; raises if it has not been built (there is no fallback path)."""
     global _lib
@@ -78,6 +99,7 @@ def lib():
         path = lib_path()
         if not os.path.exists(path):
             raise AlphaConvError("%s is not built: run `python %s`" % (path, os.path.join(_HERE, "build.py")))
+        _preload_hip_runtime()
         L = ctypes.CDLL(path)
         for name, sig in _SIGS.items():
             fn = getattr(L, name)
