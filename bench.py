@@ -247,7 +247,8 @@ def main():
 
     head = measure(pkg, torch, args.layer, op, args.steps, args.warmup)
     props = torch.cuda.get_device_properties(0)
-    cus, clk_ghz = props.multi_processor_count, props.clock_rate / 1e6
+    cus, clk_khz = pkg.device_info()
+    clk_ghz = clk_khz / 1e6
     N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[args.layer]
     out = {
         "metric": "conv fwd/bwd TFLOP/s (fp32) + % of MI355X fp32 MFMA peak, 1 GPU",

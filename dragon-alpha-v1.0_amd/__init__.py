@@ -6,4 +6,4 @@ from csrc/. This Python package is only a thin ctypes mirror of the reference's 
 falls back to a CPU or PyTorch implementation: if the library is missing, loading raises.
 """
 from .native import (Cuda_conv3D, Cuda_dconv3D_deltaX, Cuda_dconv3D_deltaW, AlphaConvError, lib, lib_path,  # noqa: F401
-                     exported_symbols)
+                     exported_symbols, device_info)

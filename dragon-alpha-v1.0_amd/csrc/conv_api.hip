@@ -181,6 +181,17 @@ extern "C" {
 const char *alpha_conv_version(void) { return "alpha-conv-hip gfx950 0.1"; }
 const char *alpha_conv_last_error(void) { return g_err; }
 
+int alpha_conv_device_info(int *compute_units, int *clock_khz)
+{
+    int dev = 0, cu = 0, clk = 0;
+    if (int e = hip_status(hipGetDevice(&dev), __func__)) return e;
+    if (int e = hip_status(hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev), __func__)) return e;
+    if (int e = hip_status(hipDeviceGetAttribute(&clk, hipDeviceAttributeClockRate, dev), __func__)) return e;
+    if (compute_units) *compute_units = cu;
+    if (clock_khz) *clock_khz = clk;
+    return 0;
+}
+
 static int g_fwd_algo = -1;
 int alpha_conv_get_fwd_algo(void)
 {

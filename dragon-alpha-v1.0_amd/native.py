@@ -68,7 +68,7 @@ def lib_path():
 
 def exported_symbols():
     """Names the C ABI must export (every function include/alpha_conv.h declares)."""
-    return sorted(list(_SIGS) + ["alpha_conv_version", "alpha_conv_last_error", "alpha_conv_set_fwd_algo",
+    return sorted(list(_SIGS) + ["alpha_conv_version", "alpha_conv_last_error", "alpha_conv_device_info", "alpha_conv_set_fwd_algo",
                                  "alpha_conv_get_fwd_algo", "alpha_winograd_filter_size"])
 
 
@@ -136,6 +136,15 @@ def _call(name, *args):
     rc = getattr(L, name)(*conv)
     if rc != 0:
         raise AlphaConvError("%s failed (%d): %s" % (name, rc, L.alpha_conv_last_error().decode()))
+
+
+def device_info():
+    """(compute units, peak clock in kHz) of the current device."""
+    cu, clk = ctypes.c_int(0), ctypes.c_int(0)
+    rc = lib().alpha_conv_device_info(ctypes.byref(cu), ctypes.byref(clk))
+    if rc != 0:
+        raise AlphaConvError("alpha_conv_device_info failed (%d): %s" % (rc, lib().alpha_conv_last_error().decode()))
+    return cu.value, clk.value
 
 
 class Cuda_conv3D:

@@ -44,6 +44,11 @@ extern "C" {
 const char *alpha_conv_version(void);
 const char *alpha_conv_last_error(void);
 
+/* Compute-unit count and peak engine clock (kHz) of the current device. Stands in for the one
+ * field of the reference's CudaDevice class this path uses: the multiprocessor count that caps the
+ * split-K factor (CudaFloat32EngineBase.java:73). */
+int alpha_conv_device_info(int *compute_units, int *clock_khz);
+
 /* Forward algorithm used inside the forward entries when the layer is 3x3, stride 1:
  * 0 = auto, 1 = implicit GEMM only, 2 = Winograd F(2x2,3x3) where eligible.
  * Also read once from the environment variable ALPHA_HIP_CONV_ALGO = auto|igemm|winograd.

@@ -1,0 +1,94 @@
+"""The JNI layer: every `static native` method of the reference's three conv classes resolves to an
+exported symbol with the JNI-mangled name, and the stubs drive the C ABI through a fake JNIEnv
+(stream-array copy, error -> Java exception). There is no JVM in this environment, so this proves the
+shim's self-consistency with the JNI specification's table layout, not execution inside a real JVM."""
+import ctypes
+import subprocess
+
+import numpy as np
+import pytest
+
+from fake_jni import FakeEnv
+from util import load_package
+
+pkg = load_package()
+
+# `static native` method names as declared in the reference's Java classes
+NATIVES = {
+    "Cuda_conv3D": ["conv3D", "conv3D_texture", "conv3DV2", "conv3D_np", "conv3D_W1", "kernel_remode", "conv3D_GemmR",
+                    "conv3D_GemmR_texture", "conv3D_GemmV2R", "conv3D_GemmR_W1"],
+    "Cuda_dconv3D_deltaX": ["dconv3D_deltaX_s1", "dconv3D_deltaX_s1_texture", "dconv3D_deltaX_V2_s1", "dconv3D_deltaX_W1",
+                            "ks_remode", "ks_remodev2", "dconv3D_deltaX_kernelSplit", "dconv3D_deltaX_ksImsR",
+                            "dconv3D_deltaX_ksImsR_texture", "dconv3D_deltaX_ksIms2R", "dconv3D_deltaX_ksIms2R_texture",
+                            "dconv3D_deltaX_ksV2_Ims2R", "dconv3D_deltaX_crossAdd"],
+    "Cuda_dconv3D_deltaW": ["dconv3D_deltaW", "dconv3D_deltaW_W1", "buf_summary", "dconv3D_deltaW_GemmSK",
+                            "dconv3D_deltaW_GemmV2SK", "dconv3D_deltaW_GemmSK_W1"],
+}
+
+
+def mangle(cls, method):
+    esc = lambda s: s.replace("_", "_1")
+    return "Java_z_dragon_engine_cuda_impl_math_%s_%s" % (esc(cls), esc(method))
+
+
+def test_all_29_jni_symbols_exported():
+    out = subprocess.check_output(["nm", "-D", "--defined-only", pkg.lib_path()], text=True)
+    exported = {l.split()[-1] for l in out.splitlines() if " T " in l}
+    want = [mangle(c, m) for c, ms in NATIVES.items() for m in ms]
+    assert len(want) == 29
+    assert not [w for w in want if w not in exported]
+    assert len([e for e in exported if e.startswith("Java_")]) == 29   # nothing extra either
+
+
+def _jni(name):
+    return getattr(pkg.lib(), name)
+
+
+def test_error_becomes_java_exception_and_streams_are_copied():
+    env = FakeEnv()
+    fn = _jni(mangle("Cuda_conv3D", "conv3D"))
+    fn.restype = None
+    L, I, P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
+    fn.argtypes = [P, P, P, I, L, I, I, L, I, I, L, I, I, I, I, I, I, I, I, I]
+    arr = env.long_array([0, 0, 0])
+    # IC = 6 is not a multiple of 4 -> the C ABI refuses before touching the GPU -> ThrowNew(CudaException)
+    fn(env.ptr, None, arr, 3, 256, 8, 8, 256, 3, 3, 256, 8, 8, 4, 6, 8, 1, 1, 1, 1)
+    assert env.thrown and env.thrown[0][0] == "z/dragon/engine/cuda/impl/CudaException"
+    assert "multiples of 4" in env.thrown[0][1]
+    # class lookup falls back when the engine's class is absent
+    env2 = FakeEnv(known_classes=("java/lang/RuntimeException",))
+    fn(env2.ptr, None, env2.long_array([0]), 1, 256, 8, 8, 256, 3, 3, 256, 8, 8, 4, 6, 8, 1, 1, 1, 1)
+    assert env2.find_calls == ["z/dragon/engine/cuda/impl/CudaException", "z/jcuda/exception/CudaException",
+                               "java/lang/RuntimeException"]
+    assert env2.cleared == 2 and env2.thrown[0][0] == "java/lang/RuntimeException"
+    # an empty stream array is refused, not dereferenced
+    env3 = FakeEnv()
+    fn(env3.ptr, None, env3.long_array([]), 0, 256, 8, 8, 256, 3, 3, 256, 8, 8, 4, 4, 8, 1, 1, 1, 1)
+    assert "stream" in env3.thrown[0][1]
+
+
+@pytest.mark.gpu
+def test_forward_through_jni_symbols_on_gpu():
+    from oracle import oracle as O
+    from util import Dev, he_normal, uniform
+    dev = Dev()
+    N, IH, IW, IC, OC, F_ = 4, 12, 12, 16, 40, 3
+    X, W = uniform((N, IH, IW, IC), 5001), he_normal(OC, F_, F_, IC, 5002)
+    x, w = dev.put(X), dev.put(W)
+    cw = dev.empty(F_ * F_ * IC * OC, fill=float("nan"))
+    y = dev.empty(N, IH, IW, OC, fill=float("nan"))
+    env = FakeEnv()
+    L, I, P, Z = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p, ctypes.c_uint8
+    remode = _jni(mangle("Cuda_conv3D", "kernel_remode"))
+    remode.restype, remode.argtypes = None, [P, P, L, L, L, I, I, I, I]
+    remode(env.ptr, None, dev.stream, w.data_ptr(), cw.data_ptr(), F_, F_, OC, IC)
+    conv = _jni(mangle("Cuda_conv3D", "conv3D_GemmV2R"))
+    conv.restype = None
+    conv.argtypes = [P, P, Z, P, I, L, I, I, L, L, I, I, L, I, I, I, I, I, I, I, I, I]
+    streams = env.long_array([dev.stream] * 3)
+    conv(env.ptr, None, 1, streams, 3, x.data_ptr(), IH, IW, w.data_ptr(), cw.data_ptr(), F_, F_, y.data_ptr(), IH, IW,
+         N, IC, OC, 1, 1, 1, 1)
+    assert not env.thrown
+    want = O.conv3D_f64(X, W, 1, 1, 1, 1)
+    floor = 1e-5 * max(1.0, float(np.sqrt(np.mean(want * want))))
+    assert O.max_err_ratio(dev.get(y), want, 1e-4, floor) <= 1.0
