@@ -179,11 +179,14 @@ def cpu_baseline(layer, op, budget_s=12.0):
     n0 = min(N, max(1, cores // 4))
     t_probe = run(n0)
     n = int(max(n0, min(N, n0 * budget_s / max(t_probe, 1e-6))))
-    t = run(n) if n > n0 else t_probe
+    t1 = run(n) if n > n0 else t_probe
     n_used = n if n > n0 else n0
+    reps = int(max(1, min(200, budget_s / max(t1, 1e-6))))   # repeat the subset until ~budget_s of CPU work is timed
+    t = sum(run(n_used) for _ in range(reps))
     return {
-        "value": round(per_image * n_used / t / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-        "sample": "%s %s on %d of %d images (%.2f s, OpenMP over n,oh; float accumulate, direct loops)" % (layer, op, n_used, N, t),
+        "value": round(per_image * n_used * reps / t / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": "%s %s on %d of %d images x %d repeats (%.1f s total, OpenMP over n,oh; float accumulate, direct loops)"
+                  % (layer, op, n_used, N, reps, t),
     }
 
 
@@ -231,6 +234,8 @@ def main():
     ap.add_argument("--op", default=None, choices=["fwd", "dx", "dw"])
     ap.add_argument("--layers", action="store_true", help="also measure every layer/op of BASELINE.json's configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--probe-copy", action="store_true",
+                    help="only run a plain 256 MiB device-to-device copy a few times (calibrates FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -239,6 +244,14 @@ def main():
         sys.exit(2)
 
     import torch
+    if args.probe_copy:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "copy", "bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}))
+        return
     from __graft_entry__ import package
     pkg = package()
     pkg.lib()   # raises if the HIP library is not built; there is no fallback

@@ -54,6 +54,14 @@ struct GatherConvArgs {
 
 hipError_t launch_gather_conv(hipStream_t stream, const GatherConvArgs &a, int TH, int TW, int OHt, int OWt, int N);
 
+// Stride-1 convolution with the input window staged once in LDS (tap_conv.hip). B must be contiguous
+// along the output channel: element (th, tw, c, co) at b_off + th*b_sth + tw*b_stw + c*b_sc + co.
+// Returns hipErrorNotSupported (nothing launched) when the shape does not fit.
+hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
+                           int N, int AH, int AW, int AC, int OH, int OW, int CO,
+                           int TH, int TW, int ph, int pw,
+                           int b_off, int b_sth, int b_stw, int b_sc);
+
 // Backward-filter implicit GEMM with split-K over k = (n, oh, ow):
 //   dst_z[oc, fh, fw, ic] = sum_{k in slice z} deltaY[k, oc] * X[n, oh*sh - ph + fh, ow*sw - pw + fw, ic]
 // slice z = [z*GK_slice, (z+1)*GK_slice), the last one running to GK; dst_0 = deltaW,

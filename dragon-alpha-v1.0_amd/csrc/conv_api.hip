@@ -56,6 +56,21 @@ int check_dims(const char *fn, int N, int IC, int OC, int IH, int IW, int OH, in
 
 enum FilterLayout { FILTER_W, FILTER_CW };
 
+int g_fwd_algo = -1;   // -1: not yet read from the environment
+
+int fwd_algo()
+{
+    if (g_fwd_algo < 0) {
+        const char *e = getenv("ALPHA_HIP_CONV_ALGO");
+        int v = 0;
+        if (e && !strcmp(e, "igemm")) v = 1;
+        else if (e && !strcmp(e, "winograd")) v = 2;
+        else if (e && !strcmp(e, "generic")) v = 3;
+        g_fwd_algo = v;
+    }
+    return g_fwd_algo;
+}
+
 // Forward: Y = conv(X, filter). FILTER_W reads W[OC,FH,FW,IC]; FILTER_CW reads CW[FH,FW,IC,OC].
 int forward(const char *fn, const int64_t *streams, int length,
             const float *X, int IH, int IW, const float *F, FilterLayout layout, int FH, int FW,
@@ -65,6 +80,12 @@ int forward(const char *fn, const int64_t *streams, int length,
     if (!X || !F || !Y || !aligned16(X) || !aligned16(F) || !aligned16(Y))
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
+
+    if (layout == FILTER_CW && sh == 1 && sw == 1 && fwd_algo() != 3) {
+        hipError_t e = launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
+                                       0, FW * IC * OC, IC * OC, OC);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
 
     GatherConvArgs a{};
     a.A = X; a.B = F; a.O = Y;
@@ -92,6 +113,12 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, 1, 1, ph, pw)) return e;
     if (FH - 1 - ph < 0 || FW - 1 - pw < 0) return fail(ALPHA_CONV_EINVAL, "%s: padding larger than FH-1", fn);
+
+    if (fwd_algo() != 3) {
+        hipError_t e = launch_tap_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, FH - 1 - ph, FW - 1 - pw,
+                                       ((FH - 1) * FW + (FW - 1)) * IC, -FW * IC, -IC, FH * FW * IC);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
 
     GatherConvArgs a{};
     a.A = dY; a.B = W; a.O = dX;
@@ -192,21 +219,10 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz)
     return 0;
 }
 
-static int g_fwd_algo = -1;
-int alpha_conv_get_fwd_algo(void)
-{
-    if (g_fwd_algo < 0) {
-        const char *e = getenv("ALPHA_HIP_CONV_ALGO");
-        int v = 0;
-        if (e && !strcmp(e, "igemm")) v = 1;
-        else if (e && !strcmp(e, "winograd")) v = 2;
-        g_fwd_algo = v;
-    }
-    return g_fwd_algo;
-}
+int alpha_conv_get_fwd_algo(void) { return fwd_algo(); }
 int alpha_conv_set_fwd_algo(int algo)
 {
-    if (algo < 0 || algo > 2) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0, 1 or 2");
+    if (algo < 0 || algo > 3) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..3");
     g_fwd_algo = algo;
     return 0;
 }

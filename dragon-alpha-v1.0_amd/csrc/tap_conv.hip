@@ -1,0 +1,282 @@
+// Stride-1 convolution with the input window staged ONCE in LDS ("tap convolution"), fp32 MFMA
+// v_mfma_f32_16x16x4_f32, gfx950. Serves forward 3x3/5x5... stride 1 and stride-1 backward-data.
+//
+// A workgroup (4 wavefronts) owns P = 16*TILES consecutive output pixels of the flattened
+// (n, oh, ow) index and a slice of 64 output channels. For each chunk of 64 input channels it
+//   1. copies the zero-padded input rows those pixels touch into LDS once
+//      (rows are "padded global rows" n*(AH+2ph) + ih + ph, so a pixel range may cross image borders);
+//   2. walks the filter in "half taps" (one tap, 32 input channels): the 32x64 filter slice is staged
+//      in one of two LDS buffers while the MFMAs of the previous half tap run (one barrier per half
+//      tap); every lane reads its pixel's 4 consecutive channels with one 128-bit LDS read at
+//      base(pixel) + tap offset — no address arithmetic or bounds tests in the inner loop.
+// Each input element is read from memory once per workgroup instead of once per tap.
+//
+// Wavefront w computes output channels [16w, 16w+16) for all TILES pixel tiles (TILES*4 accumulator
+// registers). Operand fragments are double-buffered in registers: the LDS reads of channel group
+// g+1 are issued before the MFMAs of group g.
+//
+// LDS layouts (floats):
+//   halo  [row][col][64+4]      pixel stride 68: the 16 lanes of a 128-bit read hit distinct banks
+//   filter[2][8][64 oc][4]      the 4 channels a lane needs at one output channel are contiguous, so
+//                               the B fragment is a single 128-bit read, lanes contiguous
+// K permutation inside a group of 16 channels: lane group q = lane/16 supplies channel 16g + 4q + s
+// at MFMA step s, for both operands.
+#include "common.hpp"
+
+namespace alpha {
+
+struct TapConvArgs {
+    const float *A;   // input activations [N, AH, AW, AC]
+    const float *B;   // filter; element (th, tw, c, co) at b_off + th*b_sth + tw*b_stw + c*b_sc + co
+    float *O;         // output [N, OH, OW, CO] dense
+    int M, CO;        // N*OH*OW pixels, output channels
+    int AH, AW, AC;
+    int TH, TW, ph, pw;
+    int PHt, PWt;     // AH + 2ph, AW + 2pw
+    int lds_rows;     // halo rows reserved in LDS
+    int b_off, b_sth, b_stw, b_sc;
+    FastDiv d_OW, d_OHW, d_PHt, d_PWt;
+};
+
+constexpr int TC_ICC = 64;            // input channels per halo pass
+constexpr int TC_PS = TC_ICC + 4;     // LDS pixel stride (floats)
+constexpr int TC_WBUF = 8 * 64 * 4;   // floats per filter buffer (32 channels x 64 output channels)
+constexpr int TC_OS = 64 + 4;         // output staging row stride (floats)
+
+template <int TILES>
+__global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
+{
+    constexpr int P = TILES * 16;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float *Ws = smem;                       // [2][TC_WBUF]
+    float *Hs = smem + 2 * TC_WBUF;         // [lds_rows][PWt][TC_PS]; reused as output staging [P][TC_OS]
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = t >> 6;
+    const int l16 = lane & 15, q = lane >> 4;
+
+    const int m0 = blockIdx.x * P;
+    const int oc0 = blockIdx.y * 64;
+    const int OW = p.d_OW.d, OHW = p.d_OHW.d, PHt = p.PHt, PWt = p.PWt;
+
+    // first padded global row held in LDS, and how many rows this unit needs (<= p.lds_rows, host-checked)
+    const int n_first = fdiv(m0, p.d_OHW);
+    const int oh_first = fdiv(m0 - n_first * OHW, p.d_OW);
+    const int pgr0 = n_first * PHt + oh_first;
+    const int m_last = min(m0 + P, p.M) - 1;
+    const int n_last = fdiv(m_last, p.d_OHW);
+    const int oh_last = fdiv(m_last - n_last * OHW, p.d_OW);
+    const int rows = n_last * PHt + oh_last + p.TH - 1 - pgr0 + 1;
+
+    // per-lane LDS offset (floats) of each tile's pixel at tap (0,0), plus this lane group's channel offset
+    int abase[TILES];
+#pragma unroll
+    for (int i = 0; i < TILES; i++) {
+        const int m = min(m0 + 16 * i + l16, p.M - 1);
+        const int n = fdiv(m, p.d_OHW), rem = m - n * OHW;
+        const int oh = fdiv(rem, p.d_OW), ow = rem - oh * OW;
+        abase[i] = ((n * PHt + oh - pgr0) * PWt + ow) * TC_PS + 4 * q;
+    }
+    const int bbase = (q * 64 + 16 * w + l16) * 4;
+
+    floatx4 acc[TILES];
+#pragma unroll
+    for (int i = 0; i < TILES; i++) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // ---- filter staging: thread (Q = t/32, pair = t%32) moves channels 4Q..4Q+3 of two output channels ----
+    const int w_Q = t >> 5, w_oc = (t & 31) * 2;
+    const bool w_colv = oc0 + w_oc < p.CO;
+    float2 wreg[4];
+    bool wok = false;
+    // Loads are issued unconditionally from a clamped (always valid) address; the zeroing of invalid
+    // channels happens when the registers are stored to LDS, so nothing waits on the loads before the
+    // MFMAs of the current half tap have been issued.
+    auto load_filter = [&](int icbase, int th, int tw) {   // icbase: first of the 32 channels of this half tap
+        const int base = p.b_off + th * p.b_sth + tw * p.b_stw + oc0 + w_oc;
+        const int c = icbase + 4 * w_Q;
+        wok = w_colv && c < p.AC;   // AC % 4 == 0: the four channels are valid together
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+            wreg[s] = *reinterpret_cast<const float2 *>(p.B + ((base + (c + s) * p.b_sc) & -(int)wok));
+    };
+    auto store_filter = [&](int buf) {
+        float *dst = Ws + buf * TC_WBUF + (w_Q * 64 + w_oc) * 4;
+        *reinterpret_cast<float4 *>(dst) = make_float4(wok ? wreg[0].x : 0.f, wok ? wreg[1].x : 0.f,
+                                                       wok ? wreg[2].x : 0.f, wok ? wreg[3].x : 0.f);
+        *reinterpret_cast<float4 *>(dst + 4) = make_float4(wok ? wreg[0].y : 0.f, wok ? wreg[1].y : 0.f,
+                                                           wok ? wreg[2].y : 0.f, wok ? wreg[3].y : 0.f);
+    };
+
+    const int halo_quads = rows * PWt * (TC_ICC / 4);
+    const int taps = p.TH * p.TW;
+    const int steps = taps * 2;   // half taps per 64-channel pass
+
+    for (int ic0 = 0; ic0 < p.AC; ic0 += TC_ICC) {
+        // ---- stage the halo: 16 lanes per pixel (64 channels), zero outside the image / beyond AC ----------
+        // (the barrier that ended the previous pass guarantees nobody still reads the old halo)
+        for (int base = 0; base < halo_quads; base += 256 * 8) {
+            float4 v[8];
+            unsigned okmask = 0;
+            // all eight loads are issued (unconditionally, from a clamped address) before any result is used
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int idx = base + t + 256 * u;
+                const int pix = idx >> 4, cq = (idx & 15) * 4;
+                const int r = fdiv(pix, p.d_PWt), cp = pix - r * PWt;
+                const int pgr = pgr0 + r;
+                const int n = fdiv(pgr, p.d_PHt), ih = pgr - n * PHt - p.ph, iw = cp - p.pw;
+                const bool ok = idx < halo_quads && (unsigned)ih < (unsigned)p.AH && (unsigned)iw < (unsigned)p.AW &&
+                                ic0 + cq < p.AC;
+                // branch-free clamp: offset 0 when the element is outside the image
+                const int off = (((n * p.AH + ih) * p.AW + iw) * p.AC + ic0 + cq) & -(int)ok;
+                v[u] = *reinterpret_cast<const float4 *>(p.A + off);
+                okmask |= (unsigned)ok << u;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int idx = base + t + 256 * u;
+                // threads past the end of the halo write their zeros to a spare slot behind it
+                const int dst = idx < halo_quads ? (idx >> 4) * TC_PS + (idx & 15) * 4 : p.lds_rows * PWt * TC_PS;
+                const bool ok = (okmask >> u) & 1u;   // per-component selects keep v[] in registers
+                *reinterpret_cast<float4 *>(Hs + dst) =
+                    make_float4(ok ? v[u].x : 0.f, ok ? v[u].y : 0.f, ok ? v[u].z : 0.f, ok ? v[u].w : 0.f);
+            }
+        }
+        load_filter(ic0, 0, 0);
+        store_filter(0);
+        __syncthreads();
+
+        int th = 0, tw = 0;
+        for (int step = 0; step < steps; step++) {
+            const int half = step & 1, buf = step & 1;
+            // next half tap: same tap, channels +32; or next tap, channels +0
+            int nth = th, ntw = tw;
+            if (half) { ntw = tw + 1; if (ntw == p.TW) { ntw = 0; nth = th + 1; } }
+            const bool more = step + 1 < steps;
+            if (more) load_filter(ic0 + (half ? 0 : 32), nth, ntw);
+
+            const float *hs = Hs + (th * PWt + tw) * TC_PS + 32 * half;
+            const float *ws = Ws + buf * TC_WBUF + bbase;
+            floatx4 a0[TILES], a1[TILES], b0, b1;
+            b0 = *reinterpret_cast<const floatx4 *>(ws);
+#pragma unroll
+            for (int i = 0; i < TILES; i++) a0[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i]);
+            b1 = *reinterpret_cast<const floatx4 *>(ws + 4 * 64 * 4);
+#pragma unroll
+            for (int i = 0; i < TILES; i++) a1[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i] + 16);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int i = 0; i < TILES; i++)
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[i][s], b0[s], acc[i], 0, 0, 0);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int i = 0; i < TILES; i++)
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[i][s], b1[s], acc[i], 0, 0, 0);
+
+            if (more) store_filter(buf ^ 1);
+            __syncthreads();
+            th = nth;
+            tw = ntw;
+        }
+    }
+
+    // ---- epilogue: transpose through LDS so every output pixel row is written as whole 256-byte lines ----
+    float *Os = Hs;   // [P][TC_OS]; the barrier that ended the last step makes the halo free
+#pragma unroll
+    for (int i = 0; i < TILES; i++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) Os[(16 * i + 4 * q + r) * TC_OS + 16 * w + l16] = acc[i][r];
+    __syncthreads();
+    for (int idx = t; idx < P * 16; idx += 256) {
+        const int pix = idx >> 4, cq = (idx & 15) * 4;
+        const int m = m0 + pix;
+        if (m < p.M && oc0 + cq < p.CO)
+            *reinterpret_cast<float4 *>(p.O + (size_t)m * p.CO + oc0 + cq) = *reinterpret_cast<const float4 *>(Os + pix * TC_OS + cq);
+    }
+}
+
+// Rows of LDS halo the worst unit needs: output rows spanned by P consecutive pixels, TH-1 extra rows,
+// and TH-1 more for every image border crossed.
+static int tap_conv_lds_rows(int M, int P, int OH, int OW, int TH)
+{
+    const int OHW = OH * OW, PHt = OH + TH - 1;
+    int worst = 0;
+    const int units = (M + P - 1) / P;
+    const int scan = units < 4096 ? units : 4096;
+    for (int u = 0; u < scan; u++) {
+        const long m0 = (long)u * P, m1 = (m0 + P < M ? m0 + P : M) - 1;
+        const int n0 = (int)(m0 / OHW), oh0 = (int)(m0 % OHW) / OW;
+        const int n1 = (int)(m1 / OHW), oh1 = (int)(m1 % OHW) / OW;
+        const int rows = (n1 * PHt + oh1 + TH - 1) - (n0 * PHt + oh0) + 1;
+        if (rows > worst) worst = rows;
+    }
+    if (units > scan) {   // analytic bound for what was not scanned
+        const int span = (P + OW - 2) / OW + 1;
+        const int cross = (P + OHW - 2) / OHW + 1;
+        const int bound = span + (TH - 1) * (1 + cross);
+        if (bound > worst) worst = bound;
+    }
+    return worst;
+}
+
+template <int TILES>
+static hipError_t launch_tc(hipStream_t stream, const TapConvArgs &a, size_t lds)
+{
+    auto kern = tap_conv_kernel<TILES>;
+    static size_t configured = 0;
+    if (lds > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = lds;
+    }
+    dim3 grid((a.M + TILES * 16 - 1) / (TILES * 16), (a.CO + 63) / 64, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
+    return hipGetLastError();
+}
+
+// Returns hipErrorNotSupported when the shape does not fit this kernel (caller falls back to the
+// generic implicit GEMM); otherwise launches.
+hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
+                           int N, int AH, int AW, int AC, int OH, int OW, int CO,
+                           int TH, int TW, int ph, int pw,
+                           int b_off, int b_sth, int b_stw, int b_sc)
+{
+    if (OH != AH + 2 * ph - TH + 1 || OW != AW + 2 * pw - TW + 1) return hipErrorNotSupported;
+    if (AC < 32 || TH * TW < 2 || TH > 7 || TW > 7) return hipErrorNotSupported;
+    const long M = (long)N * OH * OW;
+    if ((long)N * (AH + 2 * ph) >= (1L << 24)) return hipErrorNotSupported;
+
+    TapConvArgs a{};
+    a.A = A; a.B = B; a.O = O;
+    a.M = (int)M; a.CO = CO;
+    a.AH = AH; a.AW = AW; a.AC = AC;
+    a.TH = TH; a.TW = TW; a.ph = ph; a.pw = pw;
+    a.PHt = AH + 2 * ph; a.PWt = AW + 2 * pw;
+    a.b_off = b_off; a.b_sth = b_sth; a.b_stw = b_stw; a.b_sc = b_sc;
+    a.d_OW = make_fastdiv(OW);
+    a.d_OHW = make_fastdiv(OH * OW);
+    a.d_PHt = make_fastdiv(a.PHt);
+    a.d_PWt = make_fastdiv(a.PWt);
+
+    // pixels per workgroup: 7 tiles (112) when that divides the row/image structure better, else 8 (128)
+    const int OHW = OH * OW;
+    int tiles = 8;
+    if ((OHW % 112 == 0 || (2 * OW) % 112 == 0 || 112 % OW == 0) && !(OHW % 128 == 0 || 128 % OW == 0)) tiles = 7;
+    const size_t budget = 80 * 1024;   // two workgroups per CU
+    for (int attempt = 0; attempt < 2; attempt++) {
+        const int P = tiles * 16;
+        a.lds_rows = tap_conv_lds_rows(a.M, P, OH, OW, TH);
+        size_t halo = (size_t)a.lds_rows * a.PWt * TC_PS + 4;   // + one spare 16-byte slot
+        const size_t stage = (size_t)P * TC_OS;
+        if (halo < stage) halo = stage;
+        const size_t lds = (2 * TC_WBUF + halo) * sizeof(float);
+        if (lds <= budget) return tiles == 7 ? launch_tc<7>(stream, a, lds) : launch_tc<8>(stream, a, lds);
+        tiles = (tiles == 8) ? 7 : 8;
+    }
+    return hipErrorNotSupported;
+}
+
+}  // namespace alpha

@@ -49,9 +49,10 @@ const char *alpha_conv_last_error(void);
  * split-K factor (CudaFloat32EngineBase.java:73). */
 int alpha_conv_device_info(int *compute_units, int *clock_khz);
 
-/* Forward algorithm used inside the forward entries when the layer is 3x3, stride 1:
- * 0 = auto, 1 = implicit GEMM only, 2 = Winograd F(2x2,3x3) where eligible.
- * Also read once from the environment variable ALPHA_HIP_CONV_ALGO = auto|igemm|winograd.
+/* Kernel family used inside the stride-1 entries:
+ * 0 = auto, 1 = implicit GEMM only (LDS-halo kernel where eligible, else the generic one),
+ * 2 = Winograd F(2x2,3x3) where eligible, 3 = the generic gather kernel only (for comparisons).
+ * Also read once from the environment variable ALPHA_HIP_CONV_ALGO = auto|igemm|winograd|generic.
  * No counterpart in the reference (its Winograd experiments are compiled out, conv/conv3D.cuh:39-44). */
 int alpha_conv_set_fwd_algo(int algo);
 int alpha_conv_get_fwd_algo(void);

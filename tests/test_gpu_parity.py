@@ -129,6 +129,53 @@ def test_forward_np_and_w1_entries(dev):
     check(_run_fwd(dev, "conv3D_GemmR_W1", X, W, 1, 1, 0, 0), want, "conv3D_GemmR_W1")
 
 
+TAP_SHAPES = [
+    # stride-1 layers served by the LDS-halo kernel: N, IH, IW, IC, OC, FH, FW, ph, pw
+    (4, 56, 56, 64, 64, 3, 3, 1, 1),      # c3a / c5b geometry (units of 2 rows)
+    (8, 32, 32, 64, 64, 3, 3, 1, 1),      # c2a geometry
+    (8, 28, 28, 128, 128, 3, 3, 1, 1),    # c3b: two channel passes, two oc slices
+    (16, 14, 14, 256, 256, 3, 3, 1, 1),   # c3c: units cross image borders
+    (36, 7, 7, 512, 512, 3, 3, 1, 1),     # c3d: a unit spans several images
+    (20, 8, 8, 256, 256, 3, 3, 1, 1),     # c2c
+    (4, 13, 11, 36, 44, 3, 3, 1, 1),      # ragged IC / OC (zero-filled channel tails)
+    (4, 12, 17, 100, 132, 5, 5, 2, 2),
+    (4, 10, 10, 64, 64, 3, 3, 0, 0),      # no padding
+    (4, 9, 14, 96, 72, 2, 4, 1, 3),       # non-square filter, asymmetric pad
+    (4, 6, 5, 32, 64, 3, 3, 2, 2),        # pad larger than usual
+    (3, 5, 5, 64, 64, 3, 3, 1, 1),        # fewer pixels than one unit
+]
+
+
+@pytest.mark.parametrize("shape", TAP_SHAPES)
+def test_forward_lds_halo_kernel_vs_oracle_and_generic(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, ph, pw = shape
+    X, W = normal((N, IH, IW, IC), 1101), he_normal(OC, FH, FW, IC, 1102)
+    want = O.conv3D_f64(X, W, 1, 1, ph, pw)
+    L = pkg.lib()
+    try:
+        L.alpha_conv_set_fwd_algo(0)
+        fast = _run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, ph, pw)
+        L.alpha_conv_set_fwd_algo(3)
+        generic = _run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, ph, pw)
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+    check(fast, want, "lds-halo fwd %s" % (shape,))
+    check(generic, want, "generic fwd %s" % (shape,))
+
+
+@pytest.mark.parametrize("shape", TAP_SHAPES)
+def test_deltaX_lds_halo_kernel_vs_oracle(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, ph, pw = shape
+    if ph > FH - 1 or pw > FW - 1:
+        pytest.skip("backward-data needs ph <= FH-1")
+    OH, OW = out_dim(IH, IW, FH, FW, 1, 1, ph, pw)
+    dY, W = normal((N, OH, OW, OC), 1103), he_normal(OC, FH, FW, IC, 1104)
+    dy, w = dev.put(dY), dev.put(W)
+    dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+    DX.dconv3D_deltaX_s1(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC, ph, pw)
+    check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw), "lds-halo dX %s" % (shape,))
+
+
 def test_forward_oc_sweep_covers_every_ragged_width(dev):
     # the reference's "for OC from 1 to 128: correct" sweep (Cuda_conv3D_test.java:155-156), in steps of 4
     X = uniform((4, 9, 9, 8), 1009)
