@@ -5,20 +5,20 @@
 // (n, oh, ow) index and a slice of 64 output channels. For each chunk of 64 input channels it
 //   1. copies the zero-padded input rows those pixels touch into LDS once
 //      (rows are "padded global rows" n*(AH+2ph) + ih + ph, so a pixel range may cross image borders);
-//   2. walks the filter in "half taps" (one tap, 32 input channels): the 32x64 filter slice is staged
-//      in one of two LDS buffers while the MFMAs of the previous half tap run (one barrier per half
-//      tap); every lane reads its pixel's 4 consecutive channels with one 128-bit LDS read at
-//      base(pixel) + tap offset — no address arithmetic or bounds tests in the inner loop.
+//   2. walks the filter in "half taps" (one tap, 32 input channels). Every lane reads its pixel's 4
+//      consecutive channels with one 128-bit LDS read at base(pixel) + tap offset — no address
+//      arithmetic or bounds tests in the inner loop. The filter fragment of a half tap (8 floats per
+//      lane) comes straight from global memory (it is L2/L1 resident: every workgroup reads the same
+//      few hundred KB) and is prefetched one half tap ahead, so the main loop has no barrier at all.
 // Each input element is read from memory once per workgroup instead of once per tap.
 //
 // Wavefront w computes output channels [16w, 16w+16) for all TILES pixel tiles (TILES*4 accumulator
-// registers). Operand fragments are double-buffered in registers: the LDS reads of channel group
-// g+1 are issued before the MFMAs of group g.
+// registers).
 //
-// LDS layouts (floats):
-//   halo  [row][col][64+4]      pixel stride 68: the 16 lanes of a 128-bit read hit distinct banks
-//   filter[2][8][64 oc][4]      the 4 channels a lane needs at one output channel are contiguous, so
-//                               the B fragment is a single 128-bit read, lanes contiguous
+// LDS layout (floats): halo[row][col][64+8]. Pixel stride 72 floats = 288 bytes: measured on gfx950,
+// a 128-bit LDS read is conflict-free when the 32 lanes of each half wavefront touch 32 distinct
+// 16-byte slots modulo 512 bytes; with 16 consecutive pixels x 2 channel quads per half wavefront
+// that needs a pixel stride of 16*(4k+2) bytes (272 gives a 2-way conflict, 288 none).
 // K permutation inside a group of 16 channels: lane group q = lane/16 supplies channel 16g + 4q + s
 // at MFMA step s, for both operands.
 #include "common.hpp"
@@ -39,23 +39,29 @@ struct TapConvArgs {
 };
 
 constexpr int TC_ICC = 64;            // input channels per halo pass
-constexpr int TC_PS = TC_ICC + 4;     // LDS pixel stride (floats)
-constexpr int TC_WBUF = 8 * 64 * 4;   // floats per filter buffer (32 channels x 64 output channels)
+constexpr int TC_PS = TC_ICC + 8;     // LDS pixel stride (floats)
 constexpr int TC_OS = 64 + 4;         // output staging row stride (floats)
 
-template <int TILES>
+// RAGGED: AC is not a multiple of 64, so the last pass has channels beyond AC whose filter fragments
+// must be zeroed (kept out of the common case: the extra selects would pull the wait for the
+// prefetched fragment in front of the MFMAs).
+template <int TILES, bool RAGGED>
 __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
 {
     constexpr int P = TILES * 16;
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *Ws = smem;                       // [2][TC_WBUF]
-    float *Hs = smem + 2 * TC_WBUF;         // [lds_rows][PWt][TC_PS]; reused as output staging [P][TC_OS]
+    float *Hs = smem;   // [lds_rows][PWt][TC_PS] (+ one spare slot); reused as output staging [P][TC_OS]
 
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
     const int l16 = lane & 15, q = lane >> 4;
 
-    const int m0 = blockIdx.x * P;
+    // Consecutive units share halo rows: keep them on one XCD (workgroups are dealt round-robin to the
+    // 8 XCDs) so the shared rows are served by that XCD's L2.
+    const int G = gridDim.x;
+    const int xcd = blockIdx.x & 7, xi = blockIdx.x >> 3;
+    const int unit = xcd * (G >> 3) + min(xcd, G & 7) + xi;
+    const int m0 = unit * P;
     const int oc0 = blockIdx.y * 64;
     const int OW = p.d_OW.d, OHW = p.d_OHW.d, PHt = p.PHt, PWt = p.PWt;
 
@@ -77,43 +83,64 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
         const int oh = fdiv(rem, p.d_OW), ow = rem - oh * OW;
         abase[i] = ((n * PHt + oh - pgr0) * PWt + ow) * TC_PS + 4 * q;
     }
-    const int bbase = (q * 64 + 16 * w + l16) * 4;
 
     floatx4 acc[TILES];
 #pragma unroll
     for (int i = 0; i < TILES; i++) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // ---- filter staging: thread (Q = t/32, pair = t%32) moves channels 4Q..4Q+3 of two output channels ----
-    const int w_Q = t >> 5, w_oc = (t & 31) * 2;
-    const bool w_colv = oc0 + w_oc < p.CO;
-    float2 wreg[4];
-    bool wok = false;
-    // Loads are issued unconditionally from a clamped (always valid) address; the zeroing of invalid
-    // channels happens when the registers are stored to LDS, so nothing waits on the loads before the
-    // MFMAs of the current half tap have been issued.
-    auto load_filter = [&](int icbase, int th, int tw) {   // icbase: first of the 32 channels of this half tap
-        const int base = p.b_off + th * p.b_sth + tw * p.b_stw + oc0 + w_oc;
-        const int c = icbase + 4 * w_Q;
-        wok = w_colv && c < p.AC;   // AC % 4 == 0: the four channels are valid together
+    // ---- filter fragments straight from global memory -------------------------------------------------
+    // lane (l16, q) of wavefront w needs, for channel group g of a half tap, B[c = 16g + 4q + s][oc0 + 16w + l16].
+    const int b_co = oc0 + 16 * w + l16;
+    const bool b_cov = b_co < p.CO;   // columns beyond CO are never stored; clamp their loads to a valid address
+    auto load_b = [&](float (&b)[2][4], int icbase, int th, int tw) {
+        const int base = p.b_off + th * p.b_sth + tw * p.b_stw + (b_cov ? b_co : 0);
 #pragma unroll
-        for (int s = 0; s < 4; s++)
-            wreg[s] = *reinterpret_cast<const float2 *>(p.B + ((base + (c + s) * p.b_sc) & -(int)wok));
+        for (int g = 0; g < 2; g++) {
+            const int c = icbase + 16 * g + 4 * q;
+            const int ok = -(int)(c < p.AC);   // AC % 4 == 0: the four channels are valid together
+#pragma unroll
+            for (int s = 0; s < 4; s++) b[g][s] = p.B[(base + (c + s) * p.b_sc) & ok];
+        }
     };
-    auto store_filter = [&](int buf) {
-        float *dst = Ws + buf * TC_WBUF + (w_Q * 64 + w_oc) * 4;
-        *reinterpret_cast<float4 *>(dst) = make_float4(wok ? wreg[0].x : 0.f, wok ? wreg[1].x : 0.f,
-                                                       wok ? wreg[2].x : 0.f, wok ? wreg[3].x : 0.f);
-        *reinterpret_cast<float4 *>(dst + 4) = make_float4(wok ? wreg[0].y : 0.f, wok ? wreg[1].y : 0.f,
-                                                           wok ? wreg[2].y : 0.f, wok ? wreg[3].y : 0.f);
+    // channels beyond AC: the halo holds zeros there, but 0 * (whatever the clamped load returned) must
+    // not turn into NaN, so the fragment is zeroed when it is used
+    auto mask_b = [&](float (&b)[2][4], int icbase) {
+        if (!RAGGED) return;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const bool ok = icbase + 16 * g + 4 * q < p.AC;
+#pragma unroll
+            for (int s = 0; s < 4; s++) b[g][s] = ok ? b[g][s] : 0.f;
+        }
     };
 
     const int halo_quads = rows * PWt * (TC_ICC / 4);
     const int taps = p.TH * p.TW;
-    const int steps = taps * 2;   // half taps per 64-channel pass
 
+    auto half_tap = [&](const float (&b)[2][4], int th, int tw, int half) {
+        const float *hs = Hs + (th * PWt + tw) * TC_PS + 32 * half;
+        floatx4 a0[TILES], a1[TILES];
+#pragma unroll
+        for (int i = 0; i < TILES; i++) a0[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i]);
+#pragma unroll
+        for (int i = 0; i < TILES; i++) a1[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i] + 16);
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int i = 0; i < TILES; i++)
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[i][s], b[0][s], acc[i], 0, 0, 0);
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int i = 0; i < TILES; i++)
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[i][s], b[1][s], acc[i], 0, 0, 0);
+    };
+
+    float bA[2][4], bB[2][4];
+    load_b(bA, 0, 0, 0);   // first half tap; in flight while the halo is staged
     for (int ic0 = 0; ic0 < p.AC; ic0 += TC_ICC) {
+        if (ic0 > 0) __syncthreads();   // everyone finished reading the previous pass's halo
         // ---- stage the halo: 16 lanes per pixel (64 channels), zero outside the image / beyond AC ----------
-        // (the barrier that ended the previous pass guarantees nobody still reads the old halo)
         for (int base = 0; base < halo_quads; base += 256 * 8) {
             float4 v[8];
             unsigned okmask = 0;
@@ -142,48 +169,38 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
                     make_float4(ok ? v[u].x : 0.f, ok ? v[u].y : 0.f, ok ? v[u].z : 0.f, ok ? v[u].w : 0.f);
             }
         }
-        load_filter(ic0, 0, 0);
-        store_filter(0);
         __syncthreads();
 
+        // ---- main loop: two half taps per iteration, filter fragments ping-pong between bA and bB --------
         int th = 0, tw = 0;
-        for (int step = 0; step < steps; step++) {
-            const int half = step & 1, buf = step & 1;
-            // next half tap: same tap, channels +32; or next tap, channels +0
-            int nth = th, ntw = tw;
-            if (half) { ntw = tw + 1; if (ntw == p.TW) { ntw = 0; nth = th + 1; } }
-            const bool more = step + 1 < steps;
-            if (more) load_filter(ic0 + (half ? 0 : 32), nth, ntw);
-
-            const float *hs = Hs + (th * PWt + tw) * TC_PS + 32 * half;
-            const float *ws = Ws + buf * TC_WBUF + bbase;
-            floatx4 a0[TILES], a1[TILES], b0, b1;
-            b0 = *reinterpret_cast<const floatx4 *>(ws);
-#pragma unroll
-            for (int i = 0; i < TILES; i++) a0[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i]);
-            b1 = *reinterpret_cast<const floatx4 *>(ws + 4 * 64 * 4);
-#pragma unroll
-            for (int i = 0; i < TILES; i++) a1[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i] + 16);
-#pragma unroll
-            for (int s = 0; s < 4; s++)
-#pragma unroll
-                for (int i = 0; i < TILES; i++)
-                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[i][s], b0[s], acc[i], 0, 0, 0);
-#pragma unroll
-            for (int s = 0; s < 4; s++)
-#pragma unroll
-                for (int i = 0; i < TILES; i++)
-                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[i][s], b1[s], acc[i], 0, 0, 0);
-
-            if (more) store_filter(buf ^ 1);
-            __syncthreads();
+        for (int tap = 0; tap < taps; tap++) {
+            // The prefetch below is unconditional (a branch around it would make every wait in the loop
+            // assume the shorter queue): after the last tap it fetches the first half tap of the next
+            // pass, or harmlessly re-fetches tap (0,0) of this one at the very end.
+            int nth = th, ntw = tw + 1, nic = ic0;
+            if (ntw == p.TW) { ntw = 0; nth = th + 1; }
+            if (tap + 1 == taps) { nth = 0; ntw = 0; nic = ic0 + TC_ICC < p.AC ? ic0 + TC_ICC : ic0; }
+            // The scheduling barriers pin each prefetch in front of the half tap that hides its latency; left
+            // alone the compiler sinks the loads to just before their first use.
+            load_b(bB, ic0 + 32, th, tw);
+            __builtin_amdgcn_sched_barrier(0);
+            mask_b(bA, ic0);
+            half_tap(bA, th, tw, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_b(bA, nic, nth, ntw);
+            __builtin_amdgcn_sched_barrier(0);
+            mask_b(bB, ic0 + 32);
+            half_tap(bB, th, tw, 1);
+            __builtin_amdgcn_sched_barrier(0);
             th = nth;
             tw = ntw;
         }
     }
+    (void)bA;
 
     // ---- epilogue: transpose through LDS so every output pixel row is written as whole 256-byte lines ----
-    float *Os = Hs;   // [P][TC_OS]; the barrier that ended the last step makes the halo free
+    __syncthreads();   // all wavefronts are done reading the halo
+    float *Os = Hs;    // [P][TC_OS]
 #pragma unroll
     for (int i = 0; i < TILES; i++)
 #pragma unroll
@@ -221,10 +238,10 @@ static int tap_conv_lds_rows(int M, int P, int OH, int OW, int TH)
     return worst;
 }
 
-template <int TILES>
+template <int TILES, bool RAGGED>
 static hipError_t launch_tc(hipStream_t stream, const TapConvArgs &a, size_t lds)
 {
-    auto kern = tap_conv_kernel<TILES>;
+    auto kern = tap_conv_kernel<TILES, RAGGED>;
     static size_t configured = 0;
     if (lds > configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -272,8 +289,12 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
         size_t halo = (size_t)a.lds_rows * a.PWt * TC_PS + 4;   // + one spare 16-byte slot
         const size_t stage = (size_t)P * TC_OS;
         if (halo < stage) halo = stage;
-        const size_t lds = (2 * TC_WBUF + halo) * sizeof(float);
-        if (lds <= budget) return tiles == 7 ? launch_tc<7>(stream, a, lds) : launch_tc<8>(stream, a, lds);
+        const size_t lds = halo * sizeof(float);
+        if (lds <= budget) {
+            const bool ragged = (AC % TC_ICC) != 0;
+            if (tiles == 7) return ragged ? launch_tc<7, true>(stream, a, lds) : launch_tc<7, false>(stream, a, lds);
+            return ragged ? launch_tc<8, true>(stream, a, lds) : launch_tc<8, false>(stream, a, lds);
+        }
         tiles = (tiles == 8) ? 7 : 8;
     }
     return hipErrorNotSupported;
