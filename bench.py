@@ -87,9 +87,9 @@ class Workload:
         self.CW = torch.empty(F * F * IC * OC, device=dev)
         self.stream = int(torch.cuda.current_stream().cuda_stream)
         self.streams = [self.stream]
-        # split-K factor: the engine's clamp (CudaFloat32EngineBase.java:1707-1715) with MaxPartNum = clip(#CU,16,128)
-        GK = N * OH * OW
-        self.GridZ = max(2, min(128, GK >> 8)) if GK >= 512 else 1
+        self.engine = pkg.engine.Engine(self.stream)
+        # split-K factor for the kernel-only timing: what the host layer would pass (CudaFloat32EngineBase.java:1707-1715)
+        self.GridZ = max(1, pkg.engine.plan_deltaW(self.engine.config, IH, IW, OH, OW, F, F, N, IC, OC, s, s).GridZ)
         self.buf = torch.empty(max(1, self.GridZ - 1) * self.dW.numel(), device=dev)
         if s > 1:
             CFH = (F + s - 1) // s
@@ -111,8 +111,10 @@ class Workload:
                              self.Y.data_ptr(), self.OH, self.OW, N, IC, OC, s, s, p, p)
 
     def fwd(self):
-        self.fwd_remode()
-        self.fwd_conv()
+        # whole operator through the C++ host layer: entry selection, CW scratch, kernel_remode, conv entry
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.engine.conv3D(self.Y.data_ptr(), self.OH, self.OW, self.X.data_ptr(), IH, IW, self.W.data_ptr(), F, F,
+                           N, IC, OC, s, s, p, p)
 
     def dx(self):
         N, IH, IW, IC, OC, F, s, p = self.dims
@@ -134,8 +136,15 @@ class Workload:
                                     self.dW.data_ptr(), self.buf.data_ptr(), F, F, N, IC, OC, s, s, p, p)
 
     def dw(self):
-        self.dw_gemm()
-        self.pkg.Cuda_dconv3D_deltaW.buf_summary(self.stream, self.buf.data_ptr(), self.dW.data_ptr(), self.GridZ - 1, self.dW.numel())
+        # whole operator through the C++ host layer: GridZ, deltaW_buf scratch, split-K entry, buf_summary
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.engine.dconv3D_deltaW(self.dW.data_ptr(), F, F, self.X.data_ptr(), IH, IW, self.dY.data_ptr(), self.OH, self.OW,
+                                   N, IC, OC, s, s, p, p)
+
+    def dx_op(self):
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.engine.dconv3D_deltaX(self.dX.data_ptr(), IH, IW, self.dY.data_ptr(), self.OH, self.OW, self.W.data_ptr(), F, F,
+                                   N, IC, OC, s, s, p, p)
 
 
 def time_loop(torch, fn, steps, warmup):
@@ -203,12 +212,17 @@ def load_traffic(layer, op):
 
 def measure(pkg, torch, layer, op, steps, warmup):
     wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer))
-    step = {"fwd": wl.fwd, "dx": wl.dx, "dw": wl.dw}[op]
+    step = {"fwd": wl.fwd, "dx": wl.dx_op, "dw": wl.dw}[op]
     kernel = {"fwd": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm}[op]
     if op == "fwd":
         wl.fwd_remode()
-    wall_ms, ev_ms = time_loop(torch, step, steps, warmup)
+    def step_and_recycle():
+        step()
+    wall_ms, ev_ms = time_loop(torch, step_and_recycle, steps, warmup)
+    wl.engine.sync()
     _, k_ms = time_loop(torch, kernel, steps, max(1, warmup // 2))   # dominant kernel alone, HIP events on its stream
+    gridz = wl.GridZ
+    wl.engine.close()
     fl, by = flops(layer), algorithmic_bytes(layer)
     hbm = layer in HBM_BOUND
     roof = {
@@ -222,7 +236,7 @@ def measure(pkg, torch, layer, op, steps, warmup):
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     return {"layer": layer, "op": op, "ms_per_step": round(wall_ms, 5), "event_ms_per_step": round(ev_ms, 5),
             "tflops": round(fl / (wall_ms * 1e-3) / 1e12, 3), "gflop": round(fl / 1e9, 3),
-            "algorithmic_MB": round(by / 1e6, 2), "roofline": roof}
+            "algorithmic_MB": round(by / 1e6, 2), "GridZ": gridz if op == "dw" else None, "roofline": roof}
 
 
 def main():
@@ -269,7 +283,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "%s %s: N=%d %dx%dx%d->%d %dx%d s%d p%d NHWC; step = kernel_remode + conv entry"
+        "config": {"workload": "%s %s: N=%d %dx%dx%d->%d %dx%d s%d p%d NHWC; step = one operator call through the host layer (scratch + remode/summary + conv entry)"
                                % (args.layer, op, N, IH, IW, ICl, OC, F, F, s, p),
                    "layer": args.layer, "op": op, "gflop_per_step": head["gflop"],
                    "algorithmic_MB_per_step": head["algorithmic_MB"],

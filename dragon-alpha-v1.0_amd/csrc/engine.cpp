@@ -1,0 +1,432 @@
+// Host-side counterpart of the reference's CudaFloat32EngineBase convolution section
+// (src/alpha_src/z/dragon/engine/cuda/CudaFloat32EngineBase.java:1323-2005): which native entry is
+// called for a layer, with how many stream handles, which split-K factor and which scratch buffers.
+// The reference does this in Java above the JNI boundary; there is no JVM here, so the same integer
+// decisions are restated in C++ and exported through the C ABI (alpha_plan_* are pure functions,
+// alpha_engine_* additionally own the scratch memory the Java engine would take from its pool and
+// then call the natives exactly as the Java code does).
+#include "../../include/alpha_conv.h"
+#include "../../include/alpha_engine.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+namespace {
+
+// Tiles of the reference's power-of-two strip decomposition of one GEMM extent: whole 128-wide
+// tiles, then one strip for every set bit 64, 32, 16, 8 and one for a remainder of 4..7
+// (Cuda_conv3D.java:19-41 and its twins in the deltaX / deltaW classes).
+int strips_tiles(int g) { return (g >> 7) + __builtin_popcount(g & 0x7C); }
+
+// Kernel launches (= streams wanted) along one extent: 1 for a power of two, else one per strip
+// (Cuda_conv3D.java:70-97).
+int strips_streams(int g)
+{
+    if ((g & (g - 1)) == 0) return 1;
+    return (g > 127 ? 1 : 0) + __builtin_popcount(g & 0x7C);
+}
+
+int stream_count(int gn, int gm, int cap) { return std::min(strips_streams(gn) * strips_streams(gm), cap); }
+
+}  // namespace
+
+extern "C" {
+#pragma GCC visibility push(default)
+
+int alpha_blockNum(int GN, int GM) { return strips_tiles(GN) * strips_tiles(GM); }
+int alpha_streamSize(int GN, int GM, int cap) { return stream_count(GN, GM, cap); }
+
+double alpha_paddingScaleUp(int IH, int IW, int OH, int OW, int FH, int FW, int sh, int sw)
+{
+    // Cuda_conv3D.java:129-135
+    return 1.0 * (((OH - 1) * sh + FH) * ((OW - 1) * sw + FW)) / (IH * IW);
+}
+
+void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
+{
+    // CudaFloat32EngineBase.java:1324-1352, 1630-1663, 1765-1793 and :73 (MaxPartNum = clip(#SM, 16, 128))
+    c->conv3D_useTexture = 1;
+    c->conv3D_remode = 1;
+    c->conv3D_remode_V2_Q = 1.05f;
+    c->conv3D_V2_Q = 1.25f;
+    c->deltaW_SplitKThreshold = 512;
+    c->deltaW_SK_MaxPartNum = std::max(16, std::min(128, compute_units));
+    c->deltaW_SK_V2_Q = 1.15f;
+    c->deltaX_s1_useTexture = 1;
+    c->deltaX_ks_useTexture = 0;
+    c->deltaX_s1_V2_Q = 1.1f;
+    c->deltaX_ks_V2_Q = 1.1f;
+}
+
+// ---- forward: CudaFloat32EngineBase.conv3D (:1355-1474) ----------------------------------------------
+void alpha_plan_conv3D(const alpha_engine_config *c, int IH, int IW, int OH, int OW, int FH, int FW, int N, int IC, int OC,
+                       int sh, int sw, int ph, int pw, alpha_conv_plan *out)
+{
+    (void)IC;
+    memset(out, 0, sizeof(*out));
+    const double Q = alpha_paddingScaleUp(IH, IW, OH, OW, FH, FW, sh, sw);
+    out->Q = Q;
+    if (c->conv3D_remode && OC > 31 && N * OH * OW > 31) {
+        const bool V2 = N > 63 && OC > 63 && Q > c->conv3D_remode_V2_Q;
+        out->remode = 1;
+        out->V2 = V2;
+        out->streams = V2 ? stream_count(OC, N, 10) : stream_count(OC, N * OH * OW, 10);
+        out->useTexture = c->conv3D_useTexture;
+        // The W1 natives carry no stride or padding (1x1, stride 1, pad 0). The Java engine can send every 1x1 layer
+        // there because its argument check refuses sh > FH (EngineCore.java:650-651); this host layer also serves
+        // strided 1x1 layers, through the general entries.
+        const bool w1 = FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
+        if (w1) out->entry = ALPHA_E_conv3D_GemmR_W1;
+        else if (V2) out->entry = ALPHA_E_conv3D_GemmV2R;
+        else if (c->conv3D_useTexture) out->entry = ALPHA_E_conv3D_GemmR_texture;
+        else out->entry = ALPHA_E_conv3D_GemmR;
+        out->scratch_floats = (long)FH * FW * IC * OC;
+    } else {
+        const bool V2 = N > 127 && OC > 127 && Q >= c->conv3D_V2_Q;
+        out->V2 = V2;
+        out->streams = V2 ? stream_count(OC, N, 10) : stream_count(OC, N * OH * OW, 10);
+        out->useTexture = c->conv3D_useTexture && OC > 15;
+        if (FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0) out->entry = ALPHA_E_conv3D_W1;
+        else if (ph == 0 && pw == 0) out->entry = ALPHA_E_conv3D_np;
+        else if (V2) out->entry = ALPHA_E_conv3DV2;
+        else if (out->useTexture) out->entry = ALPHA_E_conv3D_texture;
+        else out->entry = ALPHA_E_conv3D;
+    }
+}
+
+// ---- backward-filter: CudaFloat32EngineBase.dconv3D_deltaW (:1666-1762) ------------------------------------
+void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int OW, int FH, int FW, int N, int IC, int OC,
+                       int sh, int sw, alpha_conv_plan *out)
+{
+    memset(out, 0, sizeof(*out));
+    const int GK = N * OH * OW;
+    const double Q = alpha_paddingScaleUp(IH, IW, OH, OW, FH, FW, sh, sw);
+    out->Q = Q;
+    if (GK < c->deltaW_SplitKThreshold) {
+        out->streams = stream_count(OC, FH * FW * IC, 12);
+        out->GridZ = 1;
+        out->entry = (FH == 1 && FW == 1 && sh == 1 && sw == 1) ? ALPHA_E_dconv3D_deltaW_W1 : ALPHA_E_dconv3D_deltaW;
+        return;
+    }
+    const bool V2 = OC > 63 && IC > 63 && Q >= c->deltaW_SK_V2_Q;
+    out->V2 = V2;
+    out->streams = V2 ? stream_count(OC, IC, 12) : stream_count(OC, FH * FW * IC, 12);
+    // tile counts of forward, backward-data and backward-filter (Cuda_conv3D.blockNum[V2] and twins)
+    const int b1 = V2 ? strips_tiles(OC) * strips_tiles(N) * OH * OW : strips_tiles(OC) * strips_tiles(N * OH * OW);
+    const int b2 = V2 ? strips_tiles(IC) * strips_tiles(N) * IH * IW : strips_tiles(IC) * strips_tiles(N * IH * IW);
+    const int b3 = V2 ? strips_tiles(OC) * strips_tiles(IC) * FH * FW : strips_tiles(OC) * strips_tiles(FH * FW * IC);
+    int GridZ = (b1 + b2) / (b3 << 1);
+    if (GridZ < 2) GridZ = 2;
+    if (GridZ > c->deltaW_SK_MaxPartNum) GridZ = c->deltaW_SK_MaxPartNum;
+    const int GridZ2 = GK >> 8;
+    if (GridZ > GridZ2) GridZ = GridZ2;
+    out->GridZ = GridZ;
+    out->scratch_floats = (long)OC * FH * FW * IC * (GridZ - 1);
+    if (FH == 1 && FW == 1 && sh == 1 && sw == 1) out->entry = ALPHA_E_dconv3D_deltaW_GemmSK_W1;   // W1 natives: stride 1 only
+    else if (V2) out->entry = ALPHA_E_dconv3D_deltaW_GemmV2SK;
+    else out->entry = ALPHA_E_dconv3D_deltaW_GemmSK;
+}
+
+// ---- backward-data: CudaFloat32EngineBase.dconv3D_deltaX (:1796-2005) ---------------------------------------
+void alpha_plan_deltaX(const alpha_engine_config *c, int IH, int IW, int OH, int OW, int FH, int FW, int N, int IC, int OC,
+                       int sh, int sw, alpha_conv_plan *out)
+{
+    memset(out, 0, sizeof(*out));
+    if (IC <= 8 || (IC <= 16 && sh * sw >= 4)) {
+        out->entry = ALPHA_E_dconv3D_deltaX_crossAdd;
+        out->streams = stream_count(OC, N * OH * OW, 7);
+        return;
+    }
+    if (FH == 1 && FW == 1 && sh == 1 && sw == 1) {   // the W1 native ignores stride; strided 1x1 goes to kernel split
+        out->entry = ALPHA_E_dconv3D_deltaX_W1;
+        out->streams = stream_count(IC, N * IH * IW, 10);
+        return;
+    }
+    if (sh == 1 && sw == 1) {
+        // Cuda_dconv3D_deltaX.s1_paddingScaleUp
+        const double Q = 1.0 * ((IH - 1 + FH) * (IW - 1 + FW)) / (OH * OW);
+        const bool V2 = N > 63 && IC > 63 && Q > c->deltaX_s1_V2_Q;
+        out->Q = Q;
+        out->V2 = V2;
+        out->streams = V2 ? stream_count(IC, N, 10) : stream_count(IC, N * IH * IW, 10);
+        out->useTexture = c->deltaX_s1_useTexture && IC > 15;
+        out->entry = V2 ? ALPHA_E_dconv3D_deltaX_V2_s1 : (out->useTexture ? ALPHA_E_dconv3D_deltaX_s1_texture : ALPHA_E_dconv3D_deltaX_s1);
+        return;
+    }
+    const int CFH = (FH + sh - 1) / sh, CFW = (FW + sw - 1) / sw;
+    out->remode = 1;
+    out->scratch_floats = (long)OC * CFH * CFW * IC * sh * sw;
+    out->useTexture = c->deltaX_ks_useTexture && IC > 15;
+    const int ks_streams = stream_count(IC, N * ((IH + sh - 1) / sh) * ((IW + sw - 1) / sw), 10);
+    if (sh == 2 && sw == 2 && (IH & 1) == 0 && (IW & 1) == 0) {
+        // Cuda_dconv3D_deltaX.Ims2_paddingScaleUp
+        const int OH0 = (IH >> 1) + ((FH + 1) >> 1) - 1, OW0 = (IW >> 1) + ((FW + 1) >> 1) - 1;
+        const int OH1 = (IH >> 1) + (FH >> 1) - 1, OW1 = (IW >> 1) + (FW >> 1) - 1;
+        const double Q = 0.25 * ((OH0 + OH1) * (OW0 + OW1)) / (OH * OW);
+        const bool V2 = N > 63 && IC > 63 && Q > c->deltaX_ks_V2_Q;
+        out->Q = Q;
+        out->V2 = V2;
+        out->streams = V2 ? stream_count(IC, N, 10) : ks_streams;
+        out->entry = V2 ? ALPHA_E_dconv3D_deltaX_ksV2_Ims2R
+                        : (out->useTexture ? ALPHA_E_dconv3D_deltaX_ksIms2R_texture : ALPHA_E_dconv3D_deltaX_ksIms2R);
+        return;
+    }
+    out->streams = ks_streams;
+    if (IH % sh == 0 && IW % sw == 0)
+        out->entry = out->useTexture ? ALPHA_E_dconv3D_deltaX_ksImsR_texture : ALPHA_E_dconv3D_deltaX_ksImsR;
+    else
+        out->entry = ALPHA_E_dconv3D_deltaX_kernelSplit;
+}
+
+// ---- engine object: owns scratch and calls the natives the way the Java engine does --------------------------------
+struct alpha_engine {
+    alpha_engine_config cfg;
+    int64_t stream;
+    std::mutex mu;
+    // Scratch pool, by size in bytes. Every operator is enqueued on the one stream of this engine, so a block used by
+    // one operator can be handed to the next as soon as the first has been enqueued: stream order keeps their kernels
+    // apart (the Java engine, which spreads work over several streams, waits for the operator's Syncer instead).
+    std::multimap<size_t, void *> free_blocks;
+    std::vector<std::pair<size_t, void *>> in_flight;     // blocks of the operator being enqueued
+    char err[256];
+};
+
+static void release_blocks(alpha_engine *e)
+{
+    std::lock_guard<std::mutex> g(e->mu);
+    for (auto &b : e->in_flight) e->free_blocks.emplace(b.first, b.second);
+    e->in_flight.clear();
+}
+
+struct BlockScope {   // returns the operator's scratch to the pool when the operator has been enqueued
+    alpha_engine *e;
+    ~BlockScope() { release_blocks(e); }
+};
+
+static void *take_block(alpha_engine *e, size_t bytes)
+{
+    std::lock_guard<std::mutex> g(e->mu);
+    auto it = e->free_blocks.lower_bound(bytes);
+    void *p = nullptr;
+    size_t sz = bytes;
+    if (it != e->free_blocks.end() && it->first <= bytes * 2 + 4096) {
+        p = it->second;
+        sz = it->first;
+        e->free_blocks.erase(it);
+    } else if (hipMalloc(&p, bytes) != hipSuccess) {
+        return nullptr;
+    }
+    e->in_flight.emplace_back(sz, p);
+    return p;
+}
+
+alpha_engine *alpha_engine_create(int64_t stream)
+{
+    alpha_engine *e = new alpha_engine();
+    int cu = 0, clk = 0;
+    if (alpha_conv_device_info(&cu, &clk) != 0) cu = 0;
+    alpha_engine_config_default(&e->cfg, cu);
+    e->stream = stream;
+    e->err[0] = 0;
+    return e;
+}
+
+alpha_engine_config *alpha_engine_get_config(alpha_engine *e) { return &e->cfg; }
+const char *alpha_engine_last_error(alpha_engine *e) { return e->err; }
+
+int alpha_engine_sync(alpha_engine *e)
+{
+    hipError_t rc = hipStreamSynchronize(reinterpret_cast<hipStream_t>((intptr_t)e->stream));
+    release_blocks(e);
+    return (int)rc;
+}
+
+void alpha_engine_destroy(alpha_engine *e)
+{
+    if (!e) return;
+    alpha_engine_sync(e);
+    for (auto &b : e->free_blocks) (void)hipFree(b.second);
+    delete e;
+}
+
+// EngineCore.conv3D_param_check (EngineCore.java:630-678), non-strict form, minus the sh <= FH rule (see alpha_plan_conv3D).
+// Refusing inconsistent shapes here matters: the natives trust their arguments and would write out of bounds.
+static const char *param_check(int OH, int OW, int IH, int IW, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    if (OH <= 0 || OW <= 0) return "output size <= 0";
+    if (N <= 0 || IC <= 0 || OC <= 0) return "N, IC or OC <= 0";
+    if (sh <= 0 || sw <= 0) return "stride <= 0";
+    if (ph < 0 || pw < 0) return "padding < 0";
+    if (FH <= ph || FW <= pw) return "filter size <= padding";
+    if (FH > IH + (ph << 1) || FW > IW + (pw << 1)) return "filter larger than padded input";
+    if (IH - FH + (ph << 1) < (OH - 1) * sh) return "(IH - FH + 2*ph) < (OH - 1)*sh";
+    if (IW - FW + (pw << 1) < (OW - 1) * sw) return "(IW - FW + 2*pw) < (OW - 1)*sw";
+    if ((IC & 3) || (OC & 3)) return "IC and OC must be padded to multiples of 4";
+    return nullptr;
+}
+
+const char *alpha_engine_param_check(int OH, int OW, int IH, int IW, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    return param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw);
+}
+
+static int fail(alpha_engine *e, int rc, const char *what)
+{
+    snprintf(e->err, sizeof(e->err), "%s: %s", what, rc == -1 ? "scratch allocation failed" : alpha_conv_last_error());
+    return rc;
+}
+
+int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W, int FH, int FW,
+                        int N, int IC, int OC, int sh, int sw, int ph, int pw, alpha_conv_plan *plan_out)
+{
+    if (const char *why = param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw)) {
+        snprintf(e->err, sizeof(e->err), "%s: illegal size: %s", "alpha_engine_conv3D", why);
+        return ALPHA_CONV_EINVAL;
+    }
+    BlockScope scope{e};
+    alpha_conv_plan p;
+    alpha_plan_conv3D(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, ph, pw, &p);
+    if (plan_out) *plan_out = p;
+    int64_t streams[16];
+    for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
+    int rc = 0;
+    if (p.remode) {
+        float *CW = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        if (!CW) return fail(e, -1, "conv3D");
+        if ((rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");
+        switch (p.entry) {
+        case ALPHA_E_conv3D_GemmR_W1: rc = alpha_conv3D_GemmR_W1(streams, p.streams, X, IH, IW, W, CW, Y, N, IC, OC); break;
+        case ALPHA_E_conv3D_GemmV2R:
+            rc = alpha_conv3D_GemmV2R(p.useTexture, streams, p.streams, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+            break;
+        case ALPHA_E_conv3D_GemmR_texture:
+            rc = alpha_conv3D_GemmR_texture(streams, p.streams, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+            break;
+        default: rc = alpha_conv3D_GemmR(streams, p.streams, X, IH, IW, W, CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw); break;
+        }
+    } else {
+        switch (p.entry) {
+        case ALPHA_E_conv3D_W1: rc = alpha_conv3D_W1(streams, p.streams, X, IH, IW, W, Y, N, IC, OC); break;
+        case ALPHA_E_conv3D_np: rc = alpha_conv3D_np(streams, p.streams, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw); break;
+        case ALPHA_E_conv3DV2:
+            rc = alpha_conv3DV2(p.useTexture, streams, p.streams, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+            break;
+        case ALPHA_E_conv3D_texture:
+            rc = alpha_conv3D_texture(streams, p.streams, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+            break;
+        default: rc = alpha_conv3D(streams, p.streams, X, IH, IW, W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw); break;
+        }
+    }
+    return rc ? fail(e, rc, "conv3D") : 0;
+}
+
+int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, const float *X, int IH, int IW,
+                                const float *deltaY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                alpha_conv_plan *plan_out)
+{
+    if (const char *why = param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw)) {
+        snprintf(e->err, sizeof(e->err), "%s: illegal size: %s", "alpha_engine_dconv3D_deltaW", why);
+        return ALPHA_CONV_EINVAL;
+    }
+    BlockScope scope{e};
+    alpha_conv_plan p;
+    alpha_plan_deltaW(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    if (plan_out) *plan_out = p;
+    int64_t streams[16];
+    for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
+    int rc = 0;
+    if (p.GridZ == 1) {
+        rc = p.entry == ALPHA_E_dconv3D_deltaW_W1
+                 ? alpha_dconv3D_deltaW_W1(streams, p.streams, X, IH, IW, deltaY, deltaW, N, IC, OC)
+                 : alpha_dconv3D_deltaW(streams, p.streams, X, IH, IW, deltaY, OH, OW, deltaW, FH, FW, N, IC, OC, sh, sw, ph, pw);
+        return rc ? fail(e, rc, "dconv3D_deltaW") : 0;
+    }
+    float *buf = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+    if (!buf) return fail(e, -1, "dconv3D_deltaW");
+    switch (p.entry) {
+    case ALPHA_E_dconv3D_deltaW_GemmSK_W1:
+        rc = alpha_dconv3D_deltaW_GemmSK_W1(streams, p.streams, p.GridZ, X, IH, IW, deltaY, deltaW, buf, N, IC, OC);
+        break;
+    case ALPHA_E_dconv3D_deltaW_GemmV2SK:
+        rc = alpha_dconv3D_deltaW_GemmV2SK(streams, p.streams, p.GridZ, X, IH, IW, deltaY, OH, OW, deltaW, buf, FH, FW, N, IC, OC,
+                                           sh, sw, ph, pw);
+        break;
+    default:
+        rc = alpha_dconv3D_deltaW_GemmSK(streams, p.streams, p.GridZ, X, IH, IW, deltaY, OH, OW, deltaW, buf, FH, FW, N, IC, OC,
+                                         sh, sw, ph, pw);
+        break;
+    }
+    if (rc) return fail(e, rc, "dconv3D_deltaW");
+    rc = alpha_buf_summary(streams[0], buf, deltaW, p.GridZ - 1, OC * FH * FW * IC);
+    return rc ? fail(e, rc, "buf_summary") : 0;
+}
+
+int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
+                                const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                alpha_conv_plan *plan_out)
+{
+    if (const char *why = param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw)) {
+        snprintf(e->err, sizeof(e->err), "%s: illegal size: %s", "alpha_engine_dconv3D_deltaX", why);
+        return ALPHA_CONV_EINVAL;
+    }
+    BlockScope scope{e};
+    alpha_conv_plan p;
+    alpha_plan_deltaX(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    if (plan_out) *plan_out = p;
+    int64_t streams[16];
+    for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
+    int rc = 0;
+    switch (p.entry) {
+    case ALPHA_E_dconv3D_deltaX_crossAdd:
+        rc = alpha_dconv3D_deltaX_crossAdd(streams, p.streams, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
+        break;
+    case ALPHA_E_dconv3D_deltaX_W1:
+        rc = alpha_dconv3D_deltaX_W1(streams, p.streams, deltaY, W, deltaX, IH, IW, N, IC, OC);
+        break;
+    case ALPHA_E_dconv3D_deltaX_V2_s1:
+        rc = alpha_dconv3D_deltaX_V2_s1(p.useTexture, streams, p.streams, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+        break;
+    case ALPHA_E_dconv3D_deltaX_s1_texture:
+        rc = alpha_dconv3D_deltaX_s1_texture(streams, p.streams, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+        break;
+    case ALPHA_E_dconv3D_deltaX_s1:
+        rc = alpha_dconv3D_deltaX_s1(streams, p.streams, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+        break;
+    default: {
+        const int CFH = (FH + sh - 1) / sh, CFW = (FW + sw - 1) / sw;
+        float *CW = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        if (!CW) return fail(e, -1, "dconv3D_deltaX");
+        if ((rc = alpha_ks_remodev2(streams[0], W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw))) return fail(e, rc, "ks_remodev2");
+        switch (p.entry) {
+        case ALPHA_E_dconv3D_deltaX_ksV2_Ims2R:
+            rc = alpha_dconv3D_deltaX_ksV2_Ims2R(p.useTexture, streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+            break;
+        case ALPHA_E_dconv3D_deltaX_ksIms2R_texture:
+            rc = alpha_dconv3D_deltaX_ksIms2R_texture(streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+            break;
+        case ALPHA_E_dconv3D_deltaX_ksIms2R:
+            rc = alpha_dconv3D_deltaX_ksIms2R(streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);
+            break;
+        case ALPHA_E_dconv3D_deltaX_ksImsR_texture:
+            rc = alpha_dconv3D_deltaX_ksImsR_texture(streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
+            break;
+        case ALPHA_E_dconv3D_deltaX_ksImsR:
+            rc = alpha_dconv3D_deltaX_ksImsR(streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
+            break;
+        default:
+            rc = alpha_dconv3D_deltaX_kernelSplit(streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
+            break;
+        }
+    }
+    }
+    return rc ? fail(e, rc, "dconv3D_deltaX") : 0;
+}
+
+#pragma GCC visibility pop
+}  // extern "C"

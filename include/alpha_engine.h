@@ -1,0 +1,102 @@
+/*
+ * alpha_engine.h — host-side counterpart of the reference's Java algorithm selection for the conv3D path
+ * (src/alpha_src/z/dragon/engine/cuda/CudaFloat32EngineBase.java:1323-2005), restated in C++ because there is no JVM
+ * in the build environment. Two layers:
+ *   alpha_plan_*    pure integer functions: which native entry the Java engine would call for a layer, with how many
+ *                   stream handles, whether it remodes the filter, the split-K factor GridZ and the scratch size.
+ *   alpha_engine_*  an object that owns the scratch buffers (the Java engine takes them from its memory pool and frees
+ *                   them when the returned Syncer completes) and calls the natives of alpha_conv.h in the same order
+ *                   as the Java code: remode -> conv entry; split-K entry -> buf_summary; ks_remodev2 -> kernel-split.
+ * Flags and thresholds are the reference's fluent setters with their defaults.
+ */
+#ifndef ALPHA_ENGINE_H
+#define ALPHA_ENGINE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* CudaFloat32EngineBase.java:1324-1352 (forward), :1630-1663 (deltaW), :1765-1793 (deltaX) */
+typedef struct alpha_engine_config {
+    int conv3D_useTexture;        /* true */
+    int conv3D_remode;            /* true */
+    float conv3D_remode_V2_Q;     /* 1.05 */
+    float conv3D_V2_Q;            /* 1.25 */
+    int deltaW_SplitKThreshold;   /* 512 */
+    int deltaW_SK_MaxPartNum;     /* clip(#compute units, 16, 128)  (:73) */
+    float deltaW_SK_V2_Q;         /* 1.15 */
+    int deltaX_s1_useTexture;     /* true */
+    int deltaX_ks_useTexture;     /* false */
+    float deltaX_s1_V2_Q;         /* 1.1 */
+    float deltaX_ks_V2_Q;         /* 1.1 */
+} alpha_engine_config;
+
+/* Native entry chosen by a plan; names are the Java native method names. */
+enum alpha_entry {
+    ALPHA_E_conv3D = 1, ALPHA_E_conv3D_texture, ALPHA_E_conv3DV2, ALPHA_E_conv3D_np, ALPHA_E_conv3D_W1,
+    ALPHA_E_conv3D_GemmR, ALPHA_E_conv3D_GemmR_texture, ALPHA_E_conv3D_GemmV2R, ALPHA_E_conv3D_GemmR_W1,
+    ALPHA_E_dconv3D_deltaX_s1, ALPHA_E_dconv3D_deltaX_s1_texture, ALPHA_E_dconv3D_deltaX_V2_s1, ALPHA_E_dconv3D_deltaX_W1,
+    ALPHA_E_dconv3D_deltaX_kernelSplit, ALPHA_E_dconv3D_deltaX_ksImsR, ALPHA_E_dconv3D_deltaX_ksImsR_texture,
+    ALPHA_E_dconv3D_deltaX_ksIms2R, ALPHA_E_dconv3D_deltaX_ksIms2R_texture, ALPHA_E_dconv3D_deltaX_ksV2_Ims2R,
+    ALPHA_E_dconv3D_deltaX_crossAdd,
+    ALPHA_E_dconv3D_deltaW, ALPHA_E_dconv3D_deltaW_W1, ALPHA_E_dconv3D_deltaW_GemmSK, ALPHA_E_dconv3D_deltaW_GemmV2SK,
+    ALPHA_E_dconv3D_deltaW_GemmSK_W1
+};
+
+typedef struct alpha_conv_plan {
+    int entry;            /* enum alpha_entry */
+    int streams;          /* length of the stream array the Java engine would pass */
+    int remode;           /* 1 when kernel_remode / ks_remodev2 runs first */
+    int V2;               /* the "V2" variant was chosen */
+    int useTexture;       /* flag passed to entries that take one */
+    int GridZ;            /* split-K factor (deltaW), 1 = single pass */
+    long scratch_floats;  /* CW or deltaW_buf size */
+    double Q;             /* padding scale-up the decision was based on */
+} alpha_conv_plan;
+
+/* Integer helpers of the Java native classes. GN, GM are the implicit-GEMM extents each class uses:
+ * forward (OC, N*OH*OW), deltaX (IC, N*IH*IW), deltaW (OC, FH*FW*IC); the V2 variants pass (OC, N) etc. and multiply
+ * blockNum by the spatial size themselves. Cuda_conv3D.java:19-126, Cuda_dconv3D_deltaX.java:19-190, Cuda_dconv3D_deltaW.java:19-128. */
+int alpha_blockNum(int GN, int GM);
+int alpha_streamSize(int GN, int GM, int cap);
+double alpha_paddingScaleUp(int IH, int IW, int OH, int OW, int FH, int FW, int sh, int sw);
+
+void alpha_engine_config_default(alpha_engine_config *c, int compute_units);
+
+/* EngineCore.conv3D_param_check (EngineCore.java:630-678, non-strict) minus its sh <= FH rule: NULL when the sizes are
+ * consistent, else the reason. The engine calls refuse (ALPHA_CONV_EINVAL) what this refuses. */
+const char *alpha_engine_param_check(int OH, int OW, int IH, int IW, int FH, int FW, int N, int IC, int OC,
+                                     int sh, int sw, int ph, int pw);
+
+void alpha_plan_conv3D(const alpha_engine_config *c, int IH, int IW, int OH, int OW, int FH, int FW, int N, int IC, int OC,
+                       int sh, int sw, int ph, int pw, alpha_conv_plan *out);
+void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int OW, int FH, int FW, int N, int IC, int OC,
+                       int sh, int sw, alpha_conv_plan *out);
+void alpha_plan_deltaX(const alpha_engine_config *c, int IH, int IW, int OH, int OW, int FH, int FW, int N, int IC, int OC,
+                       int sh, int sw, alpha_conv_plan *out);
+
+/* Engine object. `stream` is the hipStream_t (as int64) every call is enqueued on; it is replicated plan.streams times
+ * in the stream array handed to the natives. Argument order of the three operators follows EngineBase.java:171-199
+ * (output first). Scratch is recycled in stream order (one stream per engine); alpha_engine_sync() waits for the stream. */
+typedef struct alpha_engine alpha_engine;
+alpha_engine *alpha_engine_create(int64_t stream);
+void alpha_engine_destroy(alpha_engine *e);
+alpha_engine_config *alpha_engine_get_config(alpha_engine *e);
+const char *alpha_engine_last_error(alpha_engine *e);
+int alpha_engine_sync(alpha_engine *e);
+
+int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W, int FH, int FW,
+                        int N, int IC, int OC, int sh, int sw, int ph, int pw, alpha_conv_plan *plan_out);
+int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, const float *X, int IH, int IW,
+                                const float *deltaY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                alpha_conv_plan *plan_out);
+int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
+                                const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                alpha_conv_plan *plan_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ALPHA_ENGINE_H */

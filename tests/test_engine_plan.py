@@ -1,0 +1,123 @@
+"""The host-side selection logic (include/alpha_engine.h) against values computed by hand from the reference's Java
+formulas (CudaFloat32EngineBase.java:1355-1474, 1666-1762, 1796-2005; Cuda_conv3D.java:19-135 and twins). Pure integer
+functions: no GPU needed."""
+import pytest
+
+from util import load_package
+
+pkg = load_package()
+E = pkg.engine
+
+
+def java_blockNum(GN, GM):
+    """Independent restatement of the Java loop as arithmetic on the binary digits."""
+    def side(g):
+        return g // 128 + sum(1 for b in (64, 32, 16, 8, 4) if g % 128 & b)
+    return side(GN) * side(GM)
+
+
+def test_blockNum_and_streamSize_hand_values():
+    assert E.blockNum(64, 100352) == 784              # 1 x 784 whole 128-tiles
+    assert E.blockNum(64, 576) == 5                   # 576 = 4*128 + 64
+    assert E.blockNum(252, 4096) == (1 + 5) * 32      # 252 = 128 + 64+32+16+8+4
+    assert E.blockNum(4, 4) == 1
+    for gn, gm in [(64, 200704), (132, 36), (1024, 12544), (20, 52), (255 // 4 * 4, 100)]:
+        assert E.blockNum(gn, gm) == java_blockNum(gn, gm)
+    assert E.streamSize(64, 4096) == 1                # both powers of two
+    assert E.streamSize(252, 4096) == 6               # 128 + 64+32+16+8+4 -> 6 strips
+    assert E.streamSize(252, 100) == 10               # 6 x 3 = 18, capped at 10   (100 = 64+32+4)
+    assert E.streamSize(252, 100, 12) == 12
+    assert E.streamSize(1024, 12544) == 1             # 12544 = 98*128: one strip
+
+
+def test_forward_plans_of_the_baseline_configs():
+    cfg = E.default_config(256)
+    # c3a: N=64 > 63, OC=64 > 63, Q = 58*58/(56*56) = 1.0727 > 1.05  ->  V2 entry, one stream (64, 64 powers of two)
+    p = E.plan_conv3D(cfg, 56, 56, 56, 56, 3, 3, 64, 64, 64, 1, 1, 1, 1)
+    assert p.entry_name == "conv3D_GemmV2R" and p.remode == 1 and p.V2 == 1 and p.streams == 1
+    assert p.Q == pytest.approx(3364 / 3136) and p.scratch_floats == 3 * 3 * 64 * 64
+    # c1: N=4 -> not V2; texture flag on -> GemmR_texture
+    p = E.plan_conv3D(cfg, 32, 32, 32, 32, 3, 3, 4, 4, 64, 1, 1, 1, 1)
+    assert p.entry_name == "conv3D_GemmR_texture" and p.streams == 1
+    # c4d: 1x1 -> GemmR_W1
+    p = E.plan_conv3D(cfg, 14, 14, 14, 14, 1, 1, 64, 256, 1024, 1, 1, 0, 0)
+    assert p.entry_name == "conv3D_GemmR_W1" and p.V2 == 0
+    # c4a stem: N=64, OC=64, Q = (111*2+7)^2/224^2 = 1.045 < 1.05 -> GemmR_texture
+    p = E.plan_conv3D(cfg, 224, 224, 112, 112, 7, 7, 64, 4, 64, 2, 2, 3, 3)
+    assert p.entry_name == "conv3D_GemmR_texture" and p.Q == pytest.approx(229 * 229 / 224 / 224)
+    # small problems take the non-remode entries
+    assert E.plan_conv3D(cfg, 8, 8, 8, 8, 3, 3, 4, 8, 16, 1, 1, 1, 1).entry_name == "conv3D_texture"
+    assert E.plan_conv3D(cfg, 8, 8, 8, 8, 3, 3, 4, 8, 8, 1, 1, 1, 1).entry_name == "conv3D"       # OC <= 15: no texture
+    assert E.plan_conv3D(cfg, 8, 8, 6, 6, 3, 3, 4, 8, 16, 1, 1, 0, 0).entry_name == "conv3D_np"
+    assert E.plan_conv3D(cfg, 8, 8, 8, 8, 1, 1, 4, 8, 16, 1, 1, 0, 0).entry_name == "conv3D_W1"
+    cfg.conv3D_remode = 0
+    assert E.plan_conv3D(cfg, 8, 8, 8, 8, 3, 3, 128, 128, 128, 1, 1, 1, 1).entry_name == "conv3DV2"  # Q=1.5625 >= 1.25
+    cfg.conv3D_remode, cfg.conv3D_useTexture = 1, 0
+    assert E.plan_conv3D(cfg, 32, 32, 32, 32, 3, 3, 4, 4, 64, 1, 1, 1, 1).entry_name == "conv3D_GemmR"
+
+
+def test_deltaW_plans_and_split_k_factor():
+    cfg = E.default_config(256)
+    assert cfg.deltaW_SK_MaxPartNum == 128 and E.default_config(8).deltaW_SK_MaxPartNum == 16
+    # c5b: GK = 100352; b1 = b2 = 784, b3 = 5 -> (784+784)/10 = 156 -> capped by MaxPartNum 128 (GK>>8 = 392)
+    p = E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1)
+    assert p.entry_name == "dconv3D_deltaW_GemmSK" and p.GridZ == 128 and p.scratch_floats == 127 * 36864
+    # c5a (1x1, 256 -> 64): b1 = 784, b2 = 2*784, b3 = 2 -> 588 -> 128
+    p = E.plan_deltaW(cfg, 56, 56, 56, 56, 1, 1, 32, 256, 64, 1, 1)
+    assert p.entry_name == "dconv3D_deltaW_GemmSK_W1" and p.GridZ == 128
+    cfg.deltaW_SK_MaxPartNum = 1000
+    assert E.plan_deltaW(cfg, 56, 56, 56, 56, 1, 1, 32, 256, 64, 1, 1).GridZ == 392    # min(588, 1000, GK>>8 = 392)
+    cfg = E.default_config(256)
+    # c2c: Q = 10*10/64 = 1.5625 >= 1.15, OC, IC > 63 -> V2; b1 = b2 = 2*1*64, b3 = 2*2*9 -> 256/72 = 3
+    p = E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 128, 256, 256, 1, 1)
+    assert p.entry_name == "dconv3D_deltaW_GemmV2SK" and p.GridZ == 3 and p.V2 == 1
+    # c2b: Q = 18*18/256 = 1.266 -> V2; b1 = b2 = 256, b3 = 9 -> 512/18 = 28
+    assert E.plan_deltaW(cfg, 16, 16, 16, 16, 3, 3, 128, 128, 128, 1, 1).GridZ == 28
+    # GK < 512: single pass
+    p = E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 4, 16, 16, 1, 1)
+    assert p.entry_name == "dconv3D_deltaW" and p.GridZ == 1 and p.scratch_floats == 0
+    assert E.plan_deltaW(cfg, 8, 8, 8, 8, 1, 1, 4, 16, 16, 1, 1).entry_name == "dconv3D_deltaW_W1"
+    # GridZ floor of 2 and the GK>>8 cap: GK = 512 -> GridZ2 = 2
+    assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 8, 16, 16, 1, 1).GridZ == 2
+
+
+def test_deltaX_plans():
+    cfg = E.default_config(256)
+    assert E.plan_deltaX(cfg, 224, 224, 112, 112, 7, 7, 64, 4, 64, 2, 2).entry_name == "dconv3D_deltaX_crossAdd"   # IC <= 8
+    assert E.plan_deltaX(cfg, 16, 16, 8, 8, 3, 3, 8, 16, 32, 2, 2).entry_name == "dconv3D_deltaX_crossAdd"        # IC <= 16, s*s >= 4
+    assert E.plan_deltaX(cfg, 56, 56, 56, 56, 1, 1, 32, 256, 64, 1, 1).entry_name == "dconv3D_deltaX_W1"
+    # c5b: N=32 -> not V2; texture on, IC > 15
+    assert E.plan_deltaX(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).entry_name == "dconv3D_deltaX_s1_texture"
+    # c2a: N=128, IC=64, Q = 34*34/1024 = 1.129 > 1.1 -> V2
+    p = E.plan_deltaX(cfg, 32, 32, 32, 32, 3, 3, 128, 64, 64, 1, 1)
+    assert p.entry_name == "dconv3D_deltaX_V2_s1" and p.Q == pytest.approx(1156 / 1024)
+    cfg.deltaX_s1_useTexture = 0
+    assert E.plan_deltaX(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).entry_name == "dconv3D_deltaX_s1"
+    cfg = E.default_config(256)
+    # stride 2, even input: Ims2 family. N=32 -> not V2, ks texture off
+    p = E.plan_deltaX(cfg, 56, 56, 28, 28, 3, 3, 32, 64, 128, 2, 2)
+    assert p.entry_name == "dconv3D_deltaX_ksIms2R" and p.remode == 1 and p.scratch_floats == 128 * 2 * 2 * 64 * 4
+    # N=64, IC=64: Q = 0.25*((28+1)+(28+0))^2/(28*28) = 0.25*57*57/784 = 1.036 < 1.1 -> still not V2
+    assert E.plan_deltaX(cfg, 56, 56, 28, 28, 3, 3, 64, 64, 128, 2, 2).entry_name == "dconv3D_deltaX_ksIms2R"
+    # 8x8 input, 5x5: Q = 0.25*((4+2)+(4+1))^2/16 = 1.89 -> V2
+    assert E.plan_deltaX(cfg, 8, 8, 4, 4, 5, 5, 64, 64, 64, 2, 2).entry_name == "dconv3D_deltaX_ksV2_Ims2R"
+    assert E.plan_deltaX(cfg, 12, 9, 4, 3, 3, 3, 8, 32, 32, 3, 3).entry_name == "dconv3D_deltaX_ksImsR"          # IH%sh == 0
+    assert E.plan_deltaX(cfg, 13, 11, 5, 5, 5, 4, 8, 32, 32, 3, 2).entry_name == "dconv3D_deltaX_kernelSplit"
+    assert E.plan_deltaX(cfg, 9, 9, 4, 4, 3, 3, 8, 32, 32, 2, 2).entry_name == "dconv3D_deltaX_kernelSplit"      # odd IH, stride 2
+
+
+def test_w1_entries_only_for_stride_one_and_sizes_are_checked():
+    cfg = E.default_config(256)
+    # 1x1 stride 2 (BASELINE c4c): the W1 natives carry no stride, so the general entries must be used
+    assert E.plan_conv3D(cfg, 56, 56, 28, 28, 1, 1, 64, 64, 128, 2, 2, 0, 0).entry_name == "conv3D_GemmR_texture"
+    assert E.plan_conv3D(cfg, 56, 56, 56, 56, 1, 1, 64, 64, 128, 1, 1, 0, 0).entry_name == "conv3D_GemmR_W1"
+    assert E.plan_deltaW(cfg, 56, 56, 28, 28, 1, 1, 64, 64, 128, 2, 2).entry_name == "dconv3D_deltaW_GemmSK"
+    assert E.plan_deltaX(cfg, 56, 56, 28, 28, 1, 1, 64, 64, 128, 2, 2).entry_name == "dconv3D_deltaX_ksIms2R"
+    # EngineCore.conv3D_param_check conditions
+    ok = (28, 28, 56, 56, 3, 3, 64, 64, 128, 2, 2, 1, 1)
+    assert E.param_check(*ok) is None
+    assert "(IH - FH + 2*ph) < (OH - 1)*sh" in E.param_check(56, 28, 56, 56, 3, 3, 64, 64, 128, 2, 2, 1, 1)   # OH too large
+    assert "(IW - FW + 2*pw) < (OW - 1)*sw" in E.param_check(28, 56, 56, 56, 3, 3, 64, 64, 128, 2, 2, 1, 1)
+    assert "padding" in E.param_check(28, 28, 56, 56, 3, 3, 64, 64, 128, 2, 2, 3, 1)                           # FH <= ph
+    assert "multiples of 4" in E.param_check(28, 28, 56, 56, 3, 3, 64, 62, 128, 2, 2, 1, 1)
+    assert "stride" in E.param_check(28, 28, 56, 56, 3, 3, 64, 64, 128, 0, 2, 1, 1)

@@ -1,0 +1,83 @@
+"""GPU: the C++ host layer (alpha_engine_*) end to end — it picks the entry the Java engine would pick, owns the
+scratch, and the result matches the oracle to the parity bar of test_gpu_parity.py."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from util import Dev, he_normal, load_package, normal, out_dim
+
+pytestmark = pytest.mark.gpu
+pkg = load_package()
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return Dev()
+
+
+@pytest.fixture(scope="module")
+def eng(dev):
+    e = pkg.engine.Engine(dev.stream)
+    yield e
+    e.close()
+
+
+def check(got, want, what):
+    floor = 1e-5 * max(1.0, float(np.sqrt(np.mean(want * want))))
+    r = O.max_err_ratio(got, want, 1e-4, floor)
+    assert r <= 1.0, "%s: err/allowed = %.3f (rel 1e-4, abs floor %.3g)" % (what, r, floor)
+
+
+CASES = [
+    # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw, fwd entry, dX entry, dW entry
+    (64, 14, 14, 64, 64, 3, 3, 1, 1, 1, 1, "conv3D_GemmV2R", "dconv3D_deltaX_V2_s1", "dconv3D_deltaW_GemmV2SK"),
+    (8, 28, 28, 64, 64, 3, 3, 1, 1, 1, 1, "conv3D_GemmR_texture", "dconv3D_deltaX_s1_texture", "dconv3D_deltaW_GemmSK"),
+    (8, 14, 14, 64, 128, 1, 1, 1, 1, 0, 0, "conv3D_GemmR_W1", "dconv3D_deltaX_W1", "dconv3D_deltaW_GemmSK_W1"),
+    (8, 28, 28, 32, 64, 3, 3, 2, 2, 1, 1, "conv3D_GemmR_texture", "dconv3D_deltaX_ksIms2R", "dconv3D_deltaW_GemmSK"),
+    (4, 32, 32, 4, 64, 7, 7, 2, 2, 3, 3, "conv3D_GemmR_texture", "dconv3D_deltaX_crossAdd", "dconv3D_deltaW_GemmSK"),
+    (4, 12, 9, 32, 32, 3, 3, 3, 3, 1, 1, "conv3D_GemmR_texture", "dconv3D_deltaX_ksImsR", "dconv3D_deltaW"),
+    (4, 13, 11, 32, 16, 5, 4, 3, 2, 2, 1, "conv3D_texture", "dconv3D_deltaX_kernelSplit", "dconv3D_deltaW"),
+    (4, 9, 9, 16, 8, 3, 3, 1, 1, 0, 0, "conv3D_np", "dconv3D_deltaX_s1_texture", "dconv3D_deltaW"),
+    # 1x1 stride 2 (BASELINE c4c geometry): must NOT go to the stride-less W1 natives
+    (8, 28, 28, 64, 128, 1, 1, 2, 2, 0, 0, "conv3D_GemmR_texture", "dconv3D_deltaX_ksIms2R", "dconv3D_deltaW_GemmSK"),
+]
+
+
+def test_engine_refuses_inconsistent_sizes(dev, eng):
+    x = dev.empty(4, 8, 8, 8, fill=0.0)
+    w = dev.empty(8, 3, 3, 8, fill=0.0)
+    y = dev.empty(4, 8, 8, 8, fill=0.0)
+    with pytest.raises(pkg.AlphaConvError, match="illegal size"):
+        eng.conv3D(y.data_ptr(), 16, 16, x.data_ptr(), 8, 8, w.data_ptr(), 3, 3, 4, 8, 8, 1, 1, 1, 1)   # OH larger than the input allows
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_engine_runs_the_entry_java_would_pick(dev, eng, case):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw, e_fwd, e_dx, e_dw = case
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    X, W, dY = normal((N, IH, IW, IC), 6001), he_normal(OC, FH, FW, IC, 6002), normal((N, OH, OW, OC), 6003)
+    x, w, dy = dev.put(X), dev.put(W), dev.put(dY)
+    y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    dx = dev.empty(N, IH, IW, IC, fill=float("nan"))
+    dw = dev.empty(OC, FH, FW, IC, fill=float("nan"))
+    p1 = eng.conv3D(y.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
+    p2 = eng.dconv3D_deltaX(dx.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
+    p3 = eng.dconv3D_deltaW(dw.data_ptr(), FH, FW, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, sh, sw, ph, pw)
+    eng.sync()
+    assert (p1.entry_name, p2.entry_name, p3.entry_name) == (e_fwd, e_dx, e_dw)
+    check(dev.get(y), O.conv3D_f64(X, W, sh, sw, ph, pw), "engine conv3D %s" % (case,))
+    check(dev.get(dx), O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw), "engine deltaX %s" % (case,))
+    check(dev.get(dw), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "engine deltaW %s" % (case,))
+
+
+def test_engine_scratch_is_recycled_after_sync(dev, eng):
+    N, IH, IC, OC = 8, 16, 32, 64
+    X, W = normal((N, IH, IH, IC), 6004), he_normal(OC, 3, 3, IC, 6005)
+    x, w = dev.put(X), dev.put(W)
+    want = O.conv3D_f64(X, W, 1, 1, 1, 1)
+    for _ in range(3):
+        y = dev.empty(N, IH, IH, OC, fill=float("nan"))
+        for _ in range(4):   # several enqueues between syncs: each takes its own CW block
+            eng.conv3D(y.data_ptr(), IH, IH, x.data_ptr(), IH, IH, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1)
+        eng.sync()
+        check(dev.get(y), want, "repeat")
