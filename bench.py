@@ -91,9 +91,8 @@ class Workload:
         # split-K factor for the kernel-only timing: what the host layer would pass (CudaFloat32EngineBase.java:1707-1715)
         self.GridZ = max(1, pkg.engine.plan_deltaW(self.engine.config, IH, IW, OH, OW, F, F, N, IC, OC, s, s).GridZ)
         self.buf = torch.empty(max(1, self.GridZ - 1) * self.dW.numel(), device=dev)
-        if s > 1:
-            CFH = (F + s - 1) // s
-            self.KCW = torch.empty(s * s * OC * CFH * CFH * IC, device=dev)
+        if F == 3 and s == 1:
+            self.U = torch.empty(16 * IC * OC, device=dev)
 
     # forward: remode + GemmR entry (W1 entry for 1x1 stride 1), as CudaFloat32EngineBase.conv3D does
     def fwd_remode(self):
@@ -109,6 +108,16 @@ class Workload:
         else:
             C.conv3D_GemmV2R(True, self.streams, 1, self.X.data_ptr(), IH, IW, self.W.data_ptr(), self.CW.data_ptr(), F, F,
                              self.Y.data_ptr(), self.OH, self.OW, N, IC, OC, s, s, p, p)
+
+    def wino_conv(self):
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.pkg.Cuda_conv3D.conv3D_winograd(self.streams, 1, self.X.data_ptr(), IH, IW, self.U.data_ptr(), self.Y.data_ptr(),
+                                             self.OH, self.OW, N, IC, OC, p, p)
+
+    def wino(self):
+        self.engine.config.conv3D_winograd = 1
+        self.fwd()
+        self.engine.config.conv3D_winograd = 0
 
     def fwd(self):
         # whole operator through the C++ host layer: entry selection, CW scratch, kernel_remode, conv entry
@@ -212,10 +221,13 @@ def load_traffic(layer, op):
 
 def measure(pkg, torch, layer, op, steps, warmup):
     wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer))
-    step = {"fwd": wl.fwd, "dx": wl.dx_op, "dw": wl.dw}[op]
-    kernel = {"fwd": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm}[op]
+    step = {"fwd": wl.fwd, "dx": wl.dx_op, "dw": wl.dw, "wino": wl.wino}[op]
+    kernel = {"fwd": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "wino": wl.wino_conv}[op]
     if op == "fwd":
         wl.fwd_remode()
+    if op == "wino":
+        N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
+        pkg.Cuda_conv3D.winograd_filter_transform(wl.stream, wl.W.data_ptr(), wl.U.data_ptr(), IC_, OC_)
     def step_and_recycle():
         step()
     wall_ms, ev_ms = time_loop(torch, step_and_recycle, steps, warmup)
@@ -245,7 +257,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
-    ap.add_argument("--op", default=None, choices=["fwd", "dx", "dw"])
+    ap.add_argument("--op", default=None, choices=["fwd", "dx", "dw", "wino"],
+                    help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="also measure every layer/op of BASELINE.json's configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--probe-copy", action="store_true",
@@ -295,7 +308,10 @@ def main():
     if args.layers:
         out["layers"] = []
         for layer in sorted(LAYERS):
-            for o in LAYERS[layer][9]:
+            ops = list(LAYERS[layer][9])
+            if "fwd" in ops and LAYERS[layer][5] == 3 and LAYERS[layer][6] == 1 and LAYERS[layer][3] >= 16:
+                ops.append("wino")
+            for o in ops:
                 out["layers"].append(measure(pkg, torch, layer, o, max(5, args.steps // 5), max(2, args.warmup // 3)))
                 torch.cuda.empty_cache()
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(args.layer, op)

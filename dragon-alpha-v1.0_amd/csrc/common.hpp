@@ -80,6 +80,17 @@ struct DeltaWArgs {
 
 hipError_t launch_deltaW(hipStream_t stream, const DeltaWArgs &a);
 
+// Row-streaming backward-filter for stride-1 3x3 and 1x1 layers (delta_w_rows.hip); same split-K contract as
+// launch_deltaW. Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
+hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
+                              int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,
+                              int sh, int sw, int ph, int pw, int GK_slice, int GZ);
+
+// Winograd F(2x2,3x3) forward (winograd.hip): U = transformed filter [16][IC][OC].
+hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC);
+hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
+                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw);
+
 // Re-layout / reduction helpers.
 hipError_t launch_kernel_remode(hipStream_t s, const float *W, float *CW, int FH, int FW, int OC, int IC);
 hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, int FW, float *CW,

@@ -197,6 +197,11 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     a.GK = N * OH * OW;
     a.GZ = GridZ;
     a.GK_slice = (a.GK / GridZ) >> 3 << 3;
+    if (fwd_algo() != 3) {
+        hipError_t e = launch_deltaW_rows(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
+                                          a.GK_slice, GridZ);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     return hip_status(launch_deltaW(stream0(streams), a), fn);
 }
 
@@ -406,18 +411,26 @@ int alpha_dconv3D_deltaW_GemmSK_W1(const int64_t *streams, int length, int GridZ
     return deltaW_impl(__func__, streams, length, GridZ, X, IH, IW, deltaY, IH, IW, deltaW, deltaW_buf, 1, 1, N, IC, OC, 1, 1, 0, 0);
 }
 
-// ---- Winograd (filled in by winograd.hip once built) ------------------------------------------
+// ---- Winograd F(2x2,3x3): additional forward algorithm of this build ----------------------------------------
 long alpha_winograd_filter_size(int IC, int OC) { return 16L * IC * OC; }
 int alpha_winograd_filter_transform(int64_t stream, const float *W, float *U, int IC, int OC)
 {
-    (void)stream; (void)W; (void)U; (void)IC; (void)OC;
-    return fail(ALPHA_CONV_EINVAL, "%s: not available in this build", __func__);
+    CHECK_PTR(W);
+    CHECK_PTR(U);
+    if (IC < 4 || OC < 4 || (IC & 3) || (OC & 3)) return fail(ALPHA_CONV_EINVAL, "%s: IC and OC must be multiples of 4", __func__);
+    return hip_status(launch_winograd_filter(reinterpret_cast<hipStream_t>((intptr_t)stream), W, U, IC, OC), __func__);
 }
 int alpha_conv3D_winograd(const int64_t *streams, int length, const float *X, int IH, int IW, const float *U, float *Y,
                           int OH, int OW, int N, int IC, int OC, int ph, int pw)
 {
-    (void)streams; (void)length; (void)X; (void)IH; (void)IW; (void)U; (void)Y; (void)OH; (void)OW; (void)N; (void)IC; (void)OC; (void)ph; (void)pw;
-    return fail(ALPHA_CONV_EINVAL, "%s: not available in this build", __func__);
+    CHECK_STREAMS();
+    CHECK_PTR(X);
+    CHECK_PTR(U);
+    CHECK_PTR(Y);
+    if (int e = check_dims(__func__, N, IC, OC, IH, IW, OH, OW, 3, 3, 1, 1, ph, pw)) return e;
+    hipError_t e = launch_winograd(stream0(streams), X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw);
+    if (e == hipErrorNotSupported) return fail(ALPHA_CONV_EINVAL, "%s: needs OH = IH + 2*ph - 2, OW = IW + 2*pw - 2", __func__);
+    return hip_status(e, __func__);
 }
 
 }  // extern "C"

@@ -62,6 +62,7 @@ void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
     c->deltaX_ks_useTexture = 0;
     c->deltaX_s1_V2_Q = 1.1f;
     c->deltaX_ks_V2_Q = 1.1f;
+    c->conv3D_winograd = 0;
 }
 
 // ---- forward: CudaFloat32EngineBase.conv3D (:1355-1474) ----------------------------------------------
@@ -72,6 +73,13 @@ void alpha_plan_conv3D(const alpha_engine_config *c, int IH, int IW, int OH, int
     memset(out, 0, sizeof(*out));
     const double Q = alpha_paddingScaleUp(IH, IW, OH, OW, FH, FW, sh, sw);
     out->Q = Q;
+    if (c->conv3D_winograd && FH == 3 && FW == 3 && sh == 1 && sw == 1) {
+        out->entry = ALPHA_E_conv3D_winograd;
+        out->remode = 1;   // the filter transform takes the place of kernel_remode
+        out->streams = 1;
+        out->scratch_floats = 16L * IC * OC;
+        return;
+    }
     if (c->conv3D_remode && OC > 31 && N * OH * OW > 31) {
         const bool V2 = N > 63 && OC > 63 && Q > c->conv3D_remode_V2_Q;
         out->remode = 1;
@@ -296,7 +304,12 @@ int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *
     int64_t streams[16];
     for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
     int rc = 0;
-    if (p.remode) {
+    if (p.entry == ALPHA_E_conv3D_winograd) {
+        float *U = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        if (!U) return fail(e, -1, "conv3D");
+        if ((rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform");
+        rc = alpha_conv3D_winograd(streams, p.streams, X, IH, IW, U, Y, OH, OW, N, IC, OC, ph, pw);
+    } else if (p.remode) {
         float *CW = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
         if (!CW) return fail(e, -1, "conv3D");
         if ((rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");

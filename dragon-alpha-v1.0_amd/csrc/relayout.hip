@@ -95,49 +95,42 @@ hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, 
 }
 
 // deltaW += sum_{p < part} deltaW_buf[p], summed in the fixed order p = 0, 1, ... with fp32 Kahan
-// compensation; one thread owns four consecutive elements for the whole sum.
+// compensation (the reference's recurrence, operation for operation). The adds of one element form a serial
+// chain, but the loads do not depend on it: one thread owns ONE element (so even a 16 K-element filter gives
+// hundreds of wavefronts) and fetches 16 partials at a time before running them through the chain.
 __global__ __launch_bounds__(256) void buf_summary_kernel(const float *__restrict__ buf, float *__restrict__ dW,
                                                           int part, int sizeW)
 {
-    const int n4 = sizeW >> 2;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += gridDim.x * blockDim.x) {
-        float4 dw = *reinterpret_cast<const float4 *>(dW + (size_t)i * 4);
-        float4 c = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int p = 0; p < part; p++) {
-            float4 b = *reinterpret_cast<const float4 *>(buf + (size_t)p * sizeW + (size_t)i * 4);
-            b.x -= c.x; b.y -= c.y; b.z -= c.z; b.w -= c.w;
-            float4 s;
-            s.x = dw.x + b.x; s.y = dw.y + b.y; s.z = dw.z + b.z; s.w = dw.w + b.w;
-            c.x = (s.x - dw.x) - b.x;
-            c.y = (s.y - dw.y) - b.y;
-            c.z = (s.z - dw.z) - b.z;
-            c.w = (s.w - dw.w) - b.w;
+    constexpr int U = 16;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= sizeW) return;
+    float dw = dW[i], c = 0.f;
+    int p = 0;
+    for (; p + U <= part; p += U) {
+        float b[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) b[u] = buf[(size_t)(p + u) * sizeW + i];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float y = b[u] - c;
+            const float s = dw + y;
+            c = (s - dw) - y;
             dw = s;
         }
-        *reinterpret_cast<float4 *>(dW + (size_t)i * 4) = dw;
     }
-    // sizeW is a multiple of 4 on this path (IC % 4 == 0); a ragged tail is summed scalar-wise.
-    const int tail = sizeW & 3;
-    if (tail && blockIdx.x == 0 && threadIdx.x < tail) {
-        const int i = (n4 << 2) + threadIdx.x;
-        float dw = dW[i], c = 0.f;
-        for (int p = 0; p < part; p++) {
-            float b = buf[(size_t)p * sizeW + i] - c;
-            float s = dw + b;
-            c = (s - dw) - b;
-            dw = s;
-        }
-        dW[i] = dw;
+    for (; p < part; p++) {
+        const float y = buf[(size_t)p * sizeW + i] - c;
+        const float s = dw + y;
+        c = (s - dw) - y;
+        dw = s;
     }
+    dW[i] = dw;
 }
 
 hipError_t launch_buf_summary(hipStream_t s, const float *buf, float *dW, int part, int sizeW)
 {
     if (sizeW <= 0 || part <= 0) return hipSuccess;
-    int bx = ((sizeW >> 2) + 255) / 256;
-    if (bx < 1) bx = 1;
-    if (bx > 8192) bx = 8192;
-    hipLaunchKernelGGL(buf_summary_kernel, dim3(bx), dim3(256), 0, s, buf, dW, part, sizeW);
+    hipLaunchKernelGGL(buf_summary_kernel, dim3((sizeW + 255) / 256), dim3(256), 0, s, buf, dW, part, sizeW);
     return hipGetLastError();
 }
 

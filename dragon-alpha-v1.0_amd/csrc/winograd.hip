@@ -1,0 +1,271 @@
+// Winograd F(2x2, 3x3) forward convolution, fully fused (input transform -> 16 MFMA GEMMs -> output
+// transform in one kernel), fp32 MFMA v_mfma_f32_16x16x4_f32, gfx950. For FH = FW = 3, stride 1.
+//
+//   Y_tile = A^T [ sum_ic (G g G^T) .* (B^T d B) ] A      with 2x2 output tiles from 4x4 input patches.
+//
+// The reference ships no Winograd (its experiments are compiled out); this is an additional algorithm of this
+// build behind the same forward entries, checked against the same CPU direct convolution.
+//
+// A workgroup (4 wavefronts) owns 32 consecutive tiles of the flattened (n, tile row, tile column) index
+// (= 128 output pixels) and 64 output channels; wavefront w owns output channels [16w, 16w+16) for all 16
+// transform positions xi, i.e. 16 x 2 accumulator tiles. Because a lane then holds all 16 xi values of
+// its (tile, channel) pairs, the output transform is pure per-lane register arithmetic.
+// Input channels advance in chunks of 16: every thread loads the 4x4 patch of one (tile, channel pair) of the
+// next chunk from global memory before the MFMAs of the current chunk, transforms it afterwards and writes
+// V[xi][tile][16 channels] into the other LDS buffer. A fragment = one conflict-free 128-bit LDS read (a 16-lane
+// group reads 16 tiles x 64 contiguous bytes); the transformed-filter fragment U[xi][ic][oc] comes straight from
+// L2 four xi ahead.
+#include "common.hpp"
+
+namespace alpha {
+
+struct WinoArgs {
+    const float *X;   // [N, IH, IW, IC]
+    const float *U;   // [16][IC][OC] transformed filter
+    float *Y;         // [N, OH, OW, OC]
+    int N, IH, IW, IC, OH, OW, OC;
+    int ph, pw;
+    int TR, TC;       // tile rows / columns per image: ceil(OH/2), ceil(OW/2)
+    int ntiles;       // N*TR*TC
+    FastDiv d_TC, d_TRC;
+};
+
+constexpr int WG_TILES = 32;
+constexpr int WG_VBUF = 16 * WG_TILES * 16;   // floats per V buffer: [xi][tile][16 channels]
+
+// U[xi = 4a + b][ic][oc] = (G g G^T)[a][b],  G = [[1,0,0],[.5,.5,.5],[.5,-.5,.5],[0,0,1]],  g = W[oc][.][.][ic]
+__global__ __launch_bounds__(256) void winograd_filter_kernel(const float *__restrict__ W, float *__restrict__ U, int IC, int OC)
+{
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;   // over (ic, oc), oc fastest
+    if (idx >= IC * OC) return;
+    const int ic = idx / OC, oc = idx - ic * OC;
+    float g[3][3];
+#pragma unroll
+    for (int i = 0; i < 3; i++)
+#pragma unroll
+        for (int j = 0; j < 3; j++) g[i][j] = W[((size_t)(oc * 3 + i) * 3 + j) * IC + ic];
+    float t[4][3];
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        t[0][j] = g[0][j];
+        t[1][j] = 0.5f * (g[0][j] + g[1][j] + g[2][j]);
+        t[2][j] = 0.5f * (g[0][j] - g[1][j] + g[2][j]);
+        t[3][j] = g[2][j];
+    }
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+        const float u0 = t[a][0], u1 = 0.5f * (t[a][0] + t[a][1] + t[a][2]), u2 = 0.5f * (t[a][0] - t[a][1] + t[a][2]), u3 = t[a][2];
+        U[((size_t)(4 * a + 0) * IC + ic) * OC + oc] = u0;
+        U[((size_t)(4 * a + 1) * IC + ic) * OC + oc] = u1;
+        U[((size_t)(4 * a + 2) * IC + ic) * OC + oc] = u2;
+        U[((size_t)(4 * a + 3) * IC + ic) * OC + oc] = u3;
+    }
+}
+
+__global__ __launch_bounds__(256, 2) void winograd_f2x2_kernel(const WinoArgs p)
+{
+    extern __shared__ __attribute__((aligned(16))) float smem[];   // V[2][WG_VBUF]; reused as output staging [128 px][68]
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = t >> 6;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int tile0 = blockIdx.x * WG_TILES;
+    const int oc0 = blockIdx.y * 64;
+    const int TC = p.TC, TRC = p.d_TRC.d;
+
+    floatx4 acc[16][2];
+#pragma unroll
+    for (int x = 0; x < 16; x++) {
+        acc[x][0] = floatx4{0.f, 0.f, 0.f, 0.f};
+        acc[x][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- input transform: thread t -> (tile t/8, channel pair t%8 of the 16-channel chunk); 16 float2 loads ----------
+    const int xt = t >> 3, xq = (t & 7) * 2;
+    int x_base = 0, x_ih0 = -(1 << 28), x_iw0 = 0;
+    {
+        const int tile = tile0 + xt;
+        if (tile < p.ntiles) {
+            const int n = fdiv(tile, p.d_TRC), rem = tile - n * TRC;
+            const int ty = fdiv(rem, p.d_TC), tx = rem - ty * TC;
+            x_base = n * p.IH * p.IW * p.IC;
+            x_ih0 = 2 * ty - p.ph;
+            x_iw0 = 2 * tx - p.pw;
+        }
+    }
+    float2 d[4][4];
+    unsigned dmask = 0;
+    auto load_patch = [&](int icc) {   // icc: first channel of the 16-channel chunk
+        dmask = 0;
+        const bool cv = icc + xq < p.IC;   // IC % 4 == 0: a channel pair is valid as a whole
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int ih = x_ih0 + i, iw = x_iw0 + j;
+                const bool ok = cv && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
+                const int off = (x_base + (ih * p.IW + iw) * p.IC + icc + xq) & -(int)ok;
+                d[i][j] = *reinterpret_cast<const float2 *>(p.X + off);
+                dmask |= (unsigned)ok << (4 * i + j);
+            }
+    };
+    auto transform_store = [&](int buf) {   // V = B^T d B, B^T = [[1,0,-1,0],[0,1,1,0],[0,-1,1,0],[0,1,0,-1]]
+        float *V = smem + buf * WG_VBUF + xt * 16 + xq;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const bool ok = (dmask >> (4 * i + j)) & 1u;
+                d[i][j] = make_float2(ok ? d[i][j].x : 0.f, ok ? d[i][j].y : 0.f);
+            }
+        auto sub = [](float2 a, float2 b) { return make_float2(a.x - b.x, a.y - b.y); };
+        auto add = [](float2 a, float2 b) { return make_float2(a.x + b.x, a.y + b.y); };
+        float2 r[4][4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            r[0][j] = sub(d[0][j], d[2][j]);
+            r[1][j] = add(d[1][j], d[2][j]);
+            r[2][j] = sub(d[2][j], d[1][j]);
+            r[3][j] = sub(d[1][j], d[3][j]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float2 v0 = sub(r[i][0], r[i][2]), v1 = add(r[i][1], r[i][2]), v2 = sub(r[i][2], r[i][1]), v3 = sub(r[i][1], r[i][3]);
+            *reinterpret_cast<float2 *>(V + (4 * i + 0) * WG_TILES * 16) = v0;
+            *reinterpret_cast<float2 *>(V + (4 * i + 1) * WG_TILES * 16) = v1;
+            *reinterpret_cast<float2 *>(V + (4 * i + 2) * WG_TILES * 16) = v2;
+            *reinterpret_cast<float2 *>(V + (4 * i + 3) * WG_TILES * 16) = v3;
+        }
+    };
+
+    // ---- transformed-filter fragments from L2: lane (l16, q) needs U[xi][icc + 4q + s][oc0 + 16w + l16] ------------
+    const int b_co = oc0 + 16 * w + l16;
+    const int b_col = b_co < p.OC ? b_co : 0;   // columns beyond OC are never stored
+    const int xi_stride = p.IC * p.OC;
+    auto load_b = [&](float (&b)[4], int xi, int icc) {
+        const int c = icc + 4 * q;
+        const int ok = -(int)(c < p.IC);
+#pragma unroll
+        for (int s = 0; s < 4; s++) b[s] = p.U[(xi * xi_stride + (c + s) * p.OC + b_col) & ok];
+    };
+
+    const int nchunks = (p.IC + 15) >> 4;
+    load_patch(0);
+    transform_store(0);
+    float bring[4][4];
+#pragma unroll
+    for (int x = 0; x < 4; x++) load_b(bring[x], x, 0);
+    __syncthreads();
+
+    for (int c = 0; c < nchunks; c++) {
+        const int buf = c & 1;
+        const bool more = c + 1 < nchunks;
+        if (more) load_patch((c + 1) * 16);
+        __builtin_amdgcn_sched_barrier(0);
+
+        const float *V = smem + buf * WG_VBUF + l16 * 16 + 4 * q;
+#pragma unroll
+        for (int xi = 0; xi < 16; xi++) {
+            const floatx4 a0 = *reinterpret_cast<const floatx4 *>(V + xi * WG_TILES * 16);
+            const floatx4 a1 = *reinterpret_cast<const floatx4 *>(V + xi * WG_TILES * 16 + 16 * 16);
+            float b[4];
+#pragma unroll
+            for (int s = 0; s < 4; s++) b[s] = bring[xi & 3][s];
+            // refill this ring slot with the fragment needed four positions later (possibly in the next chunk)
+            {
+                const int nx = xi + 4;
+                const int nxi = nx & 15, nicc = (nx < 16 ? c : c + 1) * 16;
+                load_b(bring[xi & 3], nxi, nicc < p.IC ? nicc : 0);
+            }
+            if (c * 16 + 4 * q >= p.IC) {
+#pragma unroll
+                for (int s = 0; s < 4; s++) b[s] = 0.f;   // ragged last chunk: channels beyond IC
+            }
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                acc[xi][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[s], b[s], acc[xi][0], 0, 0, 0);
+                acc[xi][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[s], b[s], acc[xi][1], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) transform_store(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- output transform in registers: Y = A^T M A, A^T = [[1,1,1,0],[0,1,-1,-1]]; then LDS-staged store ---------
+    float *Os = smem;   // [128 pixels: tile*4 + 2*dy + dx][68]
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float m[4][4];
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int b = 0; b < 4; b++) m[a][b] = acc[4 * a + b][mt][r];
+            float s0[4], s1[4];
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                s0[b] = m[0][b] + m[1][b] + m[2][b];
+                s1[b] = m[1][b] - m[2][b] - m[3][b];
+            }
+            const int tl = 16 * mt + 4 * q + r;   // tile within the workgroup
+            float *o = Os + (tl * 4) * 68 + 16 * w + l16;
+            o[0 * 68] = s0[0] + s0[1] + s0[2];
+            o[1 * 68] = s0[1] - s0[2] - s0[3];
+            o[2 * 68] = s1[0] + s1[1] + s1[2];
+            o[3 * 68] = s1[1] - s1[2] - s1[3];
+        }
+    __syncthreads();
+    for (int idx = t; idx < WG_TILES * 4 * 16; idx += 256) {
+        const int px = idx >> 4, cq = (idx & 15) * 4;
+        const int tl = px >> 2, dy = (px >> 1) & 1, dx = px & 1;
+        const int tile = tile0 + tl;
+        if (tile < p.ntiles && oc0 + cq < p.OC) {
+            const int n = fdiv(tile, p.d_TRC), rem = tile - n * TRC;
+            const int ty = fdiv(rem, p.d_TC), tx = rem - ty * TC;
+            const int oh = 2 * ty + dy, ow = 2 * tx + dx;
+            if (oh < p.OH && ow < p.OW)
+                *reinterpret_cast<float4 *>(p.Y + (((size_t)n * p.OH + oh) * p.OW + ow) * p.OC + oc0 + cq) =
+                    *reinterpret_cast<const float4 *>(Os + px * 68 + cq);
+        }
+    }
+}
+
+hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC)
+{
+    if (IC <= 0 || OC <= 0) return hipSuccess;
+    hipLaunchKernelGGL(winograd_filter_kernel, dim3((IC * OC + 255) / 256), dim3(256), 0, s, W, U, IC, OC);
+    return hipGetLastError();
+}
+
+hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
+                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw)
+{
+    if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
+    WinoArgs a{};
+    a.X = X; a.U = U; a.Y = Y;
+    a.N = N; a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC;
+    a.ph = ph; a.pw = pw;
+    a.TR = (OH + 1) / 2; a.TC = (OW + 1) / 2;
+    const long nt = (long)N * a.TR * a.TC;
+    if (nt >= (1L << 30) || 16L * IC * OC >= (1L << 31)) return hipErrorNotSupported;
+    a.ntiles = (int)nt;
+    a.d_TC = make_fastdiv(a.TC);
+    a.d_TRC = make_fastdiv(a.TR * a.TC);
+    size_t lds = (size_t)2 * WG_VBUF * sizeof(float);
+    const size_t stage = (size_t)WG_TILES * 4 * 68 * sizeof(float);
+    if (lds < stage) lds = stage;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(winograd_f2x2_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    dim3 grid((a.ntiles + WG_TILES - 1) / WG_TILES, (OC + 63) / 64);
+    hipLaunchKernelGGL(winograd_f2x2_kernel, grid, dim3(256), lds, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace alpha

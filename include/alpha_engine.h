@@ -31,6 +31,7 @@ typedef struct alpha_engine_config {
     int deltaX_ks_useTexture;     /* false */
     float deltaX_s1_V2_Q;         /* 1.1 */
     float deltaX_ks_V2_Q;         /* 1.1 */
+    int conv3D_winograd;          /* this build only (no reference flag): 1 = 3x3 stride-1 forward through Winograd F(2x2,3x3); default 0 */
 } alpha_engine_config;
 
 /* Native entry chosen by a plan; names are the Java native method names. */
@@ -42,7 +43,8 @@ enum alpha_entry {
     ALPHA_E_dconv3D_deltaX_ksIms2R, ALPHA_E_dconv3D_deltaX_ksIms2R_texture, ALPHA_E_dconv3D_deltaX_ksV2_Ims2R,
     ALPHA_E_dconv3D_deltaX_crossAdd,
     ALPHA_E_dconv3D_deltaW, ALPHA_E_dconv3D_deltaW_W1, ALPHA_E_dconv3D_deltaW_GemmSK, ALPHA_E_dconv3D_deltaW_GemmV2SK,
-    ALPHA_E_dconv3D_deltaW_GemmSK_W1
+    ALPHA_E_dconv3D_deltaW_GemmSK_W1,
+    ALPHA_E_conv3D_winograd   /* this build's additional forward algorithm; never chosen unless conv3D_winograd is set */
 };
 
 typedef struct alpha_conv_plan {

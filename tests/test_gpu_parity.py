@@ -176,6 +176,48 @@ def test_deltaX_lds_halo_kernel_vs_oracle(dev, shape):
     check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw), "lds-halo dX %s" % (shape,))
 
 
+WINO_SHAPES = [
+    # N, IH, IW, IC, OC, ph, pw   (3x3, stride 1)
+    (4, 56, 56, 64, 64, 1, 1),
+    (8, 28, 28, 128, 128, 1, 1),
+    (16, 14, 14, 256, 256, 1, 1),
+    (36, 7, 7, 512, 512, 1, 1),      # odd output size: partial tiles on the right / bottom
+    (4, 13, 11, 36, 44, 1, 1),       # ragged channels, odd sizes
+    (4, 10, 12, 16, 32, 0, 0),       # no padding
+    (4, 6, 9, 32, 64, 2, 2),         # padding 2
+    (3, 5, 5, 64, 64, 1, 1),         # fewer tiles than one workgroup
+    (4, 32, 32, 4, 64, 1, 1),        # BASELINE config 1 geometry (IC = 3 stored as 4)
+]
+
+
+@pytest.mark.parametrize("shape", WINO_SHAPES)
+def test_forward_winograd_f2x2_vs_direct_oracle(dev, shape):
+    """Winograd F(2x2,3x3) against the same fp64 direct convolution; tolerance as for the direct kernels
+    (rel 1e-4, abs floor 1e-5 * max(1, rms)): the transforms only add a few ulps on unit-scale data."""
+    N, IH, IW, IC, OC, ph, pw = shape
+    OH, OW = out_dim(IH, IW, 3, 3, 1, 1, ph, pw)
+    X, W = normal((N, IH, IW, IC), 1201), he_normal(OC, 3, 3, IC, 1202)
+    x, w = dev.put(X), dev.put(W)
+    U = dev.empty(C3.winograd_filter_size(IC, OC), fill=float("nan"))
+    y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    C3.winograd_filter_transform(dev.stream, w.data_ptr(), U.data_ptr(), IC, OC)
+    C3.conv3D_winograd(dev.streams, 1, x.data_ptr(), IH, IW, U.data_ptr(), y.data_ptr(), OH, OW, N, IC, OC, ph, pw)
+    check(dev.get(y), O.conv3D_f64(X, W, 1, 1, ph, pw), "winograd %s" % (shape,))
+
+
+def test_winograd_filter_transform_matches_G_g_Gt(dev):
+    IC, OC = 8, 12
+    W = he_normal(OC, 3, 3, IC, 1203)
+    w = dev.put(W)
+    U = dev.empty(16 * IC * OC, fill=float("nan"))
+    C3.winograd_filter_transform(dev.stream, w.data_ptr(), U.data_ptr(), IC, OC)
+    G = np.array([[1, 0, 0], [.5, .5, .5], [.5, -.5, .5], [0, 0, 1]], np.float64)
+    g = W.astype(np.float64).transpose(0, 3, 1, 2)              # [oc][ic][3][3]
+    want = np.einsum("ai,ocij,bj->aboc", G, g, G)               # [4][4][oc][ic] -> U[xi][ic][oc]
+    want = want.transpose(0, 1, 3, 2).reshape(16, IC, OC)
+    np.testing.assert_allclose(dev.get(U).reshape(16, IC, OC), want, rtol=1e-6, atol=1e-7)
+
+
 def test_forward_oc_sweep_covers_every_ragged_width(dev):
     # the reference's "for OC from 1 to 128: correct" sweep (Cuda_conv3D_test.java:155-156), in steps of 4
     X = uniform((4, 9, 9, 8), 1009)
@@ -363,6 +405,59 @@ def test_deltaW_split_k_slices_follow_the_reference_partition(dev):
     parts = [dev.get(dWo)] + [b.reshape(OC, F_, F_, IC) for b in dev.get(buf)]
     for z in range(GridZ):
         check(parts[z], O.deltaW_slice_f64(X, dY, F_, F_, s, s, p, p, GridZ, z), "slice %d" % z, sp_min=0.99)
+
+
+DW_ROWS_SHAPES = [
+    # stride-1 layers served by the row-streaming kernel: N, IH, IW, IC, OC, F, p, GridZ
+    (4, 56, 56, 64, 64, 3, 1, 16),     # c5b geometry
+    (8, 32, 32, 64, 64, 3, 1, 8),      # c2a geometry
+    (16, 16, 16, 128, 128, 3, 1, 7),   # c2b: slices end inside rows and inside images
+    (32, 8, 8, 256, 256, 3, 1, 3),     # c2c with the split-K factor the Java engine would pass
+    (4, 9, 9, 16, 16, 3, 1, 5),        # GK = 324, slices of 64 pixels: boundaries in the middle of rows
+    (4, 13, 11, 36, 44, 3, 1, 3),      # ragged channel counts, OW not a multiple of 4
+    (4, 10, 12, 32, 48, 3, 0, 2),      # no padding
+    (4, 6, 7, 64, 32, 3, 2, 2),        # padding 2
+    (8, 56, 56, 256, 64, 1, 0, 16),    # c5a geometry (1x1)
+    (8, 56, 56, 64, 256, 1, 0, 16),    # c5c geometry (1x1)
+    (4, 7, 9, 20, 36, 1, 0, 2),        # 1x1 ragged
+]
+
+
+@pytest.mark.parametrize("shape", DW_ROWS_SHAPES)
+def test_deltaW_row_streaming_kernel_slices_and_sum(dev, shape):
+    N, IH, IW, IC, OC, F_, p, GridZ = shape
+    OH, OW = out_dim(IH, IW, F_, F_, 1, 1, p, p)
+    X, dY = normal((N, IH, IW, IC), 3101), normal((N, OH, OW, OC), 3102)
+    x, dy = dev.put(X), dev.put(dY)
+    sizeW = OC * F_ * F_ * IC
+    outs = {}
+    L = pkg.lib()
+    try:
+        for algo in (0, 3):   # 0: row-streaming kernel where eligible, 3: generic kernel
+            L.alpha_conv_set_fwd_algo(algo)
+            dWo = dev.empty(OC, F_, F_, IC, fill=float("nan"))
+            buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+            if F_ == 1:
+                DW.dconv3D_deltaW_GemmSK_W1(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), buf.data_ptr(),
+                                            N, IC, OC)
+            else:
+                DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(),
+                                         buf.data_ptr(), F_, F_, N, IC, OC, 1, 1, p, p)
+            outs[algo] = [dev.get(dWo)] + [b.reshape(OC, F_, F_, IC) for b in dev.get(buf)]
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+    total = np.zeros((OC, F_, F_, IC))
+    for z in range(GridZ):
+        want = O.deltaW_slice_f64(X, dY, F_, F_, 1, 1, p, p, GridZ, z)
+        total += want
+        floor = tolerance_floor(total if z else want)
+        for algo in (0, 3):
+            r = O.max_err_ratio(outs[algo][z], want, REL, max(floor, tolerance_floor(want)))
+            assert r <= 1.0, "slice %d algo %d %s: err/allowed %.3f" % (z, algo, shape, r)
+    dWs = dev.put(outs[0][0])
+    bufs = dev.put(np.stack([o.reshape(-1) for o in outs[0][1:]]))
+    DW.buf_summary(dev.stream, bufs.data_ptr(), dWs.data_ptr(), GridZ - 1, sizeW)
+    check(dev.get(dWs), O.deltaW_f64(X, dY, F_, F_, 1, 1, p, p), "row-streaming dW total %s" % (shape,))
 
 
 def test_deltaW_W1_entries(dev):
