@@ -1,0 +1,118 @@
+"""GPU: every layer of BASELINE.json's five configs at FULL size, through the C++ host layer.
+
+The CPU oracle cannot finish these sizes in seconds, so each layer is checked by
+  (1) the oracle on a few whole images of the batch (a convolution treats images independently, so image n of the
+      full-batch result must equal the oracle's result for image n alone) — forward (implicit GEMM and Winograd) and
+      backward-data;
+  (2) the adjoint identity  <conv(X,W), dY> = <X, deltaX(dY,W)> = <W, deltaW(X,dY)>  evaluated in fp64 on the device,
+      which ties the full-size backward-filter (a sum over the whole batch) to the forward result;
+  (3) for config 5: backward-filter twice, bit-identical.
+Tolerance: rel 1e-4 with abs floor 1e-5 * max(1, rms(expected)) for (1); 2e-5 relative for the inner products of (2).
+"""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from util import Dev, load_package, out_dim
+
+pytestmark = pytest.mark.gpu
+pkg = load_package()
+
+# id: N, IH, IW, IC(stored), OC, F, s, p, logical IC, input distribution
+LAYERS = {
+    "c1": (4, 32, 32, 4, 64, 3, 1, 1, 3, "uniform"),
+    "c2a": (128, 32, 32, 64, 64, 3, 1, 1, 64, "normal"),
+    "c2b": (128, 16, 16, 128, 128, 3, 1, 1, 128, "normal"),
+    "c2c": (128, 8, 8, 256, 256, 3, 1, 1, 256, "normal"),
+    "c3a": (64, 56, 56, 64, 64, 3, 1, 1, 64, "normal"),
+    "c3b": (64, 28, 28, 128, 128, 3, 1, 1, 128, "normal"),
+    "c3c": (64, 14, 14, 256, 256, 3, 1, 1, 256, "normal"),
+    "c3d": (64, 7, 7, 512, 512, 3, 1, 1, 512, "normal"),
+    "c4a": (64, 224, 224, 4, 64, 7, 2, 3, 3, "uniform"),
+    "c4b": (64, 56, 56, 64, 128, 3, 2, 1, 64, "uniform"),
+    "c4c": (64, 56, 56, 64, 128, 1, 2, 0, 64, "uniform"),
+    "c4d": (64, 14, 14, 256, 1024, 1, 1, 0, 256, "uniform"),
+    "c5a": (32, 56, 56, 256, 64, 1, 1, 0, 256, "normal"),
+    "c5b": (32, 56, 56, 64, 64, 3, 1, 1, 64, "normal"),
+    "c5c": (32, 56, 56, 64, 256, 1, 1, 0, 64, "normal"),
+}
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return Dev()
+
+
+def _tensors(dev, layer, seed):
+    torch = dev.torch
+    N, IH, IW, IC, OC, F, s, p, ICl, dist = LAYERS[layer]
+    OH, OW = out_dim(IH, IW, F, F, s, s, p, p)
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    X = torch.randn((N, IH, IW, IC), generator=g) if dist == "normal" else torch.rand((N, IH, IW, IC), generator=g) * 2 - 1
+    W = torch.randn((OC, F, F, IC), generator=g) * float(np.sqrt(2.0 / (F * F * ICl)))   # He-normal
+    if ICl < IC:
+        X[..., ICl:] = 0
+        W[..., ICl:] = 0
+    dY = torch.randn((N, OH, OW, OC), generator=g)
+    return X, W, dY, OH, OW
+
+
+def _check(got, want, what):
+    floor = 1e-5 * max(1.0, float(np.sqrt(np.mean(want * want))))
+    r = O.max_err_ratio(np.ascontiguousarray(got), want, 1e-4, floor)
+    assert r <= 1.0, "%s: err/allowed = %.3f (rel 1e-4, abs floor %.3g)" % (what, r, floor)
+
+
+@pytest.mark.parametrize("layer", sorted(LAYERS))
+def test_full_size_layer(dev, layer):
+    torch = dev.torch
+    N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[layer]
+    X, W, dY, OH, OW = _tensors(dev, layer, 7000 + sorted(LAYERS).index(layer))
+    x, w, dy = X.to(dev.dev), W.to(dev.dev), dY.to(dev.dev)
+    y = torch.full((N, OH, OW, OC), float("nan"), device=dev.dev)
+    dx = torch.full((N, IH, IW, IC), float("nan"), device=dev.dev)
+    dw = torch.full((OC, F, F, IC), float("nan"), device=dev.dev)
+    eng = pkg.engine.Engine(dev.stream)
+    try:
+        eng.conv3D(y.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), F, F, N, IC, OC, s, s, p, p)
+        eng.dconv3D_deltaX(dx.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), F, F, N, IC, OC, s, s, p, p)
+        eng.dconv3D_deltaW(dw.data_ptr(), F, F, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, s, s, p, p)
+        eng.sync()
+        yw = None
+        if F == 3 and s == 1 and IC >= 16:
+            yw = torch.full((N, OH, OW, OC), float("nan"), device=dev.dev)
+            eng.config.conv3D_winograd = 1
+            plan = eng.conv3D(yw.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), F, F, N, IC, OC, s, s, p, p)
+            eng.config.conv3D_winograd = 0
+            eng.sync()
+            assert plan.entry_name == "conv3D_winograd"
+        dw2 = None
+        if layer.startswith("c5"):
+            dw2 = torch.full((OC, F, F, IC), float("nan"), device=dev.dev)
+            eng.dconv3D_deltaW(dw2.data_ptr(), F, F, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, s, s, p, p)
+            eng.sync()
+    finally:
+        eng.close()
+
+    # (1) whole images against the oracle
+    Xn, Wn, dYn = X.numpy(), W.numpy(), dY.numpy()
+    for n in sorted({0, N // 2, N - 1}):
+        want = O.conv3D_f64(np.ascontiguousarray(Xn[n:n + 1]), Wn, s, s, p, p)
+        _check(y[n:n + 1].cpu().numpy(), want, "%s forward image %d" % (layer, n))
+        if yw is not None:
+            _check(yw[n:n + 1].cpu().numpy(), want, "%s Winograd forward image %d" % (layer, n))
+        wantx = O.deltaX_f64(np.ascontiguousarray(dYn[n:n + 1]), Wn, IH, IW, s, s, p, p)
+        _check(dx[n:n + 1].cpu().numpy(), wantx, "%s deltaX image %d" % (layer, n))
+
+    # (2) adjointness in fp64 on the device
+    a = float((y.double() * dy.double()).sum())
+    b = float((x.double() * dx.double()).sum())
+    c = float((w.double() * dw.double()).sum())
+    scale = float((y.double().abs() * dy.double().abs()).sum())   # size of the terms being summed
+    assert abs(a - b) <= 2e-5 * scale, "%s: <Y,dY> = %r vs <X,dX> = %r" % (layer, a, b)
+    assert abs(a - c) <= 2e-5 * scale, "%s: <Y,dY> = %r vs <W,dW> = %r" % (layer, a, c)
+    assert bool(torch.isfinite(dw).all()) and bool(torch.isfinite(dx).all())
+
+    # (3) run-to-run bit reproducibility of backward-filter (config 5)
+    if dw2 is not None:
+        assert torch.equal(dw, dw2), "%s: deltaW differs between two runs" % layer
