@@ -305,6 +305,13 @@ def main():
                               "fp32_mfma_peak_from_device_tflops": round(cus * 256 * clk_ghz / 1e3, 1)}},
         "roofline": head["roofline"],
     }
+    if op == "fwd" and F == 3 and s == 1 and IC >= 16:
+        # the same layer through this build's second forward algorithm, in direct-convolution-equivalent FLOPs
+        wn = measure(pkg, torch, args.layer, "wino", args.steps, args.warmup)
+        out["winograd"] = {"value": wn["tflops"], "unit": "TFLOP/s (direct-conv-equivalent)", "ms_per_step": wn["ms_per_step"],
+                           "kernel_ms": wn["roofline"]["kernel_ms"], "kernel_tflops": wn["roofline"]["achieved"],
+                           "frac_of_fp32_mfma_peak": wn["roofline"]["frac"],
+                           "note": "Winograd F(2x2,3x3): 2.25x fewer multiplies than the FLOP count credited"}
     if args.layers:
         out["layers"] = []
         for layer in sorted(LAYERS):

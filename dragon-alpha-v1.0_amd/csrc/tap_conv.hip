@@ -262,7 +262,7 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
                            int b_off, int b_sth, int b_stw, int b_sc)
 {
     if (OH != AH + 2 * ph - TH + 1 || OW != AW + 2 * pw - TW + 1) return hipErrorNotSupported;
-    if (AC < 32 || TH * TW < 2 || TH > 7 || TW > 7) return hipErrorNotSupported;
+    if (AC < 32 || TH > 7 || TW > 7) return hipErrorNotSupported;
     const long M = (long)N * OH * OW;
     if ((long)N * (AH + 2 * ph) >= (1L << 24)) return hipErrorNotSupported;
 
