@@ -66,7 +66,7 @@ def algorithmic_bytes(layer):
 class Workload:
     """Device tensors of one layer plus closures that enqueue each operator the way the Java engine does."""
 
-    def __init__(self, pkg, torch, layer, seed):
+    def __init__(self, pkg, torch, layer, seed, fill_units=False):
         self.pkg, self.torch, self.layer = pkg, torch, layer
         N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[layer]
         self.dims = (N, IH, IW, IC, OC, F, s, p)
@@ -88,6 +88,10 @@ class Workload:
         self.stream = int(torch.cuda.current_stream().cuda_stream)
         self.streams = [self.stream]
         self.engine = pkg.engine.Engine(self.stream)
+        if fill_units:
+            # this build's option: raise the split-K factor until the launch fills the device (the reference's GridZ
+            # is sized for at most 128 SMs)
+            self.engine.config.deltaW_SK_fillUnits = pkg.device_info()[0]
         # split-K factor for the kernel-only timing: what the host layer would pass (CudaFloat32EngineBase.java:1707-1715)
         self.GridZ = max(1, pkg.engine.plan_deltaW(self.engine.config, IH, IW, OH, OW, F, F, N, IC, OC, s, s).GridZ)
         self.buf = torch.empty(max(1, self.GridZ - 1) * self.dW.numel(), device=dev)
@@ -220,9 +224,9 @@ def load_traffic(layer, op):
 
 
 def measure(pkg, torch, layer, op, steps, warmup):
-    wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer))
-    step = {"fwd": wl.fwd, "dx": wl.dx_op, "dw": wl.dw, "wino": wl.wino}[op]
-    kernel = {"fwd": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "wino": wl.wino_conv}[op]
+    wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer), fill_units=(op == "dw_fill"))
+    step = {"fwd": wl.fwd, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino}[op]
+    kernel = {"fwd": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm, "wino": wl.wino_conv}[op]
     if op == "fwd":
         wl.fwd_remode()
     if op == "wino":
@@ -248,7 +252,7 @@ def measure(pkg, torch, layer, op, steps, warmup):
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     return {"layer": layer, "op": op, "ms_per_step": round(wall_ms, 5), "event_ms_per_step": round(ev_ms, 5),
             "tflops": round(fl / (wall_ms * 1e-3) / 1e12, 3), "gflop": round(fl / 1e9, 3),
-            "algorithmic_MB": round(by / 1e6, 2), "GridZ": gridz if op == "dw" else None, "roofline": roof}
+            "algorithmic_MB": round(by / 1e6, 2), "GridZ": gridz if op in ("dw", "dw_fill") else None, "roofline": roof}
 
 
 def main():
@@ -257,7 +261,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
-    ap.add_argument("--op", default=None, choices=["fwd", "dx", "dw", "wino"],
+    ap.add_argument("--op", default=None, choices=["fwd", "dx", "dw", "dw_fill", "wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="also measure every layer/op of BASELINE.json's configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -318,6 +322,8 @@ def main():
             ops = list(LAYERS[layer][9])
             if "fwd" in ops and LAYERS[layer][5] == 3 and LAYERS[layer][6] == 1 and LAYERS[layer][3] >= 16:
                 ops.append("wino")
+            if "dw" in ops:
+                ops.append("dw_fill")
             for o in ops:
                 out["layers"].append(measure(pkg, torch, layer, o, max(5, args.steps // 5), max(2, args.warmup // 3)))
                 torch.cuda.empty_cache()

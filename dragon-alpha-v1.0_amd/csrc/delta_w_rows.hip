@@ -13,8 +13,14 @@
 // Pixels outside the K slice (a slice may begin or end inside a row) are staged as zeros. No atomics: slice z
 // stores to deltaW (z = 0) or deltaW_buf[z-1]; a fixed launch gives bit-identical results.
 //
+// Narrow images: R output rows ("a chunk") are multiplied per step so that a step always has up to 64 pixels of
+// work; the ring then holds 2R + FH - 1 input rows and R new ones are fetched per step.
+//
 // LDS strides: 32-bit reads of 64 lanes are conflict-free when the four 16-lane groups (consecutive pixels) start
-// 16 banks apart: row strides are 16 or 48 floats modulo 64 (X: 80; deltaY: 48 for 32 channels, 80 for 64).
+// 16 banks apart: pixel strides are 16 or 48 floats modulo 64 (X: 80; deltaY: 48 for 32 channels, 80 for 64); with
+// 16 channels the deltaY stride is 32 (two groups share banks: a 2-way conflict on 1 of 10 reads). An unpadded,
+// XOR-permuted layout (74 KB instead of 96 KB for 56-pixel rows, so two workgroups per compute unit) was measured
+// slower: its per-tap lane offsets cost more address arithmetic and LDS instructions than the co-residency gains.
 #include "common.hpp"
 
 namespace alpha {
@@ -27,9 +33,13 @@ struct DwRowsArgs {
     int N, IH, IW, IC, OH, OW, OC;
     int ph, pw;
     int GK, GK_slice, GZ;
-    int OWp;   // OW rounded up to a multiple of 4 (pixels beyond OW are staged as zeros)
-    int PW;    // OWp + FW - 1 input columns staged per row; staged column cp holds iw = cp - pw
-    FastDiv d_OW, d_OH;
+    int OWp;     // OW rounded up to a multiple of 4 (pixels beyond OW are staged as zeros)
+    int PW;      // OWp + FW - 1 input columns staged per row; staged column cp holds iw = cp - pw
+    int R;       // output rows multiplied per step (a "chunk"); R*OWp <= 64 and R*PW <= 64
+    int CPI;     // chunks per image = ceil(OH / R)
+    int SLOTS;   // input-row slots in LDS = 2R + FH - 1
+    int steps2;  // groups of 4 pixels per chunk, rounded up to an even count (the deltaY pixels added are zeros)
+    FastDiv d_OW, d_OH, d_OWp, d_PW, d_R, d_SLOTS;
 };
 
 constexpr int DWR_XS = 80;   // X row slot pixel stride (floats): 64 channels + 16
@@ -38,15 +48,15 @@ template <int FH, int FW, int OCT>
 __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p)
 {
     constexpr int OCB = 16 * OCT;
-    constexpr int YS = OCB + 16;             // 48 or 80: both 16 or 48 modulo 64
-    constexpr int YQ = OCT;                  // float4 per thread per deltaY row   (OWp <= 64, host-checked)
-    constexpr int XQ = 4;                    // float4 per thread per X row        (PW*16 <= 1024, host-checked)
-    constexpr int SLOTS = FH + 1;
+    constexpr int YS = OCB + 16;             // deltaY pixel stride (floats): 32, 48 or 80
+    constexpr int YQ = OCT;                  // float4 per thread per deltaY chunk (R*OWp <= 64, host-checked)
+    constexpr int XQ = 4;                    // float4 per thread per R new X rows  (R*PW <= 64, host-checked)
 
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *Ybuf = smem;                               // [2][OWp][YS]
-    float *Xring = smem + 2 * p.OWp * YS;             // [SLOTS][PW][DWR_XS]
-    const int ybuf_floats = p.OWp * YS, slot_floats = p.PW * DWR_XS;
+    const int R = p.R, OWp = p.OWp, PW = p.PW, SLOTS = p.SLOTS;
+    const int ybuf_floats = p.steps2 * 4 * YS, slot_floats = PW * DWR_XS;
+    float *Ybuf = smem;                               // [2][R*OWp][YS]
+    float *Xring = smem + 2 * ybuf_floats;            // [SLOTS][PW][DWR_XS]
 
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
@@ -69,16 +79,19 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
     // ---- staging helpers (loads from clamped addresses, zeroing applied when the registers are stored) ----------
     float4 yreg[YQ], xreg[XQ];
     unsigned ymask = 0, xmask = 0;
-    const int y_quads = p.OWp * (OCB / 4), x_quads = p.PW * 16;
+    const int y_quads = p.steps2 * 4 * (OCB / 4);   // includes the zero pixels that pad the chunk to an even step count
 
-    auto load_y = [&](int gr) {   // deltaY row gr (global output row n*OH + oh)
+    // deltaY rows oh0 .. oh0+R-1 of image n; chunk pixel (rr, ow) lives at LDS pixel index rr*OWp + ow
+    auto load_y = [&](int n, int oh0) {
         ymask = 0;
 #pragma unroll
         for (int u = 0; u < YQ; u++) {
             const int idx = t + 256 * u;
-            const int ow = idx / (OCB / 4), cq = (idx % (OCB / 4)) * 4;
-            const int k = gr * OW + ow;
-            const bool ok = idx < y_quads && ow < OW && k >= k_start && k < k_end && oc0 + cq < p.OC;
+            const int px = idx / (OCB / 4), cq = (idx % (OCB / 4)) * 4;
+            const int rr = fdiv(px, p.d_OWp), ow = px - rr * OWp;
+            const int oh = oh0 + rr;
+            const int k = (n * OH + oh) * OW + ow;
+            const bool ok = idx < y_quads && rr < R && ow < OW && oh < OH && k >= k_start && k < k_end && oc0 + cq < p.OC;
             yreg[u] = *reinterpret_cast<const float4 *>(p.dY + (((size_t)k * p.OC + oc0 + cq) & (size_t)(-(long)ok)));
             ymask |= (unsigned)ok << u;
         }
@@ -88,80 +101,131 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
         for (int u = 0; u < YQ; u++) {
             const int idx = t + 256 * u;
             if (idx < y_quads) {
-                const int ow = idx / (OCB / 4), cq = (idx % (OCB / 4)) * 4;
+                const int px = idx / (OCB / 4), cq = (idx % (OCB / 4)) * 4;
                 const bool ok = (ymask >> u) & 1u;
-                *reinterpret_cast<float4 *>(Ybuf + buf * ybuf_floats + ow * YS + cq) =
+                *reinterpret_cast<float4 *>(Ybuf + buf * ybuf_floats + px * YS + cq) =
                     make_float4(ok ? yreg[u].x : 0.f, ok ? yreg[u].y : 0.f, ok ? yreg[u].z : 0.f, ok ? yreg[u].w : 0.f);
             }
         }
     };
-    auto load_x = [&](int n, int ih) {   // input row (n, ih); rows outside the image become zeros
+    // `nrows` (<= R) padded input rows rp0 .. rp0+nrows-1 of image n (padded row rp holds ih = rp - ph; rows outside
+    // the image become zeros); padded row rp lives in slot rp % SLOTS
+    auto load_x = [&](int n, int rp0, int nrows) {
         xmask = 0;
-        const bool rowv = (unsigned)ih < (unsigned)p.IH;
+        const int quads = nrows * PW * 16;
 #pragma unroll
         for (int u = 0; u < XQ; u++) {
             const int idx = t + 256 * u;
-            const int cp = idx >> 4, cq = (idx & 15) * 4;
-            const int iw = cp - p.pw;
-            const bool ok = rowv && idx < x_quads && (unsigned)iw < (unsigned)p.IW && ic0 + cq < p.IC;
+            const int px = idx >> 4, cq = (idx & 15) * 4;
+            const int rr = fdiv(px, p.d_PW), cp = px - rr * PW;
+            const int ih = rp0 + rr - p.ph, iw = cp - p.pw;
+            const bool ok = idx < quads && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW && ic0 + cq < p.IC;
             const int off = (((n * p.IH + ih) * p.IW + iw) * p.IC + ic0 + cq) & -(int)ok;
             xreg[u] = *reinterpret_cast<const float4 *>(p.X + off);
             xmask |= (unsigned)ok << u;
         }
     };
-    auto store_x = [&](int slot) {
+    auto store_x = [&](int rp0, int nrows) {
+        const int quads = nrows * PW * 16;
 #pragma unroll
         for (int u = 0; u < XQ; u++) {
             const int idx = t + 256 * u;
-            if (idx < x_quads) {
+            if (idx < quads) {
+                const int px = idx >> 4;
+                const int rr = fdiv(px, p.d_PW), cp = px - rr * PW;
+                const int rp = rp0 + rr;
+                const int slot = rp - fdiv(rp, p.d_SLOTS) * SLOTS;
                 const bool ok = (xmask >> u) & 1u;
-                *reinterpret_cast<float4 *>(Xring + slot * slot_floats + (idx >> 4) * DWR_XS + (idx & 15) * 4) =
+                *reinterpret_cast<float4 *>(Xring + slot * slot_floats + cp * DWR_XS + (idx & 15) * 4) =
                     make_float4(ok ? xreg[u].x : 0.f, ok ? xreg[u].y : 0.f, ok ? xreg[u].z : 0.f, ok ? xreg[u].w : 0.f);
             }
         }
     };
-    // all FH input rows of output row (n, oh), fetched synchronously (first row of the slice / of an image)
-    auto stage_window = [&](int n, int oh) {
+    // the whole window of chunk (n, oh0): padded rows oh0 .. oh0+R+FH-2 in up to FH pieces of R rows, all fetched
+    // before the first is stored so that their latencies overlap
+    auto stage_window = [&](int n, int oh0) {
+        float4 wreg[FH][XQ];
+        unsigned wmask[FH];
 #pragma unroll
-        for (int fh = 0; fh < FH; fh++) {
-            load_x(n, oh - p.ph + fh);
-            store_x((oh + fh) % SLOTS);
+        for (int pc = 0; pc < FH; pc++) {
+            const int nrows = min(R, R + FH - 1 - pc * R);     // <= 0: nothing left for this piece
+            load_x(n, oh0 + pc * R, nrows);
+#pragma unroll
+            for (int u = 0; u < XQ; u++) wreg[pc][u] = xreg[u];
+            wmask[pc] = xmask;
+        }
+#pragma unroll
+        for (int pc = 0; pc < FH; pc++) {
+            const int nrows = min(R, R + FH - 1 - pc * R);
+#pragma unroll
+            for (int u = 0; u < XQ; u++) xreg[u] = wreg[pc][u];
+            xmask = wmask[pc];
+            store_x(oh0 + pc * R, nrows);
         }
     };
 
     if (k_start < k_end) {
         const int gr_first = fdiv(k_start, p.d_OW), gr_last = fdiv(k_end - 1, p.d_OW);
-        int n = fdiv(gr_first, p.d_OH), oh = gr_first - n * OH;
-        load_y(gr_first);
+        int n = fdiv(gr_first, p.d_OH);
+        int ci = fdiv(gr_first - n * OH, p.d_R);                      // chunk within the image
+        const int n_last = fdiv(gr_last, p.d_OH);
+        const int ci_last = fdiv(gr_last - n_last * OH, p.d_R);
+        load_y(n, ci * R);
         store_y(0);
-        stage_window(n, oh);
+        stage_window(n, ci * R);
         __syncthreads();
 
-        const int steps = p.OWp >> 2;
-        for (int gr = gr_first, it = 0; gr <= gr_last; gr++, it++) {
-            const bool has_next = gr < gr_last;
-            int n2 = n, oh2 = oh + 1;
-            if (oh2 == OH) { oh2 = 0; n2 = n + 1; }
+        const int steps2 = p.steps2;
+        for (int it = 0;; it++) {
+            const int oh0 = ci * R;
+            const bool has_next = n < n_last || ci < ci_last;
+            int n2 = n, ci2 = ci + 1;
+            if (ci2 == p.CPI) { ci2 = 0; n2 = n + 1; }
             const bool same_image = n2 == n;
             if (has_next) {
-                load_y(gr + 1);
-                if (same_image) load_x(n, oh2 - p.ph + FH - 1);
+                load_y(n2, ci2 * R);
+                if (same_image) load_x(n, oh0 + R + FH - 1, R);   // the R new padded rows of the next chunk
             }
 
-            // ---- multiply this row: pixels in groups of 4 (lane group q takes pixel 4*k4 + q) ---------------------
+            // ---- multiply this chunk: pixels in groups of 4 (lane group q takes pixel 4*k4 + q of the chunk) --------
             const float *yb = Ybuf + (it & 1) * ybuf_floats + q * YS + l16;
-            const float *xb[FH];
+            const float *xb = Xring + q * DWR_XS + 16 * w + l16;
+            const int s0 = oh0 - fdiv(oh0, p.d_SLOTS) * SLOTS;           // ring slot of the chunk's first padded row
+
+            // Read position of the next step, kept in scalar registers: deltaY advances 4 pixels per step; the input
+            // position advances 4 columns and, at the end of an output row, one ring slot. Steps that pad the chunk
+            // to an even count (their deltaY pixels are zeros) and the read-ahead past the last step stay on the
+            // last real input position, so that nothing uninitialised is ever multiplied.
+            int yo = 0, col = 0, px = 0, xo[FH], nslot = s0 + FH;
+            nslot -= nslot >= SLOTS ? SLOTS : 0;
 #pragma unroll
-            for (int fh = 0; fh < FH; fh++) xb[fh] = Xring + ((oh + fh) % SLOTS) * slot_floats + q * DWR_XS + 16 * w + l16;
+            for (int fh = 0; fh < FH; fh++) {
+                int slot = s0 + fh;
+                slot -= slot >= SLOTS ? SLOTS : 0;
+                xo[fh] = slot * slot_floats;
+            }
+            const int px_last = R * OWp - 4;
 
             float a0[OCT], b0[FH][FW], a1[OCT], b1[FH][FW];
-            auto frags = [&](int k4, float (&a)[OCT], float (&b)[FH][FW]) {
+            auto frags = [&](float (&a)[OCT], float (&b)[FH][FW]) {
 #pragma unroll
-                for (int c = 0; c < OCT; c++) a[c] = yb[k4 * 4 * YS + 16 * c];
+                for (int c = 0; c < OCT; c++) a[c] = yb[yo + 16 * c];
 #pragma unroll
-                for (int fh = 0; fh < FH; fh++)
+                for (int fh = 0; fh < FH; fh++) {
+                    const float *xr = xb + xo[fh] + col * DWR_XS;
 #pragma unroll
-                    for (int fw = 0; fw < FW; fw++) b[fh][fw] = xb[fh][(k4 * 4 + fw) * DWR_XS];
+                    for (int fw = 0; fw < FW; fw++) b[fh][fw] = xr[fw * DWR_XS];
+                }
+                yo += 4 * YS;
+                const bool move = px < px_last;
+                const bool wrap = move && col + 4 == OWp;
+                px += 4;
+                col = wrap ? 0 : (move ? col + 4 : col);
+#pragma unroll
+                for (int fh = 0; fh + 1 < FH; fh++) xo[fh] = wrap ? xo[fh + 1] : xo[fh];
+                xo[FH - 1] = wrap ? nslot * slot_floats : xo[FH - 1];
+                const int ns = nslot + 1 == SLOTS ? 0 : nslot + 1;
+                nslot = wrap ? ns : nslot;
             };
             auto mfmas = [&](const float (&a)[OCT], const float (&b)[FH][FW]) {
 #pragma unroll
@@ -172,27 +236,40 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
                         for (int c = 0; c < OCT; c++)
                             acc[fh][fw][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[c], b[fh][fw], acc[fh][fw][c], 0, 0, 0);
             };
-            frags(0, a0, b0);
-            for (int k4 = 0; k4 < steps; k4 += 2) {
-                if (k4 + 1 < steps) frags(k4 + 1, a1, b1);
-                mfmas(a0, b0);
-                if (k4 + 1 < steps) {
-                    if (k4 + 2 < steps) frags(k4 + 2, a0, b0);
-                    mfmas(a1, b1);
+            // One step = FH*FW*OCT MFMAs on the fragments read during the previous step, with the reads and address
+            // arithmetic of the next step spread between them (a wave has the SIMD to itself, so whatever is not
+            // issued in the shadow of an MFMA is lost time). Reads are unconditional: a branch around them would turn
+            // the wait before the MFMAs into a wait for everything.
+            auto interleave = [&]() {
+#pragma unroll
+                for (int g = 0; g < FH + 1; g++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x006, 4, 0);   // up to 4 VALU / SALU
+                    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);   // up to 3 LDS reads
                 }
+            };
+            frags(a0, b0);
+            for (int k4 = 0; k4 < steps2; k4 += 2) {
+                __builtin_amdgcn_sched_barrier(0);
+                frags(a1, b1);
+                mfmas(a0, b0);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+                frags(a0, b0);
+                mfmas(a1, b1);
+                interleave();
             }
 
-            if (has_next) {
-                store_y((it + 1) & 1);
-                if (same_image) store_x((oh2 + FH - 1) % SLOTS);
-            }
+            if (!has_next) break;
+            store_y((it + 1) & 1);
+            if (same_image) store_x(oh0 + R + FH - 1, R);
             __syncthreads();
-            if (has_next && !same_image) {   // first row of the next image: its whole window is new
-                stage_window(n2, oh2);
+            if (!same_image) {   // first chunk of the next image: its whole window is new
+                stage_window(n2, 0);
                 __syncthreads();
             }
             n = n2;
-            oh = oh2;
+            ci = ci2;
         }
     }
 
@@ -212,11 +289,24 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
 }
 
 template <int FH, int FW, int OCT>
-static hipError_t launch_dwr(hipStream_t stream, const DwRowsArgs &a)
+static hipError_t launch_dwr(hipStream_t stream, DwRowsArgs a)
 {
     constexpr int OCB = 16 * OCT, YS = OCB + 16;
-    if (a.OWp > 64 || a.PW * 16 > 1024) return hipErrorNotSupported;
-    const size_t lds = ((size_t)2 * a.OWp * YS + (size_t)(FH + 1) * a.PW * DWR_XS) * sizeof(float);
+    // rows per step: as many as keep the chunk within 64 pixels and the R new input rows within 64 staged columns
+    int limit = 64 / a.PW;
+    if (limit > 64 / a.OWp) limit = 64 / a.OWp;
+    if (limit < 1) return hipErrorNotSupported;
+    if (limit > a.OH) limit = a.OH;
+    const int nchunks = (a.OH + limit - 1) / limit;
+    a.R = (a.OH + nchunks - 1) / nchunks;
+    a.CPI = (a.OH + a.R - 1) / a.R;
+    a.SLOTS = 2 * a.R + FH - 1;
+    a.steps2 = ((a.R * a.OWp) / 4 + 1) & ~1;
+    a.d_R = make_fastdiv(a.R);
+    a.d_SLOTS = make_fastdiv(a.SLOTS);
+    a.d_OWp = make_fastdiv(a.OWp);
+    a.d_PW = make_fastdiv(a.PW);
+    const size_t lds = ((size_t)2 * a.steps2 * 4 * YS + (size_t)a.SLOTS * a.PW * DWR_XS) * sizeof(float);
     if (lds > 160 * 1024) return hipErrorNotSupported;
     auto kern = delta_w_rows_kernel<FH, FW, OCT>;
     static size_t configured = 0;
@@ -247,7 +337,11 @@ hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *d
     a.PW = a.OWp + FW - 1;
     a.d_OW = make_fastdiv(OW);
     a.d_OH = make_fastdiv(OH);
-    if (FH == 3 && FW == 3) return launch_dwr<3, 3, 2>(stream, a);
+    if (FH == 3 && FW == 3) {
+        // 32 output channels per workgroup unless that leaves most of the 256 CUs without a workgroup
+        const long wgs = (long)((IC + 63) / 64) * ((OC + 31) / 32) * GZ;
+        return wgs >= 200 ? launch_dwr<3, 3, 2>(stream, a) : launch_dwr<3, 3, 1>(stream, a);
+    }
     if (FH == 1 && FW == 1) return launch_dwr<1, 1, 4>(stream, a);
     return hipErrorNotSupported;
 }

@@ -63,6 +63,7 @@ void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
     c->deltaX_s1_V2_Q = 1.1f;
     c->deltaX_ks_V2_Q = 1.1f;
     c->conv3D_winograd = 0;
+    c->deltaW_SK_fillUnits = 0;
 }
 
 // ---- forward: CudaFloat32EngineBase.conv3D (:1355-1474) ----------------------------------------------
@@ -134,6 +135,18 @@ void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int
     if (GridZ > c->deltaW_SK_MaxPartNum) GridZ = c->deltaW_SK_MaxPartNum;
     const int GridZ2 = GK >> 8;
     if (GridZ > GridZ2) GridZ = GridZ2;
+    if (c->deltaW_SK_fillUnits > 0) {
+        // The reference sizes GridZ for GPUs of at most 128 SMs; on a wider device a layer with few filter tiles leaves
+        // compute units idle. One workgroup of the backward-filter kernels covers 64 input channels x 32 output
+        // channels (64 for 1x1 filters) of one K slice.
+        const int ocb = (FH == 1 && FW == 1) ? 64 : 32;
+        const int tiles = ((IC + 63) / 64) * ((OC + ocb - 1) / ocb);
+        // rows of up to 36 pixels leave LDS for two co-resident workgroups per compute unit; wider rows for one
+        const int per_unit = (OW <= 36) ? 2 : 1;
+        int want = (per_unit * c->deltaW_SK_fillUnits + tiles - 1) / tiles;
+        if (want > GridZ2) want = GridZ2;
+        if (want > GridZ) GridZ = want;
+    }
     out->GridZ = GridZ;
     out->scratch_floats = (long)OC * FH * FW * IC * (GridZ - 1);
     if (FH == 1 && FW == 1 && sh == 1 && sw == 1) out->entry = ALPHA_E_dconv3D_deltaW_GemmSK_W1;   // W1 natives: stride 1 only

@@ -24,7 +24,7 @@ class Config(ctypes.Structure):
                 ("deltaW_SK_V2_Q", ctypes.c_float),
                 ("deltaX_s1_useTexture", ctypes.c_int), ("deltaX_ks_useTexture", ctypes.c_int),
                 ("deltaX_s1_V2_Q", ctypes.c_float), ("deltaX_ks_V2_Q", ctypes.c_float),
-                ("conv3D_winograd", ctypes.c_int)]
+                ("conv3D_winograd", ctypes.c_int), ("deltaW_SK_fillUnits", ctypes.c_int)]
 
 
 class Plan(ctypes.Structure):

@@ -32,6 +32,9 @@ typedef struct alpha_engine_config {
     float deltaX_s1_V2_Q;         /* 1.1 */
     float deltaX_ks_V2_Q;         /* 1.1 */
     int conv3D_winograd;          /* this build only (no reference flag): 1 = 3x3 stride-1 forward through Winograd F(2x2,3x3); default 0 */
+    int deltaW_SK_fillUnits;      /* this build only: when > 0, the split-K factor is raised (never lowered) until the launch has two
+                                     workgroups (one when output rows are wider than 36 pixels) for each of this many compute units,
+                                     slices staying >= 256 pixels; default 0 = the reference's GridZ exactly */
 } alpha_engine_config;
 
 /* Native entry chosen by a plan; names are the Java native method names. */

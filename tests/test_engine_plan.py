@@ -81,6 +81,30 @@ def test_deltaW_plans_and_split_k_factor():
     assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 8, 16, 16, 1, 1).GridZ == 2
 
 
+def test_deltaW_fill_option_only_raises_the_split_k_factor():
+    """deltaW_SK_fillUnits is this build's option (no reference flag): two workgroups of 64 ic x 32 oc (64 oc for 1x1) per
+    compute unit, slices of at least 256 pixels, never below the reference's GridZ."""
+    cfg = E.default_config(256)
+    assert cfg.deltaW_SK_fillUnits == 0
+    cfg.deltaW_SK_fillUnits = 256
+    # c2c: tiles = 4 x 8 = 32 -> 512/32 = 16 (reference: 3); GK>>8 = 32 does not bind
+    p = E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 128, 256, 256, 1, 1)
+    assert p.GridZ == 16 and p.scratch_floats == 15 * 256 * 9 * 256 and p.entry_name == "dconv3D_deltaW_GemmV2SK"
+    # c2b: tiles = 2 x 4 -> 64 (reference: 28)
+    assert E.plan_deltaW(cfg, 16, 16, 16, 16, 3, 3, 128, 128, 128, 1, 1).GridZ == 64
+    # rows wider than 36 pixels: one workgroup per unit. c5b: tiles = 1 x 2 -> 128 = the reference's value; c5a (1x1):
+    # tiles = 4 x 1 -> 64 < 128, unchanged; c2a (32-pixel rows): tiles = 2 -> 256 (reference: 128)
+    assert E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).GridZ == 128
+    assert E.plan_deltaW(cfg, 56, 56, 56, 56, 1, 1, 32, 256, 64, 1, 1).GridZ == 128
+    assert E.plan_deltaW(cfg, 32, 32, 32, 32, 3, 3, 128, 64, 64, 1, 1).GridZ == 256
+    # small GK: the 256-pixel floor binds (GK = 2048 -> at most 8 slices)
+    assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 32, 64, 64, 1, 1).GridZ == 8
+    # many tiles: want = 1 < reference value -> reference value kept
+    big = E.plan_deltaW(cfg, 14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1).GridZ
+    cfg.deltaW_SK_fillUnits = 0
+    assert big == E.plan_deltaW(cfg, 14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1).GridZ
+
+
 def test_deltaX_plans():
     cfg = E.default_config(256)
     assert E.plan_deltaX(cfg, 224, 224, 112, 112, 7, 7, 64, 4, 64, 2, 2).entry_name == "dconv3D_deltaX_crossAdd"   # IC <= 8

@@ -70,6 +70,27 @@ def test_engine_runs_the_entry_java_would_pick(dev, eng, case):
     check(dev.get(dw), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "engine deltaW %s" % (case,))
 
 
+def test_engine_deltaW_with_fill_option(dev):
+    """A larger split-K factor changes the summation order, not the result beyond the parity bar."""
+    N, IH, IC, OC = 32, 14, 128, 128
+    X, dY = normal((N, IH, IH, IC), 6101), normal((N, IH, IH, OC), 6102)
+    x, dy = dev.put(X), dev.put(dY)
+    want = O.deltaW_f64(X, dY, 3, 3, 1, 1, 1, 1)
+    e = pkg.engine.Engine(dev.stream)
+    try:
+        gz = []
+        for units in (0, 256):
+            e.config.deltaW_SK_fillUnits = units
+            dw = dev.empty(OC, 3, 3, IC, fill=float("nan"))
+            p = e.dconv3D_deltaW(dw.data_ptr(), 3, 3, x.data_ptr(), IH, IH, dy.data_ptr(), IH, IH, N, IC, OC, 1, 1, 1, 1)
+            e.sync()
+            gz.append(p.GridZ)
+            check(dev.get(dw), want, "engine deltaW fillUnits=%d (GridZ %d)" % (units, p.GridZ))
+        assert gz[1] > gz[0] and gz[1] == 24      # GK = 6272: 512/8 tiles = 64, capped by GK>>8 = 24
+    finally:
+        e.close()
+
+
 def test_engine_scratch_is_recycled_after_sync(dev, eng):
     N, IH, IC, OC = 8, 16, 32, 64
     X, W = normal((N, IH, IH, IC), 6004), he_normal(OC, 3, 3, IC, 6005)

@@ -420,6 +420,10 @@ DW_ROWS_SHAPES = [
     (8, 56, 56, 256, 64, 1, 0, 16),    # c5a geometry (1x1)
     (8, 56, 56, 64, 256, 1, 0, 16),    # c5c geometry (1x1)
     (4, 7, 9, 20, 36, 1, 0, 2),        # 1x1 ragged
+    (8, 12, 12, 128, 256, 3, 1, 13),   # enough workgroups for the 32-output-channel variant, 4 rows per step
+    (3, 14, 14, 64, 64, 3, 1, 2),      # c2c-sized rows: 3 rows per step, last step of an image has 2
+    (2, 5, 20, 32, 32, 3, 1, 1),       # single slice; 2 rows per step with OH odd
+    (5, 3, 40, 16, 48, 3, 1, 2),       # wide and short: one row per step, window spans the whole image
 ]
 
 
@@ -436,14 +440,14 @@ def test_deltaW_row_streaming_kernel_slices_and_sum(dev, shape):
         for algo in (0, 3):   # 0: row-streaming kernel where eligible, 3: generic kernel
             L.alpha_conv_set_fwd_algo(algo)
             dWo = dev.empty(OC, F_, F_, IC, fill=float("nan"))
-            buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+            buf = dev.empty(max(GridZ - 1, 1), sizeW, fill=float("nan"))
             if F_ == 1:
                 DW.dconv3D_deltaW_GemmSK_W1(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), buf.data_ptr(),
                                             N, IC, OC)
             else:
                 DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(),
                                          buf.data_ptr(), F_, F_, N, IC, OC, 1, 1, p, p)
-            outs[algo] = [dev.get(dWo)] + [b.reshape(OC, F_, F_, IC) for b in dev.get(buf)]
+            outs[algo] = [dev.get(dWo)] + [b.reshape(OC, F_, F_, IC) for b in dev.get(buf)[:GridZ - 1]]
     finally:
         L.alpha_conv_set_fwd_algo(0)
     total = np.zeros((OC, F_, F_, IC))
@@ -455,8 +459,9 @@ def test_deltaW_row_streaming_kernel_slices_and_sum(dev, shape):
             r = O.max_err_ratio(outs[algo][z], want, REL, max(floor, tolerance_floor(want)))
             assert r <= 1.0, "slice %d algo %d %s: err/allowed %.3f" % (z, algo, shape, r)
     dWs = dev.put(outs[0][0])
-    bufs = dev.put(np.stack([o.reshape(-1) for o in outs[0][1:]]))
-    DW.buf_summary(dev.stream, bufs.data_ptr(), dWs.data_ptr(), GridZ - 1, sizeW)
+    if GridZ > 1:
+        bufs = dev.put(np.stack([o.reshape(-1) for o in outs[0][1:]]))
+        DW.buf_summary(dev.stream, bufs.data_ptr(), dWs.data_ptr(), GridZ - 1, sizeW)
     check(dev.get(dWs), O.deltaW_f64(X, dY, F_, F_, 1, 1, p, p), "row-streaming dW total %s" % (shape,))
 
 
