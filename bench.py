@@ -203,7 +203,7 @@ def cpu_baseline(layer, op, budget_s=12.0):
     n = int(max(n0, min(N, n0 * budget_s / max(t_probe, 1e-6))))
     t1 = run(n) if n > n0 else t_probe
     n_used = n if n > n0 else n0
-    reps = int(max(1, min(200, budget_s / max(t1, 1e-6))))   # repeat the subset until ~budget_s of CPU work is timed
+    reps = int(max(1, min(5000, budget_s / max(t1, 1e-6))))   # repeat the subset until ~budget_s of CPU work is timed
     t = sum(run(n_used) for _ in range(reps))
     return {
         "value": round(per_image * n_used * reps / t / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
