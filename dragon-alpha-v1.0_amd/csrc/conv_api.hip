@@ -81,6 +81,11 @@ int forward(const char *fn, const int64_t *streams, int length,
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
 
+    if (FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
+        // W[OC][IC] is [N][K]; CW[IC][OC] is [K][N]
+        hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N * IH * IW, IC, OC, layout == FILTER_CW);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     if (layout == FILTER_CW && sh == 1 && sw == 1 && fwd_algo() != 3) {
         hipError_t e = launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
                                        0, FW * IC * OC, IC * OC, OC);
@@ -114,6 +119,11 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, 1, 1, ph, pw)) return e;
     if (FH - 1 - ph < 0 || FW - 1 - pw < 0) return fail(ALPHA_CONV_EINVAL, "%s: padding larger than FH-1", fn);
 
+    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
+        // deltaX[m][ic] = sum_oc deltaY[m][oc] * W[oc][ic]: W is [K][N]
+        hipError_t e = launch_pointwise(stream0(streams), dY, W, dX, N * IH * IW, OC, IC, 1);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     if (fwd_algo() != 3) {
         hipError_t e = launch_tap_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, FH - 1 - ph, FW - 1 - pw,
                                        ((FH - 1) * FW + (FW - 1)) * IC, -FW * IC, -IC, FH * FW * IC);

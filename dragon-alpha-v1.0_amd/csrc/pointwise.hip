@@ -1,0 +1,201 @@
+// 1x1 stride-1 convolution (forward and backward-data) as a streaming GEMM, fp32 MFMA v_mfma_f32_16x16x4_f32, gfx950.
+//
+//   O[m, n] = sum_k A[m, k] * B(k, n)        m = pixel (N*H*W of them), k = reduced channels, n = produced channels
+//
+// These layers sit at or below the ridge of the roofline (c5a/c5c: 26 FLOP/byte), so the design goal is one pass
+// over A and O at full memory rate, not MFMA occupancy:
+//   * the whole filter (K x N <= ~120 KB with padding) is copied into LDS once per workgroup, laid out [n][K+8] so
+//     that a lane's 4 consecutive k of one n are one 128-bit read and the 32 lanes of a half wavefront hit 32
+//     different 16-byte slots (row stride = 8 floats modulo 16);
+//   * one workgroup of 8 wavefronts per compute unit, persistent, owning a contiguous range of 16-pixel tiles that
+//     its wavefronts draw from a counter in LDS;
+//   * A goes from global memory straight into the MFMA operand layout: lane (l16, q) loads float4
+//     A[16t + l16][64kb + 16c + 4q ..] (K permutation: lane group q supplies channel 16c + 4q + s at step s, as the
+//     filter read does), one whole tile ahead of the tile being multiplied. No LDS, no barrier for A;
+//   * each 16 x 64 block of results is transposed through a wavefront-private LDS patch so that every pixel's 256
+//     bytes leave as whole lines.
+#include "common.hpp"
+
+namespace alpha {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+struct PointwiseArgs {
+    const float *A;   // [M][K]
+    const float *B;   // b_kmajor ? [K][N] : [N][K]
+    float *O;         // [M][N]
+    int M, K, N;
+    int b_kmajor;
+    int tiles;        // ceil(M / 16)
+};
+
+constexpr int PW_OS = 64 + 4;   // staging row stride (floats)
+
+template <int NT, int KB>   // N = 16*NT produced channels, K = 64*KB reduced channels
+__global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p)
+{
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    constexpr int K = 64 * KB, N = 16 * NT, KS = K + 8;
+    float *Bs = smem;                                 // [N][KS]
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int l16 = lane & 15, q = lane >> 4;
+    float *Os = smem + N * KS + w * (16 * PW_OS);     // [16][PW_OS], private to the wavefront
+
+    // ---- tiles: the workgroup owns the contiguous range [t_begin, t_end); its wavefronts take the first eight
+    // statically and then draw from a counter in LDS, so they finish within one tile of each other whatever the
+    // range length (a static split of 24.5 tiles over 8 wavefronts would leave a quarter of the machine idle).
+    // The first tile's A fragments are requested before anything else.
+    const int G = gridDim.x;
+    const int t_begin = (int)((long)p.tiles * blockIdx.x / G), t_end = (int)((long)p.tiles * (blockIdx.x + 1) / G);
+    int *queue = reinterpret_cast<int *>(smem + N * KS + 8 * 16 * PW_OS);
+    if (t == 0) *queue = t_begin + 8;
+
+    auto load_a = [&](floatx4 (&a)[KB][4], int tile) {
+        const int m = min(tile * 16 + l16, p.M - 1);   // rows past M are computed from a valid row and never stored
+        const float *src = p.A + (size_t)m * K + 4 * q;
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) a[kb][c] = *reinterpret_cast<const floatx4 *>(src + 64 * kb + 16 * c);
+    };
+    floatx4 aP[KB][4], aQ[KB][4];
+    int tile = t_begin + w;
+    load_a(aP, min(tile, p.tiles - 1));
+
+    // ---- filter -> LDS, once: 8 loads in flight per thread, consecutive lanes along k so that the transposing
+    // stores of the [K][N] layout fall into consecutive banks -------------------------------------------------------
+    constexpr int QUADS = N * K / 4;
+    for (int base = 0; base < QUADS; base += 512 * 8) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int idx = min(base + t + 512 * u, QUADS - 1);
+            if (!p.b_kmajor) {
+                const int n = idx / (K / 4), k4 = (idx % (K / 4)) * 4;
+                v[u] = *reinterpret_cast<const float4 *>(p.B + n * K + k4);
+            } else {
+                const int k = idx % K, n4 = (idx / K) * 4;
+                v[u] = *reinterpret_cast<const float4 *>(p.B + k * N + n4);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int idx = base + t + 512 * u;
+            if (idx < QUADS) {
+                if (!p.b_kmajor) {
+                    const int n = idx / (K / 4), k4 = (idx % (K / 4)) * 4;
+                    *reinterpret_cast<float4 *>(Bs + n * KS + k4) = v[u];
+                } else {
+                    const int k = idx % K, n4 = (idx / K) * 4;
+                    Bs[(n4 + 0) * KS + k] = v[u].x;
+                    Bs[(n4 + 1) * KS + k] = v[u].y;
+                    Bs[(n4 + 2) * KS + k] = v[u].z;
+                    Bs[(n4 + 3) * KS + k] = v[u].w;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    floatx4 acc[NT];
+    const float *bl = Bs + l16 * KS + 4 * q;
+    while (tile < t_end) {
+        // draw the next tile and start its fragments on their way while this tile is multiplied (past the end of
+        // the range: re-fetch this tile, unused)
+        int ntile = 0;
+        if (lane == 0) ntile = atomicAdd(queue, 1);
+        ntile = __builtin_amdgcn_readfirstlane(ntile);
+        load_a(aQ, ntile < t_end ? ntile : tile);
+#pragma unroll
+        for (int j = 0; j < NT; j++) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+#pragma unroll
+                for (int j = 0; j < NT; j++) {
+                    const floatx4 b = *reinterpret_cast<const floatx4 *>(bl + j * 16 * KS + kb * 64 + 16 * c);
+#pragma unroll
+                    for (int s = 0; s < 4; s++) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(aP[kb][c][s], b[s], acc[j], 0, 0, 0);
+                }
+
+        // ---- lane holds O[16*tile + 4q + r][16j + l16]; 64 columns at a time through the LDS patch -----------------
+#pragma unroll
+        for (int jg = 0; jg < NT / 4; jg++) {
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) Os[(4 * q + r) * PW_OS + 16 * jj + l16] = acc[4 * jg + jj][r];
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = 4 * i + q, m = tile * 16 + row;
+                const float4 v = *reinterpret_cast<const float4 *>(Os + row * PW_OS + 4 * l16);
+                if (m < p.M) *reinterpret_cast<float4 *>(p.O + (size_t)m * N + 64 * jg + 4 * l16) = v;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) aP[kb][c] = aQ[kb][c];
+        tile = ntile;
+    }
+}
+
+template <int NT, int KB>
+static hipError_t launch_pw(hipStream_t stream, const PointwiseArgs &a, int cus)
+{
+    constexpr size_t lds = ((size_t)16 * NT * (64 * KB + 8) + 8 * 16 * PW_OS + 4) * sizeof(float);
+    static_assert(lds <= 160 * 1024, "filter + staging must fit in LDS");
+    auto kern = pointwise_kernel<NT, KB>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    int grid = cus;
+    if (grid * 8 > a.tiles) grid = (a.tiles + 7) / 8;   // at least 8 tiles per workgroup when there are few
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
+    return hipGetLastError();
+}
+
+// O[M][N] = A[M][K] * B. Returns hipErrorNotSupported (nothing launched) unless (K, N) is one of the combinations below
+// (filter resident in LDS); the caller then uses another kernel.
+hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, float *O, int M, int K, int N, int b_kmajor)
+{
+    if (M < 1 || (K & 63) || K < 64 || K > 256) return hipErrorNotSupported;
+    if (N != 64 && N != 128 && N != 256) return hipErrorNotSupported;
+    if ((long)N * K > 128 * 128 && !(N == 64 && K == 256) && !(N == 256 && K == 64)) return hipErrorNotSupported;
+    if ((size_t)M * (size_t)(K > N ? K : N) >= (1u << 31)) return hipErrorNotSupported;
+    static int cu_count[64] = {0};   // per device; a racing first call writes the same value
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorNotSupported;
+    if (cu_count[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return hipErrorNotSupported;
+        cu_count[dev] = n;
+    }
+    const int cus = cu_count[dev];
+    PointwiseArgs a{};
+    a.A = A; a.B = B; a.O = O;
+    a.M = M; a.K = K; a.N = N; a.b_kmajor = b_kmajor;
+    a.tiles = (M + 15) / 16;
+    const int KB = K / 64;
+    if (N == 64) {
+        if (KB == 1) return launch_pw<4, 1>(stream, a, cus);
+        if (KB == 2) return launch_pw<4, 2>(stream, a, cus);
+        if (KB == 3) return launch_pw<4, 3>(stream, a, cus);
+        return launch_pw<4, 4>(stream, a, cus);
+    }
+    if (N == 128) {
+        if (KB == 1) return launch_pw<8, 1>(stream, a, cus);
+        if (KB == 2) return launch_pw<8, 2>(stream, a, cus);
+        return hipErrorNotSupported;
+    }
+    if (KB == 1) return launch_pw<16, 1>(stream, a, cus);
+    return hipErrorNotSupported;
+}
+
+}  // namespace alpha

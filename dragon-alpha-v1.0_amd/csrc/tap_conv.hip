@@ -90,16 +90,24 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
 
     // ---- filter fragments straight from global memory -------------------------------------------------
     // lane (l16, q) of wavefront w needs, for channel group g of a half tap, B[c = 16g + 4q + s][oc0 + 16w + l16].
+    // Address = (uniform base of the half tap, kept in scalar registers) + (per-lane byte offset, fixed for the whole
+    // kernel), so a load costs no vector arithmetic.
     const int b_co = oc0 + 16 * w + l16;
     const bool b_cov = b_co < p.CO;   // columns beyond CO are never stored; clamp their loads to a valid address
+    unsigned b_lane[2][4];
+#pragma unroll
+    for (int g = 0; g < 2; g++)
+#pragma unroll
+        for (int s = 0; s < 4; s++) b_lane[g][s] = (unsigned)(((16 * g + 4 * q + s) * p.b_sc + (b_cov ? b_co : 0)) * 4);
     auto load_b = [&](float (&b)[2][4], int icbase, int th, int tw) {
-        const int base = p.b_off + th * p.b_sth + tw * p.b_stw + (b_cov ? b_co : 0);
+        const int sbase = __builtin_amdgcn_readfirstlane(p.b_off + th * p.b_sth + tw * p.b_stw + icbase * p.b_sc);
+        const char *sb = reinterpret_cast<const char *>(p.B + sbase);
 #pragma unroll
         for (int g = 0; g < 2; g++) {
-            const int c = icbase + 16 * g + 4 * q;
-            const int ok = -(int)(c < p.AC);   // AC % 4 == 0: the four channels are valid together
+            // RAGGED: channels beyond AC (AC % 4 == 0: four at a time) are fetched from the half tap's first element
+            const unsigned ok = RAGGED ? (unsigned)-(int)(icbase + 16 * g + 4 * q < p.AC) : ~0u;
 #pragma unroll
-            for (int s = 0; s < 4; s++) b[g][s] = p.B[(base + (c + s) * p.b_sc) & ok];
+            for (int s = 0; s < 4; s++) b[g][s] = *reinterpret_cast<const float *>(sb + (b_lane[g][s] & ok));
         }
     };
     // channels beyond AC: the halo holds zeros there, but 0 * (whatever the clamped load returned) must
@@ -117,26 +125,30 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
     const int halo_quads = rows * PWt * (TC_ICC / 4);
     const int taps = p.TH * p.TW;
 
-    auto half_tap = [&](const float (&b)[2][4], int th, int tw, int half) {
-        const float *hs = Hs + (th * PWt + tw) * TC_PS + 32 * half;
-        floatx4 a0[TILES], a1[TILES];
+    // A fragments of one 16-channel chunk: chunk ck (0..3) of tap (th, tw) starts 16*ck floats into the pixel
+    auto read_a = [&](floatx4 (&a)[TILES], int th, int tw, int ck) {
+        const float *hs = Hs + (th * PWt + tw) * TC_PS + 16 * ck;
 #pragma unroll
-        for (int i = 0; i < TILES; i++) a0[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i]);
-#pragma unroll
-        for (int i = 0; i < TILES; i++) a1[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i] + 16);
-#pragma unroll
-        for (int s = 0; s < 4; s++)
-#pragma unroll
-            for (int i = 0; i < TILES; i++)
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[i][s], b[0][s], acc[i], 0, 0, 0);
+        for (int i = 0; i < TILES; i++) a[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i]);
+    };
+    auto mfma_chunk = [&](const floatx4 (&a)[TILES], const float (&b)[4]) {
 #pragma unroll
         for (int s = 0; s < 4; s++)
 #pragma unroll
             for (int i = 0; i < TILES; i++)
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[i][s], b[1][s], acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i][s], b[s], acc[i], 0, 0, 0);
+    };
+    // LDS reads of the next chunk issue in the shadow of this chunk's first MFMAs
+    auto spread_reads = [&]() {
+#pragma unroll
+        for (int i = 0; i < TILES; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 LDS read
+        }
     };
 
     float bA[2][4], bB[2][4];
+    floatx4 aP[TILES], aQ[TILES];   // A fragments ping-pong: the next chunk is read while the current one is multiplied
     load_b(bA, 0, 0, 0);   // first half tap; in flight while the halo is staged
     for (int ic0 = 0; ic0 < p.AC; ic0 += TC_ICC) {
         if (ic0 > 0) __syncthreads();   // everyone finished reading the previous pass's halo
@@ -171,32 +183,47 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
         }
         __syncthreads();
 
-        // ---- main loop: two half taps per iteration, filter fragments ping-pong between bA and bB --------
+        // ---- main loop: one tap (four 16-channel chunks) per iteration ------------------------------------
+        // Filter fragments ping-pong between bA and bB one half tap (two chunks) ahead, A fragments between aP
+        // and aQ one chunk ahead. Every prefetch is unconditional (a branch around it would make every wait in the
+        // loop assume the shorter queue): after the last tap it fetches the first half tap of the next pass, or
+        // harmlessly re-fetches tap (0,0) of this one at the very end. The scheduling barriers pin each prefetch in
+        // front of the chunk that hides its latency; left alone the compiler sinks the loads to their first use.
         int th = 0, tw = 0;
+        read_a(aP, 0, 0, 0);
         for (int tap = 0; tap < taps; tap++) {
-            // The prefetch below is unconditional (a branch around it would make every wait in the loop
-            // assume the shorter queue): after the last tap it fetches the first half tap of the next
-            // pass, or harmlessly re-fetches tap (0,0) of this one at the very end.
             int nth = th, ntw = tw + 1, nic = ic0;
             if (ntw == p.TW) { ntw = 0; nth = th + 1; }
             if (tap + 1 == taps) { nth = 0; ntw = 0; nic = ic0 + TC_ICC < p.AC ? ic0 + TC_ICC : ic0; }
-            // The scheduling barriers pin each prefetch in front of the half tap that hides its latency; left
-            // alone the compiler sinks the loads to just before their first use.
+            __builtin_amdgcn_sched_barrier(0);
             load_b(bB, ic0 + 32, th, tw);
             __builtin_amdgcn_sched_barrier(0);
             mask_b(bA, ic0);
-            half_tap(bA, th, tw, 0);
+            read_a(aQ, th, tw, 1);
+            mfma_chunk(aP, bA[0]);
+            spread_reads();
+            __builtin_amdgcn_sched_barrier(0);
+            read_a(aP, th, tw, 2);
+            mfma_chunk(aQ, bA[1]);
+            spread_reads();
             __builtin_amdgcn_sched_barrier(0);
             load_b(bA, nic, nth, ntw);
             __builtin_amdgcn_sched_barrier(0);
             mask_b(bB, ic0 + 32);
-            half_tap(bB, th, tw, 1);
+            read_a(aQ, th, tw, 3);
+            mfma_chunk(aP, bB[0]);
+            spread_reads();
+            __builtin_amdgcn_sched_barrier(0);
+            read_a(aP, nth, ntw, 0);   // after the last tap of a pass: re-read once the next halo is staged
+            mfma_chunk(aQ, bB[1]);
+            spread_reads();
             __builtin_amdgcn_sched_barrier(0);
             th = nth;
             tw = ntw;
         }
     }
     (void)bA;
+    (void)aP;
 
     // ---- epilogue: transpose through LDS so every output pixel row is written as whole 256-byte lines ----
     __syncthreads();   // all wavefronts are done reading the halo

@@ -286,6 +286,40 @@ def test_deltaX_W1(dev):
         check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, 0, 0), "deltaX_W1", sp_thr=1e-4)
 
 
+POINTWISE_SHAPES = [
+    # N, IH, IW, IC, OC: 1x1 stride-1 layers served by the streaming GEMM kernel (reduced side a multiple of 64,
+    # produced side 64/128/256, filter fits in LDS), forward in both filter layouts and backward-data
+    (4, 14, 14, 256, 64),     # c5a geometry: K = 256 forward, K = 64 backward
+    (4, 9, 7, 64, 256),       # c5c geometry; 252 pixels: the last 16-pixel tile is ragged
+    (3, 5, 5, 128, 128),      # 75 pixels: fewer tiles than wavefronts
+    (2, 33, 31, 64, 64),      # 2046 pixels
+    (1, 1, 3, 192, 64),       # 3 pixels: a single ragged tile; K = 192 = 3 blocks forward (backward falls to another kernel)
+]
+
+
+@pytest.mark.parametrize("shape", POINTWISE_SHAPES)
+def test_pointwise_kernel_forward_and_deltaX(dev, shape):
+    N, IH, IW, IC, OC = shape
+    X, W, dY = normal((N, IH, IW, IC), 2101), he_normal(OC, 1, 1, IC, 2102), normal((N, IH, IW, OC), 2103)
+    want_y, want_dx = O.conv3D_f64(X, W, 1, 1, 0, 0), O.deltaX_f64(dY, W, IH, IW, 1, 1, 0, 0)
+    L = pkg.lib()
+    outs = {}
+    try:
+        for algo in (0, 3):   # 0: streaming GEMM kernel, 3: generic kernel
+            L.alpha_conv_set_fwd_algo(algo)
+            outs[algo] = (_run_fwd(dev, "conv3D_W1", X, W, 1, 1, 0, 0), _run_fwd(dev, "conv3D_GemmR_W1", X, W, 1, 1, 0, 0))
+            dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+            dy, w = dev.put(dY), dev.put(W)
+            DX.dconv3D_deltaX_W1(dev.streams, 1, dy.data_ptr(), w.data_ptr(), dXo.data_ptr(), IH, IW, N, IC, OC)
+            outs[algo] += (dev.get(dXo),)
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+    for algo in (0, 3):
+        check(outs[algo][0], want_y, "conv3D_W1 algo %d %s" % (algo, shape))
+        check(outs[algo][1], want_y, "conv3D_GemmR_W1 algo %d %s" % (algo, shape))
+        check(outs[algo][2], want_dx, "deltaX_W1 algo %d %s" % (algo, shape), sp_thr=1e-4)
+
+
 KS_SHAPES = [
     # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw
     (4, 16, 16, 64, 128, 3, 3, 2, 2, 1, 1),
