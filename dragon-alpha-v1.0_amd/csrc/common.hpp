@@ -92,6 +92,11 @@ hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *d
                               int sh, int sw, int ph, int pw, int GK_slice, int GZ);
 
 // Winograd F(2x2,3x3) forward (winograd.hip): U = transformed filter [16][IC][OC].
+// Backward-filter of 1x1 stride-1 layers from registers (delta_w_pointwise.hip); same slice partition and outputs.
+// Returns hipErrorNotSupported (nothing launched) unless IC and OC are multiples of 64.
+hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
+                                   int GK, int IC, int OC, int GK_slice, int GZ);
+
 hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC);
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw);

@@ -207,6 +207,10 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     a.GK = N * OH * OW;
     a.GZ = GridZ;
     a.GK_slice = (a.GK / GridZ) >> 3 << 3;
+    if (fwd_algo() != 3 && FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0) {
+        hipError_t e = launch_deltaW_pointwise(stream0(streams), X, dY, dW, dW_buf, a.GK, IC, OC, a.GK_slice, GridZ);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     if (fwd_algo() != 3) {
         hipError_t e = launch_deltaW_rows(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
                                           a.GK_slice, GridZ);

@@ -454,6 +454,12 @@ DW_ROWS_SHAPES = [
     (8, 56, 56, 256, 64, 1, 0, 16),    # c5a geometry (1x1)
     (8, 56, 56, 64, 256, 1, 0, 16),    # c5c geometry (1x1)
     (4, 7, 9, 20, 36, 1, 0, 2),        # 1x1 ragged
+    # 1x1 with channel counts multiples of 64: the register kernel (64x64 output blocks, slice pixels split in parts)
+    (4, 14, 14, 128, 64, 1, 0, 3),     # 2 blocks, one per workgroup, 8 parts each
+    (8, 16, 16, 256, 128, 1, 0, 40),   # 8 blocks; slices of 48 pixels = 12 groups over 8 parts (1 or 2 groups each)
+    (4, 3, 3, 64, 192, 1, 0, 1),       # single slice of 36 pixels
+    (4, 8, 8, 256, 256, 1, 0, 32),     # 16 blocks, two per workgroup, 4 parts; slices of 8 pixels: parts may be empty
+    (4, 8, 8, 512, 512, 1, 0, 32),     # 64 blocks, eight per workgroup, no pixel split
     (8, 12, 12, 128, 256, 3, 1, 13),   # enough workgroups for the 32-output-channel variant, 4 rows per step
     (3, 14, 14, 64, 64, 3, 1, 2),      # c2c-sized rows: 3 rows per step, last step of an image has 2
     (2, 5, 20, 32, 32, 3, 1, 1),       # single slice; 2 rows per step with OH odd
