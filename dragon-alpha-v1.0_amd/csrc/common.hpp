@@ -63,9 +63,10 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
                            int b_off, int b_sth, int b_stw, int b_sc);
 
 // 1x1 stride-1 convolution as a streaming GEMM with the filter resident in LDS (pointwise.hip):
-// O[M][N] = A[M][K] * B, B given as [K][N] (b_kmajor) or [N][K]. Returns hipErrorNotSupported (nothing launched)
-// when the shape does not fit.
-hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, float *O, int M, int K, int N, int b_kmajor);
+// O[(n,oh,ow)][co] = sum_k A[n, oh*sh, ow*sw, k] * B(k, co), B given as [K][N] (b_kmajor) or [N][K]. Returns
+// hipErrorNotSupported (nothing launched) when the shape does not fit.
+hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, float *O, int Nimg, int AH, int AW,
+                            int OH, int OW, int sh, int sw, int K, int N, int b_kmajor);
 
 // Backward-filter implicit GEMM with split-K over k = (n, oh, ow):
 //   dst_z[oc, fh, fw, ic] = sum_{k in slice z} deltaY[k, oc] * X[n, oh*sh - ph + fh, ow*sw - pw + fw, ic]

@@ -81,9 +81,9 @@ int forward(const char *fn, const int64_t *streams, int length,
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
 
-    if (FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
-        // W[OC][IC] is [N][K]; CW[IC][OC] is [K][N]
-        hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N * IH * IW, IC, OC, layout == FILTER_CW);
+    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
+        // W[OC][IC] is [N][K]; CW[IC][OC] is [K][N]; a stride only thins the input pixels that are read
+        hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (layout == FILTER_CW && sh == 1 && sw == 1 && fwd_algo() != 3) {
@@ -121,7 +121,7 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
 
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
         // deltaX[m][ic] = sum_oc deltaY[m][oc] * W[oc][ic]: W is [K][N]
-        hipError_t e = launch_pointwise(stream0(streams), dY, W, dX, N * IH * IW, OC, IC, 1);
+        hipError_t e = launch_pointwise(stream0(streams), dY, W, dX, N, IH, IW, IH, IW, 1, 1, OC, IC, 1);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (fwd_algo() != 3) {

@@ -21,12 +21,15 @@ namespace alpha {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 struct PointwiseArgs {
-    const float *A;   // [M][K]
-    const float *B;   // b_kmajor ? [K][N] : [N][K]
-    float *O;         // [M][N]
-    int M, K, N;
+    const float *A;   // [rows][K]; output pixel m = (n, oh, ow) reads row (n*AH + oh*sh)*AW + ow*sw
+    const float *B;   // b_kmajor ? [K][ldn] : [ldn][K]
+    float *O;         // [M][ldn]
+    int M, K, ldn;    // ldn = all produced channels; a workgroup produces the 16*NT of them starting at 16*NT*blockIdx.y
     int b_kmajor;
     int tiles;        // ceil(M / 16)
+    int strided;      // 0: row = m
+    int AH, AW, sh, sw;
+    FastDiv d_OW, d_OHW;
 };
 
 constexpr int PW_OS = 64 + 4;   // staging row stride (floats)
@@ -50,8 +53,14 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
     int *queue = reinterpret_cast<int *>(smem + N * KS + 8 * 16 * PW_OS);
     if (t == 0) *queue = t_begin + 8;
 
+    const int n_off = blockIdx.y * N, ldn = p.ldn;
     auto load_a = [&](floatx4 (&a)[KB][4], int tile) {
-        const int m = min(tile * 16 + l16, p.M - 1);   // rows past M are computed from a valid row and never stored
+        int m = min(tile * 16 + l16, p.M - 1);   // rows past M are computed from a valid row and never stored
+        if (p.strided) {
+            const int n = fdiv(m, p.d_OHW), rem = m - n * p.d_OHW.d;
+            const int oh = fdiv(rem, p.d_OW), ow = rem - oh * p.d_OW.d;
+            m = (n * p.AH + oh * p.sh) * p.AW + ow * p.sw;
+        }
         const float *src = p.A + (size_t)m * K + 4 * q;
 #pragma unroll
         for (int kb = 0; kb < KB; kb++)
@@ -72,10 +81,10 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
             const int idx = min(base + t + 512 * u, QUADS - 1);
             if (!p.b_kmajor) {
                 const int n = idx / (K / 4), k4 = (idx % (K / 4)) * 4;
-                v[u] = *reinterpret_cast<const float4 *>(p.B + n * K + k4);
+                v[u] = *reinterpret_cast<const float4 *>(p.B + (size_t)(n_off + n) * K + k4);
             } else {
                 const int k = idx % K, n4 = (idx / K) * 4;
-                v[u] = *reinterpret_cast<const float4 *>(p.B + k * N + n4);
+                v[u] = *reinterpret_cast<const float4 *>(p.B + (size_t)k * ldn + n_off + n4);
             }
         }
 #pragma unroll
@@ -131,7 +140,7 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
             for (int i = 0; i < 4; i++) {
                 const int row = 4 * i + q, m = tile * 16 + row;
                 const float4 v = *reinterpret_cast<const float4 *>(Os + row * PW_OS + 4 * l16);
-                if (m < p.M) *reinterpret_cast<float4 *>(p.O + (size_t)m * N + 64 * jg + 4 * l16) = v;
+                if (m < p.M) *reinterpret_cast<float4 *>(p.O + (size_t)m * ldn + n_off + 64 * jg + 4 * l16) = v;
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -155,20 +164,24 @@ static hipError_t launch_pw(hipStream_t stream, const PointwiseArgs &a, int cus)
         if (e != hipSuccess) return e;
         configured = true;
     }
-    int grid = cus;
+    const int nblocks = a.ldn / (16 * NT);
+    int grid = cus / nblocks;                            // one workgroup per compute unit, shared among the N blocks
+    if (grid < 1) grid = 1;
     if (grid * 8 > a.tiles) grid = (a.tiles + 7) / 8;   // at least 8 tiles per workgroup when there are few
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3(grid, nblocks), dim3(512), lds, stream, a);
     return hipGetLastError();
 }
 
-// O[M][N] = A[M][K] * B. Returns hipErrorNotSupported (nothing launched) unless (K, N) is one of the combinations below
-// (filter resident in LDS); the caller then uses another kernel.
-hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, float *O, int M, int K, int N, int b_kmajor)
+// O[m][n] = sum_k A[row(m)][k] * B(k, n) for m < M = Nimg*OH*OW, n < N. The produced channels are split into blocks
+// of 256, 128 or 64 (the largest that divides N and whose filter block fits in LDS beside the staging patches); with
+// more than one block A is read once per block (from L2 for the sizes this serves). Returns hipErrorNotSupported
+// (nothing launched) unless K is 64, 128, 192 or 256 and N a multiple of 64; the caller then uses another kernel.
+hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, float *O, int Nimg, int AH, int AW,
+                            int OH, int OW, int sh, int sw, int K, int N, int b_kmajor)
 {
-    if (M < 1 || (K & 63) || K < 64 || K > 256) return hipErrorNotSupported;
-    if (N != 64 && N != 128 && N != 256) return hipErrorNotSupported;
-    if ((long)N * K > 128 * 128 && !(N == 64 && K == 256) && !(N == 256 && K == 64)) return hipErrorNotSupported;
-    if ((size_t)M * (size_t)(K > N ? K : N) >= (1u << 31)) return hipErrorNotSupported;
+    const long Ml = (long)Nimg * OH * OW;
+    if (Ml < 1 || (K & 63) || K < 64 || K > 256 || (N & 63) || N < 64) return hipErrorNotSupported;
+    if ((size_t)Nimg * AH * AW * K >= (1ull << 31) || (size_t)Ml * N >= (1ull << 31)) return hipErrorNotSupported;
     static int cu_count[64] = {0};   // per device; a racing first call writes the same value
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorNotSupported;
@@ -180,22 +193,24 @@ hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, 
     const int cus = cu_count[dev];
     PointwiseArgs a{};
     a.A = A; a.B = B; a.O = O;
-    a.M = M; a.K = K; a.N = N; a.b_kmajor = b_kmajor;
-    a.tiles = (M + 15) / 16;
+    a.M = (int)Ml; a.K = K; a.ldn = N; a.b_kmajor = b_kmajor;
+    a.tiles = (a.M + 15) / 16;
+    a.strided = !(sh == 1 && sw == 1 && OH == AH && OW == AW);
+    a.AH = AH; a.AW = AW; a.sh = sh; a.sw = sw;
+    a.d_OW = make_fastdiv(OW);
+    a.d_OHW = make_fastdiv(OH * OW);
     const int KB = K / 64;
-    if (N == 64) {
-        if (KB == 1) return launch_pw<4, 1>(stream, a, cus);
-        if (KB == 2) return launch_pw<4, 2>(stream, a, cus);
-        if (KB == 3) return launch_pw<4, 3>(stream, a, cus);
-        return launch_pw<4, 4>(stream, a, cus);
+    if (KB == 1) {
+        if (N % 256 == 0) return launch_pw<16, 1>(stream, a, cus);
+        if (N % 128 == 0) return launch_pw<8, 1>(stream, a, cus);
+        return launch_pw<4, 1>(stream, a, cus);
     }
-    if (N == 128) {
-        if (KB == 1) return launch_pw<8, 1>(stream, a, cus);
-        if (KB == 2) return launch_pw<8, 2>(stream, a, cus);
-        return hipErrorNotSupported;
+    if (KB == 2) {
+        if (N % 128 == 0) return launch_pw<8, 2>(stream, a, cus);
+        return launch_pw<4, 2>(stream, a, cus);
     }
-    if (KB == 1) return launch_pw<16, 1>(stream, a, cus);
-    return hipErrorNotSupported;
+    if (KB == 3) return launch_pw<4, 3>(stream, a, cus);
+    return launch_pw<4, 4>(stream, a, cus);
 }
 
 }  // namespace alpha

@@ -320,6 +320,20 @@ def test_pointwise_kernel_forward_and_deltaX(dev, shape):
         check(outs[algo][2], want_dx, "deltaX_W1 algo %d %s" % (algo, shape), sp_thr=1e-4)
 
 
+@pytest.mark.parametrize("shape", [
+    # N, IH, IW, IC, OC, sh, sw: strided 1x1 layers (c4c geometry and ragged ones) through the general entries
+    (8, 28, 28, 64, 128, 2, 2),
+    (4, 9, 7, 128, 192, 2, 3),
+    (2, 15, 15, 256, 320, 3, 1),
+])
+def test_pointwise_kernel_strided(dev, shape):
+    N, IH, IW, IC, OC, sh, sw = shape
+    X, W = normal((N, IH, IW, IC), 2111), he_normal(OC, 1, 1, IC, 2112)
+    want = O.conv3D_f64(X, W, sh, sw, 0, 0)
+    for entry in ("conv3D", "conv3D_GemmR", "conv3D_np"):
+        check(_run_fwd(dev, entry, X, W, sh, sw, 0, 0), want, "%s strided 1x1 %s" % (entry, shape))
+
+
 KS_SHAPES = [
     # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw
     (4, 16, 16, 64, 128, 3, 3, 2, 2, 1, 1),
