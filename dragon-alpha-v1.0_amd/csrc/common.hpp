@@ -93,6 +93,11 @@ hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *d
                               int sh, int sw, int ph, int pw, int GK_slice, int GZ);
 
 // Winograd F(2x2,3x3) forward (winograd.hip): U = transformed filter [16][IC][OC].
+// Forward convolution for IC (stored) = 4 with the filter resident in LDS (stem_conv.hip); F is W[OC,FH,FW,4] or, with
+// f_cw, CW[FH,FW,4,OC]. Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
+hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, int f_cw, float *Y,
+                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw);
+
 // Backward-filter of 1x1 stride-1 layers from registers (delta_w_pointwise.hip); same slice partition and outputs.
 // Returns hipErrorNotSupported (nothing launched) unless IC and OC are multiples of 64.
 hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,

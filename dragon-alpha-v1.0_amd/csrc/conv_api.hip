@@ -81,6 +81,10 @@ int forward(const char *fn, const int64_t *streams, int length,
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
 
+    if (IC == 4 && fwd_algo() != 3) {
+        hipError_t e = launch_stem_conv(stream0(streams), X, F, layout == FILTER_CW, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
         // W[OC][IC] is [N][K]; CW[IC][OC] is [K][N]; a stride only thins the input pixels that are read
         hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW);

@@ -184,8 +184,11 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
         __syncthreads();
     }
 
-    // ---- epilogue: row -> output offset table in LDS, then masked stores ---------------------------
-    int *rowoff = reinterpret_cast<int *>(smem);
+    // ---- epilogue: the tile goes through LDS so that every output row leaves as whole 16-byte-per-lane segments
+    // (stored straight from the MFMA layout, 4 bytes per lane, the same tile cost 8-10x its size in write traffic) ----
+    constexpr int OS = BN + 4;
+    float *Os = smem;                                            // [BM][OS]; the loop's last barrier freed the tiles
+    int *rowoff = reinterpret_cast<int *>(smem + BM * OS);       // [BM] output offset of each row, -1 beyond M
     for (int r = t; r < BM; r += 256) {
         const int m = m0 + r;
         int off = -1;
@@ -196,19 +199,24 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
         }
         rowoff[r] = off;
     }
-    __syncthreads();
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            const int col = n0 + (wn * TN + j) * 32 + l32;
+            const int col = (wn * TN + j) * 32 + l32;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                const int ro = rowoff[row];
-                if (ro >= 0 && col < CO) p.O[ro + col] = acc[i][j][r];
+                Os[row * OS + col] = acc[i][j][r];
             }
         }
+    __syncthreads();
+    for (int idx = t; idx < BM * (BN / 4); idx += 256) {
+        const int row = idx / (BN / 4), c4 = (idx % (BN / 4)) * 4;
+        const int ro = rowoff[row];
+        if (ro >= 0 && n0 + c4 < CO)   // CO % 4 == 0: the four columns are valid together
+            *reinterpret_cast<float4 *>(p.O + ro + n0 + c4) = *reinterpret_cast<const float4 *>(Os + row * OS + c4);
+    }
 }
 
 template <int WM, int WN, int TM, int TN, bool B_NMAJOR>
@@ -217,7 +225,9 @@ static hipError_t launch_cfg(hipStream_t stream, const GatherConvArgs &a)
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     constexpr int A_TILE = BM * 36;
     constexpr int B_TILE = B_NMAJOR ? 32 * (BN + 8) : BN * 36;
-    constexpr size_t lds = (size_t)(2 * A_TILE + 2 * B_TILE) * sizeof(float);
+    constexpr size_t lds_loop = (size_t)(2 * A_TILE + 2 * B_TILE) * sizeof(float);
+    constexpr size_t lds_out = (size_t)(BM * (BN + 4) + BM) * sizeof(float);   // output staging + row offsets
+    constexpr size_t lds = lds_loop > lds_out ? lds_loop : lds_out;
     auto kern = gather_conv_kernel<WM, WN, TM, TN, B_NMAJOR>;
     static bool configured = false;  // idempotent attribute; a benign race sets it twice at worst
     if (!configured) {
