@@ -85,6 +85,7 @@ class Workload:
         self.dX = torch.empty((N, IH, IW, IC), device=dev)
         self.dW = torch.empty((OC, F, F, IC), device=dev)
         self.CW = torch.empty(F * F * IC * OC, device=dev)
+        self.Bias = torch.randn((OC,), generator=g).to(dev)
         self.stream = int(torch.cuda.current_stream().cuda_stream)
         self.streams = [self.stream]
         self.engine = pkg.engine.Engine(self.stream)
@@ -122,6 +123,12 @@ class Workload:
         self.engine.config.conv3D_winograd = 1
         self.fwd()
         self.engine.config.conv3D_winograd = 0
+
+    def fwd_bias(self):
+        # conv3D_biased through the host layer: same plan as fwd, bias added in the kernel epilogue
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.engine.conv3D_biased(self.Y.data_ptr(), self.OH, self.OW, self.X.data_ptr(), IH, IW, self.W.data_ptr(), F, F,
+                                  N, IC, OC, s, s, p, p, self.Bias.data_ptr(), N * self.OH * self.OW * OC, OC)
 
     def fwd(self):
         # whole operator through the C++ host layer: entry selection, CW scratch, kernel_remode, conv entry
@@ -225,9 +232,10 @@ def load_traffic(layer, op):
 
 def measure(pkg, torch, layer, op, steps, warmup):
     wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer), fill_units=(op == "dw_fill"))
-    step = {"fwd": wl.fwd, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino}[op]
-    kernel = {"fwd": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm, "wino": wl.wino_conv}[op]
-    if op == "fwd":
+    step = {"fwd": wl.fwd, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino}[op]
+    kernel = {"fwd": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
+              "wino": wl.wino_conv}[op]
+    if op in ("fwd", "fwd_bias"):
         wl.fwd_remode()
     if op == "wino":
         N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
@@ -261,7 +269,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
-    ap.add_argument("--op", default=None, choices=["fwd", "dx", "dw", "dw_fill", "wino"],
+    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "dx", "dw", "dw_fill", "wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="also measure every layer/op of BASELINE.json's configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -324,6 +332,8 @@ def main():
                 ops.append("wino")
             if "dw" in ops:
                 ops.append("dw_fill")
+            if layer == "c3a":
+                ops.append("fwd_bias")
             for o in ops:
                 out["layers"].append(measure(pkg, torch, layer, o, max(5, args.steps // 5), max(2, args.warmup // 3)))
                 torch.cuda.empty_cache()

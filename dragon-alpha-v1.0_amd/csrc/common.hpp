@@ -49,10 +49,22 @@ struct GatherConvArgs {
     int a_sn;                       // AH*AW*AC
     int o_off, o_sn, o_sh, o_sw;    // output strides, elements
     int b_off, b_sth, b_stw, b_sc, b_sn;
+    const float *bias;              // NULL or [CO]: added to every output row
     FastDiv d_AC, d_TW, d_OWt, d_OHWt;
 };
 
 hipError_t launch_gather_conv(hipStream_t stream, const GatherConvArgs &a, int TH, int TW, int OHt, int OWt, int N);
+
+static __device__ __forceinline__ float4 add_bias4(float4 v, const float *bias, int col)
+{
+    if (bias) {   // uniform: one bias per output channel, added as the row leaves for memory
+        const float4 b = *reinterpret_cast<const float4 *>(bias + col);
+        v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+    }
+    return v;
+}
+
+// Every forward launcher takes `bias` (NULL = none): bias[co] is added to each output row in the kernel's epilogue.
 
 // Stride-1 convolution with the input window staged once in LDS (tap_conv.hip). B must be contiguous
 // along the output channel: element (th, tw, c, co) at b_off + th*b_sth + tw*b_stw + c*b_sc + co.
@@ -60,13 +72,13 @@ hipError_t launch_gather_conv(hipStream_t stream, const GatherConvArgs &a, int T
 hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
                            int N, int AH, int AW, int AC, int OH, int OW, int CO,
                            int TH, int TW, int ph, int pw,
-                           int b_off, int b_sth, int b_stw, int b_sc);
+                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias = nullptr);
 
 // 1x1 stride-1 convolution as a streaming GEMM with the filter resident in LDS (pointwise.hip):
 // O[(n,oh,ow)][co] = sum_k A[n, oh*sh, ow*sw, k] * B(k, co), B given as [K][N] (b_kmajor) or [N][K]. Returns
 // hipErrorNotSupported (nothing launched) when the shape does not fit.
 hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, float *O, int Nimg, int AH, int AW,
-                            int OH, int OW, int sh, int sw, int K, int N, int b_kmajor);
+                            int OH, int OW, int sh, int sw, int K, int N, int b_kmajor, const float *bias = nullptr);
 
 // Backward-filter implicit GEMM with split-K over k = (n, oh, ow):
 //   dst_z[oc, fh, fw, ic] = sum_{k in slice z} deltaY[k, oc] * X[n, oh*sh - ph + fh, ow*sw - pw + fw, ic]
@@ -96,7 +108,8 @@ hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *d
 // Forward convolution for IC (stored) = 4 with the filter resident in LDS (stem_conv.hip); F is W[OC,FH,FW,4] or, with
 // f_cw, CW[FH,FW,4,OC]. Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
 hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, int f_cw, float *Y,
-                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw);
+                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw,
+                            const float *bias = nullptr);
 
 // Backward-filter of 1x1 stride-1 layers from registers (delta_w_pointwise.hip); same slice partition and outputs.
 // Returns hipErrorNotSupported (nothing launched) unless IC and OC are multiples of 64.
@@ -105,7 +118,7 @@ hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const flo
 
 hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC);
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
-                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw);
+                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias = nullptr);
 
 // Re-layout / reduction helpers.
 hipError_t launch_kernel_remode(hipStream_t s, const float *W, float *CW, int FH, int FW, int OC, int IC);

@@ -74,30 +74,31 @@ int fwd_algo()
 // Forward: Y = conv(X, filter). FILTER_W reads W[OC,FH,FW,IC]; FILTER_CW reads CW[FH,FW,IC,OC].
 int forward(const char *fn, const int64_t *streams, int length,
             const float *X, int IH, int IW, const float *F, FilterLayout layout, int FH, int FW,
-            float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+            float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+            const float *bias = nullptr)
 {
     if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
-    if (!X || !F || !Y || !aligned16(X) || !aligned16(F) || !aligned16(Y))
+    if (!X || !F || !Y || !aligned16(X) || !aligned16(F) || !aligned16(Y) || !aligned16(bias))
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
 
     if (IC == 4 && fwd_algo() != 3) {
-        hipError_t e = launch_stem_conv(stream0(streams), X, F, layout == FILTER_CW, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw);
+        hipError_t e = launch_stem_conv(stream0(streams), X, F, layout == FILTER_CW, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, bias);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
         // W[OC][IC] is [N][K]; CW[IC][OC] is [K][N]; a stride only thins the input pixels that are read
-        hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW);
+        hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW, bias);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (layout == FILTER_CW && sh == 1 && sw == 1 && fwd_algo() != 3) {
         hipError_t e = launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
-                                       0, FW * IC * OC, IC * OC, OC);
+                                       0, FW * IC * OC, IC * OC, OC, bias);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
 
     GatherConvArgs a{};
-    a.A = X; a.B = F; a.O = Y;
+    a.A = X; a.B = F; a.O = Y; a.bias = bias;
     a.CO = OC;
     a.AH = IH; a.AW = IW; a.AC = IC;
     a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
@@ -447,6 +448,35 @@ int alpha_conv3D_winograd(const int64_t *streams, int length, const float *X, in
     CHECK_PTR(Y);
     if (int e = check_dims(__func__, N, IC, OC, IH, IW, OH, OW, 3, 3, 1, 1, ph, pw)) return e;
     hipError_t e = launch_winograd(stream0(streams), X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw);
+    if (e == hipErrorNotSupported) return fail(ALPHA_CONV_EINVAL, "%s: needs OH = IH + 2*ph - 2, OW = IW + 2*pw - 2", __func__);
+    return hip_status(e, __func__);
+}
+
+// ---- forward with the bias added in the kernel epilogue -------------------------------------------------------------
+int alpha_conv3D_biased(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, int FH, int FW,
+                        const float *Bias, float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    CHECK_PTR(Bias);
+    return forward(__func__, streams, length, X, IH, IW, W, FILTER_W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, Bias);
+}
+int alpha_conv3D_GemmR_biased(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, const float *CW,
+                              int FH, int FW, const float *Bias, float *Y, int OH, int OW, int N, int IC, int OC,
+                              int sh, int sw, int ph, int pw)
+{
+    (void)W;
+    CHECK_PTR(Bias);
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, Bias);
+}
+int alpha_conv3D_winograd_biased(const int64_t *streams, int length, const float *X, int IH, int IW, const float *U,
+                                 const float *Bias, float *Y, int OH, int OW, int N, int IC, int OC, int ph, int pw)
+{
+    CHECK_STREAMS();
+    CHECK_PTR(X);
+    CHECK_PTR(U);
+    CHECK_PTR(Bias);
+    CHECK_PTR(Y);
+    if (int e = check_dims(__func__, N, IC, OC, IH, IW, OH, OW, 3, 3, 1, 1, ph, pw)) return e;
+    hipError_t e = launch_winograd(stream0(streams), X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, Bias);
     if (e == hipErrorNotSupported) return fail(ALPHA_CONV_EINVAL, "%s: needs OH = IH + 2*ph - 2, OW = IW + 2*pw - 2", __func__);
     return hip_status(e, __func__);
 }

@@ -352,6 +352,45 @@ int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *
     return rc ? fail(e, rc, "conv3D") : 0;
 }
 
+// CudaFloat32EngineBase.conv3D_biased (:1478-1560): same selection as conv3D; there the bias is a second pass
+// (linear_dual2D_row on Y after an event), here it rides in the conv kernel's epilogue, so every remode entry collapses
+// onto the GemmR form and every other entry onto the plain form.
+int alpha_engine_conv3D_biased(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W,
+                               int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                               const float *Bias, int lengthv, int width, alpha_conv_plan *plan_out)
+{
+    if (const char *why = param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw)) {
+        snprintf(e->err, sizeof(e->err), "%s: illegal size: %s", "alpha_engine_conv3D_biased", why);
+        return ALPHA_CONV_EINVAL;
+    }
+    // EngineCore.func_param_check_row(lengthv, OC_4x, OC, OC_4x): the rows of Y are the OC channels of one pixel
+    if (Bias == nullptr || (long)lengthv != (long)N * OH * OW * OC || width < 1 || width > OC) {
+        snprintf(e->err, sizeof(e->err), "alpha_engine_conv3D_biased: Bias is null, or lengthv != N*OH*OW*OC, or width not in [1, OC]");
+        return ALPHA_CONV_EINVAL;
+    }
+    BlockScope scope{e};
+    alpha_conv_plan p;
+    alpha_plan_conv3D(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, ph, pw, &p);
+    if (plan_out) *plan_out = p;
+    int64_t streams[16];
+    for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
+    int rc = 0;
+    if (p.entry == ALPHA_E_conv3D_winograd) {
+        float *U = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        if (!U) return fail(e, -1, "conv3D_biased");
+        if ((rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform");
+        rc = alpha_conv3D_winograd_biased(streams, p.streams, X, IH, IW, U, Bias, Y, OH, OW, N, IC, OC, ph, pw);
+    } else if (p.remode) {
+        float *CW = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        if (!CW) return fail(e, -1, "conv3D_biased");
+        if ((rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");
+        rc = alpha_conv3D_GemmR_biased(streams, p.streams, X, IH, IW, W, CW, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+    } else {
+        rc = alpha_conv3D_biased(streams, p.streams, X, IH, IW, W, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+    }
+    return rc ? fail(e, rc, "conv3D_biased") : 0;
+}
+
 int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, const float *X, int IH, int IW,
                                 const float *deltaY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                 alpha_conv_plan *plan_out)

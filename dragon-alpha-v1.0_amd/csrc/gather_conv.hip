@@ -215,7 +215,8 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
         const int row = idx / (BN / 4), c4 = (idx % (BN / 4)) * 4;
         const int ro = rowoff[row];
         if (ro >= 0 && n0 + c4 < CO)   // CO % 4 == 0: the four columns are valid together
-            *reinterpret_cast<float4 *>(p.O + ro + n0 + c4) = *reinterpret_cast<const float4 *>(Os + row * OS + c4);
+            *reinterpret_cast<float4 *>(p.O + ro + n0 + c4) =
+                add_bias4(*reinterpret_cast<const float4 *>(Os + row * OS + c4), p.bias, n0 + c4);
     }
 }
 

@@ -28,6 +28,7 @@ struct PointwiseArgs {
     int b_kmajor;
     int tiles;        // ceil(M / 16)
     int strided;      // 0: row = m
+    const float *bias;   // NULL or [ldn]
     int AH, AW, sh, sw;
     FastDiv d_OW, d_OHW;
 };
@@ -140,7 +141,9 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
             for (int i = 0; i < 4; i++) {
                 const int row = 4 * i + q, m = tile * 16 + row;
                 const float4 v = *reinterpret_cast<const float4 *>(Os + row * PW_OS + 4 * l16);
-                if (m < p.M) *reinterpret_cast<float4 *>(p.O + (size_t)m * ldn + n_off + 64 * jg + 4 * l16) = v;
+                if (m < p.M)
+                    *reinterpret_cast<float4 *>(p.O + (size_t)m * ldn + n_off + 64 * jg + 4 * l16) =
+                        add_bias4(v, p.bias, n_off + 64 * jg + 4 * l16);
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -177,7 +180,7 @@ static hipError_t launch_pw(hipStream_t stream, const PointwiseArgs &a, int cus)
 // more than one block A is read once per block (from L2 for the sizes this serves). Returns hipErrorNotSupported
 // (nothing launched) unless K is 64, 128, 192 or 256 and N a multiple of 64; the caller then uses another kernel.
 hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, float *O, int Nimg, int AH, int AW,
-                            int OH, int OW, int sh, int sw, int K, int N, int b_kmajor)
+                            int OH, int OW, int sh, int sw, int K, int N, int b_kmajor, const float *bias)
 {
     const long Ml = (long)Nimg * OH * OW;
     if (Ml < 1 || (K & 63) || K < 64 || K > 256 || (N & 63) || N < 64) return hipErrorNotSupported;
@@ -193,7 +196,7 @@ hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, 
     const int cus = cu_count[dev];
     PointwiseArgs a{};
     a.A = A; a.B = B; a.O = O;
-    a.M = (int)Ml; a.K = K; a.ldn = N; a.b_kmajor = b_kmajor;
+    a.M = (int)Ml; a.K = K; a.ldn = N; a.b_kmajor = b_kmajor; a.bias = bias;
     a.tiles = (a.M + 15) / 16;
     a.strided = !(sh == 1 && sw == 1 && OH == AH && OW == AW);
     a.AH = AH; a.AW = AW; a.sh = sh; a.sw = sw;

@@ -35,6 +35,7 @@ struct TapConvArgs {
     int PHt, PWt;     // AH + 2ph, AW + 2pw
     int lds_rows;     // halo rows reserved in LDS
     int b_off, b_sth, b_stw, b_sc;
+    const float *bias;   // NULL or [CO]
     FastDiv d_OW, d_OHW, d_PHt, d_PWt;
 };
 
@@ -237,7 +238,8 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
         const int pix = idx >> 4, cq = (idx & 15) * 4;
         const int m = m0 + pix;
         if (m < p.M && oc0 + cq < p.CO)
-            *reinterpret_cast<float4 *>(p.O + (size_t)m * p.CO + oc0 + cq) = *reinterpret_cast<const float4 *>(Os + pix * TC_OS + cq);
+            *reinterpret_cast<float4 *>(p.O + (size_t)m * p.CO + oc0 + cq) =
+                add_bias4(*reinterpret_cast<const float4 *>(Os + pix * TC_OS + cq), p.bias, oc0 + cq);
     }
 }
 
@@ -286,7 +288,7 @@ static hipError_t launch_tc(hipStream_t stream, const TapConvArgs &a, size_t lds
 hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
                            int N, int AH, int AW, int AC, int OH, int OW, int CO,
                            int TH, int TW, int ph, int pw,
-                           int b_off, int b_sth, int b_stw, int b_sc)
+                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias)
 {
     if (OH != AH + 2 * ph - TH + 1 || OW != AW + 2 * pw - TW + 1) return hipErrorNotSupported;
     if (AC < 32 || TH > 7 || TW > 7) return hipErrorNotSupported;
@@ -294,7 +296,7 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
     if ((long)N * (AH + 2 * ph) >= (1L << 24)) return hipErrorNotSupported;
 
     TapConvArgs a{};
-    a.A = A; a.B = B; a.O = O;
+    a.A = A; a.B = B; a.O = O; a.bias = bias;
     a.M = (int)M; a.CO = CO;
     a.AH = AH; a.AW = AW; a.AC = AC;
     a.TH = TH; a.TW = TW; a.ph = ph; a.pw = pw;

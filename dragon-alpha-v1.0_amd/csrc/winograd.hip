@@ -23,6 +23,7 @@ struct WinoArgs {
     const float *X;   // [N, IH, IW, IC]
     const float *U;   // [16][IC][OC] transformed filter
     float *Y;         // [N, OH, OW, OC]
+    const float *bias;   // NULL or [OC]
     int N, IH, IW, IC, OH, OW, OC;
     int ph, pw;
     int TR, TC;       // tile rows / columns per image: ceil(OH/2), ceil(OW/2)
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(256, 2) void winograd_f2x2_kernel(const WinoArgs p)
             const int oh = 2 * ty + dy, ow = 2 * tx + dx;
             if (oh < p.OH && ow < p.OW)
                 *reinterpret_cast<float4 *>(p.Y + (((size_t)n * p.OH + oh) * p.OW + ow) * p.OC + oc0 + cq) =
-                    *reinterpret_cast<const float4 *>(Os + px * 68 + cq);
+                    add_bias4(*reinterpret_cast<const float4 *>(Os + px * 68 + cq), p.bias, oc0 + cq);
         }
     }
 }
@@ -240,11 +241,11 @@ hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int I
 }
 
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
-                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw)
+                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias)
 {
     if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
     WinoArgs a{};
-    a.X = X; a.U = U; a.Y = Y;
+    a.X = X; a.U = U; a.Y = Y; a.bias = bias;
     a.N = N; a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC;
     a.ph = ph; a.pw = pw;
     a.TR = (OH + 1) / 2; a.TC = (OW + 1) / 2;

@@ -68,6 +68,8 @@ def _lib():
         L.alpha_engine_last_error.restype = ctypes.c_char_p
         L.alpha_engine_sync.argtypes = [_P]
         L.alpha_engine_conv3D.argtypes = [_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [ctypes.POINTER(Plan)]
+        L.alpha_engine_conv3D_biased.argtypes = ([_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [_P, _I, _I]
+                                                 + [ctypes.POINTER(Plan)])
         L.alpha_engine_dconv3D_deltaW.argtypes = [_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [ctypes.POINTER(Plan)]
         L.alpha_engine_dconv3D_deltaX.argtypes = [_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [ctypes.POINTER(Plan)]
         _bound = True
@@ -136,6 +138,12 @@ class Engine:
     def conv3D(self, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw):
         p = Plan()
         self._check(self._L.alpha_engine_conv3D(self._h, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, ctypes.byref(p)))
+        return p
+
+    def conv3D_biased(self, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, Bias, lengthv, width):
+        p = Plan()
+        self._check(self._L.alpha_engine_conv3D_biased(self._h, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw,
+                                                       Bias, lengthv, width, ctypes.byref(p)))
         return p
 
     def dconv3D_deltaW(self, deltaW, FH, FW, X, IH, IW, deltaY, OH, OW, N, IC, OC, sh, sw, ph, pw):

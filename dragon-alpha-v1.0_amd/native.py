@@ -54,6 +54,9 @@ _SIGS = {
     "alpha_dconv3D_deltaW_GemmSK_W1": "siipiipppiii",
     "alpha_winograd_filter_transform": "lppii",
     "alpha_conv3D_winograd": "sipiippiiiiiii",
+    "alpha_conv3D_biased": "sipiipiippiiiiiiiii",
+    "alpha_conv3D_GemmR_biased": "sipiippiippiiiiiiiii",
+    "alpha_conv3D_winograd_biased": "sipiipppiiiiiii",
 }
 _CT = {"s": _S, "i": _I, "p": _P, "l": _L}
 
@@ -206,6 +209,20 @@ class Cuda_conv3D:
     @staticmethod
     def conv3D_winograd(streamArray, length, X, IH, IW, U, Y, OH, OW, N, IC, OC, ph, pw):
         _call("alpha_conv3D_winograd", streamArray, length, X, IH, IW, U, Y, OH, OW, N, IC, OC, ph, pw)
+
+    # forward with the bias added in the kernel epilogue (the reference composes conv3D + linear_dual2D_row)
+    @staticmethod
+    def conv3D_biased(streamArray, length, X, IH, IW, W, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D_biased", streamArray, length, X, IH, IW, W, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_GemmR_biased(streamArray, length, X, IH, IW, W, CW, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D_GemmR_biased", streamArray, length, X, IH, IW, W, CW, FH, FW, Bias, Y, OH, OW, N, IC, OC,
+              sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_winograd_biased(streamArray, length, X, IH, IW, U, Bias, Y, OH, OW, N, IC, OC, ph, pw):
+        _call("alpha_conv3D_winograd_biased", streamArray, length, X, IH, IW, U, Bias, Y, OH, OW, N, IC, OC, ph, pw)
 
 
 class Cuda_dconv3D_deltaX:

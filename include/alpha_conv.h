@@ -266,6 +266,30 @@ int alpha_conv3D_winograd(const int64_t *streams, int length,
                           float *Y, int OH, int OW,
                           int N, int IC, int OC, int ph, int pw);
 
+/* ---- forward with the bias added in the kernel's epilogue --------------------------------------
+ * The reference has no native for this: its engine method conv3D_biased (CudaFloat32EngineBase.java:1478-1560,
+ * EngineBase.java:178-185) runs the conv3D entry and then Cuda_function.linear_dual2D_row(Y, Bias, ...) =
+ * Y[., oc] = 1*Y[., oc] + 1*Bias[oc] + 0 as a second pass over Y on its own stream. These entries give the same
+ * result (Bias has OC entries, OC the stored, x4-padded channel count) without the second pass; a maintainer binds
+ * them as new natives of Cuda_conv3D next to conv3D / conv3D_GemmR and calls them from conv3D_biased. */
+int alpha_conv3D_biased(const int64_t *streams, int length,
+                        const float *X, int IH, int IW,
+                        const float *W, int FH, int FW,
+                        const float *Bias,
+                        float *Y, int OH, int OW,
+                        int N, int IC, int OC, int sh, int sw, int ph, int pw);
+int alpha_conv3D_GemmR_biased(const int64_t *streams, int length,
+                              const float *X, int IH, int IW,
+                              const float *W, const float *CW, int FH, int FW,
+                              const float *Bias,
+                              float *Y, int OH, int OW,
+                              int N, int IC, int OC, int sh, int sw, int ph, int pw);
+int alpha_conv3D_winograd_biased(const int64_t *streams, int length,
+                                 const float *X, int IH, int IW,
+                                 const float *U, const float *Bias,
+                                 float *Y, int OH, int OW,
+                                 int N, int IC, int OC, int ph, int pw);
+
 #ifdef __cplusplus
 }
 #endif

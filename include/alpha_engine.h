@@ -94,6 +94,12 @@ int alpha_engine_sync(alpha_engine *e);
 
 int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W, int FH, int FW,
                         int N, int IC, int OC, int sh, int sw, int ph, int pw, alpha_conv_plan *plan_out);
+/* EngineBase.conv3D_biased (EngineBase.java:178-185; CudaFloat32EngineBase.java:1478-1560): the plan is conv3D's; the
+ * bias is added in the convolution kernel's epilogue instead of by a second pass over Y. lengthv and width are the
+ * reference's row-function arguments (N*OH*OW*OC and the logical OC): checked for consistency, otherwise unused. */
+int alpha_engine_conv3D_biased(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W,
+                               int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                               const float *Bias, int lengthv, int width, alpha_conv_plan *plan_out);
 int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, const float *X, int IH, int IW,
                                 const float *deltaY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                 alpha_conv_plan *plan_out);

@@ -70,6 +70,27 @@ def test_engine_runs_the_entry_java_would_pick(dev, eng, case):
     check(dev.get(dw), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "engine deltaW %s" % (case,))
 
 
+def test_engine_conv3D_biased(dev, eng):
+    N, IH, IC, OC = 8, 14, 64, 64
+    X, W, B = normal((N, IH, IH, IC), 6201), he_normal(OC, 3, 3, IC, 6202), normal((OC,), 6203)
+    want = O.conv3D_f64(X, W, 1, 1, 1, 1) + B.astype(np.float64)[None, None, None, :]
+    x, w, b = dev.put(X), dev.put(W), dev.put(B)
+    for wino in (0, 1):
+        eng.config.conv3D_winograd = wino
+        try:
+            y = dev.empty(N, IH, IH, OC, fill=float("nan"))
+            p = eng.conv3D_biased(y.data_ptr(), IH, IH, x.data_ptr(), IH, IH, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1,
+                                  b.data_ptr(), N * IH * IH * OC, OC)
+            eng.sync()
+        finally:
+            eng.config.conv3D_winograd = 0
+        assert p.entry_name == ("conv3D_winograd" if wino else "conv3D_GemmR_texture")
+        check(dev.get(y), want, "engine conv3D_biased (winograd %d)" % wino)
+    with pytest.raises(pkg.AlphaConvError, match="lengthv"):
+        eng.conv3D_biased(y.data_ptr(), IH, IH, x.data_ptr(), IH, IH, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1,
+                          b.data_ptr(), N * IH * IH * OC - 4, OC)
+
+
 def test_engine_deltaW_with_fill_option(dev):
     """A larger split-K factor changes the summation order, not the result beyond the parity bar."""
     N, IH, IC, OC = 32, 14, 128, 128

@@ -334,6 +334,43 @@ def test_pointwise_kernel_strided(dev, shape):
         check(_run_fwd(dev, entry, X, W, sh, sw, 0, 0), want, "%s strided 1x1 %s" % (entry, shape))
 
 
+BIAS_SHAPES = [
+    # N, IH, IW, IC, OC, F, s, p: one layer per forward kernel (the bias rides in each kernel's epilogue)
+    (4, 14, 14, 64, 64, 3, 1, 1),      # LDS-halo kernel
+    (4, 9, 9, 64, 128, 1, 1, 0),       # streaming 1x1 GEMM
+    (4, 16, 16, 4, 64, 7, 2, 3),       # stem kernel
+    (4, 13, 11, 32, 48, 3, 2, 1),      # generic kernel (strided)
+    (4, 6, 5, 12, 20, 3, 1, 1),        # generic kernel, ragged channels
+]
+
+
+@pytest.mark.parametrize("shape", BIAS_SHAPES)
+def test_forward_with_bias_in_the_epilogue(dev, shape):
+    """Y = conv(X, W) + Bias[oc] (the reference: conv3D then linear_dual2D_row(Y, Bias), CudaFloat32EngineBase.java:1548-1557)."""
+    N, IH, IW, IC, OC, F_, s_, p_ = shape
+    OH, OW = out_dim(IH, IW, F_, F_, s_, s_, p_, p_)
+    X, W, B = normal((N, IH, IW, IC), 2201), he_normal(OC, F_, F_, IC, 2202), normal((OC,), 2203)
+    want = O.conv3D_f64(X, W, s_, s_, p_, p_) + B.astype(np.float64)[None, None, None, :]
+    x, w, b = dev.put(X), dev.put(W), dev.put(B)
+    cw = dev.empty(F_ * F_ * IC * OC, fill=float("nan"))
+    C3.kernel_remode(dev.stream, w.data_ptr(), cw.data_ptr(), F_, F_, OC, IC)
+    y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    C3.conv3D_biased(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), F_, F_, b.data_ptr(), y.data_ptr(), OH, OW, N, IC, OC,
+                     s_, s_, p_, p_)
+    check(dev.get(y), want, "conv3D_biased %s" % (shape,))
+    y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    C3.conv3D_GemmR_biased(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), cw.data_ptr(), F_, F_, b.data_ptr(), y.data_ptr(),
+                           OH, OW, N, IC, OC, s_, s_, p_, p_)
+    check(dev.get(y), want, "conv3D_GemmR_biased %s" % (shape,))
+    if F_ == 3 and s_ == 1:
+        U = dev.empty(16 * IC * OC, fill=float("nan"))
+        C3.winograd_filter_transform(dev.stream, w.data_ptr(), U.data_ptr(), IC, OC)
+        y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+        C3.conv3D_winograd_biased(dev.streams, 1, x.data_ptr(), IH, IW, U.data_ptr(), b.data_ptr(), y.data_ptr(), OH, OW, N, IC, OC,
+                                  p_, p_)
+        check(dev.get(y), want, "conv3D_winograd_biased %s" % (shape,))
+
+
 KS_SHAPES = [
     # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw
     (4, 16, 16, 64, 128, 3, 3, 2, 2, 1, 1),
