@@ -130,6 +130,12 @@ class Workload:
         self.engine.conv3D_biased(self.Y.data_ptr(), self.OH, self.OW, self.X.data_ptr(), IH, IW, self.W.data_ptr(), F, F,
                                   N, IC, OC, s, s, p, p, self.Bias.data_ptr(), N * self.OH * self.OW * OC, OC)
 
+    def fwd_cached(self):
+        # as fwd, with this build's option that keeps the re-laid-out filter between calls (inference, or training with
+        # the weight update reported to the engine)
+        self.engine.config.cache_filter_transforms = 1
+        self.fwd()
+
     def fwd(self):
         # whole operator through the C++ host layer: entry selection, CW scratch, kernel_remode, conv entry
         N, IH, IW, IC, OC, F, s, p = self.dims
@@ -232,10 +238,10 @@ def load_traffic(layer, op):
 
 def measure(pkg, torch, layer, op, steps, warmup):
     wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer), fill_units=(op == "dw_fill"))
-    step = {"fwd": wl.fwd, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino}[op]
-    kernel = {"fwd": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
+    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd_cached, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino}[op]
+    kernel = {"fwd": wl.fwd_conv, "fwd_cached": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
               "wino": wl.wino_conv}[op]
-    if op in ("fwd", "fwd_bias"):
+    if op in ("fwd", "fwd_bias", "fwd_cached"):
         wl.fwd_remode()
     if op == "wino":
         N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
@@ -269,7 +275,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
-    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "dx", "dw", "dw_fill", "wino"],
+    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "dx", "dw", "dw_fill", "wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="also measure every layer/op of BASELINE.json's configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -333,7 +339,7 @@ def main():
             if "dw" in ops:
                 ops.append("dw_fill")
             if layer == "c3a":
-                ops.append("fwd_bias")
+                ops += ["fwd_bias", "fwd_cached"]
             for o in ops:
                 out["layers"].append(measure(pkg, torch, layer, o, max(5, args.steps // 5), max(2, args.warmup // 3)))
                 torch.cuda.empty_cache()

@@ -14,6 +14,7 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <tuple>
 #include <mutex>
 #include <vector>
 
@@ -64,6 +65,7 @@ void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
     c->deltaX_ks_V2_Q = 1.1f;
     c->conv3D_winograd = 0;
     c->deltaW_SK_fillUnits = 0;
+    c->cache_filter_transforms = 0;
 }
 
 // ---- forward: CudaFloat32EngineBase.conv3D (:1355-1474) ----------------------------------------------
@@ -215,6 +217,16 @@ struct alpha_engine {
     // apart (the Java engine, which spreads work over several streams, waits for the operator's Syncer instead).
     std::multimap<size_t, void *> free_blocks;
     std::vector<std::pair<size_t, void *>> in_flight;     // blocks of the operator being enqueued
+    // Transformed filters kept between calls (cfg.cache_filter_transforms): key -> (bytes, block)
+    struct FilterKey {
+        const void *W;
+        int kind, FH, FW, IC, OC, sh, sw;   // kind 0: CW of kernel_remode, 1: Winograd U, 2: kernel-split CW (ks_remodev2)
+        bool operator<(const FilterKey &o) const
+        {
+            return std::tie(W, kind, FH, FW, IC, OC, sh, sw) < std::tie(o.W, o.kind, o.FH, o.FW, o.IC, o.OC, o.sh, o.sw);
+        }
+    };
+    std::map<FilterKey, std::pair<size_t, void *>> filter_cache;
     char err[256];
 };
 
@@ -247,6 +259,52 @@ static void *take_block(alpha_engine *e, size_t bytes)
     return p;
 }
 
+// Scratch for a transformed filter. Without the cache it is an ordinary pool block and *fresh is always set (the caller
+// runs the transform); with it, the block of an earlier call with the same filter address and geometry is returned with
+// *fresh = false, and a new block stays out of the pool until alpha_engine_filter_changed() names its filter.
+static float *filter_block(alpha_engine *e, int kind, const float *W, int FH, int FW, int IC, int OC, int sh, int sw,
+                           size_t bytes, bool *fresh)
+{
+    *fresh = true;
+    if (!e->cfg.cache_filter_transforms) return static_cast<float *>(take_block(e, bytes));
+    const alpha_engine::FilterKey key{W, kind, FH, FW, IC, OC, sh, sw};
+    {
+        std::lock_guard<std::mutex> g(e->mu);
+        auto it = e->filter_cache.find(key);
+        if (it != e->filter_cache.end()) {
+            *fresh = false;
+            return static_cast<float *>(it->second.second);
+        }
+    }
+    void *p = take_block(e, bytes);
+    if (!p) return nullptr;
+    std::lock_guard<std::mutex> g(e->mu);
+    size_t sz = bytes;
+    for (auto it = e->in_flight.begin(); it != e->in_flight.end(); ++it)
+        if (it->second == p) {   // keep it: it is no longer the operator's to give back
+            sz = it->first;
+            e->in_flight.erase(it);
+            break;
+        }
+    e->filter_cache[key] = std::make_pair(sz, p);
+    return static_cast<float *>(p);
+}
+
+void alpha_engine_filter_changed(alpha_engine *e, const float *W)
+{
+    std::lock_guard<std::mutex> g(e->mu);
+    for (auto it = e->filter_cache.begin(); it != e->filter_cache.end();) {
+        if (W == nullptr || it->first.W == W) {
+            // kernels already enqueued may still read the block; whoever takes it from the pool next writes to it on
+            // the same stream, after them
+            e->free_blocks.emplace(it->second.first, it->second.second);
+            it = e->filter_cache.erase(it);
+        } else {
+            ++it;
+        }
+    }
+}
+
 alpha_engine *alpha_engine_create(int64_t stream)
 {
     alpha_engine *e = new alpha_engine();
@@ -273,6 +331,7 @@ void alpha_engine_destroy(alpha_engine *e)
     if (!e) return;
     alpha_engine_sync(e);
     for (auto &b : e->free_blocks) (void)hipFree(b.second);
+    for (auto &b : e->filter_cache) (void)hipFree(b.second.second);
     delete e;
 }
 
@@ -318,14 +377,16 @@ int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *
     for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
     int rc = 0;
     if (p.entry == ALPHA_E_conv3D_winograd) {
-        float *U = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        bool fresh;
+        float *U = filter_block(e, 1, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!U) return fail(e, -1, "conv3D");
-        if ((rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform");
+        if (fresh && (rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform");
         rc = alpha_conv3D_winograd(streams, p.streams, X, IH, IW, U, Y, OH, OW, N, IC, OC, ph, pw);
     } else if (p.remode) {
-        float *CW = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        bool fresh;
+        float *CW = filter_block(e, 0, W, FH, FW, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!CW) return fail(e, -1, "conv3D");
-        if ((rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");
+        if (fresh && (rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");
         switch (p.entry) {
         case ALPHA_E_conv3D_GemmR_W1: rc = alpha_conv3D_GemmR_W1(streams, p.streams, X, IH, IW, W, CW, Y, N, IC, OC); break;
         case ALPHA_E_conv3D_GemmV2R:
@@ -376,14 +437,16 @@ int alpha_engine_conv3D_biased(alpha_engine *e, float *Y, int OH, int OW, const 
     for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
     int rc = 0;
     if (p.entry == ALPHA_E_conv3D_winograd) {
-        float *U = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        bool fresh;
+        float *U = filter_block(e, 1, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!U) return fail(e, -1, "conv3D_biased");
-        if ((rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform");
+        if (fresh && (rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform");
         rc = alpha_conv3D_winograd_biased(streams, p.streams, X, IH, IW, U, Bias, Y, OH, OW, N, IC, OC, ph, pw);
     } else if (p.remode) {
-        float *CW = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        bool fresh;
+        float *CW = filter_block(e, 0, W, FH, FW, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!CW) return fail(e, -1, "conv3D_biased");
-        if ((rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");
+        if (fresh && (rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");
         rc = alpha_conv3D_GemmR_biased(streams, p.streams, X, IH, IW, W, CW, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
     } else {
         rc = alpha_conv3D_biased(streams, p.streams, X, IH, IW, W, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
@@ -465,9 +528,10 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
         break;
     default: {
         const int CFH = (FH + sh - 1) / sh, CFW = (FW + sw - 1) / sw;
-        float *CW = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
+        bool fresh;
+        float *CW = filter_block(e, 2, W, FH, FW, IC, OC, sh, sw, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!CW) return fail(e, -1, "dconv3D_deltaX");
-        if ((rc = alpha_ks_remodev2(streams[0], W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw))) return fail(e, rc, "ks_remodev2");
+        if (fresh && (rc = alpha_ks_remodev2(streams[0], W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw))) return fail(e, rc, "ks_remodev2");
         switch (p.entry) {
         case ALPHA_E_dconv3D_deltaX_ksV2_Ims2R:
             rc = alpha_dconv3D_deltaX_ksV2_Ims2R(p.useTexture, streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);

@@ -24,7 +24,8 @@ class Config(ctypes.Structure):
                 ("deltaW_SK_V2_Q", ctypes.c_float),
                 ("deltaX_s1_useTexture", ctypes.c_int), ("deltaX_ks_useTexture", ctypes.c_int),
                 ("deltaX_s1_V2_Q", ctypes.c_float), ("deltaX_ks_V2_Q", ctypes.c_float),
-                ("conv3D_winograd", ctypes.c_int), ("deltaW_SK_fillUnits", ctypes.c_int)]
+                ("conv3D_winograd", ctypes.c_int), ("deltaW_SK_fillUnits", ctypes.c_int),
+                ("cache_filter_transforms", ctypes.c_int)]
 
 
 class Plan(ctypes.Structure):
@@ -67,6 +68,8 @@ def _lib():
         L.alpha_engine_last_error.argtypes = [_P]
         L.alpha_engine_last_error.restype = ctypes.c_char_p
         L.alpha_engine_sync.argtypes = [_P]
+        L.alpha_engine_filter_changed.argtypes = [_P, _P]
+        L.alpha_engine_filter_changed.restype = None
         L.alpha_engine_conv3D.argtypes = [_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [ctypes.POINTER(Plan)]
         L.alpha_engine_conv3D_biased.argtypes = ([_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [_P, _I, _I]
                                                  + [ctypes.POINTER(Plan)])
@@ -139,6 +142,9 @@ class Engine:
         p = Plan()
         self._check(self._L.alpha_engine_conv3D(self._h, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, ctypes.byref(p)))
         return p
+
+    def filter_changed(self, W=None):
+        self._L.alpha_engine_filter_changed(self._h, W)
 
     def conv3D_biased(self, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, Bias, lengthv, width):
         p = Plan()

@@ -35,6 +35,10 @@ typedef struct alpha_engine_config {
     int deltaW_SK_fillUnits;      /* this build only: when > 0, the split-K factor is raised (never lowered) until the launch has two
                                      workgroups (one when output rows are wider than 36 pixels) for each of this many compute units,
                                      slices staying >= 256 pixels; default 0 = the reference's GridZ exactly */
+    int cache_filter_transforms;  /* this build only: 1 = keep kernel_remode / ks_remodev2 / Winograd filter transforms between calls,
+                                     keyed by the filter's address and geometry; the caller reports weight updates with
+                                     alpha_engine_filter_changed(). Default 0: re-transform on every call like the reference
+                                     (CudaFloat32EngineBase.java:1373-1380, 1879-1889) */
 } alpha_engine_config;
 
 /* Native entry chosen by a plan; names are the Java native method names. */
@@ -91,6 +95,8 @@ void alpha_engine_destroy(alpha_engine *e);
 alpha_engine_config *alpha_engine_get_config(alpha_engine *e);
 const char *alpha_engine_last_error(alpha_engine *e);
 int alpha_engine_sync(alpha_engine *e);
+/* With cache_filter_transforms: the values at W (NULL = every filter) changed; their cached transforms are dropped. */
+void alpha_engine_filter_changed(alpha_engine *e, const float *W);
 
 int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W, int FH, int FW,
                         int N, int IC, int OC, int sh, int sw, int ph, int pw, alpha_conv_plan *plan_out);

@@ -91,6 +91,45 @@ def test_engine_conv3D_biased(dev, eng):
                           b.data_ptr(), N * IH * IH * OC - 4, OC)
 
 
+def test_engine_filter_transform_cache(dev):
+    """With cache_filter_transforms the re-layout runs once per filter; a weight update must be reported."""
+    N, IH, IC, OC = 8, 12, 64, 64
+    X, W1, W2 = normal((N, IH, IH, IC), 6301), he_normal(OC, 3, 3, IC, 6302), he_normal(OC, 3, 3, IC, 6303)
+    dY = normal((N, 6, 6, OC), 6304)
+    x, w, dy = dev.put(X), dev.put(W1), dev.put(dY)
+    e = pkg.engine.Engine(dev.stream)
+    try:
+        e.config.cache_filter_transforms = 1
+        for wino in (0, 1):
+            e.config.conv3D_winograd = wino
+            w.copy_(dev.put(W1))
+            e.filter_changed(w.data_ptr())
+            y = dev.empty(N, IH, IH, OC, fill=float("nan"))
+            for _ in range(2):   # second call: transform taken from the cache
+                e.conv3D(y.data_ptr(), IH, IH, x.data_ptr(), IH, IH, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1)
+            e.sync()
+            check(dev.get(y), O.conv3D_f64(X, W1, 1, 1, 1, 1), "cached transform, first weights (winograd %d)" % wino)
+            w.copy_(dev.put(W2))              # optimizer step: same address, new values
+            e.conv3D(y.data_ptr(), IH, IH, x.data_ptr(), IH, IH, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1)
+            e.sync()
+            stale = dev.get(y)
+            check(stale, O.conv3D_f64(X, W1, 1, 1, 1, 1), "unreported update keeps the old transform (winograd %d)" % wino)
+            e.filter_changed(w.data_ptr())
+            e.conv3D(y.data_ptr(), IH, IH, x.data_ptr(), IH, IH, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1)
+            e.sync()
+            check(dev.get(y), O.conv3D_f64(X, W2, 1, 1, 1, 1), "after filter_changed (winograd %d)" % wino)
+        # kernel-split backward-data shares the cache (another kind under the same address)
+        e.config.conv3D_winograd = 0
+        dx = dev.empty(N, IH, IH, IC, fill=float("nan"))
+        for _ in range(2):
+            p = e.dconv3D_deltaX(dx.data_ptr(), IH, IH, dy.data_ptr(), 6, 6, w.data_ptr(), 3, 3, N, IC, OC, 2, 2, 1, 1)
+        e.sync()
+        assert p.remode == 1
+        check(dev.get(dx), O.deltaX_f64(dY, W2, IH, IH, 2, 2, 1, 1), "cached kernel-split filter")
+    finally:
+        e.close()
+
+
 def test_engine_deltaW_with_fill_option(dev):
     """A larger split-K factor changes the summation order, not the result beyond the parity bar."""
     N, IH, IC, OC = 32, 14, 128, 128
