@@ -102,7 +102,7 @@ hipError_t launch_deltaW(hipStream_t stream, const DeltaWArgs &a);
 // launch_deltaW. Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
 hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
                               int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,
-                              int sh, int sw, int ph, int pw, int GK_slice, int GZ);
+                              int sh, int sw, int ph, int pw, int GK_slice, int GZ, float *dB = nullptr, float *dB_buf = nullptr);
 
 // Winograd F(2x2,3x3) forward (winograd.hip): U = transformed filter [16][IC][OC].
 // Forward convolution for IC (stored) = 4 with the filter resident in LDS (stem_conv.hip); F is W[OC,FH,FW,4] or, with
@@ -114,7 +114,7 @@ hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, 
 // Backward-filter of 1x1 stride-1 layers from registers (delta_w_pointwise.hip); same slice partition and outputs.
 // Returns hipErrorNotSupported (nothing launched) unless IC and OC are multiples of 64.
 hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
-                                   int GK, int IC, int OC, int GK_slice, int GZ);
+                                   int GK, int IC, int OC, int GK_slice, int GZ, float *dB = nullptr, float *dB_buf = nullptr);
 
 hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC);
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
@@ -125,5 +125,7 @@ hipError_t launch_kernel_remode(hipStream_t s, const float *W, float *CW, int FH
 hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, int FW, float *CW,
                             int mCFH, int mCFW, int OC, int IC, int sh, int sw);
 hipError_t launch_buf_summary(hipStream_t s, const float *buf, float *dW, int part, int sizeW);
+// Column sums of deltaY[GK][OC] per K slice (bias gradient), same slice partition and destinations as backward-filter.
+hipError_t launch_col_sum(hipStream_t s, const float *dY, float *dB, float *dB_buf, int OC, int GK, int GK_slice, int GZ);
 
 }  // namespace alpha

@@ -195,13 +195,15 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
 
 int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
            const float *X, int IH, int IW, const float *dY, int OH, int OW,
-           float *dW, float *dW_buf, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+           float *dW, float *dW_buf, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+           float *dB = nullptr, float *dB_buf = nullptr)
 {
     if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
-    if (!X || !dY || !dW || !aligned16(X) || !aligned16(dY) || !aligned16(dW))
+    if (!X || !dY || !dW || !aligned16(X) || !aligned16(dY) || !aligned16(dW) || !aligned16(dB) || !aligned16(dB_buf))
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (GridZ < 1) return fail(ALPHA_CONV_EINVAL, "%s: GridZ must be >= 1", fn);
     if (GridZ > 1 && (!dW_buf || !aligned16(dW_buf))) return fail(ALPHA_CONV_EINVAL, "%s: deltaW_buf is null or misaligned", fn);
+    if (dB && GridZ > 1 && !dB_buf) return fail(ALPHA_CONV_EINVAL, "%s: deltaB_buf is null", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
 
     DeltaWArgs a{};
@@ -213,14 +215,17 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     a.GZ = GridZ;
     a.GK_slice = (a.GK / GridZ) >> 3 << 3;
     if (fwd_algo() != 3 && FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0) {
-        hipError_t e = launch_deltaW_pointwise(stream0(streams), X, dY, dW, dW_buf, a.GK, IC, OC, a.GK_slice, GridZ);
+        hipError_t e = launch_deltaW_pointwise(stream0(streams), X, dY, dW, dW_buf, a.GK, IC, OC, a.GK_slice, GridZ, dB, dB_buf);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (fwd_algo() != 3) {
         hipError_t e = launch_deltaW_rows(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
-                                          a.GK_slice, GridZ);
+                                          a.GK_slice, GridZ, dB, dB_buf);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
+    // the generic kernel has no bias-gradient path: the column sums of deltaY get a pass of their own
+    if (dB)
+        if (int e = hip_status(launch_col_sum(stream0(streams), dY, dB, dB_buf, OC, a.GK, a.GK_slice, GridZ), fn)) return e;
     return hip_status(launch_deltaW(stream0(streams), a), fn);
 }
 
@@ -450,6 +455,17 @@ int alpha_conv3D_winograd(const int64_t *streams, int length, const float *X, in
     hipError_t e = launch_winograd(stream0(streams), X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw);
     if (e == hipErrorNotSupported) return fail(ALPHA_CONV_EINVAL, "%s: needs OH = IH + 2*ph - 2, OW = IW + 2*pw - 2", __func__);
     return hip_status(e, __func__);
+}
+
+// ---- backward-filter with the bias gradient (column sums of deltaY) from the same pass over deltaY -------------------
+int alpha_dconv3D_deltaW_GemmSK_deltaB(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
+                                       const float *deltaY, int OH, int OW, float *deltaW, float *deltaW_buf,
+                                       float *deltaB, float *deltaB_buf, int FH, int FW, int N, int IC, int OC,
+                                       int sh, int sw, int ph, int pw)
+{
+    CHECK_PTR(deltaB);
+    return deltaW_impl(__func__, streams, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC,
+                       sh, sw, ph, pw, deltaB, deltaB_buf);
 }
 
 // ---- forward with the bias added in the kernel epilogue -------------------------------------------------------------

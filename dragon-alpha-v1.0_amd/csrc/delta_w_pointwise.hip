@@ -25,6 +25,8 @@ struct DwPointwiseArgs {
     const float *dY;
     float *dW;
     float *dW_buf;
+    float *dB;       // NULL, or the bias gradient (column sums of deltaY): slice z writes to dB (z = 0)
+    float *dB_buf;   // or dB_buf[z-1][OC]
     int IC, OC;
     int GK, GK_slice, GZ;
     int tiles, icb_count;   // 64 x 64 output blocks: tiles = (OC/64) * (IC/64), block index = ocb * icb_count + icb
@@ -61,6 +63,8 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
     const float *py = p.dY + (size_t)q * p.OC + ocb * 64 + 4 * l16;
     const float *px = p.X + (size_t)q * p.IC + icb * 64 + 4 * l16;
     floatx4 ya[DWP_D], xa[DWP_D];
+    const bool do_bias = p.dB != nullptr && live && icb == 0;   // one wavefront set per block row of deltaW
+    floatx4 bsum = floatx4{0.f, 0.f, 0.f, 0.f};
     auto load = [&](int d, int g) {   // g is clamped by the caller to a group of this part
         ya[d] = *reinterpret_cast<const floatx4 *>(py + (size_t)g * 4 * p.OC);
         xa[d] = *reinterpret_cast<const floatx4 *>(px + (size_t)g * 4 * p.IC);
@@ -77,11 +81,24 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
 #pragma unroll
                         for (int j = 0; j < 4; j++)
                             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ya[d][i], xa[d][j], acc[i][j], 0, 0, 0);
+                    if (do_bias) bsum += ya[d];
                 }
                 load(d, min(g + d + DWP_D, g1 - 1));
             }
         }
     }
+
+    // ---- bias gradient: lanes q = 0..3 hold different pixels of the same 4 channels (wavefront shuffles), the parts
+    // follow through LDS below ---------------------------------------------------------------------------------------
+    if (do_bias) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            bsum[i] += __shfl_xor(bsum[i], 16);
+            bsum[i] += __shfl_xor(bsum[i], 32);
+        }
+    }
+    floatx4 *bred = reinterpret_cast<floatx4 *>(smem) + (size_t)(KSPLIT - 1) * TPW * 16 * 64;   // [KSPLIT-1][TPW][16 lanes]
+    if (do_bias && kpart > 0 && q == 0) bred[((kpart - 1) * TPW + tw) * 16 + l16] = bsum;
 
     // ---- sum the parts in the order 0, 1, 2, ... and store ------------------------------------------------------
     floatx4 *red = reinterpret_cast<floatx4 *>(smem);
@@ -101,6 +118,11 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
                     const floatx4 v = red[(((part - 1) * TPW + tw) * 16 + i * 4 + j) * 64 + lane];
                     acc[i][j] += v;
                 }
+        if (do_bias && q == 0) {
+            for (int part = 1; part < KSPLIT; part++) bsum += bred[((part - 1) * TPW + tw) * 16 + l16];
+            float *bdst = (z == 0) ? p.dB : p.dB_buf + (size_t)(z - 1) * p.OC;
+            *reinterpret_cast<float4 *>(bdst + ocb * 64 + 4 * l16) = make_float4(bsum[0], bsum[1], bsum[2], bsum[3]);
+        }
         float *dst = (z == 0) ? p.dW : p.dW_buf + (size_t)(z - 1) * p.OC * p.IC;
         // acc[i][j][r] = deltaW[oc = 64 ocb + 4 (4q + r) + i][ic = 64 icb + 4 l16 + j]
 #pragma unroll
@@ -117,7 +139,7 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
 // Returns hipErrorNotSupported (nothing launched) unless IC and OC are multiples of 64; the caller then uses another
 // kernel.
 hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
-                                   int GK, int IC, int OC, int GK_slice, int GZ)
+                                   int GK, int IC, int OC, int GK_slice, int GZ, float *dB, float *dB_buf)
 {
     if ((IC & 63) || (OC & 63) || IC < 64 || OC < 64 || (GK & 3) || (GK_slice & 3) || GK < 4) return hipErrorNotSupported;
     if ((size_t)GK * (size_t)(IC > OC ? IC : OC) >= (1ull << 31)) return hipErrorNotSupported;
@@ -130,7 +152,7 @@ hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const flo
         cu_count[dev] = n;
     }
     DwPointwiseArgs a{};
-    a.X = X; a.dY = dY; a.dW = dW; a.dW_buf = dW_buf;
+    a.X = X; a.dY = dY; a.dW = dW; a.dW_buf = dW_buf; a.dB = dB; a.dB_buf = dB_buf;
     a.IC = IC; a.OC = OC; a.GK = GK; a.GK_slice = GK_slice; a.GZ = GZ;
     a.icb_count = IC / 64;
     a.tiles = (OC / 64) * a.icb_count;
@@ -138,7 +160,7 @@ hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const flo
     a.TPW = 1;
     for (int tpw = 8; tpw > 1; tpw >>= 1)
         if (tpw <= a.tiles && (long)((a.tiles + tpw - 1) / tpw) * GZ >= cu_count[dev]) { a.TPW = tpw; break; }
-    const size_t lds = (size_t)(8 / a.TPW - 1) * a.TPW * 16 * 64 * sizeof(floatx4) + 16;
+    const size_t lds = (size_t)(8 / a.TPW - 1) * a.TPW * (16 * 64 + 16) * sizeof(floatx4) + 16;   // accumulators + bias sums of the parts
     static size_t configured = 0;
     if (lds > configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(delta_w_pointwise_kernel),

@@ -30,6 +30,8 @@ struct DwRowsArgs {
     const float *dY;
     float *dW;
     float *dW_buf;
+    float *dB;        // NULL, or the bias gradient: slice z writes sum over its pixels of deltaY[., oc] to dB (z = 0)
+    float *dB_buf;    // or dB_buf[z-1][OC]
     int N, IH, IW, IC, OH, OW, OC;
     int ph, pw;
     int GK, GK_slice, GZ;
@@ -68,6 +70,9 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
     const int k_end = (z != p.GZ - 1) ? k_start + p.GK_slice : p.GK;
     float *dst = (z == 0) ? p.dW : p.dW_buf + (size_t)(z - 1) * p.OC * (FH * FW) * p.IC;
 
+    constexpr int BG = 64 / OCB;             // lane groups of a wavefront when lanes run over the OCB channels
+    const bool do_bias = p.dB != nullptr && blockIdx.x == 0;
+    float bsum = 0.f;
     floatx4 acc[FH][FW][OCT];
 #pragma unroll
     for (int a = 0; a < FH; a++)
@@ -187,6 +192,17 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
                 if (same_image) load_x(n, oh0 + R + FH - 1, R);   // the R new padded rows of the next chunk
             }
 
+            // ---- bias gradient: column sums of the staged deltaY chunk (its masked pixels are zeros). Wavefront w adds
+            // pixels [16w, 16w+16) in a fixed order; only the workgroups of the first input-channel block do it. --------
+            if (do_bias) {
+                const float *yc = Ybuf + (it & 1) * ybuf_floats + (lane & (OCB - 1));
+#pragma unroll
+                for (int j = 0; j < 16 / BG; j++) {
+                    const int px = 16 * w + BG * j + (lane / OCB);
+                    if (px < p.steps2 * 4) bsum += yc[px * YS];
+                }
+            }
+
             // ---- multiply this chunk: pixels in groups of 4 (lane group q takes pixel 4*k4 + q of the chunk) --------
             const float *yb = Ybuf + (it & 1) * ybuf_floats + q * YS + l16;
             const float *xb = Xring + q * DWR_XS + 16 * w + l16;
@@ -273,6 +289,19 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
         }
     }
 
+    if (do_bias) {
+        // lanes of a wavefront that share a channel (wavefront shuffles), then the four wavefronts through LDS in order
+        if (BG >= 2) bsum += __shfl_xor(bsum, 32);
+        if (BG >= 4) bsum += __shfl_xor(bsum, 16);
+        __syncthreads();   // the staging buffers are free
+        if (lane < OCB) smem[w * OCB + lane] = bsum;
+        __syncthreads();
+        if (t < OCB && oc0 + t < p.OC) {
+            float *bdst = (z == 0) ? p.dB : p.dB_buf + (size_t)(z - 1) * p.OC;
+            bdst[oc0 + t] = ((smem[t] + smem[OCB + t]) + smem[2 * OCB + t]) + smem[3 * OCB + t];
+        }
+    }
+
     // ---- store: lane holds input channel ic0 + 16w + l16 and output channels 16c + 4q + r --------------------------
     const int ic = ic0 + 16 * w + l16;
 #pragma unroll
@@ -323,13 +352,13 @@ static hipError_t launch_dwr(hipStream_t stream, DwRowsArgs a)
 // Returns hipErrorNotSupported (nothing launched) when the layer does not fit; the caller then uses the generic kernel.
 hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
                               int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,
-                              int sh, int sw, int ph, int pw, int GK_slice, int GZ)
+                              int sh, int sw, int ph, int pw, int GK_slice, int GZ, float *dB, float *dB_buf)
 {
     if (sh != 1 || sw != 1) return hipErrorNotSupported;
     if (OH != IH + 2 * ph - FH + 1 || OW != IW + 2 * pw - FW + 1) return hipErrorNotSupported;
     if (IC < 16 || OC < 16) return hipErrorNotSupported;
     DwRowsArgs a{};
-    a.X = X; a.dY = dY; a.dW = dW; a.dW_buf = dW_buf;
+    a.X = X; a.dY = dY; a.dW = dW; a.dW_buf = dW_buf; a.dB = dB; a.dB_buf = dB_buf;
     a.N = N; a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC;
     a.ph = ph; a.pw = pw;
     a.GK = N * OH * OW; a.GK_slice = GK_slice; a.GZ = GZ;

@@ -495,6 +495,40 @@ int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, 
     return rc ? fail(e, rc, "buf_summary") : 0;
 }
 
+// Backward-filter and bias gradient in one operator: nn/unit/simple/Conv3D.java:150-162 calls eg.dconv3D_deltaW and then
+// eg.field_sum(deltaY, OC); here the column sums ride in the backward-filter kernel (one pass over deltaY) and both
+// results are finished by the same Kahan buf_summary.
+int alpha_engine_dconv3D_deltaW_deltaB(alpha_engine *e, float *deltaW, float *deltaB, int FH, int FW, const float *X, int IH, int IW,
+                                       const float *deltaY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                       alpha_conv_plan *plan_out)
+{
+    if (const char *why = param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw)) {
+        snprintf(e->err, sizeof(e->err), "%s: illegal size: %s", "alpha_engine_dconv3D_deltaW_deltaB", why);
+        return ALPHA_CONV_EINVAL;
+    }
+    BlockScope scope{e};
+    alpha_conv_plan p;
+    alpha_plan_deltaW(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    if (plan_out) *plan_out = p;
+    int64_t streams[16];
+    for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
+    const size_t sizeW = (size_t)OC * FH * FW * IC;
+    float *buf = nullptr, *bbuf = nullptr;
+    if (p.GridZ > 1) {
+        buf = static_cast<float *>(take_block(e, (sizeW + OC) * (p.GridZ - 1) * sizeof(float)));
+        if (!buf) return fail(e, -1, "dconv3D_deltaW_deltaB");
+        bbuf = buf + sizeW * (p.GridZ - 1);
+    }
+    int rc = alpha_dconv3D_deltaW_GemmSK_deltaB(streams, p.streams, p.GridZ, X, IH, IW, deltaY, OH, OW, deltaW, buf, deltaB, bbuf,
+                                                FH, FW, N, IC, OC, sh, sw, ph, pw);
+    if (rc) return fail(e, rc, "dconv3D_deltaW_deltaB");
+    if (p.GridZ > 1) {
+        if ((rc = alpha_buf_summary(streams[0], buf, deltaW, p.GridZ - 1, (int)sizeW))) return fail(e, rc, "buf_summary");
+        if ((rc = alpha_buf_summary(streams[0], bbuf, deltaB, p.GridZ - 1, OC))) return fail(e, rc, "buf_summary");
+    }
+    return 0;
+}
+
 int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
                                 const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                 alpha_conv_plan *plan_out)

@@ -134,4 +134,39 @@ hipError_t launch_buf_summary(hipStream_t s, const float *buf, float *dW, int pa
     return hipGetLastError();
 }
 
+// Bias gradient without a backward-filter kernel to ride in: dst_z[oc] = sum over the pixels k of K slice z of
+// deltaY[k, oc], slice 0 -> dB, slice z -> dB_buf[z-1] (the partition of the split-K entries). One workgroup per
+// (64 channels, slice): 16 lanes cover the channels with 128-bit loads, the 16 lane rows take pixels k, k+16, ...; the
+// rows are added through LDS in a fixed order, so the result is bit-reproducible.
+__global__ __launch_bounds__(256) void col_sum_kernel(const float *__restrict__ dY, float *__restrict__ dB,
+                                                      float *__restrict__ dB_buf, int OC, int GK, int GK_slice, int GZ)
+{
+    __shared__ float4 part[16][17];
+    const int z = blockIdx.y, oc = blockIdx.x * 64 + (threadIdx.x & 15) * 4, row = threadIdx.x >> 4;
+    const int k_start = GK_slice * z, k_end = (z != GZ - 1) ? k_start + GK_slice : GK;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (oc < OC)   // OC % 4 == 0
+        for (int k = k_start + row; k < k_end; k += 16) {
+            const float4 v = *reinterpret_cast<const float4 *>(dY + (size_t)k * OC + oc);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+    part[row][threadIdx.x & 15] = s;
+    __syncthreads();
+    if (row == 0 && oc < OC) {
+        for (int r = 1; r < 16; r++) {
+            const float4 v = part[r][threadIdx.x & 15];
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        float *dst = (z == 0) ? dB : dB_buf + (size_t)(z - 1) * OC;
+        *reinterpret_cast<float4 *>(dst + oc) = s;
+    }
+}
+
+hipError_t launch_col_sum(hipStream_t s, const float *dY, float *dB, float *dB_buf, int OC, int GK, int GK_slice, int GZ)
+{
+    if (OC <= 0 || GK <= 0) return hipSuccess;
+    hipLaunchKernelGGL(col_sum_kernel, dim3((OC + 63) / 64, GZ), dim3(256), 0, s, dY, dB, dB_buf, OC, GK, GK_slice, GZ);
+    return hipGetLastError();
+}
+
 }  // namespace alpha

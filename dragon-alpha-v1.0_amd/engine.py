@@ -74,6 +74,8 @@ def _lib():
         L.alpha_engine_conv3D_biased.argtypes = ([_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [_P, _I, _I]
                                                  + [ctypes.POINTER(Plan)])
         L.alpha_engine_dconv3D_deltaW.argtypes = [_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [ctypes.POINTER(Plan)]
+        L.alpha_engine_dconv3D_deltaW_deltaB.argtypes = ([_P, _P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7
+                                                         + [ctypes.POINTER(Plan)])
         L.alpha_engine_dconv3D_deltaX.argtypes = [_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [ctypes.POINTER(Plan)]
         _bound = True
     return L
@@ -156,6 +158,12 @@ class Engine:
         p = Plan()
         self._check(self._L.alpha_engine_dconv3D_deltaW(self._h, deltaW, FH, FW, X, IH, IW, deltaY, OH, OW, N, IC, OC,
                                                         sh, sw, ph, pw, ctypes.byref(p)))
+        return p
+
+    def dconv3D_deltaW_deltaB(self, deltaW, deltaB, FH, FW, X, IH, IW, deltaY, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        p = Plan()
+        self._check(self._L.alpha_engine_dconv3D_deltaW_deltaB(self._h, deltaW, deltaB, FH, FW, X, IH, IW, deltaY, OH, OW,
+                                                               N, IC, OC, sh, sw, ph, pw, ctypes.byref(p)))
         return p
 
     def dconv3D_deltaX(self, deltaX, IH, IW, deltaY, OH, OW, W, FH, FW, N, IC, OC, sh, sw, ph, pw):

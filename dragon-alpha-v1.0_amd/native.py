@@ -54,6 +54,7 @@ _SIGS = {
     "alpha_dconv3D_deltaW_GemmSK_W1": "siipiipppiii",
     "alpha_winograd_filter_transform": "lppii",
     "alpha_conv3D_winograd": "sipiippiiiiiii",
+    "alpha_dconv3D_deltaW_GemmSK_deltaB": "siipiipiippppiiiiiiiii",
     "alpha_conv3D_biased": "sipiipiippiiiiiiiii",
     "alpha_conv3D_GemmR_biased": "sipiippiippiiiiiiiii",
     "alpha_conv3D_winograd_biased": "sipiipppiiiiiii",
@@ -307,3 +308,10 @@ class Cuda_dconv3D_deltaW:
     @staticmethod
     def dconv3D_deltaW_GemmSK_W1(streamArray, length, GridZ, X, IH, IW, deltaY, deltaW, deltaW_buf, N, IC, OC):
         _call("alpha_dconv3D_deltaW_GemmSK_W1", streamArray, length, GridZ, X, IH, IW, deltaY, deltaW, deltaW_buf, N, IC, OC)
+
+    # backward-filter plus the bias gradient (the reference: dconv3D_deltaW, then field_sum over deltaY)
+    @staticmethod
+    def dconv3D_deltaW_GemmSK_deltaB(streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf,
+                                     deltaB, deltaB_buf, FH, FW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaW_GemmSK_deltaB", streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf,
+              deltaB, deltaB_buf, FH, FW, N, IC, OC, sh, sw, ph, pw)

@@ -290,6 +290,19 @@ int alpha_conv3D_winograd_biased(const int64_t *streams, int length,
                                  float *Y, int OH, int OW,
                                  int N, int IC, int OC, int ph, int pw);
 
+/* Backward-filter plus the bias gradient deltaB[oc] = sum over all pixels of deltaY[., oc] (the reference computes it
+ * with a separate reduction, eg.field_sum(deltaY, OC), nn/unit/simple/Conv3D.java:160). Same split-K contract as
+ * alpha_dconv3D_deltaW_GemmSK: slice z of GK_slice = (GK/GridZ)>>3<<3 pixels writes its partial column sums to deltaB
+ * (z = 0) or deltaB_buf[(z-1)*OC ..]; the caller finishes with alpha_buf_summary(stream, deltaB_buf, deltaB, GridZ-1, OC)
+ * next to the one for deltaW. deltaB_buf holds (GridZ-1)*OC floats (may be NULL when GridZ = 1). Bit-reproducible. */
+int alpha_dconv3D_deltaW_GemmSK_deltaB(const int64_t *streams, int length, int GridZ,
+                                       const float *X, int IH, int IW,
+                                       const float *deltaY, int OH, int OW,
+                                       float *deltaW, float *deltaW_buf,
+                                       float *deltaB, float *deltaB_buf,
+                                       int FH, int FW, int N, int IC, int OC,
+                                       int sh, int sw, int ph, int pw);
+
 #ifdef __cplusplus
 }
 #endif

@@ -109,6 +109,11 @@ int alpha_engine_conv3D_biased(alpha_engine *e, float *Y, int OH, int OW, const 
 int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, const float *X, int IH, int IW,
                                 const float *deltaY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                 alpha_conv_plan *plan_out);
+/* dconv3D_deltaW followed by field_sum(deltaY, OC) (nn/unit/simple/Conv3D.java:150-162) as one operator: deltaB[OC] is
+ * produced by the backward-filter kernel from the deltaY it reads anyway. */
+int alpha_engine_dconv3D_deltaW_deltaB(alpha_engine *e, float *deltaW, float *deltaB, int FH, int FW, const float *X, int IH, int IW,
+                                       const float *deltaY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                       alpha_conv_plan *plan_out);
 int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
                                 const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                 alpha_conv_plan *plan_out);

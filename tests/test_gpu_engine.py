@@ -91,6 +91,35 @@ def test_engine_conv3D_biased(dev, eng):
                           b.data_ptr(), N * IH * IH * OC - 4, OC)
 
 
+@pytest.mark.parametrize("shape", [
+    # N, IH, IW, IC, OC, F, s, p: row-streaming kernel (32 and 16 channels per workgroup), register 1x1 kernel, 1x1 through
+    # the row kernel (ragged channels), generic kernel (strided), single-pass entry (GK < 512)
+    (16, 14, 14, 64, 128, 3, 1, 1),
+    (32, 8, 8, 256, 256, 3, 1, 1),
+    (8, 14, 14, 128, 64, 1, 1, 0),
+    (8, 12, 12, 36, 44, 1, 1, 0),
+    (8, 20, 20, 32, 48, 3, 2, 1),
+    (4, 9, 9, 16, 24, 3, 1, 1),
+])
+def test_engine_deltaW_with_bias_gradient(dev, eng, shape):
+    """deltaB[oc] = sum over all pixels of deltaY (the reference: field_sum(deltaY, OC) after dconv3D_deltaW)."""
+    N, IH, IW, IC, OC, F_, s_, p_ = shape
+    OH, OW = out_dim(IH, IW, F_, F_, s_, s_, p_, p_)
+    X, dY = normal((N, IH, IW, IC), 6401), normal((N, OH, OW, OC), 6402)
+    x, dy = dev.put(X), dev.put(dY)
+    got = []
+    for _ in range(2):
+        dw = dev.empty(OC, F_, F_, IC, fill=float("nan"))
+        db = dev.empty(OC, fill=float("nan"))
+        eng.dconv3D_deltaW_deltaB(dw.data_ptr(), db.data_ptr(), F_, F_, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC,
+                                  s_, s_, p_, p_)
+        eng.sync()
+        got.append((dev.get(dw), dev.get(db)))
+    check(got[0][0], O.deltaW_f64(X, dY, F_, F_, s_, s_, p_, p_), "deltaW with deltaB %s" % (shape,))
+    check(got[0][1], dY.astype(np.float64).sum(axis=(0, 1, 2)), "deltaB %s" % (shape,))
+    assert np.array_equal(got[0][0], got[1][0]) and np.array_equal(got[0][1], got[1][1]), "run-to-run bits differ"
+
+
 def test_engine_filter_transform_cache(dev):
     """With cache_filter_transforms the re-layout runs once per filter; a weight update must be reported."""
     N, IH, IC, OC = 8, 12, 64, 64
