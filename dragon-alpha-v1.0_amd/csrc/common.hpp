@@ -72,7 +72,7 @@ static __device__ __forceinline__ float4 add_bias4(float4 v, const float *bias, 
 hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
                            int N, int AH, int AW, int AC, int OH, int OW, int CO,
                            int TH, int TW, int ph, int pw,
-                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias = nullptr);
+                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias = nullptr, int sh = 1, int sw = 1);
 
 // 1x1 stride-1 convolution as a streaming GEMM with the filter resident in LDS (pointwise.hip):
 // O[(n,oh,ow)][co] = sum_k A[n, oh*sh, ow*sw, k] * B(k, co), B given as [K][N] (b_kmajor) or [N][K]. Returns

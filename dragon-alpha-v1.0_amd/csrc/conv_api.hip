@@ -91,9 +91,9 @@ int forward(const char *fn, const int64_t *streams, int length,
         hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW, bias);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (layout == FILTER_CW && sh == 1 && sw == 1 && fwd_algo() != 3) {
+    if (layout == FILTER_CW && fwd_algo() != 3) {
         hipError_t e = launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
-                                       0, FW * IC * OC, IC * OC, OC, bias);
+                                       0, FW * IC * OC, IC * OC, OC, bias, sh, sw);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
 

@@ -33,10 +33,12 @@ struct TapConvArgs {
     int AH, AW, AC;
     int TH, TW, ph, pw;
     int PHt, PWt;     // AH + 2ph, AW + 2pw
+    int sh, sw;       // output pixel (oh, ow) reads the padded input window at (oh*sh, ow*sw)
+    int PWp, RP;      // LDS row: sw planes of PWp = ceil(PWt/sw) pixels (padded column cp in plane cp % sw at cp / sw); RP = sw*PWp
     int lds_rows;     // halo rows reserved in LDS
     int b_off, b_sth, b_stw, b_sc;
     const float *bias;   // NULL or [CO]
-    FastDiv d_OW, d_OHW, d_PHt, d_PWt;
+    FastDiv d_OW, d_OHW, d_PHt, d_PWt, d_sw;
 };
 
 constexpr int TC_ICC = 64;            // input channels per halo pass
@@ -51,7 +53,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
 {
     constexpr int P = TILES * 16;
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *Hs = smem;   // [lds_rows][PWt][TC_PS] (+ one spare slot); reused as output staging [P][TC_OS]
+    float *Hs = smem;   // [lds_rows][sw planes][PWp][TC_PS] (+ one spare slot); reused as output staging [P][TC_OS]
 
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
@@ -64,16 +66,16 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
     const int unit = xcd * (G >> 3) + min(xcd, G & 7) + xi;
     const int m0 = unit * P;
     const int oc0 = blockIdx.y * 64;
-    const int OW = p.d_OW.d, OHW = p.d_OHW.d, PHt = p.PHt, PWt = p.PWt;
+    const int OW = p.d_OW.d, OHW = p.d_OHW.d, PHt = p.PHt, PWt = p.PWt, RP = p.RP;
 
     // first padded global row held in LDS, and how many rows this unit needs (<= p.lds_rows, host-checked)
     const int n_first = fdiv(m0, p.d_OHW);
     const int oh_first = fdiv(m0 - n_first * OHW, p.d_OW);
-    const int pgr0 = n_first * PHt + oh_first;
+    const int pgr0 = n_first * PHt + oh_first * p.sh;
     const int m_last = min(m0 + P, p.M) - 1;
     const int n_last = fdiv(m_last, p.d_OHW);
     const int oh_last = fdiv(m_last - n_last * OHW, p.d_OW);
-    const int rows = n_last * PHt + oh_last + p.TH - 1 - pgr0 + 1;
+    const int rows = n_last * PHt + oh_last * p.sh + p.TH - 1 - pgr0 + 1;
 
     // per-lane LDS offset (floats) of each tile's pixel at tap (0,0), plus this lane group's channel offset
     int abase[TILES];
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
         const int m = min(m0 + 16 * i + l16, p.M - 1);
         const int n = fdiv(m, p.d_OHW), rem = m - n * OHW;
         const int oh = fdiv(rem, p.d_OW), ow = rem - oh * OW;
-        abase[i] = ((n * PHt + oh - pgr0) * PWt + ow) * TC_PS + 4 * q;
+        abase[i] = ((n * PHt + oh * p.sh - pgr0) * RP + ow) * TC_PS + 4 * q;
     }
 
     floatx4 acc[TILES];
@@ -128,7 +130,10 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
 
     // A fragments of one 16-channel chunk: chunk ck (0..3) of tap (th, tw) starts 16*ck floats into the pixel
     auto read_a = [&](floatx4 (&a)[TILES], int th, int tw, int ck) {
-        const float *hs = Hs + (th * PWt + tw) * TC_PS + 16 * ck;
+        // a strided layer keeps the columns of a row de-interleaved (plane tw % sw), so that the 16 pixels of a tile
+        // are neighbours in LDS whatever the stride and the bank pattern is the stride-1 one
+        const int twq = fdiv(tw, p.d_sw), twr = tw - twq * p.sw;
+        const float *hs = Hs + (th * RP + twr * p.PWp + twq) * TC_PS + 16 * ck;
 #pragma unroll
         for (int i = 0; i < TILES; i++) a[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i]);
     };
@@ -176,7 +181,10 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
             for (int u = 0; u < 8; u++) {
                 const int idx = base + t + 256 * u;
                 // threads past the end of the halo write their zeros to a spare slot behind it
-                const int dst = idx < halo_quads ? (idx >> 4) * TC_PS + (idx & 15) * 4 : p.lds_rows * PWt * TC_PS;
+                const int pix = idx >> 4;
+                const int r = fdiv(pix, p.d_PWt), cp = pix - r * PWt;
+                const int cq = fdiv(cp, p.d_sw), cr = cp - cq * p.sw;
+                const int dst = idx < halo_quads ? (r * RP + cr * p.PWp + cq) * TC_PS + (idx & 15) * 4 : p.lds_rows * RP * TC_PS;
                 const bool ok = (okmask >> u) & 1u;   // per-component selects keep v[] in registers
                 *reinterpret_cast<float4 *>(Hs + dst) =
                     make_float4(ok ? v[u].x : 0.f, ok ? v[u].y : 0.f, ok ? v[u].z : 0.f, ok ? v[u].w : 0.f);
@@ -245,9 +253,9 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
 
 // Rows of LDS halo the worst unit needs: output rows spanned by P consecutive pixels, TH-1 extra rows,
 // and TH-1 more for every image border crossed.
-static int tap_conv_lds_rows(int M, int P, int OH, int OW, int TH)
+static int tap_conv_lds_rows(int M, int P, int OH, int OW, int TH, int sh, int PHt)
 {
-    const int OHW = OH * OW, PHt = OH + TH - 1;
+    const int OHW = OH * OW;
     int worst = 0;
     const int units = (M + P - 1) / P;
     const int scan = units < 4096 ? units : 4096;
@@ -255,13 +263,13 @@ static int tap_conv_lds_rows(int M, int P, int OH, int OW, int TH)
         const long m0 = (long)u * P, m1 = (m0 + P < M ? m0 + P : M) - 1;
         const int n0 = (int)(m0 / OHW), oh0 = (int)(m0 % OHW) / OW;
         const int n1 = (int)(m1 / OHW), oh1 = (int)(m1 % OHW) / OW;
-        const int rows = (n1 * PHt + oh1 + TH - 1) - (n0 * PHt + oh0) + 1;
+        const int rows = (n1 * PHt + oh1 * sh + TH - 1) - (n0 * PHt + oh0 * sh) + 1;
         if (rows > worst) worst = rows;
     }
     if (units > scan) {   // analytic bound for what was not scanned
         const int span = (P + OW - 2) / OW + 1;
         const int cross = (P + OHW - 2) / OHW + 1;
-        const int bound = span + (TH - 1) * (1 + cross);
+        const int bound = (span - 1) * sh + TH + cross * (PHt - OH * sh > 0 ? PHt - OH * sh : 0);
         if (bound > worst) worst = bound;
     }
     return worst;
@@ -288,9 +296,10 @@ static hipError_t launch_tc(hipStream_t stream, const TapConvArgs &a, size_t lds
 hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
                            int N, int AH, int AW, int AC, int OH, int OW, int CO,
                            int TH, int TW, int ph, int pw,
-                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias)
+                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias, int sh, int sw)
 {
-    if (OH != AH + 2 * ph - TH + 1 || OW != AW + 2 * pw - TW + 1) return hipErrorNotSupported;
+    if (sh < 1 || sw < 1 || sh > 4 || sw > 4) return hipErrorNotSupported;
+    if (OH != (AH + 2 * ph - TH) / sh + 1 || OW != (AW + 2 * pw - TW) / sw + 1) return hipErrorNotSupported;
     if (AC < 32 || TH > 7 || TW > 7) return hipErrorNotSupported;
     const long M = (long)N * OH * OW;
     if ((long)N * (AH + 2 * ph) >= (1L << 24)) return hipErrorNotSupported;
@@ -301,6 +310,9 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
     a.AH = AH; a.AW = AW; a.AC = AC;
     a.TH = TH; a.TW = TW; a.ph = ph; a.pw = pw;
     a.PHt = AH + 2 * ph; a.PWt = AW + 2 * pw;
+    a.sh = sh; a.sw = sw;
+    a.PWp = (a.PWt + sw - 1) / sw; a.RP = sw * a.PWp;
+    a.d_sw = make_fastdiv(sw);
     a.b_off = b_off; a.b_sth = b_sth; a.b_stw = b_stw; a.b_sc = b_sc;
     a.d_OW = make_fastdiv(OW);
     a.d_OHW = make_fastdiv(OH * OW);
@@ -311,11 +323,12 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
     const int OHW = OH * OW;
     int tiles = 8;
     if ((OHW % 112 == 0 || (2 * OW) % 112 == 0 || 112 % OW == 0) && !(OHW % 128 == 0 || 128 % OW == 0)) tiles = 7;
-    const size_t budget = 80 * 1024;   // two workgroups per CU
+    // stride 1: two workgroups per CU; a strided layer touches sh*sw input pixels per output pixel and gets the whole LDS
+    const size_t budget = (sh == 1 && sw == 1) ? 80 * 1024 : 160 * 1024;
     for (int attempt = 0; attempt < 2; attempt++) {
         const int P = tiles * 16;
-        a.lds_rows = tap_conv_lds_rows(a.M, P, OH, OW, TH);
-        size_t halo = (size_t)a.lds_rows * a.PWt * TC_PS + 4;   // + one spare 16-byte slot
+        a.lds_rows = tap_conv_lds_rows(a.M, P, OH, OW, TH, sh, a.PHt);
+        size_t halo = (size_t)a.lds_rows * a.RP * TC_PS + 4;   // + one spare 16-byte slot
         const size_t stage = (size_t)P * TC_OS;
         if (halo < stage) halo = stage;
         const size_t lds = halo * sizeof(float);

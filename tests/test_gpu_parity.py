@@ -334,6 +334,40 @@ def test_pointwise_kernel_strided(dev, shape):
         check(_run_fwd(dev, entry, X, W, sh, sw, 0, 0), want, "%s strided 1x1 %s" % (entry, shape))
 
 
+STRIDED_TAP_SHAPES = [
+    # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw: strided layers with >= 32 input channels through the LDS-halo kernel
+    # (columns of the halo de-interleaved by ow parity class), remode entries
+    (4, 28, 28, 64, 128, 3, 3, 2, 2, 1, 1),     # c4b geometry (56 -> 28 there)
+    (4, 15, 13, 64, 64, 3, 3, 2, 2, 1, 1),      # odd sizes: units cross rows and images
+    (4, 17, 19, 32, 96, 5, 3, 2, 3, 2, 1),      # mixed strides, non-square filter
+    (2, 16, 16, 96, 64, 2, 2, 2, 2, 0, 0),      # 2x2 stride 2 (no overlap), ragged channel pass
+    (3, 9, 30, 64, 64, 3, 3, 1, 2, 1, 1),       # stride only along the width
+]
+
+
+@pytest.mark.parametrize("shape", STRIDED_TAP_SHAPES)
+def test_strided_forward_through_the_halo_kernel(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
+    X, W, B = normal((N, IH, IW, IC), 2301), he_normal(OC, FH, FW, IC, 2302), normal((OC,), 2303)
+    want = O.conv3D_f64(X, W, sh, sw, ph, pw)
+    L = pkg.lib()
+    try:
+        for algo in (0, 3):   # 0: halo kernel, 3: generic kernel
+            L.alpha_conv_set_fwd_algo(algo)
+            for entry in ("conv3D_GemmR", "conv3D_GemmV2R"):
+                check(_run_fwd(dev, entry, X, W, sh, sw, ph, pw), want, "%s algo %d %s" % (entry, algo, shape))
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    x, w, b = dev.put(X), dev.put(W), dev.put(B)
+    cw = dev.empty(FH * FW * IC * OC, fill=float("nan"))
+    C3.kernel_remode(dev.stream, w.data_ptr(), cw.data_ptr(), FH, FW, OC, IC)
+    y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    C3.conv3D_GemmR_biased(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), cw.data_ptr(), FH, FW, b.data_ptr(), y.data_ptr(),
+                           OH, OW, N, IC, OC, sh, sw, ph, pw)
+    check(dev.get(y), want + B.astype(np.float64)[None, None, None, :], "strided biased %s" % (shape,))
+
+
 BIAS_SHAPES = [
     # N, IH, IW, IC, OC, F, s, p: one layer per forward kernel (the bias rides in each kernel's epilogue)
     (4, 14, 14, 64, 64, 3, 1, 1),      # LDS-halo kernel
