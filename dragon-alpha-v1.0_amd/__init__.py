@@ -8,3 +8,5 @@ falls back to a CPU or PyTorch implementation: if the library is missing, loadin
 from .native import (Cuda_conv3D, Cuda_dconv3D_deltaX, Cuda_dconv3D_deltaW, AlphaConvError, lib, lib_path,  # noqa: F401
                      exported_symbols, device_info)
 from . import engine  # noqa: F401,E402
+from . import runtime  # noqa: F401,E402
+from .runtime import Cuda  # noqa: F401,E402

@@ -38,6 +38,35 @@ def test_every_declared_symbol_is_exported():
     assert sorted(pkg.exported_symbols()) == declared  # the ctypes mirror binds exactly the header
 
 
+def test_runtime_header_symbols_and_jni_names():
+    """include/alpha_rt.h: every declared function is exported, and so is every native of the reference's runtime class
+    Cuda under its JNI long name (overloads carry their signature, as in the reference's Cuda_Stream.cuh / Cuda_float.cuh)."""
+    hdr = open(os.path.join(ROOT, "include", "alpha_rt.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(alpha_rt_\w+)\s*\(", hdr)))
+    assert len(declared) >= 55
+    exported = _exported()
+    assert not [f for f in declared if f not in exported]
+    P = "Java_z_dragon_engine_cuda_impl_Cuda_"
+    natives = ["malloc", "free", "mallocHost", "freeHost", "memsetAsync", "memcpyAsyncHostToDevice", "memcpyAsyncHostToHost",
+               "memcpyAsyncDeviceToHost", "memcpyAsyncDeviceToDevice", "memcpyAsyncDefault", "getDeviceId", "getDeviceCount",
+               "setDevice", "resetDevice", "deviceSynchronize", "isDeviceP2PAccessEnabled", "enableDeviceP2PAccess",
+               "disableDeviceP2PAccess", "getStreamPriorityRange", "newStream_1Blocking__", "newStream_1Blocking__I",
+               "newStream_1NonBlocking__", "newStream_1NonBlocking__I", "deleteStream__J", "deleteStream___3JI", "streamQuery",
+               "streamSynchronize__J", "streamSynchronize___3JI", "newEvent_1Default", "newEvent_1BlockingSync",
+               "newEvent_1DisableTiming", "newEvent_1Interprocess", "deleteEvent", "eventRecord__JJ", "eventRecord__J_3JI",
+               "eventSynchronize", "eventElapsedTime", "streamWaitEvent_1default", "streamWaitEvent_1external",
+               "streamsWaitEvent_1default", "streamsWaitEvent_1external", "getExceptionName", "getExceptionInfo",
+               "getLastExceptionType", "get1D", "get2D", "get1D_1v2", "get2D_1v2", "set1D__JJFI", "set2D__JJFIII",
+               "set1D__JJ_3BI", "set1D__JJ_3FI", "set1D_1v2__JJ_3BJI", "set1D_1v2__JJ_3FJI", "set2D__JJ_3BIII", "set2D__JJ_3FIII",
+               "set2D_1v2__JJ_3BJIII", "set2D_1v2__JJ_3FJIII", "setFrom1Dto2D", "setFrom2Dto1D", "setFrom2Dto2D",
+               "get1D_1int", "get2D_1int", "get1D_1v2_1int", "get2D_1v2_1int", "set1D_1int", "set2D_1int", "set1D_1v2_1int",
+               "set2D_1v2_1int", "get1D_1char", "get2D_1char", "get1D_1v2_1char", "get2D_1v2_1char", "set1D_1char", "set2D_1char",
+               "set1D_1v2_1char", "set2D_1v2_1char", "set2D_1v2_1char_1W3S4"]
+    assert len(natives) == 78
+    assert not [n for n in natives if P + n not in exported]
+
+
 def test_argument_validation_without_gpu():
     L = pkg.lib()
     one = (ctypes.c_int64 * 1)(0)

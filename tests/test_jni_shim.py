@@ -37,7 +37,7 @@ def test_all_29_jni_symbols_exported():
     want = [mangle(c, m) for c, ms in NATIVES.items() for m in ms]
     assert len(want) == 29
     assert not [w for w in want if w not in exported]
-    assert len([e for e in exported if e.startswith("Java_")]) == 29   # nothing extra either
+    assert len([e for e in exported if e.startswith("Java_z_dragon_engine_cuda_impl_math_")]) == 29   # nothing extra either
 
 
 def _jni(name):
@@ -92,3 +92,25 @@ def test_forward_through_jni_symbols_on_gpu():
     want = O.conv3D_f64(X, W, 1, 1, 1, 1)
     floor = 1e-5 * max(1.0, float(np.sqrt(np.mean(want * want))))
     assert O.max_err_ratio(dev.get(y), want, 1e-4, floor) <= 1.0
+
+
+def test_runtime_class_stubs_that_need_no_device():
+    """Natives of the runtime class (Cuda.java:19-182) whose answer does not depend on a GPU: argument validation throws
+    the Java exception, error names and the priority range come back as a jstring and an int[2]."""
+    env = FakeEnv()
+    L, I, P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
+    lib = pkg.lib()
+
+    def jni(name, restype, *argtypes):
+        fn = getattr(lib, "Java_z_dragon_engine_cuda_impl_Cuda_" + name)
+        fn.restype, fn.argtypes = restype, [P, P] + list(argtypes)
+        return lambda *a: fn(env.ptr, None, *a)
+
+    jni("memsetAsync", None, L, L, I, L)(0, 0, 0, -4)
+    assert env.thrown == [("z/dragon/engine/cuda/impl/CudaException", "alpha-rt-hip error 1: alpha_rt_memsetAsync: negative size")]
+    assert env.strings[jni("getExceptionName", P, I)(1)] == "hipErrorInvalidValue"
+    assert env.strings[jni("getExceptionInfo", P, I)(2)] == "out of memory"
+    assert env.arrays[jni("getStreamPriorityRange", P)()] == [0, 0]
+    jni("deleteStream__J", None, L)(0)                      # a zero handle is skipped without touching the device
+    jni("deleteStream___3JI", None, P, I)(env.long_array([0, 0]), 2)
+    assert len(env.thrown) == 1
