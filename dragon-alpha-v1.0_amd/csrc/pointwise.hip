@@ -34,6 +34,7 @@ struct PointwiseArgs {
 };
 
 constexpr int PW_OS = 64 + 4;   // staging row stride (floats)
+template <int V> struct IntC { static constexpr int value = V; };
 
 template <int NT, int KB>   // N = 16*NT produced channels, K = 64*KB reduced channels
 __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p)
@@ -48,9 +49,15 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
     // ---- tiles: the workgroup owns the contiguous range [t_begin, t_end); its wavefronts take the first eight
     // statically and then draw from a counter in LDS, so they finish within one tile of each other whatever the
     // range length (a static split of 24.5 tiles over 8 wavefronts would leave a quarter of the machine idle).
-    // The first tile's A fragments are requested before anything else.
+    // With more than one group of 64 produced channels per tile, the tiles beyond the last multiple of eight are
+    // split further, into (tile, group) units dealt to the wavefronts in order (wavefronts w and w + 4 share a SIMD):
+    // a 25th tile costs every SIMD a quarter of a tile instead of costing one SIMD a whole one.
     const int G = gridDim.x;
     const int t_begin = (int)((long)p.tiles * blockIdx.x / G), t_end = (int)((long)p.tiles * (blockIdx.x + 1) / G);
+    constexpr int NG = NT / 4;
+    const int t_main = NG > 1 ? t_begin + ((t_end - t_begin) & ~7) : t_end;
+    const int units = (t_end - t_main) * NG;          // 0 when NG == 1
+    const int unit_tile = t_main + w / NG;            // tile of this wavefront's first unit, if it has one (w < units)
     int *queue = reinterpret_cast<int *>(smem + N * KS + 8 * 16 * PW_OS);
     if (t == 0) *queue = t_begin + 8;
 
@@ -70,10 +77,12 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
     };
     floatx4 aP[KB][4], aQ[KB][4];
     int tile = t_begin + w;
-    load_a(aP, min(tile, p.tiles - 1));
 
     // ---- filter -> LDS, once: 8 loads in flight per thread, consecutive lanes along k so that the transposing
-    // stores of the [K][N] layout fall into consecutive banks -------------------------------------------------------
+    // stores of the [K][N] layout fall into consecutive banks. The first tile's A fragments are requested right
+    // after the first batch of filter loads: behind them (loads return in order, and the A fragments of all
+    // workgroups together are a third of a 256-channel input, far more memory time than the filter,
+    // which comes from L2), but before the filter is written to LDS ---------------------------------------------------
     constexpr int QUADS = N * K / 4;
     for (int base = 0; base < QUADS; base += 512 * 8) {
         float4 v[8];
@@ -88,6 +97,7 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
                 v[u] = *reinterpret_cast<const float4 *>(p.B + (size_t)k * ldn + n_off + n4);
             }
         }
+        if (base + 512 * 8 >= QUADS) load_a(aP, tile < t_main ? tile : w < units ? unit_tile : t_end - 1);
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             const int idx = base + t + 512 * u;
@@ -107,51 +117,108 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
     }
     __syncthreads();
 
-    floatx4 acc[NT];
     const float *bl = Bs + l16 * KS + 4 * q;
-    while (tile < t_end) {
-        // draw the next tile and start its fragments on their way while this tile is multiplied (past the end of
-        // the range: re-fetch this tile, unused)
-        int ntile = 0;
-        if (lane == 0) ntile = atomicAdd(queue, 1);
-        ntile = __builtin_amdgcn_readfirstlane(ntile);
-        load_a(aQ, ntile < t_end ? ntile : tile);
+    // bias of the columns this lane stores (zeros without one: the add is unconditional, the loop branch-free)
+    floatx4 bias4[NT / 4];
 #pragma unroll
-        for (int j = 0; j < NT; j++) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int jg = 0; jg < NT / 4; jg++)
+        bias4[jg] = p.bias ? *reinterpret_cast<const floatx4 *>(p.bias + n_off + 64 * jg + 4 * l16) : floatx4{0.f, 0.f, 0.f, 0.f};
+    // the bias and the first tile's fragments are waited for here, so that no load is outstanding when the loop is
+    // entered (a load pending at the loop head would make every iteration start with a wait for the previous
+    // iteration's stores)
 #pragma unroll
-        for (int kb = 0; kb < KB; kb++)
+    for (int jg = 0; jg < NT / 4; jg++) asm volatile("" : "+v"(bias4[jg]));
 #pragma unroll
-            for (int c = 0; c < 4; c++)
+    for (int kb = 0; kb < KB; kb++)
 #pragma unroll
-                for (int j = 0; j < NT; j++) {
-                    const floatx4 b = *reinterpret_cast<const floatx4 *>(bl + j * 16 * KS + kb * 64 + 16 * c);
+        for (int c = 0; c < 4; c++) asm volatile("" : "+v"(aP[kb][c]));
+    // One tile = NG groups of 64 produced channels; a group = GS steps of one filter fragment (128-bit LDS read, two
+    // steps ahead of its use) and four MFMAs. The results of a group leave while the next group is multiplied: its
+    // patch writes, patch reads and global stores sit in steps 1, 3 and 5 of the following group, so the first
+    // lines of a tile are on their way to memory after a quarter of its MFMAs (the 256-channel layers are bound by
+    // the rate at which the output can be written, and nothing is written while a workgroup only multiplies).
+    constexpr int GS = KB * 16;
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    // groups g0 .. g0 + NGX - 1 of one tile from the fragments a
+    auto process = [&](auto ngx, int tile, int g0, const floatx4 (&a)[KB][4]) {
+        constexpr int NGX = decltype(ngx)::value, STEPS = NGX * GS;
+        const float *blg = bl + g0 * 64 * KS;
+        auto read_b = [&](int i) {
+            const int g = i / GS, r = i % GS;
+            return *reinterpret_cast<const floatx4 *>(blg + (4 * g + (r & 3)) * 16 * KS + (r >> 2) * 16);
+        };
+        // Rows past M repeat row M-1 (their fragments were loaded from it, so they hold the same values) and are
+        // stored to it again: no store is conditional, and the waits of the loop can be counted exactly. A wait
+        // placed after a store whose execution is uncertain would have to wait for every store to be acknowledged.
+        float *dst[4];
 #pragma unroll
-                    for (int s = 0; s < 4; s++) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(aP[kb][c][s], b[s], acc[j], 0, 0, 0);
-                }
+        for (int i = 0; i < 4; i++) dst[i] = p.O + (size_t)min(tile * 16 + 4 * i + q, p.M - 1) * ldn + n_off + 64 * g0 + 4 * l16;
+        floatx4 bsel[NGX];
+        if constexpr (NGX == NG) {
+#pragma unroll
+            for (int g = 0; g < NG; g++) bsel[g] = bias4[g];
+        } else {
+            bsel[0] = bias4[0];
+#pragma unroll
+            for (int g = 1; g < NG; g++) bsel[0] = g0 == g ? bias4[g] : bsel[0];
+        }
 
-        // ---- lane holds O[16*tile + 4q + r][16j + l16]; 64 columns at a time through the LDS patch -----------------
-#pragma unroll
-        for (int jg = 0; jg < NT / 4; jg++) {
+        floatx4 acc[NGX][4], v[4], b[3];
+        auto patch_write = [&](const floatx4 (&c)[4]) {
 #pragma unroll
             for (int jj = 0; jj < 4; jj++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) Os[(4 * q + r) * PW_OS + 16 * jj + l16] = acc[4 * jg + jj][r];
-            __builtin_amdgcn_wave_barrier();
+                for (int r = 0; r < 4; r++) Os[(4 * q + r) * PW_OS + 16 * jj + l16] = c[jj][r];
+            __builtin_amdgcn_wave_barrier();   // LDS operations of one wavefront execute in order
+        };
+        auto patch_read = [&]() {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int row = 4 * i + q, m = tile * 16 + row;
-                const float4 v = *reinterpret_cast<const float4 *>(Os + row * PW_OS + 4 * l16);
-                if (m < p.M)
-                    *reinterpret_cast<float4 *>(p.O + (size_t)m * ldn + n_off + 64 * jg + 4 * l16) =
-                        add_bias4(v, p.bias, n_off + 64 * jg + 4 * l16);
-            }
+            for (int i = 0; i < 4; i++) v[i] = *reinterpret_cast<const floatx4 *>(Os + (4 * i + q) * PW_OS + 4 * l16);
             __builtin_amdgcn_wave_barrier();
+        };
+        auto store = [&](int g) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) *reinterpret_cast<floatx4 *>(dst[i] + 64 * g) = v[i] + bsel[g];
+        };
+        b[0] = read_b(0);
+        b[1] = read_b(1);
+#pragma unroll
+        for (int i = 0; i < STEPS; i++) {
+            const int g = i / GS, r = i % GS, jj = r & 3, kc = r >> 2;
+            if (i + 2 < STEPS) b[(i + 2) % 3] = read_b(i + 2);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+                acc[g][jj] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[kc >> 2][kc & 3][s], b[i % 3][s],
+                                                                  kc == 0 && s == 0 ? zero : acc[g][jj], 0, 0, 0);
+            if (g > 0 && r == 1) patch_write(acc[g - 1]);
+            if (g > 0 && r == 3) patch_read();
+            if (g > 0 && r == 5) store(g - 1);
+            __builtin_amdgcn_sched_barrier(0);   // nothing moves between steps
         }
+        patch_write(acc[NGX - 1]);
+        patch_read();
+        store(NGX - 1);
+    };
+
+    while (tile < t_main) {
+        // draw the next tile and start its fragments on their way while this tile is multiplied (past the end:
+        // the tile of this wavefront's first unit, or this tile again, unused)
+        int ntile = 0;
+        if (lane == 0) ntile = atomicAdd(queue, 1);
+        ntile = __builtin_amdgcn_readfirstlane(ntile);
+        load_a(aQ, ntile < t_main ? ntile : w < units ? unit_tile : tile);
+        process(IntC<NG>{}, tile, 0, aP);
 #pragma unroll
         for (int kb = 0; kb < KB; kb++)
 #pragma unroll
             for (int c = 0; c < 4; c++) aP[kb][c] = aQ[kb][c];
         tile = ntile;
+    }
+    if constexpr (NG > 1) {
+        for (int u = w; u < units; u += 8) {
+            if (u != w) load_a(aP, t_main + u / NG);   // only the first unit's fragments were requested ahead
+            process(IntC<1>{}, t_main + u / NG, u % NG, aP);
+        }
     }
 }
 
