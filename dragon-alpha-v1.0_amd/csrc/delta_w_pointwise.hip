@@ -69,23 +69,34 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
         ya[d] = *reinterpret_cast<const floatx4 *>(py + (size_t)g * 4 * p.OC);
         xa[d] = *reinterpret_cast<const floatx4 *>(px + (size_t)g * 4 * p.IC);
     };
+    // The ring loop is free of branches on purpose: the loads of a slot are waited for by count (14 younger loads may
+    // stay in flight), and the count is only known when every load and every use is executed unconditionally. With a
+    // branch around the MFMAs of a slot each round of the ring began with a wait for all 16 loads.
+    const float bias_on = do_bias ? 1.f : 0.f;
+    auto multiply = [&](int d) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ya[d][i], xa[d][j], acc[i][j], 0, 0, 0);
+        bsum += ya[d] * bias_on;
+    };
     if (g0 < g1) {
 #pragma unroll
         for (int d = 0; d < DWP_D; d++) load(d, min(g0 + d, g1 - 1));
-        for (int g = g0; g < g1; g += DWP_D) {
+        int g = g0;
+        for (; g + DWP_D <= g1; g += DWP_D) {
 #pragma unroll
             for (int d = 0; d < DWP_D; d++) {
-                if (g + d < g1) {   // uniform; the refill below stays unconditional so the waits stay short
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-#pragma unroll
-                        for (int j = 0; j < 4; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ya[d][i], xa[d][j], acc[i][j], 0, 0, 0);
-                    if (do_bias) bsum += ya[d];
-                }
-                load(d, min(g + d + DWP_D, g1 - 1));
+                multiply(d);
+                load(d, min(g + d + DWP_D, g1 - 1));   // past the end: the last group again, unused
+                __builtin_amdgcn_sched_barrier(0);      // keeps the refill next to its slot (the scheduler batches them)
             }
         }
+        const int rest = g1 - g;   // < DWP_D groups, already in slots 0 .. rest-1
+#pragma unroll
+        for (int d = 0; d < DWP_D - 1; d++)
+            if (d < rest) multiply(d);
     }
 
     // ---- bias gradient: lanes q = 0..3 hold different pixels of the same 4 channels (wavefront shuffles), the parts

@@ -38,6 +38,7 @@ struct StemArgs {
 
 constexpr int ST_OS = 64 + 4;       // output staging row stride (floats)
 constexpr int ST_MAXG = 13;         // tap groups supported (52 taps)
+template <int V> struct StemChannels { static constexpr int value = V; };
 
 __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
 {
@@ -49,7 +50,10 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
     const int oc0 = blockIdx.y * 64;
     const int IWB = p.IWB, taps = p.taps;
 
-    // ---- filter -> LDS, once --------------------------------------------------------------------------------------
+    // ---- filter -> LDS, once. Layers with 3 logical channels arrive with the fourth stored channel zero-filled in X
+    // and in the filter: when every weight of channel 3 in this workgroup's 64 output channels is zero, the MFMA step
+    // of that channel (a quarter of all steps) is left out ------------------------------------------------------------
+    int ch3 = 0;
     for (int idx = t; idx < p.groups * 4 * 64; idx += 256) {
         const int slot = idx >> 6, ocl = idx & 63, oc = oc0 + ocl;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -61,8 +65,10 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
                 v = make_float4(f[0], f[p.OC], f[2 * p.OC], f[3 * p.OC]);
             }
         }
+        ch3 |= v.w != 0.f;
         *reinterpret_cast<float4 *>(Ws + ((slot << 6) + (ocl ^ ((slot & 1) << 4))) * 4) = v;
     }
+    const bool use_ch3 = __syncthreads_or(ch3) != 0;
 
     // ---- per-lane offsets (floats) ---------------------------------------------------------------------------------
     int toff[ST_MAXG];   // input offset of tap 4g + q relative to the output pixel's window origin
@@ -117,23 +123,28 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
         for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        auto multiply = [&](auto sc) {
+            constexpr int SC = decltype(sc)::value;   // channels multiplied: 4, or 3 when channel 3 has zero weights
 #pragma unroll
-        for (int g = 0; g < ST_MAXG; g++) {
-            if (g < p.groups) {   // uniform
-                floatx4 a[4], b[4];
+            for (int g = 0; g < ST_MAXG; g++) {
+                if (g < p.groups) {   // uniform
+                    floatx4 a[4], b[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) a[i] = *reinterpret_cast<const floatx4 *>(Xs + xbase[i] + toff[g]);
+                    for (int i = 0; i < 4; i++) a[i] = *reinterpret_cast<const floatx4 *>(Xs + xbase[i] + toff[g]);
 #pragma unroll
-                for (int j = 0; j < 4; j++) b[j] = *reinterpret_cast<const floatx4 *>(Ws + wl[j] + g * (4 * 64 * 4));
+                    for (int j = 0; j < 4; j++) b[j] = *reinterpret_cast<const floatx4 *>(Ws + wl[j] + g * (4 * 64 * 4));
 #pragma unroll
-                for (int s = 0; s < 4; s++)
+                    for (int s = 0; s < SC; s++)
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
+                        for (int i = 0; i < 4; i++)
 #pragma unroll
-                        for (int j = 0; j < 4; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+                            for (int j = 0; j < 4; j++)
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+                }
             }
-        }
+        };
+        if (use_ch3) multiply(StemChannels<4>{});
+        else multiply(StemChannels<3>{});
         __syncthreads();   // every wavefront is done with the window: its space becomes the output patches
 
         // ---- lane holds Y[oh0 + 4w + i][ow0 + 4q + r][oc0 + 16j + l16] ---------------------------------------------------
@@ -181,7 +192,7 @@ hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, 
     a.d_IWB = make_fastdiv(a.IWB);
     const size_t window = (size_t)a.IHB * a.IWB * 4, patches = 4 * 16 * ST_OS;
     const size_t lds = ((size_t)a.groups * 4 * 64 * 4 + (window > patches ? window : patches)) * sizeof(float);
-    if (lds > 80 * 1024) return hipErrorNotSupported;   // two workgroups per compute unit
+    if (lds + 256 > 80 * 1024) return hipErrorNotSupported;   // two workgroups per compute unit (256 bytes: the block-wide OR)
     static int cu_count[64] = {0};   // per device; a racing first call writes the same value
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorNotSupported;

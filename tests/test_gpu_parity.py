@@ -112,6 +112,19 @@ def test_forward_general_entries(dev, shape, entry):
     check(_run_fwd(dev, entry, X, W, sh, sw, ph, pw), want, "%s %s" % (entry, shape))
 
 
+@pytest.mark.parametrize("entry", ["conv3D", "conv3D_GemmR"])
+def test_forward_three_channels_stored_as_four(dev, entry):
+    """The kernel for 4 stored channels leaves out the MFMA step of channel 3 for every block of 64 output channels whose
+    weights of that channel are all zero (a 3-channel layer as the engine pads it). Here the first 64 output channels are
+    padded like that and the other 64 use all four channels, so one launch runs both paths; the pad channel of X holds
+    data on purpose: it must not reach the first 64 outputs and must reach the others."""
+    N, IH, IW, OC, F_, s_, p_ = 4, 30, 30, 128, 7, 2, 3
+    X = uniform((N, IH, IW, 4), 1011)
+    W = he_normal(OC, F_, F_, 4, 1012)
+    W[:64, :, :, 3] = 0.0
+    check(_run_fwd(dev, entry, X, W, s_, s_, p_, p_), O.conv3D_f64(X, W, s_, s_, p_, p_), entry)
+
+
 @pytest.mark.parametrize("entry", ["conv3D_texture", "conv3DV2", "conv3D_GemmR_texture", "conv3D_GemmV2R"])
 def test_forward_hint_variants_give_same_result(dev, entry):
     shape = (8, 12, 12, 32, 96, 3, 3, 1, 1, 1, 1)
