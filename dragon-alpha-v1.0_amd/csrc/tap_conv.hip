@@ -41,6 +41,7 @@ struct TapConvArgs {
     FastDiv d_OW, d_OHW, d_PHt, d_PWt, d_sw;
 };
 
+template <int V> struct TapInt { static constexpr int value = V; };
 constexpr int TC_ICC = 64;            // input channels per halo pass
 constexpr int TC_PS = TC_ICC + 8;     // LDS pixel stride (floats)
 constexpr int TC_OS = 64 + 4;         // output staging row stride (floats)
@@ -125,7 +126,6 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
         }
     };
 
-    const int halo_quads = rows * PWt * (TC_ICC / 4);
     const int taps = p.TH * p.TW;
 
     // A fragments of one 16-channel chunk: chunk ck (0..3) of tap (th, tw) starts 16*ck floats into the pixel
@@ -158,38 +158,68 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
     load_b(bA, 0, 0, 0);   // first half tap; in flight while the halo is staged
     for (int ic0 = 0; ic0 < p.AC; ic0 += TC_ICC) {
         if (ic0 > 0) __syncthreads();   // everyone finished reading the previous pass's halo
-        // ---- stage the halo: 16 lanes per pixel (64 channels), zero outside the image / beyond AC ----------
-        for (int base = 0; base < halo_quads; base += 256 * 8) {
-            float4 v[8];
-            unsigned okmask = 0;
-            // all eight loads are issued (unconditionally, from a clamped address) before any result is used
+        // Two workgroups share a compute unit so that one stages while the other multiplies. A wavefront that issues
+        // MFMAs back to back keeps the SIMD's vector issue port occupied, and the address arithmetic of a staging
+        // wavefront of the other workgroup at the same priority hardly ever gets a turn: staging ended exactly
+        // when the other workgroup's MFMA loop did. Staging and the epilogue therefore run at a raised priority.
+        __builtin_amdgcn_s_setprio(2);
+        // ---- stage the halo row by row, zero outside the image / beyond AC. A thread keeps its place in the row:
+        // 16 lanes per pixel (64 channels), padded column 16*cg + t/16 of column group cg. What depends on the
+        // column is computed once per 64 columns, what depends on the row is uniform (scalar registers); per
+        // element the vector unit is left with two address operations and the zero-fill selects. (Computing
+        // pixel, row and column of every element from a flat index cost ~60 vector instructions per element, and
+        // those take issue slots from the MFMAs of the workgroup that shares the compute unit.)
+        // A step stages RS rows of CGS column groups (16 columns each), at most eight loads in flight per thread;
+        // narrow images take more rows per step, wide ones more column groups (and several trips along the row).
+        auto stage = [&](auto cgs_c, auto rs_c) {
+            constexpr int CGS = decltype(cgs_c)::value, RS = decltype(rs_c)::value;
+            const int cq4 = (t & 15) * 4;
+            const bool ch_ok = ic0 + cq4 < p.AC;
+            const int row_floats = RP * TC_PS, spare = p.lds_rows * row_floats;
+            for (int c0 = 0; c0 < PWt; c0 += 16 * CGS) {
+                int goff[CGS], loff[CGS];
+                bool cok[CGS];
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
-                const int idx = base + t + 256 * u;
-                const int pix = idx >> 4, cq = (idx & 15) * 4;
-                const int r = fdiv(pix, p.d_PWt), cp = pix - r * PWt;
-                const int pgr = pgr0 + r;
-                const int n = fdiv(pgr, p.d_PHt), ih = pgr - n * PHt - p.ph, iw = cp - p.pw;
-                const bool ok = idx < halo_quads && (unsigned)ih < (unsigned)p.AH && (unsigned)iw < (unsigned)p.AW &&
-                                ic0 + cq < p.AC;
-                // branch-free clamp: offset 0 when the element is outside the image
-                const int off = (((n * p.AH + ih) * p.AW + iw) * p.AC + ic0 + cq) & -(int)ok;
-                v[u] = *reinterpret_cast<const float4 *>(p.A + off);
-                okmask |= (unsigned)ok << u;
-            }
+                for (int cg = 0; cg < CGS; cg++) {
+                    const int cp = c0 + 16 * cg + (t >> 4), iw = cp - p.pw;
+                    cok[cg] = cp < PWt && (unsigned)iw < (unsigned)p.AW && ch_ok;
+                    goff[cg] = cok[cg] ? iw * p.AC + ic0 + cq4 : 0;
+                    const int cq = fdiv(cp, p.d_sw), cr = cp - cq * p.sw;
+                    // threads past the end of the row write their zeros to a spare slot behind the halo
+                    loff[cg] = cp < PWt ? (cr * p.PWp + cq) * TC_PS + cq4 : spare;
+                }
+                for (int r = 0; r < rows; r += RS) {
+                    float4 v[RS][CGS];
+                    bool rok[RS];
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
-                const int idx = base + t + 256 * u;
-                // threads past the end of the halo write their zeros to a spare slot behind it
-                const int pix = idx >> 4;
-                const int r = fdiv(pix, p.d_PWt), cp = pix - r * PWt;
-                const int cq = fdiv(cp, p.d_sw), cr = cp - cq * p.sw;
-                const int dst = idx < halo_quads ? (r * RP + cr * p.PWp + cq) * TC_PS + (idx & 15) * 4 : p.lds_rows * RP * TC_PS;
-                const bool ok = (okmask >> u) & 1u;   // per-component selects keep v[] in registers
-                *reinterpret_cast<float4 *>(Hs + dst) =
-                    make_float4(ok ? v[u].x : 0.f, ok ? v[u].y : 0.f, ok ? v[u].z : 0.f, ok ? v[u].w : 0.f);
+                    for (int rr = 0; rr < RS; rr++) {
+                        const int pgr = pgr0 + min(r + rr, rows - 1);   // past the last row: the last row again
+                        const int n = fdiv(pgr, p.d_PHt), ih = pgr - n * PHt - p.ph;
+                        rok[rr] = (unsigned)ih < (unsigned)p.AH;
+                        const int rowbase = rok[rr] ? (n * p.AH + ih) * p.AW * p.AC : 0;
+                        const int rowmask = rok[rr] ? -1 : 0;
+#pragma unroll
+                        for (int cg = 0; cg < CGS; cg++)   // outside the image: element 0, zeroed below
+                            v[rr][cg] = *reinterpret_cast<const float4 *>(p.A + rowbase + (goff[cg] & rowmask));
+                    }
+#pragma unroll
+                    for (int rr = 0; rr < RS; rr++) {
+                        const int rowoff = min(r + rr, rows - 1) * row_floats;
+#pragma unroll
+                        for (int cg = 0; cg < CGS; cg++) {
+                            const bool ok = rok[rr] && cok[cg];   // per-component selects keep v[] in registers
+                            const int dst = loff[cg] == spare ? spare : rowoff + loff[cg];
+                            *reinterpret_cast<float4 *>(Hs + dst) = make_float4(ok ? v[rr][cg].x : 0.f, ok ? v[rr][cg].y : 0.f,
+                                                                                ok ? v[rr][cg].z : 0.f, ok ? v[rr][cg].w : 0.f);
+                        }
+                    }
+                }
             }
-        }
+        };
+        if (PWt <= 16) stage(TapInt<1>{}, TapInt<8>{});
+        else if (PWt <= 32) stage(TapInt<2>{}, TapInt<4>{});
+        else if (PWt <= 48) stage(TapInt<3>{}, TapInt<2>{});
+        else stage(TapInt<4>{}, TapInt<2>{});
         __syncthreads();
 
         // ---- main loop: one tap (four 16-channel chunks) per iteration ------------------------------------
@@ -198,6 +228,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
         // loop assume the shorter queue): after the last tap it fetches the first half tap of the next pass, or
         // harmlessly re-fetches tap (0,0) of this one at the very end. The scheduling barriers pin each prefetch in
         // front of the chunk that hides its latency; left alone the compiler sinks the loads to their first use.
+        __builtin_amdgcn_s_setprio(0);
         int th = 0, tw = 0;
         read_a(aP, 0, 0, 0);
         for (int tap = 0; tap < taps; tap++) {
@@ -233,6 +264,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
     }
     (void)bA;
     (void)aP;
+    __builtin_amdgcn_s_setprio(2);
 
     // ---- epilogue: transpose through LDS so every output pixel row is written as whole 256-byte lines ----
     __syncthreads();   // all wavefronts are done reading the halo
