@@ -81,34 +81,60 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
 #pragma unroll
             for (int c = 0; c < OCT; c++) acc[a][b][c] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // ---- staging helpers (loads from clamped addresses, zeroing applied when the registers are stored) ----------
+    // ---- staging helpers (loads from clamped addresses, zeroing applied when the registers are stored). A thread
+    // stages the same places of every chunk: pixel, channel quad, row within the chunk, LDS offset and the part of
+    // the global offset that does not depend on the chunk are computed once; per chunk a load costs an add for the
+    // chunk's base and the compares of the slice and image borders. (Vector instructions issued while staging take
+    // issue slots from the MFMAs; recomputing these from a flat index cost ~40 of them per element.) -----------------
     float4 yreg[YQ], xreg[XQ];
     unsigned ymask = 0, xmask = 0;
     const int y_quads = p.steps2 * 4 * (OCB / 4);   // includes the zero pixels that pad the chunk to an even step count
+    int y_koff[YQ], y_goff[YQ], y_rr[YQ], y_lds[YQ];
+    bool y_ok[YQ];
+#pragma unroll
+    for (int u = 0; u < YQ; u++) {
+        const int idx = t + 256 * u;
+        const int px = idx / (OCB / 4), cq = (idx % (OCB / 4)) * 4;
+        const int rr = fdiv(px, p.d_OWp), ow = px - rr * OWp;
+        y_ok[u] = idx < y_quads && rr < R && ow < OW && oc0 + cq < p.OC;
+        y_rr[u] = rr;
+        y_koff[u] = rr * OW + ow;
+        y_goff[u] = y_koff[u] * p.OC + oc0 + cq;
+        y_lds[u] = idx < y_quads ? px * YS + cq : -1;
+    }
+    int x_goff[XQ], x_rr[XQ], x_lds[XQ];
+    bool x_ok[XQ];
+#pragma unroll
+    for (int u = 0; u < XQ; u++) {
+        const int idx = t + 256 * u;
+        const int px = idx >> 4, cq = (idx & 15) * 4;
+        const int rr = fdiv(px, p.d_PW), cp = px - rr * PW;
+        const int iw = cp - p.pw;
+        x_ok[u] = (unsigned)iw < (unsigned)p.IW && ic0 + cq < p.IC;
+        x_rr[u] = rr;
+        x_goff[u] = (rr * p.IW + iw) * p.IC + ic0 + cq;
+        x_lds[u] = cp * DWR_XS + cq;
+    }
 
     // deltaY rows oh0 .. oh0+R-1 of image n; chunk pixel (rr, ow) lives at LDS pixel index rr*OWp + ow
     auto load_y = [&](int n, int oh0) {
         ymask = 0;
+        const int kbase = (n * OH + oh0) * OW;           // uniform
+        const unsigned kspan = (unsigned)(k_end - k_start);
 #pragma unroll
         for (int u = 0; u < YQ; u++) {
-            const int idx = t + 256 * u;
-            const int px = idx / (OCB / 4), cq = (idx % (OCB / 4)) * 4;
-            const int rr = fdiv(px, p.d_OWp), ow = px - rr * OWp;
-            const int oh = oh0 + rr;
-            const int k = (n * OH + oh) * OW + ow;
-            const bool ok = idx < y_quads && rr < R && ow < OW && oh < OH && k >= k_start && k < k_end && oc0 + cq < p.OC;
-            yreg[u] = *reinterpret_cast<const float4 *>(p.dY + (((size_t)k * p.OC + oc0 + cq) & (size_t)(-(long)ok)));
+            const bool ok = y_ok[u] && y_rr[u] < OH - oh0 && (unsigned)(kbase + y_koff[u] - k_start) < kspan;
+            const size_t off = ok ? (size_t)kbase * p.OC + y_goff[u] : 0;
+            yreg[u] = *reinterpret_cast<const float4 *>(p.dY + off);
             ymask |= (unsigned)ok << u;
         }
     };
     auto store_y = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < YQ; u++) {
-            const int idx = t + 256 * u;
-            if (idx < y_quads) {
-                const int px = idx / (OCB / 4), cq = (idx % (OCB / 4)) * 4;
+            if (y_lds[u] >= 0) {
                 const bool ok = (ymask >> u) & 1u;
-                *reinterpret_cast<float4 *>(Ybuf + buf * ybuf_floats + px * YS + cq) =
+                *reinterpret_cast<float4 *>(Ybuf + buf * ybuf_floats + y_lds[u]) =
                     make_float4(ok ? yreg[u].x : 0.f, ok ? yreg[u].y : 0.f, ok ? yreg[u].z : 0.f, ok ? yreg[u].w : 0.f);
             }
         }
@@ -117,31 +143,24 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
     // the image become zeros); padded row rp lives in slot rp % SLOTS
     auto load_x = [&](int n, int rp0, int nrows) {
         xmask = 0;
-        const int quads = nrows * PW * 16;
+        const int base = ((n * p.IH + rp0 - p.ph) * p.IW) * p.IC;   // uniform; may point before the image (then no row is valid)
 #pragma unroll
         for (int u = 0; u < XQ; u++) {
-            const int idx = t + 256 * u;
-            const int px = idx >> 4, cq = (idx & 15) * 4;
-            const int rr = fdiv(px, p.d_PW), cp = px - rr * PW;
-            const int ih = rp0 + rr - p.ph, iw = cp - p.pw;
-            const bool ok = idx < quads && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW && ic0 + cq < p.IC;
-            const int off = (((n * p.IH + ih) * p.IW + iw) * p.IC + ic0 + cq) & -(int)ok;
+            const bool ok = x_ok[u] && x_rr[u] < nrows && (unsigned)(rp0 - p.ph + x_rr[u]) < (unsigned)p.IH;
+            const int off = ok ? base + x_goff[u] : 0;
             xreg[u] = *reinterpret_cast<const float4 *>(p.X + off);
             xmask |= (unsigned)ok << u;
         }
     };
     auto store_x = [&](int rp0, int nrows) {
-        const int quads = nrows * PW * 16;
+        const int s0 = rp0 - fdiv(rp0, p.d_SLOTS) * SLOTS;          // uniform
 #pragma unroll
         for (int u = 0; u < XQ; u++) {
-            const int idx = t + 256 * u;
-            if (idx < quads) {
-                const int px = idx >> 4;
-                const int rr = fdiv(px, p.d_PW), cp = px - rr * PW;
-                const int rp = rp0 + rr;
-                const int slot = rp - fdiv(rp, p.d_SLOTS) * SLOTS;
+            if (x_rr[u] < nrows) {
+                int slot = s0 + x_rr[u];                             // x_rr < R <= SLOTS
+                slot -= slot >= SLOTS ? SLOTS : 0;
                 const bool ok = (xmask >> u) & 1u;
-                *reinterpret_cast<float4 *>(Xring + slot * slot_floats + cp * DWR_XS + (idx & 15) * 4) =
+                *reinterpret_cast<float4 *>(Xring + slot * slot_floats + x_lds[u]) =
                     make_float4(ok ? xreg[u].x : 0.f, ok ? xreg[u].y : 0.f, ok ? xreg[u].z : 0.f, ok ? xreg[u].w : 0.f);
             }
         }
