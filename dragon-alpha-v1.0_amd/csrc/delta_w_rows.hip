@@ -37,6 +37,7 @@ struct DwRowsArgs {
     int GK, GK_slice, GZ;
     int OWp;     // OW rounded up to a multiple of 4 (pixels beyond OW are staged as zeros)
     int PW;      // OWp + FW - 1 input columns staged per row; staged column cp holds iw = cp - pw
+    int PWA;     // columns allocated per row slot: PW, or PW + 8 zero columns when R = 1 (see the single-row loop)
     int R;       // output rows multiplied per step (a "chunk"); R*OWp <= 64 and R*PW <= 64
     int CPI;     // chunks per image = ceil(OH / R)
     int SLOTS;   // input-row slots in LDS = 2R + FH - 1
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
 
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int R = p.R, OWp = p.OWp, PW = p.PW, SLOTS = p.SLOTS;
-    const int ybuf_floats = p.steps2 * 4 * YS, slot_floats = PW * DWR_XS;
+    const int ybuf_floats = p.steps2 * 4 * YS, slot_floats = p.PWA * DWR_XS;
     float *Ybuf = smem;                               // [2][R*OWp][YS]
     float *Xring = smem + 2 * ybuf_floats;            // [SLOTS][PW][DWR_XS]
 
@@ -197,6 +198,12 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
         load_y(n, ci * R);
         store_y(0);
         stage_window(n, ci * R);
+        // columns PW .. PWA-1 of every slot stay zero for the whole kernel (nothing is staged there)
+        for (int idx = t; idx < SLOTS * (p.PWA - PW) * (DWR_XS / 4); idx += 256) {
+            const int per_slot = (p.PWA - PW) * (DWR_XS / 4);
+            const int slot = idx / per_slot, rest = idx - slot * per_slot;
+            *reinterpret_cast<float4 *>(Xring + slot * slot_floats + PW * DWR_XS + rest * 4) = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
         __syncthreads();
 
         const int steps2 = p.steps2;
@@ -283,16 +290,50 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
                     __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);   // up to 3 LDS reads
                 }
             };
-            frags(a0, b0);
-            for (int k4 = 0; k4 < steps2; k4 += 2) {
-                __builtin_amdgcn_sched_barrier(0);
-                frags(a1, b1);
-                mfmas(a0, b0);
-                interleave();
-                __builtin_amdgcn_sched_barrier(0);
+            if (R == 1) {
+                // One output row per chunk: the read positions only ever advance by 4 pixels, so they live in
+                // per-lane pointers bumped by a constant (scalar bookkeeping is not free either: every scalar
+                // instruction of the wave delays its next MFMA by two to three cycles, and the general path below
+                // spends ~23 of them per step). The step that pads the chunk to an even count and the read-ahead
+                // past the last step run into the 8 zero columns behind the row.
+                const float *yp = yb;
+                const float *xp[FH];
+#pragma unroll
+                for (int fh = 0; fh < FH; fh++) xp[fh] = xb + xo[fh];
+                auto frags1 = [&](float (&a)[OCT], float (&b)[FH][FW]) {
+#pragma unroll
+                    for (int c = 0; c < OCT; c++) a[c] = yp[16 * c];
+#pragma unroll
+                    for (int fh = 0; fh < FH; fh++) {
+#pragma unroll
+                        for (int fw = 0; fw < FW; fw++) b[fh][fw] = xp[fh][fw * DWR_XS];
+                        xp[fh] += 4 * DWR_XS;
+                    }
+                    yp += 4 * YS;
+                };
+                frags1(a0, b0);
+                for (int k4 = 0; k4 < steps2; k4 += 2) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags1(a1, b1);
+                    mfmas(a0, b0);
+                    interleave();
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags1(a0, b0);
+                    mfmas(a1, b1);
+                    interleave();
+                }
+            } else {
                 frags(a0, b0);
-                mfmas(a1, b1);
-                interleave();
+                for (int k4 = 0; k4 < steps2; k4 += 2) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags(a1, b1);
+                    mfmas(a0, b0);
+                    interleave();
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags(a0, b0);
+                    mfmas(a1, b1);
+                    interleave();
+                }
             }
 
             if (!has_next) break;
@@ -349,12 +390,13 @@ static hipError_t launch_dwr(hipStream_t stream, DwRowsArgs a)
     a.R = (a.OH + nchunks - 1) / nchunks;
     a.CPI = (a.OH + a.R - 1) / a.R;
     a.SLOTS = 2 * a.R + FH - 1;
+    a.PWA = a.R == 1 ? a.PW + 8 : a.PW;
     a.steps2 = ((a.R * a.OWp) / 4 + 1) & ~1;
     a.d_R = make_fastdiv(a.R);
     a.d_SLOTS = make_fastdiv(a.SLOTS);
     a.d_OWp = make_fastdiv(a.OWp);
     a.d_PW = make_fastdiv(a.PW);
-    const size_t lds = ((size_t)2 * a.steps2 * 4 * YS + (size_t)a.SLOTS * a.PW * DWR_XS) * sizeof(float);
+    const size_t lds = ((size_t)2 * a.steps2 * 4 * YS + (size_t)a.SLOTS * a.PWA * DWR_XS) * sizeof(float);
     if (lds > 160 * 1024) return hipErrorNotSupported;
     auto kern = delta_w_rows_kernel<FH, FW, OCT>;
     static size_t configured = 0;

@@ -94,8 +94,10 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
 
     // ---- filter fragments straight from global memory -------------------------------------------------
     // lane (l16, q) of wavefront w needs, for channel group g of a half tap, B[c = 16g + 4q + s][oc0 + 16w + l16].
-    // Address = (uniform base of the half tap, kept in scalar registers) + (per-lane byte offset, fixed for the whole
-    // kernel), so a load costs no vector arithmetic.
+    // Address = (uniform base of the half tap, kept in scalar registers) + (per-lane 32-bit byte offset, fixed for the
+    // whole kernel): the scalar-base form of the load instruction, no vector arithmetic. The empty asm keeps the
+    // zero-extension of the offset next to the load; hoisted out of the tap loop (as it is otherwise) the offsets
+    // become 64-bit register pairs and every load is preceded by a 64-bit vector add.
     const int b_co = oc0 + 16 * w + l16;
     const bool b_cov = b_co < p.CO;   // columns beyond CO are never stored; clamp their loads to a valid address
     unsigned b_lane[2][4];
@@ -111,7 +113,10 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
             // RAGGED: channels beyond AC (AC % 4 == 0: four at a time) are fetched from the half tap's first element
             const unsigned ok = RAGGED ? (unsigned)-(int)(icbase + 16 * g + 4 * q < p.AC) : ~0u;
 #pragma unroll
-            for (int s = 0; s < 4; s++) b[g][s] = *reinterpret_cast<const float *>(sb + (b_lane[g][s] & ok));
+            for (int s = 0; s < 4; s++) {
+                if (!RAGGED) asm volatile("" : "+v"(b_lane[g][s]));   // value unchanged
+                b[g][s] = *reinterpret_cast<const float *>(sb + (b_lane[g][s] & ok));
+            }
         }
     };
     // channels beyond AC: the halo holds zeros there, but 0 * (whatever the clamped load returned) must
@@ -128,14 +133,22 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
 
     const int taps = p.TH * p.TW;
 
-    // A fragments of one 16-channel chunk: chunk ck (0..3) of tap (th, tw) starts 16*ck floats into the pixel
-    auto read_a = [&](floatx4 (&a)[TILES], int th, int tw, int ck) {
-        // a strided layer keeps the columns of a row de-interleaved (plane tw % sw), so that the 16 pixels of a tile
-        // are neighbours in LDS whatever the stride and the bank pattern is the stride-1 one
-        const int twq = fdiv(tw, p.d_sw), twr = tw - twq * p.sw;
-        const float *hs = Hs + (th * RP + twr * p.PWp + twq) * TC_PS + 16 * ck;
+    // A fragments of one 16-channel chunk: chunk ck (0..3) of the current tap starts 16*ck floats into the pixel. The
+    // per-lane offsets cur[] point at the current tap and are moved by a uniform amount from tap to tap (adding the
+    // tap's offset at every read cost one vector add per tile and chunk, and a vector instruction takes five to
+    // nine cycles from the MFMAs). A strided layer keeps the columns of a row de-interleaved
+    // (plane tw % sw), so that the 16 pixels of a tile are neighbours in LDS whatever the stride and the bank
+    // pattern is the stride-1 one.
+    int cur[TILES];
 #pragma unroll
-        for (int i = 0; i < TILES; i++) a[i] = *reinterpret_cast<const floatx4 *>(hs + abase[i]);
+    for (int i = 0; i < TILES; i++) cur[i] = abase[i];
+    auto tap_offset = [&](int th, int tw) {
+        const int twq = fdiv(tw, p.d_sw), twr = tw - twq * p.sw;
+        return (th * RP + twr * p.PWp + twq) * TC_PS;
+    };
+    auto read_a = [&](floatx4 (&a)[TILES], int ck) {
+#pragma unroll
+        for (int i = 0; i < TILES; i++) a[i] = *reinterpret_cast<const floatx4 *>(Hs + cur[i] + 16 * ck);
     };
     auto mfma_chunk = [&](const floatx4 (&a)[TILES], const float (&b)[4]) {
 #pragma unroll
@@ -229,8 +242,8 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
         // harmlessly re-fetches tap (0,0) of this one at the very end. The scheduling barriers pin each prefetch in
         // front of the chunk that hides its latency; left alone the compiler sinks the loads to their first use.
         __builtin_amdgcn_s_setprio(0);
-        int th = 0, tw = 0;
-        read_a(aP, 0, 0, 0);
+        int th = 0, tw = 0, coff = 0;   // cur[] is at tap (0, 0) here
+        read_a(aP, 0);
         for (int tap = 0; tap < taps; tap++) {
             int nth = th, ntw = tw + 1, nic = ic0;
             if (ntw == p.TW) { ntw = 0; nth = th + 1; }
@@ -239,22 +252,28 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
             load_b(bB, ic0 + 32, th, tw);
             __builtin_amdgcn_sched_barrier(0);
             mask_b(bA, ic0);
-            read_a(aQ, th, tw, 1);
+            read_a(aQ, 1);
             mfma_chunk(aP, bA[0]);
             spread_reads();
             __builtin_amdgcn_sched_barrier(0);
-            read_a(aP, th, tw, 2);
+            read_a(aP, 2);
             mfma_chunk(aQ, bA[1]);
             spread_reads();
             __builtin_amdgcn_sched_barrier(0);
             load_b(bA, nic, nth, ntw);
             __builtin_amdgcn_sched_barrier(0);
             mask_b(bB, ic0 + 32);
-            read_a(aQ, th, tw, 3);
+            read_a(aQ, 3);
             mfma_chunk(aP, bB[0]);
             spread_reads();
             __builtin_amdgcn_sched_barrier(0);
-            read_a(aP, nth, ntw, 0);   // after the last tap of a pass: re-read once the next halo is staged
+            {   // on to the next tap (after the last one: back to tap (0, 0))
+                const int noff = tap_offset(nth, ntw), d = noff - coff;
+                coff = noff;
+#pragma unroll
+                for (int i = 0; i < TILES; i++) cur[i] += d;
+            }
+            read_a(aP, 0);   // after the last tap of a pass: re-read once the next halo is staged
             mfma_chunk(aQ, bB[1]);
             spread_reads();
             __builtin_amdgcn_sched_barrier(0);
