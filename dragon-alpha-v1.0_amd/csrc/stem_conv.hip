@@ -86,6 +86,21 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
     float *Os = Xs + w * (16 * ST_OS);
 
     const int window_quads = p.IHB * IWB;
+    // A thread stages the same window positions for every block: row, column and relative offset are computed once
+    // (the first eight of them; a window of more than 2048 pixels takes the general path below).
+    int st_r[8], st_c[8], st_off[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        const int idx = min(t + 256 * u, window_quads - 1);
+        st_r[u] = fdiv(idx, p.d_IWB);
+        st_c[u] = idx - st_r[u] * IWB;
+        st_off[u] = (st_r[u] * p.IW + st_c[u]) * 4;
+    }
+    // columns of the output block this lane stores: pixel 4*pp + q, channels oc0 + 4*l16 .. +3
+    int out_off[4];
+#pragma unroll
+    for (int pp = 0; pp < 4; pp++) out_off[pp] = (4 * pp + q) * p.OC + oc0 + 4 * l16;
+    const bool oc_ok = oc0 + 4 * l16 < p.OC;   // OC % 4 == 0: four channels valid together
     for (int blk = blockIdx.x; blk < p.blocks; blk += gridDim.x) {
         const int n = fdiv(blk, p.d_bhw), rem = blk - n * p.d_bhw.d;
         const int bh = fdiv(rem, p.d_bw), bw = rem - bh * p.d_bw.d;
@@ -94,7 +109,27 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
 
         __syncthreads();   // filter staged (first block) / previous block's output patches drained
         // ---- input window -> LDS: 8 loads in flight per thread, zeros outside the image ------------------------------
-        for (int base = 0; base < window_quads; base += 256 * 8) {
+        {
+            float4 v[8];
+            unsigned okmask = 0;
+            const int blockbase = ((n * p.IH + ih0) * p.IW + iw0) * 4;   // uniform; may lie before the image
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const bool ok = t + 256 * u < window_quads && (unsigned)(ih0 + st_r[u]) < (unsigned)p.IH &&
+                                (unsigned)(iw0 + st_c[u]) < (unsigned)p.IW;
+                v[u] = *reinterpret_cast<const float4 *>(p.X + (ok ? blockbase + st_off[u] : 0));
+                okmask |= (unsigned)ok << u;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int idx = t + 256 * u;
+                const bool ok = (okmask >> u) & 1u;
+                if (idx < window_quads)
+                    *reinterpret_cast<float4 *>(Xs + idx * 4) =
+                        make_float4(ok ? v[u].x : 0.f, ok ? v[u].y : 0.f, ok ? v[u].z : 0.f, ok ? v[u].w : 0.f);
+            }
+        }
+        for (int base = 256 * 8; base < window_quads; base += 256 * 8) {   // windows of more than 2048 pixels
             float4 v[8];
             unsigned okmask = 0;
 #pragma unroll
@@ -151,6 +186,7 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int oh = oh0 + 4 * w + i;
+            float *yrow = p.Y + ((size_t)(n * p.OH + oh) * p.OW + ow0) * p.OC;   // uniform
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -160,9 +196,8 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
             for (int pp = 0; pp < 4; pp++) {
                 const int col = 4 * pp + q, ow = ow0 + col;
                 const float4 v = *reinterpret_cast<const float4 *>(Os + col * ST_OS + 4 * l16);
-                if (oh < p.OH && ow < p.OW && oc0 + 4 * l16 < p.OC)   // OC % 4 == 0: four channels valid together
-                    *reinterpret_cast<float4 *>(p.Y + ((size_t)(n * p.OH + oh) * p.OW + ow) * p.OC + oc0 + 4 * l16) =
-                        add_bias4(v, p.bias, oc0 + 4 * l16);
+                if (oh < p.OH && ow < p.OW && oc_ok)
+                    *reinterpret_cast<float4 *>(yrow + out_off[pp]) = add_bias4(v, p.bias, oc0 + 4 * l16);
             }
             __builtin_amdgcn_wave_barrier();
         }
