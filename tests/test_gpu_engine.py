@@ -191,3 +191,46 @@ def test_engine_scratch_is_recycled_after_sync(dev, eng):
             eng.conv3D(y.data_ptr(), IH, IH, x.data_ptr(), IH, IH, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1)
         eng.sync()
         check(dev.get(y), want, "repeat")
+
+
+def _random_cases(count, seed):
+    """Seeded random layer geometries inside what the Java engine accepts (EngineCore.java:630-678: sh <= FH, sw <= FW,
+    pads below the filter size, N/IC/OC multiples of 4): the analogue of the reference's sweeps over ragged sizes
+    (Cuda_conv3D_test.java:155-156), with image widths on both sides of the kernels' row-width classes (16/32/48
+    padded columns), channel counts on both sides of 64 and all filter sizes the specialised kernels serve."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    cases = []
+    while len(cases) < count:
+        F_ = int(rng.choice([1, 2, 3, 3, 3, 4, 5, 7]))
+        FW_ = F_ if rng.random() < 0.8 else int(rng.choice([1, 2, 3, 4, 5]))
+        sh = int(rng.integers(1, min(F_, 3) + 1)) if rng.random() < 0.4 else 1
+        sw = min(sh, FW_) if rng.random() < 0.8 else int(rng.integers(1, min(FW_, 3) + 1))
+        ph, pw = int(rng.integers(0, F_)), int(rng.integers(0, FW_))
+        IH, IW = int(rng.integers(F_, 41)), int(rng.integers(FW_, 61))
+        IC = 4 * int(rng.choice([1, 2, 3, 8, 16, 17, 24, 32, 40]))
+        OC = 4 * int(rng.choice([1, 2, 5, 8, 16, 16, 19, 32, 48]))
+        N = int(rng.choice([4, 8]))
+        OH, OW = out_dim(IH, IW, F_, FW_, sh, sw, ph, pw)
+        if OH < 1 or OW < 1 or N * IH * IW * IC > 3_000_000 or N * OH * OW * OC > 3_000_000:
+            continue
+        cases.append((N, IH, IW, IC, OC, F_, FW_, sh, sw, ph, pw))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(36, 20240611))
+def test_engine_random_geometries(dev, eng, case):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = case
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    seed = 7000 + (hash(case) % 1000)
+    X, W, dY = normal((N, IH, IW, IC), seed), he_normal(OC, FH, FW, IC, seed + 1), normal((N, OH, OW, OC), seed + 2)
+    x, w, dy = dev.put(X), dev.put(W), dev.put(dY)
+    y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    dx = dev.empty(N, IH, IW, IC, fill=float("nan"))
+    dw = dev.empty(OC, FH, FW, IC, fill=float("nan"))
+    eng.conv3D(y.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
+    eng.dconv3D_deltaX(dx.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
+    eng.dconv3D_deltaW(dw.data_ptr(), FH, FW, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, sh, sw, ph, pw)
+    eng.sync()
+    check(dev.get(y), O.conv3D_f64(X, W, sh, sw, ph, pw), "conv3D %s" % (case,))
+    check(dev.get(dx), O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw), "deltaX %s" % (case,))
+    check(dev.get(dw), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "deltaW %s" % (case,))
