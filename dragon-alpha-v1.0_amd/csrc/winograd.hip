@@ -28,6 +28,7 @@ struct WinoArgs {
     int ph, pw;
     int TR, TC;       // tile rows / columns per image: ceil(OH/2), ceil(OW/2)
     int ntiles;       // N*TR*TC
+    int x_bytes;      // size of X in bytes (< 2 GB)
     FastDiv d_TC, d_TRC;
 };
 
@@ -94,31 +95,37 @@ __global__ __launch_bounds__(256, 2) void winograd_f2x2_kernel(const WinoArgs p)
             x_iw0 = 2 * tx - p.pw;
         }
     }
+    // Loads go through buffer descriptors: address = descriptor base + uniform offset (scalar register: the chunk's
+    // first channel) + per-lane 32-bit offset (fixed for the whole kernel), and an offset beyond the descriptor's size
+    // returns 0. A thread loads the same 16 pixels of its tile for every channel chunk, so the per-lane offsets are
+    // computed once, pixels outside the image get an offset that is out of range (their zeros come from the range
+    // check), and a load costs no vector arithmetic. (Computing a 64-bit address per load took ~5 vector instructions
+    // for each of the 80 loads of a chunk - more issue slots than the chunk's 128 MFMAs.)
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
+    constexpr unsigned OUT_OF_RANGE = 0x80000000u;   // descriptors are below 2 GB (host-checked)
     float2 d[4][4];
-    unsigned dmask = 0;
+    unsigned p_off[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int ih = x_ih0 + i, iw = x_iw0 + j;
+            const bool ok = (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
+            p_off[i][j] = ok ? (unsigned)(x_base + (ih * p.IW + iw) * p.IC + xq) * 4u : OUT_OF_RANGE;
+        }
     auto load_patch = [&](int icc) {   // icc: first channel of the 16-channel chunk
-        dmask = 0;
-        const bool cv = icc + xq < p.IC;   // IC % 4 == 0: a channel pair is valid as a whole
+        // IC % 4 == 0: a channel pair is valid as a whole; only the last chunk of a ragged IC has invalid pairs
+        const bool cv = icc + xq < p.IC;
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int ih = x_ih0 + i, iw = x_iw0 + j;
-                const bool ok = cv && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
-                const int off = (x_base + (ih * p.IW + iw) * p.IC + icc + xq) & -(int)ok;
-                d[i][j] = *reinterpret_cast<const float2 *>(p.X + off);
-                dmask |= (unsigned)ok << (4 * i + j);
+                const unsigned off = (icc + 16 <= p.IC || cv) ? p_off[i][j] : OUT_OF_RANGE;
+                d[i][j] = __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, off, icc * 4, 0));
             }
     };
     auto transform_store = [&](int buf) {   // V = B^T d B, B^T = [[1,0,-1,0],[0,1,1,0],[0,-1,1,0],[0,1,0,-1]]
         float *V = smem + buf * WG_VBUF + xt * 16 + xq;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const bool ok = (dmask >> (4 * i + j)) & 1u;
-                d[i][j] = make_float2(ok ? d[i][j].x : 0.f, ok ? d[i][j].y : 0.f);
-            }
         auto sub = [](float2 a, float2 b) { return make_float2(a.x - b.x, a.y - b.y); };
         auto add = [](float2 a, float2 b) { return make_float2(a.x + b.x, a.y + b.y); };
         float2 r[4][4];
@@ -143,11 +150,16 @@ __global__ __launch_bounds__(256, 2) void winograd_f2x2_kernel(const WinoArgs p)
     const int b_co = oc0 + 16 * w + l16;
     const int b_col = b_co < p.OC ? b_co : 0;   // columns beyond OC are never stored
     const int xi_stride = p.IC * p.OC;
-    auto load_b = [&](float (&b)[4], int xi, int icc) {
-        const int c = icc + 4 * q;
-        const int ok = -(int)(c < p.IC);
+    const __amdgpu_buffer_rsrc_t u_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.U), 0, 16 * xi_stride * 4, 0x00020000);
+    unsigned u_lane[4];   // byte offset of this lane's elements inside a (frequency, 16-channel chunk) block of U
 #pragma unroll
-        for (int s = 0; s < 4; s++) b[s] = p.U[(xi * xi_stride + (c + s) * p.OC + b_col) & ok];
+    for (int s = 0; s < 4; s++) u_lane[s] = (unsigned)((4 * q + s) * p.OC + b_col) * 4u;
+    auto load_b = [&](float (&b)[4], int xi, int icc) {
+        // channels beyond IC (last chunk of a ragged IC) read the next frequency's block or, at the very end, get the
+        // range check's zero; the fragment is zeroed where it is used
+        const int block = (xi * xi_stride + icc * p.OC) * 4;   // uniform
+#pragma unroll
+        for (int s = 0; s < 4; s++) b[s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(u_rsrc, u_lane[s], block, 0));
     };
 
     const int nchunks = (p.IC + 15) >> 4;
@@ -250,7 +262,8 @@ hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, f
     a.ph = ph; a.pw = pw;
     a.TR = (OH + 1) / 2; a.TC = (OW + 1) / 2;
     const long nt = (long)N * a.TR * a.TC;
-    if (nt >= (1L << 30) || 16L * IC * OC >= (1L << 31)) return hipErrorNotSupported;
+    if (nt >= (1L << 30) || 16L * IC * OC * 4 >= (1L << 31) || (long)N * IH * IW * IC * 4 >= (1L << 31)) return hipErrorNotSupported;   // buffer descriptors below 2 GB
+    a.x_bytes = (int)((long)N * IH * IW * IC * 4);
     a.ntiles = (int)nt;
     a.d_TC = make_fastdiv(a.TC);
     a.d_TRC = make_fastdiv(a.TR * a.TC);
