@@ -51,8 +51,9 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
     const int k_end = (z != p.GZ - 1) ? k_start + p.GK_slice : p.GK;
     // pixel groups (4 pixels) of this wavefront's part; GK and GK_slice are multiples of 4
     const int groups = (k_end - k_start) >> 2;
-    const int g0 = (k_start >> 2) + (int)((long)groups * kpart / KSPLIT);
-    const int g1 = live ? (k_start >> 2) + (int)((long)groups * (kpart + 1) / KSPLIT) : g0;
+    // (uniform over the wavefront; said so explicitly, because the pixel-group offset of a load must be a scalar)
+    const int g0 = __builtin_amdgcn_readfirstlane((k_start >> 2) + (int)((long)groups * kpart / KSPLIT));
+    const int g1 = __builtin_amdgcn_readfirstlane(live ? (k_start >> 2) + (int)((long)groups * (kpart + 1) / KSPLIT) : g0);
 
     floatx4 acc[4][4];
 #pragma unroll
@@ -60,14 +61,18 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    const float *py = p.dY + (size_t)q * p.OC + ocb * 64 + 4 * l16;
-    const float *px = p.X + (size_t)q * p.IC + icb * 64 + 4 * l16;
+    // Loads through buffer descriptors: descriptor base + uniform offset of the pixel group (scalar register) + fixed
+    // per-lane offset, no vector arithmetic per load (a 64-bit address per load cost 6 vector instructions per 16 MFMAs).
+    const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.dY), 0, p.GK * p.OC * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.GK * p.IC * 4, 0x00020000);
+    const unsigned y_lane = (unsigned)(q * p.OC + ocb * 64 + 4 * l16) * 4u;
+    const unsigned x_lane = (unsigned)(q * p.IC + icb * 64 + 4 * l16) * 4u;
     floatx4 ya[DWP_D], xa[DWP_D];
     const bool do_bias = p.dB != nullptr && live && icb == 0;   // one wavefront set per block row of deltaW
     floatx4 bsum = floatx4{0.f, 0.f, 0.f, 0.f};
     auto load = [&](int d, int g) {   // g is clamped by the caller to a group of this part
-        ya[d] = *reinterpret_cast<const floatx4 *>(py + (size_t)g * 4 * p.OC);
-        xa[d] = *reinterpret_cast<const floatx4 *>(px + (size_t)g * 4 * p.IC);
+        ya[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, y_lane, g * 16 * p.OC, 0));
+        xa[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_lane, g * 16 * p.IC, 0));
     };
     // The ring loop is free of branches on purpose: the loads of a slot are waited for by count (14 younger loads may
     // stay in flight), and the count is only known when every load and every use is executed unconditionally. With a
@@ -153,7 +158,7 @@ hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const flo
                                    int GK, int IC, int OC, int GK_slice, int GZ, float *dB, float *dB_buf)
 {
     if ((IC & 63) || (OC & 63) || IC < 64 || OC < 64 || (GK & 3) || (GK_slice & 3) || GK < 4) return hipErrorNotSupported;
-    if ((size_t)GK * (size_t)(IC > OC ? IC : OC) >= (1ull << 31)) return hipErrorNotSupported;
+    if ((size_t)GK * (size_t)(IC > OC ? IC : OC) * 4 >= (1ull << 31)) return hipErrorNotSupported;   // buffer descriptors below 2 GB
     static int cu_count[64] = {0};   // per device; a racing first call writes the same value
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorNotSupported;
