@@ -33,6 +33,7 @@ struct DwPointwiseArgs {
     int TPW;                // blocks per workgroup (1, 2, 4 or 8); 8 / TPW wavefronts share a block
 };
 
+template <int V> struct DwpFlag { static constexpr int value = V; };
 constexpr int DWP_D = 8;    // pixel groups in flight per wavefront
 
 __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPointwiseArgs p)
@@ -77,16 +78,18 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
     // The ring loop is free of branches on purpose: the loads of a slot are waited for by count (14 younger loads may
     // stay in flight), and the count is only known when every load and every use is executed unconditionally. With a
     // branch around the MFMAs of a slot each round of the ring began with a wait for all 16 loads.
-    const float bias_on = do_bias ? 1.f : 0.f;
-    auto multiply = [&](int d) {
+    // The ring exists twice, with and without the column sums of deltaY for the bias gradient (4 vector instructions
+    // per 16 MFMAs that a call without deltaB, and every workgroup but those of the first input-channel block, skip).
+    auto ring = [&](auto with_bias) {
+        constexpr bool WB = decltype(with_bias)::value != 0;
+        auto multiply = [&](int d) {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+            for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ya[d][i], xa[d][j], acc[i][j], 0, 0, 0);
-        bsum += ya[d] * bias_on;
-    };
-    if (g0 < g1) {
+                for (int j = 0; j < 4; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ya[d][i], xa[d][j], acc[i][j], 0, 0, 0);
+            if (WB) bsum += ya[d];
+        };
 #pragma unroll
         for (int d = 0; d < DWP_D; d++) load(d, min(g0 + d, g1 - 1));
         int g = g0;
@@ -102,6 +105,10 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
 #pragma unroll
         for (int d = 0; d < DWP_D - 1; d++)
             if (d < rest) multiply(d);
+    };
+    if (g0 < g1) {
+        if (__builtin_amdgcn_readfirstlane((int)do_bias)) ring(DwpFlag<1>{});
+        else ring(DwpFlag<0>{});
     }
 
     // ---- bias gradient: lanes q = 0..3 hold different pixels of the same 4 channels (wavefront shuffles), the parts
