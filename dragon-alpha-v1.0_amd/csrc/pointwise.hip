@@ -28,6 +28,7 @@ struct PointwiseArgs {
     int b_kmajor;
     int tiles;        // ceil(M / 16)
     int strided;      // 0: row = m
+    int a_bytes;      // size of A in bytes (< 2 GB)
     const float *bias;   // NULL or [ldn]
     int AH, AW, sh, sw;
     FastDiv d_OW, d_OHW;
@@ -62,21 +63,35 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
     if (t == 0) *queue = t_begin + 8;
 
     const int n_off = blockIdx.y * N, ldn = p.ldn;
-    auto load_a = [&](floatx4 (&a)[KB][4], int tile) {
-        int m = min(tile * 16 + l16, p.M - 1);   // rows past M are computed from a valid row and never stored
+    // A and O are addressed through buffer descriptors: descriptor base + uniform offset of the tile (scalar register)
+    // + a per-lane offset that is fixed for the whole kernel, no vector arithmetic per load or store. Rows past M are
+    // beyond the descriptors: their loads return zeros and their stores are dropped, so nothing in the tile loop is
+    // conditional and every wait can be counted exactly (a wait placed after a store whose execution is uncertain would
+    // have to wait for every store to be acknowledged). A strided layer (input rows thinned) computes its lane offsets
+    // per tile.
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.O, 0, p.M * ldn * 4, 0x00020000);
+    const unsigned a_lane = (unsigned)(l16 * K + 4 * q) * 4u;
+    const unsigned o_lane = (unsigned)(q * ldn + n_off + 4 * l16) * 4u;
+    auto load_a = [&](floatx4 (&a)[KB][4], int tile_) {
+        const int tile = __builtin_amdgcn_readfirstlane(tile_);   // uniform, said so: the tile offset must be a scalar
+        unsigned voff = a_lane;
+        int soff = tile * 16 * K * 4;
         if (p.strided) {
+            const int m = min(tile * 16 + l16, p.M - 1);
             const int n = fdiv(m, p.d_OHW), rem = m - n * p.d_OHW.d;
             const int oh = fdiv(rem, p.d_OW), ow = rem - oh * p.d_OW.d;
-            m = (n * p.AH + oh * p.sh) * p.AW + ow * p.sw;
+            voff = (unsigned)(((n * p.AH + oh * p.sh) * p.AW + ow * p.sw) * K + 4 * q) * 4u;
+            soff = 0;
         }
-        const float *src = p.A + (size_t)m * K + 4 * q;
 #pragma unroll
         for (int kb = 0; kb < KB; kb++)
 #pragma unroll
-            for (int c = 0; c < 4; c++) a[kb][c] = *reinterpret_cast<const floatx4 *>(src + 64 * kb + 16 * c);
+            for (int c = 0; c < 4; c++)
+                a[kb][c] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, voff + (64 * kb + 16 * c) * 4, soff, 0));
     };
     floatx4 aP[KB][4], aQ[KB][4];
-    int tile = t_begin + w;
+    int tile = __builtin_amdgcn_readfirstlane(t_begin + w);
 
     // ---- filter -> LDS, once: 8 loads in flight per thread, consecutive lanes along k so that the transposing
     // stores of the [K][N] layout fall into consecutive banks. The first tile's A fragments are requested right
@@ -147,12 +162,7 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
             const int g = i / GS, r = i % GS;
             return *reinterpret_cast<const floatx4 *>(blg + (4 * g + (r & 3)) * 16 * KS + (r >> 2) * 16);
         };
-        // Rows past M repeat row M-1 (their fragments were loaded from it, so they hold the same values) and are
-        // stored to it again: no store is conditional, and the waits of the loop can be counted exactly. A wait
-        // placed after a store whose execution is uncertain would have to wait for every store to be acknowledged.
-        float *dst[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) dst[i] = p.O + (size_t)min(tile * 16 + 4 * i + q, p.M - 1) * ldn + n_off + 64 * g0 + 4 * l16;
+        const int o_tile = __builtin_amdgcn_readfirstlane((tile * 16 * ldn + 64 * g0) * 4);   // uniform
         floatx4 bsel[NGX];
         if constexpr (NGX == NG) {
 #pragma unroll
@@ -178,7 +188,9 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
         };
         auto store = [&](int g) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) *reinterpret_cast<floatx4 *>(dst[i] + 64 * g) = v[i] + bsel[g];
+            for (int i = 0; i < 4; i++)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v[i] + bsel[g]),
+                                                       o_rsrc, o_lane, o_tile + (4 * i * ldn + 64 * g) * 4, 0);
         };
         b[0] = read_b(0);
         b[1] = read_b(1);
@@ -251,7 +263,7 @@ hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, 
 {
     const long Ml = (long)Nimg * OH * OW;
     if (Ml < 1 || (K & 63) || K < 64 || K > 256 || (N & 63) || N < 64) return hipErrorNotSupported;
-    if ((size_t)Nimg * AH * AW * K >= (1ull << 31) || (size_t)Ml * N >= (1ull << 31)) return hipErrorNotSupported;
+    if ((size_t)Nimg * AH * AW * K * 4 >= (1ull << 31) || (size_t)Ml * N * 4 >= (1ull << 31)) return hipErrorNotSupported;   // buffer descriptors below 2 GB
     static int cu_count[64] = {0};   // per device; a racing first call writes the same value
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorNotSupported;
@@ -267,6 +279,7 @@ hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, 
     a.tiles = (a.M + 15) / 16;
     a.strided = !(sh == 1 && sw == 1 && OH == AH && OW == AW);
     a.AH = AH; a.AW = AW; a.sh = sh; a.sw = sw;
+    a.a_bytes = (int)((size_t)Nimg * AH * AW * K * 4);
     a.d_OW = make_fastdiv(OW);
     a.d_OHW = make_fastdiv(OH * OW);
     const int KB = K / 64;
