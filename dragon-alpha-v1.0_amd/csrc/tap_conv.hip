@@ -38,6 +38,9 @@ struct TapConvArgs {
     int lds_rows;     // halo rows reserved in LDS
     int b_off, b_sth, b_stw, b_sc;
     const float *bias;   // NULL or [CO]
+    int full_units;   // units of 16*TILES pixels that are processed whole, dealt round-robin to the persistent workgroups
+    int pieces;       // the remaining units cut into piece_split pieces of piece_tiles tiles each, one piece per workgroup
+    int piece_split, piece_tiles;
     FastDiv d_OW, d_OHW, d_PHt, d_PWt, d_sw;
 };
 
@@ -49,31 +52,23 @@ constexpr int TC_OS = 64 + 4;         // output staging row stride (floats)
 // RAGGED: AC is not a multiple of 64, so the last pass has channels beyond AC whose filter fragments
 // must be zeroed (kept out of the common case: the extra selects would pull the wait for the
 // prefetched fragment in front of the MFMAs).
+// One unit: output pixels [m0, min(m0 + 16*TILES, m_lim)) x output channels [oc0, oc0 + 64).
 template <int TILES, bool RAGGED>
-__global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
+__device__ __forceinline__ void tap_conv_unit(const TapConvArgs &p, float *smem, const int m0, const int m_lim, const int oc0)
 {
     constexpr int P = TILES * 16;
-    extern __shared__ __attribute__((aligned(16))) float smem[];
     float *Hs = smem;   // [lds_rows][sw planes][PWp][TC_PS] (+ one spare slot); reused as output staging [P][TC_OS]
 
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
     const int l16 = lane & 15, q = lane >> 4;
-
-    // Consecutive units share halo rows: keep them on one XCD (workgroups are dealt round-robin to the
-    // 8 XCDs) so the shared rows are served by that XCD's L2.
-    const int G = gridDim.x;
-    const int xcd = blockIdx.x & 7, xi = blockIdx.x >> 3;
-    const int unit = xcd * (G >> 3) + min(xcd, G & 7) + xi;
-    const int m0 = unit * P;
-    const int oc0 = blockIdx.y * 64;
     const int OW = p.d_OW.d, OHW = p.d_OHW.d, PHt = p.PHt, PWt = p.PWt, RP = p.RP;
 
     // first padded global row held in LDS, and how many rows this unit needs (<= p.lds_rows, host-checked)
     const int n_first = fdiv(m0, p.d_OHW);
     const int oh_first = fdiv(m0 - n_first * OHW, p.d_OW);
     const int pgr0 = n_first * PHt + oh_first * p.sh;
-    const int m_last = min(m0 + P, p.M) - 1;
+    const int m_last = min(m0 + P, m_lim) - 1;
     const int n_last = fdiv(m_last, p.d_OHW);
     const int oh_last = fdiv(m_last - n_last * OHW, p.d_OW);
     const int rows = n_last * PHt + oh_last * p.sh + p.TH - 1 - pgr0 + 1;
@@ -82,7 +77,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
     int abase[TILES];
 #pragma unroll
     for (int i = 0; i < TILES; i++) {
-        const int m = min(m0 + 16 * i + l16, p.M - 1);
+        const int m = min(m0 + 16 * i + l16, m_lim - 1);
         const int n = fdiv(m, p.d_OHW), rem = m - n * OHW;
         const int oh = fdiv(rem, p.d_OW), ow = rem - oh * OW;
         abase[i] = ((n * PHt + oh * p.sh - pgr0) * RP + ow) * TC_PS + 4 * q;
@@ -140,12 +135,12 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
     // (plane tw % sw), so that the 16 pixels of a tile are neighbours in LDS whatever the stride and the bank
     // pattern is the stride-1 one.
     int cur[TILES];
-#pragma unroll
-    for (int i = 0; i < TILES; i++) cur[i] = abase[i];
     auto tap_offset = [&](int th, int tw) {
         const int twq = fdiv(tw, p.d_sw), twr = tw - twq * p.sw;
         return (th * RP + twr * p.PWp + twq) * TC_PS;
     };
+#pragma unroll
+    for (int i = 0; i < TILES; i++) cur[i] = abase[i];
     auto read_a = [&](floatx4 (&a)[TILES], int ck) {
 #pragma unroll
         for (int i = 0; i < TILES; i++) a[i] = *reinterpret_cast<const floatx4 *>(Hs + cur[i] + 16 * ck);
@@ -296,10 +291,53 @@ __global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
     for (int idx = t; idx < P * 16; idx += 256) {
         const int pix = idx >> 4, cq = (idx & 15) * 4;
         const int m = m0 + pix;
-        if (m < p.M && oc0 + cq < p.CO)
+        if (m < m_lim && oc0 + cq < p.CO)
             *reinterpret_cast<float4 *>(p.O + (size_t)m * p.CO + oc0 + cq) =
                 add_bias4(*reinterpret_cast<const float4 *>(Os + pix * TC_OS + cq), p.bias, oc0 + cq);
     }
+}
+
+// The grid is persistent: as many workgroups as the device holds at once (per block of 64 output channels), each taking
+// whole units round-robin. Units that would make a partial last round are cut into pieces of fewer tiles, one piece
+// per workgroup, so that every workgroup does the same amount of work (c4b: 896 units on 512 workgroups).
+// Consecutive units share halo rows: each XCD (workgroups are dealt round-robin to the 8 XCDs) works on a contiguous
+// run of units, so the shared rows are served by that XCD's L2.
+template <int TILES, bool RAGGED>
+__global__ __launch_bounds__(256, 2) void tap_conv_kernel(const TapConvArgs p)
+{
+    constexpr int P = TILES * 16;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    const int oc0 = blockIdx.y * 64;
+    const int G = gridDim.x;
+    const int xcd = blockIdx.x & 7, xi = blockIdx.x >> 3;
+    const int wgs = (G >> 3) + (xcd < (G & 7) ? 1 : 0);   // workgroups on this XCD
+    bool first = true;
+    auto whole_units = [&]() {
+        const int U = p.full_units;
+        const int lo = xcd * (U >> 3) + min(xcd, U & 7), n = (U >> 3) + (xcd < (U & 7) ? 1 : 0);
+        for (int i = xi; i < n; i += wgs) {
+            if (!first) __syncthreads();   // the previous unit's output staging has been read
+            first = false;
+            tap_conv_unit<TILES, RAGGED>(p, smem, (lo + i) * P, p.M, oc0);
+        }
+    };
+    auto one_piece = [&]() {
+        const int U = p.pieces;
+        const int lo = xcd * (U >> 3) + min(xcd, U & 7), n = (U >> 3) + (xcd < (U & 7) ? 1 : 0);
+        for (int i = xi; i < n; i += wgs) {
+            const int piece = lo + i;
+            const int unit = p.full_units + piece / p.piece_split, k = piece - (piece / p.piece_split) * p.piece_split;
+            const int m0 = unit * P + k * 16 * p.piece_tiles;
+            const int m_lim = min(min(m0 + 16 * p.piece_tiles, (unit + 1) * P), p.M);
+            if (m0 >= m_lim) continue;
+            if (!first) __syncthreads();
+            first = false;
+            if (p.piece_tiles > 2) tap_conv_unit<4, RAGGED>(p, smem, m0, m_lim, oc0);
+            else tap_conv_unit<2, RAGGED>(p, smem, m0, m_lim, oc0);
+        }
+    };
+    whole_units();
+    one_piece();
 }
 
 // Rows of LDS halo the worst unit needs: output rows spanned by P consecutive pixels, TH-1 extra rows,
@@ -327,7 +365,7 @@ static int tap_conv_lds_rows(int M, int P, int OH, int OW, int TH, int sh, int P
 }
 
 template <int TILES, bool RAGGED>
-static hipError_t launch_tc(hipStream_t stream, const TapConvArgs &a, size_t lds)
+static hipError_t launch_tc(hipStream_t stream, TapConvArgs a, size_t lds, int cus)
 {
     auto kern = tap_conv_kernel<TILES, RAGGED>;
     static size_t configured = 0;
@@ -337,8 +375,26 @@ static hipError_t launch_tc(hipStream_t stream, const TapConvArgs &a, size_t lds
         if (e != hipSuccess) return e;
         configured = lds;
     }
-    dim3 grid((a.M + TILES * 16 - 1) / (TILES * 16), (a.CO + 63) / 64, 1);
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
+    const int units = (a.M + TILES * 16 - 1) / (TILES * 16), ocb = (a.CO + 63) / 64;
+    const int slots = cus * (2 * lds <= 160 * 1024 ? 2 : 1);   // workgroups the device holds at once
+    int G = slots / ocb;
+    if (G < 1) G = 1;
+    if (G > units) G = units;
+    a.full_units = (units / G) * G;
+    a.pieces = 0; a.piece_split = 1; a.piece_tiles = TILES;
+    const int left = units - a.full_units;
+    if (left > 0) {
+        int split = G / left;                  // pieces per left-over unit that still give every workgroup at most one
+        if (split > TILES / 2) split = TILES / 2;
+        if (split >= 2) {
+            a.piece_split = split;
+            a.piece_tiles = (TILES + split - 1) / split;   // <= 4 for TILES <= 8
+            a.pieces = left * split;
+        } else {
+            a.full_units = units;              // more than half a round is left: whole units for the first workgroups
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(G, ocb, 1), dim3(256), lds, stream, a);
     return hipGetLastError();
 }
 
@@ -370,6 +426,15 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
     a.d_PHt = make_fastdiv(a.PHt);
     a.d_PWt = make_fastdiv(a.PWt);
 
+    static int cu_count[64] = {0};   // per device; a racing first call writes the same value
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorNotSupported;
+    if (cu_count[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return hipErrorNotSupported;
+        cu_count[dev] = n;
+    }
+    const int cus = cu_count[dev];
     // pixels per workgroup: 7 tiles (112) when that divides the row/image structure better, else 8 (128)
     const int OHW = OH * OW;
     int tiles = 8;
@@ -385,8 +450,8 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
         const size_t lds = halo * sizeof(float);
         if (lds <= budget) {
             const bool ragged = (AC % TC_ICC) != 0;
-            if (tiles == 7) return ragged ? launch_tc<7, true>(stream, a, lds) : launch_tc<7, false>(stream, a, lds);
-            return ragged ? launch_tc<8, true>(stream, a, lds) : launch_tc<8, false>(stream, a, lds);
+            if (tiles == 7) return ragged ? launch_tc<7, true>(stream, a, lds, cus) : launch_tc<7, false>(stream, a, lds, cus);
+            return ragged ? launch_tc<8, true>(stream, a, lds, cus) : launch_tc<8, false>(stream, a, lds, cus);
         }
         tiles = (tiles == 8) ? 7 : 8;
     }
