@@ -398,6 +398,11 @@ static hipError_t launch_tc(hipStream_t stream, TapConvArgs a, size_t lds, int c
     return hipGetLastError();
 }
 
+hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const float *B, float *O,
+                                    int N, int AH, int AW, int AC, int OH, int OW, int CO,
+                                    int TH, int TW, int ph, int pw,
+                                    int b_off, int b_sth, int b_stw, int b_sc, const float *bias, int cus);
+
 // Returns hipErrorNotSupported when the shape does not fit this kernel (caller falls back to the
 // generic implicit GEMM); otherwise launches.
 hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
@@ -435,6 +440,11 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
         cu_count[dev] = n;
     }
     const int cus = cu_count[dev];
+    if (sh == 1 && sw == 1) {   // the variant that prefetches the halo, where it applies
+        const hipError_t e = launch_tap_conv_prefetch(stream, A, B, O, N, AH, AW, AC, OH, OW, CO, TH, TW, ph, pw,
+                                                      b_off, b_sth, b_stw, b_sc, bias, cus);
+        if (e != hipErrorNotSupported) return e;
+    }
     // pixels per workgroup: 7 tiles (112) when that divides the row/image structure better, else 8 (128)
     const int OHW = OH * OW;
     int tiles = 8;
