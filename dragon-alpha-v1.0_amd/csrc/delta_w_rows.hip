@@ -48,7 +48,7 @@ struct DwRowsArgs {
 constexpr int DWR_XS = 80;   // X row slot pixel stride (floats): 64 channels + 16
 
 template <int FH, int FW, int OCT>
-__global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p)
+__global__ __launch_bounds__(256, OCT <= 2 ? 2 : 1) void delta_w_rows_kernel(const DwRowsArgs p)   // <= 256 registers where two workgroups fit a compute unit
 {
     constexpr int OCB = 16 * OCT;
     constexpr int YS = OCB + 16;             // deltaY pixel stride (floats): 32, 48 or 80
@@ -82,87 +82,83 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
 #pragma unroll
             for (int c = 0; c < OCT; c++) acc[a][b][c] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // ---- staging helpers (loads from clamped addresses, zeroing applied when the registers are stored). A thread
-    // stages the same places of every chunk: pixel, channel quad, row within the chunk, LDS offset and the part of
-    // the global offset that does not depend on the chunk are computed once; per chunk a load costs an add for the
-    // chunk's base and the compares of the slice and image borders. (Vector instructions issued while staging take
-    // issue slots from the MFMAs; recomputing these from a flat index cost ~40 of them per element.) -----------------
+    // ---- staging helpers. Loads go through buffer descriptors, one over this slice's pixels of deltaY and one over
+    // the image of X that is being read: an offset outside the descriptor returns zeros, which is exactly what pixels
+    // outside the slice, rows above and below the image and (through a per-thread offset that is out of range from the
+    // start) padding columns, padding pixels and channels past the end need. A thread stages the same places of every
+    // chunk: its byte offset within the chunk and its LDS place are computed once, per chunk a load costs one add.
+    // (Vector instructions issued while staging take issue slots from the MFMAs - a wave has its SIMD to itself here -
+    // and compares, selects and 64-bit address arithmetic per element were a tenth of the kernel's time.)
+    // Threads beyond the last element repeat the last element (same bytes to the same place). ---------------------
+    constexpr int NEVER = 0x40000000;   // plus any offset within a slice or an image (host-checked < 2^29): still out of range
+    const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(p.dY) + (size_t)k_start * p.OC, 0, k_start < k_end ? (k_end - k_start) * p.OC * 4 : 0, 0x00020000);
+    const int x_image_bytes = p.IH * p.IW * p.IC * 4;
     float4 yreg[YQ], xreg[XQ];
-    unsigned ymask = 0, xmask = 0;
     const int y_quads = p.steps2 * 4 * (OCB / 4);   // includes the zero pixels that pad the chunk to an even step count
-    int y_koff[YQ], y_goff[YQ], y_rr[YQ], y_lds[YQ];
-    bool y_ok[YQ];
+    int y_voff[YQ], y_rr[YQ], y_lds[YQ];
 #pragma unroll
     for (int u = 0; u < YQ; u++) {
-        const int idx = t + 256 * u;
+        const int idx = min(t + 256 * u, y_quads - 1);
         const int px = idx / (OCB / 4), cq = (idx % (OCB / 4)) * 4;
         const int rr = fdiv(px, p.d_OWp), ow = px - rr * OWp;
-        y_ok[u] = idx < y_quads && rr < R && ow < OW && oc0 + cq < p.OC;
+        const bool ok = rr < R && ow < OW && oc0 + cq < p.OC;
         y_rr[u] = rr;
-        y_koff[u] = rr * OW + ow;
-        y_goff[u] = y_koff[u] * p.OC + oc0 + cq;
-        y_lds[u] = idx < y_quads ? px * YS + cq : -1;
+        y_voff[u] = ok ? ((rr * OW + ow) * p.OC + oc0 + cq) * 4 : NEVER;
+        y_lds[u] = px * YS + cq;
     }
-    int x_goff[XQ], x_rr[XQ], x_lds[XQ];
-    bool x_ok[XQ];
+    const int x_quads = R * PW * 16;
+    int x_voff[XQ], x_rr[XQ], x_lds[XQ];
 #pragma unroll
     for (int u = 0; u < XQ; u++) {
-        const int idx = t + 256 * u;
+        const int idx = min(t + 256 * u, x_quads - 1);
         const int px = idx >> 4, cq = (idx & 15) * 4;
         const int rr = fdiv(px, p.d_PW), cp = px - rr * PW;
         const int iw = cp - p.pw;
-        x_ok[u] = (unsigned)iw < (unsigned)p.IW && ic0 + cq < p.IC;
+        const bool ok = (unsigned)iw < (unsigned)p.IW && ic0 + cq < p.IC;
         x_rr[u] = rr;
-        x_goff[u] = (rr * p.IW + iw) * p.IC + ic0 + cq;
+        x_voff[u] = ok ? ((rr * p.IW + iw) * p.IC + ic0 + cq) * 4 : NEVER;
         x_lds[u] = cp * DWR_XS + cq;
     }
 
     // deltaY rows oh0 .. oh0+R-1 of image n; chunk pixel (rr, ow) lives at LDS pixel index rr*OWp + ow
     auto load_y = [&](int n, int oh0) {
-        ymask = 0;
-        const int kbase = (n * OH + oh0) * OW;           // uniform
-        const unsigned kspan = (unsigned)(k_end - k_start);
+        const int rel = __builtin_amdgcn_readfirstlane((((n * OH + oh0) * OW) - k_start) * p.OC * 4);   // may be negative
 #pragma unroll
         for (int u = 0; u < YQ; u++) {
-            const bool ok = y_ok[u] && y_rr[u] < OH - oh0 && (unsigned)(kbase + y_koff[u] - k_start) < kspan;
-            const size_t off = ok ? (size_t)kbase * p.OC + y_goff[u] : 0;
-            yreg[u] = *reinterpret_cast<const float4 *>(p.dY + off);
-            ymask |= (unsigned)ok << u;
+            int off = y_voff[u] + rel;
+            if (R > 1) off = y_rr[u] < OH - oh0 ? off : NEVER;   // the image's last chunk may have fewer rows
+            yreg[u] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, off, 0, 0));
         }
     };
     auto store_y = [&](int buf) {
 #pragma unroll
-        for (int u = 0; u < YQ; u++) {
-            if (y_lds[u] >= 0) {
-                const bool ok = (ymask >> u) & 1u;
-                *reinterpret_cast<float4 *>(Ybuf + buf * ybuf_floats + y_lds[u]) =
-                    make_float4(ok ? yreg[u].x : 0.f, ok ? yreg[u].y : 0.f, ok ? yreg[u].z : 0.f, ok ? yreg[u].w : 0.f);
-            }
-        }
+        for (int u = 0; u < YQ; u++) *reinterpret_cast<float4 *>(Ybuf + buf * ybuf_floats + y_lds[u]) = yreg[u];
     };
-    // `nrows` (<= R) padded input rows rp0 .. rp0+nrows-1 of image n (padded row rp holds ih = rp - ph; rows outside
-    // the image become zeros); padded row rp lives in slot rp % SLOTS
-    auto load_x = [&](int n, int rp0, int nrows) {
-        xmask = 0;
-        const int base = ((n * p.IH + rp0 - p.ph) * p.IW) * p.IC;   // uniform; may point before the image (then no row is valid)
+    // R padded input rows rp0 .. rp0+R-1 of image n (padded row rp holds ih = rp - ph; rows outside the image are out
+    // of the descriptor's range: zeros); padded row rp lives in slot rp % SLOTS
+    auto load_x = [&](int n, int rp0) {
+        const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(p.X) + (size_t)n * p.IH * p.IW * p.IC, 0, x_image_bytes, 0x00020000);
+        const int rel = __builtin_amdgcn_readfirstlane((rp0 - p.ph) * p.IW * p.IC * 4);   // may be negative
 #pragma unroll
-        for (int u = 0; u < XQ; u++) {
-            const bool ok = x_ok[u] && x_rr[u] < nrows && (unsigned)(rp0 - p.ph + x_rr[u]) < (unsigned)p.IH;
-            const int off = ok ? base + x_goff[u] : 0;
-            xreg[u] = *reinterpret_cast<const float4 *>(p.X + off);
-            xmask |= (unsigned)ok << u;
-        }
+        for (int u = 0; u < XQ; u++)
+            xreg[u] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_voff[u] + rel, 0, 0));
     };
-    auto store_x = [&](int rp0, int nrows) {
+    auto store_x = [&](int rp0, int nrows) {   // nrows < R: only the first nrows of the R rows are kept
         const int s0 = rp0 - fdiv(rp0, p.d_SLOTS) * SLOTS;          // uniform
+        if (R == 1) {
+            float *slot = Xring + s0 * slot_floats;
 #pragma unroll
-        for (int u = 0; u < XQ; u++) {
-            if (x_rr[u] < nrows) {
-                int slot = s0 + x_rr[u];                             // x_rr < R <= SLOTS
-                slot -= slot >= SLOTS ? SLOTS : 0;
-                const bool ok = (xmask >> u) & 1u;
-                *reinterpret_cast<float4 *>(Xring + slot * slot_floats + x_lds[u]) =
-                    make_float4(ok ? xreg[u].x : 0.f, ok ? xreg[u].y : 0.f, ok ? xreg[u].z : 0.f, ok ? xreg[u].w : 0.f);
+            for (int u = 0; u < XQ; u++) *reinterpret_cast<float4 *>(slot + x_lds[u]) = xreg[u];
+        } else {
+#pragma unroll
+            for (int u = 0; u < XQ; u++) {
+                if (x_rr[u] < nrows) {
+                    int slot = s0 + x_rr[u];                             // x_rr < R <= SLOTS
+                    slot -= slot >= SLOTS ? SLOTS : 0;
+                    *reinterpret_cast<float4 *>(Xring + slot * slot_floats + x_lds[u]) = xreg[u];
+                }
             }
         }
     };
@@ -170,22 +166,18 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
     // before the first is stored so that their latencies overlap
     auto stage_window = [&](int n, int oh0) {
         float4 wreg[FH][XQ];
-        unsigned wmask[FH];
 #pragma unroll
         for (int pc = 0; pc < FH; pc++) {
-            const int nrows = min(R, R + FH - 1 - pc * R);     // <= 0: nothing left for this piece
-            load_x(n, oh0 + pc * R, nrows);
+            load_x(n, oh0 + pc * R);
 #pragma unroll
             for (int u = 0; u < XQ; u++) wreg[pc][u] = xreg[u];
-            wmask[pc] = xmask;
         }
 #pragma unroll
         for (int pc = 0; pc < FH; pc++) {
-            const int nrows = min(R, R + FH - 1 - pc * R);
+            const int nrows = min(R, R + FH - 1 - pc * R);     // <= 0: nothing left for this piece
 #pragma unroll
             for (int u = 0; u < XQ; u++) xreg[u] = wreg[pc][u];
-            xmask = wmask[pc];
-            store_x(oh0 + pc * R, nrows);
+            if (nrows > 0) store_x(oh0 + pc * R, nrows);
         }
     };
 
@@ -215,7 +207,7 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
             const bool same_image = n2 == n;
             if (has_next) {
                 load_y(n2, ci2 * R);
-                if (same_image) load_x(n, oh0 + R + FH - 1, R);   // the R new padded rows of the next chunk
+                if (same_image) load_x(n, oh0 + R + FH - 1);   // the R new padded rows of the next chunk
             }
 
             // ---- bias gradient: column sums of the staged deltaY chunk (its masked pixels are zeros). Wavefront w adds
@@ -290,6 +282,17 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
                     __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);   // up to 3 LDS reads
                 }
             };
+            // Half-way through the chunk the next chunk's rows (requested above, arrived by now) go to their LDS places:
+            // the other deltaY buffer and the ring slots the current chunk does not read. Done after the loop instead,
+            // these stores, their barrier and the refill of the read pipeline cost 2500 cycles per chunk with no MFMA
+            // in flight (a chunk of 56 pixels multiplies for 11400).
+            const int mid = (steps2 / 2) & ~1;
+            auto store_next = [&]() {
+                if (has_next) {
+                    store_y((it + 1) & 1);
+                    if (same_image) store_x(oh0 + R + FH - 1, R);
+                }
+            };
             if (R == 1) {
                 // One output row per chunk: the read positions only ever advance by 4 pixels, so they live in
                 // per-lane pointers bumped by a constant (scalar bookkeeping is not free either: every scalar
@@ -312,7 +315,18 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
                     yp += 4 * YS;
                 };
                 frags1(a0, b0);
-                for (int k4 = 0; k4 < steps2; k4 += 2) {
+                for (int k4 = 0; k4 < mid; k4 += 2) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags1(a1, b1);
+                    mfmas(a0, b0);
+                    interleave();
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags1(a0, b0);
+                    mfmas(a1, b1);
+                    interleave();
+                }
+                store_next();
+                for (int k4 = mid; k4 < steps2; k4 += 2) {
                     __builtin_amdgcn_sched_barrier(0);
                     frags1(a1, b1);
                     mfmas(a0, b0);
@@ -324,7 +338,18 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
                 }
             } else {
                 frags(a0, b0);
-                for (int k4 = 0; k4 < steps2; k4 += 2) {
+                for (int k4 = 0; k4 < mid; k4 += 2) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags(a1, b1);
+                    mfmas(a0, b0);
+                    interleave();
+                    __builtin_amdgcn_sched_barrier(0);
+                    frags(a0, b0);
+                    mfmas(a1, b1);
+                    interleave();
+                }
+                store_next();
+                for (int k4 = mid; k4 < steps2; k4 += 2) {
                     __builtin_amdgcn_sched_barrier(0);
                     frags(a1, b1);
                     mfmas(a0, b0);
@@ -337,8 +362,6 @@ __global__ __launch_bounds__(256, 1) void delta_w_rows_kernel(const DwRowsArgs p
             }
 
             if (!has_next) break;
-            store_y((it + 1) & 1);
-            if (same_image) store_x(oh0 + R + FH - 1, R);
             __syncthreads();
             if (!same_image) {   // first chunk of the next image: its whole window is new
                 stage_window(n2, 0);
@@ -396,6 +419,12 @@ static hipError_t launch_dwr(hipStream_t stream, DwRowsArgs a)
     a.d_SLOTS = make_fastdiv(a.SLOTS);
     a.d_OWp = make_fastdiv(a.OWp);
     a.d_PW = make_fastdiv(a.PW);
+    {   // the staging loads address a slice of deltaY and an image of X with 32-bit offsets that must stay below 2^29
+        const long last = (long)a.GK - (long)a.GK_slice * (a.GZ - 1);
+        const long slice = last > a.GK_slice ? last : a.GK_slice;
+        if ((slice + (long)a.R * a.OW) * a.OC * 4 >= (1L << 29)) return hipErrorNotSupported;
+        if ((long)(a.IH + a.R + FH) * a.IW * a.IC * 4 >= (1L << 29)) return hipErrorNotSupported;
+    }
     const size_t lds = ((size_t)2 * a.steps2 * 4 * YS + (size_t)a.SLOTS * a.PWA * DWR_XS) * sizeof(float);
     if (lds > 160 * 1024) return hipErrorNotSupported;
     auto kern = delta_w_rows_kernel<FH, FW, OCT>;

@@ -12,9 +12,9 @@
 // left-over unit), which is what lets it fetch the next unit's rows early.
 //
 // LDS: two buffers of [lds_rows][PWt][40] floats (32 channels + 8: a pixel stride of 160 bytes = 16*(4k+2) keeps the
-// 128-bit reads conflict-free) and one spare 16-byte slot. The buffer a unit's last pass has used holds the output
-// staging [P][68] afterwards. Synchronisation: one barrier per pass (everyone has finished reading the current
-// buffer, everyone's prefetch writes into the other one have landed), two more per unit around the output transpose.
+// 128-bit reads conflict-free) and one spare 16-byte slot. Synchronisation: one barrier per pass (everyone has
+// finished reading the current buffer, everyone's prefetch writes into the other one have landed); the output goes
+// from the accumulators straight to memory.
 //
 // Restrictions (the launcher answers hipErrorNotSupported and the caller uses tap_conv.hip): 3x3 taps, stride 1, AC a
 // multiple of 32, padded rows of 17..64 pixels, both buffers within 80 KB.
@@ -50,7 +50,6 @@ static __device__ __forceinline__ void pf_static_for(F &&f)
 }
 constexpr int PF_ICC = 32;            // input channels per pass
 constexpr int PF_PS = PF_ICC + 8;     // LDS pixel stride (floats)
-constexpr int PF_OS = 64 + 4;         // output staging row stride (floats)
 constexpr unsigned PF_OUT_OF_RANGE = 0x80000000u;   // beyond any descriptor (< 2 GB, host-checked): the load returns zeros
 
 // Halo of the pixels [m0, m_hi): first padded global row (n*PHt + ih + ph) and number of rows.
@@ -184,6 +183,8 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
     // SIMD's vector issue port, and the other workgroup's address arithmetic and stores at the same priority wait for
     // thousands of cycles (unit set-up 15000 cycles instead of 1000, measured).
     __builtin_amdgcn_s_setprio(3);
+    const float bias_v = (p.bias != nullptr && b_cov) ? p.bias[b_co] : 0.f;
+    const int o_lane = b_cov ? (4 * q * p.CO + b_co) * 4 : (int)PF_OUT_OF_RANGE;   // output byte offset of this lane within a tile
     int buf = 0;          // buffer that holds the halo of the pass about to run
     float bA[2][4];       // filter fragment of that pass's first tap
     load_b(bA, 0, 0, 0);
@@ -329,23 +330,20 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
             }
         }
 
-        // ---- epilogue: transpose through LDS so every output pixel row is written as whole 256-byte lines --------
-        float *Os = Hs + (buf ^ 1) * p.buf_floats;   // [16*T][PF_OS] in the buffer the last pass used
+        // ---- epilogue: accumulators straight to memory ----------------------------------------------------------------
+        // Lane (l16, q) holds pixels 16i + 4q + r, channel 16w + l16: one store instruction writes 64 contiguous bytes
+        // of four pixel rows; the other three quarters of those rows come from the other wavefronts and meet in L2.
+        // (A transpose through LDS gives whole 256-byte rows per instruction but needs two barriers, and its LDS traffic
+        // queues behind the reads of the other workgroup's MFMA loop: 12000 cycles per unit, measured.)
+        // The descriptor ends at the unit's last pixel, so rows past it are dropped by the range check.
+        const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.O, 0, m_hi * p.CO * 4, 0x00020000);
 #pragma unroll
         for (int i = 0; i < T; i++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) Os[(16 * i + 4 * q + r) * PF_OS + 16 * w + l16] = acc[i][r];
-        __syncthreads();
-        float4 o[T];
-#pragma unroll
-        for (int i = 0; i < T; i++) o[i] = *reinterpret_cast<const float4 *>(Os + (16 * i + (t >> 4)) * PF_OS + (t & 15) * 4);
-#pragma unroll
-        for (int i = 0; i < T; i++) {
-            const int m = m0 + 16 * i + (t >> 4), cq = (t & 15) * 4;
-            if (m < m_hi && oc0 + cq < p.CO)
-                *reinterpret_cast<float4 *>(p.O + (size_t)m * p.CO + oc0 + cq) = add_bias4(o[i], p.bias, oc0 + cq);
-        }
-        __syncthreads();   // the next unit's prefetch writes into this buffer
+            for (int r = 0; r < 4; r++) {
+                const int soff = __builtin_amdgcn_readfirstlane((m0 + 16 * i + r) * p.CO * 4);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[i][r] + bias_v), o_rsrc, o_lane, soff, 0);
+            }
     };
 
     while (idx < n_items) {
@@ -431,7 +429,7 @@ hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const fl
     const long M = (long)N * OH * OW;
     if ((long)N * PHt >= (1L << 24) || M >= (1L << 30)) return hipErrorNotSupported;
     const long a_bytes = (long)N * AH * AW * AC * 4;
-    if (a_bytes >= (1L << 31)) return hipErrorNotSupported;
+    if (a_bytes >= (1L << 31) || M * CO * 4 >= (1L << 31)) return hipErrorNotSupported;
 
     TapPfArgs a{};
     a.A = A; a.B = B; a.O = O; a.bias = bias;
@@ -453,8 +451,7 @@ hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const fl
     for (int attempt = 0; attempt < 2; attempt++) {
         const int P = tiles * 16;
         a.lds_rows = tap_pf_lds_rows(a.M, P, OH, OW, TH, PHt);
-        size_t bufsz = (size_t)a.lds_rows * PWt * PF_PS;
-        if (bufsz < (size_t)P * PF_OS) bufsz = (size_t)P * PF_OS;
+        const size_t bufsz = (size_t)a.lds_rows * PWt * PF_PS;
         a.buf_floats = (int)bufsz;
         const size_t lds = (2 * bufsz + 4) * sizeof(float);
         const int elems = a.lds_rows * cg, ept = (elems + TH * TW - 2) / (TH * TW - 1);
