@@ -47,7 +47,8 @@ struct DwRowsArgs {
 
 constexpr int DWR_XS = 80;   // X row slot pixel stride (floats): 64 channels + 16
 
-template <int FH, int FW, int OCT>
+// ONE_ROW: one output row per chunk (p.R == 1), which lets the compiler drop the multi-row loop and its bookkeeping.
+template <int FH, int FW, int OCT, bool ONE_ROW>
 __global__ __launch_bounds__(256, OCT <= 2 ? 2 : 1) void delta_w_rows_kernel(const DwRowsArgs p)   // <= 256 registers where two workgroups fit a compute unit
 {
     constexpr int OCB = 16 * OCT;
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256, OCT <= 2 ? 2 : 1) void delta_w_rows_kernel(con
     constexpr int XQ = 4;                    // float4 per thread per R new X rows  (R*PW <= 64, host-checked)
 
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    const int R = p.R, OWp = p.OWp, PW = p.PW, SLOTS = p.SLOTS;
+    const int R = ONE_ROW ? 1 : p.R, OWp = p.OWp, PW = p.PW, SLOTS = p.SLOTS;
     const int ybuf_floats = p.steps2 * 4 * YS, slot_floats = p.PWA * DWR_XS;
     float *Ybuf = smem;                               // [2][R*OWp][YS]
     float *Xring = smem + 2 * ybuf_floats;            // [SLOTS][PW][DWR_XS]
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(256, OCT <= 2 ? 2 : 1) void delta_w_rows_kernel(con
 #pragma unroll
         for (int u = 0; u < YQ; u++) {
             int off = y_voff[u] + rel;
-            if (R > 1) off = y_rr[u] < OH - oh0 ? off : NEVER;   // the image's last chunk may have fewer rows
+            if (!ONE_ROW) off = y_rr[u] < OH - oh0 ? off : NEVER;   // the image's last chunk may have fewer rows
             yreg[u] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, off, 0, 0));
         }
     };
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(256, OCT <= 2 ? 2 : 1) void delta_w_rows_kernel(con
     };
     auto store_x = [&](int rp0, int nrows) {   // nrows < R: only the first nrows of the R rows are kept
         const int s0 = rp0 - fdiv(rp0, p.d_SLOTS) * SLOTS;          // uniform
-        if (R == 1) {
+        if (ONE_ROW) {
             float *slot = Xring + s0 * slot_floats;
 #pragma unroll
             for (int u = 0; u < XQ; u++) *reinterpret_cast<float4 *>(slot + x_lds[u]) = xreg[u];
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(256, OCT <= 2 ? 2 : 1) void delta_w_rows_kernel(con
                     if (same_image) store_x(oh0 + R + FH - 1, R);
                 }
             };
-            if (R == 1) {
+            if constexpr (ONE_ROW) {
                 // One output row per chunk: the read positions only ever advance by 4 pixels, so they live in
                 // per-lane pointers bumped by a constant (scalar bookkeeping is not free either: every scalar
                 // instruction of the wave delays its next MFMA by two to three cycles, and the general path below
@@ -400,6 +401,22 @@ __global__ __launch_bounds__(256, OCT <= 2 ? 2 : 1) void delta_w_rows_kernel(con
                 }
 }
 
+template <int FH, int FW, int OCT, bool ONE_ROW>
+static hipError_t launch_dwr_rows(hipStream_t stream, const DwRowsArgs &a, size_t lds)
+{
+    auto kern = delta_w_rows_kernel<FH, FW, OCT, ONE_ROW>;
+    static size_t configured = 0;
+    if (lds > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = lds;
+    }
+    constexpr int OCB = 16 * OCT;
+    dim3 grid((a.IC + 63) / 64, (a.OC + OCB - 1) / OCB, a.GZ);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
+    return hipGetLastError();
+}
+
 template <int FH, int FW, int OCT>
 static hipError_t launch_dwr(hipStream_t stream, DwRowsArgs a)
 {
@@ -427,16 +444,7 @@ static hipError_t launch_dwr(hipStream_t stream, DwRowsArgs a)
     }
     const size_t lds = ((size_t)2 * a.steps2 * 4 * YS + (size_t)a.SLOTS * a.PWA * DWR_XS) * sizeof(float);
     if (lds > 160 * 1024) return hipErrorNotSupported;
-    auto kern = delta_w_rows_kernel<FH, FW, OCT>;
-    static size_t configured = 0;
-    if (lds > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = lds;
-    }
-    dim3 grid((a.IC + 63) / 64, (a.OC + OCB - 1) / OCB, a.GZ);
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
-    return hipGetLastError();
+    return a.R == 1 ? launch_dwr_rows<FH, FW, OCT, true>(stream, a, lds) : launch_dwr_rows<FH, FW, OCT, false>(stream, a, lds);
 }
 
 // Returns hipErrorNotSupported (nothing launched) when the layer does not fit; the caller then uses the generic kernel.
