@@ -66,13 +66,15 @@ static __device__ __forceinline__ float4 add_bias4(float4 v, const float *bias, 
 
 // Every forward launcher takes `bias` (NULL = none): bias[co] is added to each output row in the kernel's epilogue.
 
-// Stride-1 convolution with the input window staged once in LDS (tap_conv.hip). B must be contiguous
-// along the output channel: element (th, tw, c, co) at b_off + th*b_sth + tw*b_stw + c*b_sc + co.
+// Convolution with the input window staged in LDS (tap_conv.hip, tap_conv_prefetch.hip). Filter element (th, tw, c, co)
+// at b_off + th*b_sth + tw*b_stw + c*b_sc + co*b_sn; b_sn = 1 (contiguous along the output channel) fits every shape
+// these kernels take, b_sn != 1 with b_sc = 1 (contiguous along the input channel) the 3x3 stride-1 ones.
 // Returns hipErrorNotSupported (nothing launched) when the shape does not fit.
 hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
                            int N, int AH, int AW, int AC, int OH, int OW, int CO,
                            int TH, int TW, int ph, int pw,
-                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias = nullptr, int sh = 1, int sw = 1);
+                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias = nullptr, int sh = 1, int sw = 1,
+                           int b_sn = 1);
 
 // 1x1 stride-1 convolution as a streaming GEMM with the filter resident in LDS (pointwise.hip):
 // O[(n,oh,ow)][co] = sum_k A[n, oh*sh, ow*sw, k] * B(k, co), B given as [K][N] (b_kmajor) or [N][K]. Returns

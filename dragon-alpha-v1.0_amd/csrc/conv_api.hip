@@ -91,9 +91,14 @@ int forward(const char *fn, const int64_t *streams, int length,
         hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW, bias);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (layout == FILTER_CW && fwd_algo() != 3) {
-        hipError_t e = launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
-                                       0, FW * IC * OC, IC * OC, OC, bias, sh, sw);
+    if (fwd_algo() != 3) {
+        // W[OC,FH,FW,IC] as it is: taken by the 3x3 stride-1 kernel (128-bit fragment loads; measured the same speed as
+        // from CW), refused by the others, which then leaves the generic kernel
+        hipError_t e = layout == FILTER_CW
+            ? launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
+                              0, FW * IC * OC, IC * OC, OC, bias, sh, sw)
+            : launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
+                              0, FW * IC, IC, 1, bias, sh, sw, FH * FW * IC);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
 

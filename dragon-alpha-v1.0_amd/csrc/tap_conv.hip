@@ -401,14 +401,14 @@ static hipError_t launch_tc(hipStream_t stream, TapConvArgs a, size_t lds, int c
 hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const float *B, float *O,
                                     int N, int AH, int AW, int AC, int OH, int OW, int CO,
                                     int TH, int TW, int ph, int pw,
-                                    int b_off, int b_sth, int b_stw, int b_sc, const float *bias, int cus);
+                                    int b_off, int b_sth, int b_stw, int b_sc, int b_sn, const float *bias, int cus);
 
 // Returns hipErrorNotSupported when the shape does not fit this kernel (caller falls back to the
 // generic implicit GEMM); otherwise launches.
 hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
                            int N, int AH, int AW, int AC, int OH, int OW, int CO,
                            int TH, int TW, int ph, int pw,
-                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias, int sh, int sw)
+                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias, int sh, int sw, int b_sn)
 {
     if (sh < 1 || sw < 1 || sh > 4 || sw > 4) return hipErrorNotSupported;
     if (OH != (AH + 2 * ph - TH) / sh + 1 || OW != (AW + 2 * pw - TW) / sw + 1) return hipErrorNotSupported;
@@ -442,9 +442,10 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
     const int cus = cu_count[dev];
     if (sh == 1 && sw == 1) {   // the variant that prefetches the halo, where it applies
         const hipError_t e = launch_tap_conv_prefetch(stream, A, B, O, N, AH, AW, AC, OH, OW, CO, TH, TW, ph, pw,
-                                                      b_off, b_sth, b_stw, b_sc, bias, cus);
+                                                      b_off, b_sth, b_stw, b_sc, b_sn, bias, cus);
         if (e != hipErrorNotSupported) return e;
     }
+    if (b_sn != 1) return hipErrorNotSupported;   // the kernel below reads the filter along the output channel only
     // pixels per workgroup: 7 tiles (112) when that divides the row/image structure better, else 8 (128)
     const int OHW = OH * OW;
     int tiles = 8;

@@ -24,7 +24,7 @@ namespace alpha {
 
 struct TapPfArgs {
     const float *A;   // input activations [N, AH, AW, AC]
-    const float *B;   // filter; element (th, tw, c, co) at b_off + th*b_sth + tw*b_stw + c*b_sc + co
+    const float *B;   // filter; element (th, tw, c, co) at b_off + th*b_sth + tw*b_stw + c*b_sc + co*b_sn
     float *O;         // output [N, OH, OW, CO] dense
     const float *bias;   // NULL or [CO]
     int M, CO;        // N*OH*OW pixels, output channels
@@ -34,7 +34,7 @@ struct TapPfArgs {
     int lds_rows;     // halo rows reserved per buffer
     int buf_floats;   // floats per LDS buffer
     int a_bytes;      // size of A, < 2^31
-    int b_off, b_sth, b_stw, b_sc;
+    int b_off, b_sth, b_stw, b_sc, b_sn;   // either b_sn == 1 (output channel contiguous) or b_sc == 1 (input channel contiguous)
     int full_units, pieces, piece_split, piece_tiles;   // as in tap_conv.hip
     FastDiv d_OW, d_OHW, d_PHt;
 };
@@ -72,8 +72,9 @@ static __device__ __forceinline__ PfHalo pf_halo(const TapPfArgs &p, int m0, int
 }
 
 // TILES: tiles of a whole unit; CG: column groups of 32 padded pixels per row (1 or 2); EPT: halo elements a thread
-// requests per tap.
-template <int TILES, int CG, int EPT>
+// requests per tap; BK: the filter is contiguous along the input channel (W[OC,FH,FW,IC] as it is) instead of along the
+// output channel.
+template <int TILES, int CG, int EPT, bool BK>
 __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -160,23 +161,35 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
     };
 
     // ---- filter fragments straight from global memory (see tap_conv.hip) ----------------------------------------
+    // lane (l16, q) of wavefront w needs, for channel group g of a tap, B[c = 16g + 4q + s][oc0 + 16w + l16], s = 0..3.
+    // Output channel contiguous: eight 32-bit loads at (scalar base of the tap) + (fixed per-lane offset). Input
+    // channel contiguous: the four s of a group are neighbours, two 128-bit loads.
     const int b_co = oc0 + 16 * w + l16;
     const bool b_cov = b_co < p.CO;   // columns beyond CO are never stored; clamp their loads to a valid address
     unsigned b_lane[2][4];
 #pragma unroll
     for (int g = 0; g < 2; g++)
 #pragma unroll
-        for (int s = 0; s < 4; s++) b_lane[g][s] = (unsigned)(((16 * g + 4 * q + s) * p.b_sc + (b_cov ? b_co : 0)) * 4);
+        for (int s = 0; s < 4; s++)
+            b_lane[g][s] = BK ? (unsigned)(((b_cov ? b_co : 0) * p.b_sn + 16 * g + 4 * q) * 4)
+                              : (unsigned)(((16 * g + 4 * q + s) * p.b_sc + (b_cov ? b_co : 0)) * 4);
     auto load_b = [&](float (&b)[2][4], int icbase, int th, int tw) {
         const int sbase = __builtin_amdgcn_readfirstlane(p.b_off + th * p.b_sth + tw * p.b_stw + icbase * p.b_sc);
         const char *sb = reinterpret_cast<const char *>(p.B + sbase);
 #pragma unroll
-        for (int g = 0; g < 2; g++)
+        for (int g = 0; g < 2; g++) {
+            if (BK) {
+                asm volatile("" : "+v"(b_lane[g][0]));   // value unchanged; keeps the zero-extension next to the load
+                const float4 v = *reinterpret_cast<const float4 *>(sb + b_lane[g][0]);
+                b[g][0] = v.x; b[g][1] = v.y; b[g][2] = v.z; b[g][3] = v.w;
+            } else {
 #pragma unroll
-            for (int s = 0; s < 4; s++) {
-                asm volatile("" : "+v"(b_lane[g][s]));   // value unchanged; keeps the zero-extension next to the load
-                b[g][s] = *reinterpret_cast<const float *>(sb + b_lane[g][s]);
+                for (int s = 0; s < 4; s++) {
+                    asm volatile("" : "+v"(b_lane[g][s]));
+                    b[g][s] = *reinterpret_cast<const float *>(sb + b_lane[g][s]);
+                }
             }
+        }
     };
 
     // Everything outside the MFMA loops runs at a raised priority: a wavefront that issues MFMAs back to back keeps the
@@ -383,10 +396,10 @@ static int tap_pf_lds_rows(int M, int P, int OH, int OW, int TH, int PHt)
     return worst;
 }
 
-template <int TILES, int CG, int EPT>
-static hipError_t launch_pf(hipStream_t stream, TapPfArgs a, size_t lds, int cus)
+template <int TILES, int CG, int EPT, bool BK>
+static hipError_t launch_pf2(hipStream_t stream, TapPfArgs a, size_t lds, int cus)
 {
-    auto kern = tap_conv_prefetch_kernel<TILES, CG, EPT>;
+    auto kern = tap_conv_prefetch_kernel<TILES, CG, EPT, BK>;
     static size_t configured = 0;
     if (lds > configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -416,12 +429,19 @@ static hipError_t launch_pf(hipStream_t stream, TapPfArgs a, size_t lds, int cus
     return hipGetLastError();
 }
 
+template <int TILES, int CG, int EPT>
+static hipError_t launch_pf(hipStream_t stream, const TapPfArgs &a, size_t lds, int cus)
+{
+    return a.b_sn != 1 ? launch_pf2<TILES, CG, EPT, true>(stream, a, lds, cus) : launch_pf2<TILES, CG, EPT, false>(stream, a, lds, cus);
+}
+
 // Returns hipErrorNotSupported when the shape does not fit this kernel; otherwise launches.
 hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const float *B, float *O,
                                     int N, int AH, int AW, int AC, int OH, int OW, int CO,
                                     int TH, int TW, int ph, int pw,
-                                    int b_off, int b_sth, int b_stw, int b_sc, const float *bias, int cus)
+                                    int b_off, int b_sth, int b_stw, int b_sc, int b_sn, const float *bias, int cus)
 {
+    if (b_sn != 1 && (b_sc != 1 || (b_sn | b_sth | b_stw | b_off) % 4 != 0)) return hipErrorNotSupported;   // 128-bit fragment loads
     if (OH != AH + 2 * ph - TH + 1 || OW != AW + 2 * pw - TW + 1) return hipErrorNotSupported;
     if (AC % PF_ICC != 0 || TH != 3 || TW != 3) return hipErrorNotSupported;
     const int PHt = AH + 2 * ph, PWt = AW + 2 * pw;
@@ -438,7 +458,7 @@ hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const fl
     a.TH = TH; a.TW = TW; a.ph = ph; a.pw = pw;
     a.PHt = PHt; a.PWt = PWt;
     a.a_bytes = (int)a_bytes;
-    a.b_off = b_off; a.b_sth = b_sth; a.b_stw = b_stw; a.b_sc = b_sc;
+    a.b_off = b_off; a.b_sth = b_sth; a.b_stw = b_stw; a.b_sc = b_sc; a.b_sn = b_sn;
     a.d_OW = make_fastdiv(OW);
     a.d_OHW = make_fastdiv(OH * OW);
     a.d_PHt = make_fastdiv(PHt);

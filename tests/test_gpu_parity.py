@@ -156,6 +156,11 @@ TAP_SHAPES = [
     (4, 9, 14, 96, 72, 2, 4, 1, 3),       # non-square filter, asymmetric pad
     (4, 6, 5, 32, 64, 3, 3, 2, 2),        # pad larger than usual
     (3, 5, 5, 64, 64, 3, 3, 1, 1),        # fewer pixels than one unit
+    (5, 17, 19, 32, 48, 3, 3, 1, 1),      # halo-prefetching kernel: one pass, ragged OC, last unit partial
+    (2, 30, 62, 96, 80, 3, 3, 1, 1),      # ... widest row it takes (64 padded pixels), three passes, two oc slices
+    (3, 18, 18, 64, 64, 3, 3, 0, 0),      # ... no padding
+    (7, 40, 24, 64, 64, 3, 3, 2, 2),      # ... pad 2
+    (180, 20, 20, 32, 64, 3, 3, 1, 1),    # ... more units than workgroup slots: several units per workgroup, 2-tile pieces
 ]
 
 
@@ -168,11 +173,13 @@ def test_forward_lds_halo_kernel_vs_oracle_and_generic(dev, shape):
     try:
         L.alpha_conv_set_fwd_algo(0)
         fast = _run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, ph, pw)
+        fast_w = _run_fwd(dev, "conv3D", X, W, 1, 1, ph, pw)   # W[OC,FH,FW,IC] as it is (3x3: 128-bit filter fragment loads)
         L.alpha_conv_set_fwd_algo(3)
         generic = _run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, ph, pw)
     finally:
         L.alpha_conv_set_fwd_algo(0)
     check(fast, want, "lds-halo fwd %s" % (shape,))
+    check(fast_w, want, "lds-halo fwd from W %s" % (shape,))
     check(generic, want, "generic fwd %s" % (shape,))
 
 
