@@ -75,7 +75,7 @@ def _run_fwd(dev, entry, X, W, sh, sw, ph, pw):
     OC, FH, FW, _ = W.shape
     OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
     dXd, dWd = dev.put(X), dev.put(W)
-    Y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    Y = dev.guarded(N, OH, OW, OC)
     S, L = dev.streams, 1
     x, w, y = dXd.data_ptr(), dWd.data_ptr(), Y.data_ptr()
     if entry in ("conv3D", "conv3D_texture"):
@@ -191,7 +191,7 @@ def test_deltaX_lds_halo_kernel_vs_oracle(dev, shape):
     OH, OW = out_dim(IH, IW, FH, FW, 1, 1, ph, pw)
     dY, W = normal((N, OH, OW, OC), 1103), he_normal(OC, FH, FW, IC, 1104)
     dy, w = dev.put(dY), dev.put(W)
-    dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+    dXo = dev.guarded(N, IH, IW, IC)
     DX.dconv3D_deltaX_s1(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC, ph, pw)
     check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw), "lds-halo dX %s" % (shape,))
 
@@ -288,7 +288,7 @@ def test_deltaX_s1_entries(dev, shape):
     want = O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw)
     dy, w = dev.put(dY), dev.put(W)
     for entry in ("dconv3D_deltaX_s1", "dconv3D_deltaX_s1_texture", "dconv3D_deltaX_V2_s1"):
-        dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+        dXo = dev.guarded(N, IH, IW, IC)
         args = (dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC, ph, pw)
         if entry == "dconv3D_deltaX_V2_s1":
             DX.dconv3D_deltaX_V2_s1(True, *args)
@@ -300,7 +300,7 @@ def test_deltaX_s1_entries(dev, shape):
 def test_deltaX_W1(dev):
     for (N, IH, IW, IC, OC) in [(4, 14, 14, 256, 64), (4, 9, 7, 64, 256), (4, 5, 5, 12, 20)]:
         dY, W = normal((N, IH, IW, OC), 2003), he_normal(OC, 1, 1, IC, 2004)
-        dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+        dXo = dev.guarded(N, IH, IW, IC)
         dy, w = dev.put(dY), dev.put(W)  # keep the device buffers alive across the call
         DX.dconv3D_deltaX_W1(dev.streams, 1, dy.data_ptr(), w.data_ptr(), dXo.data_ptr(), IH, IW, N, IC, OC)
         check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, 0, 0), "deltaX_W1", sp_thr=1e-4)
@@ -328,7 +328,7 @@ def test_pointwise_kernel_forward_and_deltaX(dev, shape):
         for algo in (0, 3):   # 0: streaming GEMM kernel, 3: generic kernel
             L.alpha_conv_set_fwd_algo(algo)
             outs[algo] = (_run_fwd(dev, "conv3D_W1", X, W, 1, 1, 0, 0), _run_fwd(dev, "conv3D_GemmR_W1", X, W, 1, 1, 0, 0))
-            dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+            dXo = dev.guarded(N, IH, IW, IC)
             dy, w = dev.put(dY), dev.put(W)
             DX.dconv3D_deltaX_W1(dev.streams, 1, dy.data_ptr(), w.data_ptr(), dXo.data_ptr(), IH, IW, N, IC, OC)
             outs[algo] += (dev.get(dXo),)
@@ -459,7 +459,7 @@ def test_deltaX_kernel_split_family(dev, shape):
     if sh == 2 and sw == 2 and IH % 2 == 0 and IW % 2 == 0:
         entries += ["dconv3D_deltaX_ksIms2R", "dconv3D_deltaX_ksIms2R_texture", "dconv3D_deltaX_ksV2_Ims2R"]
     for entry in entries:
-        dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+        dXo = dev.guarded(N, IH, IW, IC)
         base = (dev.streams, 1, dy.data_ptr(), OH, OW, CW.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC)
         if entry == "dconv3D_deltaX_ksV2_Ims2R":
             DX.dconv3D_deltaX_ksV2_Ims2R(False, *base, ph, pw)
@@ -483,7 +483,7 @@ def test_deltaX_crossAdd_is_deterministic_gather(dev, shape):
     dy, w = dev.put(dY), dev.put(W)
     outs = []
     for _ in range(2):
-        dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+        dXo = dev.guarded(N, IH, IW, IC)
         DX.dconv3D_deltaX_crossAdd(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW,
                                    N, IC, OC, sh, sw, ph, pw)
         outs.append(dev.get(dXo))
@@ -517,13 +517,13 @@ def test_deltaW_entries(dev, shape):
     X, dY = normal((N, IH, IW, IC), 3001), normal((N, OH, OW, OC), 3002)
     want = O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw)
     x, dy = dev.put(X), dev.put(dY)
-    dWo = dev.empty(OC, FH, FW, IC, fill=float("nan"))
+    dWo = dev.guarded(OC, FH, FW, IC)
     DW.dconv3D_deltaW(dev.streams, 1, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
     check(dev.get(dWo), want, "dconv3D_deltaW %s" % (shape,), sp_min=1.0)
     sizeW = OC * FH * FW * IC
     for entry in ("dconv3D_deltaW_GemmSK", "dconv3D_deltaW_GemmV2SK"):
         for GridZ in (2, 5, 16):
-            dWo = dev.empty(OC, FH, FW, IC, fill=float("nan"))
+            dWo = dev.guarded(OC, FH, FW, IC)
             buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
             getattr(DW, entry)(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
                                FH, FW, N, IC, OC, sh, sw, ph, pw)
@@ -537,7 +537,7 @@ def test_deltaW_split_k_slices_follow_the_reference_partition(dev):
     X, dY = normal((N, IH, IW, IC), 3003), normal((N, OH, OW, OC), 3004)
     x, dy = dev.put(X), dev.put(dY)
     GridZ, sizeW = 5, OC * F_ * F_ * IC
-    dWo = dev.empty(OC, F_, F_, IC, fill=float("nan"))
+    dWo = dev.guarded(OC, F_, F_, IC)
     buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
     DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
                              F_, F_, N, IC, OC, s, s, p, p)
@@ -584,7 +584,7 @@ def test_deltaW_row_streaming_kernel_slices_and_sum(dev, shape):
     try:
         for algo in (0, 3):   # 0: row-streaming kernel where eligible, 3: generic kernel
             L.alpha_conv_set_fwd_algo(algo)
-            dWo = dev.empty(OC, F_, F_, IC, fill=float("nan"))
+            dWo = dev.guarded(OC, F_, F_, IC)
             buf = dev.empty(max(GridZ - 1, 1), sizeW, fill=float("nan"))
             if F_ == 1:
                 DW.dconv3D_deltaW_GemmSK_W1(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), buf.data_ptr(),
@@ -615,11 +615,11 @@ def test_deltaW_W1_entries(dev):
         X, dY = normal((N, IH, IW, IC), 3005), normal((N, IH, IW, OC), 3006)
         want = O.deltaW_f64(X, dY, 1, 1, 1, 1, 0, 0)
         x, dy = dev.put(X), dev.put(dY)
-        dWo = dev.empty(OC, 1, 1, IC, fill=float("nan"))
+        dWo = dev.guarded(OC, 1, 1, IC)
         DW.dconv3D_deltaW_W1(dev.streams, 1, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), N, IC, OC)
         check(dev.get(dWo), want, "deltaW_W1", sp_min=1.0)
         GridZ = 3
-        dWo = dev.empty(OC, 1, 1, IC, fill=float("nan"))
+        dWo = dev.guarded(OC, 1, 1, IC)
         buf = dev.empty(GridZ - 1, OC * IC, fill=float("nan"))
         DW.dconv3D_deltaW_GemmSK_W1(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), buf.data_ptr(), N, IC, OC)
         check(_sum_partials(dev, dWo, buf, GridZ), want, "deltaW_GemmSK_W1", sp_min=1.0)
@@ -643,7 +643,7 @@ def test_deltaW_bit_reproducible_run_to_run(dev):
     GridZ, sizeW = 16, OC * 9 * IC
     outs = []
     for _ in range(3):
-        dWo = dev.empty(OC, 3, 3, IC, fill=float("nan"))
+        dWo = dev.guarded(OC, 3, 3, IC)
         buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
         DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), IH, IW, dWo.data_ptr(), buf.data_ptr(),
                                  3, 3, N, IC, OC, 1, 1, 1, 1)
@@ -669,7 +669,7 @@ def test_reference_style_criterion_deltaX(dev):
     N, IH, IW, IC, OC, F_, p = 4, 31, 31, 128, 32, 4, 1
     OH, OW = out_dim(IH, IW, F_, F_, 1, 1, p, p)
     dY, W = uniform((N, OH, OW, OC), 4003, 0, 1), uniform((OC, F_, F_, IC), 4004, 0, 1)
-    dXo = dev.empty(N, IH, IW, IC, fill=float("nan"))
+    dXo = dev.guarded(N, IH, IW, IC)
     dy, w = dev.put(dY), dev.put(W)
     DX.dconv3D_deltaX_s1(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), F_, F_, dXo.data_ptr(), IH, IW,
                          N, IC, OC, p, p)
@@ -684,7 +684,7 @@ def test_reference_style_criterion_deltaW(dev):
     cpu = O.deltaW_naive(X, dY, F_, F_, s, s, p, p)
     x, dy = dev.put(X), dev.put(dY)
     GridZ, sizeW = 4, OC * F_ * F_ * IC
-    dWo = dev.empty(OC, F_, F_, IC, fill=float("nan"))
+    dWo = dev.guarded(OC, F_, F_, IC)
     buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
     DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
                              F_, F_, N, IC, OC, s, s, p, p)

@@ -38,6 +38,10 @@ def he_normal(OC, FH, FW, IC, seed):
     return normal((OC, FH, FW, IC), seed, std=float(np.sqrt(2.0 / (FH * FW * IC))))
 
 
+GUARD = 16384          # floats on either side of a guarded output (a multiple of 4: the tensor stays 16-byte aligned)
+SENTINEL = 1.5e30
+
+
 class Dev:
     """Device-side helpers built on torch (allocation, copies, the current stream handle)."""
 
@@ -58,8 +62,28 @@ class Dev:
             t.fill_(fill)
         return t
 
+    def guarded(self, *shape):
+        """An output tensor filled with NaN that sits between two guard bands of a sentinel value; `check_guards`
+        tells whether a kernel wrote outside the tensor."""
+        n = int(np.prod(shape))
+        flat = self.torch.full((2 * GUARD + n,), SENTINEL, dtype=self.torch.float32, device=self.dev)
+        inner = flat[GUARD:GUARD + n].view(*shape)
+        inner.fill_(float("nan"))
+        inner._guard_owner = flat
+        return inner
+
+    def check_guards(self, t):
+        flat = t._guard_owner
+        self.torch.cuda.synchronize()
+        n = flat.numel() - 2 * GUARD
+        lo, hi = flat[:GUARD].cpu().numpy(), flat[GUARD + n:].cpu().numpy()
+        assert np.all(lo == np.float32(SENTINEL)), "write before the output tensor"
+        assert np.all(hi == np.float32(SENTINEL)), "write past the output tensor"
+
     def get(self, t):
         self.torch.cuda.synchronize()
+        if hasattr(t, "_guard_owner"):
+            self.check_guards(t)
         return t.cpu().numpy()
 
     def sync(self):
