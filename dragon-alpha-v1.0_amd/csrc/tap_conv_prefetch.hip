@@ -17,7 +17,7 @@
 // from the accumulators straight to memory.
 //
 // Restrictions (the launcher answers hipErrorNotSupported and the caller uses tap_conv.hip): 3x3 taps, stride 1, AC a
-// multiple of 32, padded rows of 17..64 pixels, both buffers within 80 KB.
+// multiple of 32, padded rows of at most 64 pixels, at most 32 halo rows per unit, both buffers within 80 KB.
 #include "common.hpp"
 
 namespace alpha {
@@ -73,8 +73,8 @@ static __device__ __forceinline__ PfHalo pf_halo(const TapPfArgs &p, int m0, int
 
 // TILES: tiles of a whole unit; CG: column groups of 32 padded pixels per row (1 or 2); EPT: halo elements a thread
 // requests per tap; BK: the filter is contiguous along the input channel (W[OC,FH,FW,IC] as it is) instead of along the
-// output channel.
-template <int TILES, int CG, int EPT, bool BK>
+// output channel; RP2: rows of at most 16 padded pixels, a halo element is this thread's share of TWO rows (CG = 1).
+template <int TILES, int CG, int EPT, bool BK, bool RP2>
 __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -124,40 +124,69 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
 
     // ---- halo mover ------------------------------------------------------------------------------------------------
     // Thread t moves channels [4*(t&7), +4) of padded column 32*cg + (t>>3) of a row; element e of a pass is (row
-    // e / CG, column group e % CG). Columns past the end of the row repeat the last column (the same bytes to the same
-    // place), rows past the halo's last row repeat the last row. The row is uniform: its terms live in scalar
-    // registers, the load takes (descriptor, per-thread offset, scalar offset); padding columns and rows make the
-    // per-thread offset out of range and zeros arrive without a select.
+    // e / CG, column group e % CG). Rows of at most 16 pixels (RP2): column (t>>3)&15 of row 2e + (t>>7). Columns past
+    // the end of the row repeat the last column (the same bytes to the same place), rows past the halo's last row
+    // repeat the last row. What depends on the row - where it starts in A, whether it lies inside the image, where it
+    // goes in LDS - is the same for every pass of a unit: lane i of a wavefront computes it for row i once per unit
+    // (two registers), and a tap fetches the rows it requests with v_readlane into scalar registers. The load takes
+    // (descriptor, per-thread offset, scalar offset); padding columns and rows make the per-thread offset out of range
+    // and zeros arrive without a select.
+    constexpr unsigned NEVER = 0x40000000u;   // RP2 adds a column and a row offset: two of these still do not wrap (A < 1 GB, host-checked)
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
     unsigned voff[CG];
     int loff[CG];
 #pragma unroll
     for (int cg = 0; cg < CG; cg++) {
-        const int cp = min(32 * cg + (t >> 3), PWt - 1), iw = cp - p.pw;
-        voff[cg] = (unsigned)iw < (unsigned)p.AW ? (unsigned)((iw * p.AC + (t & 7) * 4) * 4) : PF_OUT_OF_RANGE;
+        const int cp = min(RP2 ? (t >> 3) & 15 : 32 * cg + (t >> 3), PWt - 1), iw = cp - p.pw;
+        voff[cg] = (unsigned)iw < (unsigned)p.AW ? (unsigned)((iw * p.AC + (t & 7) * 4) * 4) : (RP2 ? NEVER : PF_OUT_OF_RANGE);
         loff[cg] = cp * PF_PS + (t & 7) * 4;
     }
-    // A halo row being requested: scalar offset of its first pixel in A (channels of the pass included), whether it
-    // lies inside the image, and where it goes in LDS.
-    struct RowState {
-        int soff, rowoff;
-        unsigned kill;
+    const bool second_row = RP2 && t >= 128;
+    // per-lane table of a halo's rows: byte offset of the row in A (-1: padding row) and float offset of the row in a buffer
+    struct RowTable {
+        int g, l;
     };
-    // row r (clamped to the halo's last row) of halo h, channels [ic0, ic0 + 32), for the buffer at float offset tb
-    auto next_row = [&](RowState &row, auto r_c, const PfHalo &h, int ic0, int tb, bool on) {
-        const int r = min((int)decltype(r_c)::value, h.rows - 1);
+    auto row_table = [&](const PfHalo &h, bool on) {
+        const int r = min(lane, h.rows - 1);
         const int pgr = h.pgr0 + r;
         const int n = fdiv(pgr, p.d_PHt), ih = pgr - n * PHt - p.ph;
-        const bool rok = (unsigned)ih < (unsigned)p.AH && on;
-        row.soff = __builtin_amdgcn_readfirstlane(rok ? ((n * p.AH + ih) * p.AW * p.AC + ic0) * 4 : 0);
-        row.kill = __builtin_amdgcn_readfirstlane(rok ? 0u : PF_OUT_OF_RANGE);
-        row.rowoff = __builtin_amdgcn_readfirstlane(tb + r * row_floats);
+        RowTable tb_;
+        tb_.g = ((unsigned)ih < (unsigned)p.AH && on) ? (n * p.AH + ih) * p.AW * p.AC * 4 : -1;
+        tb_.l = r * row_floats;
+        return tb_;
+    };
+    // The row(s) being requested: scalar offset in A (channels of the pass included), padding or not, place in LDS.
+    struct RowState {
+        int soff, rowoff;     // first (or only) row
+        unsigned kill;
+        int soff2, rowoff2;   // RP2: second row; soff/soff2 are then NEVER for a padding row
+    };
+    // row index (RP2: rows 2*index, 2*index+1) of the table, channels [ic0, ic0 + 32), for the buffer at float offset tb
+    auto next_row = [&](RowState &row, int index, const RowTable &tab, int ic0, int tb) {
+        if (!RP2) {
+            const int g = __builtin_amdgcn_readlane(tab.g, index);
+            row.soff = g >= 0 ? g + ic0 * 4 : 0;
+            row.kill = g >= 0 ? 0u : PF_OUT_OF_RANGE;
+            row.rowoff = tb + __builtin_amdgcn_readlane(tab.l, index);
+        } else {
+            const int g = __builtin_amdgcn_readlane(tab.g, 2 * index), g2 = __builtin_amdgcn_readlane(tab.g, 2 * index + 1);
+            row.soff = g >= 0 ? g + ic0 * 4 : (int)NEVER;
+            row.soff2 = g2 >= 0 ? g2 + ic0 * 4 : (int)NEVER;
+            row.rowoff = tb + __builtin_amdgcn_readlane(tab.l, 2 * index);
+            row.rowoff2 = tb + __builtin_amdgcn_readlane(tab.l, 2 * index + 1);
+        }
     };
     // request this thread's element of column group cg of that row; `on` false: zeros to the spare slot
     auto request = [&](auto cg_c, const RowState &row, bool on, float4 &v, int &dst) {
         constexpr int cg = decltype(cg_c)::value;
-        v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(voff[cg] | row.kill), row.soff, 0));
-        dst = on ? row.rowoff + loff[cg] : spare;
+        if (!RP2) {
+            v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(voff[cg] | row.kill), row.soff, 0));
+            dst = on ? row.rowoff + loff[cg] : spare;
+        } else {
+            const int so = second_row ? row.soff2 : row.soff;
+            v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(voff[0] + (unsigned)so), 0, 0));
+            dst = on ? (second_row ? row.rowoff2 : row.rowoff) + loff[0] : spare;
+        }
     };
 
     // ---- filter fragments straight from global memory (see tap_conv.hip) ----------------------------------------
@@ -206,21 +235,17 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
     int m0 = 0, m_hi = 0, body = 0;
     int idx = next_item(0, m0, m_hi, body);
     if (idx >= n_items) return;
+    RowTable tab_cur = row_table(pf_halo(p, m0, m_hi), true);
     {
         const PfHalo h = pf_halo(p, m0, m_hi);
-        for (int r0 = 0; r0 < h.rows; r0 += 8 / CG) {
+        constexpr int ROWS8 = RP2 ? 16 : 8 / CG;   // rows that eight elements cover
+        for (int r0 = 0; r0 < h.rows; r0 += ROWS8) {
             float4 v[8];
             int dst[8];
             pf_static_for<0, 8>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
                 RowState row;
-                const int r = min(r0 + i / CG, h.rows - 1);
-                const int pgr = h.pgr0 + r;
-                const int n = fdiv(pgr, p.d_PHt), ih = pgr - n * PHt - p.ph;
-                const bool rok = (unsigned)ih < (unsigned)p.AH;
-                row.soff = __builtin_amdgcn_readfirstlane(rok ? ((n * p.AH + ih) * p.AW * p.AC) * 4 : 0);
-                row.kill = __builtin_amdgcn_readfirstlane(rok ? 0u : PF_OUT_OF_RANGE);
-                row.rowoff = __builtin_amdgcn_readfirstlane(r * row_floats);
+                next_row(row, min((RP2 ? r0 / 2 : r0) + i / CG, 31), tab_cur, 0, 0);
                 request(PfInt<i % CG>{}, row, true, v[i], dst[i]);
             });
 #pragma unroll
@@ -230,7 +255,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
     }
 
     // ---- one unit ------------------------------------------------------------------------------------------------------
-    auto run_unit = [&](auto tiles_c, const int m0, const int m_hi, const bool has_next, const PfHalo nh) {
+    auto run_unit = [&](auto tiles_c, const int m0, const int m_hi, const bool has_next, const RowTable &tab_next) {
         constexpr int T = decltype(tiles_c)::value;
         const PfHalo h = pf_halo(p, m0, m_hi);
 
@@ -278,7 +303,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
             const int ic0 = pass * PF_ICC;
             const bool last_pass = pass + 1 == npass;
             // what to prefetch: the next 32 channels of this halo, or the first 32 of the next unit's
-            const PfHalo th_ = last_pass ? nh : h;
+            const RowTable &tab = last_pass ? tab_next : tab_cur;
             const int t_ic0 = last_pass ? 0 : ic0 + PF_ICC;
             const bool t_on = !last_pass || has_next;
             const int tb = (buf ^ 1) * p.buf_floats;
@@ -303,7 +328,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
                 if (!TAIL) {
                     pf_static_for<0, EPT>([&](auto ic) {
                         constexpr int i = decltype(ic)::value, e = K * EPT + i;
-                        if (e % CG == 0) next_row(row, PfInt<e / CG>{}, th_, t_ic0, tb, t_on);
+                        if (e % CG == 0) next_row(row, e / CG, tab, t_ic0, tb);
                         request(PfInt<e % CG>{}, row, t_on, pv[PAR][i], pd[PAR][i]);
                     });
                 }
@@ -365,10 +390,12 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
         const bool has_next = nidx < n_items;
         PfHalo nh{0, 1};
         if (has_next) nh = pf_halo(p, n_m0, n_hi);
-        if (body == 0) run_unit(PfInt<TILES>{}, m0, m_hi, has_next, nh);
-        else if (body == 1) run_unit(PfInt<4>{}, m0, m_hi, has_next, nh);
-        else run_unit(PfInt<2>{}, m0, m_hi, has_next, nh);
+        const RowTable tab_next = row_table(nh, has_next);
+        if (body == 0) run_unit(PfInt<TILES>{}, m0, m_hi, has_next, tab_next);
+        else if (body == 1) run_unit(PfInt<4>{}, m0, m_hi, has_next, tab_next);
+        else run_unit(PfInt<2>{}, m0, m_hi, has_next, tab_next);
         idx = nidx; m0 = n_m0; m_hi = n_hi; body = n_body;
+        tab_cur = tab_next;
     }
 }
 
@@ -396,10 +423,10 @@ static int tap_pf_lds_rows(int M, int P, int OH, int OW, int TH, int PHt)
     return worst;
 }
 
-template <int TILES, int CG, int EPT, bool BK>
+template <int TILES, int CG, int EPT, bool BK, bool RP2>
 static hipError_t launch_pf2(hipStream_t stream, TapPfArgs a, size_t lds, int cus)
 {
-    auto kern = tap_conv_prefetch_kernel<TILES, CG, EPT, BK>;
+    auto kern = tap_conv_prefetch_kernel<TILES, CG, EPT, BK, RP2>;
     static size_t configured = 0;
     if (lds > configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -429,10 +456,10 @@ static hipError_t launch_pf2(hipStream_t stream, TapPfArgs a, size_t lds, int cu
     return hipGetLastError();
 }
 
-template <int TILES, int CG, int EPT>
+template <int TILES, int CG, int EPT, bool RP2 = false>
 static hipError_t launch_pf(hipStream_t stream, const TapPfArgs &a, size_t lds, int cus)
 {
-    return a.b_sn != 1 ? launch_pf2<TILES, CG, EPT, true>(stream, a, lds, cus) : launch_pf2<TILES, CG, EPT, false>(stream, a, lds, cus);
+    return a.b_sn != 1 ? launch_pf2<TILES, CG, EPT, true, RP2>(stream, a, lds, cus) : launch_pf2<TILES, CG, EPT, false, RP2>(stream, a, lds, cus);
 }
 
 // Returns hipErrorNotSupported when the shape does not fit this kernel; otherwise launches.
@@ -445,11 +472,13 @@ hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const fl
     if (OH != AH + 2 * ph - TH + 1 || OW != AW + 2 * pw - TW + 1) return hipErrorNotSupported;
     if (AC % PF_ICC != 0 || TH != 3 || TW != 3) return hipErrorNotSupported;
     const int PHt = AH + 2 * ph, PWt = AW + 2 * pw;
-    if (PWt <= 16 || PWt > 64) return hipErrorNotSupported;
+    if (PWt < 3 || PWt > 64) return hipErrorNotSupported;
+    const bool rp2 = PWt <= 16;
     const long M = (long)N * OH * OW;
     if ((long)N * PHt >= (1L << 24) || M >= (1L << 30)) return hipErrorNotSupported;
     const long a_bytes = (long)N * AH * AW * AC * 4;
     if (a_bytes >= (1L << 31) || M * CO * 4 >= (1L << 31)) return hipErrorNotSupported;
+    if (PWt <= 16 && a_bytes >= (1L << 30)) return hipErrorNotSupported;
 
     TapPfArgs a{};
     a.A = A; a.B = B; a.O = O; a.bias = bias;
@@ -474,7 +503,11 @@ hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const fl
         const size_t bufsz = (size_t)a.lds_rows * PWt * PF_PS;
         a.buf_floats = (int)bufsz;
         const size_t lds = (2 * bufsz + 4) * sizeof(float);
-        const int elems = a.lds_rows * cg, ept = (elems + TH * TW - 2) / (TH * TW - 1);
+        const int elems = rp2 ? (a.lds_rows + 1) / 2 : a.lds_rows * cg, ept = (elems + TH * TW - 2) / (TH * TW - 1);
+        if (lds <= 80 * 1024 && ept <= 2 && rp2) {
+            if (tiles == 7) return ept == 1 ? launch_pf<7, 1, 1, true>(stream, a, lds, cus) : launch_pf<7, 1, 2, true>(stream, a, lds, cus);
+            return ept == 1 ? launch_pf<8, 1, 1, true>(stream, a, lds, cus) : launch_pf<8, 1, 2, true>(stream, a, lds, cus);
+        }
         if (lds <= 80 * 1024 && ept <= 2) {
             if (tiles == 7) {
                 if (cg == 1) return ept == 1 ? launch_pf<7, 1, 1>(stream, a, lds, cus) : launch_pf<7, 1, 2>(stream, a, lds, cus);
