@@ -139,10 +139,10 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
     for (int cg = 0; cg < CG; cg++) {
         const int cp = min(RP2 ? (t >> 3) & 15 : 32 * cg + (t >> 3), PWt - 1), iw = cp - p.pw;
         voff[cg] = (unsigned)iw < (unsigned)p.AW ? (unsigned)((iw * p.AC + (t & 7) * 4) * 4) : (RP2 ? NEVER : PF_OUT_OF_RANGE);
-        loff[cg] = cp * PF_PS + (t & 7) * 4;
+        loff[cg] = (cp * PF_PS + (t & 7) * 4) * 4;   // bytes
     }
     const bool second_row = RP2 && t >= 128;
-    // per-lane table of a halo's rows: byte offset of the row in A (-1: padding row) and float offset of the row in a buffer
+    // per-lane table of a halo's rows: byte offset of the row in A (-1: padding row) and byte offset of the row in a buffer
     struct RowTable {
         int g, l;
     };
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
         const int n = fdiv(pgr, p.d_PHt), ih = pgr - n * PHt - p.ph;
         RowTable tb_;
         tb_.g = ((unsigned)ih < (unsigned)p.AH && on) ? (n * p.AH + ih) * p.AW * p.AC * 4 : -1;
-        tb_.l = r * row_floats;
+        tb_.l = r * row_floats * 4;
         return tb_;
     };
     // The row(s) being requested: scalar offset in A (channels of the pass included), padding or not, place in LDS.
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
         unsigned kill;
         int soff2, rowoff2;   // RP2: second row; soff/soff2 are then NEVER for a padding row
     };
-    // row index (RP2: rows 2*index, 2*index+1) of the table, channels [ic0, ic0 + 32), for the buffer at float offset tb
+    // row index (RP2: rows 2*index, 2*index+1) of the table, channels [ic0, ic0 + 32), for the buffer at byte offset tb
     auto next_row = [&](RowState &row, int index, const RowTable &tab, int ic0, int tb) {
         if (!RP2) {
             const int g = __builtin_amdgcn_readlane(tab.g, index);
@@ -176,16 +176,17 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
             row.rowoff2 = tb + __builtin_amdgcn_readlane(tab.l, 2 * index + 1);
         }
     };
-    // request this thread's element of column group cg of that row; `on` false: zeros to the spare slot
-    auto request = [&](auto cg_c, const RowState &row, bool on, float4 &v, int &dst) {
+    // request this thread's element of column group cg of that row; dst: its place in LDS (bytes). With nothing to
+    // prefetch (the table says padding everywhere) zeros go to the buffer nobody will read.
+    auto request = [&](auto cg_c, const RowState &row, float4 &v, int &dst) {
         constexpr int cg = decltype(cg_c)::value;
         if (!RP2) {
             v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(voff[cg] | row.kill), row.soff, 0));
-            dst = on ? row.rowoff + loff[cg] : spare;
+            dst = row.rowoff + loff[cg];
         } else {
             const int so = second_row ? row.soff2 : row.soff;
             v = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(voff[0] + (unsigned)so), 0, 0));
-            dst = on ? (second_row ? row.rowoff2 : row.rowoff) + loff[0] : spare;
+            dst = (second_row ? row.rowoff2 : row.rowoff) + loff[0];
         }
     };
 
@@ -246,10 +247,10 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
                 constexpr int i = decltype(ic)::value;
                 RowState row;
                 next_row(row, min((RP2 ? r0 / 2 : r0) + i / CG, 31), tab_cur, 0, 0);
-                request(PfInt<i % CG>{}, row, true, v[i], dst[i]);
+                request(PfInt<i % CG>{}, row, v[i], dst[i]);
             });
 #pragma unroll
-            for (int i = 0; i < 8; i++) *reinterpret_cast<float4 *>(Hs + dst[i]) = v[i];
+            for (int i = 0; i < 8; i++) *reinterpret_cast<float4 *>(reinterpret_cast<char *>(Hs) + dst[i]) = v[i];
         }
         __syncthreads();
     }
@@ -305,11 +306,10 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
             // what to prefetch: the next 32 channels of this halo, or the first 32 of the next unit's
             const RowTable &tab = last_pass ? tab_next : tab_cur;
             const int t_ic0 = last_pass ? 0 : ic0 + PF_ICC;
-            const bool t_on = !last_pass || has_next;
-            const int tb = (buf ^ 1) * p.buf_floats;
+            const int tb = (buf ^ 1) * p.buf_floats * 4;   // bytes
             const int n_ic = last_pass ? 0 : ic0 + PF_ICC;   // filter fragment after this pass's last tap
 #pragma unroll
-            for (int i = 0; i < EPT; i++) pd[1][i] = spare;   // tap 0 commits "the tap before": nothing
+            for (int i = 0; i < EPT; i++) pd[1][i] = spare * 4;   // tap 0 commits "the tap before": nothing
             RowState row;
 
             __builtin_amdgcn_s_setprio(0);
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
                     pf_static_for<0, EPT>([&](auto ic) {
                         constexpr int i = decltype(ic)::value, e = K * EPT + i;
                         if (e % CG == 0) next_row(row, e / CG, tab, t_ic0, tb);
-                        request(PfInt<e % CG>{}, row, t_on, pv[PAR][i], pd[PAR][i]);
+                        request(PfInt<e % CG>{}, row, pv[PAR][i], pd[PAR][i]);
                     });
                 }
                 load_b(bL, TAIL ? n_ic : ic0, NK / 3, NK % 3);
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < EPT; i++)   // the elements requested one tap ago
-                    *reinterpret_cast<float4 *>(Hs + pd[PAR ^ 1][i]) = pv[PAR ^ 1][i];
+                    *reinterpret_cast<float4 *>(reinterpret_cast<char *>(Hs) + pd[PAR ^ 1][i]) = pv[PAR ^ 1][i];
                 if (!TAIL) {
                     if (TW_ == 2) {   // on to the next filter row
 #pragma unroll
