@@ -32,6 +32,24 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
     return (__umulhi(n, f.mul) + n) >> f.shift;
 }
 
+// The dynamic LDS limit is a property of (kernel, device): raise it the first time a device needs more than it has.
+// One instantiation, and so one table, per kernel. A racing first call sets the same value twice.
+template <auto KERNEL>
+inline hipError_t ensure_dynamic_lds(size_t bytes)
+{
+    static size_t configured[64] = {0};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    if (bytes > configured[dev]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) return e;
+        configured[dev] = bytes;
+    }
+    return hipSuccess;
+}
+
 // One launch of the generic implicit-GEMM "gather convolution":
 //   O[o_off + n*o_sn + i*o_sh + j*o_sw + co] =
 //       sum_{th<TH, tw<TW, c<AC}  A[n, i*sh - ph + th, j*sw - pw + tw, c] * B[b_off + th*b_sth + tw*b_stw + c*b_sc + co*b_sn]

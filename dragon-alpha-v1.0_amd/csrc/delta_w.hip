@@ -144,14 +144,8 @@ static hipError_t launch_dw_cfg(hipStream_t stream, const DeltaWArgs &a)
 {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     constexpr size_t lds = (size_t)2 * 32 * ((BM + 8) + (BN + 8)) * sizeof(float);
-    auto kern = delta_w_kernel<WM, WN, TM, TN>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    constexpr auto kern = delta_w_kernel<WM, WN, TM, TN>;
+    if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     dim3 grid((a.GM + BN - 1) / BN, (a.OC + BM - 1) / BM, a.GZ);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
     return hipGetLastError();

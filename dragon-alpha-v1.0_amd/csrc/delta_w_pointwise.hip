@@ -184,13 +184,7 @@ hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const flo
     for (int tpw = 8; tpw > 1; tpw >>= 1)
         if (tpw <= a.tiles && (long)((a.tiles + tpw - 1) / tpw) * GZ >= cu_count[dev]) { a.TPW = tpw; break; }
     const size_t lds = (size_t)(8 / a.TPW - 1) * a.TPW * (16 * 64 + 16) * sizeof(floatx4) + 16;   // accumulators + bias sums of the parts
-    static size_t configured = 0;
-    if (lds > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(delta_w_pointwise_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = lds;
-    }
+    if (hipError_t e = ensure_dynamic_lds<delta_w_pointwise_kernel>(lds); e != hipSuccess) return e;
     dim3 grid((a.tiles + a.TPW - 1) / a.TPW, GZ);
     hipLaunchKernelGGL(delta_w_pointwise_kernel, grid, dim3(512), lds, stream, a);
     return hipGetLastError();

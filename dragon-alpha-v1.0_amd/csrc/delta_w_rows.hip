@@ -404,13 +404,8 @@ __global__ __launch_bounds__(256, OCT <= 2 ? 2 : 1) void delta_w_rows_kernel(con
 template <int FH, int FW, int OCT, bool ONE_ROW>
 static hipError_t launch_dwr_rows(hipStream_t stream, const DwRowsArgs &a, size_t lds)
 {
-    auto kern = delta_w_rows_kernel<FH, FW, OCT, ONE_ROW>;
-    static size_t configured = 0;
-    if (lds > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = lds;
-    }
+    constexpr auto kern = delta_w_rows_kernel<FH, FW, OCT, ONE_ROW>;
+    if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     constexpr int OCB = 16 * OCT;
     dim3 grid((a.IC + 63) / 64, (a.OC + OCB - 1) / OCB, a.GZ);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);

@@ -229,14 +229,8 @@ static hipError_t launch_cfg(hipStream_t stream, const GatherConvArgs &a)
     constexpr size_t lds_loop = (size_t)(2 * A_TILE + 2 * B_TILE) * sizeof(float);
     constexpr size_t lds_out = (size_t)(BM * (BN + 4) + BM) * sizeof(float);   // output staging + row offsets
     constexpr size_t lds = lds_loop > lds_out ? lds_loop : lds_out;
-    auto kern = gather_conv_kernel<WM, WN, TM, TN, B_NMAJOR>;
-    static bool configured = false;  // idempotent attribute; a benign race sets it twice at worst
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    constexpr auto kern = gather_conv_kernel<WM, WN, TM, TN, B_NMAJOR>;
+    if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     dim3 grid((a.M + BM - 1) / BM, (a.CO + BN - 1) / BN, 1);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
     return hipGetLastError();

@@ -239,13 +239,8 @@ static hipError_t launch_pw(hipStream_t stream, const PointwiseArgs &a, int cus)
 {
     constexpr size_t lds = ((size_t)16 * NT * (64 * KB + 8) + 8 * 16 * PW_OS + 4) * sizeof(float);
     static_assert(lds <= 160 * 1024, "filter + staging must fit in LDS");
-    auto kern = pointwise_kernel<NT, KB>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    constexpr auto kern = pointwise_kernel<NT, KB>;
+    if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     const int nblocks = a.ldn / (16 * NT);
     int grid = cus / nblocks;                            // one workgroup per compute unit, shared among the N blocks
     if (grid < 1) grid = 1;

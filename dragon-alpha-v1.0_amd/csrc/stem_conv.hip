@@ -236,13 +236,7 @@ hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, 
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return hipErrorNotSupported;
         cu_count[dev] = n;
     }
-    static size_t configured = 0;
-    if (lds > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(stem_conv_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = lds;
-    }
+    if (hipError_t e = ensure_dynamic_lds<stem_conv_kernel>(lds); e != hipSuccess) return e;
     const int ocb = (OC + 63) / 64;
     int gx = 2 * cu_count[dev] / ocb;
     if (gx < 1) gx = 1;

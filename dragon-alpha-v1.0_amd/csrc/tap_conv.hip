@@ -367,14 +367,8 @@ static int tap_conv_lds_rows(int M, int P, int OH, int OW, int TH, int sh, int P
 template <int TILES, bool RAGGED>
 static hipError_t launch_tc(hipStream_t stream, TapConvArgs a, size_t lds, int cus)
 {
-    auto kern = tap_conv_kernel<TILES, RAGGED>;
-    static size_t configured = 0;
-    if (lds > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = lds;
-    }
+    constexpr auto kern = tap_conv_kernel<TILES, RAGGED>;
+    if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     const int units = (a.M + TILES * 16 - 1) / (TILES * 16), ocb = (a.CO + 63) / 64;
     const int slots = cus * (2 * lds <= 160 * 1024 ? 2 : 1);   // workgroups the device holds at once
     int G = slots / ocb;

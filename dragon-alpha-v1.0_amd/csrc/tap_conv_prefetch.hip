@@ -426,14 +426,8 @@ static int tap_pf_lds_rows(int M, int P, int OH, int OW, int TH, int PHt)
 template <int TILES, int CG, int EPT, bool BK, bool RP2>
 static hipError_t launch_pf2(hipStream_t stream, TapPfArgs a, size_t lds, int cus)
 {
-    auto kern = tap_conv_prefetch_kernel<TILES, CG, EPT, BK, RP2>;
-    static size_t configured = 0;
-    if (lds > configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = lds;
-    }
+    constexpr auto kern = tap_conv_prefetch_kernel<TILES, CG, EPT, BK, RP2>;
+    if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     const int units = (a.M + TILES * 16 - 1) / (TILES * 16), ocb = (a.CO + 63) / 64;
     int G = 2 * cus / ocb;   // two workgroups per compute unit
     if (G < 1) G = 1;

@@ -270,13 +270,7 @@ hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, f
     size_t lds = (size_t)2 * WG_VBUF * sizeof(float);
     const size_t stage = (size_t)WG_TILES * 4 * 68 * sizeof(float);
     if (lds < stage) lds = stage;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(winograd_f2x2_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    if (hipError_t e = ensure_dynamic_lds<winograd_f2x2_kernel>(lds); e != hipSuccess) return e;
     dim3 grid((a.ntiles + WG_TILES - 1) / WG_TILES, (OC + 63) / 64);
     hipLaunchKernelGGL(winograd_f2x2_kernel, grid, dim3(256), lds, stream, a);
     return hipGetLastError();
