@@ -50,15 +50,16 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
     // ---- tiles: the workgroup owns the contiguous range [t_begin, t_end); its wavefronts take the first eight
     // statically and then draw from a counter in LDS, so they finish within one tile of each other whatever the
     // range length (a static split of 24.5 tiles over 8 wavefronts would leave a quarter of the machine idle).
-    // With more than one group of 64 produced channels per tile, the tiles beyond the last multiple of eight are
-    // split further, into (tile, group) units dealt to the wavefronts in order (wavefronts w and w + 4 share a SIMD):
-    // a 25th tile costs every SIMD a quarter of a tile instead of costing one SIMD a whole one.
+    // The tiles beyond the last multiple of eight are split further, into (tile, group of 64 produced channels) units
+    // or, with a single group, (tile, 16 channels) units, dealt to the wavefronts in order (wavefronts w and w + 4
+    // share a SIMD): a 25th tile costs every SIMD a quarter of a tile instead of costing one SIMD a whole one.
     const int G = gridDim.x;
     const int t_begin = (int)((long)p.tiles * blockIdx.x / G), t_end = (int)((long)p.tiles * (blockIdx.x + 1) / G);
     constexpr int NG = NT / 4;
-    const int t_main = NG > 1 ? t_begin + ((t_end - t_begin) & ~7) : t_end;
-    const int units = (t_end - t_main) * NG;          // 0 when NG == 1
-    const int unit_tile = t_main + w / NG;            // tile of this wavefront's first unit, if it has one (w < units)
+    constexpr int UPT = NG > 1 ? NG : 4;              // units per tile
+    const int t_main = t_begin + ((t_end - t_begin) & ~7);
+    const int units = (t_end - t_main) * UPT;
+    const int unit_tile = t_main + w / UPT;           // tile of this wavefront's first unit, if it has one (w < units)
     int *queue = reinterpret_cast<int *>(smem + N * KS + 8 * 16 * PW_OS);
     if (t == 0) *queue = t_begin + 8;
 
@@ -230,6 +231,30 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
         for (int u = w; u < units; u += 8) {
             if (u != w) load_a(aP, t_main + u / NG);   // only the first unit's fragments were requested ahead
             process(IntC<1>{}, t_main + u / NG, u % NG, aP);
+        }
+    } else {
+        // 16 produced channels of one tile: one accumulator tile, stored straight from the MFMA layout (lane (l16, q)
+        // holds pixels 4q + r of channel l16: 64 contiguous bytes of four pixel rows per store)
+        for (int u = w; u < units; u += 8) {
+            const int utile = t_main + u / 4, jj = u % 4;
+            if (u != w) load_a(aP, utile);
+            const float *blj = bl + jj * 16 * KS;
+            const float bias_l = p.bias ? p.bias[n_off + 16 * jj + l16] : 0.f;
+            floatx4 acc = zero, b[3];
+            b[0] = *reinterpret_cast<const floatx4 *>(blj);
+            b[1] = *reinterpret_cast<const floatx4 *>(blj + 16);
+#pragma unroll
+            for (int kc = 0; kc < KB * 4; kc++) {
+                if (kc + 2 < KB * 4) b[(kc + 2) % 3] = *reinterpret_cast<const floatx4 *>(blj + (kc + 2) * 16);
+#pragma unroll
+                for (int s = 0; s < 4; s++)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(aP[kc >> 2][kc & 3][s], b[kc % 3][s], acc, 0, 0, 0);
+            }
+            const int o_unit = __builtin_amdgcn_readfirstlane((utile * 16 * ldn + 16 * jj) * 4);
+            const unsigned o_lane_q = (unsigned)(4 * q * ldn + n_off + l16) * 4u;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[r] + bias_l), o_rsrc, o_lane_q, o_unit + r * ldn * 4, 0);
         }
     }
 }
