@@ -100,34 +100,54 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
     // workgroups together are a third of a 256-channel input, far more memory time than the filter,
     // which comes from L2), but before the filter is written to LDS ---------------------------------------------------
     constexpr int QUADS = N * K / 4;
-    for (int base = 0; base < QUADS; base += 512 * 8) {
-        float4 v[8];
+    const int first_tile = tile < t_main ? tile : w < units ? unit_tile : t_end - 1;
+    if (!p.b_kmajor) {
+        // [N][K]: a row of the filter is a row of Bs
+        for (int base = 0; base < QUADS; base += 512 * 8) {
+            float4 v[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int idx = min(base + t + 512 * u, QUADS - 1);
-            if (!p.b_kmajor) {
+            for (int u = 0; u < 8; u++) {
+                const int idx = min(base + t + 512 * u, QUADS - 1);
                 const int n = idx / (K / 4), k4 = (idx % (K / 4)) * 4;
                 v[u] = *reinterpret_cast<const float4 *>(p.B + (size_t)(n_off + n) * K + k4);
-            } else {
-                const int k = idx % K, n4 = (idx / K) * 4;
-                v[u] = *reinterpret_cast<const float4 *>(p.B + (size_t)k * ldn + n_off + n4);
             }
-        }
-        if (base + 512 * 8 >= QUADS) load_a(aP, tile < t_main ? tile : w < units ? unit_tile : t_end - 1);
+            if (base + 512 * 8 >= QUADS) load_a(aP, first_tile);
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int idx = base + t + 512 * u;
-            if (idx < QUADS) {
-                if (!p.b_kmajor) {
+            for (int u = 0; u < 8; u++) {
+                const int idx = base + t + 512 * u;
+                if (idx < QUADS) {
                     const int n = idx / (K / 4), k4 = (idx % (K / 4)) * 4;
                     *reinterpret_cast<float4 *>(Bs + n * KS + k4) = v[u];
-                } else {
-                    const int k = idx % K, n4 = (idx / K) * 4;
-                    Bs[(n4 + 0) * KS + k] = v[u].x;
-                    Bs[(n4 + 1) * KS + k] = v[u].y;
-                    Bs[(n4 + 2) * KS + k] = v[u].z;
-                    Bs[(n4 + 3) * KS + k] = v[u].w;
                 }
+            }
+        }
+    } else {
+        // [K][ldn]: transposed on the way. A thread takes a cell of 4 k x 4 n: four 128-bit loads (rows k..k+3), a 4x4
+        // transpose in registers, four 128-bit LDS stores (rows n..n+3 of Bs). The 64 lanes of a wavefront form a tile
+        // of 8 cells along k x 8 along n: a load touches 8 rows x 128 contiguous bytes, and the 32 lanes of a half
+        // wavefront store to 32 different 16-byte slots (a row of Bs is 8 floats modulo 16 longer than a power of two).
+        // (One lane per k with scalar transposing stores touched 64 cache lines per load and staged in 12-17 k cycles.)
+        constexpr int CELLS = 64 * NT * KB, TKT = 2 * KB, ITER = (CELLS + 511) / 512;
+        float4 v[ITER][4];
+        int k0[ITER], n0[ITER];
+#pragma unroll
+        for (int it = 0; it < ITER; it++) {
+            const int tile8 = min(w + 8 * it, CELLS / 64 - 1);
+            k0[it] = 4 * (8 * (tile8 % TKT) + (lane & 7));
+            n0[it] = 4 * (8 * (tile8 / TKT) + (lane >> 3));
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                v[it][r] = *reinterpret_cast<const float4 *>(p.B + (size_t)(k0[it] + r) * ldn + n_off + n0[it]);
+        }
+        load_a(aP, first_tile);
+#pragma unroll
+        for (int it = 0; it < ITER; it++) {
+            if (w + 8 * it < CELLS / 64) {
+                float *dst = Bs + n0[it] * KS + k0[it];
+                *reinterpret_cast<float4 *>(dst) = make_float4(v[it][0].x, v[it][1].x, v[it][2].x, v[it][3].x);
+                *reinterpret_cast<float4 *>(dst + KS) = make_float4(v[it][0].y, v[it][1].y, v[it][2].y, v[it][3].y);
+                *reinterpret_cast<float4 *>(dst + 2 * KS) = make_float4(v[it][0].z, v[it][1].z, v[it][2].z, v[it][3].z);
+                *reinterpret_cast<float4 *>(dst + 3 * KS) = make_float4(v[it][0].w, v[it][1].w, v[it][2].w, v[it][3].w);
             }
         }
     }
