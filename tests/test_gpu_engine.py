@@ -234,3 +234,45 @@ def test_engine_random_geometries(dev, eng, case):
     check(dev.get(y), O.conv3D_f64(X, W, sh, sw, ph, pw), "conv3D %s" % (case,))
     check(dev.get(dx), O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw), "deltaX %s" % (case,))
     check(dev.get(dw), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "deltaW %s" % (case,))
+
+
+def _random_3x3_cases(count, seed):
+    """Seeded random 3x3 stride-1 layers with channel counts the LDS-halo kernels take: row widths from 3 to 62 (both
+    row-width classes of the halo-prefetching kernel and its limits), batch sizes that give anything from a fraction of
+    a unit to several units per workgroup plus left-over pieces, pads 0..2, ragged output channel counts."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    cases = []
+    while len(cases) < count:
+        IH, IW = int(rng.integers(3, 41)), int(rng.integers(3, 63))
+        IC = int(rng.choice([32, 64, 96, 128]))
+        OC = int(rng.choice([16, 48, 64, 80, 128]))
+        ph, pw = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        N = int(rng.choice([1, 3, 4, 8, 20, 60, 150]))
+        OH, OW = out_dim(IH, IW, 3, 3, 1, 1, ph, pw)
+        if OH < 1 or OW < 1 or N * OH * OW * OC * IC * 18 > 1.5e9 or N * IH * IW * IC > 6_000_000:
+            continue
+        cases.append((N, IH, IW, IC, OC, ph, pw))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_3x3_cases(20, 20241125))
+def test_engine_random_3x3_stride1_layers(dev, eng, case):
+    N, IH, IW, IC, OC, ph, pw = case
+    OH, OW = out_dim(IH, IW, 3, 3, 1, 1, ph, pw)
+    seed = 9000 + (hash(case) % 1000)
+    X, W, dY = normal((N, IH, IW, IC), seed), he_normal(OC, 3, 3, IC, seed + 1), normal((N, OH, OW, OC), seed + 2)
+    x, w, dy = dev.put(X), dev.put(W), dev.put(dY)
+    y, y_w = dev.guarded(N, OH, OW, OC), dev.guarded(N, OH, OW, OC)
+    dx = dev.guarded(N, IH, IW, IC)
+    dw = dev.guarded(OC, 3, 3, IC)
+    eng.conv3D(y.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, ph, pw)
+    pkg.Cuda_conv3D.conv3D(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), 3, 3, y_w.data_ptr(), OH, OW, N, IC, OC, 1, 1, ph, pw)
+    eng.dconv3D_deltaX(dx.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, ph, pw)
+    eng.dconv3D_deltaW(dw.data_ptr(), 3, 3, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, 1, 1, ph, pw)
+    eng.sync()
+    want = O.conv3D_f64(X, W, 1, 1, ph, pw)
+    check(dev.get(y), want, "conv3D %s" % (case,))
+    check(dev.get(y_w), want, "conv3D from W %s" % (case,))
+    check(dev.get(dx), O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw), "deltaX %s" % (case,))
+    check(dev.get(dw), O.deltaW_f64(X, dY, 3, 3, 1, 1, ph, pw), "deltaW %s" % (case,))
+
