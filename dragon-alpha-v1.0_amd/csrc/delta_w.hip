@@ -52,15 +52,16 @@ __global__ __launch_bounds__(256, 2) void delta_w_kernel(const DeltaWArgs p)
     const bool ycolv = ycol < OC;
     const int ykrow = t / LPR_Y;
 
-    float4 yreg[Y_PASSES], xreg[X_PASSES];
-    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    // (the vector type, not the float4 struct: copies of the struct keep these arrays in scratch memory)
+    floatx4 yreg[Y_PASSES], xreg[X_PASSES];
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
     auto load_global = [&](int kbase) {
 #pragma unroll
         for (int q = 0; q < Y_PASSES; q++) {
             const int k = kbase + ykrow + RPP_Y * q;
             const bool ok = ycolv && k < k_end;
-            yreg[q] = ok ? *reinterpret_cast<const float4 *>(p.dY + (size_t)k * OC + ycol) : zero4;
+            yreg[q] = ok ? *reinterpret_cast<const floatx4 *>(p.dY + (size_t)k * OC + ycol) : zero4;
         }
 #pragma unroll
         for (int q = 0; q < X_PASSES; q++) {
@@ -70,16 +71,16 @@ __global__ __launch_bounds__(256, 2) void delta_w_kernel(const DeltaWArgs p)
             const int ih = oh * p.sh - p.ph + x_fh, iw = ow * p.sw - p.pw + x_fw;
             const bool ok = xcolv && k < k_end && (unsigned)ih < (unsigned)IH && (unsigned)iw < (unsigned)IW;
             const int off = ((n * IH + ih) * IW + iw) * IC + x_ic;
-            xreg[q] = ok ? *reinterpret_cast<const float4 *>(p.X + off) : zero4;
+            xreg[q] = ok ? *reinterpret_cast<const floatx4 *>(p.X + off) : zero4;
         }
     };
     auto store_lds = [&](int buf) {
 #pragma unroll
         for (int q = 0; q < Y_PASSES; q++)
-            *reinterpret_cast<float4 *>(Ys + buf * Y_TILE + (ykrow + RPP_Y * q) * YS + (t % LPR_Y) * 4) = yreg[q];
+            *reinterpret_cast<floatx4 *>(Ys + buf * Y_TILE + (ykrow + RPP_Y * q) * YS + (t % LPR_Y) * 4) = yreg[q];
 #pragma unroll
         for (int q = 0; q < X_PASSES; q++)
-            *reinterpret_cast<float4 *>(Xs + buf * X_TILE + (xkrow + RPP_X * q) * XS + (t % LPR_X) * 4) = xreg[q];
+            *reinterpret_cast<floatx4 *>(Xs + buf * X_TILE + (xkrow + RPP_X * q) * XS + (t % LPR_X) * 4) = xreg[q];
     };
 
     floatx16 acc[TM][TN];

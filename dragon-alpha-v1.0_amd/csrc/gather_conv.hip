@@ -80,8 +80,9 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
     const int b_col = B_NMAJOR ? n0 + (t % LPR) * 4 : 0;
     const int b_krow = t / LPR;
 
-    float4 areg[A_PASSES], breg[B_PASSES];
-    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    // (the vector type, not the float4 struct: copies of the struct keep these arrays in scratch memory)
+    floatx4 areg[A_PASSES], breg[B_PASSES];
+    const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
     auto load_global = [&](int it) {
         const int k = it * BK + kq;
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
             const int ih = a_ih0[q] + th, iw = a_iw0[q] + tw;
             const bool ok = kv && (unsigned)ih < (unsigned)AH && (unsigned)iw < (unsigned)AW;
             const int off = a_base[q] + (ih * AW + iw) * AC + c;
-            areg[q] = ok ? *reinterpret_cast<const float4 *>(p.A + off) : zero4;
+            areg[q] = ok ? *reinterpret_cast<const floatx4 *>(p.A + off) : zero4;
         }
         if (B_NMAJOR) {
 #pragma unroll
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
                 const int thb = fdiv(tapb, p.d_TW), twb = tapb - thb * TW;
                 const bool ok = kb < K && b_col < CO;
                 const int off = p.b_off + thb * p.b_sth + twb * p.b_stw + cb * p.b_sc + b_col;
-                breg[q] = ok ? *reinterpret_cast<const float4 *>(p.B + off) : zero4;
+                breg[q] = ok ? *reinterpret_cast<const floatx4 *>(p.B + off) : zero4;
             }
         } else {
             const int koff = p.b_off + th * p.b_sth + tw * p.b_stw + c;
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
                 const int col = n0 + (t >> 3) + 32 * q;
                 const bool ok = kv && col < CO;
                 const int off = koff + col * p.b_sn;
-                breg[q] = ok ? *reinterpret_cast<const float4 *>(p.B + off) : zero4;
+                breg[q] = ok ? *reinterpret_cast<const floatx4 *>(p.B + off) : zero4;
             }
         }
     };
@@ -122,15 +123,15 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
         float *bs = Bs + buf * B_TILE;
 #pragma unroll
         for (int q = 0; q < A_PASSES; q++)
-            *reinterpret_cast<float4 *>(as + ((t >> 3) + 32 * q) * AS + kq) = areg[q];
+            *reinterpret_cast<floatx4 *>(as + ((t >> 3) + 32 * q) * AS + kq) = areg[q];
         if (B_NMAJOR) {
 #pragma unroll
             for (int q = 0; q < B_PASSES; q++)
-                *reinterpret_cast<float4 *>(bs + (b_krow + RPP * q) * BSN + (t % LPR) * 4) = breg[q];
+                *reinterpret_cast<floatx4 *>(bs + (b_krow + RPP * q) * BSN + (t % LPR) * 4) = breg[q];
         } else {
 #pragma unroll
             for (int q = 0; q < B_PASSES; q++)
-                *reinterpret_cast<float4 *>(bs + ((t >> 3) + 32 * q) * BSK + kq) = breg[q];
+                *reinterpret_cast<floatx4 *>(bs + ((t >> 3) + 32 * q) * BSK + kq) = breg[q];
         }
     };
 

@@ -190,9 +190,9 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
 #pragma unroll
             for (int g = 0; g < NG; g++) bsel[g] = bias4[g];
         } else {
-            bsel[0] = bias4[0];
-#pragma unroll
-            for (int g = 1; g < NG; g++) bsel[0] = g0 == g ? bias4[g] : bsel[0];
+            // one group of a tile (the units behind the last multiple of eight tiles): its bias comes from memory (picked
+            // out of bias4[] by g0 the compiler indexes the array, which puts it into scratch)
+            bsel[0] = p.bias ? *reinterpret_cast<const floatx4 *>(p.bias + n_off + 64 * g0 + 4 * l16) : zero;
         }
 
         floatx4 acc[NGX][4], v[4], b[3];
