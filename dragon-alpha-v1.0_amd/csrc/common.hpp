@@ -50,6 +50,20 @@ inline hipError_t ensure_dynamic_lds(size_t bytes)
     return hipSuccess;
 }
 
+// Compute units of the current device (0 if it cannot be read); cached per device, a racing first call writes the same value.
+inline int device_cu_count()
+{
+    static int cu_count[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cu_count[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return 0;
+        cu_count[dev] = n;
+    }
+    return cu_count[dev];
+}
+
 // One launch of the generic implicit-GEMM "gather convolution":
 //   O[o_off + n*o_sn + i*o_sh + j*o_sw + co] =
 //       sum_{th<TH, tw<TW, c<AC}  A[n, i*sh - ph + th, j*sw - pw + tw, c] * B[b_off + th*b_sth + tw*b_stw + c*b_sc + co*b_sn]
@@ -139,6 +153,10 @@ hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const flo
 hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC);
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias = nullptr);
+// The same as one MFMA stream per persistent workgroup (winograd_stream.hip), for IC % 16 == 0; returns
+// hipErrorNotSupported (nothing launched) otherwise.
+hipError_t launch_winograd_stream(hipStream_t stream, const float *X, const float *U, float *Y,
+                                  int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias = nullptr);
 
 // Re-layout / reduction helpers.
 hipError_t launch_kernel_remode(hipStream_t s, const float *W, float *CW, int FH, int FW, int OC, int IC);

@@ -425,15 +425,8 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
     a.d_PHt = make_fastdiv(a.PHt);
     a.d_PWt = make_fastdiv(a.PWt);
 
-    static int cu_count[64] = {0};   // per device; a racing first call writes the same value
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorNotSupported;
-    if (cu_count[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return hipErrorNotSupported;
-        cu_count[dev] = n;
-    }
-    const int cus = cu_count[dev];
+    const int cus = device_cu_count();
+    if (cus < 1) return hipErrorNotSupported;
     if (sh == 1 && sw == 1) {   // the variant that prefetches the halo, where it applies
         const hipError_t e = launch_tap_conv_prefetch(stream, A, B, O, N, AH, AW, AC, OH, OW, CO, TH, TW, ph, pw,
                                                       b_off, b_sth, b_stw, b_sc, b_sn, bias, cus);

@@ -256,6 +256,8 @@ hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, f
                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias)
 {
     if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
+    if (const hipError_t e = launch_winograd_stream(stream, X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, bias); e != hipErrorNotSupported)
+        return e;   // the persistent variant, where it applies
     WinoArgs a{};
     a.X = X; a.U = U; a.Y = Y; a.bias = bias;
     a.N = N; a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC;

@@ -1,0 +1,330 @@
+// Winograd F(2x2, 3x3) forward convolution as one uninterrupted MFMA stream per workgroup, gfx950, for input channel
+// counts that are multiples of 16. Same arithmetic as winograd.hip (input transform -> 16 MFMA GEMMs, one per transform
+// position xi -> output transform, v_mfma_f32_16x16x4_f32, the transformed filter U[16][IC][OC] fetched from L2 through
+// a register ring); what differs is what happens between two output blocks.
+//
+// An item is 32 consecutive tiles of the flattened (n, tile row, tile column) index (2x2 output pixels each) times 64
+// output channels; a step is one 16-channel chunk of one item. The grid is persistent (two workgroups of 4 wavefronts
+// per compute unit) and a workgroup walks a contiguous range of items as one sequence of steps. Three cursors run along
+// that sequence, none of them stops at an item boundary:
+//   * the MFMAs of step k (wavefront w: output channels [16w, 16w+16) x 32 tiles x 16 xi = 128 accumulator registers),
+//   * the filter ring, four xi ahead of the MFMAs,
+//   * the input patches: the 4x4 patch of (tile, channel pair) for step k+2 is requested from memory during step k,
+//     transformed (B^T d B, per thread) and written as V[xi][tile][16 channels] into the other LDS buffer during step
+//     k+1, in the shadow of that step's MFMAs, and multiplied in step k+2.
+// So the only thing outside the MFMA stream is an item's output transform (A^T m A per lane, which holds all 16 xi of
+// its (tile, channel) pairs) and its stores, which leave the registers directly: 16 lanes write 64 consecutive bytes.
+// Items that do not divide evenly among the workgroups are cut into halves of 16 tiles (the second MFMA row block is
+// left out), so the longest workgroup is half an item above the shortest.
+#include "common.hpp"
+#include <type_traits>
+
+namespace alpha {
+
+struct WinoStreamArgs {
+    const float *X;      // [N, IH, IW, IC]
+    const float *U;      // [16][IC][OC]
+    float *Y;            // [N, OH, OW, OC]
+    const float *bias;   // NULL or [OC]
+    int IH, IW, IC, OH, OW, OC, ph, pw;
+    int TC, TRC;         // tile columns per image row, tiles per image
+    int ntiles, groups;  // N*TRC; groups of 32 tiles; item id = (block of 64 output channels) * groups + group
+    int x_bytes, u_bytes, y_bytes;   // each below 2 GB
+    int whole;           // items every workgroup takes: workgroup b owns [b*whole, (b+1)*whole)
+    int extra;           // workgroups below this take item gridDim.x*whole + b as well
+    int halves;          // or: workgroups below this take half (b & 1) of item gridDim.x*whole + b/2
+    FastDiv d_TC, d_TRC, d_groups;
+};
+
+constexpr int WS_TILES = 32;
+constexpr int WS_VBUF = 16 * WS_TILES * 16;   // floats per V buffer: [xi][tile][16 channels]
+constexpr unsigned WS_OOR = 0x80000000u;      // beyond every descriptor: loads return 0, stores are dropped
+
+__global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStreamArgs p)
+{
+    extern __shared__ __attribute__((aligned(16))) float ws_smem[];   // V[2][WS_VBUF]
+    float *smem = ws_smem;
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = t >> 6;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int xt = t >> 3, xq = (t & 7) * 2;   // input transform: thread -> (tile xt, channel pair xq of the chunk)
+    const int b = blockIdx.x, G = gridDim.x;
+    const int nitems = p.whole + (b < p.extra ? 1 : 0) + (b < p.halves ? 1 : 0);
+    const int nchunks = p.IC >> 4;
+    const unsigned xi_stride4 = (unsigned)p.IC * p.OC * 4;   // bytes between two transform positions of U
+    const unsigned chunk_stride4 = 16u * p.OC * 4;           // bytes between two 16-channel chunks of U
+
+    struct Item {
+        int tile_first, tile_end, oc0, half;
+    };
+    auto item_of = [&](int k) {   // uniform
+        Item it;
+        int id, hoff = 0;
+        it.half = 0;
+        if (k < p.whole) id = b * p.whole + k;
+        else if (p.extra) id = G * p.whole + b;
+        else {
+            id = G * p.whole + (b >> 1);
+            it.half = 1;
+            hoff = (b & 1) * 16;
+        }
+        const int ocb = fdiv(id, p.d_groups), g = id - ocb * p.groups;
+        it.oc0 = ocb * 64;
+        it.tile_first = g * WS_TILES + hoff;
+        const int end = it.tile_first + (it.half ? 16 : WS_TILES);
+        it.tile_end = end < p.ntiles ? end : p.ntiles;
+        return it;
+    };
+
+    floatx4 acc[16][2];
+#pragma unroll
+    for (int x = 0; x < 16; x++) {
+        acc[x][0] = floatx4{0.f, 0.f, 0.f, 0.f};
+        acc[x][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- input patches: descriptor base + uniform channel offset + per-lane pixel offset (fixed for an item) ----------
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
+    float2 d[4][4];
+    unsigned p_off[4][4];
+    auto patch_offsets = [&](const Item &it) {
+        // computed for every lane, selected at the end: no divergent branches in the MFMA stream
+        const int tile = it.tile_first + xt;
+        const bool tile_ok = tile < it.tile_end;
+        const int n = fdiv(tile, p.d_TRC), rem = tile - n * p.TRC;
+        const int ty = fdiv(rem, p.d_TC), tx = rem - ty * p.TC;
+        const int ih0 = 2 * ty - p.ph, iw0 = 2 * tx - p.pw;
+        const int x_base = n * p.IH * p.IW * p.IC + xq;
+        int rowpart[4], colpart[4];
+        bool row_ok[4], col_ok[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            row_ok[i] = tile_ok && (unsigned)(ih0 + i) < (unsigned)p.IH;
+            rowpart[i] = x_base + (ih0 + i) * p.IW * p.IC;
+            col_ok[i] = (unsigned)(iw0 + i) < (unsigned)p.IW;
+            colpart[i] = (iw0 + i) * p.IC;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                p_off[i][j] = (row_ok[i] && col_ok[j]) ? (unsigned)(rowpart[i] + colpart[j]) * 4u : WS_OOR;
+    };
+    auto load_patch = [&](int icc) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                d[i][j] = __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, p_off[i][j], icc * 4, 0));
+    };
+    // V = B^T d B, B^T = [[1,0,-1,0],[0,1,1,0],[0,-1,1,0],[0,1,0,-1]]
+    auto sub = [](float2 a, float2 c) { return make_float2(a.x - c.x, a.y - c.y); };
+    auto add = [](float2 a, float2 c) { return make_float2(a.x + c.x, a.y + c.y); };
+    float2 r[4][4];   // B^T d, alive between the two halves of the transform
+    auto transform_columns = [&]() {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            r[0][j] = sub(d[0][j], d[2][j]);
+            r[1][j] = add(d[1][j], d[2][j]);
+            r[2][j] = sub(d[2][j], d[1][j]);
+            r[3][j] = sub(d[1][j], d[3][j]);
+        }
+    };
+    auto transform_row_store = [&](float *Vw, int i) {
+        const float2 v0 = sub(r[i][0], r[i][2]), v1 = add(r[i][1], r[i][2]), v2 = sub(r[i][2], r[i][1]), v3 = sub(r[i][1], r[i][3]);
+        *reinterpret_cast<float2 *>(Vw + (4 * i + 0) * WS_TILES * 16) = v0;
+        *reinterpret_cast<float2 *>(Vw + (4 * i + 1) * WS_TILES * 16) = v1;
+        *reinterpret_cast<float2 *>(Vw + (4 * i + 2) * WS_TILES * 16) = v2;
+        *reinterpret_cast<float2 *>(Vw + (4 * i + 3) * WS_TILES * 16) = v3;
+    };
+
+    // ---- transformed filter: lane (l16, q) needs U[xi][chunk*16 + 4q + s][oc0 + 16w + l16]; columns beyond OC read
+    //      something finite or the range check's zero and are never stored --------------------------------------------
+    const __amdgpu_buffer_rsrc_t u_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.U), 0, p.u_bytes, 0x00020000);
+    unsigned u_lane[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) u_lane[s] = (unsigned)((4 * q + s) * p.OC + 16 * w + l16) * 4u;
+    float bring[4][4];
+    auto load_b = [&](float (&bb)[4], unsigned block) {   // block: uniform byte offset of (xi, chunk, oc0)
+#pragma unroll
+        for (int s = 0; s < 4; s++) bb[s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(u_rsrc, u_lane[s], block, 0));
+    };
+
+    // ---- output: lane (l16, q) holds tiles 16mt + 4q + r (r = accumulator component) of channel oc0 + 16w + l16 ---------
+    const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.Y, 0, p.y_bytes, 0x00020000);
+    auto store_item = [&](auto half_c, const Item &it) {
+        constexpr bool HALF = decltype(half_c)::value;
+        const int col = it.oc0 + 16 * w + l16;
+        const bool col_ok = col < p.OC;
+        float bias_v = 0.f;
+        if (p.bias && col_ok) bias_v = p.bias[col];
+        const unsigned row4 = (unsigned)p.OW * p.OC * 4u, px4 = (unsigned)p.OC * 4u;
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) {
+            if (mt == 1 && HALF) break;
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+                const int tile = it.tile_first + 16 * mt + 4 * q + rr;
+                const bool ok = tile < it.tile_end && col_ok;
+                const int n = fdiv(tile, p.d_TRC), rem = tile - n * p.TRC;
+                const int ty = fdiv(rem, p.d_TC), tx = rem - ty * p.TC;
+                const int oh = 2 * ty, ow = 2 * tx;
+                const unsigned o = (unsigned)(((n * p.OH + oh) * p.OW + ow) * p.OC + col) * 4u;
+                const bool right = ok && ow + 1 < p.OW, below = ok && oh + 1 < p.OH;
+                const unsigned o00 = ok ? o : WS_OOR, o01 = right ? o + px4 : WS_OOR;
+                const unsigned o10 = below ? o + row4 : WS_OOR, o11 = (right && below) ? o + row4 + px4 : WS_OOR;
+                // Y = A^T m A, A^T = [[1,1,1,0],[0,1,-1,-1]], m[a][c] = acc[4a + c]
+                float s0[4], s1[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const float m0 = acc[c][mt][rr], m1 = acc[4 + c][mt][rr], m2 = acc[8 + c][mt][rr], m3 = acc[12 + c][mt][rr];
+                    s0[c] = m0 + m1 + m2;
+                    s1[c] = m1 - m2 - m3;
+                }
+                const float y00 = s0[0] + s0[1] + s0[2] + bias_v, y01 = s0[1] - s0[2] - s0[3] + bias_v;
+                const float y10 = s1[0] + s1[1] + s1[2] + bias_v, y11 = s1[1] - s1[2] - s1[3] + bias_v;
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y00), y_rsrc, o00, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y01), y_rsrc, o01, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y10), y_rsrc, o10, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y11), y_rsrc, o11, 0, 0);
+            }
+        }
+    };
+
+    // ---- start: V of step 0, the patch of step 1 on its way, the ring filled ------------------------------------------
+    Item cur = item_of(0);
+    int pk = 0, pc = 0;   // patch cursor: item and chunk of the patch in d
+    auto advance_patch = [&]() {   // moves the cursor one step on and requests that step's patch
+        pc++;
+        if (pc == nchunks) {
+            pc = 0;
+            pk++;
+            if (pk < nitems) patch_offsets(item_of(pk));
+        }
+        load_patch(pc * 16);   // beyond the last step: a patch nobody multiplies (its addresses are valid)
+    };
+    patch_offsets(cur);
+    load_patch(0);
+    transform_columns();
+#pragma unroll
+    for (int i = 0; i < 4; i++) transform_row_store(smem + xt * 16 + xq, i);
+    advance_patch();
+    {
+        const unsigned u0 = (unsigned)cur.oc0 * 4u;
+#pragma unroll
+        for (int x = 0; x < 4; x++) load_b(bring[x], u0 + x * xi_stride4);
+    }
+    __syncthreads();
+
+    // ---- one step: 16 xi x (2 LDS fragments, 4 filter elements, 8 MFMAs); in their shadow the next step's V ----------
+    // Every xi is a scheduling region of its own (nothing crosses its borders), in program order: the LDS fragments of
+    // the next xi, the ring refill, 8 MFMAs, and in their shadow a slice of the next step's preparation. Left to
+    // itself the scheduler dissolves the ring (loads issued right before their use) and moves the patch loads to the
+    // end of the step and their transform to the start of the next one, with nothing in between to cover the latency.
+    auto chunk = [&](auto half_c, int buf, unsigned ucur, unsigned unext) {
+        constexpr bool HALF = decltype(half_c)::value;
+        const float *V = smem + buf * WS_VBUF + l16 * 16 + 4 * q;
+        float *Vw = smem + (buf ^ 1) * WS_VBUF + xt * 16 + xq;
+        floatx4 a0 = *reinterpret_cast<const floatx4 *>(V);
+        floatx4 a1 = a0;
+        if (!HALF) a1 = *reinterpret_cast<const floatx4 *>(V + 16 * 16);
+#pragma unroll
+        for (int xi = 0; xi < 16; xi++) {
+            __builtin_amdgcn_sched_barrier(0);
+            floatx4 a0n = a0, a1n = a1;
+            if (xi < 15) {
+                a0n = *reinterpret_cast<const floatx4 *>(V + (xi + 1) * WS_TILES * 16);
+                if (!HALF) a1n = *reinterpret_cast<const floatx4 *>(V + (xi + 1) * WS_TILES * 16 + 16 * 16);
+            }
+            float bb[4];
+#pragma unroll
+            for (int s = 0; s < 4; s++) bb[s] = bring[xi & 3][s];
+            {   // refill this ring slot with the fragment needed four positions later (possibly in the next step)
+                const int nx = xi + 4;
+                load_b(bring[xi & 3], nx < 16 ? ucur + nx * xi_stride4 : unext + (nx - 16) * xi_stride4);
+            }
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                acc[xi][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[s], bb[s], acc[xi][0], 0, 0, 0);
+                if (!HALF) acc[xi][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[s], bb[s], acc[xi][1], 0, 0, 0);
+            }
+            if (xi == 3) transform_columns();                // consumes the patch of the next step
+            if (xi == 4 || xi == 5) {                        // writes that step's V
+                transform_row_store(Vw, 2 * (xi - 4));
+                transform_row_store(Vw, 2 * (xi - 4) + 1);
+            }
+            if (xi == 6) advance_patch();                    // requests the patch of the step after it
+            a0 = a0n;
+            a1 = a1n;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // whole items first, then the half item if this workgroup has one: two copies of the step, one after the other
+    int buf = 0;
+    auto run_item = [&](auto half_c, int k) {
+        const bool has_next = k + 1 < nitems;
+        Item nxt = cur;
+        if (has_next) nxt = item_of(k + 1);
+        const unsigned u_item = (unsigned)cur.oc0 * 4u;
+        for (int c = 0; c < nchunks; c++) {
+            const unsigned ucur = u_item + c * chunk_stride4;
+            const unsigned unext = c + 1 < nchunks ? ucur + chunk_stride4 : (has_next ? (unsigned)nxt.oc0 * 4u : 0u);
+            chunk(half_c, buf, ucur, unext);
+            __syncthreads();
+            buf ^= 1;
+        }
+        store_item(half_c, cur);
+#pragma unroll
+        for (int x = 0; x < 16; x++) {
+            acc[x][0] = floatx4{0.f, 0.f, 0.f, 0.f};
+            acc[x][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+        cur = nxt;
+    };
+    const int nfull = b < p.halves ? nitems - 1 : nitems;
+    for (int k = 0; k < nfull; k++) run_item(std::false_type{}, k);
+    if (nfull < nitems) run_item(std::true_type{}, nfull);
+}
+
+hipError_t launch_winograd_stream(hipStream_t stream, const float *X, const float *U, float *Y,
+                                  int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias)
+{
+    if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
+    if (IC < 16 || IC % 16 != 0 || OC < 1 || N < 1 || OH < 1 || OW < 1) return hipErrorNotSupported;
+    const long x_bytes = (long)N * IH * IW * IC * 4, y_bytes = (long)N * OH * OW * OC * 4, u_bytes = 16L * IC * OC * 4;
+    if (x_bytes >= (1L << 31) || y_bytes >= (1L << 31) || u_bytes >= (1L << 31)) return hipErrorNotSupported;
+    const int cus = device_cu_count();
+    if (cus < 1) return hipErrorNotSupported;
+
+    WinoStreamArgs a{};
+    a.X = X; a.U = U; a.Y = Y; a.bias = bias;
+    a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC; a.ph = ph; a.pw = pw;
+    a.TC = (OW + 1) / 2;
+    a.TRC = ((OH + 1) / 2) * a.TC;
+    const long nt = (long)N * a.TRC;
+    if (nt >= (1L << 30)) return hipErrorNotSupported;
+    a.ntiles = (int)nt;
+    a.groups = (a.ntiles + WS_TILES - 1) / WS_TILES;
+    a.x_bytes = (int)x_bytes; a.y_bytes = (int)y_bytes; a.u_bytes = (int)u_bytes;
+    a.d_TC = make_fastdiv(a.TC);
+    a.d_TRC = make_fastdiv(a.TRC);
+    a.d_groups = make_fastdiv(a.groups);
+    const long items = (long)a.groups * ((OC + 63) / 64);
+    if (items >= (1L << 30)) return hipErrorNotSupported;
+    const int slots = 2 * cus;
+    const int grid = items < slots ? (int)items : slots;
+    a.whole = (int)(items / grid);
+    const int left = (int)(items - (long)a.whole * grid);   // < grid
+    if (2 * left <= grid) a.halves = 2 * left;
+    else a.extra = left;
+
+    constexpr auto kern = winograd_stream_kernel;
+    const size_t lds = (size_t)2 * WS_VBUF * sizeof(float);
+    if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace alpha

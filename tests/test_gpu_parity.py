@@ -207,6 +207,12 @@ WINO_SHAPES = [
     (4, 6, 9, 32, 64, 2, 2),         # padding 2
     (3, 5, 5, 64, 64, 1, 1),         # fewer tiles than one workgroup
     (4, 32, 32, 4, 64, 1, 1),        # BASELINE config 1 geometry (IC = 3 stored as 4)
+    # persistent kernel (IC % 16 == 0), 512 workgroups on 256 compute units:
+    (25, 56, 56, 16, 16, 1, 1),      # 613 items: one whole item each, 101 left over -> 202 half items, ragged last group
+    (40, 56, 56, 16, 20, 1, 1),      # 980 items: 468 left over -> whole extra items; 20 of 64 output channels
+    (16, 56, 56, 32, 128, 1, 1),     # 784 items in two blocks of output channels, two chunks
+    (66, 55, 53, 16, 16, 1, 1),      # 1560 items: three whole items each, 24 left over -> 48 half items; odd sizes
+    (2, 9, 9, 48, 72, 1, 1),         # fewer items than workgroups, ragged block of output channels
 ]
 
 
@@ -219,7 +225,7 @@ def test_forward_winograd_f2x2_vs_direct_oracle(dev, shape):
     X, W = normal((N, IH, IW, IC), 1201), he_normal(OC, 3, 3, IC, 1202)
     x, w = dev.put(X), dev.put(W)
     U = dev.empty(C3.winograd_filter_size(IC, OC), fill=float("nan"))
-    y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    y = dev.guarded(N, OH, OW, OC)
     C3.winograd_filter_transform(dev.stream, w.data_ptr(), U.data_ptr(), IC, OC)
     C3.conv3D_winograd(dev.streams, 1, x.data_ptr(), IH, IW, U.data_ptr(), y.data_ptr(), OH, OW, N, IC, OC, ph, pw)
     check(dev.get(y), O.conv3D_f64(X, W, 1, 1, ph, pw), "winograd %s" % (shape,))
