@@ -29,7 +29,7 @@ struct WinoStreamArgs {
     int IH, IW, IC, OH, OW, OC, ph, pw;
     int TC, TRC;         // tile columns per image row, tiles per image
     int ntiles, groups;  // N*TRC; groups of 32 tiles; item id = (block of 64 output channels) * groups + group
-    int x_bytes, u_bytes, y_bytes;   // each below 2 GB
+    int x_bytes, u_bytes, y_bytes;   // X and U below 2 GB, Y at most 1 GB
     int whole;           // items every workgroup takes: workgroup b owns [b*whole, (b+1)*whole)
     int extra;           // workgroups below this take item gridDim.x*whole + b as well
     int halves;          // or: workgroups below this take half (b & 1) of item gridDim.x*whole + b/2
@@ -42,7 +42,7 @@ constexpr unsigned WS_OOR = 0x80000000u;      // beyond every descriptor: loads 
 
 __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStreamArgs p)
 {
-    extern __shared__ __attribute__((aligned(16))) float ws_smem[];   // V[2][WS_VBUF]
+    extern __shared__ __attribute__((aligned(16))) float ws_smem[];   // V[2][WS_VBUF], otab[2][32][4]
     float *smem = ws_smem;
 
     const int t = threadIdx.x;
@@ -77,12 +77,7 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
         return it;
     };
 
-    floatx4 acc[16][2];
-#pragma unroll
-    for (int x = 0; x < 16; x++) {
-        acc[x][0] = floatx4{0.f, 0.f, 0.f, 0.f};
-        acc[x][1] = floatx4{0.f, 0.f, 0.f, 0.f};
-    }
+    floatx4 acc[16][2];   // every item's first step starts them from zero
 
     // ---- input patches: descriptor base + uniform channel offset + per-lane pixel offset (fixed for an item) ----------
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
@@ -111,12 +106,12 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
             for (int j = 0; j < 4; j++)
                 p_off[i][j] = (row_ok[i] && col_ok[j]) ? (unsigned)(rowpart[i] + colpart[j]) * 4u : WS_OOR;
     };
+    auto load_patch_element = [&](int e, int icc) {   // e = 4i + j
+        d[e >> 2][e & 3] = __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, p_off[e >> 2][e & 3], icc * 4, 0));
+    };
     auto load_patch = [&](int icc) {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                d[i][j] = __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, p_off[i][j], icc * 4, 0));
+        for (int e = 0; e < 16; e++) load_patch_element(e, icc);
     };
     // V = B^T d B, B^T = [[1,0,-1,0],[0,1,1,0],[0,-1,1,0],[0,1,0,-1]]
     auto sub = [](float2 a, float2 c) { return make_float2(a.x - c.x, a.y - c.y); };
@@ -131,12 +126,11 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
             r[3][j] = sub(d[1][j], d[3][j]);
         }
     };
-    auto transform_row_store = [&](float *Vw, int i) {
-        const float2 v0 = sub(r[i][0], r[i][2]), v1 = add(r[i][1], r[i][2]), v2 = sub(r[i][2], r[i][1]), v3 = sub(r[i][1], r[i][3]);
-        *reinterpret_cast<float2 *>(Vw + (4 * i + 0) * WS_TILES * 16) = v0;
-        *reinterpret_cast<float2 *>(Vw + (4 * i + 1) * WS_TILES * 16) = v1;
-        *reinterpret_cast<float2 *>(Vw + (4 * i + 2) * WS_TILES * 16) = v2;
-        *reinterpret_cast<float2 *>(Vw + (4 * i + 3) * WS_TILES * 16) = v3;
+    auto transform_half_row_store = [&](float *Vw, int i, int h) {   // V positions 4i + 2h, 4i + 2h + 1
+        const float2 va = h == 0 ? sub(r[i][0], r[i][2]) : sub(r[i][2], r[i][1]);
+        const float2 vb = h == 0 ? add(r[i][1], r[i][2]) : sub(r[i][1], r[i][3]);
+        *reinterpret_cast<float2 *>(Vw + (4 * i + 2 * h + 0) * WS_TILES * 16) = va;
+        *reinterpret_cast<float2 *>(Vw + (4 * i + 2 * h + 1) * WS_TILES * 16) = vb;
     };
 
     // ---- transformed filter: lane (l16, q) needs U[xi][chunk*16 + 4q + s][oc0 + 16w + l16]; columns beyond OC read
@@ -152,28 +146,44 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
     };
 
     // ---- output: lane (l16, q) holds tiles 16mt + 4q + r (r = accumulator component) of channel oc0 + 16w + l16 ---------
+    // The byte offsets of a tile's four pixels (channel 0; beyond the descriptor where the tile or the pixel does not
+    // exist) are computed once per item by 32 threads, in the shadow of the item's first step, and kept in LDS:
+    // otab[item parity][tile][4]. The output transform then costs one LDS read and four additions per tile for addresses.
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.Y, 0, p.y_bytes, 0x00020000);
-    auto store_item = [&](auto half_c, const Item &it) {
-        constexpr bool HALF = decltype(half_c)::value;
+    unsigned *otab = reinterpret_cast<unsigned *>(smem + 2 * WS_VBUF);
+    auto write_offset_table = [&](const Item &it, int parity) {
+        const int tile = it.tile_first + (t & 31);
+        const bool ok = tile < it.tile_end;
+        const int n = fdiv(tile, p.d_TRC), rem = tile - n * p.TRC;
+        const int ty = fdiv(rem, p.d_TC), tx = rem - ty * p.TC;
+        const int oh = 2 * ty, ow = 2 * tx;
+        const unsigned row4 = (unsigned)p.OW * p.OC * 4u, px4 = (unsigned)p.OC * 4u;
+        const unsigned o = (unsigned)(((n * p.OH + oh) * p.OW + ow) * p.OC) * 4u;
+        const bool right = ok && ow + 1 < p.OW, below = ok && oh + 1 < p.OH;
+        uint4 e;
+        e.x = ok ? o : WS_OOR;
+        e.y = right ? o + px4 : WS_OOR;
+        e.z = below ? o + row4 : WS_OOR;
+        e.w = (right && below) ? o + row4 + px4 : WS_OOR;
+        if (t < 32) *reinterpret_cast<uint4 *>(otab + parity * 128 + t * 4) = e;
+    };
+    float bias_v = 0.f;     // of the current item's channel
+    unsigned col4 = 0;      // its byte offset; 1 GB (beyond the descriptor, also when added to WS_OOR) for channels >= OC
+    auto item_column = [&](const Item &it) {
         const int col = it.oc0 + 16 * w + l16;
         const bool col_ok = col < p.OC;
-        float bias_v = 0.f;
-        if (p.bias && col_ok) bias_v = p.bias[col];
-        const unsigned row4 = (unsigned)p.OW * p.OC * 4u, px4 = (unsigned)p.OC * 4u;
+        col4 = col_ok ? (unsigned)col * 4u : 0x40000000u;
+        bias_v = 0.f;
+        if (p.bias) bias_v = p.bias[col_ok ? col : 0];
+    };
+    auto store_item = [&](auto half_c, int parity) {
+        constexpr bool HALF = decltype(half_c)::value;
 #pragma unroll
         for (int mt = 0; mt < 2; mt++) {
             if (mt == 1 && HALF) break;
 #pragma unroll
             for (int rr = 0; rr < 4; rr++) {
-                const int tile = it.tile_first + 16 * mt + 4 * q + rr;
-                const bool ok = tile < it.tile_end && col_ok;
-                const int n = fdiv(tile, p.d_TRC), rem = tile - n * p.TRC;
-                const int ty = fdiv(rem, p.d_TC), tx = rem - ty * p.TC;
-                const int oh = 2 * ty, ow = 2 * tx;
-                const unsigned o = (unsigned)(((n * p.OH + oh) * p.OW + ow) * p.OC + col) * 4u;
-                const bool right = ok && ow + 1 < p.OW, below = ok && oh + 1 < p.OH;
-                const unsigned o00 = ok ? o : WS_OOR, o01 = right ? o + px4 : WS_OOR;
-                const unsigned o10 = below ? o + row4 : WS_OOR, o11 = (right && below) ? o + row4 + px4 : WS_OOR;
+                const uint4 o = *reinterpret_cast<const uint4 *>(otab + parity * 128 + (16 * mt + 4 * q + rr) * 4);
                 // Y = A^T m A, A^T = [[1,1,1,0],[0,1,-1,-1]], m[a][c] = acc[4a + c]
                 float s0[4], s1[4];
 #pragma unroll
@@ -184,10 +194,10 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
                 }
                 const float y00 = s0[0] + s0[1] + s0[2] + bias_v, y01 = s0[1] - s0[2] - s0[3] + bias_v;
                 const float y10 = s1[0] + s1[1] + s1[2] + bias_v, y11 = s1[1] - s1[2] - s1[3] + bias_v;
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y00), y_rsrc, o00, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y01), y_rsrc, o01, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y10), y_rsrc, o10, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y11), y_rsrc, o11, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y00), y_rsrc, o.x + col4, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y01), y_rsrc, o.y + col4, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y10), y_rsrc, o.z + col4, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, y11), y_rsrc, o.w + col4, 0, 0);
             }
         }
     };
@@ -195,21 +205,24 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
     // ---- start: V of step 0, the patch of step 1 on its way, the ring filled ------------------------------------------
     Item cur = item_of(0);
     int pk = 0, pc = 0;   // patch cursor: item and chunk of the patch in d
-    auto advance_patch = [&]() {   // moves the cursor one step on and requests that step's patch
+    auto advance_patch_cursor = [&]() {   // one step on; a new item brings new pixel offsets
         pc++;
         if (pc == nchunks) {
             pc = 0;
             pk++;
-            if (pk < nitems) patch_offsets(item_of(pk));
+            if (pk < nitems) patch_offsets(item_of(pk));   // beyond the last step: patches nobody multiplies, valid addresses
         }
-        load_patch(pc * 16);   // beyond the last step: a patch nobody multiplies (its addresses are valid)
     };
     patch_offsets(cur);
     load_patch(0);
     transform_columns();
 #pragma unroll
-    for (int i = 0; i < 4; i++) transform_row_store(smem + xt * 16 + xq, i);
-    advance_patch();
+    for (int i = 0; i < 4; i++) {
+        transform_half_row_store(smem + xt * 16 + xq, i, 0);
+        transform_half_row_store(smem + xt * 16 + xq, i, 1);
+    }
+    advance_patch_cursor();
+    load_patch(pc * 16);
     {
         const unsigned u0 = (unsigned)cur.oc0 * 4u;
 #pragma unroll
@@ -219,16 +232,26 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
 
     // ---- one step: 16 xi x (2 LDS fragments, 4 filter elements, 8 MFMAs); in their shadow the next step's V ----------
     // Every xi is a scheduling region of its own (nothing crosses its borders), in program order: the LDS fragments of
-    // the next xi, the ring refill, 8 MFMAs, and in their shadow a slice of the next step's preparation. Left to
-    // itself the scheduler dissolves the ring (loads issued right before their use) and moves the patch loads to the
-    // end of the step and their transform to the start of the next one, with nothing in between to cover the latency.
-    auto chunk = [&](auto half_c, int buf, unsigned ucur, unsigned unext) {
+    // the next xi, the ring refill, 8 MFMAs, and a slice of the preparation of the steps to come. Left to itself the
+    // scheduler dissolves the ring (loads issued right before their use) and moves the patch loads to the end of the
+    // step and their transform to the start of the next one, with nothing in between to cover the latency. The slices
+    // are thin because the four wavefronts of a compute unit run in step and share its memory pipelines: 16 patch loads
+    // or 8 LDS writes per wavefront at one place keep them all waiting (measured: 930 and 570 cycles of a 6300-cycle
+    // step); two loads and one write per xi pass unnoticed.
+    //   xi 0      columns of B^T d B for the next step's patch (it arrived during the last step)
+    //   xi 1-8    half a row of the transform each: 2 of the 16 V positions written to the other LDS buffer
+    //   xi 2      the patch cursor moves on to the step after the next
+    //   xi 3-10   two of its 16 loads each, into the registers the finished rows have left
+    //   xi 12     first step of an item only: the item's output offsets into LDS
+    auto chunk = [&](auto half_c, auto first_c, int buf, unsigned ucur, unsigned unext, int k) {
         constexpr bool HALF = decltype(half_c)::value;
+        constexpr bool FIRST = decltype(first_c)::value;   // first step of an item: the accumulators start from zero
         const float *V = smem + buf * WS_VBUF + l16 * 16 + 4 * q;
         float *Vw = smem + (buf ^ 1) * WS_VBUF + xt * 16 + xq;
         floatx4 a0 = *reinterpret_cast<const floatx4 *>(V);
         floatx4 a1 = a0;
         if (!HALF) a1 = *reinterpret_cast<const floatx4 *>(V + 16 * 16);
+        const floatx4 zero = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int xi = 0; xi < 16; xi++) {
             __builtin_amdgcn_sched_barrier(0);
@@ -246,41 +269,51 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
             }
 #pragma unroll
             for (int s = 0; s < 4; s++) {
-                acc[xi][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[s], bb[s], acc[xi][0], 0, 0, 0);
-                if (!HALF) acc[xi][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[s], bb[s], acc[xi][1], 0, 0, 0);
+                acc[xi][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[s], bb[s], (FIRST && s == 0) ? zero : acc[xi][0], 0, 0, 0);
+                if (!HALF) acc[xi][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[s], bb[s], (FIRST && s == 0) ? zero : acc[xi][1], 0, 0, 0);
             }
-            if (xi == 3) transform_columns();                // consumes the patch of the next step
-            if (xi == 4 || xi == 5) {                        // writes that step's V
-                transform_row_store(Vw, 2 * (xi - 4));
-                transform_row_store(Vw, 2 * (xi - 4) + 1);
+            if (xi == 0) transform_columns();
+            if (xi >= 1 && xi <= 8) transform_half_row_store(Vw, (xi - 1) >> 1, (xi - 1) & 1);
+            if (xi == 2) advance_patch_cursor();
+            if (xi >= 3 && xi <= 10) {
+                load_patch_element(2 * (xi - 3), pc * 16);
+                load_patch_element(2 * (xi - 3) + 1, pc * 16);
             }
-            if (xi == 6) advance_patch();                    // requests the patch of the step after it
+            if (FIRST && xi == 12) write_offset_table(cur, k & 1);
+            // order inside the region: each MFMA is followed by at most one memory instruction of each kind and a few
+            // vector ALU instructions, so that no run of them is longer than the MFMA in front of it
+#pragma unroll
+            for (int m = 0; m < 8; m++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // 1 load from memory
+                __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);   // 1 LDS instruction
+                __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // vector ALU
+            }
             a0 = a0n;
             a1 = a1n;
         }
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    // whole items first, then the half item if this workgroup has one: two copies of the step, one after the other
+    // whole items first, then the half item if this workgroup has one: two copies of the steps, one after the other
     int buf = 0;
     auto run_item = [&](auto half_c, int k) {
         const bool has_next = k + 1 < nitems;
         Item nxt = cur;
         if (has_next) nxt = item_of(k + 1);
+        item_column(cur);
         const unsigned u_item = (unsigned)cur.oc0 * 4u;
-        for (int c = 0; c < nchunks; c++) {
+        const unsigned u_after = has_next ? (unsigned)nxt.oc0 * 4u : 0u;   // where the ring goes on after this item
+        chunk(half_c, std::true_type{}, buf, u_item, nchunks > 1 ? u_item + chunk_stride4 : u_after, k);
+        __syncthreads();
+        buf ^= 1;
+        for (int c = 1; c < nchunks; c++) {
             const unsigned ucur = u_item + c * chunk_stride4;
-            const unsigned unext = c + 1 < nchunks ? ucur + chunk_stride4 : (has_next ? (unsigned)nxt.oc0 * 4u : 0u);
-            chunk(half_c, buf, ucur, unext);
+            chunk(half_c, std::false_type{}, buf, ucur, c + 1 < nchunks ? ucur + chunk_stride4 : u_after, k);
             __syncthreads();
             buf ^= 1;
         }
-        store_item(half_c, cur);
-#pragma unroll
-        for (int x = 0; x < 16; x++) {
-            acc[x][0] = floatx4{0.f, 0.f, 0.f, 0.f};
-            acc[x][1] = floatx4{0.f, 0.f, 0.f, 0.f};
-        }
+        store_item(half_c, k & 1);
         cur = nxt;
     };
     const int nfull = b < p.halves ? nitems - 1 : nitems;
@@ -294,7 +327,7 @@ hipError_t launch_winograd_stream(hipStream_t stream, const float *X, const floa
     if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
     if (IC < 16 || IC % 16 != 0 || OC < 1 || N < 1 || OH < 1 || OW < 1) return hipErrorNotSupported;
     const long x_bytes = (long)N * IH * IW * IC * 4, y_bytes = (long)N * OH * OW * OC * 4, u_bytes = 16L * IC * OC * 4;
-    if (x_bytes >= (1L << 31) || y_bytes >= (1L << 31) || u_bytes >= (1L << 31)) return hipErrorNotSupported;
+    if (x_bytes >= (1L << 31) || y_bytes > (1L << 30) || u_bytes >= (1L << 31)) return hipErrorNotSupported;
     const int cus = device_cu_count();
     if (cus < 1) return hipErrorNotSupported;
 
@@ -321,7 +354,7 @@ hipError_t launch_winograd_stream(hipStream_t stream, const float *X, const floa
     else a.extra = left;
 
     constexpr auto kern = winograd_stream_kernel;
-    const size_t lds = (size_t)2 * WS_VBUF * sizeof(float);
+    const size_t lds = (size_t)2 * WS_VBUF * sizeof(float) + 2 * WS_TILES * 4 * sizeof(unsigned);   // V[2], otab[2]
     if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, a);
     return hipGetLastError();
