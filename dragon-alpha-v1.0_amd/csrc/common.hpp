@@ -150,6 +150,9 @@ hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, 
 hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
                                    int GK, int IC, int OC, int GK_slice, int GZ, float *dB = nullptr, float *dB_buf = nullptr);
 
+// Which of the two layouts of the transformed filter a layer uses (a function of IC alone: the transform does not know
+// the rest of the layer): grouped U[16][IC/4][OC][4] for the persistent kernel, else U[16][IC][OC].
+inline bool winograd_grouped_filter(int IC) { return IC >= 16 && IC % 16 == 0; }
 hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC);
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias = nullptr);

@@ -35,12 +35,26 @@ struct WinoArgs {
 constexpr int WG_TILES = 32;
 constexpr int WG_VBUF = 16 * WG_TILES * 16;   // floats per V buffer: [xi][tile][16 channels]
 
-// U[xi = 4a + b][ic][oc] = (G g G^T)[a][b],  G = [[1,0,0],[.5,.5,.5],[.5,-.5,.5],[0,0,1]],  g = W[oc][.][.][ic]
-__global__ __launch_bounds__(256) void winograd_filter_kernel(const float *__restrict__ W, float *__restrict__ U, int IC, int OC)
+// U[xi = 4a + b](ic, oc) = (G g G^T)[a][b],  G = [[1,0,0],[.5,.5,.5],[.5,-.5,.5],[0,0,1]],  g = W[oc][.][.][ic].
+// Two layouts, chosen by IC alone so that the transform and the kernel that reads it agree: U[xi][ic][oc] for the kernel
+// below, and for IC % 16 == 0 (winograd_stream.hip) U[xi][ic / 4][oc][ic % 4], where the four input channels of an
+// MFMA operand are one 128-bit element.
+__global__ __launch_bounds__(256) void winograd_filter_kernel(const float *__restrict__ W, float *__restrict__ U, int IC, int OC, int grouped)
 {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;   // over (ic, oc), oc fastest
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= IC * OC) return;
-    const int ic = idx / OC, oc = idx - ic * OC;
+    int ic, oc, pos, xi_stride = IC * OC, step;   // element (xi, ic, oc) at U[xi * xi_stride + pos]
+    if (grouped) {   // threads over (ic / 4, oc, ic % 4), ic % 4 fastest: consecutive threads write consecutive elements
+        const int g = idx / (4 * OC), r = idx - g * 4 * OC;
+        oc = r >> 2;
+        ic = 4 * g + (r & 3);
+        pos = idx;
+    } else {         // threads over (ic, oc), oc fastest
+        ic = idx / OC;
+        oc = idx - ic * OC;
+        pos = idx;
+    }
+    step = xi_stride;
     float g[3][3];
 #pragma unroll
     for (int i = 0; i < 3; i++)
@@ -57,10 +71,10 @@ __global__ __launch_bounds__(256) void winograd_filter_kernel(const float *__res
 #pragma unroll
     for (int a = 0; a < 4; a++) {
         const float u0 = t[a][0], u1 = 0.5f * (t[a][0] + t[a][1] + t[a][2]), u2 = 0.5f * (t[a][0] - t[a][1] + t[a][2]), u3 = t[a][2];
-        U[((size_t)(4 * a + 0) * IC + ic) * OC + oc] = u0;
-        U[((size_t)(4 * a + 1) * IC + ic) * OC + oc] = u1;
-        U[((size_t)(4 * a + 2) * IC + ic) * OC + oc] = u2;
-        U[((size_t)(4 * a + 3) * IC + ic) * OC + oc] = u3;
+        U[(size_t)(4 * a + 0) * step + pos] = u0;
+        U[(size_t)(4 * a + 1) * step + pos] = u1;
+        U[(size_t)(4 * a + 2) * step + pos] = u2;
+        U[(size_t)(4 * a + 3) * step + pos] = u3;
     }
 }
 
@@ -248,7 +262,7 @@ __global__ __launch_bounds__(256, 2) void winograd_f2x2_kernel(const WinoArgs p)
 hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC)
 {
     if (IC <= 0 || OC <= 0) return hipSuccess;
-    hipLaunchKernelGGL(winograd_filter_kernel, dim3((IC * OC + 255) / 256), dim3(256), 0, s, W, U, IC, OC);
+    hipLaunchKernelGGL(winograd_filter_kernel, dim3((IC * OC + 255) / 256), dim3(256), 0, s, W, U, IC, OC, winograd_grouped_filter(IC) ? 1 : 0);
     return hipGetLastError();
 }
 
@@ -256,8 +270,8 @@ hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, f
                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias)
 {
     if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
-    if (const hipError_t e = launch_winograd_stream(stream, X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, bias); e != hipErrorNotSupported)
-        return e;   // the persistent variant, where it applies
+    if (winograd_grouped_filter(IC))   // the persistent variant and its filter layout; no other kernel reads that layout
+        return launch_winograd_stream(stream, X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, bias);
     WinoArgs a{};
     a.X = X; a.U = U; a.Y = Y; a.bias = bias;
     a.N = N; a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC;

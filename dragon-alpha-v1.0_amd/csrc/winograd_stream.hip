@@ -1,6 +1,6 @@
 // Winograd F(2x2, 3x3) forward convolution as one uninterrupted MFMA stream per workgroup, gfx950, for input channel
 // counts that are multiples of 16. Same arithmetic as winograd.hip (input transform -> 16 MFMA GEMMs, one per transform
-// position xi -> output transform, v_mfma_f32_16x16x4_f32, the transformed filter U[16][IC][OC] fetched from L2 through
+// position xi -> output transform, v_mfma_f32_16x16x4_f32, the transformed filter U[16][IC/4][OC][4] fetched from L2 through
 // a register ring); what differs is what happens between two output blocks.
 //
 // An item is 32 consecutive tiles of the flattened (n, tile row, tile column) index (2x2 output pixels each) times 64
@@ -23,7 +23,7 @@ namespace alpha {
 
 struct WinoStreamArgs {
     const float *X;      // [N, IH, IW, IC]
-    const float *U;      // [16][IC][OC]
+    const float *U;      // [16][IC/4][OC][4]
     float *Y;            // [N, OH, OW, OC]
     const float *bias;   // NULL or [OC]
     int IH, IW, IC, OH, OW, OC, ph, pw;
@@ -133,16 +133,14 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
         *reinterpret_cast<float2 *>(Vw + (4 * i + 2 * h + 1) * WS_TILES * 16) = vb;
     };
 
-    // ---- transformed filter: lane (l16, q) needs U[xi][chunk*16 + 4q + s][oc0 + 16w + l16]; columns beyond OC read
+    // ---- transformed filter U[16][IC/4][OC][4]: lane (l16, q) needs channels chunk*16 + 4q .. + 3 of column
+    //      oc0 + 16w + l16, one 128-bit element (a ring refill is one load instead of four); columns beyond OC read
     //      something finite or the range check's zero and are never stored --------------------------------------------
     const __amdgpu_buffer_rsrc_t u_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.U), 0, p.u_bytes, 0x00020000);
-    unsigned u_lane[4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) u_lane[s] = (unsigned)((4 * q + s) * p.OC + 16 * w + l16) * 4u;
-    float bring[4][4];
-    auto load_b = [&](float (&bb)[4], unsigned block) {   // block: uniform byte offset of (xi, chunk, oc0)
-#pragma unroll
-        for (int s = 0; s < 4; s++) bb[s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(u_rsrc, u_lane[s], block, 0));
+    const unsigned u_lane = (unsigned)(q * p.OC + 16 * w + l16) * 16u;   // group q of the chunk's four groups of 4 channels
+    floatx4 bring[4];
+    auto load_b = [&](floatx4 &bb, unsigned block) {   // block: uniform byte offset of (xi, chunk, oc0)
+        bb = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(u_rsrc, u_lane, block, 0));
     };
 
     // ---- output: lane (l16, q) holds tiles 16mt + 4q + r (r = accumulator component) of channel oc0 + 16w + l16 ---------
@@ -224,7 +222,7 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
     advance_patch_cursor();
     load_patch(pc * 16);
     {
-        const unsigned u0 = (unsigned)cur.oc0 * 4u;
+        const unsigned u0 = (unsigned)cur.oc0 * 16u;
 #pragma unroll
         for (int x = 0; x < 4; x++) load_b(bring[x], u0 + x * xi_stride4);
     }
@@ -260,9 +258,7 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
                 a0n = *reinterpret_cast<const floatx4 *>(V + (xi + 1) * WS_TILES * 16);
                 if (!HALF) a1n = *reinterpret_cast<const floatx4 *>(V + (xi + 1) * WS_TILES * 16 + 16 * 16);
             }
-            float bb[4];
-#pragma unroll
-            for (int s = 0; s < 4; s++) bb[s] = bring[xi & 3][s];
+            const floatx4 bb = bring[xi & 3];
             {   // refill this ring slot with the fragment needed four positions later (possibly in the next step)
                 const int nx = xi + 4;
                 load_b(bring[xi & 3], nx < 16 ? ucur + nx * xi_stride4 : unext + (nx - 16) * xi_stride4);
@@ -302,8 +298,8 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
         Item nxt = cur;
         if (has_next) nxt = item_of(k + 1);
         item_column(cur);
-        const unsigned u_item = (unsigned)cur.oc0 * 4u;
-        const unsigned u_after = has_next ? (unsigned)nxt.oc0 * 4u : 0u;   // where the ring goes on after this item
+        const unsigned u_item = (unsigned)cur.oc0 * 16u;
+        const unsigned u_after = has_next ? (unsigned)nxt.oc0 * 16u : 0u;   // where the ring goes on after this item
         chunk(half_c, std::true_type{}, buf, u_item, nchunks > 1 ? u_item + chunk_stride4 : u_after, k);
         __syncthreads();
         buf ^= 1;
