@@ -257,7 +257,8 @@ int alpha_dconv3D_deltaW_GemmSK_W1(const int64_t *streams, int length, int GridZ
 /* Winograd F(2x2,3x3) forward for FH = FW = 3, stride 1. No counterpart among the reference's
  * JNI methods. U is scratch of alpha_winograd_filter_size(IC, OC) floats supplied by the caller
  * (the transformed filter, 16 * IC * OC); alpha_winograd_filter_transform fills it from
- * W[OC,3,3,IC]; alpha_conv3D_winograd then consumes it. */
+ * W[OC,3,3,IC]; alpha_conv3D_winograd then consumes it. U is opaque: its element order depends on IC
+ * (the two calls agree on it) and only these two entries may interpret it. */
 long alpha_winograd_filter_size(int IC, int OC);
 int alpha_winograd_filter_transform(int64_t stream, const float *W, float *U, int IC, int OC);
 int alpha_conv3D_winograd(const int64_t *streams, int length,
