@@ -97,25 +97,36 @@ hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, 
 // deltaW += sum_{p < part} deltaW_buf[p], summed in the fixed order p = 0, 1, ... with fp32 Kahan
 // compensation (the reference's recurrence, operation for operation). The adds of one element form a serial
 // chain, but the loads do not depend on it: one thread owns ONE element (so even a 16 K-element filter gives
-// hundreds of wavefronts) and fetches 16 partials at a time before running them through the chain.
+// hundreds of wavefronts) and fetches 24 partials at a time, the next batch while the current one runs through the chain.
 __global__ __launch_bounds__(256) void buf_summary_kernel(const float *__restrict__ buf, float *__restrict__ dW,
                                                           int part, int sizeW)
 {
-    constexpr int U = 16;
+    constexpr int U = 24;   // partials per batch; two batches in flight (the next one is requested before this one is added)
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= sizeW) return;
     float dw = dW[i], c = 0.f;
     int p = 0;
-    for (; p + U <= part; p += U) {
-        float b[U];
+    float b[U], nb[U];
+    if (U <= part) {
 #pragma unroll
-        for (int u = 0; u < U; u++) b[u] = buf[(size_t)(p + u) * sizeW + i];
+        for (int u = 0; u < U; u++) b[u] = buf[(size_t)u * sizeW + i];
+    }
+    for (; p + U <= part; p += U) {
+        const bool more = p + 2 * U <= part;
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < U; u++) nb[u] = buf[(size_t)(p + U + u) * sizeW + i];
+        }
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const float y = b[u] - c;
             const float s = dw + y;
             c = (s - dw) - y;
             dw = s;
+        }
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < U; u++) b[u] = nb[u];
         }
     }
     for (; p < part; p++) {
