@@ -401,6 +401,8 @@ BIAS_SHAPES = [
     (4, 16, 16, 4, 64, 7, 2, 3),       # stem kernel
     (4, 13, 11, 32, 48, 3, 2, 1),      # generic kernel (strided)
     (4, 6, 5, 12, 20, 3, 1, 1),        # generic kernel, ragged channels
+    (25, 40, 40, 16, 72, 3, 1, 1),     # persistent Winograd kernel: 626 items in two blocks of output channels (the second
+                                       # with 8 of 64), whole and half items
 ]
 
 
