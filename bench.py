@@ -167,6 +167,16 @@ class Workload:
         self.engine.dconv3D_deltaW(self.dW.data_ptr(), F, F, self.X.data_ptr(), IH, IW, self.dY.data_ptr(), self.OH, self.OW,
                                    N, IC, OC, s, s, p, p)
 
+    def dx_wino_conv(self):
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.pkg.Cuda_dconv3D_deltaX.dconv3D_deltaX_winograd(self.streams, 1, self.dY.data_ptr(), self.OH, self.OW, self.U.data_ptr(),
+                                                             self.dX.data_ptr(), IH, IW, N, IC, OC, p, p)
+
+    def dx_wino(self):
+        self.engine.config.deltaX_winograd = 1
+        self.dx_op()
+        self.engine.config.deltaX_winograd = 0
+
     def dx_op(self):
         N, IH, IW, IC, OC, F, s, p = self.dims
         self.engine.dconv3D_deltaX(self.dX.data_ptr(), IH, IW, self.dY.data_ptr(), self.OH, self.OW, self.W.data_ptr(), F, F,
@@ -238,14 +248,18 @@ def load_traffic(layer, op):
 
 def measure(pkg, torch, layer, op, steps, warmup):
     wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer), fill_units=(op == "dw_fill"))
-    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd_cached, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino}[op]
+    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd_cached, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino,
+            "dx_wino": wl.dx_wino}[op]
     kernel = {"fwd": wl.fwd_conv, "fwd_cached": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
-              "wino": wl.wino_conv}[op]
+              "wino": wl.wino_conv, "dx_wino": wl.dx_wino_conv}[op]
     if op in ("fwd", "fwd_bias", "fwd_cached"):
         wl.fwd_remode()
     if op == "wino":
         N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
         pkg.Cuda_conv3D.winograd_filter_transform(wl.stream, wl.W.data_ptr(), wl.U.data_ptr(), IC_, OC_)
+    if op == "dx_wino":
+        N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
+        pkg.Cuda_dconv3D_deltaX.winograd_filter_transform_deltaX(wl.stream, wl.W.data_ptr(), wl.U.data_ptr(), IC_, OC_)
     def step_and_recycle():
         step()
     wall_ms, ev_ms = time_loop(torch, step_and_recycle, steps, warmup)
@@ -275,7 +289,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
-    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "dx", "dw", "dw_fill", "wino"],
+    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "dx", "dw", "dw_fill", "wino", "dx_wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="also measure every layer/op of BASELINE.json's configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -336,6 +350,8 @@ def main():
             ops = list(LAYERS[layer][9])
             if "fwd" in ops and LAYERS[layer][5] == 3 and LAYERS[layer][6] == 1 and LAYERS[layer][3] >= 16:
                 ops.append("wino")
+            if "dx" in ops and LAYERS[layer][5] == 3 and LAYERS[layer][6] == 1:
+                ops.append("dx_wino")
             if "dw" in ops:
                 ops.append("dw_fill")
             if layer == "c3a":

@@ -153,7 +153,9 @@ hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const flo
 // Which of the two layouts of the transformed filter a layer uses (a function of IC alone: the transform does not know
 // the rest of the layer): grouped U[16][IC/4][OC][4] for the persistent kernel, else U[16][IC][OC].
 inline bool winograd_grouped_filter(int IC) { return IC >= 16 && IC % 16 == 0; }
-hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC);
+// backward: the filter of backward-data as a forward convolution of deltaY (OC reduced, IC produced, taps rotated);
+// launch_winograd(deltaY, U, deltaX, N, OH, OW, OC, IH, IW, IC, 2 - ph, 2 - pw) then computes deltaX.
+hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC, bool backward = false);
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias = nullptr);
 // The same as one MFMA stream per persistent workgroup (winograd_stream.hip), for IC % 16 == 0; returns

@@ -462,6 +462,29 @@ int alpha_conv3D_winograd(const int64_t *streams, int length, const float *X, in
     return hip_status(e, __func__);
 }
 
+// Backward-data of a 3x3 stride-1 layer is a forward convolution of deltaY (OC channels in, IC out, padding 2 - p, taps
+// rotated): the same Winograd kernels compute it from a filter transformed accordingly.
+int alpha_winograd_filter_transform_deltaX(int64_t stream, const float *W, float *U, int IC, int OC)
+{
+    CHECK_PTR(W);
+    CHECK_PTR(U);
+    if (IC < 4 || OC < 4 || (IC & 3) || (OC & 3)) return fail(ALPHA_CONV_EINVAL, "%s: IC and OC must be multiples of 4", __func__);
+    return hip_status(launch_winograd_filter(reinterpret_cast<hipStream_t>((intptr_t)stream), W, U, IC, OC, true), __func__);
+}
+int alpha_dconv3D_deltaX_winograd(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *U,
+                                  float *deltaX, int IH, int IW, int N, int IC, int OC, int ph, int pw)
+{
+    CHECK_STREAMS();
+    CHECK_PTR(deltaY);
+    CHECK_PTR(U);
+    CHECK_PTR(deltaX);
+    if (int e = check_dims(__func__, N, IC, OC, IH, IW, OH, OW, 3, 3, 1, 1, ph, pw)) return e;
+    if (ph > 2 || pw > 2) return fail(ALPHA_CONV_EINVAL, "%s: padding must be at most 2", __func__);
+    hipError_t e = launch_winograd(stream0(streams), deltaY, U, deltaX, N, OH, OW, OC, IH, IW, IC, 2 - ph, 2 - pw);
+    if (e == hipErrorNotSupported) return fail(ALPHA_CONV_EINVAL, "%s: needs OH = IH + 2*ph - 2, OW = IW + 2*pw - 2", __func__);
+    return hip_status(e, __func__);
+}
+
 // ---- backward-filter with the bias gradient (column sums of deltaY) from the same pass over deltaY -------------------
 int alpha_dconv3D_deltaW_GemmSK_deltaB(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
                                        const float *deltaY, int OH, int OW, float *deltaW, float *deltaW_buf,

@@ -64,6 +64,7 @@ void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
     c->deltaX_s1_V2_Q = 1.1f;
     c->deltaX_ks_V2_Q = 1.1f;
     c->conv3D_winograd = 0;
+    c->deltaX_winograd = 0;
     c->deltaW_SK_fillUnits = 0;
     c->cache_filter_transforms = 0;
 }
@@ -171,6 +172,12 @@ void alpha_plan_deltaX(const alpha_engine_config *c, int IH, int IW, int OH, int
         out->streams = stream_count(IC, N * IH * IW, 10);
         return;
     }
+    if (c->deltaX_winograd && sh == 1 && sw == 1 && FH == 3 && FW == 3 && OH - IH + 2 <= 4 && OW - IW + 2 <= 4) {   // padding <= 2
+        out->entry = ALPHA_E_dconv3D_deltaX_winograd;
+        out->streams = 1;
+        out->scratch_floats = 16L * IC * OC;
+        return;
+    }
     if (sh == 1 && sw == 1) {
         // Cuda_dconv3D_deltaX.s1_paddingScaleUp
         const double Q = 1.0 * ((IH - 1 + FH) * (IW - 1 + FW)) / (OH * OW);
@@ -220,7 +227,7 @@ struct alpha_engine {
     // Transformed filters kept between calls (cfg.cache_filter_transforms): key -> (bytes, block)
     struct FilterKey {
         const void *W;
-        int kind, FH, FW, IC, OC, sh, sw;   // kind 0: CW of kernel_remode, 1: Winograd U, 2: kernel-split CW (ks_remodev2)
+        int kind, FH, FW, IC, OC, sh, sw;   // kind 0: CW of kernel_remode, 1: Winograd U, 2: kernel-split CW (ks_remodev2), 3: Winograd U of backward-data
         bool operator<(const FilterKey &o) const
         {
             return std::tie(W, kind, FH, FW, IC, OC, sh, sw) < std::tie(o.W, o.kind, o.FH, o.FW, o.IC, o.OC, o.sh, o.sw);
@@ -548,6 +555,14 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
     case ALPHA_E_dconv3D_deltaX_crossAdd:
         rc = alpha_dconv3D_deltaX_crossAdd(streams, p.streams, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
         break;
+    case ALPHA_E_dconv3D_deltaX_winograd: {
+        bool fresh;
+        float *U = filter_block(e, 3, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
+        if (!U) return fail(e, -1, "dconv3D_deltaX");
+        if (fresh && (rc = alpha_winograd_filter_transform_deltaX(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform_deltaX");
+        rc = alpha_dconv3D_deltaX_winograd(streams, p.streams, deltaY, OH, OW, U, deltaX, IH, IW, N, IC, OC, ph, pw);
+        break;
+    }
     case ALPHA_E_dconv3D_deltaX_W1:
         rc = alpha_dconv3D_deltaX_W1(streams, p.streams, deltaY, W, deltaX, IH, IW, N, IC, OC);
         break;

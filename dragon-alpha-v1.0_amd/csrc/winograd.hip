@@ -39,7 +39,12 @@ constexpr int WG_VBUF = 16 * WG_TILES * 16;   // floats per V buffer: [xi][tile]
 // Two layouts, chosen by IC alone so that the transform and the kernel that reads it agree: U[xi][ic][oc] for the kernel
 // below, and for IC % 16 == 0 (winograd_stream.hip) U[xi][ic / 4][oc][ic % 4], where the four input channels of an
 // MFMA operand are one 128-bit element.
-__global__ __launch_bounds__(256) void winograd_filter_kernel(const float *__restrict__ W, float *__restrict__ U, int IC, int OC, int grouped)
+// With `backward` the transform is that of the filter of backward-data seen as a forward convolution of deltaY: reduced
+// channels = the layer's OC, produced channels = the layer's IC, taps rotated by 180 degrees,
+// g'[i][j](reduced oc, produced ic) = W[oc][2-i][2-j][ic]. IC and OC below are then the reduced and the produced count
+// (the layer's OC and IC), LD the layer's IC (the stride of W's taps).
+__global__ __launch_bounds__(256) void winograd_filter_kernel(const float *__restrict__ W, float *__restrict__ U, int IC, int OC, int grouped,
+                                                              int backward)
 {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= IC * OC) return;
@@ -59,7 +64,8 @@ __global__ __launch_bounds__(256) void winograd_filter_kernel(const float *__res
 #pragma unroll
     for (int i = 0; i < 3; i++)
 #pragma unroll
-        for (int j = 0; j < 3; j++) g[i][j] = W[((size_t)(oc * 3 + i) * 3 + j) * IC + ic];
+        for (int j = 0; j < 3; j++)
+            g[i][j] = backward ? W[((size_t)(ic * 3 + (2 - i)) * 3 + (2 - j)) * OC + oc] : W[((size_t)(oc * 3 + i) * 3 + j) * IC + ic];
     float t[4][3];
 #pragma unroll
     for (int j = 0; j < 3; j++) {
@@ -259,10 +265,12 @@ __global__ __launch_bounds__(256, 2) void winograd_f2x2_kernel(const WinoArgs p)
     }
 }
 
-hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC)
+hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC, bool backward)
 {
     if (IC <= 0 || OC <= 0) return hipSuccess;
-    hipLaunchKernelGGL(winograd_filter_kernel, dim3((IC * OC + 255) / 256), dim3(256), 0, s, W, U, IC, OC, winograd_grouped_filter(IC) ? 1 : 0);
+    const int red = backward ? OC : IC, prod = backward ? IC : OC;   // reduced and produced channels of the convolution that reads U
+    hipLaunchKernelGGL(winograd_filter_kernel, dim3((IC * OC + 255) / 256), dim3(256), 0, s, W, U, red, prod,
+                       winograd_grouped_filter(red) ? 1 : 0, backward ? 1 : 0);
     return hipGetLastError();
 }
 

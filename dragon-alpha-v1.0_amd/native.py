@@ -54,6 +54,8 @@ _SIGS = {
     "alpha_dconv3D_deltaW_GemmSK_W1": "siipiipppiii",
     "alpha_winograd_filter_transform": "lppii",
     "alpha_conv3D_winograd": "sipiippiiiiiii",
+    "alpha_winograd_filter_transform_deltaX": "lppii",
+    "alpha_dconv3D_deltaX_winograd": "sipiippiiiiiii",
     "alpha_dconv3D_deltaW_GemmSK_deltaB": "siipiipiippppiiiiiiiii",
     "alpha_conv3D_biased": "sipiipiippiiiiiiiii",
     "alpha_conv3D_GemmR_biased": "sipiippiippiiiiiiiii",
@@ -232,6 +234,15 @@ class Cuda_dconv3D_deltaX:
     @staticmethod
     def dconv3D_deltaX_s1(streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):
         _call("alpha_dconv3D_deltaX_s1", streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def winograd_filter_transform_deltaX(stream, W, U, IC, OC):
+        """This build's Winograd path for backward-data (no reference counterpart): U as for the forward transform."""
+        _call("alpha_winograd_filter_transform_deltaX", stream, W, U, IC, OC)
+
+    @staticmethod
+    def dconv3D_deltaX_winograd(streamArray, length, deltaY, OH, OW, U, deltaX, IH, IW, N, IC, OC, ph, pw):
+        _call("alpha_dconv3D_deltaX_winograd", streamArray, length, deltaY, OH, OW, U, deltaX, IH, IW, N, IC, OC, ph, pw)
 
     @staticmethod
     def dconv3D_deltaX_s1_texture(streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):

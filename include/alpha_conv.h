@@ -267,6 +267,17 @@ int alpha_conv3D_winograd(const int64_t *streams, int length,
                           float *Y, int OH, int OW,
                           int N, int IC, int OC, int ph, int pw);
 
+/* The same algorithm for backward-data of a 3x3 stride-1 layer (deltaX = forward convolution of deltaY with the
+ * rotated filter, OC channels in, IC out, padding 2 - p). No counterpart in the reference (its backward-data natives,
+ * Cuda_dconv3D_deltaX.java:311-478, take W and no scratch); a caller that wants it supplies U
+ * (alpha_winograd_filter_size(IC, OC) floats) like CW of the kernel-split entries. ph, pw <= 2. */
+int alpha_winograd_filter_transform_deltaX(int64_t stream, const float *W, float *U, int IC, int OC);
+int alpha_dconv3D_deltaX_winograd(const int64_t *streams, int length,
+                                  const float *deltaY, int OH, int OW,
+                                  const float *U,
+                                  float *deltaX, int IH, int IW,
+                                  int N, int IC, int OC, int ph, int pw);
+
 /* ---- forward with the bias added in the kernel's epilogue --------------------------------------
  * The reference has no native for this: its engine method conv3D_biased (CudaFloat32EngineBase.java:1478-1560,
  * EngineBase.java:178-185) runs the conv3D entry and then Cuda_function.linear_dual2D_row(Y, Bias, ...) =

@@ -39,6 +39,8 @@ typedef struct alpha_engine_config {
                                      keyed by the filter's address and geometry; the caller reports weight updates with
                                      alpha_engine_filter_changed(). Default 0: re-transform on every call like the reference
                                      (CudaFloat32EngineBase.java:1373-1380, 1879-1889) */
+    int deltaX_winograd;          /* this build only: 1 = backward-data of 3x3 stride-1 layers (padding <= 2, more than 8 input
+                                     channels) through Winograd F(2x2,3x3); default 0 */
 } alpha_engine_config;
 
 /* Native entry chosen by a plan; names are the Java native method names. */
@@ -51,7 +53,8 @@ enum alpha_entry {
     ALPHA_E_dconv3D_deltaX_crossAdd,
     ALPHA_E_dconv3D_deltaW, ALPHA_E_dconv3D_deltaW_W1, ALPHA_E_dconv3D_deltaW_GemmSK, ALPHA_E_dconv3D_deltaW_GemmV2SK,
     ALPHA_E_dconv3D_deltaW_GemmSK_W1,
-    ALPHA_E_conv3D_winograd   /* this build's additional forward algorithm; never chosen unless conv3D_winograd is set */
+    ALPHA_E_conv3D_winograd,  /* this build's additional forward algorithm; never chosen unless conv3D_winograd is set */
+    ALPHA_E_dconv3D_deltaX_winograd   /* the same for backward-data; never chosen unless deltaX_winograd is set */
 };
 
 typedef struct alpha_conv_plan {

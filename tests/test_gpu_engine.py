@@ -70,6 +70,31 @@ def test_engine_runs_the_entry_java_would_pick(dev, eng, case):
     check(dev.get(dw), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "engine deltaW %s" % (case,))
 
 
+def test_engine_deltaX_winograd_flag(dev, eng):
+    """deltaX_winograd = 1 sends 3x3 stride-1 backward-data through the Winograd entry (scratch from the engine's pool);
+    off, the plan is the reference's."""
+    N, IH, IC, OC = 8, 14, 64, 32
+    dY, W = normal((N, IH, IH, OC), 6211), he_normal(OC, 3, 3, IC, 6212)
+    want = O.deltaX_f64(dY, W, IH, IH, 1, 1, 1, 1)
+    dy, w = dev.put(dY), dev.put(W)
+    for wino in (0, 1):
+        eng.config.deltaX_winograd = wino
+        try:
+            dx = dev.empty(N, IH, IH, IC, fill=float("nan"))
+            p = eng.dconv3D_deltaX(dx.data_ptr(), IH, IH, dy.data_ptr(), IH, IH, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1)
+            eng.sync()
+        finally:
+            eng.config.deltaX_winograd = 0
+        assert p.entry_name == ("dconv3D_deltaX_winograd" if wino else "dconv3D_deltaX_s1_texture")
+        check(dev.get(dx), want, "engine deltaX (winograd %d)" % wino)
+    # a strided layer keeps the reference's plan with the flag set
+    eng.config.deltaX_winograd = 1
+    try:
+        assert pkg.engine.plan_deltaX(eng.config, 14, 14, 7, 7, 3, 3, N, IC, OC, 2, 2).entry_name != "dconv3D_deltaX_winograd"
+    finally:
+        eng.config.deltaX_winograd = 0
+
+
 def test_engine_conv3D_biased(dev, eng):
     N, IH, IC, OC = 8, 14, 64, 64
     X, W, B = normal((N, IH, IH, IC), 6201), he_normal(OC, 3, 3, IC, 6202), normal((OC,), 6203)

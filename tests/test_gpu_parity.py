@@ -231,6 +231,21 @@ def test_forward_winograd_f2x2_vs_direct_oracle(dev, shape):
     check(dev.get(y), O.conv3D_f64(X, W, 1, 1, ph, pw), "winograd %s" % (shape,))
 
 
+@pytest.mark.parametrize("shape", WINO_SHAPES)
+def test_deltaX_winograd_vs_oracle(dev, shape):
+    """Backward-data of a 3x3 stride-1 layer as a Winograd convolution of deltaY (rotated filter, padding 2 - p);
+    same bar as the direct kernels. The table's layers read as (N, IH, IW, IC, OC) of the layer whose deltaX is wanted."""
+    N, IH, IW, IC, OC, ph, pw = shape
+    OH, OW = out_dim(IH, IW, 3, 3, 1, 1, ph, pw)
+    dY, W = normal((N, OH, OW, OC), 1211), he_normal(OC, 3, 3, IC, 1212)
+    dy, w = dev.put(dY), dev.put(W)
+    U = dev.empty(C3.winograd_filter_size(IC, OC), fill=float("nan"))
+    dXo = dev.guarded(N, IH, IW, IC)
+    DX.winograd_filter_transform_deltaX(dev.stream, w.data_ptr(), U.data_ptr(), IC, OC)
+    DX.dconv3D_deltaX_winograd(dev.streams, 1, dy.data_ptr(), OH, OW, U.data_ptr(), dXo.data_ptr(), IH, IW, N, IC, OC, ph, pw)
+    check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw), "winograd dX %s" % (shape,))
+
+
 def test_winograd_filter_transform_matches_G_g_Gt(dev):
     IC, OC = 8, 12
     W = he_normal(OC, 3, 3, IC, 1203)
