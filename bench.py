@@ -66,7 +66,7 @@ def algorithmic_bytes(layer):
 class Workload:
     """Device tensors of one layer plus closures that enqueue each operator the way the Java engine does."""
 
-    def __init__(self, pkg, torch, layer, seed, fill_units=False):
+    def __init__(self, pkg, torch, layer, seed, fill_units=False, dw_winograd=False):
         self.pkg, self.torch, self.layer = pkg, torch, layer
         N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[layer]
         self.dims = (N, IH, IW, IC, OC, F, s, p)
@@ -93,6 +93,9 @@ class Workload:
             # this build's option: raise the split-K factor until the launch fills the device (the reference's GridZ
             # is sized for at most 128 SMs)
             self.engine.config.deltaW_SK_fillUnits = pkg.device_info()[0]
+        if dw_winograd:
+            # this build's Winograd backward-filter, its split-K factor sized for the device's compute units
+            self.engine.config.deltaW_winograd = pkg.device_info()[0]
         # split-K factor for the kernel-only timing: what the host layer would pass (CudaFloat32EngineBase.java:1707-1715)
         self.GridZ = max(1, pkg.engine.plan_deltaW(self.engine.config, IH, IW, OH, OW, F, F, N, IC, OC, s, s).GridZ)
         self.buf = torch.empty(max(1, self.GridZ - 1) * self.dW.numel(), device=dev)
@@ -166,6 +169,12 @@ class Workload:
         N, IH, IW, IC, OC, F, s, p = self.dims
         self.engine.dconv3D_deltaW(self.dW.data_ptr(), F, F, self.X.data_ptr(), IH, IW, self.dY.data_ptr(), self.OH, self.OW,
                                    N, IC, OC, s, s, p, p)
+
+    def dw_wino_gemm(self):
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.pkg.Cuda_dconv3D_deltaW.dconv3D_deltaW_GemmSK_winograd(self.streams, 1, self.GridZ, self.X.data_ptr(), IH, IW,
+                                                                    self.dY.data_ptr(), self.OH, self.OW, self.dW.data_ptr(),
+                                                                    self.buf.data_ptr(), N, IC, OC, p, p)
 
     def dx_wino_conv(self):
         N, IH, IW, IC, OC, F, s, p = self.dims
@@ -247,11 +256,11 @@ def load_traffic(layer, op):
 
 
 def measure(pkg, torch, layer, op, steps, warmup):
-    wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer), fill_units=(op == "dw_fill"))
+    wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer), fill_units=(op == "dw_fill"), dw_winograd=(op == "dw_wino"))
     step = {"fwd": wl.fwd, "fwd_cached": wl.fwd_cached, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino,
-            "dx_wino": wl.dx_wino}[op]
+            "dx_wino": wl.dx_wino, "dw_wino": wl.dw}[op]
     kernel = {"fwd": wl.fwd_conv, "fwd_cached": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
-              "wino": wl.wino_conv, "dx_wino": wl.dx_wino_conv}[op]
+              "wino": wl.wino_conv, "dx_wino": wl.dx_wino_conv, "dw_wino": wl.dw_wino_gemm}[op]
     if op in ("fwd", "fwd_bias", "fwd_cached"):
         wl.fwd_remode()
     if op == "wino":
@@ -289,7 +298,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
-    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "dx", "dw", "dw_fill", "wino", "dx_wino"],
+    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "dx", "dw", "dw_fill", "wino", "dx_wino", "dw_wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="also measure every layer/op of BASELINE.json's configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -354,6 +363,8 @@ def main():
                 ops.append("dx_wino")
             if "dw" in ops:
                 ops.append("dw_fill")
+            if "dw" in ops and LAYERS[layer][5] == 3 and LAYERS[layer][6] == 1:
+                ops.append("dw_wino")
             if layer == "c3a":
                 ops += ["fwd_bias", "fwd_cached"]
             for o in ops:

@@ -163,6 +163,11 @@ hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, f
 hipError_t launch_winograd_stream(hipStream_t stream, const float *X, const float *U, float *Y,
                                   int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias = nullptr);
 
+// Backward-filter of 3x3 stride-1 layers by Winograd F(3x3,2x2) (winograd_dw.hip); slice z (a range of 2x2 output tiles)
+// -> deltaW or deltaW_buf[z-1]. Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
+hipError_t launch_deltaW_winograd(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
+                                  int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, int GZ);
+
 // Re-layout / reduction helpers.
 hipError_t launch_kernel_remode(hipStream_t s, const float *W, float *CW, int FH, int FW, int OC, int IC);
 hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, int FW, float *CW,

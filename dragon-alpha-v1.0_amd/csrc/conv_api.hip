@@ -485,6 +485,24 @@ int alpha_dconv3D_deltaX_winograd(const int64_t *streams, int length, const floa
     return hip_status(e, __func__);
 }
 
+// Backward-filter of a 3x3 stride-1 layer by Winograd F(3x3,2x2): the split-K contract of dconv3D_deltaW_GemmSK (slice z ->
+// deltaW or deltaW_buf[z-1], buf_summary finishes), the slices being ranges of 2x2 output tiles.
+int alpha_dconv3D_deltaW_GemmSK_winograd(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
+                                         const float *deltaY, int OH, int OW, float *deltaW, float *deltaW_buf,
+                                         int N, int IC, int OC, int ph, int pw)
+{
+    CHECK_STREAMS();
+    CHECK_PTR(X);
+    CHECK_PTR(deltaY);
+    CHECK_PTR(deltaW);
+    if (GridZ < 1) return fail(ALPHA_CONV_EINVAL, "%s: GridZ must be >= 1", __func__);
+    if (GridZ > 1 && (!deltaW_buf || !aligned16(deltaW_buf))) return fail(ALPHA_CONV_EINVAL, "%s: deltaW_buf is null or misaligned", __func__);
+    if (int e = check_dims(__func__, N, IC, OC, IH, IW, OH, OW, 3, 3, 1, 1, ph, pw)) return e;
+    hipError_t e = launch_deltaW_winograd(stream0(streams), X, deltaY, deltaW, deltaW_buf, N, IH, IW, IC, OH, OW, OC, ph, pw, GridZ);
+    if (e == hipErrorNotSupported) return fail(ALPHA_CONV_EINVAL, "%s: needs a 3x3 stride-1 layer with tensors below 2 GB", __func__);
+    return hip_status(e, __func__);
+}
+
 // ---- backward-filter with the bias gradient (column sums of deltaY) from the same pass over deltaY -------------------
 int alpha_dconv3D_deltaW_GemmSK_deltaB(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
                                        const float *deltaY, int OH, int OW, float *deltaW, float *deltaW_buf,

@@ -65,6 +65,7 @@ void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
     c->deltaX_ks_V2_Q = 1.1f;
     c->conv3D_winograd = 0;
     c->deltaX_winograd = 0;
+    c->deltaW_winograd = 0;
     c->deltaW_SK_fillUnits = 0;
     c->cache_filter_transforms = 0;
 }
@@ -150,8 +151,24 @@ void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int
         if (want > GridZ2) want = GridZ2;
         if (want > GridZ) GridZ = want;
     }
+    const bool winograd = c->deltaW_winograd && FH == 3 && FW == 3 && sh == 1 && sw == 1;
+    if (winograd && c->deltaW_winograd > 1) {
+        // One workgroup of the Winograd kernel covers 32 input x 64 output channels of one slice of tiles and has a
+        // compute unit to itself: values above 1 are the number of compute units to fill (slices of at least 64 tiles).
+        const int tiles = ((IC + 31) / 32) * ((OC + 63) / 64);
+        int want = (c->deltaW_winograd + tiles - 1) / tiles;
+        const int most = N * ((OH + 1) / 2) * ((OW + 1) / 2) / 64;
+        if (want > most) want = most;
+        if (want < 1) want = 1;
+        GridZ = want;
+    }
     out->GridZ = GridZ;
     out->scratch_floats = (long)OC * FH * FW * IC * (GridZ - 1);
+    if (winograd) {
+        out->entry = ALPHA_E_dconv3D_deltaW_GemmSK_winograd;
+        out->streams = 1;
+        return;
+    }
     if (FH == 1 && FW == 1 && sh == 1 && sw == 1) out->entry = ALPHA_E_dconv3D_deltaW_GemmSK_W1;   // W1 natives: stride 1 only
     else if (V2) out->entry = ALPHA_E_dconv3D_deltaW_GemmV2SK;
     else out->entry = ALPHA_E_dconv3D_deltaW_GemmSK;
@@ -476,6 +493,10 @@ int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, 
     int64_t streams[16];
     for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
     int rc = 0;
+    if (p.GridZ == 1 && p.entry == ALPHA_E_dconv3D_deltaW_GemmSK_winograd) {
+        rc = alpha_dconv3D_deltaW_GemmSK_winograd(streams, p.streams, 1, X, IH, IW, deltaY, OH, OW, deltaW, nullptr, N, IC, OC, ph, pw);
+        return rc ? fail(e, rc, "dconv3D_deltaW") : 0;
+    }
     if (p.GridZ == 1) {
         rc = p.entry == ALPHA_E_dconv3D_deltaW_W1
                  ? alpha_dconv3D_deltaW_W1(streams, p.streams, X, IH, IW, deltaY, deltaW, N, IC, OC)
@@ -485,6 +506,9 @@ int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, 
     float *buf = static_cast<float *>(take_block(e, (size_t)p.scratch_floats * sizeof(float)));
     if (!buf) return fail(e, -1, "dconv3D_deltaW");
     switch (p.entry) {
+    case ALPHA_E_dconv3D_deltaW_GemmSK_winograd:
+        rc = alpha_dconv3D_deltaW_GemmSK_winograd(streams, p.streams, p.GridZ, X, IH, IW, deltaY, OH, OW, deltaW, buf, N, IC, OC, ph, pw);
+        break;
     case ALPHA_E_dconv3D_deltaW_GemmSK_W1:
         rc = alpha_dconv3D_deltaW_GemmSK_W1(streams, p.streams, p.GridZ, X, IH, IW, deltaY, deltaW, buf, N, IC, OC);
         break;

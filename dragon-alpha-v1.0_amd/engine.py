@@ -14,7 +14,7 @@ ENTRY_NAMES = [None,
                "dconv3D_deltaX_ksIms2R", "dconv3D_deltaX_ksIms2R_texture", "dconv3D_deltaX_ksV2_Ims2R",
                "dconv3D_deltaX_crossAdd",
                "dconv3D_deltaW", "dconv3D_deltaW_W1", "dconv3D_deltaW_GemmSK", "dconv3D_deltaW_GemmV2SK",
-               "dconv3D_deltaW_GemmSK_W1", "conv3D_winograd", "dconv3D_deltaX_winograd"]
+               "dconv3D_deltaW_GemmSK_W1", "conv3D_winograd", "dconv3D_deltaX_winograd", "dconv3D_deltaW_GemmSK_winograd"]
 
 
 class Config(ctypes.Structure):
@@ -25,7 +25,7 @@ class Config(ctypes.Structure):
                 ("deltaX_s1_useTexture", ctypes.c_int), ("deltaX_ks_useTexture", ctypes.c_int),
                 ("deltaX_s1_V2_Q", ctypes.c_float), ("deltaX_ks_V2_Q", ctypes.c_float),
                 ("conv3D_winograd", ctypes.c_int), ("deltaW_SK_fillUnits", ctypes.c_int),
-                ("cache_filter_transforms", ctypes.c_int), ("deltaX_winograd", ctypes.c_int)]
+                ("cache_filter_transforms", ctypes.c_int), ("deltaX_winograd", ctypes.c_int), ("deltaW_winograd", ctypes.c_int)]
 
 
 class Plan(ctypes.Structure):

@@ -55,6 +55,7 @@ _SIGS = {
     "alpha_winograd_filter_transform": "lppii",
     "alpha_conv3D_winograd": "sipiippiiiiiii",
     "alpha_winograd_filter_transform_deltaX": "lppii",
+    "alpha_dconv3D_deltaW_GemmSK_winograd": "siipiipiippiiiii",
     "alpha_dconv3D_deltaX_winograd": "sipiippiiiiiii",
     "alpha_dconv3D_deltaW_GemmSK_deltaB": "siipiipiippppiiiiiiiii",
     "alpha_conv3D_biased": "sipiipiippiiiiiiiii",
@@ -311,6 +312,11 @@ class Cuda_dconv3D_deltaW:
     @staticmethod
     def dconv3D_deltaW_GemmSK(streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw):
         _call("alpha_dconv3D_deltaW_GemmSK", streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaW_GemmSK_winograd(streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, N, IC, OC, ph, pw):
+        """This build's Winograd F(3x3,2x2) backward-filter for 3x3 stride-1 layers (no reference counterpart)."""
+        _call("alpha_dconv3D_deltaW_GemmSK_winograd", streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, N, IC, OC, ph, pw)
 
     @staticmethod
     def dconv3D_deltaW_GemmV2SK(streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf, FH, FW, N, IC, OC, sh, sw, ph, pw):

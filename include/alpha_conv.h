@@ -278,6 +278,17 @@ int alpha_dconv3D_deltaX_winograd(const int64_t *streams, int length,
                                   float *deltaX, int IH, int IW,
                                   int N, int IC, int OC, int ph, int pw);
 
+/* Backward-filter of a 3x3 stride-1 layer by Winograd F(3x3,2x2): arguments and split-K contract of
+ * alpha_dconv3D_deltaW_GemmSK (slice z writes deltaW, z = 0, or deltaW_buf[z-1]; alpha_buf_summary finishes), without FH, FW,
+ * sh, sw. The slices are ranges of 2x2 output tiles instead of the reference's pixel ranges
+ * (cu32/dW/dconv3d_dW_GemmSK_kernel.cuh:131-262), so the partial results differ from the direct entry's while their sum
+ * is the same up to rounding. No counterpart in the reference. */
+int alpha_dconv3D_deltaW_GemmSK_winograd(const int64_t *streams, int length, int GridZ,
+                                         const float *X, int IH, int IW,
+                                         const float *deltaY, int OH, int OW,
+                                         float *deltaW, float *deltaW_buf,
+                                         int N, int IC, int OC, int ph, int pw);
+
 /* ---- forward with the bias added in the kernel's epilogue --------------------------------------
  * The reference has no native for this: its engine method conv3D_biased (CudaFloat32EngineBase.java:1478-1560,
  * EngineBase.java:178-185) runs the conv3D entry and then Cuda_function.linear_dual2D_row(Y, Bias, ...) =

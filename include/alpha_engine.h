@@ -41,6 +41,9 @@ typedef struct alpha_engine_config {
                                      (CudaFloat32EngineBase.java:1373-1380, 1879-1889) */
     int deltaX_winograd;          /* this build only: 1 = backward-data of 3x3 stride-1 layers (padding <= 2, more than 8 input
                                      channels) through Winograd F(2x2,3x3); default 0 */
+    int deltaW_winograd;          /* this build only: > 0 = backward-filter of 3x3 stride-1 layers (split-K case) through Winograd
+                                     F(3x3,2x2). 1: with the reference's GridZ; > 1: the number of compute units to fill - GridZ becomes
+                                     that many workgroups' worth of slices (at least 64 tiles each). Default 0 */
 } alpha_engine_config;
 
 /* Native entry chosen by a plan; names are the Java native method names. */
@@ -54,7 +57,8 @@ enum alpha_entry {
     ALPHA_E_dconv3D_deltaW, ALPHA_E_dconv3D_deltaW_W1, ALPHA_E_dconv3D_deltaW_GemmSK, ALPHA_E_dconv3D_deltaW_GemmV2SK,
     ALPHA_E_dconv3D_deltaW_GemmSK_W1,
     ALPHA_E_conv3D_winograd,  /* this build's additional forward algorithm; never chosen unless conv3D_winograd is set */
-    ALPHA_E_dconv3D_deltaX_winograd   /* the same for backward-data; never chosen unless deltaX_winograd is set */
+    ALPHA_E_dconv3D_deltaX_winograd,  /* the same for backward-data; never chosen unless deltaX_winograd is set */
+    ALPHA_E_dconv3D_deltaW_GemmSK_winograd   /* Winograd F(3x3,2x2) backward-filter; never chosen unless deltaW_winograd is set */
 };
 
 typedef struct alpha_conv_plan {

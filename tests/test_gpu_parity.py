@@ -633,6 +633,42 @@ def test_deltaW_row_streaming_kernel_slices_and_sum(dev, shape):
     check(dev.get(dWs), O.deltaW_f64(X, dY, F_, F_, 1, 1, p, p), "row-streaming dW total %s" % (shape,))
 
 
+DW_WINO_SHAPES = [
+    # N, IH, IW, IC, OC, ph, pw, GridZ   (3x3, stride 1)
+    (4, 56, 56, 64, 64, 1, 1, 16),
+    (8, 32, 32, 64, 64, 1, 1, 5),       # slices that end inside an image
+    (16, 16, 16, 128, 128, 1, 1, 7),    # four blocks of input channels, two of output channels
+    (36, 7, 7, 64, 96, 1, 1, 3),        # odd sizes: partial tiles on the right / bottom; ragged block of output channels
+    (4, 13, 11, 36, 44, 1, 1, 4),       # ragged channels
+    (4, 10, 12, 32, 64, 0, 0, 2),       # no padding
+    (4, 6, 9, 32, 64, 2, 2, 1),         # padding 2, one slice (no partial buffers)
+    (2, 5, 5, 64, 64, 1, 1, 9),         # more slices than chunks of tiles: empty slices must write zeros
+]
+
+
+@pytest.mark.parametrize("shape", DW_WINO_SHAPES)
+def test_deltaW_winograd_slices_sum_to_the_oracle(dev, shape):
+    """Winograd F(3x3,2x2) backward-filter: the slices are ranges of 2x2 tiles (not the reference's pixel ranges), so only
+    their Kahan sum (buf_summary, as after the GemmSK entry) is compared with the fp64 oracle; same bar as the direct
+    kernels. Two runs must agree bit for bit (no atomics)."""
+    N, IH, IW, IC, OC, ph, pw, GridZ = shape
+    OH, OW = out_dim(IH, IW, 3, 3, 1, 1, ph, pw)
+    X, dY = normal((N, IH, IW, IC), 3201), normal((N, OH, OW, OC), 3202)
+    x, dy = dev.put(X), dev.put(dY)
+    sizeW = OC * 9 * IC
+    runs = []
+    for _ in range(2):
+        dWo = dev.guarded(OC, 3, 3, IC)
+        buf = dev.empty(max(GridZ - 1, 1), sizeW, fill=float("nan"))
+        DW.dconv3D_deltaW_GemmSK_winograd(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(),
+                                          buf.data_ptr(), N, IC, OC, ph, pw)
+        if GridZ > 1:
+            DW.buf_summary(dev.stream, buf.data_ptr(), dWo.data_ptr(), GridZ - 1, sizeW)
+        runs.append(dev.get(dWo))
+    assert np.array_equal(runs[0], runs[1]), "two runs differ"
+    check(runs[0], O.deltaW_f64(X, dY, 3, 3, 1, 1, ph, pw), "winograd dW %s" % (shape,))
+
+
 def test_deltaW_W1_entries(dev):
     for (N, IH, IW, IC, OC) in [(4, 14, 14, 256, 64), (4, 12, 12, 64, 256), (4, 7, 9, 12, 20)]:
         X, dY = normal((N, IH, IW, IC), 3005), normal((N, IH, IW, OC), 3006)
