@@ -13,13 +13,14 @@
 // gives bit-identical results. (The partition is over tiles, not over the reference's pixel ranges: the partial results
 // differ from the direct kernels', their sum does not, up to rounding.)
 //
-// A workgroup (4 wavefronts) owns one slice, 64 output channels and 32 input channels: wavefront w accumulates output
-// channels [16w, 16w+16) x 32 input channels x 16 xi = 128 registers. Tiles advance in chunks of 8: every thread loads
-// the 4x4 patch of one (tile, input channel) and the 2x2 tile of one (tile, pair of output channels) two chunks ahead
-// (two register sets), transforms them one chunk ahead and writes Xh[xi][tile][32 + pad], Yh[xi][tile][64 + pad] into the
-// other LDS buffer, all in the shadow of the current chunk's 64 MFMAs per wavefront. MFMA operands are 32-bit LDS reads
-// with lanes across channels (the reduction index is the tile, the slow axis of both arrays); the tile strides 48 and 80
-// floats put the four tiles of an operand in different banks.
+// A workgroup owns one slice, 64 output channels and 32 input channels. Four of its eight wavefronts multiply: wavefront w
+// accumulates output channels [16w, 16w+16) x 32 input channels x 16 xi = 128 registers. The other four stage: tiles
+// advance in chunks of 8; a staging thread loads the 4x4 patch of one (tile, input channel) and the 2x2 tile of one (tile,
+// pair of output channels) a chunk before they are transformed, and writes Xh[tile][32][16 xi], Yh[tile][64][16 xi] into
+// the LDS buffer that is multiplied in the chunk after. In LDS the 16 xi of a (tile, channel) are contiguous, so a lane's
+// operand for four xi is one 128-bit read (an operand per xi as a 32-bit read - three LDS instructions per two MFMAs -
+// cost 30 cycles per pair of MFMAs); the four 16-byte groups of a (tile, channel) are stored permuted (group g at position
+// g ^ (channel / 4 % 4)), which spreads the 16 lanes of a read over all banks.
 #include "common.hpp"
 #include <type_traits>
 
@@ -42,15 +43,13 @@ struct WinoDwArgs {
 };
 
 constexpr int WD_TK = 8;                        // tiles per chunk
-constexpr int WD_XS = 48, WD_YS = 80;           // floats per tile: 32 input channels + 16, 64 output channels + 16
-constexpr int WD_XBUF = 16 * WD_TK * WD_XS;     // Xh[xi][tile][WD_XS]
-constexpr int WD_YBUF = 16 * WD_TK * WD_YS;     // Yh[xi][tile][WD_YS]
+constexpr int WD_XBUF = WD_TK * 32 * 16;        // Xh[tile][32 input channels][16 xi]
+constexpr int WD_YBUF = WD_TK * 64 * 16;        // Yh[tile][64 output channels][16 xi]
 constexpr int WD_BUF = WD_XBUF + WD_YBUF;
 constexpr unsigned WD_OOR = 0x80000000u;        // beyond both descriptors: the load returns 0
 constexpr unsigned WD_OOR_COL = 0x40000000u;    // added to a valid offset of X (at most 1 GB) or to WD_OOR: beyond too
 
-__global__ __launch_bounds__(256, 2) void winograd_dw_kernel(const WinoDwArgs p)   // <= 256 registers: the accumulators stay in
-                                                                                       // ordinary registers (no copies to and from AGPRs)
+__global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float wd_smem[];   // [2][WD_BUF]
     float *smem = wd_smem;
@@ -75,8 +74,9 @@ __global__ __launch_bounds__(256, 2) void winograd_dw_kernel(const WinoDwArgs p)
     //      size, tiles past the slice, channels past the end) are beyond the descriptors and read as zeros. The thread's
     //      tile position is kept from chunk to chunk and moved on by additions only (no division, no multiplication:
     //      recomputing 20 offsets per chunk from the tile index cost more issue slots than the chunk's 64 MFMAs). --------
-    const int st = t >> 5, sc = t & 31;
+    const int pt = t & 255, st = pt >> 5, sc = pt & 31;   // staging wavefronts (t >= 256) only
     const bool xc_ok = ic0 + sc < p.IC, yc_ok = oc0 + 2 * sc < p.OC;   // OC % 4 == 0: a pair is valid as a whole
+    const int swz_w = (sc >> 2) & 3, swz_wy = (sc >> 1) & 3;            // (channel / 4) % 4 of the channel(s) this thread writes
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.dY), 0, p.y_bytes, 0x00020000);
     const int row_elems = p.IW * p.IC;
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256, 2) void winograd_dw_kernel(const WinoDwArgs p)
         yo[1][0] = (ok && below) ? o + (unsigned)y_row * 4u : WD_OOR;
         yo[1][1] = (ok && right && below) ? o + (unsigned)(y_row + y_px) * 4u : WD_OOR;
     };
-    float xr[2][4][4];     // raw patches, two chunks in flight
+    float xr[2][4][4];     // raw patches: set s holds a chunk of parity s, requested two chunks before it is transformed
     float2 yr[2][2][2];    // raw deltaY tiles
     auto load_one = [&](auto set_c, int e) {   // e < 16: patch element e; 16..19: deltaY element e - 16
         constexpr int SET = decltype(set_c)::value;
@@ -150,11 +150,9 @@ __global__ __launch_bounds__(256, 2) void winograd_dw_kernel(const WinoDwArgs p)
             xrow[3][j] = xr[SET][3][j] - xr[SET][1][j];
         }
     };
-    auto x_store = [&](float *Xh, int i) {
-        Xh[(4 * i + 0) * WD_TK * WD_XS] = xrow[i][0] - xrow[i][2];
-        Xh[(4 * i + 1) * WD_TK * WD_XS] = xrow[i][1] + xrow[i][2];
-        Xh[(4 * i + 2) * WD_TK * WD_XS] = xrow[i][2] - xrow[i][1];
-        Xh[(4 * i + 3) * WD_TK * WD_XS] = xrow[i][3] - xrow[i][1];
+    auto x_store = [&](float *Xh, int i) {   // xi = 4i .. 4i+3: group i of this (tile, channel)
+        const floatx4 v = floatx4{xrow[i][0] - xrow[i][2], xrow[i][1] + xrow[i][2], xrow[i][2] - xrow[i][1], xrow[i][3] - xrow[i][1]};
+        *reinterpret_cast<floatx4 *>(Xh + ((i ^ swz_w) << 2)) = v;
     };
     auto add2 = [](float2 a, float2 c) { return make_float2(a.x + c.x, a.y + c.y); };
     auto sub2 = [](float2 a, float2 c) { return make_float2(a.x - c.x, a.y - c.y); };
@@ -168,95 +166,98 @@ __global__ __launch_bounds__(256, 2) void winograd_dw_kernel(const WinoDwArgs p)
             yg[3][b] = yr[SET][1][b];
         }
     };
-    auto y_store = [&](float *Yh, int a) {
-        *reinterpret_cast<float2 *>(Yh + (4 * a + 0) * WD_TK * WD_YS) = yg[a][0];
-        *reinterpret_cast<float2 *>(Yh + (4 * a + 1) * WD_TK * WD_YS) = add2(yg[a][0], yg[a][1]);
-        *reinterpret_cast<float2 *>(Yh + (4 * a + 2) * WD_TK * WD_YS) = sub2(yg[a][0], yg[a][1]);
-        *reinterpret_cast<float2 *>(Yh + (4 * a + 3) * WD_TK * WD_YS) = yg[a][1];
+    auto y_store = [&](float *Yh, int a) {   // xi = 4a .. 4a+3 of the thread's two channels
+        const float2 v1 = add2(yg[a][0], yg[a][1]), v2 = sub2(yg[a][0], yg[a][1]);
+        *reinterpret_cast<floatx4 *>(Yh + ((a ^ swz_wy) << 2)) = floatx4{yg[a][0].x, v1.x, v2.x, yg[a][1].x};
+        *reinterpret_cast<floatx4 *>(Yh + 16 + ((a ^ swz_wy) << 2)) = floatx4{yg[a][0].y, v1.y, v2.y, yg[a][1].y};
     };
-    const int xh_write = st * WD_XS + sc, yh_write = WD_XBUF + st * WD_YS + 2 * sc;
+    const int xh_write = (st * 32 + sc) * 16, yh_write = WD_XBUF + (st * 64 + 2 * sc) * 16;
+
+    // Wavefronts 0-3 multiply, wavefronts 4-7 stage: each SIMD holds one of either kind, so the staging instructions
+    // (loads, transforms, LDS writes: about 150 per chunk) fill the issue slots between the other wavefront's MFMAs without
+    // any of them sharing registers with the 128 accumulators. One barrier per chunk joins them: while chunk c is
+    // multiplied out of LDS buffer c & 1, chunk c+1 (requested from memory a chunk earlier) is transformed and written to
+    // the other buffer and chunk c+2 is requested.
+    typedef std::integral_constant<int, 0> Set0;
+    typedef std::integral_constant<int, 1> Set1;
+    if (t >= 256) {
+        if (nchunks > 0) {
+            auto request = [&](auto set_c) {   // the 20 loads of the chunk the tile cursor stands on
+                x_terms();
+#pragma unroll
+                for (int i = 0; i < 4; i++) x_offsets(i);
+                y_offsets();
+#pragma unroll
+                for (int e = 0; e < 20; e++) load_one(set_c, e);   // past the slice: out of range, zeros
+            };
+            auto transform = [&](auto set_c, int buf, bool store) {
+                x_rows(set_c);
+                y_rows(set_c);
+                if (store) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        x_store(smem + buf * WD_BUF + xh_write, i);
+                        y_store(smem + buf * WD_BUF + yh_write, i);
+                    }
+                }
+            };
+            request(Set0{});
+            transform(Set0{}, 0, true);   // chunk 0, waited for
+            advance_tile();
+            request(Set1{});              // chunk 1
+            advance_tile();
+            request(Set0{});              // chunk 2
+            __syncthreads();
+            // chunk c: chunk c+1 (requested two chunks ago) is transformed into the other buffer, chunk c+3 requested into
+            // the set it leaves. Two chunks per round so that the sets are fixed registers; the loads of the second half
+            // are issued even when that chunk does not exist (only its LDS writes and its barrier are skipped).
+            for (int c = 0; c < nchunks; c += 2) {
+                transform(Set1{}, 1, true);
+                advance_tile();
+                request(Set1{});
+                __syncthreads();
+                const bool more = c + 1 < nchunks;
+                transform(Set0{}, 0, more);
+                advance_tile();
+                request(Set0{});
+                if (more) __syncthreads();
+            }
+        }
+        return;
+    }
 
     if (nchunks > 0) {
-        // chunk 0 into LDS buffer 0, chunk 1 into register set 1 (chunk c requests chunk c+2 into set c & 1)
-        x_terms();
+        // One chunk = 8 groups of 8 MFMAs: (4 tiles kk, 4 xi) x (two blocks of input channels); three 128-bit LDS reads per
+        // group, one group ahead. The two MFMAs into one accumulator (kk = 0, 1) are 4 groups apart.
+        const int swz_r = (l16 >> 2) & 3;
+        int rdx[4], rdy[4];   // float offsets of this lane's operands for xi group gx (tile q, channel l16 / 16w + l16)
 #pragma unroll
-        for (int i = 0; i < 4; i++) x_offsets(i);
-        y_offsets();
-#pragma unroll
-        for (int e = 0; e < 20; e++) load_one(std::integral_constant<int, 0>{}, e);
-        x_rows(std::integral_constant<int, 0>{});
-        y_rows(std::integral_constant<int, 0>{});
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            x_store(smem + xh_write, i);
-            y_store(smem + yh_write, i);
+        for (int gx = 0; gx < 4; gx++) {
+            rdx[gx] = (q * 32 + l16) * 16 + ((gx ^ swz_r) << 2);
+            rdy[gx] = WD_XBUF + (q * 64 + 16 * w + l16) * 16 + ((gx ^ swz_r) << 2);
         }
-        advance_tile();
-        x_terms();
-#pragma unroll
-        for (int i = 0; i < 4; i++) x_offsets(i);
-        y_offsets();
-#pragma unroll
-        for (int e = 0; e < 20; e++) load_one(std::integral_constant<int, 1>{}, e);
         __syncthreads();
-
-        // One chunk = 32 groups of (one deltaY fragment, two patch fragments, two MFMAs): 16 xi x 2 sets of 4 tiles. Each
-        // group is a scheduling region with a slice of the staging work behind its MFMAs (a wavefront has its SIMD to
-        // itself: what is not issued in the shadow of an MFMA is lost time):
-        //   groups 0-7    the thread's tile moves on to the chunk after next; its 20 offsets
-        //   groups 8-17   that chunk's 20 loads, into the register set the previous chunk freed
-        //   groups 18-27  the next chunk (loaded during the previous one) is transformed and written to the other buffer
-        auto chunk = [&](auto par_c) {
-            constexpr int PAR = decltype(par_c)::value;   // chunk number & 1 = its LDS buffer
-            const float *Yb = smem + PAR * WD_BUF + WD_XBUF + q * WD_YS + 16 * w + l16;
-            const float *Xb = smem + PAR * WD_BUF + q * WD_XS + l16;
-            float *Xh = smem + (PAR ^ 1) * WD_BUF + xh_write, *Yh = smem + (PAR ^ 1) * WD_BUF + yh_write;
-            // fragments are read two groups ahead of their MFMAs (an LDS read takes longer than one group's 64 cycles)
-            auto frag = [&](int g, float &fa, float &fb0, float &fb1) {
-                const int xi = g >> 1, kk = g & 1;
-                fa = Yb[(xi * WD_TK + 4 * kk) * WD_YS];
-                fb0 = Xb[(xi * WD_TK + 4 * kk) * WD_XS];
-                fb1 = Xb[(xi * WD_TK + 4 * kk) * WD_XS + 16];
+        for (int c = 0; c < nchunks; c++) {
+            const float *B = smem + (c & 1) * WD_BUF;
+            auto frag = [&](int g, floatx4 &fa, floatx4 &fb0, floatx4 &fb1) {
+                const int kk = g >> 2, gx = g & 3;
+                fa = *reinterpret_cast<const floatx4 *>(B + rdy[gx] + kk * 4 * 64 * 16);
+                fb0 = *reinterpret_cast<const floatx4 *>(B + rdx[gx] + kk * 4 * 32 * 16);
+                fb1 = *reinterpret_cast<const floatx4 *>(B + rdx[gx] + kk * 4 * 32 * 16 + 16 * 16);
             };
-            float a[3], b0[3], b1[3];
+            floatx4 a[2], b0[2], b1[2];
             frag(0, a[0], b0[0], b1[0]);
-            frag(1, a[1], b0[1], b1[1]);
 #pragma unroll
-            for (int g = 0; g < 32; g++) {
-                __builtin_amdgcn_sched_barrier(0);
-                if (g + 2 < 32) frag(g + 2, a[(g + 2) % 3], b0[(g + 2) % 3], b1[(g + 2) % 3]);
-                acc[g >> 1][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g % 3], b0[g % 3], acc[g >> 1][0], 0, 0, 0);
-                acc[g >> 1][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g % 3], b1[g % 3], acc[g >> 1][1], 0, 0, 0);
-                if (g == 0) advance_tile();
-                if (g == 1) x_terms();
-                if (g >= 2 && g < 6) x_offsets(g - 2);
-                if (g == 6) y_offsets();
-                if (g >= 8 && g < 18) {
-                    load_one(std::integral_constant<int, PAR>{}, 2 * (g - 8));
-                    load_one(std::integral_constant<int, PAR>{}, 2 * (g - 8) + 1);
+            for (int g = 0; g < 8; g++) {
+                if (g + 1 < 8) frag(g + 1, a[(g + 1) & 1], b0[(g + 1) & 1], b1[(g + 1) & 1]);
+#pragma unroll
+                for (int x = 0; x < 4; x++) {
+                    const int xi = 4 * (g & 3) + x;
+                    acc[xi][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g & 1][x], b0[g & 1][x], acc[xi][0], 0, 0, 0);
+                    acc[xi][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g & 1][x], b1[g & 1][x], acc[xi][1], 0, 0, 0);
                 }
-                if (g == 18) x_rows(std::integral_constant<int, PAR ^ 1>{});
-                if (g >= 19 && g < 23) x_store(Xh, g - 19);
-                if (g == 23) y_rows(std::integral_constant<int, PAR ^ 1>{});
-                if (g >= 24 && g < 28) y_store(Yh, g - 24);
-                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);   // LDS reads of the group after next
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);   // vector ALU
-                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // a load
-                __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);   // LDS writes
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
             __syncthreads();
-        };
-        // Always two chunks per round (the second may lie past the slice: its loads are out of range, it adds zeros): with
-        // a branch around it the register sets meet at a join, and the copies made there wait for every load in flight.
-        for (int c = 0; c < nchunks; c += 2) {
-            chunk(std::integral_constant<int, 0>{});
-            chunk(std::integral_constant<int, 1>{});
         }
     }
 
@@ -333,7 +334,7 @@ hipError_t launch_deltaW_winograd(hipStream_t stream, const float *X, const floa
     constexpr auto kern = winograd_dw_kernel;
     const size_t lds = (size_t)2 * WD_BUF * sizeof(float);
     if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((IC + 31) / 32, (OC + 63) / 64, GZ), dim3(256), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3((IC + 31) / 32, (OC + 63) / 64, GZ), dim3(512), lds, stream, a);
     return hipGetLastError();
 }
 
