@@ -19,8 +19,10 @@
 // pair of output channels) a chunk before they are transformed, and writes Xh[tile][32][16 xi], Yh[tile][64][16 xi] into
 // the LDS buffer that is multiplied in the chunk after. In LDS the 16 xi of a (tile, channel) are contiguous, so a lane's
 // operand for four xi is one 128-bit read (an operand per xi as a 32-bit read - three LDS instructions per two MFMAs -
-// cost 30 cycles per pair of MFMAs); the four 16-byte groups of a (tile, channel) are stored permuted (group g at position
-// g ^ (channel / 4 % 4)), which spreads the 16 lanes of a read over all banks.
+// cost 30 cycles per pair of MFMAs). A (tile, channel) takes 80 bytes, its four 16-byte groups of xi stored permuted (group
+// g at position g ^ (channel / 16 % 4)): the 16 lanes of a read (16 consecutive channels) and the 16 lanes of a staging
+// write (channels 2 or 4 apart) then both touch 16 different 16-byte bank groups. With 64 bytes per channel the writes of
+// the deltaY stagers were 4-way bank conflicts.
 #include "common.hpp"
 #include <type_traits>
 
@@ -43,8 +45,9 @@ struct WinoDwArgs {
 };
 
 constexpr int WD_TK = 8;                        // tiles per chunk
-constexpr int WD_XBUF = WD_TK * 32 * 16;        // Xh[tile][32 input channels][16 xi]
-constexpr int WD_YBUF = WD_TK * 64 * 16;        // Yh[tile][64 output channels][16 xi]
+constexpr int WD_CS = 20;                       // floats per (tile, channel): 16 xi + 4 (see the layout note above)
+constexpr int WD_XBUF = WD_TK * 32 * WD_CS;     // Xh[tile][32 input channels][16 xi + 4]
+constexpr int WD_YBUF = WD_TK * 64 * WD_CS;     // Yh[tile][64 output channels][16 xi + 4]
 constexpr int WD_BUF = WD_XBUF + WD_YBUF;
 constexpr unsigned WD_OOR = 0x80000000u;        // beyond both descriptors: the load returns 0
 constexpr unsigned WD_OOR_COL = 0x40000000u;    // added to a valid offset of X (at most 1 GB) or to WD_OOR: beyond too
@@ -69,24 +72,31 @@ __global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
         acc[x][1] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // ---- staging: thread -> tile st of the chunk; input channel ic0 + sc for the patch, output channels oc0 + 2 sc,
-    //      oc0 + 2 sc + 1 for the deltaY tile. Offsets outside the tensors (padding, rows / columns past an odd output
-    //      size, tiles past the slice, channels past the end) are beyond the descriptors and read as zeros. The thread's
-    //      tile position is kept from chunk to chunk and moved on by additions only (no division, no multiplication:
-    //      recomputing 20 offsets per chunk from the tile index cost more issue slots than the chunk's 64 MFMAs). --------
-    const int pt = t & 255, st = pt >> 5, sc = pt & 31;   // staging wavefronts (t >= 256) only
-    const bool xc_ok = ic0 + sc < p.IC, yc_ok = oc0 + 2 * sc < p.OC;   // OC % 4 == 0: a pair is valid as a whole
-    const int swz_w = (sc >> 2) & 3, swz_wy = (sc >> 1) & 3;            // (channel / 4) % 4 of the channel(s) this thread writes
+    // ---- staging (wavefronts 4-7). Wavefronts 4 and 7 stage the patches: a thread takes (tile, pair of input channels),
+    //      16 64-bit loads; wavefronts 5 and 6 stage deltaY: a thread takes (tile, four output channels), four 128-bit
+    //      loads. Either way 16 threads per tile, 8 tiles per chunk, and about 90 instructions per thread and chunk. (One
+    //      channel per thread with 32-bit loads took 215, and the 80 load instructions per chunk of a compute unit's four
+    //      staging wavefronts alone kept its address pipeline busy for most of the chunk.) Offsets outside the tensors
+    //      (padding, rows / columns past an odd output size, tiles past the slice, channels past the end) are beyond the
+    //      descriptors and read as zeros. A thread's tile position is kept from chunk to chunk and moved on by
+    //      additions only (no division, no multiplication). ------------------------------------------------------------------
+    const int sw = w - 4;                                  // staging wavefront
+    const bool x_role = sw == 0 || sw == 3;
+    const int item = ((sw == 0 || sw == 1) ? 0 : 64) + lane;   // of the role's 128 items
+    const int st = item >> 4, sub = item & 15;
+    const int x_ch = 2 * sub, y_ch = 4 * sub;              // first channel of the thread's pair / quad within the block
+    const bool xc_ok = ic0 + x_ch < p.IC, yc_ok = oc0 + y_ch < p.OC;   // IC, OC % 4 == 0: valid as a whole
+    const int swz_wx = (x_ch >> 4) & 3, swz_wy = (y_ch >> 4) & 3;   // (channel / 16) % 4 of the channels this thread writes
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.dY), 0, p.y_bytes, 0x00020000);
     const int row_elems = p.IW * p.IC;
-    int tile_cur = tile_begin + st, ty, tx, x00, y00;   // x00: element offset of X[n, 2ty-ph, 2tx-pw, ic0+sc] (may be negative)
+    int tile_cur = tile_begin + st, ty, tx, x00, y00;   // x00: element offset of X[n, 2ty-ph, 2tx-pw, ic0+x_ch] (may be negative)
     {
         const int n = fdiv(tile_cur, p.d_TRC), rem = tile_cur - n * p.TRC;
         ty = fdiv(rem, p.d_TC);
         tx = rem - ty * p.TC;
-        x00 = (n * p.IH + 2 * ty - p.ph) * row_elems + (2 * tx - p.pw) * p.IC + ic0 + sc;
-        y00 = ((n * p.OH + 2 * ty) * p.OW + 2 * tx) * p.OC + oc0 + 2 * sc;
+        x00 = (n * p.IH + 2 * ty - p.ph) * row_elems + (2 * tx - p.pw) * p.IC + ic0 + x_ch;
+        y00 = ((n * p.OH + 2 * ty) * p.OW + 2 * tx) * p.OC + oc0 + y_ch;
     }
     auto advance_tile = [&]() {
         tile_cur += WD_TK;
@@ -104,124 +114,132 @@ __global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
         x00 += w2 ? p.wx2 : 0;
         y00 += w2 ? p.wy2 : 0;
     };
-    unsigned xo[4][4], yo[2][2], rowterm[4], colterm[4];
-    auto x_terms = [&]() {
-        const bool ok = tile_cur < tile_end && xc_ok;
-        const int ih0 = 2 * ty - p.ph, iw0 = 2 * tx - p.pw;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const unsigned rv = (unsigned)x00 * 4u + (unsigned)(i * row_elems) * 4u, cv = (unsigned)(i * p.IC) * 4u;   // i-th terms are uniform
-            rowterm[i] = (ok && (unsigned)(ih0 + i) < (unsigned)p.IH) ? rv : WD_OOR;
-            colterm[i] = ((unsigned)(iw0 + i) < (unsigned)p.IW) ? cv : WD_OOR_COL;
-        }
-    };
-    auto x_offsets = [&](int i) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) xo[i][j] = rowterm[i] + colterm[j];
-    };
-    const int y_px = p.OC, y_row = p.OW * p.OC;
-    auto y_offsets = [&]() {   // everything computed, then selected: no divergent branches among the MFMAs
-        const bool ok = tile_cur < tile_end && yc_ok;
-        const bool right = 2 * tx + 1 < p.OW, below = 2 * ty + 1 < p.OH;
-        const unsigned o = (unsigned)y00 * 4u;
-        yo[0][0] = ok ? o : WD_OOR;
-        yo[0][1] = (ok && right) ? o + (unsigned)y_px * 4u : WD_OOR;
-        yo[1][0] = (ok && below) ? o + (unsigned)y_row * 4u : WD_OOR;
-        yo[1][1] = (ok && right && below) ? o + (unsigned)(y_row + y_px) * 4u : WD_OOR;
-    };
-    float xr[2][4][4];     // raw patches: set s holds a chunk of parity s, requested two chunks before it is transformed
-    float2 yr[2][2][2];    // raw deltaY tiles
-    auto load_one = [&](auto set_c, int e) {   // e < 16: patch element e; 16..19: deltaY element e - 16
-        constexpr int SET = decltype(set_c)::value;
-        if (e < 16) xr[SET][e >> 2][e & 3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, xo[e >> 2][e & 3], 0, 0));
-        else yr[SET][(e - 16) >> 1][(e - 16) & 1] = __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(y_rsrc, yo[(e - 16) >> 1][(e - 16) & 1], 0, 0));
-    };
-    // Xh = B^T x B; Yh' = G' y G'^T with G' = [[1,0],[1,1],[1,-1],[0,1]] = G without its factors 1/2, which are applied to
-    // the accumulators once, at the end
-    float xrow[4][4];
-    float2 yg[4][2];
-    auto x_rows = [&](auto set_c) {
-        constexpr int SET = decltype(set_c)::value;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            xrow[0][j] = xr[SET][0][j] - xr[SET][2][j];
-            xrow[1][j] = xr[SET][1][j] + xr[SET][2][j];
-            xrow[2][j] = xr[SET][2][j] - xr[SET][1][j];
-            xrow[3][j] = xr[SET][3][j] - xr[SET][1][j];
-        }
-    };
-    auto x_store = [&](float *Xh, int i) {   // xi = 4i .. 4i+3: group i of this (tile, channel)
-        const floatx4 v = floatx4{xrow[i][0] - xrow[i][2], xrow[i][1] + xrow[i][2], xrow[i][2] - xrow[i][1], xrow[i][3] - xrow[i][1]};
-        *reinterpret_cast<floatx4 *>(Xh + ((i ^ swz_w) << 2)) = v;
-    };
-    auto add2 = [](float2 a, float2 c) { return make_float2(a.x + c.x, a.y + c.y); };
-    auto sub2 = [](float2 a, float2 c) { return make_float2(a.x - c.x, a.y - c.y); };
-    auto y_rows = [&](auto set_c) {
-        constexpr int SET = decltype(set_c)::value;
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-            yg[0][b] = yr[SET][0][b];
-            yg[1][b] = add2(yr[SET][0][b], yr[SET][1][b]);
-            yg[2][b] = sub2(yr[SET][0][b], yr[SET][1][b]);
-            yg[3][b] = yr[SET][1][b];
-        }
-    };
-    auto y_store = [&](float *Yh, int a) {   // xi = 4a .. 4a+3 of the thread's two channels
-        const float2 v1 = add2(yg[a][0], yg[a][1]), v2 = sub2(yg[a][0], yg[a][1]);
-        *reinterpret_cast<floatx4 *>(Yh + ((a ^ swz_wy) << 2)) = floatx4{yg[a][0].x, v1.x, v2.x, yg[a][1].x};
-        *reinterpret_cast<floatx4 *>(Yh + 16 + ((a ^ swz_wy) << 2)) = floatx4{yg[a][0].y, v1.y, v2.y, yg[a][1].y};
-    };
-    const int xh_write = (st * 32 + sc) * 16, yh_write = WD_XBUF + (st * 64 + 2 * sc) * 16;
-
-    // Wavefronts 0-3 multiply, wavefronts 4-7 stage: each SIMD holds one of either kind, so the staging instructions
-    // (loads, transforms, LDS writes: about 150 per chunk) fill the issue slots between the other wavefront's MFMAs without
-    // any of them sharing registers with the 128 accumulators. One barrier per chunk joins them: while chunk c is
-    // multiplied out of LDS buffer c & 1, chunk c+1 (requested from memory a chunk earlier) is transformed and written to
-    // the other buffer and chunk c+2 is requested.
     typedef std::integral_constant<int, 0> Set0;
     typedef std::integral_constant<int, 1> Set1;
-    if (t >= 256) {
-        if (nchunks > 0) {
-            auto request = [&](auto set_c) {   // the 20 loads of the chunk the tile cursor stands on
-                x_terms();
+
+    if (t >= 256) __builtin_amdgcn_s_setprio(3);   // staging instructions go first: they are few, and the multiplying wavefront of the SIMD waits for them at the barrier
+    if (t >= 256 && x_role) {
+        if (nchunks == 0) return;
+        float2 xr[2][4][4];   // raw patches: set s holds a chunk of parity s, requested two chunks before it is transformed
+        auto request = [&](auto set_c) {   // the 16 loads of the chunk the tile cursor stands on
+            constexpr int SET = decltype(set_c)::value;
+            const bool ok = tile_cur < tile_end && xc_ok;
+            const int ih0 = 2 * ty - p.ph, iw0 = 2 * tx - p.pw;
+            unsigned rowterm[4], colterm[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) x_offsets(i);
-                y_offsets();
+            for (int i = 0; i < 4; i++) {
+                const unsigned rv = (unsigned)x00 * 4u + (unsigned)(i * row_elems) * 4u, cv = (unsigned)(i * p.IC) * 4u;
+                rowterm[i] = (ok && (unsigned)(ih0 + i) < (unsigned)p.IH) ? rv : WD_OOR;
+                colterm[i] = ((unsigned)(iw0 + i) < (unsigned)p.IW) ? cv : WD_OOR_COL;
+            }
 #pragma unroll
-                for (int e = 0; e < 20; e++) load_one(set_c, e);   // past the slice: out of range, zeros
-            };
-            auto transform = [&](auto set_c, int buf, bool store) {
-                x_rows(set_c);
-                y_rows(set_c);
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    xr[SET][i][j] = __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, rowterm[i] + colterm[j], 0, 0));
+        };
+        // Xh = B^T x B per channel; the 4 xi of a row are one 128-bit element of the (tile, channel)
+        auto transform = [&](auto set_c, int buf, bool store) {
+            constexpr int SET = decltype(set_c)::value;
+            float *Xh = smem + buf * WD_BUF + (st * 32 + x_ch) * WD_CS;
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                float r[4][4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float x0 = k ? xr[SET][0][j].y : xr[SET][0][j].x, x1 = k ? xr[SET][1][j].y : xr[SET][1][j].x;
+                    const float x2 = k ? xr[SET][2][j].y : xr[SET][2][j].x, x3 = k ? xr[SET][3][j].y : xr[SET][3][j].x;
+                    r[0][j] = x0 - x2;
+                    r[1][j] = x1 + x2;
+                    r[2][j] = x2 - x1;
+                    r[3][j] = x3 - x1;
+                }
                 if (store) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        x_store(smem + buf * WD_BUF + xh_write, i);
-                        y_store(smem + buf * WD_BUF + yh_write, i);
-                    }
+                    for (int i = 0; i < 4; i++)
+                        *reinterpret_cast<floatx4 *>(Xh + k * WD_CS + ((i ^ swz_wx) << 2)) =
+                            floatx4{r[i][0] - r[i][2], r[i][1] + r[i][2], r[i][2] - r[i][1], r[i][3] - r[i][1]};
                 }
-            };
-            request(Set0{});
-            transform(Set0{}, 0, true);   // chunk 0, waited for
-            advance_tile();
-            request(Set1{});              // chunk 1
-            advance_tile();
-            request(Set0{});              // chunk 2
-            __syncthreads();
-            // chunk c: chunk c+1 (requested two chunks ago) is transformed into the other buffer, chunk c+3 requested into
-            // the set it leaves. Two chunks per round so that the sets are fixed registers; the loads of the second half
-            // are issued even when that chunk does not exist (only its LDS writes and its barrier are skipped).
-            for (int c = 0; c < nchunks; c += 2) {
-                transform(Set1{}, 1, true);
-                advance_tile();
-                request(Set1{});
-                __syncthreads();
-                const bool more = c + 1 < nchunks;
-                transform(Set0{}, 0, more);
-                advance_tile();
-                request(Set0{});
-                if (more) __syncthreads();
             }
+        };
+        request(Set0{});
+        transform(Set0{}, 0, true);   // chunk 0, waited for
+        advance_tile();
+        request(Set1{});              // chunk 1
+        advance_tile();
+        request(Set0{});              // chunk 2
+        __syncthreads();
+        // chunk c: chunk c+1 (requested two chunks ago) is transformed into the other buffer, chunk c+3 requested into the
+        // set it leaves. Two chunks per round so that the sets are fixed registers; the loads of the second half are issued
+        // even when that chunk does not exist (only its LDS writes and its barrier are skipped).
+        for (int c = 0; c < nchunks; c += 2) {
+            transform(Set1{}, 1, true);
+            advance_tile();
+            request(Set1{});
+            __syncthreads();
+            const bool more = c + 1 < nchunks;
+            transform(Set0{}, 0, more);
+            advance_tile();
+            request(Set0{});
+            if (more) __syncthreads();
+        }
+        return;
+    }
+    if (t >= 256) {
+        if (nchunks == 0) return;
+        floatx4 yr[2][2][2];   // raw deltaY tiles
+        const int y_px = p.OC, y_row = p.OW * p.OC;
+        auto request = [&](auto set_c) {
+            constexpr int SET = decltype(set_c)::value;
+            const bool ok = tile_cur < tile_end && yc_ok;
+            const bool right = 2 * tx + 1 < p.OW, below = 2 * ty + 1 < p.OH;
+            const unsigned o = (unsigned)y00 * 4u;
+            const unsigned o00 = ok ? o : WD_OOR, o01 = (ok && right) ? o + (unsigned)y_px * 4u : WD_OOR;
+            const unsigned o10 = (ok && below) ? o + (unsigned)y_row * 4u : WD_OOR;
+            const unsigned o11 = (ok && right && below) ? o + (unsigned)(y_row + y_px) * 4u : WD_OOR;
+            yr[SET][0][0] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, o00, 0, 0));
+            yr[SET][0][1] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, o01, 0, 0));
+            yr[SET][1][0] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, o10, 0, 0));
+            yr[SET][1][1] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, o11, 0, 0));
+        };
+        // Yh' = G' y G'^T per channel with G' = [[1,0],[1,1],[1,-1],[0,1]] = G without its factors 1/2, which are applied to
+        // the accumulators once, at the end
+        auto transform = [&](auto set_c, int buf, bool store) {
+            constexpr int SET = decltype(set_c)::value;
+            float *Yh = smem + buf * WD_BUF + WD_XBUF + (st * 64 + y_ch) * WD_CS;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float y00v = yr[SET][0][0][k], y01v = yr[SET][0][1][k], y10v = yr[SET][1][0][k], y11v = yr[SET][1][1][k];
+                float g[4][2];
+                g[0][0] = y00v; g[0][1] = y01v;
+                g[1][0] = y00v + y10v; g[1][1] = y01v + y11v;
+                g[2][0] = y00v - y10v; g[2][1] = y01v - y11v;
+                g[3][0] = y10v; g[3][1] = y11v;
+                if (store) {
+#pragma unroll
+                    for (int a = 0; a < 4; a++)
+                        *reinterpret_cast<floatx4 *>(Yh + k * WD_CS + ((a ^ swz_wy) << 2)) =
+                            floatx4{g[a][0], g[a][0] + g[a][1], g[a][0] - g[a][1], g[a][1]};
+                }
+            }
+        };
+        request(Set0{});
+        transform(Set0{}, 0, true);
+        advance_tile();
+        request(Set1{});
+        advance_tile();
+        request(Set0{});
+        __syncthreads();
+        for (int c = 0; c < nchunks; c += 2) {
+            transform(Set1{}, 1, true);
+            advance_tile();
+            request(Set1{});
+            __syncthreads();
+            const bool more = c + 1 < nchunks;
+            transform(Set0{}, 0, more);
+            advance_tile();
+            request(Set0{});
+            if (more) __syncthreads();
         }
         return;
     }
@@ -229,21 +247,21 @@ __global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
     if (nchunks > 0) {
         // One chunk = 8 groups of 8 MFMAs: (4 tiles kk, 4 xi) x (two blocks of input channels); three 128-bit LDS reads per
         // group, one group ahead. The two MFMAs into one accumulator (kk = 0, 1) are 4 groups apart.
-        const int swz_r = (l16 >> 2) & 3;
-        int rdx[4], rdy[4];   // float offsets of this lane's operands for xi group gx (tile q, channel l16 / 16w + l16)
+        int rdx0[4], rdx1[4], rdy[4];   // float offsets of this lane's operands for xi group gx (tile q; channels l16, 16 + l16, 16w + l16)
 #pragma unroll
         for (int gx = 0; gx < 4; gx++) {
-            rdx[gx] = (q * 32 + l16) * 16 + ((gx ^ swz_r) << 2);
-            rdy[gx] = WD_XBUF + (q * 64 + 16 * w + l16) * 16 + ((gx ^ swz_r) << 2);
+            rdx0[gx] = (q * 32 + l16) * WD_CS + (gx << 2);
+            rdx1[gx] = (q * 32 + 16 + l16) * WD_CS + ((gx ^ 1) << 2);
+            rdy[gx] = WD_XBUF + (q * 64 + 16 * w + l16) * WD_CS + ((gx ^ w) << 2);
         }
         __syncthreads();
         for (int c = 0; c < nchunks; c++) {
             const float *B = smem + (c & 1) * WD_BUF;
             auto frag = [&](int g, floatx4 &fa, floatx4 &fb0, floatx4 &fb1) {
                 const int kk = g >> 2, gx = g & 3;
-                fa = *reinterpret_cast<const floatx4 *>(B + rdy[gx] + kk * 4 * 64 * 16);
-                fb0 = *reinterpret_cast<const floatx4 *>(B + rdx[gx] + kk * 4 * 32 * 16);
-                fb1 = *reinterpret_cast<const floatx4 *>(B + rdx[gx] + kk * 4 * 32 * 16 + 16 * 16);
+                fa = *reinterpret_cast<const floatx4 *>(B + rdy[gx] + kk * 4 * 64 * WD_CS);
+                fb0 = *reinterpret_cast<const floatx4 *>(B + rdx0[gx] + kk * 4 * 32 * WD_CS);
+                fb1 = *reinterpret_cast<const floatx4 *>(B + rdx1[gx] + kk * 4 * 32 * WD_CS);
             };
             floatx4 a[2], b0[2], b1[2];
             frag(0, a[0], b0[0], b1[0]);
