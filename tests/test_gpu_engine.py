@@ -95,6 +95,40 @@ def test_engine_deltaX_winograd_flag(dev, eng):
         eng.config.deltaX_winograd = 0
 
 
+def test_engine_deltaW_winograd_flag(dev, eng):
+    """deltaW_winograd > 0 sends the split-K backward-filter of a 3x3 stride-1 layer through the Winograd F(3x3,2x2) entry
+    (1: the reference's GridZ; > 1: GridZ sized for that many compute units); off, the plan is the reference's."""
+    N, IH, IC, OC = 8, 16, 64, 64
+    X, dY = normal((N, IH, IH, IC), 6221), normal((N, IH, IH, OC), 6222)
+    want = O.deltaW_f64(X, dY, 3, 3, 1, 1, 1, 1)
+    x, dy = dev.put(X), dev.put(dY)
+    ref_plan = pkg.engine.plan_deltaW(eng.config, IH, IH, IH, IH, 3, 3, N, IC, OC, 1, 1)
+    for flag in (0, 1, 64):
+        eng.config.deltaW_winograd = flag
+        try:
+            dw = dev.empty(OC, 3, 3, IC, fill=float("nan"))
+            p = eng.dconv3D_deltaW(dw.data_ptr(), 3, 3, x.data_ptr(), IH, IH, dy.data_ptr(), IH, IH, N, IC, OC, 1, 1, 1, 1)
+            eng.sync()
+        finally:
+            eng.config.deltaW_winograd = 0
+        if flag:
+            assert p.entry_name == "dconv3D_deltaW_GemmSK_winograd"
+            if flag == 1:
+                assert p.GridZ == ref_plan.GridZ
+            else:
+                assert p.GridZ == min(64 // 2, N * 8 * 8 // 64)   # 2 channel blocks; slices of at least 64 tiles
+        else:
+            assert p.entry_name == ref_plan.entry_name
+        check(dev.get(dw), want, "engine deltaW (winograd %d)" % flag)
+    # strided and 1x1 layers keep the reference's plan with the flag set
+    eng.config.deltaW_winograd = 1
+    try:
+        assert pkg.engine.plan_deltaW(eng.config, 16, 16, 8, 8, 3, 3, N, IC, OC, 2, 2).entry_name != "dconv3D_deltaW_GemmSK_winograd"
+        assert pkg.engine.plan_deltaW(eng.config, 16, 16, 16, 16, 1, 1, N, IC, OC, 1, 1).entry_name != "dconv3D_deltaW_GemmSK_winograd"
+    finally:
+        eng.config.deltaW_winograd = 0
+
+
 def test_engine_conv3D_biased(dev, eng):
     N, IH, IC, OC = 8, 14, 64, 64
     X, W, B = normal((N, IH, IH, IC), 6201), he_normal(OC, 3, 3, IC, 6202), normal((OC,), 6203)
