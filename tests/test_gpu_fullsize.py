@@ -86,6 +86,20 @@ def test_full_size_layer(dev, layer):
             eng.config.conv3D_winograd = 0
             eng.sync()
             assert plan.entry_name == "conv3D_winograd"
+        dxw = dww = dww2 = None
+        if F == 3 and s == 1 and IC >= 16:   # the same layer through the Winograd backward paths of this build
+            dxw = torch.full((N, IH, IW, IC), float("nan"), device=dev.dev)
+            dww = torch.full((OC, F, F, IC), float("nan"), device=dev.dev)
+            dww2 = torch.full((OC, F, F, IC), float("nan"), device=dev.dev)
+            eng.config.deltaX_winograd = 1
+            eng.config.deltaW_winograd = pkg.device_info()[0]
+            px = eng.dconv3D_deltaX(dxw.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), F, F, N, IC, OC, s, s, p, p)
+            pw_ = eng.dconv3D_deltaW(dww.data_ptr(), F, F, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, s, s, p, p)
+            eng.dconv3D_deltaW(dww2.data_ptr(), F, F, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, s, s, p, p)
+            eng.config.deltaX_winograd = 0
+            eng.config.deltaW_winograd = 0
+            eng.sync()
+            assert px.entry_name == "dconv3D_deltaX_winograd" and pw_.entry_name == "dconv3D_deltaW_GemmSK_winograd"
         dw2 = None
         if layer.startswith("c5"):
             dw2 = torch.full((OC, F, F, IC), float("nan"), device=dev.dev)
@@ -103,6 +117,8 @@ def test_full_size_layer(dev, layer):
             _check(yw[n:n + 1].cpu().numpy(), want, "%s Winograd forward image %d" % (layer, n))
         wantx = O.deltaX_f64(np.ascontiguousarray(dYn[n:n + 1]), Wn, IH, IW, s, s, p, p)
         _check(dx[n:n + 1].cpu().numpy(), wantx, "%s deltaX image %d" % (layer, n))
+        if dxw is not None:
+            _check(dxw[n:n + 1].cpu().numpy(), wantx, "%s Winograd deltaX image %d" % (layer, n))
 
     # (2) adjointness in fp64 on the device
     a = float((y.double() * dy.double()).sum())
@@ -112,6 +128,15 @@ def test_full_size_layer(dev, layer):
     assert abs(a - b) <= 2e-5 * scale, "%s: <Y,dY> = %r vs <X,dX> = %r" % (layer, a, b)
     assert abs(a - c) <= 2e-5 * scale, "%s: <Y,dY> = %r vs <W,dW> = %r" % (layer, a, c)
     assert bool(torch.isfinite(dw).all()) and bool(torch.isfinite(dx).all())
+    if dww is not None:
+        cw = float((w.double() * dww.double()).sum())
+        assert abs(a - cw) <= 2e-5 * scale, "%s: <Y,dY> = %r vs <W,dW Winograd> = %r" % (layer, a, cw)
+        # element-wise against the direct kernel's result (both within the bar of the oracle: twice the bar between them)
+        ref = dw.double()
+        floor = 1e-5 * max(1.0, float(ref.pow(2).mean().sqrt()))
+        err = (dww.double() - ref).abs() - 2 * torch.clamp(1e-4 * ref.abs(), min=floor)
+        assert float(err.max()) <= 0.0, "%s: Winograd deltaW differs from the direct kernel's beyond twice the bar" % layer
+        assert torch.equal(dww, dww2), "%s: Winograd deltaW differs between two runs" % layer
 
     # (3) run-to-run bit reproducibility of backward-filter (config 5)
     if dw2 is not None:
