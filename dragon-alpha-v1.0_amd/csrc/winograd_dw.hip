@@ -13,16 +13,18 @@
 // gives bit-identical results. (The partition is over tiles, not over the reference's pixel ranges: the partial results
 // differ from the direct kernels', their sum does not, up to rounding.)
 //
-// A workgroup owns one slice, 64 output channels and 32 input channels. Four of its eight wavefronts multiply: wavefront w
-// accumulates output channels [16w, 16w+16) x 32 input channels x 16 xi = 128 registers. The other four stage: tiles
-// advance in chunks of 8; a staging thread loads the 4x4 patch of one (tile, input channel) and the 2x2 tile of one (tile,
-// pair of output channels) a chunk before they are transformed, and writes Xh[tile][32][16 xi], Yh[tile][64][16 xi] into
-// the LDS buffer that is multiplied in the chunk after. In LDS the 16 xi of a (tile, channel) are contiguous, so a lane's
-// operand for four xi is one 128-bit read (an operand per xi as a 32-bit read - three LDS instructions per two MFMAs -
-// cost 30 cycles per pair of MFMAs). A (tile, channel) takes 80 bytes, its four 16-byte groups of xi stored permuted (group
-// g at position g ^ (channel / 16 % 4)): the 16 lanes of a read (16 consecutive channels) and the 16 lanes of a staging
-// write (channels 2 or 4 apart) then both touch 16 different 16-byte bank groups. With 64 bytes per channel the writes of
-// the deltaY stagers were 4-way bank conflicts.
+// A workgroup owns one slice, 64 output channels and 32 input channels, and has six wavefronts. Four multiply: wavefront w
+// accumulates output channels [16w, 16w+16) x 32 input channels x 16 xi = 128 registers. Tiles advance in chunks of 8.
+// Two wavefronts stage the patches: a thread loads the 4x4 patch of one (tile, pair of input channels) two chunks before
+// it is transformed and writes Xh[tile][32][16 xi] into the LDS buffer that is multiplied in the chunk after; one barrier
+// per chunk joins the two kinds (wavefronts of one kind doing both jobs needed scheduling directives, spilled, or moved
+// the accumulators through AGPRs). deltaY does not pass through LDS: a multiplying wavefront is the only user of its 16
+// output channels, so its lanes load their own 2x2 tiles and transform them in registers into MFMA operands.
+// In LDS the 16 xi of a (tile, channel) are contiguous, so a lane's patch operand for four xi is one 128-bit read (an
+// operand per xi as a 32-bit read - three LDS instructions per two MFMAs - cost 30 cycles per pair of MFMAs). A (tile,
+// channel) takes 80 bytes, its four 16-byte groups of xi stored permuted (group g at position g ^ (channel / 16 % 4)): the
+// 16 lanes of a read (16 consecutive channels) and the 16 lanes of a staging write (channels 2 apart) then both touch 16
+// different 16-byte bank groups.
 #include "common.hpp"
 #include <type_traits>
 
@@ -46,15 +48,14 @@ struct WinoDwArgs {
 
 constexpr int WD_TK = 8;                        // tiles per chunk
 constexpr int WD_CS = 20;                       // floats per (tile, channel): 16 xi + 4 (see the layout note above)
-constexpr int WD_XBUF = WD_TK * 32 * WD_CS;     // Xh[tile][32 input channels][16 xi + 4]
-constexpr int WD_YBUF = WD_TK * 64 * WD_CS;     // Yh[tile][64 output channels][16 xi + 4]
-constexpr int WD_BUF = WD_XBUF + WD_YBUF;
+constexpr int WD_XBUF = WD_TK * 32 * WD_CS;     // Xh[tile][32 input channels][16 xi + 4]: one LDS buffer
+constexpr int WD_BUF = WD_XBUF;
 constexpr unsigned WD_OOR = 0x80000000u;        // beyond both descriptors: the load returns 0
 constexpr unsigned WD_OOR_COL = 0x40000000u;    // added to a valid offset of X (at most 1 GB) or to WD_OOR: beyond too
 
-__global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
+__global__ __launch_bounds__(384) void winograd_dw_kernel(const WinoDwArgs p)
 {
-    extern __shared__ __attribute__((aligned(16))) float wd_smem[];   // [2][WD_BUF]
+    extern __shared__ __attribute__((aligned(16))) float wd_smem[];   // Xh[2][WD_BUF]
     float *smem = wd_smem;
 
     const int t = threadIdx.x;
@@ -72,63 +73,61 @@ __global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
         acc[x][1] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // ---- staging (wavefronts 4-7). Wavefronts 4 and 7 stage the patches: a thread takes (tile, pair of input channels),
-    //      16 64-bit loads; wavefronts 5 and 6 stage deltaY: a thread takes (tile, four output channels), four 128-bit
-    //      loads. Either way 16 threads per tile, 8 tiles per chunk, and about 90 instructions per thread and chunk. (One
-    //      channel per thread with 32-bit loads took 215, and the 80 load instructions per chunk of a compute unit's four
-    //      staging wavefronts alone kept its address pipeline busy for most of the chunk.) Offsets outside the tensors
-    //      (padding, rows / columns past an odd output size, tiles past the slice, channels past the end) are beyond the
-    //      descriptors and read as zeros. A thread's tile position is kept from chunk to chunk and moved on by
-    //      additions only (no division, no multiplication). ------------------------------------------------------------------
-    const int sw = w - 4;                                  // staging wavefront
-    const bool x_role = sw == 0 || sw == 3;
-    const int item = ((sw == 0 || sw == 1) ? 0 : 64) + lane;   // of the role's 128 items
-    const int st = item >> 4, sub = item & 15;
-    const int x_ch = 2 * sub, y_ch = 4 * sub;              // first channel of the thread's pair / quad within the block
-    const bool xc_ok = ic0 + x_ch < p.IC, yc_ok = oc0 + y_ch < p.OC;   // IC, OC % 4 == 0: valid as a whole
-    const int swz_wx = (x_ch >> 4) & 3, swz_wy = (y_ch >> 4) & 3;   // (channel / 16) % 4 of the channels this thread writes
+    // Tile positions are kept per thread from chunk to chunk and moved on by additions only (no division, no multiplication:
+    // recomputing a chunk's offsets from tile indices cost more issue slots than the chunk's MFMAs).
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.dY), 0, p.y_bytes, 0x00020000);
     const int row_elems = p.IW * p.IC;
-    int tile_cur = tile_begin + st, ty, tx, x00, y00;   // x00: element offset of X[n, 2ty-ph, 2tx-pw, ic0+x_ch] (may be negative)
-    {
-        const int n = fdiv(tile_cur, p.d_TRC), rem = tile_cur - n * p.TRC;
-        ty = fdiv(rem, p.d_TC);
-        tx = rem - ty * p.TC;
-        x00 = (n * p.IH + 2 * ty - p.ph) * row_elems + (2 * tx - p.pw) * p.IC + ic0 + x_ch;
-        y00 = ((n * p.OH + 2 * ty) * p.OW + 2 * tx) * p.OC + oc0 + y_ch;
-    }
-    auto advance_tile = [&]() {
-        tile_cur += WD_TK;
-        tx += p.adv_tx;
-        ty += p.adv_ty;
-        x00 += p.dx0;
-        y00 += p.dy0;
-        const bool w1 = tx >= p.TC;
-        tx -= w1 ? p.TC : 0;
-        ty += w1 ? 1 : 0;
-        x00 += w1 ? p.wx1 : 0;
-        y00 += w1 ? p.wy1 : 0;
-        const bool w2 = ty >= p.TR;
-        ty -= w2 ? p.TR : 0;
-        x00 += w2 ? p.wx2 : 0;
-        y00 += w2 ? p.wy2 : 0;
+    struct TileCur {
+        int tile, ty, tx, x00, y00;   // x00 / y00: element offsets of X[n, 2ty-ph, 2tx-pw, channel] (may be negative) / deltaY[n, 2ty, 2tx, channel]
+    };
+    auto cur_init = [&](TileCur &c, int tile, int x_channel, int y_channel) {
+        c.tile = tile;
+        const int n = fdiv(tile, p.d_TRC), rem = tile - n * p.TRC;
+        c.ty = fdiv(rem, p.d_TC);
+        c.tx = rem - c.ty * p.TC;
+        c.x00 = (n * p.IH + 2 * c.ty - p.ph) * row_elems + (2 * c.tx - p.pw) * p.IC + x_channel;
+        c.y00 = ((n * p.OH + 2 * c.ty) * p.OW + 2 * c.tx) * p.OC + y_channel;
+    };
+    auto cur_advance = [&](TileCur &c) {   // 8 tiles on
+        c.tile += WD_TK;
+        c.tx += p.adv_tx;
+        c.ty += p.adv_ty;
+        c.x00 += p.dx0;
+        c.y00 += p.dy0;
+        const bool w1 = c.tx >= p.TC;
+        c.tx -= w1 ? p.TC : 0;
+        c.ty += w1 ? 1 : 0;
+        c.x00 += w1 ? p.wx1 : 0;
+        c.y00 += w1 ? p.wy1 : 0;
+        const bool w2 = c.ty >= p.TR;
+        c.ty -= w2 ? p.TR : 0;
+        c.x00 += w2 ? p.wx2 : 0;
+        c.y00 += w2 ? p.wy2 : 0;
     };
     typedef std::integral_constant<int, 0> Set0;
     typedef std::integral_constant<int, 1> Set1;
 
-    if (t >= 256) __builtin_amdgcn_s_setprio(3);   // staging instructions go first: they are few, and the multiplying wavefront of the SIMD waits for them at the barrier
-    if (t >= 256 && x_role) {
+    // ---- wavefronts 4 and 5 stage the patches: a thread takes (tile, pair of input channels) - 16 64-bit loads two chunks
+    //      ahead, B^T x B, eight 128-bit LDS writes into the buffer that is multiplied in the next chunk. Offsets outside the
+    //      tensor (padding, tiles past the slice, channels past the end) are beyond the descriptor and read as zeros. -------
+    if (t >= 256) {
         if (nchunks == 0) return;
+        __builtin_amdgcn_s_setprio(3);   // few instructions, and the multiplying wavefronts wait for them at the barrier
+        const int item = t - 256, st = item >> 4, x_ch = 2 * (item & 15);
+        const bool xc_ok = ic0 + x_ch < p.IC;          // IC % 4 == 0: a pair is valid as a whole
+        const int swz_wx = (x_ch >> 4) & 3;            // (channel / 16) % 4 of the channels this thread writes
+        TileCur cur;
+        cur_init(cur, tile_begin + st, ic0 + x_ch, 0);
         float2 xr[2][4][4];   // raw patches: set s holds a chunk of parity s, requested two chunks before it is transformed
         auto request = [&](auto set_c) {   // the 16 loads of the chunk the tile cursor stands on
             constexpr int SET = decltype(set_c)::value;
-            const bool ok = tile_cur < tile_end && xc_ok;
-            const int ih0 = 2 * ty - p.ph, iw0 = 2 * tx - p.pw;
+            const bool ok = cur.tile < tile_end && xc_ok;
+            const int ih0 = 2 * cur.ty - p.ph, iw0 = 2 * cur.tx - p.pw;
             unsigned rowterm[4], colterm[4];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const unsigned rv = (unsigned)x00 * 4u + (unsigned)(i * row_elems) * 4u, cv = (unsigned)(i * p.IC) * 4u;
+                const unsigned rv = (unsigned)cur.x00 * 4u + (unsigned)(i * row_elems) * 4u, cv = (unsigned)(i * p.IC) * 4u;
                 rowterm[i] = (ok && (unsigned)(ih0 + i) < (unsigned)p.IH) ? rv : WD_OOR;
                 colterm[i] = ((unsigned)(iw0 + i) < (unsigned)p.IW) ? cv : WD_OOR_COL;
             }
@@ -164,9 +163,9 @@ __global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
         };
         request(Set0{});
         transform(Set0{}, 0, true);   // chunk 0, waited for
-        advance_tile();
+        cur_advance(cur);
         request(Set1{});              // chunk 1
-        advance_tile();
+        cur_advance(cur);
         request(Set0{});              // chunk 2
         __syncthreads();
         // chunk c: chunk c+1 (requested two chunks ago) is transformed into the other buffer, chunk c+3 requested into the
@@ -174,108 +173,119 @@ __global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
         // even when that chunk does not exist (only its LDS writes and its barrier are skipped).
         for (int c = 0; c < nchunks; c += 2) {
             transform(Set1{}, 1, true);
-            advance_tile();
+            cur_advance(cur);
             request(Set1{});
             __syncthreads();
             const bool more = c + 1 < nchunks;
             transform(Set0{}, 0, more);
-            advance_tile();
-            request(Set0{});
-            if (more) __syncthreads();
-        }
-        return;
-    }
-    if (t >= 256) {
-        if (nchunks == 0) return;
-        floatx4 yr[2][2][2];   // raw deltaY tiles
-        const int y_px = p.OC, y_row = p.OW * p.OC;
-        auto request = [&](auto set_c) {
-            constexpr int SET = decltype(set_c)::value;
-            const bool ok = tile_cur < tile_end && yc_ok;
-            const bool right = 2 * tx + 1 < p.OW, below = 2 * ty + 1 < p.OH;
-            const unsigned o = (unsigned)y00 * 4u;
-            const unsigned o00 = ok ? o : WD_OOR, o01 = (ok && right) ? o + (unsigned)y_px * 4u : WD_OOR;
-            const unsigned o10 = (ok && below) ? o + (unsigned)y_row * 4u : WD_OOR;
-            const unsigned o11 = (ok && right && below) ? o + (unsigned)(y_row + y_px) * 4u : WD_OOR;
-            yr[SET][0][0] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, o00, 0, 0));
-            yr[SET][0][1] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, o01, 0, 0));
-            yr[SET][1][0] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, o10, 0, 0));
-            yr[SET][1][1] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, o11, 0, 0));
-        };
-        // Yh' = G' y G'^T per channel with G' = [[1,0],[1,1],[1,-1],[0,1]] = G without its factors 1/2, which are applied to
-        // the accumulators once, at the end
-        auto transform = [&](auto set_c, int buf, bool store) {
-            constexpr int SET = decltype(set_c)::value;
-            float *Yh = smem + buf * WD_BUF + WD_XBUF + (st * 64 + y_ch) * WD_CS;
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const float y00v = yr[SET][0][0][k], y01v = yr[SET][0][1][k], y10v = yr[SET][1][0][k], y11v = yr[SET][1][1][k];
-                float g[4][2];
-                g[0][0] = y00v; g[0][1] = y01v;
-                g[1][0] = y00v + y10v; g[1][1] = y01v + y11v;
-                g[2][0] = y00v - y10v; g[2][1] = y01v - y11v;
-                g[3][0] = y10v; g[3][1] = y11v;
-                if (store) {
-#pragma unroll
-                    for (int a = 0; a < 4; a++)
-                        *reinterpret_cast<floatx4 *>(Yh + k * WD_CS + ((a ^ swz_wy) << 2)) =
-                            floatx4{g[a][0], g[a][0] + g[a][1], g[a][0] - g[a][1], g[a][1]};
-                }
-            }
-        };
-        request(Set0{});
-        transform(Set0{}, 0, true);
-        advance_tile();
-        request(Set1{});
-        advance_tile();
-        request(Set0{});
-        __syncthreads();
-        for (int c = 0; c < nchunks; c += 2) {
-            transform(Set1{}, 1, true);
-            advance_tile();
-            request(Set1{});
-            __syncthreads();
-            const bool more = c + 1 < nchunks;
-            transform(Set0{}, 0, more);
-            advance_tile();
+            cur_advance(cur);
             request(Set0{});
             if (more) __syncthreads();
         }
         return;
     }
 
+    // ---- wavefronts 0-3 multiply. deltaY does not go through LDS: wavefront w is the only one that needs output channels
+    //      [16w, 16w+16), so lane (l16, q) loads the 2x2 tiles of channel 16w + l16 for its two tiles of a chunk (q and
+    //      4 + q) itself, two chunks ahead, and transforms them in registers into the 32 MFMA operands of the chunk. The
+    //      patches come from LDS. ------------------------------------------------------------------------------------------
     if (nchunks > 0) {
-        // One chunk = 8 groups of 8 MFMAs: (4 tiles kk, 4 xi) x (two blocks of input channels); three 128-bit LDS reads per
-        // group, one group ahead. The two MFMAs into one accumulator (kk = 0, 1) are 4 groups apart.
-        int rdx0[4], rdx1[4], rdy[4];   // float offsets of this lane's operands for xi group gx (tile q; channels l16, 16 + l16, 16w + l16)
+        const int y_ch = oc0 + 16 * w + l16;
+        const bool yc_ok = y_ch < p.OC;
+        const int y_px = p.OC, y_row = p.OW * p.OC;
+        TileCur ca, cb;
+        cur_init(ca, tile_begin + q, 0, y_ch);
+        cur_init(cb, tile_begin + 4 + q, 0, y_ch);
+        float yraw[2][2][4];   // [set][kk][pixel]
+        auto request_one = [&](const TileCur &c, float (&y)[4]) {
+            const bool ok = c.tile < tile_end && yc_ok;
+            const bool right = 2 * c.tx + 1 < p.OW, below = 2 * c.ty + 1 < p.OH;
+            const unsigned o = (unsigned)c.y00 * 4u;
+            const unsigned o00 = ok ? o : WD_OOR, o01 = (ok && right) ? o + (unsigned)y_px * 4u : WD_OOR;
+            const unsigned o10 = (ok && below) ? o + (unsigned)y_row * 4u : WD_OOR;
+            const unsigned o11 = (ok && right && below) ? o + (unsigned)(y_row + y_px) * 4u : WD_OOR;
+            y[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o00, 0, 0));
+            y[1] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o01, 0, 0));
+            y[2] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o10, 0, 0));
+            y[3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o11, 0, 0));
+        };
+        auto request = [&](auto set_c) {
+            constexpr int SET = decltype(set_c)::value;
+            request_one(ca, yraw[SET][0]);
+            request_one(cb, yraw[SET][1]);
+        };
+        // Yh' = G' y G'^T with G' = [[1,0],[1,1],[1,-1],[0,1]] = G without its factors 1/2, which are applied to the
+        // accumulators once, at the end
+        float ya[2][16];
+        auto transform = [&](auto set_c) {
+            constexpr int SET = decltype(set_c)::value;
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                const float y00v = yraw[SET][kk][0], y01v = yraw[SET][kk][1], y10v = yraw[SET][kk][2], y11v = yraw[SET][kk][3];
+                float g[4][2];
+                g[0][0] = y00v; g[0][1] = y01v;
+                g[1][0] = y00v + y10v; g[1][1] = y01v + y11v;
+                g[2][0] = y00v - y10v; g[2][1] = y01v - y11v;
+                g[3][0] = y10v; g[3][1] = y11v;
+#pragma unroll
+                for (int a = 0; a < 4; a++) {
+                    ya[kk][4 * a + 0] = g[a][0];
+                    ya[kk][4 * a + 1] = g[a][0] + g[a][1];
+                    ya[kk][4 * a + 2] = g[a][0] - g[a][1];
+                    ya[kk][4 * a + 3] = g[a][1];
+                }
+            }
+        };
+        int rdx0[4], rdx1[4];   // float offsets of this lane's patch operands for xi group gx (tile q; channels l16, 16 + l16)
 #pragma unroll
         for (int gx = 0; gx < 4; gx++) {
             rdx0[gx] = (q * 32 + l16) * WD_CS + (gx << 2);
             rdx1[gx] = (q * 32 + 16 + l16) * WD_CS + ((gx ^ 1) << 2);
-            rdy[gx] = WD_XBUF + (q * 64 + 16 * w + l16) * WD_CS + ((gx ^ w) << 2);
         }
-        __syncthreads();
-        for (int c = 0; c < nchunks; c++) {
-            const float *B = smem + (c & 1) * WD_BUF;
-            auto frag = [&](int g, floatx4 &fa, floatx4 &fb0, floatx4 &fb1) {
+        // One chunk = 8 groups of 8 MFMAs: (4 tiles kk, 4 xi) x (two blocks of input channels); two 128-bit LDS reads per
+        // group, one group ahead. The two MFMAs into one accumulator (kk = 0, 1) are 4 groups apart.
+        auto multiply = [&](int buf) {
+            const float *B = smem + buf * WD_BUF;
+            auto frag = [&](int g, floatx4 &fb0, floatx4 &fb1) {
                 const int kk = g >> 2, gx = g & 3;
-                fa = *reinterpret_cast<const floatx4 *>(B + rdy[gx] + kk * 4 * 64 * WD_CS);
                 fb0 = *reinterpret_cast<const floatx4 *>(B + rdx0[gx] + kk * 4 * 32 * WD_CS);
                 fb1 = *reinterpret_cast<const floatx4 *>(B + rdx1[gx] + kk * 4 * 32 * WD_CS);
             };
-            floatx4 a[2], b0[2], b1[2];
-            frag(0, a[0], b0[0], b1[0]);
+            floatx4 b0[2], b1[2];
+            frag(0, b0[0], b1[0]);
 #pragma unroll
             for (int g = 0; g < 8; g++) {
-                if (g + 1 < 8) frag(g + 1, a[(g + 1) & 1], b0[(g + 1) & 1], b1[(g + 1) & 1]);
+                if (g + 1 < 8) frag(g + 1, b0[(g + 1) & 1], b1[(g + 1) & 1]);
 #pragma unroll
                 for (int x = 0; x < 4; x++) {
                     const int xi = 4 * (g & 3) + x;
-                    acc[xi][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g & 1][x], b0[g & 1][x], acc[xi][0], 0, 0, 0);
-                    acc[xi][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[g & 1][x], b1[g & 1][x], acc[xi][1], 0, 0, 0);
+                    const float a = ya[g >> 2][xi];
+                    acc[xi][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b0[g & 1][x], acc[xi][0], 0, 0, 0);
+                    acc[xi][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b1[g & 1][x], acc[xi][1], 0, 0, 0);
                 }
             }
+        };
+        request(Set0{});       // chunk 0
+        cur_advance(ca);
+        cur_advance(cb);
+        request(Set1{});       // chunk 1
+        __syncthreads();
+        for (int c = 0; c < nchunks; c += 2) {
+            transform(Set0{});
+            cur_advance(ca);
+            cur_advance(cb);
+            request(Set0{});   // chunk c + 2
+            multiply(0);
             __syncthreads();
+            const bool more = c + 1 < nchunks;
+            transform(Set1{});
+            cur_advance(ca);
+            cur_advance(cb);
+            request(Set1{});   // chunk c + 3
+            if (more) {
+                multiply(1);
+                __syncthreads();
+            }
         }
     }
 
@@ -352,7 +362,7 @@ hipError_t launch_deltaW_winograd(hipStream_t stream, const float *X, const floa
     constexpr auto kern = winograd_dw_kernel;
     const size_t lds = (size_t)2 * WD_BUF * sizeof(float);
     if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((IC + 31) / 32, (OC + 63) / 64, GZ), dim3(512), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3((IC + 31) / 32, (OC + 63) / 64, GZ), dim3(384), lds, stream, a);
     return hipGetLastError();
 }
 
