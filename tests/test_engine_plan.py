@@ -145,3 +145,40 @@ def test_w1_entries_only_for_stride_one_and_sizes_are_checked():
     assert "padding" in E.param_check(28, 28, 56, 56, 3, 3, 64, 64, 128, 2, 2, 3, 1)                           # FH <= ph
     assert "multiples of 4" in E.param_check(28, 28, 56, 56, 3, 3, 64, 62, 128, 2, 2, 1, 1)
     assert "stride" in E.param_check(28, 28, 56, 56, 3, 3, 64, 64, 128, 0, 2, 1, 1)
+
+
+def test_winograd_backward_flags_change_only_3x3_stride1_plans():
+    """This build's options deltaX_winograd / deltaW_winograd (no reference counterpart): off by default; on, they take
+    3x3 stride-1 layers only, with scratch 16*IC*OC for backward-data and a split-K factor sized for the device for
+    backward-filter (values above 1 = compute units to fill; 32 x 64 channel blocks; slices of at least 64 tiles)."""
+    cfg = E.default_config(256)
+    assert cfg.deltaX_winograd == 0 and cfg.deltaW_winograd == 0
+    ref_dx = E.plan_deltaX(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).entry_name
+    ref_dw = E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1)
+    cfg.deltaX_winograd = 1
+    p = E.plan_deltaX(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1)
+    assert p.entry_name == "dconv3D_deltaX_winograd" and p.scratch_floats == 16 * 64 * 64 and p.streams == 1
+    assert E.plan_deltaX(cfg, 56, 56, 28, 28, 3, 3, 32, 64, 128, 2, 2).entry_name != "dconv3D_deltaX_winograd"   # stride 2
+    assert E.plan_deltaX(cfg, 56, 56, 56, 56, 1, 1, 32, 256, 64, 1, 1).entry_name == "dconv3D_deltaX_W1"          # 1x1
+    assert E.plan_deltaX(cfg, 32, 32, 32, 32, 3, 3, 4, 4, 64, 1, 1).entry_name == "dconv3D_deltaX_crossAdd"       # IC <= 8
+    cfg.deltaX_winograd = 0
+    assert E.plan_deltaX(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).entry_name == ref_dx
+
+    cfg.deltaW_winograd = 1   # the reference's GridZ
+    p = E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1)
+    assert p.entry_name == "dconv3D_deltaW_GemmSK_winograd" and p.GridZ == ref_dw.GridZ
+    assert p.scratch_floats == 64 * 9 * 64 * (p.GridZ - 1)
+    cfg.deltaW_winograd = 256   # c5b: 2 x 1 channel blocks -> 128 slices of 196 tiles
+    p = E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1)
+    assert p.GridZ == 128 and p.scratch_floats == 64 * 9 * 64 * 127
+    # c2c: 8 x 4 channel blocks -> 8 slices; 2048 tiles / 64 = 32 would allow more
+    assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 128, 256, 256, 1, 1).GridZ == 8
+    # below the split-K threshold (N*OH*OW = 256 < 512) the reference's plain entry stays
+    p = E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 4, 64, 64, 1, 1)
+    assert p.entry_name == "dconv3D_deltaW" and p.GridZ == 1
+    # 16 images of 8x8: 256 tiles, at most 4 slices of 64 tiles although 256 units / 2 channel blocks would ask for 128
+    assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 16, 64, 64, 1, 1).GridZ == 4
+    assert E.plan_deltaW(cfg, 56, 56, 28, 28, 3, 3, 32, 64, 128, 2, 2).entry_name != "dconv3D_deltaW_GemmSK_winograd"
+    assert E.plan_deltaW(cfg, 56, 56, 56, 56, 1, 1, 32, 256, 64, 1, 1).entry_name == "dconv3D_deltaW_GemmSK_W1"
+    cfg.deltaW_winograd = 0
+    assert E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).entry_name == ref_dw.entry_name
