@@ -334,4 +334,20 @@ def test_engine_random_3x3_stride1_layers(dev, eng, case):
     check(dev.get(y_w), want, "conv3D from W %s" % (case,))
     check(dev.get(dx), O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw), "deltaX %s" % (case,))
     check(dev.get(dw), O.deltaW_f64(X, dY, 3, 3, 1, 1, ph, pw), "deltaW %s" % (case,))
+    # the same layer through this build's three Winograd paths
+    y2, dx2, dw2 = dev.guarded(N, OH, OW, OC), dev.guarded(N, IH, IW, IC), dev.guarded(OC, 3, 3, IC)
+    eng.config.conv3D_winograd, eng.config.deltaX_winograd, eng.config.deltaW_winograd = 1, 1, 40
+    try:
+        p1 = eng.conv3D(y2.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, ph, pw)
+        p2 = eng.dconv3D_deltaX(dx2.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, ph, pw)
+        p3 = eng.dconv3D_deltaW(dw2.data_ptr(), 3, 3, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, 1, 1, ph, pw)
+        eng.sync()
+    finally:
+        eng.config.conv3D_winograd, eng.config.deltaX_winograd, eng.config.deltaW_winograd = 0, 0, 0
+    assert p1.entry_name == "conv3D_winograd" and p2.entry_name == "dconv3D_deltaX_winograd"
+    check(dev.get(y2), want, "Winograd conv3D %s" % (case,))
+    check(dev.get(dx2), O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw), "Winograd deltaX %s" % (case,))
+    if N * OH * OW >= 512:   # below the split-K threshold the plain entry stays
+        assert p3.entry_name == "dconv3D_deltaW_GemmSK_winograd"
+    check(dev.get(dw2), O.deltaW_f64(X, dY, 3, 3, 1, 1, ph, pw), "Winograd deltaW %s" % (case,))
 
