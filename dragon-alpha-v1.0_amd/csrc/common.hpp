@@ -1,6 +1,7 @@
 // Shared declarations of the gfx950 conv kernels: launch-argument structs, exact integer
 // division by launch-time constants, and the host-side launcher prototypes called by the C ABI.
 #pragma once
+#include "winograd_limits.hpp"
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -150,9 +151,7 @@ hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, 
 hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
                                    int GK, int IC, int OC, int GK_slice, int GZ, float *dB = nullptr, float *dB_buf = nullptr);
 
-// Which of the two layouts of the transformed filter a layer uses (a function of IC alone: the transform does not know
-// the rest of the layer): grouped U[16][IC/4][OC][4] for the persistent kernel, else U[16][IC][OC].
-inline bool winograd_grouped_filter(int IC) { return IC >= 16 && IC % 16 == 0; }
+// winograd_grouped_filter(IC) and the size limits of the Winograd kernels: winograd_limits.hpp
 // backward: the filter of backward-data as a forward convolution of deltaY (OC reduced, IC produced, taps rotated);
 // launch_winograd(deltaY, U, deltaX, N, OH, OW, OC, IH, IW, IC, 2 - ph, 2 - pw) then computes deltaX.
 hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC, bool backward = false);

@@ -7,6 +7,7 @@
 // then call the natives exactly as the Java code does).
 #include "../../include/alpha_conv.h"
 #include "../../include/alpha_engine.h"
+#include "winograd_limits.hpp"
 
 #include <hip/hip_runtime.h>
 
@@ -74,11 +75,11 @@ void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
 void alpha_plan_conv3D(const alpha_engine_config *c, int IH, int IW, int OH, int OW, int FH, int FW, int N, int IC, int OC,
                        int sh, int sw, int ph, int pw, alpha_conv_plan *out)
 {
-    (void)IC;
     memset(out, 0, sizeof(*out));
     const double Q = alpha_paddingScaleUp(IH, IW, OH, OW, FH, FW, sh, sw);
     out->Q = Q;
-    if (c->conv3D_winograd && FH == 3 && FW == 3 && sh == 1 && sw == 1) {
+    // a layer beyond the Winograd kernels' 32-bit offsets stays on the entries below
+    if (c->conv3D_winograd && FH == 3 && FW == 3 && sh == 1 && sw == 1 && alpha::winograd_forward_fits(N, IH, IW, IC, OH, OW, OC)) {
         out->entry = ALPHA_E_conv3D_winograd;
         out->remode = 1;   // the filter transform takes the place of kernel_remode
         out->streams = 1;
@@ -151,7 +152,8 @@ void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int
         if (want > GridZ2) want = GridZ2;
         if (want > GridZ) GridZ = want;
     }
-    const bool winograd = c->deltaW_winograd && FH == 3 && FW == 3 && sh == 1 && sw == 1;
+    const bool winograd = c->deltaW_winograd && FH == 3 && FW == 3 && sh == 1 && sw == 1 &&
+                          alpha::winograd_deltaW_fits(N, IH, IW, IC, OH, OW, OC);
     if (winograd && c->deltaW_winograd > 1) {
         // One workgroup of the Winograd kernel covers 32 input x 64 output channels of one slice of tiles and has a
         // compute unit to itself: values above 1 are the number of compute units to fill (slices of at least 64 tiles).
@@ -189,7 +191,8 @@ void alpha_plan_deltaX(const alpha_engine_config *c, int IH, int IW, int OH, int
         out->streams = stream_count(IC, N * IH * IW, 10);
         return;
     }
-    if (c->deltaX_winograd && sh == 1 && sw == 1 && FH == 3 && FW == 3 && OH - IH + 2 <= 4 && OW - IW + 2 <= 4) {   // padding <= 2
+    if (c->deltaX_winograd && sh == 1 && sw == 1 && FH == 3 && FW == 3 && OH - IH + 2 <= 4 && OW - IW + 2 <= 4 &&   // padding <= 2
+        alpha::winograd_forward_fits(N, OH, OW, OC, IH, IW, IC)) {
         out->entry = ALPHA_E_dconv3D_deltaX_winograd;
         out->streams = 1;
         out->scratch_floats = 16L * IC * OC;

@@ -278,6 +278,7 @@ hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, f
                            int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias)
 {
     if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
+    if (!winograd_forward_fits(N, IH, IW, IC, OH, OW, OC)) return hipErrorNotSupported;
     if (winograd_grouped_filter(IC))   // the persistent variant and its filter layout; no other kernel reads that layout
         return launch_winograd_stream(stream, X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, bias);
     WinoArgs a{};

@@ -329,6 +329,7 @@ hipError_t launch_deltaW_winograd(hipStream_t stream, const float *X, const floa
 {
     if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
     if (IC < 4 || OC < 4 || (OC & 3) || N < 1 || OH < 1 || OW < 1 || GZ < 1) return hipErrorNotSupported;
+    if (!winograd_deltaW_fits(N, IH, IW, IC, OH, OW, OC)) return hipErrorNotSupported;
     const long x_bytes = (long)N * IH * IW * IC * 4, y_bytes = (long)N * OH * OW * OC * 4;
     // the patch offsets are sums of a row term and a column term that mark "outside" by 2 GB and 1 GB: X must end below 1 GB
     if (x_bytes + 8L * IC > (1L << 30) || y_bytes >= (1L << 31)) return hipErrorNotSupported;

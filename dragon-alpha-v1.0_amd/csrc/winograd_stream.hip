@@ -322,6 +322,7 @@ hipError_t launch_winograd_stream(hipStream_t stream, const float *X, const floa
 {
     if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
     if (IC < 16 || IC % 16 != 0 || OC < 1 || N < 1 || OH < 1 || OW < 1) return hipErrorNotSupported;
+    if (!winograd_forward_fits(N, IH, IW, IC, OH, OW, OC)) return hipErrorNotSupported;
     const long x_bytes = (long)N * IH * IW * IC * 4, y_bytes = (long)N * OH * OW * OC * 4, u_bytes = 16L * IC * OC * 4;
     if (x_bytes >= (1L << 31) || y_bytes > (1L << 30) || u_bytes >= (1L << 31)) return hipErrorNotSupported;
     const int cus = device_cu_count();

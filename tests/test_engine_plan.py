@@ -182,3 +182,26 @@ def test_winograd_backward_flags_change_only_3x3_stride1_plans():
     assert E.plan_deltaW(cfg, 56, 56, 56, 56, 1, 1, 32, 256, 64, 1, 1).entry_name == "dconv3D_deltaW_GemmSK_W1"
     cfg.deltaW_winograd = 0
     assert E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).entry_name == ref_dw.entry_name
+
+
+def test_winograd_flags_leave_layers_beyond_32bit_offsets_on_the_default_entries():
+    """The Winograd kernels address with 32-bit offsets that keep the top bits for "outside" marks: the persistent forward
+    kernel needs the output within 1 GB (input and transformed filter within 2 GB), the backward-filter kernel X within
+    1 GB. With the flags set, a layer beyond that keeps the plan it has without them instead of failing at the call."""
+    cfg = E.default_config(256)
+    big = (128, 128, 128, 128, 3, 3, 64, 256, 256, 1, 1)      # X = Y = 1 GiB exactly
+    bigger = (128, 128, 128, 128, 3, 3, 64, 256, 512, 1, 1)   # Y = 2 GiB
+    ref = {k: (E.plan_conv3D(cfg, *k[:11], 1, 1).entry_name, E.plan_deltaX(cfg, *k).entry_name, E.plan_deltaW(cfg, *k).entry_name)
+           for k in (big, bigger)}
+    cfg.conv3D_winograd, cfg.deltaX_winograd, cfg.deltaW_winograd = 1, 1, 256
+    # 1 GiB output fits the forward kernel (limit inclusive); X + one pixel beyond 1 GiB does not fit backward-filter
+    assert E.plan_conv3D(cfg, *big, 1, 1).entry_name == "conv3D_winograd"
+    assert E.plan_deltaX(cfg, *big).entry_name == "dconv3D_deltaX_winograd"
+    assert E.plan_deltaW(cfg, *big).entry_name == ref[big][2]
+    # 2 GiB of Y: forward output too large, backward-data input too large, backward-filter deltaY too large
+    assert E.plan_conv3D(cfg, *bigger, 1, 1).entry_name == ref[bigger][0]
+    assert E.plan_deltaX(cfg, *bigger).entry_name == ref[bigger][1]
+    assert E.plan_deltaW(cfg, *bigger).entry_name == ref[bigger][2]
+    # just inside: half the images
+    inside = (128, 128, 128, 128, 3, 3, 32, 256, 256, 1, 1)
+    assert E.plan_deltaW(cfg, *inside).entry_name == "dconv3D_deltaW_GemmSK_winograd"
