@@ -49,6 +49,28 @@ constexpr int TC_ICC = 64;            // input channels per halo pass
 constexpr int TC_PS = TC_ICC + 8;     // LDS pixel stride (floats)
 constexpr int TC_OS = 64 + 4;         // output staging row stride (floats)
 
+// Where a lane reads its filter fragment: element index = half-tap base (uniform) + lane offset. The three functions
+// below are the whole address computation of the filter loads, shared by the kernel and by the host-side walk
+// alpha_selfcheck_tap_filter_extent, which the CPU tests use to prove that no load leaves the filter.
+// RAGGED: the second half tap of the last pass may start at or beyond AC (AC % 64 in [4, 32]); every lane of such a
+// half tap is masked, and its base is pulled back to the last channel quad so that the masked lanes' address
+// (base + 0) stays inside the filter.
+template <bool RAGGED>
+__host__ __device__ __forceinline__ int tap_filter_half_tap_base(int b_off, int b_sth, int b_stw, int b_sc, int AC, int icbase, int th, int tw)
+{
+    const int icb = RAGGED ? (icbase < AC - 4 ? icbase : AC - 4) : icbase;
+    return b_off + th * b_sth + tw * b_stw + icb * b_sc;
+}
+template <bool RAGGED>
+__host__ __device__ __forceinline__ unsigned tap_filter_lane_mask(int AC, int icbase, int g, int q)
+{
+    return RAGGED ? (unsigned)-(int)(icbase + 16 * g + 4 * q < AC) : ~0u;
+}
+__host__ __device__ __forceinline__ unsigned tap_filter_lane_bytes(int b_sc, int g, int q, int s, int co)
+{
+    return (unsigned)(((16 * g + 4 * q + s) * b_sc + co) * 4);
+}
+
 // RAGGED: AC is not a multiple of 64, so the last pass has channels beyond AC whose filter fragments
 // must be zeroed (kept out of the common case: the extra selects would pull the wait for the
 // prefetched fragment in front of the MFMAs).
@@ -99,14 +121,14 @@ __device__ __forceinline__ void tap_conv_unit(const TapConvArgs &p, float *smem,
 #pragma unroll
     for (int g = 0; g < 2; g++)
 #pragma unroll
-        for (int s = 0; s < 4; s++) b_lane[g][s] = (unsigned)(((16 * g + 4 * q + s) * p.b_sc + (b_cov ? b_co : 0)) * 4);
+        for (int s = 0; s < 4; s++) b_lane[g][s] = tap_filter_lane_bytes(p.b_sc, g, q, s, b_cov ? b_co : 0);
     auto load_b = [&](float (&b)[2][4], int icbase, int th, int tw) {
-        const int sbase = __builtin_amdgcn_readfirstlane(p.b_off + th * p.b_sth + tw * p.b_stw + icbase * p.b_sc);
+        const int sbase = __builtin_amdgcn_readfirstlane(tap_filter_half_tap_base<RAGGED>(p.b_off, p.b_sth, p.b_stw, p.b_sc, p.AC, icbase, th, tw));
         const char *sb = reinterpret_cast<const char *>(p.B + sbase);
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             // RAGGED: channels beyond AC (AC % 4 == 0: four at a time) are fetched from the half tap's first element
-            const unsigned ok = RAGGED ? (unsigned)-(int)(icbase + 16 * g + 4 * q < p.AC) : ~0u;
+            const unsigned ok = tap_filter_lane_mask<RAGGED>(p.AC, icbase, g, q);
 #pragma unroll
             for (int s = 0; s < 4; s++) {
                 if (!RAGGED) asm volatile("" : "+v"(b_lane[g][s]));   // value unchanged
@@ -457,3 +479,52 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
 }
 
 }  // namespace alpha
+
+// Host-side walk over every filter address tap_conv_kernel generates for one block of 64 output channels per lane
+// (same loop structure as tap_conv_unit: first half tap, then per tap the second half tap and the next tap's first
+// one), using the kernel's own address functions. Writes the smallest and largest element index read.
+#pragma GCC visibility push(default)
+extern "C" int alpha_selfcheck_tap_filter_extent(int AC, int CO, int TH, int TW, int b_off, int b_sth, int b_stw, int b_sc,
+                                                 long *lo_out, long *hi_out)
+{
+    using namespace alpha;
+    if (AC < 4 || (AC & 3) || CO < 4 || TH < 1 || TW < 1 || !lo_out || !hi_out) return -1;
+    const bool ragged = (AC % TC_ICC) != 0;
+    long lo = (1L << 62), hi = -(1L << 62);
+    auto visit = [&](int icbase, int th, int tw) {
+        const int sbase = ragged ? tap_filter_half_tap_base<true>(b_off, b_sth, b_stw, b_sc, AC, icbase, th, tw)
+                                 : tap_filter_half_tap_base<false>(b_off, b_sth, b_stw, b_sc, AC, icbase, th, tw);
+        for (int oc0 = 0; oc0 < CO; oc0 += 64)
+            for (int w = 0; w < 4; w++)
+                for (int lane = 0; lane < 64; lane++) {
+                    const int l16 = lane & 15, q = lane >> 4;
+                    const int b_co = oc0 + 16 * w + l16;
+                    const int co = b_co < CO ? b_co : 0;
+                    for (int g = 0; g < 2; g++) {
+                        const unsigned ok = ragged ? tap_filter_lane_mask<true>(AC, icbase, g, q) : tap_filter_lane_mask<false>(AC, icbase, g, q);
+                        for (int s = 0; s < 4; s++) {
+                            const long idx = (long)sbase + (long)((tap_filter_lane_bytes(b_sc, g, q, s, co) & ok) / 4);
+                            if (idx < lo) lo = idx;
+                            if (idx > hi) hi = idx;
+                        }
+                    }
+                }
+    };
+    visit(0, 0, 0);
+    const int taps = TH * TW;
+    for (int ic0 = 0; ic0 < AC; ic0 += TC_ICC) {
+        int th = 0, tw = 0;
+        for (int tap = 0; tap < taps; tap++) {
+            int nth = th, ntw = tw + 1, nic = ic0;
+            if (ntw == TW) { ntw = 0; nth = th + 1; }
+            if (tap + 1 == taps) { nth = 0; ntw = 0; nic = ic0 + TC_ICC < AC ? ic0 + TC_ICC : ic0; }
+            visit(ic0 + 32, th, tw);
+            visit(nic, nth, ntw);
+            th = nth; tw = ntw;
+        }
+    }
+    *lo_out = lo;
+    *hi_out = hi;
+    return 0;
+}
+#pragma GCC visibility pop

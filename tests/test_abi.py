@@ -84,3 +84,31 @@ def test_argument_validation_without_gpu():
     assert rc == 10001 and b"deltaW_buf" in L.alpha_conv_last_error()
     with pytest.raises(pkg.AlphaConvError):
         pkg.Cuda_conv3D.kernel_remode(0, 0, 0, 3, 3, 8, 4)
+
+
+def _tap_filter_extent(AC, CO, TH, TW, b_off, b_sth, b_stw, b_sc):
+    L = pkg.lib()
+    fn = L.alpha_selfcheck_tap_filter_extent
+    fn.argtypes = [ctypes.c_int] * 8 + [ctypes.POINTER(ctypes.c_long)] * 2
+    fn.restype = ctypes.c_int
+    lo, hi = ctypes.c_long(), ctypes.c_long()
+    assert fn(AC, CO, TH, TW, b_off, b_sth, b_stw, b_sc, ctypes.byref(lo), ctypes.byref(hi)) == 0
+    return lo.value, hi.value
+
+
+@pytest.mark.parametrize("AC", [32, 36, 64, 68, 80, 92, 96, 100, 128, 160, 196])
+@pytest.mark.parametrize("CO", [4, 20, 64, 100])
+@pytest.mark.parametrize("TH,TW", [(3, 3), (5, 3), (2, 2), (7, 7), (1, 1)])
+def test_tap_conv_filter_loads_stay_inside_the_filter(AC, CO, TH, TW):
+    """The library walks the filter addresses of the LDS-halo kernel with the kernel's own address functions
+    (same loop structure: the second half tap of every tap and the prefetch of the next). Every element index must lie
+    inside the filter for both layouts the kernel is given: CW[TH,TW,AC,CO] (forward) and W[AC,TH,TW,CO] read in place
+    with rotated taps (backward-data: reduced channel = OC of W, produced channel = IC of W). Channel counts with
+    AC % 64 in [4, 32] are the ones whose last pass has an all-masked second half tap."""
+    size = TH * TW * AC * CO
+    lo, hi = _tap_filter_extent(AC, CO, TH, TW, 0, TW * AC * CO, AC * CO, CO)
+    assert 0 <= lo and hi < size, ("CW", lo, hi, size)
+    lo, hi = _tap_filter_extent(AC, CO, TH, TW, ((TH - 1) * TW + (TW - 1)) * CO, -TW * CO, -CO, TH * TW * CO)
+    assert 0 <= lo and hi < size, ("W rotated", lo, hi, size)
+    if AC % 64 == 0 and CO % 64 == 0:   # nothing is masked or clamped: the walk touches the first and the last element
+        assert (lo, hi) == (0, size - 1)
