@@ -4,6 +4,7 @@
 #include "../../include/alpha_conv.h"
 #include "common.hpp"
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -234,6 +235,38 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     return hip_status(launch_deltaW(stream0(streams), a), fn);
 }
 
+// ---- split-K partial sums in device memory that belongs to the library ---------------------------------------------
+// For callers that cannot allocate (HIP graph capture, serving loops, harnesses that forbid hipMalloc): the partial
+// sums of alpha_dconv3D_deltaW_GemmSK_static live in this file-scope array instead of a deltaW_buf from the caller.
+// Every device that loads the library holds its own copy until the process ends. In host code the array's name is
+// only a handle: its device address is asked for once per device (with that device current) and kept here.
+constexpr size_t STATIC_SCRATCH_FLOATS = ALPHA_CONV_STATIC_SCRATCH_BYTES / sizeof(float);
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<float *> g_scratch_ptr[MAX_DEVICES];
+
+// Device address of `scratch` on the current device, or nullptr with the error recorded.
+float *static_scratch(const char *fn)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { hip_status(e, fn); return nullptr; }
+    if (dev < 0 || dev >= MAX_DEVICES) { fail(ALPHA_CONV_EINVAL, "%s: device index %d out of range", fn, dev); return nullptr; }
+    float *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {   // a racing first call asks twice and stores the same address
+        void *sym = nullptr;
+        e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || sym == nullptr) {
+            fail(e != hipSuccess ? (int)e : ALPHA_CONV_EINVAL, "%s: hipGetSymbolAddress(scratch): %s", fn, hipGetErrorString(e));
+            return nullptr;
+        }
+        ptr = static_cast<float *>(sym);
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    return ptr;
+}
+
 }  // namespace
 
 #pragma GCC visibility push(default)
@@ -250,6 +283,9 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz)
     if (int e = hip_status(hipDeviceGetAttribute(&clk, hipDeviceAttributeClockRate, dev), __func__)) return e;
     if (compute_units) *compute_units = cu;
     if (clock_khz) *clock_khz = clk;
+    // the per-device set-up call of the library: also resolves this device's copy of the static scratch array, so that a
+    // caller who asks for the device first never triggers that lookup inside a captured region
+    if (static_scratch(__func__) == nullptr) return ALPHA_CONV_EINVAL;
     return 0;
 }
 
@@ -438,6 +474,31 @@ int alpha_dconv3D_deltaW_GemmSK_W1(const int64_t *streams, int length, int GridZ
                                    const float *deltaY, float *deltaW, float *deltaW_buf, int N, int IC, int OC)
 {
     return deltaW_impl(__func__, streams, length, GridZ, X, IH, IW, deltaY, IH, IW, deltaW, deltaW_buf, 1, 1, N, IC, OC, 1, 1, 0, 0);
+}
+
+// Split-K backward-filter that allocates nothing and takes no workspace: the GridZ - 1 partial results go to the
+// library's static array, and the Kahan sum over them (buf_summary) is enqueued behind the split-K kernel on streams[0],
+// so deltaW is complete when the stream reaches the end of this call's work. Same kernels, slices and summation order as
+// alpha_dconv3D_deltaW_GemmSK followed by alpha_buf_summary: the results are bit-identical to that pair.
+// Every slice's kernel overwrites its whole partial tensor (empty slices write zeros), so nothing of an earlier call
+// is read. All calls on one device share the array: two calls whose work overlaps in time on one device race.
+int alpha_dconv3D_deltaW_GemmSK_static(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
+                                       const float *deltaY, int OH, int OW, float *deltaW, int FH, int FW,
+                                       int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    CHECK_STREAMS();
+    if (GridZ < 1) return fail(ALPHA_CONV_EINVAL, "%s: GridZ must be >= 1", __func__);
+    if (int e = check_dims(__func__, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
+    const size_t sizeW = (size_t)OC * FH * FW * IC, need = (size_t)(GridZ - 1) * sizeW;
+    if (need > STATIC_SCRATCH_FLOATS)
+        return fail(ALPHA_CONV_EINVAL, "%s: (GridZ - 1) * OC*FH*FW*IC = %zu floats of partial sums exceed the static scratch of %zu floats; "
+                                       "lower GridZ or use alpha_dconv3D_deltaW_GemmSK with a deltaW_buf", __func__, need, STATIC_SCRATCH_FLOATS);
+    float *buf = static_scratch(__func__);
+    if (buf == nullptr) return ALPHA_CONV_EINVAL;
+    if (int e = deltaW_impl(__func__, streams, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, buf, FH, FW, N, IC, OC, sh, sw, ph, pw))
+        return e;
+    if (GridZ == 1) return 0;
+    return hip_status(launch_buf_summary(stream0(streams), buf, deltaW, GridZ - 1, (int)sizeW), __func__);
 }
 
 // ---- Winograd F(2x2,3x3): additional forward algorithm of this build ----------------------------------------

@@ -52,6 +52,7 @@ _SIGS = {
     "alpha_dconv3D_deltaW_GemmSK": "siipiipiippiiiiiiiii",
     "alpha_dconv3D_deltaW_GemmV2SK": "siipiipiippiiiiiiiii",
     "alpha_dconv3D_deltaW_GemmSK_W1": "siipiipppiii",
+    "alpha_dconv3D_deltaW_GemmSK_static": "siipiipiipiiiiiiiii",
     "alpha_winograd_filter_transform": "lppii",
     "alpha_conv3D_winograd": "sipiippiiiiiii",
     "alpha_winograd_filter_transform_deltaX": "lppii",
@@ -325,6 +326,12 @@ class Cuda_dconv3D_deltaW:
     @staticmethod
     def dconv3D_deltaW_GemmSK_W1(streamArray, length, GridZ, X, IH, IW, deltaY, deltaW, deltaW_buf, N, IC, OC):
         _call("alpha_dconv3D_deltaW_GemmSK_W1", streamArray, length, GridZ, X, IH, IW, deltaY, deltaW, deltaW_buf, N, IC, OC)
+
+    @staticmethod
+    def dconv3D_deltaW_GemmSK_static(streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, FH, FW, N, IC, OC, sh, sw, ph, pw):
+        """Split-K backward-filter plus the sum of its partial results, with the partials in the library's static device
+        array: allocates nothing, takes no deltaW_buf (no reference counterpart)."""
+        _call("alpha_dconv3D_deltaW_GemmSK_static", streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, FH, FW, N, IC, OC, sh, sw, ph, pw)
 
     # backward-filter plus the bias gradient (the reference: dconv3D_deltaW, then field_sum over deltaY)
     @staticmethod

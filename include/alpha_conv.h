@@ -252,6 +252,24 @@ int alpha_dconv3D_deltaW_GemmSK_W1(const int64_t *streams, int length, int GridZ
                                    const float *deltaY, float *deltaW, float *deltaW_buf,
                                    int N, int IC, int OC);
 
+/* No counterpart in the reference. For callers that cannot allocate device memory or hand over a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same computation as alpha_dconv3D_deltaW_GemmSK followed by alpha_buf_summary(deltaW_buf, deltaW,
+ * GridZ - 1, OC*FH*FW*IC) on streams[0], bit for bit, but the GridZ - 1 partial results live in a
+ * static device array of ALPHA_CONV_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held
+ * until the process ends) and the call neither allocates nor frees anything. deltaW is complete
+ * when streams[0] has run the enqueued work. (GridZ - 1) * OC*FH*FW*IC * 4 bytes beyond the array's
+ * size is refused with ALPHA_CONV_EINVAL. All calls on one GPU share the array: calls whose work
+ * overlaps in time on one GPU race (order them on one stream or with events).
+ * alpha_conv_device_info() resolves the array's address for the current device; a caller that
+ * captures graphs calls it once per device before capturing. */
+#define ALPHA_CONV_STATIC_SCRATCH_BYTES (32u << 20)
+int alpha_dconv3D_deltaW_GemmSK_static(const int64_t *streams, int length, int GridZ,
+                                       const float *X, int IH, int IW,
+                                       const float *deltaY, int OH, int OW,
+                                       float *deltaW, int FH, int FW,
+                                       int N, int IC, int OC, int sh, int sw, int ph, int pw);
+
 /* ---- this build's additional forward algorithm ------------------------------------------- */
 
 /* Winograd F(2x2,3x3) forward for FH = FW = 3, stride 1. No counterpart among the reference's
