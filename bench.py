@@ -6,9 +6,12 @@ forward, N=64, 56x56x64 -> 64 (config "c3a") — called the way the reference's 
 (kernel_remode then the GemmR entry, both per step; CudaFloat32EngineBase.java:1363-1420), inputs
 resident in HBM. One "step" = one forward pass over that batch. Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--layer c3a] [--op fwd|dx|dw] [--layers]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--layer c3a] [--op fwd|dx|dw] [--no-layers] [--no-parity]
 
---layers adds a "layers" array with every layer of BASELINE.json's configs (fewer iterations each).
+The line also carries a "layers" array: every layer and operator of BASELINE.json's five configs (fewer iterations
+each), each row with its time, its roofline fraction and its parity against the fp64 CPU oracle on a subset of the
+same seeded tensors (images for forward / backward-data, output channels over the full batch for backward-filter),
+with the tolerance it is held to stated in the row. --no-layers leaves the array out.
 The cpu_baseline leg times the CPU oracle's float-accumulate direct convolution on a bounded batch
 subset of the same workload on the host cores (baseline only, never a target).
 """
@@ -36,15 +39,17 @@ LAYERS = {
     "c3b": (64, 28, 28, 128, 128, 3, 1, 1, 128, ("fwd",)),
     "c3c": (64, 14, 14, 256, 256, 3, 1, 1, 256, ("fwd",)),
     "c3d": (64, 7, 7, 512, 512, 3, 1, 1, 512, ("fwd",)),
-    "c4a": (64, 224, 224, 4, 64, 7, 2, 3, 3, ("fwd",)),
-    "c4b": (64, 56, 56, 64, 128, 3, 2, 1, 64, ("fwd",)),
-    "c4c": (64, 56, 56, 64, 128, 1, 2, 0, 64, ("fwd",)),
+    "c4a": (64, 224, 224, 4, 64, 7, 2, 3, 3, ("fwd", "dx")),   # dx rows of config 4: the strided backward-data family,
+    "c4b": (64, 56, 56, 64, 128, 3, 2, 1, 64, ("fwd", "dx")),  # not asked for by BASELINE.json, measured all the same
+    "c4c": (64, 56, 56, 64, 128, 1, 2, 0, 64, ("fwd", "dx")),
     "c4d": (64, 14, 14, 256, 1024, 1, 1, 0, 256, ("fwd",)),
     "c5a": (32, 56, 56, 256, 64, 1, 1, 0, 256, ("dx", "dw")),
     "c5b": (32, 56, 56, 64, 64, 3, 1, 1, 64, ("dx", "dw")),
     "c5c": (32, 56, 56, 64, 256, 1, 1, 0, 64, ("dx", "dw")),
 }
 HBM_BOUND = {"c1", "c4c", "c5a", "c5c"}   # arithmetic intensity below the ridge
+UNIFORM_INPUT = {"c1", "c4a", "c4b", "c4c", "c4d"}   # BASELINE.json: inputs uniform[-1,1] (the others N(0,1)); filters He-normal
+REL_TOL, ABS_TOL = 1e-4, 1e-5
 
 
 def out_dim(IH, F, s, p):
@@ -66,7 +71,7 @@ def algorithmic_bytes(layer):
 class Workload:
     """Device tensors of one layer plus closures that enqueue each operator the way the Java engine does."""
 
-    def __init__(self, pkg, torch, layer, seed, fill_units=False, dw_winograd=False):
+    def __init__(self, pkg, torch, layer, seed):
         self.pkg, self.torch, self.layer = pkg, torch, layer
         N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[layer]
         self.dims = (N, IH, IW, IC, OC, F, s, p)
@@ -74,33 +79,52 @@ class Workload:
         self.OH, self.OW = OH, OW
         dev = torch.device("cuda:0")
         g = torch.Generator(device="cpu").manual_seed(seed)
-        X = torch.randn((N, IH, IW, IC), generator=g)
+        if layer in UNIFORM_INPUT:
+            X = torch.rand((N, IH, IW, IC), generator=g) * 2 - 1
+        else:
+            X = torch.randn((N, IH, IW, IC), generator=g)
         W = torch.randn((OC, F, F, IC), generator=g) * float(np.sqrt(2.0 / (F * F * ICl)))
         if ICl < IC:
             X[..., ICl:] = 0
             W[..., ICl:] = 0
         dY = torch.randn((N, OH, OW, OC), generator=g)
+        self.Xh, self.Wh, self.dYh = X, W, dY   # host copies: what the oracle is given
         self.X, self.W, self.dY = X.to(dev), W.to(dev), dY.to(dev)
         self.Y = torch.empty((N, OH, OW, OC), device=dev)
         self.dX = torch.empty((N, IH, IW, IC), device=dev)
         self.dW = torch.empty((OC, F, F, IC), device=dev)
         self.CW = torch.empty(F * F * IC * OC, device=dev)
-        self.Bias = torch.randn((OC,), generator=g).to(dev)
+        self.Bias = torch.randn((OC,), generator=g)
+        self.Biash, self.Bias = self.Bias, self.Bias.to(dev)
         self.stream = int(torch.cuda.current_stream().cuda_stream)
         self.streams = [self.stream]
         self.engine = pkg.engine.Engine(self.stream)
-        if fill_units:
-            # this build's option: raise the split-K factor until the launch fills the device (the reference's GridZ
-            # is sized for at most 128 SMs)
-            self.engine.config.deltaW_SK_fillUnits = pkg.device_info()[0]
-        if dw_winograd:
-            # this build's Winograd backward-filter, its split-K factor sized for the device's compute units
-            self.engine.config.deltaW_winograd = pkg.device_info()[0]
-        # split-K factor for the kernel-only timing: what the host layer would pass (CudaFloat32EngineBase.java:1707-1715)
-        self.GridZ = max(1, pkg.engine.plan_deltaW(self.engine.config, IH, IW, OH, OW, F, F, N, IC, OC, s, s).GridZ)
-        self.buf = torch.empty(max(1, self.GridZ - 1) * self.dW.numel(), device=dev)
+        self.dx_plan = pkg.engine.plan_deltaX(self.engine.config, IH, IW, OH, OW, F, F, N, IC, OC, s, s)
+        if s > 1:
+            cf = (F + s - 1) // s
+            self.ksCW = torch.empty(s * s * OC * cf * cf * IC, device=dev)
         if F == 3 and s == 1:
             self.U = torch.empty(16 * IC * OC, device=dev)
+        self.set_op("fwd")
+
+    def set_op(self, op):
+        """Engine options of one bench row (all of them this build's additions, off by default) and the split-K factor the
+        host layer passes with them (CudaFloat32EngineBase.java:1707-1715)."""
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        cfg = self.engine.config
+        cus = self.pkg.device_info()[0]
+        cfg.deltaW_SK_fillUnits = cus if op == "dw_fill" else 0
+        cfg.deltaW_winograd = cus if op == "dw_wino" else 0
+        cfg.conv3D_winograd = 1 if op == "wino" else 0
+        cfg.deltaX_winograd = 1 if op == "dx_wino" else 0
+        cfg.cache_filter_transforms = 1 if op == "fwd_cached" else 0
+        self.GridZ = max(1, self.pkg.engine.plan_deltaW(cfg, IH, IW, self.OH, self.OW, F, F, N, IC, OC, s, s).GridZ)
+        need = max(1, self.GridZ - 1) * self.dW.numel()
+        if getattr(self, "buf", None) is None or self.buf.numel() < need:
+            self.buf = self.torch.empty(need, device=self.X.device)
+
+    def close(self):
+        self.engine.close()
 
     # forward: remode + GemmR entry (W1 entry for 1x1 stride 1), as CudaFloat32EngineBase.conv3D does
     def fwd_remode(self):
@@ -122,22 +146,11 @@ class Workload:
         self.pkg.Cuda_conv3D.conv3D_winograd(self.streams, 1, self.X.data_ptr(), IH, IW, self.U.data_ptr(), self.Y.data_ptr(),
                                              self.OH, self.OW, N, IC, OC, p, p)
 
-    def wino(self):
-        self.engine.config.conv3D_winograd = 1
-        self.fwd()
-        self.engine.config.conv3D_winograd = 0
-
     def fwd_bias(self):
         # conv3D_biased through the host layer: same plan as fwd, bias added in the kernel epilogue
         N, IH, IW, IC, OC, F, s, p = self.dims
         self.engine.conv3D_biased(self.Y.data_ptr(), self.OH, self.OW, self.X.data_ptr(), IH, IW, self.W.data_ptr(), F, F,
                                   N, IC, OC, s, s, p, p, self.Bias.data_ptr(), N * self.OH * self.OW * OC, OC)
-
-    def fwd_cached(self):
-        # as fwd, with this build's option that keeps the re-laid-out filter between calls (inference, or training with
-        # the weight update reported to the engine)
-        self.engine.config.cache_filter_transforms = 1
-        self.fwd()
 
     def fwd(self):
         # whole operator through the C++ host layer: entry selection, CW scratch, kernel_remode, conv entry
@@ -146,13 +159,26 @@ class Workload:
                            N, IC, OC, s, s, p, p)
 
     def dx(self):
+        # the backward-data entry alone; strided layers: the entry the host layer picks, filter re-layout done beforehand
         N, IH, IW, IC, OC, F, s, p = self.dims
         D = self.pkg.Cuda_dconv3D_deltaX
-        if F == 1:
+        if F == 1 and s == 1:
             D.dconv3D_deltaX_W1(self.streams, 1, self.dY.data_ptr(), self.W.data_ptr(), self.dX.data_ptr(), IH, IW, N, IC, OC)
-        else:
+        elif s == 1:
             D.dconv3D_deltaX_V2_s1(True, self.streams, 1, self.dY.data_ptr(), self.OH, self.OW, self.W.data_ptr(), F, F,
                                    self.dX.data_ptr(), IH, IW, N, IC, OC, p, p)
+        elif self.dx_plan.entry_name == "dconv3D_deltaX_crossAdd":
+            D.dconv3D_deltaX_crossAdd(self.streams, 1, self.dY.data_ptr(), self.OH, self.OW, self.W.data_ptr(), F, F,
+                                      self.dX.data_ptr(), IH, IW, N, IC, OC, s, s, p, p)
+        else:
+            D.dconv3D_deltaX_kernelSplit(self.streams, 1, self.dY.data_ptr(), self.OH, self.OW, self.ksCW.data_ptr(), F, F,
+                                         self.dX.data_ptr(), IH, IW, N, IC, OC, s, s, p, p)
+
+    def dx_prepare(self):
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        if s > 1:
+            cf = (F + s - 1) // s
+            self.pkg.Cuda_dconv3D_deltaX.ks_remodev2(self.stream, self.W.data_ptr(), F, F, self.ksCW.data_ptr(), cf, cf, OC, IC, s, s)
 
     def dw_gemm(self):
         N, IH, IW, IC, OC, F, s, p = self.dims
@@ -180,11 +206,6 @@ class Workload:
         N, IH, IW, IC, OC, F, s, p = self.dims
         self.pkg.Cuda_dconv3D_deltaX.dconv3D_deltaX_winograd(self.streams, 1, self.dY.data_ptr(), self.OH, self.OW, self.U.data_ptr(),
                                                              self.dX.data_ptr(), IH, IW, N, IC, OC, p, p)
-
-    def dx_wino(self):
-        self.engine.config.deltaX_winograd = 1
-        self.dx_op()
-        self.engine.config.deltaX_winograd = 0
 
     def dx_op(self):
         N, IH, IW, IC, OC, F, s, p = self.dims
@@ -255,27 +276,83 @@ def load_traffic(layer, op):
     return None
 
 
-def measure(pkg, torch, layer, op, steps, warmup):
-    wl = Workload(pkg, torch, layer, seed=1000 + sorted(LAYERS).index(layer), fill_units=(op == "dw_fill"), dw_winograd=(op == "dw_wino"))
-    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd_cached, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.wino,
-            "dx_wino": wl.dx_wino, "dw_wino": wl.dw}[op]
+ORACLE_MACS = 2.5e8   # multiply-adds of fp64 oracle work per bench row (a fraction of a second on the host cores)
+
+
+def parity(wl, op, step):
+    """Runs `step` once and compares part of its output with the fp64 oracle on the same tensors. Forward and backward-data:
+    a subset of images (the first ones and the last one). Backward-filter: the full batch for four output channels (the
+    first two and the last two), i.e. every element of deltaW[oc] for those oc. Reports the bar of the GPU tests
+    (|err| <= max(1e-4*|want|, 1e-5*max(1, rms(want)))), the same with the literal absolute floor 1e-5, and the reference's
+    own criterion (Vector.samePercentRelative, threshold 1e-4)."""
+    from oracle import oracle as O
+    torch = wl.torch
+    N, IH, IW, IC, OC, F, s, p = wl.dims
+    OH, OW = wl.OH, wl.OW
+    out = {"fwd": wl.Y, "dx": wl.dX, "dw": wl.dW}[kind_of(op)]
+    out.fill_(float("nan"))
+    step()
+    wl.engine.sync()
+    torch.cuda.synchronize()
+    extra = {}
+    if kind_of(op) == "dw":
+        ocs = sorted(set([0, 1, OC - 2, OC - 1]))
+        dYs = np.ascontiguousarray(wl.dYh.numpy()[..., ocs])
+        want = O.deltaW_f64(wl.Xh.numpy(), dYs, F, F, s, s, p, p)
+        got = out[ocs].cpu().numpy()
+        subset = "all %d images, output channels %s" % (N, ocs)
+        first = out.clone()
+        step()
+        wl.engine.sync()
+        torch.cuda.synchronize()
+        extra["bit_reproducible_run_to_run"] = bool(torch.equal(first.view(torch.int32), out.view(torch.int32)))
+    else:
+        per_image = float(OH) * OW * OC * F * F * IC
+        n = int(max(2, min(N, ORACLE_MACS // per_image)))
+        imgs = list(range(n - 1)) + [N - 1]
+        if kind_of(op) == "fwd":
+            want = O.conv3D_f64(np.ascontiguousarray(wl.Xh.numpy()[imgs]), wl.Wh.numpy(), s, s, p, p)
+            if op == "fwd_bias":
+                want = want + wl.Biash.numpy().astype(np.float64)
+        else:
+            want = O.deltaX_f64(np.ascontiguousarray(wl.dYh.numpy()[imgs]), wl.Wh.numpy(), IH, IW, s, s, p, p)
+        got = out[imgs].cpu().numpy()
+        subset = "images %s of %d, all channels" % (imgs, N)
+    rms = float(np.sqrt(np.mean(want * want)))
+    tol_abs = ABS_TOL * max(1.0, rms)
+    r = {"vs": "fp64 CPU oracle", "subset": subset, "checked": int(want.size), "tol_rel": REL_TOL, "tol_abs": float("%.3g" % tol_abs),
+         "max_err_ratio": round(O.max_err_ratio(got, want, REL_TOL, tol_abs), 4),
+         "max_err_ratio_at_abs_1e-5": round(O.max_err_ratio(got, want, REL_TOL, ABS_TOL), 4),
+         "max_abs_err": float("%.3g" % float(np.max(np.abs(got.astype(np.float64) - want)))), "rms_expected": float("%.4g" % rms),
+         "samePercentRelative_1e-4": round(O.samePercentRelative(want.astype(np.float32), got, 1e-4), 6)}
+    r["ok"] = bool(r["max_err_ratio"] <= 1.0 and np.isfinite(got).all())
+    r.update(extra)
+    return r
+
+
+def kind_of(op):
+    return "fwd" if op in ("fwd", "fwd_bias", "fwd_cached", "wino") else "dx" if op in ("dx", "dx_wino") else "dw"
+
+
+def measure(wl, op, steps, warmup, with_parity=True):
+    pkg, torch, layer = wl.pkg, wl.torch, wl.layer
+    wl.set_op(op)
+    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.fwd,
+            "dx_wino": wl.dx_op, "dw_wino": wl.dw}[op]
     kernel = {"fwd": wl.fwd_conv, "fwd_cached": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
               "wino": wl.wino_conv, "dx_wino": wl.dx_wino_conv, "dw_wino": wl.dw_wino_gemm}[op]
+    N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
     if op in ("fwd", "fwd_bias", "fwd_cached"):
         wl.fwd_remode()
     if op == "wino":
-        N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
         pkg.Cuda_conv3D.winograd_filter_transform(wl.stream, wl.W.data_ptr(), wl.U.data_ptr(), IC_, OC_)
     if op == "dx_wino":
-        N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
         pkg.Cuda_dconv3D_deltaX.winograd_filter_transform_deltaX(wl.stream, wl.W.data_ptr(), wl.U.data_ptr(), IC_, OC_)
-    def step_and_recycle():
-        step()
-    wall_ms, ev_ms = time_loop(torch, step_and_recycle, steps, warmup)
+    if op == "dx":
+        wl.dx_prepare()
+    wall_ms, ev_ms = time_loop(torch, step, steps, warmup)
     wl.engine.sync()
     _, k_ms = time_loop(torch, kernel, steps, max(1, warmup // 2))   # dominant kernel alone, HIP events on its stream
-    gridz = wl.GridZ
-    wl.engine.close()
     fl, by = flops(layer), algorithmic_bytes(layer)
     hbm = layer in HBM_BOUND
     roof = {
@@ -287,9 +364,31 @@ def measure(pkg, torch, layer, op, steps, warmup):
         "traffic": load_traffic(layer, op),
     }
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
-    return {"layer": layer, "op": op, "ms_per_step": round(wall_ms, 5), "event_ms_per_step": round(ev_ms, 5),
-            "tflops": round(fl / (wall_ms * 1e-3) / 1e12, 3), "gflop": round(fl / 1e9, 3),
-            "algorithmic_MB": round(by / 1e6, 2), "GridZ": gridz if op in ("dw", "dw_fill") else None, "roofline": roof}
+    if op in ("wino", "dx_wino", "dw_wino"):
+        roof["note"] = "Winograd: FLOPs credited are the direct convolution's (2.25x the multiplies executed); frac is not a roofline fraction"
+    row = {"layer": layer, "op": op, "ms_per_step": round(wall_ms, 5), "event_ms_per_step": round(ev_ms, 5),
+           "tflops": round(fl / (wall_ms * 1e-3) / 1e12, 3), "gflop": round(fl / 1e9, 3),
+           "algorithmic_MB": round(by / 1e6, 2), "GridZ": wl.GridZ if kind_of(op) == "dw" else None, "roofline": roof}
+    if with_parity:
+        row["parity"] = parity(wl, op, step)
+    wl.set_op("fwd")
+    return row
+
+
+def layer_ops(layer):
+    N, IH, IW, IC, OC, F, s, p, ICl, ops = LAYERS[layer]
+    ops = list(ops)
+    if "fwd" in ops and F == 3 and s == 1 and IC >= 16:
+        ops.append("wino")
+    if "dx" in ops and F == 3 and s == 1:
+        ops.append("dx_wino")
+    if "dw" in ops:
+        ops.append("dw_fill")
+    if "dw" in ops and F == 3 and s == 1:
+        ops.append("dw_wino")
+    if layer == "c3a":
+        ops += ["fwd_bias", "fwd_cached"]
+    return ops
 
 
 def main():
@@ -300,7 +399,9 @@ def main():
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
     ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "dx", "dw", "dw_fill", "wino", "dx_wino", "dw_wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
-    ap.add_argument("--layers", action="store_true", help="also measure every layer/op of BASELINE.json's configs")
+    ap.add_argument("--layers", action="store_true", help="accepted for compatibility: the layers array is part of the default line")
+    ap.add_argument("--no-layers", action="store_true", help="leave out the array with every layer/op of BASELINE.json's configs")
+    ap.add_argument("--no-parity", action="store_true", help="leave out the per-row comparison with the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--probe-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy a few times (calibrates FETCH_SIZE/WRITE_SIZE counters)")
@@ -326,7 +427,11 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     op = args.op or LAYERS[args.layer][9][0]
 
-    head = measure(pkg, torch, args.layer, op, args.steps, args.warmup)
+    def seed_of(layer):
+        return 1000 + sorted(LAYERS).index(layer)
+
+    wl = Workload(pkg, torch, args.layer, seed_of(args.layer))
+    head = measure(wl, op, args.steps, args.warmup, with_parity=not args.no_parity)
     props = torch.cuda.get_device_properties(0)
     cus, clk_khz = pkg.device_info()
     clk_ghz = clk_khz / 1e6
@@ -342,34 +447,41 @@ def main():
                    "layer": args.layer, "op": op, "gflop_per_step": head["gflop"],
                    "algorithmic_MB_per_step": head["algorithmic_MB"],
                    "frac_of_fp32_mfma_peak": round(head["tflops"] / PEAK_MFMA_F32_TFLOPS, 4),
+                   "tolerance": "rel 1e-4, abs 1e-5*max(1, rms(expected)) against the fp64 CPU oracle; each row's parity states its own "
+                                "figures, also against the literal abs 1e-5",
                    "device": {"name": props.name, "cus": cus, "clock_ghz": round(clk_ghz, 3),
                               "fp32_mfma_peak_from_device_tflops": round(cus * 256 * clk_ghz / 1e3, 1)}},
         "roofline": head["roofline"],
     }
+    if "parity" in head:
+        out["parity"] = head["parity"]
     if op == "fwd" and F == 3 and s == 1 and IC >= 16:
         # the same layer through this build's second forward algorithm, in direct-convolution-equivalent FLOPs
-        wn = measure(pkg, torch, args.layer, "wino", args.steps, args.warmup)
+        wn = measure(wl, "wino", args.steps, args.warmup, with_parity=not args.no_parity)
         out["winograd"] = {"value": wn["tflops"], "unit": "TFLOP/s (direct-conv-equivalent)", "ms_per_step": wn["ms_per_step"],
                            "kernel_ms": wn["roofline"]["kernel_ms"], "kernel_tflops": wn["roofline"]["achieved"],
-                           "frac_of_fp32_mfma_peak": wn["roofline"]["frac"],
-                           "note": "Winograd F(2x2,3x3): 2.25x fewer multiplies than the FLOP count credited"}
-    if args.layers:
+                           "direct_equivalent_over_fp32_mfma_peak": wn["roofline"]["frac"],
+                           "executed_flop_frac_of_fp32_mfma_peak": round(wn["roofline"]["frac"] / 2.25, 4),
+                           "note": "Winograd F(2x2,3x3): 2.25x fewer multiplies than the FLOP count credited; the executed-FLOP figure "
+                                   "counts the 16 GEMMs only, not the transforms",
+                           "parity": wn.get("parity")}
+    wl.close()
+    del wl
+    if not args.no_layers:
         out["layers"] = []
+        lsteps, lwarm = max(5, args.steps // 5), max(2, args.warmup // 3)
         for layer in sorted(LAYERS):
-            ops = list(LAYERS[layer][9])
-            if "fwd" in ops and LAYERS[layer][5] == 3 and LAYERS[layer][6] == 1 and LAYERS[layer][3] >= 16:
-                ops.append("wino")
-            if "dx" in ops and LAYERS[layer][5] == 3 and LAYERS[layer][6] == 1:
-                ops.append("dx_wino")
-            if "dw" in ops:
-                ops.append("dw_fill")
-            if "dw" in ops and LAYERS[layer][5] == 3 and LAYERS[layer][6] == 1:
-                ops.append("dw_wino")
-            if layer == "c3a":
-                ops += ["fwd_bias", "fwd_cached"]
-            for o in ops:
-                out["layers"].append(measure(pkg, torch, layer, o, max(5, args.steps // 5), max(2, args.warmup // 3)))
-                torch.cuda.empty_cache()
+            wl = Workload(pkg, torch, layer, seed_of(layer))
+            for o in layer_ops(layer):
+                out["layers"].append(measure(wl, o, lsteps, lwarm, with_parity=not args.no_parity))
+            wl.close()
+            del wl
+            torch.cuda.empty_cache()
+        rows = [r for r in out["layers"] if "parity" in r]
+        if rows:
+            out["parity_summary"] = {"rows": len(rows), "rows_ok": sum(1 for r in rows if r["parity"]["ok"]),
+                                     "worst_max_err_ratio": max(r["parity"]["max_err_ratio"] for r in rows),
+                                     "worst_max_err_ratio_at_abs_1e-5": max(r["parity"]["max_err_ratio_at_abs_1e-5"] for r in rows)}
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(args.layer, op)
     print(json.dumps(out))
 

@@ -64,7 +64,9 @@ void oracle_set_num_threads(int n)
  * ---------------------------------------------------------------------------------------- */
 
 /* Tense.conv3D_naive (Tense.java:143-173): float tensors, DOUBLE accumulator, taps visited in
- * (fh, fw, ic) order, out-of-bounds taps skipped, result rounded to float once. */
+ * (fh, fw, ic) order, out-of-bounds taps skipped, result rounded to float once. The product is a
+ * FLOAT product (Tense.java:168: `v += X[..] * W[..]` with float operands: Java rounds it to float
+ * before widening it for the addition). */
 void oracle_conv3D_naive(const float *X, int IH, int IW,
                          const float *W, int FH, int FW,
                          float *Y, int OH, int OW,
@@ -84,7 +86,7 @@ void oracle_conv3D_naive(const float *X, int IH, int IW,
                             if (ih < 0 || iw < 0 || ih >= IH || iw >= IW) continue;
                             const float *x = &X_AT(n, ih, iw, 0);
                             const float *w = &W_AT(oc, fh, fw, 0);
-                            for (int ic = 0; ic < IC; ic++) v += (double)x[ic] * (double)w[ic];
+                            for (int ic = 0; ic < IC; ic++) v += (double)(float)(x[ic] * w[ic]);
                         }
                     Y_AT(n, oh, ow, oc) = (float)v;
                 }
@@ -255,7 +257,7 @@ void oracle_deltaW_naive(const float *X, int IH, int IW,
                             const int iw = ow * sw - pw + fw;
                             if (iw < 0 || iw >= IW) continue;
                             for (int n = 0; n < N; n++)
-                                v += (double)X_AT(n, ih, iw, ic) * (double)DY_AT(n, oh, ow, oc);
+                                v += (double)(float)(X_AT(n, ih, iw, ic) * DY_AT(n, oh, ow, oc));   /* float product, as conv3D_naive */
                         }
                     }
                     DW_AT(oc, fh, fw, ic) = (float)v;

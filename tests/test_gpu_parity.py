@@ -36,7 +36,7 @@ def tolerance_floor(want64):
     return ABS * max(1.0, float(np.sqrt(np.mean(np.square(want64)))))
 
 
-def check(got, want64, what, **_):
+def check(got, want64, what):
     floor = tolerance_floor(want64)
     ratio = O.max_err_ratio(got, want64, REL, floor)
     assert ratio <= 1.0, "%s: err/allowed = %.3f (rel %g, abs floor %.3g)" % (what, ratio, REL, floor)
@@ -315,7 +315,7 @@ def test_deltaX_s1_entries(dev, shape):
             DX.dconv3D_deltaX_V2_s1(True, *args)
         else:
             getattr(DX, entry)(*args)
-        check(dev.get(dXo), want, "%s %s" % (entry, shape), sp_thr=1e-4)
+        check(dev.get(dXo), want, "%s %s" % (entry, shape))
 
 
 def test_deltaX_W1(dev):
@@ -324,7 +324,7 @@ def test_deltaX_W1(dev):
         dXo = dev.guarded(N, IH, IW, IC)
         dy, w = dev.put(dY), dev.put(W)  # keep the device buffers alive across the call
         DX.dconv3D_deltaX_W1(dev.streams, 1, dy.data_ptr(), w.data_ptr(), dXo.data_ptr(), IH, IW, N, IC, OC)
-        check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, 0, 0), "deltaX_W1", sp_thr=1e-4)
+        check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, 0, 0), "deltaX_W1")
 
 
 POINTWISE_SHAPES = [
@@ -358,7 +358,7 @@ def test_pointwise_kernel_forward_and_deltaX(dev, shape):
     for algo in (0, 3):
         check(outs[algo][0], want_y, "conv3D_W1 algo %d %s" % (algo, shape))
         check(outs[algo][1], want_y, "conv3D_GemmR_W1 algo %d %s" % (algo, shape))
-        check(outs[algo][2], want_dx, "deltaX_W1 algo %d %s" % (algo, shape), sp_thr=1e-4)
+        check(outs[algo][2], want_dx, "deltaX_W1 algo %d %s" % (algo, shape))
 
 
 @pytest.mark.parametrize("shape", [
@@ -490,7 +490,7 @@ def test_deltaX_kernel_split_family(dev, shape):
             getattr(DX, entry)(*base, ph, pw)
         else:
             getattr(DX, entry)(*base, sh, sw, ph, pw)
-        check(dev.get(dXo), want, "%s %s" % (entry, shape), sp_thr=1e-4)
+        check(dev.get(dXo), want, "%s %s" % (entry, shape))
 
 
 @pytest.mark.parametrize("shape", [
@@ -510,7 +510,7 @@ def test_deltaX_crossAdd_is_deterministic_gather(dev, shape):
         DX.dconv3D_deltaX_crossAdd(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW,
                                    N, IC, OC, sh, sw, ph, pw)
         outs.append(dev.get(dXo))
-    check(outs[0], O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw), "crossAdd %s" % (shape,), sp_thr=1e-4)
+    check(outs[0], O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw), "crossAdd %s" % (shape,))
     assert np.array_equal(outs[0], outs[1])
 
 
@@ -542,7 +542,7 @@ def test_deltaW_entries(dev, shape):
     x, dy = dev.put(X), dev.put(dY)
     dWo = dev.guarded(OC, FH, FW, IC)
     DW.dconv3D_deltaW(dev.streams, 1, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
-    check(dev.get(dWo), want, "dconv3D_deltaW %s" % (shape,), sp_min=1.0)
+    check(dev.get(dWo), want, "dconv3D_deltaW %s" % (shape,))
     sizeW = OC * FH * FW * IC
     for entry in ("dconv3D_deltaW_GemmSK", "dconv3D_deltaW_GemmV2SK"):
         for GridZ in (2, 5, 16):
@@ -550,7 +550,7 @@ def test_deltaW_entries(dev, shape):
             buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
             getattr(DW, entry)(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
                                FH, FW, N, IC, OC, sh, sw, ph, pw)
-            check(_sum_partials(dev, dWo, buf, GridZ), want, "%s GridZ=%d %s" % (entry, GridZ, shape), sp_min=1.0)
+            check(_sum_partials(dev, dWo, buf, GridZ), want, "%s GridZ=%d %s" % (entry, GridZ, shape))
 
 
 def test_deltaW_split_k_slices_follow_the_reference_partition(dev):
@@ -566,7 +566,7 @@ def test_deltaW_split_k_slices_follow_the_reference_partition(dev):
                              F_, F_, N, IC, OC, s, s, p, p)
     parts = [dev.get(dWo)] + [b.reshape(OC, F_, F_, IC) for b in dev.get(buf)]
     for z in range(GridZ):
-        check(parts[z], O.deltaW_slice_f64(X, dY, F_, F_, s, s, p, p, GridZ, z), "slice %d" % z, sp_min=0.99)
+        check(parts[z], O.deltaW_slice_f64(X, dY, F_, F_, s, s, p, p, GridZ, z), "slice %d" % z)
 
 
 DW_ROWS_SHAPES = [
@@ -676,12 +676,12 @@ def test_deltaW_W1_entries(dev):
         x, dy = dev.put(X), dev.put(dY)
         dWo = dev.guarded(OC, 1, 1, IC)
         DW.dconv3D_deltaW_W1(dev.streams, 1, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), N, IC, OC)
-        check(dev.get(dWo), want, "deltaW_W1", sp_min=1.0)
+        check(dev.get(dWo), want, "deltaW_W1")
         GridZ = 3
         dWo = dev.guarded(OC, 1, 1, IC)
         buf = dev.empty(GridZ - 1, OC * IC, fill=float("nan"))
         DW.dconv3D_deltaW_GemmSK_W1(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), dWo.data_ptr(), buf.data_ptr(), N, IC, OC)
-        check(_sum_partials(dev, dWo, buf, GridZ), want, "deltaW_GemmSK_W1", sp_min=1.0)
+        check(_sum_partials(dev, dWo, buf, GridZ), want, "deltaW_GemmSK_W1")
 
 
 def test_buf_summary_bit_exact_kahan(dev):
@@ -708,7 +708,7 @@ def test_deltaW_bit_reproducible_run_to_run(dev):
                                  3, 3, N, IC, OC, 1, 1, 1, 1)
         outs.append(_sum_partials(dev, dWo, buf, GridZ))
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
-    check(outs[0], O.deltaW_f64(X, dY, 3, 3, 1, 1, 1, 1), "config-5b dW (N=4)", sp_min=1.0)
+    check(outs[0], O.deltaW_f64(X, dY, 3, 3, 1, 1, 1, 1), "config-5b dW (N=4)")
 
 
 # ----------------------------------------------------------------------------------------------

@@ -65,8 +65,8 @@ def test_forward_vs_torch_fp64(shape):
     got64 = O.conv3D_f64(X, W, sh, sw, ph, pw)
     assert got64.shape == want.shape
     np.testing.assert_allclose(got64, want, rtol=1e-12, atol=1e-12)
-    # double-accumulate float-out variant: correctly rounded up to one ulp of double noise
-    np.testing.assert_allclose(O.conv3D_naive(X, W, sh, sw, ph, pw), want, rtol=2e-7, atol=1e-7)
+    # double accumulator over FLOAT products (Tense.java:168), float out: each term carries one float rounding
+    np.testing.assert_allclose(O.conv3D_naive(X, W, sh, sw, ph, pw), want, rtol=2e-6, atol=2e-6)
     np.testing.assert_allclose(O.conv3D_f32acc(X, W, sh, sw, ph, pw), want, rtol=1e-4, atol=1e-5)
 
 
@@ -87,7 +87,7 @@ def test_deltaW_vs_torch_fp64(shape):
     X, dY = _rand((N, IH, IW, IC), 5), _rand((N, OH, OW, OC), 6)
     want = _torch_dw(X, dY, FH, FW, sh, sw, ph, pw)
     np.testing.assert_allclose(O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), want, rtol=1e-12, atol=1e-12)
-    np.testing.assert_allclose(O.deltaW_naive(X, dY, FH, FW, sh, sw, ph, pw), want, rtol=2e-7, atol=1e-7)
+    np.testing.assert_allclose(O.deltaW_naive(X, dY, FH, FW, sh, sw, ph, pw), want, rtol=2e-6, atol=2e-6)
     np.testing.assert_allclose(O.deltaW_f32acc(X, dY, FH, FW, sh, sw, ph, pw), want, rtol=1e-4, atol=1e-5)
 
 
@@ -109,6 +109,38 @@ def test_forward_brute_force_tiny():
         X, W = _rand((1, IH, IW, 2), 7), _rand((3, FH, FW, 2), 8)
         np.testing.assert_allclose(O.conv3D_f64(X, W, sh, sw, ph, pw), _brute_forward(X, W, sh, sw, ph, pw),
                                    rtol=1e-13, atol=1e-13)
+
+
+def test_naive_variants_add_float_products_to_a_double_accumulator():
+    """Tense.conv3D_naive (Tense.java:168) computes `v += X[..] * W[..]` with float operands and a double v: Java rounds the
+    product to float first. Emulated term by term with numpy scalars in the reference's (fh, fw, ic) order; a product taken
+    in double instead gives different bits in some outputs, which the last assertion shows for this data."""
+    IH, IW, IC, OC, F_, p = 5, 4, 4, 4, 3, 1
+    X, W = _rand((1, IH, IW, IC), 21), _rand((OC, F_, F_, IC), 22)
+    want = np.zeros((1, IH, IW, OC), np.float32)
+    dbl = np.zeros((1, IH, IW, OC), np.float32)
+    for oh, ow, oc in itertools.product(range(IH), range(IW), range(OC)):
+        v, vd = np.float64(0), np.float64(0)
+        for fh, fw, ic in itertools.product(range(F_), range(F_), range(IC)):
+            ih, iw = oh - p + fh, ow - p + fw
+            if 0 <= ih < IH and 0 <= iw < IW:
+                v = v + np.float64(np.float32(X[0, ih, iw, ic] * W[oc, fh, fw, ic]))
+                vd = vd + np.float64(X[0, ih, iw, ic]) * np.float64(W[oc, fh, fw, ic])
+        want[0, oh, ow, oc], dbl[0, oh, ow, oc] = np.float32(v), np.float32(vd)
+    got = O.conv3D_naive(X, W, 1, 1, p, p)
+    assert np.array_equal(got, want)
+    assert not np.array_equal(want, dbl)
+    # deltaW_naive is the same routine with deltaY as the filter (Tense.java:1277-1320): sum over (oh, ow, n)
+    dY = _rand((1, IH, IW, OC), 23)
+    wantW = np.zeros((OC, F_, F_, IC), np.float32)
+    for oc, fh, fw, ic in itertools.product(range(OC), range(F_), range(F_), range(IC)):
+        v = np.float64(0)
+        for oh, ow in itertools.product(range(IH), range(IW)):
+            ih, iw = oh - p + fh, ow - p + fw
+            if 0 <= ih < IH and 0 <= iw < IW:
+                v = v + np.float64(np.float32(X[0, ih, iw, ic] * dY[0, oh, ow, oc]))
+        wantW[oc, fh, fw, ic] = np.float32(v)
+    assert np.array_equal(O.deltaW_naive(X, dY, F_, F_, 1, 1, p, p), wantW)
 
 
 def test_all_ones_counts_in_bounds_taps():
