@@ -36,6 +36,9 @@ def _compile(src):
 
 def build(jobs=8, verbose=False):
     os.makedirs(OBJ, exist_ok=True)
+    # jni_shim.cpp is generated from the method table in gen_jni_shim.py and the C ABI header: regenerate it on every
+    # build so that the committed file cannot drift from its generator
+    subprocess.check_call([sys.executable, os.path.join(CSRC, "gen_jni_shim.py")], stdout=subprocess.DEVNULL)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         results = list(ex.map(_compile, sources()))
     for _, out in results:

@@ -3,6 +3,7 @@
 #pragma once
 #include "winograd_limits.hpp"
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 
 namespace alpha {
@@ -33,12 +34,26 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
     return (__umulhi(n, f.mul) + n) >> f.shift;
 }
 
+// Bumped by alpha_rt_resetDevice: a device reset drops function attributes and symbol addresses, so whatever this
+// library remembers per device is only valid for the generation it was recorded in.
+inline std::atomic<unsigned> &device_generation()
+{
+    static std::atomic<unsigned> gen{0};
+    return gen;
+}
+
 // The dynamic LDS limit is a property of (kernel, device): raise it the first time a device needs more than it has.
 // One instantiation, and so one table, per kernel. A racing first call sets the same value twice.
 template <auto KERNEL>
 inline hipError_t ensure_dynamic_lds(size_t bytes)
 {
     static size_t configured[64] = {0};
+    static unsigned seen_generation = 0;
+    const unsigned gen = device_generation().load(std::memory_order_acquire);
+    if (gen != seen_generation) {   // a device was reset since: every device's attribute is asked for again
+        for (size_t &c : configured) c = 0;
+        seen_generation = gen;
+    }
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;

@@ -52,24 +52,33 @@ int check_dims(const char *fn, int N, int IC, int OC, int IH, int IW, int OH, in
     if ((IC & 3) || (OC & 3)) return fail(ALPHA_CONV_EINVAL, "%s: IC and OC must be multiples of 4 (got %d, %d)", fn, IC, OC);
     if ((long)N * IH * IW * IC >= (1L << 31) || (long)N * OH * OW * OC >= (1L << 31) || (long)OC * FH * FW * IC >= (1L << 31))
         return fail(ALPHA_CONV_EINVAL, "%s: tensor exceeds 2^31 elements", fn);
+    // every output pixel's window must lie inside the padded input, as the engine's own check demands
+    // (EngineCore.java:653-665); a smaller output than the formula's is legal there and here
+    if ((long)(OH - 1) * sh + FH > (long)IH + 2 * ph || (long)(OW - 1) * sw + FW > (long)IW + 2 * pw)
+        return fail(ALPHA_CONV_EINVAL, "%s: output %dx%d does not fit input %dx%d with filter %dx%d, stride %d,%d, padding %d,%d",
+                    fn, OH, OW, IH, IW, FH, FW, sh, sw, ph, pw);
     return 0;
 }
 
 enum FilterLayout { FILTER_W, FILTER_CW };
 
-int g_fwd_algo = -1;   // -1: not yet read from the environment
+// Debugging switch (tests and comparisons force the generic kernels with it); not part of the drop-in contract. The only
+// mutable process-wide setting of the library: atomic, read once per call, so a call sees one value throughout.
+std::atomic<int> g_fwd_algo{-1};   // -1: not yet read from the environment
 
 int fwd_algo()
 {
-    if (g_fwd_algo < 0) {
+    int v = g_fwd_algo.load(std::memory_order_relaxed);
+    if (v < 0) {
         const char *e = getenv("ALPHA_HIP_CONV_ALGO");
-        int v = 0;
+        v = 0;
         if (e && !strcmp(e, "igemm")) v = 1;
         else if (e && !strcmp(e, "winograd")) v = 2;
         else if (e && !strcmp(e, "generic")) v = 3;
-        g_fwd_algo = v;
+        int expected = -1;
+        if (!g_fwd_algo.compare_exchange_strong(expected, v)) v = expected;   // a setter was quicker
     }
-    return g_fwd_algo;
+    return v;
 }
 
 // Forward: Y = conv(X, filter). FILTER_W reads W[OC,FH,FW,IC]; FILTER_CW reads CW[FH,FW,IC,OC].
@@ -245,6 +254,7 @@ static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
 
 constexpr int MAX_DEVICES = 64;
 std::atomic<float *> g_scratch_ptr[MAX_DEVICES];
+std::atomic<unsigned> g_scratch_generation{0};   // device_generation() the addresses above were asked in
 
 // Device address of `scratch` on the current device, or nullptr with the error recorded.
 float *static_scratch(const char *fn)
@@ -253,6 +263,11 @@ float *static_scratch(const char *fn)
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) { hip_status(e, fn); return nullptr; }
     if (dev < 0 || dev >= MAX_DEVICES) { fail(ALPHA_CONV_EINVAL, "%s: device index %d out of range", fn, dev); return nullptr; }
+    const unsigned gen = device_generation().load(std::memory_order_acquire);
+    if (g_scratch_generation.load(std::memory_order_acquire) != gen) {   // a device was reset: ask again
+        for (auto &q : g_scratch_ptr) q.store(nullptr, std::memory_order_release);
+        g_scratch_generation.store(gen, std::memory_order_release);
+    }
     float *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (ptr == nullptr) {   // a racing first call asks twice and stores the same address
         void *sym = nullptr;
@@ -293,7 +308,7 @@ int alpha_conv_get_fwd_algo(void) { return fwd_algo(); }
 int alpha_conv_set_fwd_algo(int algo)
 {
     if (algo < 0 || algo > 3) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..3");
-    g_fwd_algo = algo;
+    g_fwd_algo.store(algo);
     return 0;
 }
 

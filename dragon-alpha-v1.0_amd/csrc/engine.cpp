@@ -79,7 +79,9 @@ void alpha_plan_conv3D(const alpha_engine_config *c, int IH, int IW, int OH, int
     const double Q = alpha_paddingScaleUp(IH, IW, OH, OW, FH, FW, sh, sw);
     out->Q = Q;
     // a layer beyond the Winograd kernels' 32-bit offsets stays on the entries below
-    if (c->conv3D_winograd && FH == 3 && FW == 3 && sh == 1 && sw == 1 && alpha::winograd_forward_fits(N, IH, IW, IC, OH, OW, OC)) {
+    // (and so does one whose output is smaller than the formula's, which the engine's check allows and the kernels do not take)
+    if (c->conv3D_winograd && FH == 3 && FW == 3 && sh == 1 && sw == 1 && OH == IH + 2 * ph - 2 && OW == IW + 2 * pw - 2 &&
+        alpha::winograd_forward_fits(N, IH, IW, IC, OH, OW, OC)) {
         out->entry = ALPHA_E_conv3D_winograd;
         out->remode = 1;   // the filter transform takes the place of kernel_remode
         out->streams = 1;
@@ -317,6 +319,18 @@ static float *filter_block(alpha_engine *e, int kind, const float *W, int FH, in
     return static_cast<float *>(p);
 }
 
+// A transform into a freshly cached block failed: the block must not be handed out as a finished transform.
+static void forget_filter_block(alpha_engine *e, const float *block)
+{
+    std::lock_guard<std::mutex> g(e->mu);
+    for (auto it = e->filter_cache.begin(); it != e->filter_cache.end(); ++it)
+        if (it->second.second == block) {
+            e->free_blocks.emplace(it->second.first, it->second.second);
+            e->filter_cache.erase(it);
+            return;
+        }
+}
+
 void alpha_engine_filter_changed(alpha_engine *e, const float *W)
 {
     std::lock_guard<std::mutex> g(e->mu);
@@ -407,13 +421,13 @@ int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *
         bool fresh;
         float *U = filter_block(e, 1, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!U) return fail(e, -1, "conv3D");
-        if (fresh && (rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform");
+        if (fresh && (rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) { forget_filter_block(e, U); return fail(e, rc, "winograd_filter_transform"); }
         rc = alpha_conv3D_winograd(streams, p.streams, X, IH, IW, U, Y, OH, OW, N, IC, OC, ph, pw);
     } else if (p.remode) {
         bool fresh;
         float *CW = filter_block(e, 0, W, FH, FW, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!CW) return fail(e, -1, "conv3D");
-        if (fresh && (rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");
+        if (fresh && (rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) { forget_filter_block(e, CW); return fail(e, rc, "kernel_remode"); }
         switch (p.entry) {
         case ALPHA_E_conv3D_GemmR_W1: rc = alpha_conv3D_GemmR_W1(streams, p.streams, X, IH, IW, W, CW, Y, N, IC, OC); break;
         case ALPHA_E_conv3D_GemmV2R:
@@ -467,13 +481,13 @@ int alpha_engine_conv3D_biased(alpha_engine *e, float *Y, int OH, int OW, const 
         bool fresh;
         float *U = filter_block(e, 1, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!U) return fail(e, -1, "conv3D_biased");
-        if (fresh && (rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform");
+        if (fresh && (rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) { forget_filter_block(e, U); return fail(e, rc, "winograd_filter_transform"); }
         rc = alpha_conv3D_winograd_biased(streams, p.streams, X, IH, IW, U, Bias, Y, OH, OW, N, IC, OC, ph, pw);
     } else if (p.remode) {
         bool fresh;
         float *CW = filter_block(e, 0, W, FH, FW, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!CW) return fail(e, -1, "conv3D_biased");
-        if (fresh && (rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) return fail(e, rc, "kernel_remode");
+        if (fresh && (rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) { forget_filter_block(e, CW); return fail(e, rc, "kernel_remode"); }
         rc = alpha_conv3D_GemmR_biased(streams, p.streams, X, IH, IW, W, CW, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
     } else {
         rc = alpha_conv3D_biased(streams, p.streams, X, IH, IW, W, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
@@ -492,6 +506,12 @@ int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, 
     BlockScope scope{e};
     alpha_conv_plan p;
     alpha_plan_deltaW(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    if (p.entry == ALPHA_E_dconv3D_deltaW_GemmSK_winograd && (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2)) {
+        // an output smaller than the formula's is legal for the engine but not for the Winograd kernel: the default plan
+        alpha_engine_config plain = e->cfg;
+        plain.deltaW_winograd = 0;
+        alpha_plan_deltaW(&plain, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    }
     if (plan_out) *plan_out = p;
     int64_t streams[16];
     for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
@@ -543,6 +563,12 @@ int alpha_engine_dconv3D_deltaW_deltaB(alpha_engine *e, float *deltaW, float *de
     BlockScope scope{e};
     alpha_conv_plan p;
     alpha_plan_deltaW(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    if (p.entry == ALPHA_E_dconv3D_deltaW_GemmSK_winograd && (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2)) {
+        // an output smaller than the formula's is legal for the engine but not for the Winograd kernel: the default plan
+        alpha_engine_config plain = e->cfg;
+        plain.deltaW_winograd = 0;
+        alpha_plan_deltaW(&plain, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    }
     if (plan_out) *plan_out = p;
     int64_t streams[16];
     for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
@@ -574,6 +600,12 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
     BlockScope scope{e};
     alpha_conv_plan p;
     alpha_plan_deltaX(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    if (p.entry == ALPHA_E_dconv3D_deltaX_winograd && (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2)) {
+        // an output smaller than the formula's is legal for the engine but not for the Winograd kernels: the default plan
+        alpha_engine_config plain = e->cfg;
+        plain.deltaX_winograd = 0;
+        alpha_plan_deltaX(&plain, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    }
     if (plan_out) *plan_out = p;
     int64_t streams[16];
     for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
@@ -586,7 +618,7 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
         bool fresh;
         float *U = filter_block(e, 3, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!U) return fail(e, -1, "dconv3D_deltaX");
-        if (fresh && (rc = alpha_winograd_filter_transform_deltaX(streams[0], W, U, IC, OC))) return fail(e, rc, "winograd_filter_transform_deltaX");
+        if (fresh && (rc = alpha_winograd_filter_transform_deltaX(streams[0], W, U, IC, OC))) { forget_filter_block(e, U); return fail(e, rc, "winograd_filter_transform_deltaX"); }
         rc = alpha_dconv3D_deltaX_winograd(streams, p.streams, deltaY, OH, OW, U, deltaX, IH, IW, N, IC, OC, ph, pw);
         break;
     }
@@ -607,7 +639,7 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
         bool fresh;
         float *CW = filter_block(e, 2, W, FH, FW, IC, OC, sh, sw, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!CW) return fail(e, -1, "dconv3D_deltaX");
-        if (fresh && (rc = alpha_ks_remodev2(streams[0], W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw))) return fail(e, rc, "ks_remodev2");
+        if (fresh && (rc = alpha_ks_remodev2(streams[0], W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw))) { forget_filter_block(e, CW); return fail(e, rc, "ks_remodev2"); }
         switch (p.entry) {
         case ALPHA_E_dconv3D_deltaX_ksV2_Ims2R:
             rc = alpha_dconv3D_deltaX_ksV2_Ims2R(p.useTexture, streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);

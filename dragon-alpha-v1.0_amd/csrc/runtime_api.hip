@@ -3,6 +3,7 @@
 // small device kernels (fills and re-strides). Nothing here is on the convolution path; it exists so that a process can
 // obtain the device addresses and stream handles that path consumes from the same library.
 #include "../../include/alpha_rt.h"
+#include "common.hpp"
 
 #include <hip/hip_runtime.h>
 
@@ -41,13 +42,16 @@ int copy(const char *fn, int64_t stream, int64_t dst, int64_t src, int64_t size,
 __global__ __launch_bounds__(256) void fill_kernel(float *__restrict__ X, float value, int lengthv, int width, int stride)
 {
     // element k is data when k % stride < width, padding (zero) otherwise; width == stride for the 1-D fill
-    for (int k = blockIdx.x * 256 + threadIdx.x; k < lengthv; k += gridDim.x * 256) X[k] = (k % stride) < width ? value : 0.f;
+    // 64-bit loop index: k + gridDim.x*256 must not wrap for lengths close to 2^31
+    for (long k = (long)blockIdx.x * 256 + threadIdx.x; k < lengthv; k += (long)gridDim.x * 256) X[k] = ((int)k % stride) < width ? value : 0.f;
 }
 __global__ __launch_bounds__(256) void restride_kernel(const float *__restrict__ X, int XW, int XS, float *__restrict__ Y,
                                                        int YW, int YS, int length)
 {
-    for (int k = blockIdx.x * 256 + threadIdx.x; k < length; k += gridDim.x * 256)
-        Y[(k / YW) * YS + (k % YW)] = X[(k / XW) * XS + (k % XW)];
+    for (long kk = (long)blockIdx.x * 256 + threadIdx.x; kk < length; kk += (long)gridDim.x * 256) {
+        const int k = (int)kk;
+        Y[(size_t)(k / YW) * YS + (k % YW)] = X[(size_t)(k / XW) * XS + (k % XW)];
+    }
 }
 
 // memset by kernel rather than hipMemsetAsync, so that the call behaves the same when the caller's stream is being
@@ -146,7 +150,15 @@ int alpha_rt_memcpyAsyncDefault(int64_t stream, int64_t dst, int64_t src, int64_
 int alpha_rt_getDeviceId(int *id) { return id ? status(hipGetDevice(id), __func__) : invalid(__func__, "null"); }
 int alpha_rt_getDeviceCount(int *count) { return count ? status(hipGetDeviceCount(count), __func__) : invalid(__func__, "null"); }
 int alpha_rt_setDevice(int dev_id) { return status(hipSetDevice(dev_id), __func__); }
-int alpha_rt_resetDevice(void) { return status(hipDeviceReset(), __func__); }
+// hipDeviceReset drops what the library configured on the device (function attributes, the address of the static
+// scratch array) and frees every allocation, including the scratch pools of engines: destroy engines before a reset.
+// The generation counter makes the conv launchers configure their kernels again afterwards.
+int alpha_rt_resetDevice(void)
+{
+    const int rc = status(hipDeviceReset(), __func__);
+    alpha::device_generation().fetch_add(1, std::memory_order_acq_rel);
+    return rc;
+}
 int alpha_rt_deviceSynchronize(void) { return status(hipDeviceSynchronize(), __func__); }
 int alpha_rt_isDeviceP2PAccessEnabled(int dev1_id, int dev2_id, int *enabled)
 {

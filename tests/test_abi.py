@@ -84,6 +84,14 @@ def test_argument_validation_without_gpu():
     assert rc == 10001 and b"deltaW_buf" in L.alpha_conv_last_error()
     with pytest.raises(pkg.AlphaConvError):
         pkg.Cuda_conv3D.kernel_remode(0, 0, 0, 3, 3, 8, 4)
+    # an output whose windows leave the padded input is refused at the C ABI too; a smaller one than the formula's is not
+    # a size error (the call then fails later, on the null stream array of this test, not on the sizes)
+    rc = L.alpha_conv3D(one, 1, p, 8, 8, p, 3, 3, p, 9, 8, 4, 4, 8, 1, 1, 1, 1)
+    assert rc == 10001 and b"does not fit" in L.alpha_conv_last_error()
+    rc = L.alpha_dconv3D_deltaX_s1(one, 1, p, 8, 12, p, 3, 3, p, 8, 8, 4, 4, 8, 1, 1)
+    assert rc == 10001 and b"does not fit" in L.alpha_conv_last_error()
+    rc = L.alpha_dconv3D_deltaW_GemmSK(one, 1, 2, p, 8, 8, p, 5, 5, p, p, 3, 3, 4, 4, 8, 2, 2, 1, 1)
+    assert rc == 10001 and b"does not fit" in L.alpha_conv_last_error()
 
 
 def _tap_filter_extent(AC, CO, TH, TW, b_off, b_sth, b_stw, b_sc):

@@ -205,3 +205,17 @@ def test_winograd_flags_leave_layers_beyond_32bit_offsets_on_the_default_entries
     # just inside: half the images
     inside = (128, 128, 128, 128, 3, 3, 32, 256, 256, 1, 1)
     assert E.plan_deltaW(cfg, *inside).entry_name == "dconv3D_deltaW_GemmSK_winograd"
+
+
+def test_winograd_forward_flag_leaves_layers_with_a_smaller_output_on_the_default_entry():
+    """The engine's size check is not strict (EngineCore.java:653-665: the output may be smaller than the formula's); the
+    Winograd kernels take exact-size layers only, so such a layer keeps the plan it has without the flag."""
+    cfg = E.default_config(256)
+    base = E.plan_conv3D(cfg, 12, 12, 11, 12, 3, 3, 8, 64, 64, 1, 1, 1, 1)
+    cfg.conv3D_winograd = 1
+    assert E.plan_conv3D(cfg, 12, 12, 12, 12, 3, 3, 8, 64, 64, 1, 1, 1, 1).entry_name == "conv3D_winograd"
+    for OH, OW in ((11, 12), (12, 10), (9, 9)):
+        p = E.plan_conv3D(cfg, 12, 12, OH, OW, 3, 3, 8, 64, 64, 1, 1, 1, 1)
+        assert p.entry_name == base.entry_name and p.entry_name != "conv3D_winograd"
+    assert E.param_check(11, 12, 12, 12, 3, 3, 8, 64, 64, 1, 1, 1, 1) is None
+    assert E.param_check(13, 12, 12, 12, 3, 3, 8, 64, 64, 1, 1, 1, 1) is not None

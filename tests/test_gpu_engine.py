@@ -218,6 +218,37 @@ def test_engine_filter_transform_cache(dev):
         e.close()
 
 
+def test_engine_winograd_flags_and_a_smaller_output_than_the_formula(dev):
+    """The engine accepts an output smaller than (IH + 2p - F)/s + 1 (EngineCore.java:653-665); the Winograd kernels need the
+    exact size, so with every Winograd flag on such a layer runs on its default entries and gives the leading block of
+    the full result (forward) / the gradients of a deltaY that is zero outside that block (backward)."""
+    N, IH, IW, IC, OC = 4, 12, 12, 32, 32
+    OH, OW = 11, 10
+    X, W, dY = normal((N, IH, IW, IC), 6401), he_normal(OC, 3, 3, IC, 6402), normal((N, OH, OW, OC), 6403)
+    dYfull = np.zeros((N, IH, IW, OC), np.float32)
+    dYfull[:, :OH, :OW] = dY
+    x, w, dy = dev.put(X), dev.put(W), dev.put(dY)
+    e = pkg.engine.Engine(dev.stream)
+    try:
+        e.config.conv3D_winograd = 1
+        e.config.deltaX_winograd = 1
+        e.config.deltaW_winograd = 1
+        e.config.deltaW_SplitKThreshold = 64
+        y = dev.guarded(N, OH, OW, OC)
+        dx = dev.guarded(N, IH, IW, IC)
+        dw = dev.guarded(OC, 3, 3, IC)
+        p1 = e.conv3D(y.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1)
+        p2 = e.dconv3D_deltaX(dx.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), 3, 3, N, IC, OC, 1, 1, 1, 1)
+        p3 = e.dconv3D_deltaW(dw.data_ptr(), 3, 3, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, 1, 1, 1, 1)
+        e.sync()
+        assert "winograd" not in p1.entry_name + p2.entry_name + p3.entry_name
+        check(dev.get(y), np.ascontiguousarray(O.conv3D_f64(X, W, 1, 1, 1, 1)[:, :OH, :OW]), "smaller output, forward")
+        check(dev.get(dx), O.deltaX_f64(dYfull, W, IH, IW, 1, 1, 1, 1), "smaller output, deltaX")
+        check(dev.get(dw), O.deltaW_f64(X, dYfull, 3, 3, 1, 1, 1, 1), "smaller output, deltaW")
+    finally:
+        e.close()
+
+
 def test_engine_deltaW_with_fill_option(dev):
     """A larger split-K factor changes the summation order, not the result beyond the parity bar."""
     N, IH, IC, OC = 32, 14, 128, 128

@@ -6,7 +6,10 @@ The CPU oracle cannot finish these sizes in seconds, so each layer is checked by
       backward-data;
   (2) the adjoint identity  <conv(X,W), dY> = <X, deltaX(dY,W)> = <W, deltaW(X,dY)>  evaluated in fp64 on the device,
       which ties the full-size backward-filter (a sum over the whole batch) to the forward result;
-  (3) for config 5: backward-filter twice, bit-identical.
+  (3) for config 5: backward-filter twice, bit-identical;
+  (4) backward-filter element by element: deltaW[oc] depends on deltaY[..., oc] only, so the oracle run on the FULL batch
+      with deltaY restricted to a few output channels (first, middle, last) must give those channels' whole filters - for
+      the direct kernels and for the Winograd backward-filter.
 Tolerance: rel 1e-4 with abs floor 1e-5 * max(1, rms(expected)) for (1); 2e-5 relative for the inner products of (2).
 """
 import numpy as np
@@ -137,6 +140,13 @@ def test_full_size_layer(dev, layer):
         err = (dww.double() - ref).abs() - 2 * torch.clamp(1e-4 * ref.abs(), min=floor)
         assert float(err.max()) <= 0.0, "%s: Winograd deltaW differs from the direct kernel's beyond twice the bar" % layer
         assert torch.equal(dww, dww2), "%s: Winograd deltaW differs between two runs" % layer
+
+    # (4) backward-filter element by element on the full batch, for a few output channels (Tense.java:1277-1320 restated)
+    ocs = sorted({0, 1, OC // 2 + 1, OC - 2, OC - 1})
+    wantw = O.deltaW_f64(Xn, np.ascontiguousarray(dYn[..., ocs]), F, F, s, s, p, p)
+    _check(dw[ocs].cpu().numpy(), wantw, "%s deltaW, output channels %s, all %d images" % (layer, ocs, N))
+    if dww is not None:
+        _check(dww[ocs].cpu().numpy(), wantw, "%s Winograd deltaW, output channels %s, all %d images" % (layer, ocs, N))
 
     # (3) run-to-run bit reproducibility of backward-filter (config 5)
     if dw2 is not None:
