@@ -154,6 +154,12 @@ hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *d
                               int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,
                               int sh, int sw, int ph, int pw, int GK_slice, int GZ, float *dB = nullptr, float *dB_buf = nullptr);
 
+// Backward-filter with the filter tap in the grid and both operands straight from memory (delta_w_taps.hip): any filter,
+// stride and padding; same slice partition and outputs. Returns hipErrorNotSupported (nothing launched) when it does not fit.
+hipError_t launch_deltaW_taps(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
+                              int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,
+                              int sh, int sw, int ph, int pw, int GK_slice, int GZ);
+
 // Winograd F(2x2,3x3) forward (winograd.hip): U = transformed filter [16][IC][OC].
 // Forward convolution for IC (stored) = 4 with the filter resident in LDS (stem_conv.hip); F is W[OC,FH,FW,4] or, with
 // f_cw, CW[FH,FW,4,OC]. Returns hipErrorNotSupported (nothing launched) when the layer does not fit.

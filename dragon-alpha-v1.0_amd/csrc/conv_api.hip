@@ -229,6 +229,12 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     a.GK = N * OH * OW;
     a.GZ = GridZ;
     a.GK_slice = (a.GK / GridZ) >> 3 << 3;
+    if (fwd_algo() == 4) {   // comparisons: the tap-per-workgroup kernel wherever it fits
+        if (dB)
+            if (int e = hip_status(launch_col_sum(stream0(streams), dY, dB, dB_buf, OC, a.GK, a.GK_slice, GridZ), fn)) return e;
+        hipError_t e = launch_deltaW_taps(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, a.GK_slice, GridZ);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     if (fwd_algo() != 3 && FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0) {
         hipError_t e = launch_deltaW_pointwise(stream0(streams), X, dY, dW, dW_buf, a.GK, IC, OC, a.GK_slice, GridZ, dB, dB_buf);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
@@ -307,7 +313,7 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz)
 int alpha_conv_get_fwd_algo(void) { return fwd_algo(); }
 int alpha_conv_set_fwd_algo(int algo)
 {
-    if (algo < 0 || algo > 3) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..3");
+    if (algo < 0 || algo > 4) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..4");
     g_fwd_algo.store(algo);
     return 0;
 }

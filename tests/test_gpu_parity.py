@@ -633,6 +633,58 @@ def test_deltaW_row_streaming_kernel_slices_and_sum(dev, shape):
     check(dev.get(dWs), O.deltaW_f64(X, dY, F_, F_, 1, 1, p, p), "row-streaming dW total %s" % (shape,))
 
 
+DW_TAPS_SHAPES = [
+    # the tap-per-workgroup kernel takes any geometry: N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw, GridZ
+    (32, 8, 8, 256, 256, 3, 3, 1, 1, 1, 1, 3),      # c2c with the Java engine's split-K factor (slices end inside rows)
+    (16, 16, 16, 128, 128, 3, 3, 1, 1, 1, 1, 7),    # c2b geometry: 14 sharing groups, linear block order
+    (8, 32, 32, 64, 64, 3, 3, 1, 1, 1, 1, 8),       # c2a geometry: 8 sharing groups, one per XCD
+    (4, 56, 56, 64, 64, 3, 3, 1, 1, 1, 1, 16),      # c5b geometry
+    (4, 9, 9, 16, 16, 3, 3, 1, 1, 1, 1, 5),         # slices of 64 pixels: boundaries in the middle of rows, channels < 64
+    (4, 13, 11, 36, 44, 3, 3, 1, 1, 1, 1, 3),       # ragged channel counts, OW not a multiple of 4
+    (4, 10, 12, 32, 48, 3, 3, 1, 1, 0, 0, 2),       # no padding
+    (4, 6, 7, 64, 32, 3, 3, 1, 1, 2, 2, 2),         # padding 2
+    (4, 14, 14, 64, 128, 3, 3, 2, 2, 1, 1, 4),      # c4b geometry: stride 2
+    (4, 15, 13, 68, 132, 3, 3, 2, 2, 1, 1, 3),      # stride 2, odd sizes, ragged channels over several blocks
+    (4, 30, 30, 4, 64, 7, 7, 2, 2, 3, 3, 6),        # stem-like: 4 stored input channels, 49 taps
+    (4, 9, 11, 12, 20, 5, 4, 2, 3, 2, 1, 2),        # rectangular filter, different strides
+    (4, 14, 14, 64, 128, 1, 1, 2, 2, 0, 0, 5),      # 1x1 stride 2 (c4c geometry)
+    (8, 14, 14, 128, 64, 1, 1, 1, 1, 0, 0, 3),      # 1x1 stride 1
+    (4, 8, 8, 64, 64, 3, 3, 1, 1, 1, 1, 1),         # a single slice
+    (4, 4, 4, 64, 64, 3, 3, 1, 1, 1, 1, 16),        # GK = 64 < 8 * GridZ: GK_slice = 0, every slice but the last is empty
+    (4, 5, 6, 8, 8, 3, 3, 1, 1, 1, 1, 9),           # fewer rows in a slice than wavefronts in a workgroup
+]
+
+
+@pytest.mark.parametrize("shape", DW_TAPS_SHAPES)
+def test_deltaW_tap_per_workgroup_kernel_slices_and_sum(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw, GridZ = shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    X, dY = normal((N, IH, IW, IC), 3301), normal((N, OH, OW, OC), 3302)
+    x, dy = dev.put(X), dev.put(dY)
+    sizeW = OC * FH * FW * IC
+    L = pkg.lib()
+    runs = []
+    try:
+        L.alpha_conv_set_fwd_algo(4)   # the tap-per-workgroup kernel wherever it fits (it fits everything here)
+        for _ in range(2):
+            dWo = dev.guarded(OC, FH, FW, IC)
+            buf = dev.empty(max(GridZ - 1, 1), sizeW, fill=float("nan"))
+            DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(),
+                                     buf.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
+            runs.append([dev.get(dWo)] + [b.reshape(OC, FH, FW, IC) for b in dev.get(buf)[:GridZ - 1]])
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+    for z in range(GridZ):
+        want = O.deltaW_slice_f64(X, dY, FH, FW, sh, sw, ph, pw, GridZ, z)
+        check(runs[0][z], want, "tap kernel slice %d %s" % (z, shape))
+        assert np.array_equal(runs[0][z].view(np.uint32), runs[1][z].view(np.uint32)), "slice %d differs between two runs" % z
+    dWs = dev.put(runs[0][0])
+    if GridZ > 1:
+        bufs = dev.put(np.stack([o.reshape(-1) for o in runs[0][1:]]))
+        DW.buf_summary(dev.stream, bufs.data_ptr(), dWs.data_ptr(), GridZ - 1, sizeW)
+    check(dev.get(dWs), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "tap kernel dW total %s" % (shape,))
+
+
 DW_WINO_SHAPES = [
     # N, IH, IW, IC, OC, ph, pw, GridZ   (3x3, stride 1)
     (4, 56, 56, 64, 64, 1, 1, 16),
