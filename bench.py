@@ -183,7 +183,7 @@ class Workload:
     def dw_gemm(self):
         N, IH, IW, IC, OC, F, s, p = self.dims
         D = self.pkg.Cuda_dconv3D_deltaW
-        if F == 1:
+        if F == 1 and s == 1:   # the W1 natives carry no stride: 1x1 stride 1 only
             D.dconv3D_deltaW_GemmSK_W1(self.streams, 1, self.GridZ, self.X.data_ptr(), IH, IW, self.dY.data_ptr(),
                                        self.dW.data_ptr(), self.buf.data_ptr(), N, IC, OC)
         else:

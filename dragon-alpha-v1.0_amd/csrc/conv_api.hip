@@ -75,6 +75,8 @@ int fwd_algo()
         if (e && !strcmp(e, "igemm")) v = 1;
         else if (e && !strcmp(e, "winograd")) v = 2;
         else if (e && !strcmp(e, "generic")) v = 3;
+        else if (e && !strcmp(e, "taps")) v = 4;
+        else if (e && !strcmp(e, "rows")) v = 5;
         int expected = -1;
         if (!g_fwd_algo.compare_exchange_strong(expected, v)) v = expected;   // a setter was quicker
     }
@@ -229,17 +231,29 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     a.GK = N * OH * OW;
     a.GZ = GridZ;
     a.GK_slice = (a.GK / GridZ) >> 3 << 3;
-    if (fwd_algo() == 4) {   // comparisons: the tap-per-workgroup kernel wherever it fits
-        if (dB)
-            if (int e = hip_status(launch_col_sum(stream0(streams), dY, dB, dB_buf, OC, a.GK, a.GK_slice, GridZ), fn)) return e;
-        hipError_t e = launch_deltaW_taps(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, a.GK_slice, GridZ);
-        if (e != hipErrorNotSupported) return hip_status(e, fn);
-    }
-    if (fwd_algo() != 3 && FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0) {
+    const int algo = fwd_algo();
+    // Which kernel (all share the slice partition and the outputs):
+    //  - 1x1 stride 1 with channel counts in multiples of 64: the register kernel of delta_w_pointwise.hip;
+    //  - layers whose channel counts fill the 64 x 64 blocks of the tap-per-workgroup kernel to 75 % or more: that kernel
+    //    (any filter, stride and padding); the bias gradient, when asked for, then takes a pass of its own over deltaY -
+    //    unless the row-streaming kernel, which produces it on the way, would fill the device anyway;
+    //  - other stride-1 3x3 / 1x1 layers: the row-streaming kernel; whatever is left: the generic kernel.
+    // algo 3 forces the generic kernel, 4 the tap-per-workgroup kernel wherever it fits, 5 the row-streaming kernel
+    // wherever it fits (comparisons and tests).
+    const bool w1 = FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
+    if (algo != 3 && algo != 4 && algo != 5 && w1) {
         hipError_t e = launch_deltaW_pointwise(stream0(streams), X, dY, dW, dW_buf, a.GK, IC, OC, a.GK_slice, GridZ, dB, dB_buf);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (fwd_algo() != 3) {
+    const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
+    const bool blocks_filled = 4L * IC * OC >= 3L * icb * 64 * ocb * 64;
+    const bool rows_fill = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1)) && icb * ((OC + 31) / 32) * GridZ >= 2L * device_cu_count();
+    if (algo == 4 || (algo != 3 && algo != 5 && blocks_filled && !(dB && rows_fill))) {
+        hipError_t e = launch_deltaW_taps(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, a.GK_slice, GridZ);
+        if (e == hipSuccess && dB) e = launch_col_sum(stream0(streams), dY, dB, dB_buf, OC, a.GK, a.GK_slice, GridZ);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
+    if (algo != 3) {
         hipError_t e = launch_deltaW_rows(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
                                           a.GK_slice, GridZ, dB, dB_buf);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
@@ -313,7 +327,7 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz)
 int alpha_conv_get_fwd_algo(void) { return fwd_algo(); }
 int alpha_conv_set_fwd_algo(int algo)
 {
-    if (algo < 0 || algo > 4) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..4");
+    if (algo < 0 || algo > 5) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..5");
     g_fwd_algo.store(algo);
     return 0;
 }

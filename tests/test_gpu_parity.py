@@ -605,7 +605,7 @@ def test_deltaW_row_streaming_kernel_slices_and_sum(dev, shape):
     outs = {}
     L = pkg.lib()
     try:
-        for algo in (0, 3):   # 0: row-streaming kernel where eligible, 3: generic kernel
+        for algo in (5, 3):   # 5: row-streaming kernel where eligible, 3: generic kernel
             L.alpha_conv_set_fwd_algo(algo)
             dWo = dev.guarded(OC, F_, F_, IC)
             buf = dev.empty(max(GridZ - 1, 1), sizeW, fill=float("nan"))
@@ -623,12 +623,12 @@ def test_deltaW_row_streaming_kernel_slices_and_sum(dev, shape):
         want = O.deltaW_slice_f64(X, dY, F_, F_, 1, 1, p, p, GridZ, z)
         total += want
         floor = tolerance_floor(total if z else want)
-        for algo in (0, 3):
+        for algo in (5, 3):
             r = O.max_err_ratio(outs[algo][z], want, REL, max(floor, tolerance_floor(want)))
             assert r <= 1.0, "slice %d algo %d %s: err/allowed %.3f" % (z, algo, shape, r)
-    dWs = dev.put(outs[0][0])
+    dWs = dev.put(outs[5][0])
     if GridZ > 1:
-        bufs = dev.put(np.stack([o.reshape(-1) for o in outs[0][1:]]))
+        bufs = dev.put(np.stack([o.reshape(-1) for o in outs[5][1:]]))
         DW.buf_summary(dev.stream, bufs.data_ptr(), dWs.data_ptr(), GridZ - 1, sizeW)
     check(dev.get(dWs), O.deltaW_f64(X, dY, F_, F_, 1, 1, p, p), "row-streaming dW total %s" % (shape,))
 
