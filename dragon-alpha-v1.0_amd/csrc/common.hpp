@@ -80,6 +80,29 @@ inline int device_cu_count()
     return cu_count[dev];
 }
 
+// What happens to a result on its way to memory. Forward:
+//     y = leakyRelu( A[c] * ((acc + bias[c] - mean[c]) * rsqrt(var[c] + eps)) + B[c], slope )
+// i.e. the bias row-add, batch normalisation with given statistics (with or without its affine part) and the leaky
+// ReLU that the reference runs as separate passes over Y (linear_dual2D_row, batchNorm2D_row / batchNorm_affined2D_row,
+// leakyRelu2D: Cuda_function.java:1607, 3829, 3862). Every pointer may be NULL (that step is left out; mean and var
+// go together, A and B go together); slope = 1 leaves the sign alone. Backward (gate != NULL): the result is
+// multiplied by (gate[same element] > 0 ? 1 : slope), the backward of the leaky ReLU whose OUTPUT is `gate`
+// (leakyRelu2D_deltaX_v1, Cuda_function.java:1640); nothing else is applied then.
+struct Epilogue {
+    const float *bias, *mean, *var, *A, *B;
+    const float *gate;   // a tensor of the output's shape and layout
+    float eps, slope;
+    int fused;           // 0: only `bias` is applied (the fast path every kernel has); 1: all of the above
+};
+
+inline Epilogue bias_epilogue(const float *bias)
+{
+    Epilogue e{};
+    e.bias = bias;
+    e.slope = 1.f;
+    return e;
+}
+
 // One launch of the generic implicit-GEMM "gather convolution":
 //   O[o_off + n*o_sn + i*o_sh + j*o_sw + co] =
 //       sum_{th<TH, tw<TW, c<AC}  A[n, i*sh - ph + th, j*sw - pw + tw, c] * B[b_off + th*b_sth + tw*b_stw + c*b_sc + co*b_sn]
@@ -97,7 +120,7 @@ struct GatherConvArgs {
     int a_sn;                       // AH*AW*AC
     int o_off, o_sn, o_sh, o_sw;    // output strides, elements
     int b_off, b_sth, b_stw, b_sc, b_sn;
-    const float *bias;              // NULL or [CO]: added to every output row
+    Epilogue ep;                    // bias / normalisation / activation applied as the rows leave for memory
     FastDiv d_AC, d_TW, d_OWt, d_OHWt;
 };
 
@@ -112,7 +135,51 @@ static __device__ __forceinline__ float4 add_bias4(float4 v, const float *bias, 
     return v;
 }
 
+// per-channel constants of the forward form: y = (acc - sub) * mul + add
+static __device__ __forceinline__ void ep_channel(const Epilogue &ep, int c, float &sub, float &mul, float &add)
+{
+    sub = ep.bias ? -ep.bias[c] : 0.f;
+    mul = 1.f;
+    add = 0.f;
+    if (ep.mean) {
+        sub += ep.mean[c];
+        mul = rsqrtf(ep.var[c] + ep.eps);
+    }
+    if (ep.A) {
+        mul *= ep.A[c];
+        add = ep.B[c];
+    }
+}
+static __device__ __forceinline__ float ep_finish(float acc, float sub, float mul, float add, float slope)
+{
+    const float y = (acc - sub) * mul + add;
+    return y > 0.f ? y : y * slope;
+}
+static __device__ __forceinline__ float ep_gate(float acc, float g, float slope) { return g > 0.f ? acc : acc * slope; }
+
+// Four consecutive channels col .. col+3 of one output pixel; `elem` = offset of that float4 in the output tensor (where
+// the gate is read).
+static __device__ __forceinline__ float4 epilogue4(float4 v, const Epilogue &ep, int col, size_t elem)
+{
+    if (!ep.fused) return add_bias4(v, ep.bias, col);
+    if (ep.gate) {
+        const float4 g = *reinterpret_cast<const float4 *>(ep.gate + elem);
+        return make_float4(ep_gate(v.x, g.x, ep.slope), ep_gate(v.y, g.y, ep.slope), ep_gate(v.z, g.z, ep.slope), ep_gate(v.w, g.w, ep.slope));
+    }
+    float r[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float sub, mul, add;
+        ep_channel(ep, col + j, sub, mul, add);
+        r[j] = ep_finish(r[j], sub, mul, add, ep.slope);
+    }
+    return make_float4(r[0], r[1], r[2], r[3]);
+}
+
 // Every forward launcher takes `bias` (NULL = none): bias[co] is added to each output row in the kernel's epilogue.
+// Launchers that also take `ep` apply the whole Epilogue when ep != NULL (bias is then ignored); the others are followed
+// by launch_epilogue_rows, one more pass over the output.
+hipError_t launch_epilogue_rows(hipStream_t s, const float *X, float *Y, const Epilogue &ep, long lengthv, int width, int stride);
 
 // Convolution with the input window staged in LDS (tap_conv.hip, tap_conv_prefetch.hip). Filter element (th, tw, c, co)
 // at b_off + th*b_sth + tw*b_stw + c*b_sc + co*b_sn; b_sn = 1 (contiguous along the output channel) fits every shape
@@ -122,7 +189,7 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
                            int N, int AH, int AW, int AC, int OH, int OW, int CO,
                            int TH, int TW, int ph, int pw,
                            int b_off, int b_sth, int b_stw, int b_sc, const float *bias = nullptr, int sh = 1, int sw = 1,
-                           int b_sn = 1);
+                           int b_sn = 1, const Epilogue *ep = nullptr);
 
 // 1x1 stride-1 convolution as a streaming GEMM with the filter resident in LDS (pointwise.hip):
 // O[(n,oh,ow)][co] = sum_k A[n, oh*sh, ow*sw, k] * B(k, co), B given as [K][N] (b_kmajor) or [N][K]. Returns
@@ -165,7 +232,7 @@ hipError_t launch_deltaW_taps(hipStream_t stream, const float *X, const float *d
 // f_cw, CW[FH,FW,4,OC]. Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
 hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, int f_cw, float *Y,
                             int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw,
-                            const float *bias = nullptr);
+                            const float *bias = nullptr, const Epilogue *ep = nullptr);
 
 // Backward-filter of 1x1 stride-1 layers from registers (delta_w_pointwise.hip); same slice partition and outputs.
 // Returns hipErrorNotSupported (nothing launched) unless IC and OC are multiples of 64.
@@ -177,7 +244,8 @@ hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const flo
 // launch_winograd(deltaY, U, deltaX, N, OH, OW, OC, IH, IW, IC, 2 - ph, 2 - pw) then computes deltaX.
 hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int IC, int OC, bool backward = false);
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
-                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias = nullptr);
+                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias = nullptr,
+                           const Epilogue *ep = nullptr);
 // The same as one MFMA stream per persistent workgroup (winograd_stream.hip), for IC % 16 == 0; returns
 // hipErrorNotSupported (nothing launched) otherwise.
 hipError_t launch_winograd_stream(hipStream_t stream, const float *X, const float *U, float *Y,

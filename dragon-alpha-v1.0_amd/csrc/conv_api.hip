@@ -83,39 +83,49 @@ int fwd_algo()
     return v;
 }
 
-// Forward: Y = conv(X, filter). FILTER_W reads W[OC,FH,FW,IC]; FILTER_CW reads CW[FH,FW,IC,OC].
+// The rest of a fused epilogue as a pass of its own over a dense [pixels, C] output (kernels that add a bias only).
+int epilogue_pass(const char *fn, hipStream_t s, float *Y, const Epilogue &ep, long pixels, int C)
+{
+    return hip_status(launch_epilogue_rows(s, Y, Y, ep, pixels * C, C, C), fn);
+}
+
+// Forward: Y = conv(X, filter). FILTER_W reads W[OC,FH,FW,IC]; FILTER_CW reads CW[FH,FW,IC,OC]. `ep` (when not NULL
+// and fused) replaces `bias`: applied inside the kernel where it has the fused form, else by one more pass over Y.
 int forward(const char *fn, const int64_t *streams, int length,
             const float *X, int IH, int IW, const float *F, FilterLayout layout, int FH, int FW,
             float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
-            const float *bias = nullptr)
+            const float *bias = nullptr, const Epilogue *ep = nullptr)
 {
     if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
     if (!X || !F || !Y || !aligned16(X) || !aligned16(F) || !aligned16(Y) || !aligned16(bias))
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, sh, sw, ph, pw)) return e;
+    if (ep && !ep->fused) { bias = ep->bias; ep = nullptr; }
+    const int algo = fwd_algo();
 
-    if (IC == 4 && fwd_algo() != 3) {
-        hipError_t e = launch_stem_conv(stream0(streams), X, F, layout == FILTER_CW, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, bias);
+    if (IC == 4 && algo != 3) {
+        hipError_t e = launch_stem_conv(stream0(streams), X, F, layout == FILTER_CW, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, bias, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
+    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && algo != 3) {
         // W[OC][IC] is [N][K]; CW[IC][OC] is [K][N]; a stride only thins the input pixels that are read
-        hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW, bias);
+        hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW, ep ? nullptr : bias);
+        if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), Y, *ep, (long)N * OH * OW, OC);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (fwd_algo() != 3) {
+    if (algo != 3) {
         // W[OC,FH,FW,IC] as it is: taken by the 3x3 stride-1 kernel (128-bit fragment loads; measured the same speed as
         // from CW), refused by the others, which then leaves the generic kernel
         hipError_t e = layout == FILTER_CW
             ? launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
-                              0, FW * IC * OC, IC * OC, OC, bias, sh, sw)
+                              0, FW * IC * OC, IC * OC, OC, bias, sh, sw, 1, ep)
             : launch_tap_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, ph, pw,
-                              0, FW * IC, IC, 1, bias, sh, sw, FH * FW * IC);
+                              0, FW * IC, IC, 1, bias, sh, sw, FH * FW * IC, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
 
     GatherConvArgs a{};
-    a.A = X; a.B = F; a.O = Y; a.bias = bias;
+    a.A = X; a.B = F; a.O = Y; a.ep = ep ? *ep : bias_epilogue(bias);
     a.CO = OC;
     a.AH = IH; a.AW = IW; a.AC = IC;
     a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
@@ -131,29 +141,32 @@ int forward(const char *fn, const int64_t *streams, int length,
 
 // Backward-data, stride 1, reading W[OC,FH,FW,IC] in place rotated by 180 degrees:
 // deltaX[n,ih,iw,ic] = sum_{t_h,t_w,oc} deltaY[n, ih - (FH-1-ph) + t_h, iw - (FW-1-pw) + t_w, oc] * W[oc, FH-1-t_h, FW-1-t_w, ic]
+// `ep` (NULL, or a gate epilogue): deltaX is multiplied by the derivative of the leaky ReLU that produced this layer's input.
 int deltaX_s1(const char *fn, const int64_t *streams, int length,
               const float *dY, int OH, int OW, const float *W, int FH, int FW,
-              float *dX, int IH, int IW, int N, int IC, int OC, int ph, int pw)
+              float *dX, int IH, int IW, int N, int IC, int OC, int ph, int pw, const Epilogue *ep = nullptr)
 {
     if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
     if (!dY || !W || !dX || !aligned16(dY) || !aligned16(W) || !aligned16(dX))
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
     if (int e = check_dims(fn, N, IC, OC, IH, IW, OH, OW, FH, FW, 1, 1, ph, pw)) return e;
     if (FH - 1 - ph < 0 || FW - 1 - pw < 0) return fail(ALPHA_CONV_EINVAL, "%s: padding larger than FH-1", fn);
+    const int algo = fwd_algo();
 
-    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && fwd_algo() != 3) {
+    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && algo != 3) {
         // deltaX[m][ic] = sum_oc deltaY[m][oc] * W[oc][ic]: W is [K][N]
         hipError_t e = launch_pointwise(stream0(streams), dY, W, dX, N, IH, IW, IH, IW, 1, 1, OC, IC, 1);
+        if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), dX, *ep, (long)N * IH * IW, IC);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (fwd_algo() != 3) {
+    if (algo != 3) {
         hipError_t e = launch_tap_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, FH - 1 - ph, FW - 1 - pw,
-                                       ((FH - 1) * FW + (FW - 1)) * IC, -FW * IC, -IC, FH * FW * IC);
+                                       ((FH - 1) * FW + (FW - 1)) * IC, -FW * IC, -IC, FH * FW * IC, nullptr, 1, 1, 1, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
 
     GatherConvArgs a{};
-    a.A = dY; a.B = W; a.O = dX;
+    a.A = dY; a.B = W; a.O = dX; a.ep = ep ? *ep : bias_epilogue(nullptr);
     a.CO = IC;
     a.AH = OH; a.AW = OW; a.AC = OC;
     a.sh = 1; a.sw = 1; a.ph = FH - 1 - ph; a.pw = FW - 1 - pw;
@@ -637,6 +650,109 @@ int alpha_conv3D_winograd_biased(const int64_t *streams, int length, const float
     hipError_t e = launch_winograd(stream0(streams), X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, Bias);
     if (e == hipErrorNotSupported) return fail(ALPHA_CONV_EINVAL, "%s: needs OH = IH + 2*ph - 2, OW = IW + 2*pw - 2", __func__);
     return hip_status(e, __func__);
+}
+
+// ---- fused epilogues: batch normalisation and leaky ReLU around the convolution ---------------------------------------
+namespace {
+// The C-ABI epilogue as the kernels' Epilogue; 0 when it is inconsistent.
+int make_epilogue(const char *fn, const alpha_conv_epilogue *in, Epilogue *out)
+{
+    if (in == nullptr) return fail(ALPHA_CONV_EINVAL, "%s: epilogue is null", fn);
+    if ((in->X_mean == nullptr) != (in->X_var == nullptr)) return fail(ALPHA_CONV_EINVAL, "%s: X_mean and X_var go together", fn);
+    if ((in->A == nullptr) != (in->B == nullptr)) return fail(ALPHA_CONV_EINVAL, "%s: A and B go together", fn);
+    if (!aligned16(in->Bias) || !aligned16(in->X_mean) || !aligned16(in->X_var) || !aligned16(in->A) || !aligned16(in->B))
+        return fail(ALPHA_CONV_EINVAL, "%s: misaligned epilogue pointer", fn);
+    Epilogue e{};
+    e.bias = in->Bias; e.mean = in->X_mean; e.var = in->X_var; e.A = in->A; e.B = in->B;
+    e.eps = in->eps; e.slope = in->k;
+    e.fused = (in->X_mean || in->A || in->k != 1.f) ? 1 : 0;   // a bias alone is every kernel's fast path
+    *out = e;
+    return 0;
+}
+int row_function(const char *fn, int64_t stream, const float *X, float *Y, const Epilogue &ep, int lengthv, int mem_width, int mem_stride)
+{
+    if (!X || !Y || !aligned16(X) || !aligned16(Y)) return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
+    if (lengthv < 0 || mem_stride < 4 || (mem_stride & 3) || mem_width < 1 || mem_width > mem_stride || lengthv % mem_stride != 0)
+        return fail(ALPHA_CONV_EINVAL, "%s: need lengthv = height * mem_stride, mem_stride a multiple of 4, 1 <= mem_width <= mem_stride", fn);
+    return hip_status(launch_epilogue_rows(reinterpret_cast<hipStream_t>((intptr_t)stream), X, Y, ep, lengthv, mem_width, mem_stride), fn);
+}
+}  // namespace
+
+int alpha_conv3D_fused(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, int FH, int FW,
+                       const alpha_conv_epilogue *epilogue, float *Y, int OH, int OW, int N, int IC, int OC,
+                       int sh, int sw, int ph, int pw)
+{
+    Epilogue ep;
+    if (int e = make_epilogue(__func__, epilogue, &ep)) return e;
+    return forward(__func__, streams, length, X, IH, IW, W, FILTER_W, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, nullptr, &ep);
+}
+int alpha_conv3D_GemmR_fused(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, const float *CW,
+                             int FH, int FW, const alpha_conv_epilogue *epilogue, float *Y, int OH, int OW, int N, int IC, int OC,
+                             int sh, int sw, int ph, int pw)
+{
+    (void)W;
+    Epilogue ep;
+    if (int e = make_epilogue(__func__, epilogue, &ep)) return e;
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, nullptr, &ep);
+}
+int alpha_conv3D_winograd_fused(const int64_t *streams, int length, const float *X, int IH, int IW, const float *U,
+                                const alpha_conv_epilogue *epilogue, float *Y, int OH, int OW, int N, int IC, int OC, int ph, int pw)
+{
+    CHECK_STREAMS();
+    CHECK_PTR(X);
+    CHECK_PTR(U);
+    CHECK_PTR(Y);
+    Epilogue ep;
+    if (int e = make_epilogue(__func__, epilogue, &ep)) return e;
+    if (int e = check_dims(__func__, N, IC, OC, IH, IW, OH, OW, 3, 3, 1, 1, ph, pw)) return e;
+    hipError_t e = launch_winograd(stream0(streams), X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, nullptr, &ep);
+    if (e == hipErrorNotSupported) return fail(ALPHA_CONV_EINVAL, "%s: needs OH = IH + 2*ph - 2, OW = IW + 2*pw - 2", __func__);
+    return hip_status(e, __func__);
+}
+int alpha_dconv3D_deltaX_s1_leakyRelu(const int64_t *streams, int length, const float *deltaY, int OH, int OW, const float *W,
+                                      int FH, int FW, const float *Xf, float k, float *deltaX, int IH, int IW,
+                                      int N, int IC, int OC, int ph, int pw)
+{
+    CHECK_PTR(Xf);
+    Epilogue ep{};
+    ep.gate = Xf; ep.slope = k; ep.fused = 1;
+    return deltaX_s1(__func__, streams, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw, &ep);
+}
+int alpha_leakyRelu2D(int64_t stream, const float *X, float k, float *Y, int lengthv, int mem_width, int mem_stride)
+{
+    Epilogue ep{};
+    ep.slope = k; ep.fused = 1;
+    return row_function(__func__, stream, X, Y, ep, lengthv, mem_width, mem_stride);
+}
+int alpha_leakyRelu2D_deltaX_v1(int64_t stream, float *deltaX, const float *deltaY, const float *Y, float k,
+                                int lengthv, int mem_width, int mem_stride)
+{
+    CHECK_PTR(Y);
+    Epilogue ep{};
+    ep.gate = Y; ep.slope = k; ep.fused = 1;
+    return row_function(__func__, stream, deltaY, deltaX, ep, lengthv, mem_width, mem_stride);
+}
+int alpha_batchNorm2D_row(int64_t stream, const float *X, const float *X_mean, const float *X_var, float eps, int row_lengthv,
+                          float *Y, int lengthv, int mem_width, int mem_stride)
+{
+    CHECK_PTR(X_mean);
+    CHECK_PTR(X_var);
+    if (row_lengthv != mem_stride) return fail(ALPHA_CONV_EINVAL, "%s: row_lengthv must equal mem_stride", __func__);
+    Epilogue ep{};
+    ep.mean = X_mean; ep.var = X_var; ep.eps = eps; ep.slope = 1.f; ep.fused = 1;
+    return row_function(__func__, stream, X, Y, ep, lengthv, mem_width, mem_stride);
+}
+int alpha_batchNorm_affined2D_row(int64_t stream, const float *X, const float *X_mean, const float *X_var, float eps,
+                                  const float *A, const float *B, int row_lengthv, float *Y, int lengthv, int mem_width, int mem_stride)
+{
+    CHECK_PTR(X_mean);
+    CHECK_PTR(X_var);
+    CHECK_PTR(A);
+    CHECK_PTR(B);
+    if (row_lengthv != mem_stride) return fail(ALPHA_CONV_EINVAL, "%s: row_lengthv must equal mem_stride", __func__);
+    Epilogue ep{};
+    ep.mean = X_mean; ep.var = X_var; ep.eps = eps; ep.A = A; ep.B = B; ep.slope = 1.f; ep.fused = 1;
+    return row_function(__func__, stream, X, Y, ep, lengthv, mem_width, mem_stride);
 }
 
 }  // extern "C"

@@ -457,6 +457,35 @@ int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *
 // CudaFloat32EngineBase.conv3D_biased (:1478-1560): same selection as conv3D; there the bias is a second pass
 // (linear_dual2D_row on Y after an event), here it rides in the conv kernel's epilogue, so every remode entry collapses
 // onto the GemmR form and every other entry onto the plain form.
+static int conv3D_with_epilogue(alpha_engine *e, const char *what, float *Y, int OH, int OW, const float *X, int IH, int IW,
+                                const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                const alpha_conv_epilogue *ep, alpha_conv_plan *plan_out)
+{
+    BlockScope scope{e};
+    alpha_conv_plan p;
+    alpha_plan_conv3D(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, ph, pw, &p);
+    if (plan_out) *plan_out = p;
+    int64_t streams[16];
+    for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
+    int rc = 0;
+    if (p.entry == ALPHA_E_conv3D_winograd) {
+        bool fresh;
+        float *U = filter_block(e, 1, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
+        if (!U) return fail(e, -1, what);
+        if (fresh && (rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) { forget_filter_block(e, U); return fail(e, rc, "winograd_filter_transform"); }
+        rc = alpha_conv3D_winograd_fused(streams, p.streams, X, IH, IW, U, ep, Y, OH, OW, N, IC, OC, ph, pw);
+    } else if (p.remode) {
+        bool fresh;
+        float *CW = filter_block(e, 0, W, FH, FW, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
+        if (!CW) return fail(e, -1, what);
+        if (fresh && (rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) { forget_filter_block(e, CW); return fail(e, rc, "kernel_remode"); }
+        rc = alpha_conv3D_GemmR_fused(streams, p.streams, X, IH, IW, W, CW, FH, FW, ep, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+    } else {
+        rc = alpha_conv3D_fused(streams, p.streams, X, IH, IW, W, FH, FW, ep, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+    }
+    return rc ? fail(e, rc, what) : 0;
+}
+
 int alpha_engine_conv3D_biased(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W,
                                int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                const float *Bias, int lengthv, int width, alpha_conv_plan *plan_out)
@@ -470,29 +499,28 @@ int alpha_engine_conv3D_biased(alpha_engine *e, float *Y, int OH, int OW, const 
         snprintf(e->err, sizeof(e->err), "alpha_engine_conv3D_biased: Bias is null, or lengthv != N*OH*OW*OC, or width not in [1, OC]");
         return ALPHA_CONV_EINVAL;
     }
-    BlockScope scope{e};
-    alpha_conv_plan p;
-    alpha_plan_conv3D(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, ph, pw, &p);
-    if (plan_out) *plan_out = p;
-    int64_t streams[16];
-    for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
-    int rc = 0;
-    if (p.entry == ALPHA_E_conv3D_winograd) {
-        bool fresh;
-        float *U = filter_block(e, 1, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
-        if (!U) return fail(e, -1, "conv3D_biased");
-        if (fresh && (rc = alpha_winograd_filter_transform(streams[0], W, U, IC, OC))) { forget_filter_block(e, U); return fail(e, rc, "winograd_filter_transform"); }
-        rc = alpha_conv3D_winograd_biased(streams, p.streams, X, IH, IW, U, Bias, Y, OH, OW, N, IC, OC, ph, pw);
-    } else if (p.remode) {
-        bool fresh;
-        float *CW = filter_block(e, 0, W, FH, FW, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
-        if (!CW) return fail(e, -1, "conv3D_biased");
-        if (fresh && (rc = alpha_kernel_remode(streams[0], W, CW, FH, FW, OC, IC))) { forget_filter_block(e, CW); return fail(e, rc, "kernel_remode"); }
-        rc = alpha_conv3D_GemmR_biased(streams, p.streams, X, IH, IW, W, CW, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
-    } else {
-        rc = alpha_conv3D_biased(streams, p.streams, X, IH, IW, W, FH, FW, Bias, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+    alpha_conv_epilogue ep{};
+    ep.Bias = Bias;
+    ep.k = 1.f;
+    return conv3D_with_epilogue(e, "conv3D_biased", Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, &ep, plan_out);
+}
+
+// conv3D followed by batch normalisation with given statistics and leaky ReLU (the inference form of the reference's
+// conv -> bn -> leakyRelu blocks, experiments/alpha_code/src/cifar10/resnet18/Net.java:42-58), as one operator: same plan
+// as conv3D, the row functions in the convolution kernel's epilogue.
+int alpha_engine_conv3D_fused(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W,
+                              int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                              const alpha_conv_epilogue *epilogue, alpha_conv_plan *plan_out)
+{
+    if (const char *why = param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw)) {
+        snprintf(e->err, sizeof(e->err), "%s: illegal size: %s", "alpha_engine_conv3D_fused", why);
+        return ALPHA_CONV_EINVAL;
     }
-    return rc ? fail(e, rc, "conv3D_biased") : 0;
+    if (epilogue == nullptr) {
+        snprintf(e->err, sizeof(e->err), "alpha_engine_conv3D_fused: epilogue is null");
+        return ALPHA_CONV_EINVAL;
+    }
+    return conv3D_with_epilogue(e, "conv3D_fused", Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, epilogue, plan_out);
 }
 
 int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, const float *X, int IH, int IW,
@@ -589,12 +617,14 @@ int alpha_engine_dconv3D_deltaW_deltaB(alpha_engine *e, float *deltaW, float *de
     return 0;
 }
 
-int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
-                                const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
-                                alpha_conv_plan *plan_out)
+// Xf != NULL: deltaX is multiplied by the derivative of the leaky ReLU (slope k) whose output Xf is this layer's input - in
+// the kernel's epilogue for the stride-1 entries, by leakyRelu2D_deltaX_v1 in place after the others.
+static int deltaX_impl(alpha_engine *e, const char *what, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
+                       const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                       const float *Xf, float k, alpha_conv_plan *plan_out)
 {
     if (const char *why = param_check(OH, OW, IH, IW, FH, FW, N, IC, OC, sh, sw, ph, pw)) {
-        snprintf(e->err, sizeof(e->err), "%s: illegal size: %s", "alpha_engine_dconv3D_deltaX", why);
+        snprintf(e->err, sizeof(e->err), "%s: illegal size: %s", what, why);
         return ALPHA_CONV_EINVAL;
     }
     BlockScope scope{e};
@@ -610,6 +640,14 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
     int64_t streams[16];
     for (int i = 0; i < p.streams; i++) streams[i] = e->stream;
     int rc = 0;
+    bool gated = Xf == nullptr;   // nothing to apply, or applied by the kernel
+    if (Xf != nullptr && (p.entry == ALPHA_E_dconv3D_deltaX_W1 || p.entry == ALPHA_E_dconv3D_deltaX_V2_s1 ||
+                          p.entry == ALPHA_E_dconv3D_deltaX_s1_texture || p.entry == ALPHA_E_dconv3D_deltaX_s1)) {
+        const bool w1 = p.entry == ALPHA_E_dconv3D_deltaX_W1;
+        rc = alpha_dconv3D_deltaX_s1_leakyRelu(streams, p.streams, deltaY, w1 ? IH : OH, w1 ? IW : OW, W, FH, FW, Xf, k, deltaX, IH, IW,
+                                               N, IC, OC, w1 ? 0 : ph, w1 ? 0 : pw);
+        return rc ? fail(e, rc, what) : 0;
+    }
     switch (p.entry) {
     case ALPHA_E_dconv3D_deltaX_crossAdd:
         rc = alpha_dconv3D_deltaX_crossAdd(streams, p.streams, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw);
@@ -617,7 +655,7 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
     case ALPHA_E_dconv3D_deltaX_winograd: {
         bool fresh;
         float *U = filter_block(e, 3, W, 3, 3, IC, OC, 1, 1, (size_t)p.scratch_floats * sizeof(float), &fresh);
-        if (!U) return fail(e, -1, "dconv3D_deltaX");
+        if (!U) return fail(e, -1, what);
         if (fresh && (rc = alpha_winograd_filter_transform_deltaX(streams[0], W, U, IC, OC))) { forget_filter_block(e, U); return fail(e, rc, "winograd_filter_transform_deltaX"); }
         rc = alpha_dconv3D_deltaX_winograd(streams, p.streams, deltaY, OH, OW, U, deltaX, IH, IW, N, IC, OC, ph, pw);
         break;
@@ -638,7 +676,7 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
         const int CFH = (FH + sh - 1) / sh, CFW = (FW + sw - 1) / sw;
         bool fresh;
         float *CW = filter_block(e, 2, W, FH, FW, IC, OC, sh, sw, (size_t)p.scratch_floats * sizeof(float), &fresh);
-        if (!CW) return fail(e, -1, "dconv3D_deltaX");
+        if (!CW) return fail(e, -1, what);
         if (fresh && (rc = alpha_ks_remodev2(streams[0], W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw))) { forget_filter_block(e, CW); return fail(e, rc, "ks_remodev2"); }
         switch (p.entry) {
         case ALPHA_E_dconv3D_deltaX_ksV2_Ims2R:
@@ -662,7 +700,30 @@ int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, 
         }
     }
     }
-    return rc ? fail(e, rc, "dconv3D_deltaX") : 0;
+    if (rc == 0 && !gated)
+        rc = alpha_leakyRelu2D_deltaX_v1(streams[0], deltaX, deltaX, Xf, k, N * IH * IW * IC, IC, IC);
+    return rc ? fail(e, rc, what) : 0;
+}
+
+int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
+                                const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                alpha_conv_plan *plan_out)
+{
+    return deltaX_impl(e, "alpha_engine_dconv3D_deltaX", deltaX, IH, IW, deltaY, OH, OW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, nullptr, 1.f,
+                       plan_out);
+}
+
+int alpha_engine_dconv3D_deltaX_leakyRelu(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
+                                          const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                          const float *Xf, float k, alpha_conv_plan *plan_out)
+{
+    if (Xf == nullptr) {
+        snprintf(e->err, sizeof(e->err), "alpha_engine_dconv3D_deltaX_leakyRelu: Xf is null");
+        return ALPHA_CONV_EINVAL;
+    }
+    return deltaX_impl(e, "alpha_engine_dconv3D_deltaX_leakyRelu", deltaX, IH, IW, deltaY, OH, OW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, Xf, k,
+                       plan_out);
+
 }
 
 #pragma GCC visibility pop

@@ -217,7 +217,7 @@ __global__ __launch_bounds__(256, 2) void gather_conv_kernel(const GatherConvArg
         const int ro = rowoff[row];
         if (ro >= 0 && n0 + c4 < CO)   // CO % 4 == 0: the four columns are valid together
             *reinterpret_cast<float4 *>(p.O + ro + n0 + c4) =
-                add_bias4(*reinterpret_cast<const float4 *>(Os + row * OS + c4), p.bias, n0 + c4);
+                epilogue4(*reinterpret_cast<const float4 *>(Os + row * OS + c4), p.ep, n0 + c4, (size_t)(ro + n0 + c4));
     }
 }
 

@@ -29,7 +29,7 @@ struct StemArgs {
     int N, IH, IW, OH, OW, OC;
     int FW, sh, sw, ph, pw;
     int f_cw;
-    const float *bias;   // NULL or [OC]
+    Epilogue ep;         // applied as the rows leave for memory
     int taps, groups;   // FH*FW and ceil(taps / 4)
     int IHB, IWB;       // input window of a block: 15*sh + FH rows, 15*sw + FW columns
     int blocks;         // N * bh_count * bw_count
@@ -197,7 +197,8 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
                 const int col = 4 * pp + q, ow = ow0 + col;
                 const float4 v = *reinterpret_cast<const float4 *>(Os + col * ST_OS + 4 * l16);
                 if (oh < p.OH && ow < p.OW && oc_ok)
-                    *reinterpret_cast<float4 *>(yrow + out_off[pp]) = add_bias4(v, p.bias, oc0 + 4 * l16);
+                    *reinterpret_cast<float4 *>(yrow + out_off[pp]) =
+                        epilogue4(v, p.ep, oc0 + 4 * l16, (size_t)(yrow - p.Y) + out_off[pp]);
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -207,12 +208,12 @@ __global__ __launch_bounds__(256, 2) void stem_conv_kernel(const StemArgs p)
 // Returns hipErrorNotSupported (nothing launched) unless IC (stored) is 4 and the filter has at most 52 taps.
 hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, int f_cw, float *Y,
                             int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw,
-                            const float *bias)
+                            const float *bias, const Epilogue *ep)
 {
     if (IC != 4 || FH * FW > 4 * ST_MAXG || OC < 4 || (OC & 3)) return hipErrorNotSupported;
     if ((size_t)N * IH * IW * 4 >= (1ull << 31) || (size_t)N * OH * OW * OC >= (1ull << 31)) return hipErrorNotSupported;
     StemArgs a{};
-    a.X = X; a.F = F; a.Y = Y; a.f_cw = f_cw; a.bias = bias;
+    a.X = X; a.F = F; a.Y = Y; a.f_cw = f_cw; a.ep = ep ? *ep : bias_epilogue(bias);
     a.N = N; a.IH = IH; a.IW = IW; a.OH = OH; a.OW = OW; a.OC = OC;
     a.FW = FW; a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
     a.taps = FH * FW;

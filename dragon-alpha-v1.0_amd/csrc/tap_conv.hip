@@ -37,7 +37,7 @@ struct TapConvArgs {
     int PWp, RP;      // LDS row: sw planes of PWp = ceil(PWt/sw) pixels (padded column cp in plane cp % sw at cp / sw); RP = sw*PWp
     int lds_rows;     // halo rows reserved in LDS
     int b_off, b_sth, b_stw, b_sc;
-    const float *bias;   // NULL or [CO]
+    Epilogue ep;         // applied as the rows leave for memory
     int full_units;   // units of 16*TILES pixels that are processed whole, dealt round-robin to the persistent workgroups
     int pieces;       // the remaining units cut into piece_split pieces of piece_tiles tiles each, one piece per workgroup
     int piece_split, piece_tiles;
@@ -315,7 +315,7 @@ __device__ __forceinline__ void tap_conv_unit(const TapConvArgs &p, float *smem,
         const int m = m0 + pix;
         if (m < m_lim && oc0 + cq < p.CO)
             *reinterpret_cast<float4 *>(p.O + (size_t)m * p.CO + oc0 + cq) =
-                add_bias4(*reinterpret_cast<const float4 *>(Os + pix * TC_OS + cq), p.bias, oc0 + cq);
+                epilogue4(*reinterpret_cast<const float4 *>(Os + pix * TC_OS + cq), p.ep, oc0 + cq, (size_t)m * p.CO + oc0 + cq);
     }
 }
 
@@ -417,14 +417,14 @@ static hipError_t launch_tc(hipStream_t stream, TapConvArgs a, size_t lds, int c
 hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const float *B, float *O,
                                     int N, int AH, int AW, int AC, int OH, int OW, int CO,
                                     int TH, int TW, int ph, int pw,
-                                    int b_off, int b_sth, int b_stw, int b_sc, int b_sn, const float *bias, int cus);
+                                    int b_off, int b_sth, int b_stw, int b_sc, int b_sn, const Epilogue &ep, int cus);
 
 // Returns hipErrorNotSupported when the shape does not fit this kernel (caller falls back to the
 // generic implicit GEMM); otherwise launches.
 hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, float *O,
                            int N, int AH, int AW, int AC, int OH, int OW, int CO,
                            int TH, int TW, int ph, int pw,
-                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias, int sh, int sw, int b_sn)
+                           int b_off, int b_sth, int b_stw, int b_sc, const float *bias, int sh, int sw, int b_sn, const Epilogue *ep)
 {
     if (sh < 1 || sw < 1 || sh > 4 || sw > 4) return hipErrorNotSupported;
     if (OH != (AH + 2 * ph - TH) / sh + 1 || OW != (AW + 2 * pw - TW) / sw + 1) return hipErrorNotSupported;
@@ -433,7 +433,7 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
     if ((long)N * (AH + 2 * ph) >= (1L << 24)) return hipErrorNotSupported;
 
     TapConvArgs a{};
-    a.A = A; a.B = B; a.O = O; a.bias = bias;
+    a.A = A; a.B = B; a.O = O; a.ep = ep ? *ep : bias_epilogue(bias);
     a.M = (int)M; a.CO = CO;
     a.AH = AH; a.AW = AW; a.AC = AC;
     a.TH = TH; a.TW = TW; a.ph = ph; a.pw = pw;
@@ -451,7 +451,7 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
     if (cus < 1) return hipErrorNotSupported;
     if (sh == 1 && sw == 1) {   // the variant that prefetches the halo, where it applies
         const hipError_t e = launch_tap_conv_prefetch(stream, A, B, O, N, AH, AW, AC, OH, OW, CO, TH, TW, ph, pw,
-                                                      b_off, b_sth, b_stw, b_sc, b_sn, bias, cus);
+                                                      b_off, b_sth, b_stw, b_sc, b_sn, a.ep, cus);
         if (e != hipErrorNotSupported) return e;
     }
     if (b_sn != 1) return hipErrorNotSupported;   // the kernel below reads the filter along the output channel only

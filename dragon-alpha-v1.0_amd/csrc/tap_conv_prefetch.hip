@@ -26,7 +26,7 @@ struct TapPfArgs {
     const float *A;   // input activations [N, AH, AW, AC]
     const float *B;   // filter; element (th, tw, c, co) at b_off + th*b_sth + tw*b_stw + c*b_sc + co*b_sn
     float *O;         // output [N, OH, OW, CO] dense
-    const float *bias;   // NULL or [CO]
+    Epilogue ep;         // EPI = false: only ep.bias is applied; EPI = true: the whole epilogue
     int M, CO;        // N*OH*OW pixels, output channels
     int AH, AW, AC;
     int TH, TW, ph, pw;
@@ -74,7 +74,7 @@ static __device__ __forceinline__ PfHalo pf_halo(const TapPfArgs &p, int m0, int
 // TILES: tiles of a whole unit; CG: column groups of 32 padded pixels per row (1 or 2); EPT: halo elements a thread
 // requests per tap; BK: the filter is contiguous along the input channel (W[OC,FH,FW,IC] as it is) instead of along the
 // output channel; RP2: rows of at most 16 padded pixels, a halo element is this thread's share of TWO rows (CG = 1).
-template <int TILES, int CG, int EPT, bool BK, bool RP2>
+template <int TILES, int CG, int EPT, bool BK, bool RP2, bool EPI>
 __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -226,7 +226,10 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
     // SIMD's vector issue port, and the other workgroup's address arithmetic and stores at the same priority wait for
     // thousands of cycles (unit set-up 15000 cycles instead of 1000, measured).
     __builtin_amdgcn_s_setprio(3);
-    const float bias_v = (p.bias != nullptr && b_cov) ? p.bias[b_co] : 0.f;
+    const float bias_v = (p.ep.bias != nullptr && b_cov) ? p.ep.bias[b_co] : 0.f;
+    // EPI: this lane's channel constants of the fused epilogue (the channel is the same for every unit of the workgroup)
+    float e_sub = 0.f, e_mul = 1.f, e_add = 0.f;
+    if (EPI && b_cov) ep_channel(p.ep, b_co, e_sub, e_mul, e_add);
     const int o_lane = b_cov ? (4 * q * p.CO + b_co) * 4 : (int)PF_OUT_OF_RANGE;   // output byte offset of this lane within a tile
     int buf = 0;          // buffer that holds the halo of the pass about to run
     float bA[2][4];       // filter fragment of that pass's first tap
@@ -375,13 +378,41 @@ __global__ __launch_bounds__(256, 2) void tap_conv_prefetch_kernel(const TapPfAr
         // queues behind the reads of the other workgroup's MFMA loop: 12000 cycles per unit, measured.)
         // The descriptor ends at the unit's last pixel, so rows past it are dropped by the range check.
         const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.O, 0, m_hi * p.CO * 4, 0x00020000);
+        if constexpr (!EPI) {
 #pragma unroll
-        for (int i = 0; i < T; i++)
+            for (int i = 0; i < T; i++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int soff = __builtin_amdgcn_readfirstlane((m0 + 16 * i + r) * p.CO * 4);
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[i][r] + bias_v), o_rsrc, o_lane, soff, 0);
+                for (int r = 0; r < 4; r++) {
+                    const int soff = __builtin_amdgcn_readfirstlane((m0 + 16 * i + r) * p.CO * 4);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, acc[i][r] + bias_v), o_rsrc, o_lane, soff, 0);
+                }
+        } else if (p.ep.gate != nullptr) {   // uniform: backward of the leaky ReLU that produced this tensor's twin `gate`
+            const __amdgpu_buffer_rsrc_t g_rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.ep.gate), 0, m_hi * p.CO * 4, 0x00020000);
+#pragma unroll
+            for (int i = 0; i < T; i++) {
+                float g[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int soff = __builtin_amdgcn_readfirstlane((m0 + 16 * i + r) * p.CO * 4);
+                    g[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(g_rsrc, o_lane, soff, 0));
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int soff = __builtin_amdgcn_readfirstlane((m0 + 16 * i + r) * p.CO * 4);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, ep_gate(acc[i][r], g[r], p.ep.slope)), o_rsrc, o_lane, soff, 0);
+                }
             }
+        } else {
+#pragma unroll
+            for (int i = 0; i < T; i++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int soff = __builtin_amdgcn_readfirstlane((m0 + 16 * i + r) * p.CO * 4);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, ep_finish(acc[i][r], e_sub, e_mul, e_add, p.ep.slope)),
+                                                          o_rsrc, o_lane, soff, 0);
+                }
+        }
     };
 
     while (idx < n_items) {
@@ -423,10 +454,10 @@ static int tap_pf_lds_rows(int M, int P, int OH, int OW, int TH, int PHt)
     return worst;
 }
 
-template <int TILES, int CG, int EPT, bool BK, bool RP2>
-static hipError_t launch_pf2(hipStream_t stream, TapPfArgs a, size_t lds, int cus)
+template <int TILES, int CG, int EPT, bool BK, bool RP2, bool EPI>
+static hipError_t launch_pf3(hipStream_t stream, TapPfArgs a, size_t lds, int cus)
 {
-    constexpr auto kern = tap_conv_prefetch_kernel<TILES, CG, EPT, BK, RP2>;
+    constexpr auto kern = tap_conv_prefetch_kernel<TILES, CG, EPT, BK, RP2, EPI>;
     if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     const int units = (a.M + TILES * 16 - 1) / (TILES * 16), ocb = (a.CO + 63) / 64;
     int G = 2 * cus / ocb;   // two workgroups per compute unit
@@ -450,6 +481,12 @@ static hipError_t launch_pf2(hipStream_t stream, TapPfArgs a, size_t lds, int cu
     return hipGetLastError();
 }
 
+template <int TILES, int CG, int EPT, bool BK, bool RP2>
+static hipError_t launch_pf2(hipStream_t stream, const TapPfArgs &a, size_t lds, int cus)
+{
+    return a.ep.fused ? launch_pf3<TILES, CG, EPT, BK, RP2, true>(stream, a, lds, cus) : launch_pf3<TILES, CG, EPT, BK, RP2, false>(stream, a, lds, cus);
+}
+
 template <int TILES, int CG, int EPT, bool RP2 = false>
 static hipError_t launch_pf(hipStream_t stream, const TapPfArgs &a, size_t lds, int cus)
 {
@@ -460,7 +497,7 @@ static hipError_t launch_pf(hipStream_t stream, const TapPfArgs &a, size_t lds, 
 hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const float *B, float *O,
                                     int N, int AH, int AW, int AC, int OH, int OW, int CO,
                                     int TH, int TW, int ph, int pw,
-                                    int b_off, int b_sth, int b_stw, int b_sc, int b_sn, const float *bias, int cus)
+                                    int b_off, int b_sth, int b_stw, int b_sc, int b_sn, const Epilogue &ep, int cus)
 {
     if (b_sn != 1 && (b_sc != 1 || (b_sn | b_sth | b_stw | b_off) % 4 != 0)) return hipErrorNotSupported;   // 128-bit fragment loads
     if (OH != AH + 2 * ph - TH + 1 || OW != AW + 2 * pw - TW + 1) return hipErrorNotSupported;
@@ -475,7 +512,7 @@ hipError_t launch_tap_conv_prefetch(hipStream_t stream, const float *A, const fl
     if (PWt <= 16 && a_bytes >= (1L << 30)) return hipErrorNotSupported;
 
     TapPfArgs a{};
-    a.A = A; a.B = B; a.O = O; a.bias = bias;
+    a.A = A; a.B = B; a.O = O; a.ep = ep;
     a.M = (int)M; a.CO = CO;
     a.AH = AH; a.AW = AW; a.AC = AC;
     a.TH = TH; a.TW = TW; a.ph = ph; a.pw = pw;

@@ -23,7 +23,7 @@ struct WinoArgs {
     const float *X;   // [N, IH, IW, IC]
     const float *U;   // [16][IC][OC] transformed filter
     float *Y;         // [N, OH, OW, OC]
-    const float *bias;   // NULL or [OC]
+    Epilogue ep;         // applied as the rows leave for memory
     int N, IH, IW, IC, OH, OW, OC;
     int ph, pw;
     int TR, TC;       // tile rows / columns per image: ceil(OH/2), ceil(OW/2)
@@ -258,9 +258,10 @@ __global__ __launch_bounds__(256, 2) void winograd_f2x2_kernel(const WinoArgs p)
             const int n = fdiv(tile, p.d_TRC), rem = tile - n * TRC;
             const int ty = fdiv(rem, p.d_TC), tx = rem - ty * TC;
             const int oh = 2 * ty + dy, ow = 2 * tx + dx;
-            if (oh < p.OH && ow < p.OW)
-                *reinterpret_cast<float4 *>(p.Y + (((size_t)n * p.OH + oh) * p.OW + ow) * p.OC + oc0 + cq) =
-                    add_bias4(*reinterpret_cast<const float4 *>(Os + px * 68 + cq), p.bias, oc0 + cq);
+            if (oh < p.OH && ow < p.OW) {
+                const size_t elem = (((size_t)n * p.OH + oh) * p.OW + ow) * p.OC + oc0 + cq;
+                *reinterpret_cast<float4 *>(p.Y + elem) = epilogue4(*reinterpret_cast<const float4 *>(Os + px * 68 + cq), p.ep, oc0 + cq, elem);
+            }
         }
     }
 }
@@ -275,14 +276,18 @@ hipError_t launch_winograd_filter(hipStream_t s, const float *W, float *U, int I
 }
 
 hipError_t launch_winograd(hipStream_t stream, const float *X, const float *U, float *Y,
-                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias)
+                           int N, int IH, int IW, int IC, int OH, int OW, int OC, int ph, int pw, const float *bias, const Epilogue *ep)
 {
     if (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2) return hipErrorNotSupported;
     if (!winograd_forward_fits(N, IH, IW, IC, OH, OW, OC)) return hipErrorNotSupported;
-    if (winograd_grouped_filter(IC))   // the persistent variant and its filter layout; no other kernel reads that layout
-        return launch_winograd_stream(stream, X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, bias);
+    if (winograd_grouped_filter(IC)) {   // the persistent variant and its filter layout; no other kernel reads that layout
+        if (ep == nullptr || !ep->fused) return launch_winograd_stream(stream, X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, ep ? ep->bias : bias);
+        // that kernel adds a bias only: the rest of the epilogue is one more pass over Y
+        if (hipError_t e = launch_winograd_stream(stream, X, U, Y, N, IH, IW, IC, OH, OW, OC, ph, pw, nullptr); e != hipSuccess) return e;
+        return launch_epilogue_rows(stream, Y, Y, *ep, (long)N * OH * OW * OC, OC, OC);
+    }
     WinoArgs a{};
-    a.X = X; a.U = U; a.Y = Y; a.bias = bias;
+    a.X = X; a.U = U; a.Y = Y; a.ep = ep ? *ep : bias_epilogue(bias);
     a.N = N; a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC;
     a.ph = ph; a.pw = pw;
     a.TR = (OH + 1) / 2; a.TC = (OW + 1) / 2;

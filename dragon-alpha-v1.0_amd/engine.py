@@ -77,6 +77,10 @@ def _lib():
         L.alpha_engine_dconv3D_deltaW_deltaB.argtypes = ([_P, _P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7
                                                          + [ctypes.POINTER(Plan)])
         L.alpha_engine_dconv3D_deltaX.argtypes = [_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7 + [ctypes.POINTER(Plan)]
+        L.alpha_engine_conv3D_fused.argtypes = ([_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7
+                                                + [ctypes.POINTER(native.Epilogue), ctypes.POINTER(Plan)])
+        L.alpha_engine_dconv3D_deltaX_leakyRelu.argtypes = ([_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7
+                                                            + [_P, ctypes.c_float, ctypes.POINTER(Plan)])
         _bound = True
     return L
 
@@ -152,6 +156,19 @@ class Engine:
         p = Plan()
         self._check(self._L.alpha_engine_conv3D_biased(self._h, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw,
                                                        Bias, lengthv, width, ctypes.byref(p)))
+        return p
+
+    def conv3D_fused(self, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, epilogue):
+        """conv3D + batch normalisation (given statistics) + leaky ReLU as one operator; `epilogue` is a native.Epilogue."""
+        p = Plan()
+        self._check(self._L.alpha_engine_conv3D_fused(self._h, Y, OH, OW, X, IH, IW, W, FH, FW, N, IC, OC, sh, sw, ph, pw,
+                                                      ctypes.byref(epilogue), ctypes.byref(p)))
+        return p
+
+    def dconv3D_deltaX_leakyRelu(self, deltaX, IH, IW, deltaY, OH, OW, W, FH, FW, N, IC, OC, sh, sw, ph, pw, Xf, k):
+        p = Plan()
+        self._check(self._L.alpha_engine_dconv3D_deltaX_leakyRelu(self._h, deltaX, IH, IW, deltaY, OH, OW, W, FH, FW, N, IC, OC,
+                                                                  sh, sw, ph, pw, Xf, k, ctypes.byref(p)))
         return p
 
     def dconv3D_deltaW(self, deltaW, FH, FW, X, IH, IW, deltaY, OH, OW, N, IC, OC, sh, sw, ph, pw):

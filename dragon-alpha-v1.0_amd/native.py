@@ -62,8 +62,26 @@ _SIGS = {
     "alpha_conv3D_biased": "sipiipiippiiiiiiiii",
     "alpha_conv3D_GemmR_biased": "sipiippiippiiiiiiiii",
     "alpha_conv3D_winograd_biased": "sipiipppiiiiiii",
+    "alpha_conv3D_fused": "sipiipiiepiiiiiiiii",
+    "alpha_conv3D_GemmR_fused": "sipiippiiepiiiiiiiii",
+    "alpha_conv3D_winograd_fused": "sipiipepiiiiiii",
+    "alpha_dconv3D_deltaX_s1_leakyRelu": "sipiipiipfpiiiiiii",
+    "alpha_leakyRelu2D": "lpfpiii",
+    "alpha_leakyRelu2D_deltaX_v1": "lpppfiii",
+    "alpha_batchNorm2D_row": "lpppfipiii",
+    "alpha_batchNorm_affined2D_row": "lpppfppipiii",
 }
-_CT = {"s": _S, "i": _I, "p": _P, "l": _L}
+
+
+class Epilogue(ctypes.Structure):
+    """alpha_conv_epilogue of include/alpha_conv.h: device addresses as integers (0 = absent), eps and k as floats."""
+    _fields_ = [("Bias", _P), ("X_mean", _P), ("X_var", _P), ("eps", ctypes.c_float), ("A", _P), ("B", _P), ("k", ctypes.c_float)]
+
+    def __init__(self, Bias=0, X_mean=0, X_var=0, eps=1e-5, A=0, B=0, k=1.0):
+        super().__init__(Bias or None, X_mean or None, X_var or None, eps, A or None, B or None, k)
+
+
+_CT = {"s": _S, "i": _I, "p": _P, "l": _L, "f": ctypes.c_float, "e": ctypes.POINTER(Epilogue)}
 
 
 class AlphaConvError(RuntimeError):
@@ -139,6 +157,11 @@ def _call(name, *args):
             conv.append(ctypes.c_void_p(int(a)))
         elif c == "l":
             conv.append(ctypes.c_int64(int(a)))
+        elif c == "f":
+            conv.append(ctypes.c_float(float(a)))
+        elif c == "e":
+            keep.append(a)
+            conv.append(ctypes.byref(a))
         else:
             conv.append(int(a))
     rc = getattr(L, name)(*conv)
@@ -229,6 +252,19 @@ class Cuda_conv3D:
     def conv3D_winograd_biased(streamArray, length, X, IH, IW, U, Bias, Y, OH, OW, N, IC, OC, ph, pw):
         _call("alpha_conv3D_winograd_biased", streamArray, length, X, IH, IW, U, Bias, Y, OH, OW, N, IC, OC, ph, pw)
 
+    # forward with bias, batch normalisation (given statistics) and leaky ReLU in the kernel epilogue; `epilogue` is an Epilogue
+    @staticmethod
+    def conv3D_fused(streamArray, length, X, IH, IW, W, FH, FW, epilogue, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D_fused", streamArray, length, X, IH, IW, W, FH, FW, epilogue, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_GemmR_fused(streamArray, length, X, IH, IW, W, CW, FH, FW, epilogue, Y, OH, OW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_conv3D_GemmR_fused", streamArray, length, X, IH, IW, W, CW, FH, FW, epilogue, Y, OH, OW, N, IC, OC, sh, sw, ph, pw)
+
+    @staticmethod
+    def conv3D_winograd_fused(streamArray, length, X, IH, IW, U, epilogue, Y, OH, OW, N, IC, OC, ph, pw):
+        _call("alpha_conv3D_winograd_fused", streamArray, length, X, IH, IW, U, epilogue, Y, OH, OW, N, IC, OC, ph, pw)
+
 
 class Cuda_dconv3D_deltaX:
     """Backward-data natives (Cuda_dconv3D_deltaX.java)."""
@@ -245,6 +281,11 @@ class Cuda_dconv3D_deltaX:
     @staticmethod
     def dconv3D_deltaX_winograd(streamArray, length, deltaY, OH, OW, U, deltaX, IH, IW, N, IC, OC, ph, pw):
         _call("alpha_dconv3D_deltaX_winograd", streamArray, length, deltaY, OH, OW, U, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_s1_leakyRelu(streamArray, length, deltaY, OH, OW, W, FH, FW, Xf, k, deltaX, IH, IW, N, IC, OC, ph, pw):
+        """Backward-data times the derivative of the leaky ReLU whose output Xf is this layer's input (fused epilogue)."""
+        _call("alpha_dconv3D_deltaX_s1_leakyRelu", streamArray, length, deltaY, OH, OW, W, FH, FW, Xf, k, deltaX, IH, IW, N, IC, OC, ph, pw)
 
     @staticmethod
     def dconv3D_deltaX_s1_texture(streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):
@@ -339,3 +380,24 @@ class Cuda_dconv3D_deltaW:
                                      deltaB, deltaB_buf, FH, FW, N, IC, OC, sh, sw, ph, pw):
         _call("alpha_dconv3D_deltaW_GemmSK_deltaB", streamArray, length, GridZ, X, IH, IW, deltaY, OH, OW, deltaW, deltaW_buf,
               deltaB, deltaB_buf, FH, FW, N, IC, OC, sh, sw, ph, pw)
+
+
+class Cuda_function:
+    """The row functions the reference applies to convolution outputs (Cuda_function.java:1607, 1640, 3829, 3862), same
+    argument order; one HBM-bound pass each. Only these four: the class's other natives are outside this library."""
+
+    @staticmethod
+    def leakyRelu2D(stream, X, k, Y, lengthv, mem_width, mem_stride):
+        _call("alpha_leakyRelu2D", stream, X, k, Y, lengthv, mem_width, mem_stride)
+
+    @staticmethod
+    def leakyRelu2D_deltaX_v1(stream, deltaX, deltaY, Y, k, lengthv, mem_width, mem_stride):
+        _call("alpha_leakyRelu2D_deltaX_v1", stream, deltaX, deltaY, Y, k, lengthv, mem_width, mem_stride)
+
+    @staticmethod
+    def batchNorm2D_row(stream, X, X_mean, X_var, eps, row_lengthv, Y, lengthv, mem_width, mem_stride):
+        _call("alpha_batchNorm2D_row", stream, X, X_mean, X_var, eps, row_lengthv, Y, lengthv, mem_width, mem_stride)
+
+    @staticmethod
+    def batchNorm_affined2D_row(stream, X, X_mean, X_var, eps, A, B, row_lengthv, Y, lengthv, mem_width, mem_stride):
+        _call("alpha_batchNorm_affined2D_row", stream, X, X_mean, X_var, eps, A, B, row_lengthv, Y, lengthv, mem_width, mem_stride)

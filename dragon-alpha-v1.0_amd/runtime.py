@@ -251,3 +251,52 @@ class Cuda:
     setFrom2Dto1D = staticmethod(lambda s, src, h, w, st, dst, n: _ck(_lib().alpha_rt_setFrom2Dto1D(s, src, h, w, st, dst, n)))
     setFrom2Dto2D = staticmethod(
         lambda s, src, h, w, st, dst, dh, dw, dst_stride: _ck(_lib().alpha_rt_setFrom2Dto2D(s, src, h, w, st, dst, dh, dw, dst_stride)))
+
+
+class DeviceProperties(ctypes.Structure):
+    """alpha_device_properties of include/alpha_rt.h (member for member)."""
+    _I3, _I2 = ctypes.c_int * 3, ctypes.c_int * 2
+    _fields_ = (
+        [("name", ctypes.c_char * 256), ("uuid", ctypes.c_ubyte * 16), ("luid", ctypes.c_ubyte * 8)]
+        + [(n, _I) for n in ("luidDeviceNodeMask", "major", "minor", "pciBusID", "pciDeviceID", "pciDomainID", "multiGpuBoardGroupID",
+                             "computeMode", "deviceOverlap", "integrated", "kernelExecTimeoutEnabled", "unifiedAddressing",
+                             "canMapHostMemory", "canUseHostPointerForRegisteredMem", "directManagedMemAccessFromHost",
+                             "concurrentKernels", "ECCEnabled", "tccDriver", "streamPrioritiesSupported", "globalL1CacheSupported",
+                             "localL1CacheSupported", "managedMemory", "multiGpuBoard", "hostNativeAtomicSupported",
+                             "pageableMemoryAccess", "cooperativeLaunch", "concurrentManagedAccess", "computePreemptionSupported",
+                             "clockRate", "memoryClockRate", "memoryBusWidth")]
+        + [("totalGlobalMemory", _L), ("totalConstMemory", _L)]
+        + [(n, _I) for n in ("l2CacheSize", "persistingL2CacheMaxSize", "multiProcessorCount", "asyncEngineCount")]
+        + [("maxGridSize", _I3), ("singleToDoublePrecisionPerfRatio", _I), ("accessPolicyMaxWindowSize", _I), ("memoryPitch", _L),
+           ("maxThreadsPerMultiProcessor", _I), ("sharedMemPerMultiprocessor", _L), ("regsPerMultiprocessor", _I),
+           ("maxBlocksPerMultiProcessor", _I), ("sharedMemPerBlock", _L), ("reservedSharedMemPerBlock", _L),
+           ("sharedMemPerBlockOptin", _L), ("regsPerBlock", _I), ("maxThreadsPerBlock", _I), ("maxThreadsDim", _I3), ("warpSize", _I),
+           ("textureAlignment", _L), ("texturePitchAlignment", _L), ("maxTexture1D", _I), ("maxTexture1DMipmap", _I),
+           ("maxTexture1DLinear", _I), ("maxTexture2D", _I2), ("maxTexture2DMipmap", _I2), ("maxTexture2DLinear", _I3),
+           ("maxTexture2DGather", _I2), ("maxTexture3D", _I3), ("maxTexture3DAlt", _I3), ("maxTexture1DLayered", _I2),
+           ("maxTexture2DLayered", _I3), ("maxTextureCubemapLayered", _I2), ("surfaceAlignment", _L), ("maxSurface1D", _I),
+           ("maxSurface2D", _I2), ("maxSurface3D", _I3), ("maxSurface1DLayered", _I2), ("maxSurface2DLayered", _I3),
+           ("maxSurfaceCubemap", _I), ("maxSurfaceCubemapLayered", _I2)])
+
+
+class CudaDevice:
+    """Mirror of z.dragon.engine.cuda.impl.CudaDevice (CudaDevice.java:16-215): constructing it runs the class's one native,
+    setProperty(device_id); the properties are then attributes under the Java field names (arrays as lists, the name as str)."""
+
+    def __init__(self, device_id=None):
+        self.id = Cuda.getDeviceId() if device_id is None else int(device_id)
+        props = DeviceProperties()
+        L = _lib()
+        L.alpha_rt_getDeviceProperties.argtypes = [_I, ctypes.POINTER(DeviceProperties)]
+        _ck(L.alpha_rt_getDeviceProperties(self.id, ctypes.byref(props)))
+        for name, ctype in DeviceProperties._fields_:
+            v = getattr(props, name)
+            if name == "name":
+                v = v.decode()
+            elif hasattr(v, "__len__"):
+                v = list(v)
+            setattr(self, name, v)
+
+    @staticmethod
+    def getDevices():
+        return [CudaDevice(i) for i in range(Cuda.getDeviceCount())]

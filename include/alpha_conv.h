@@ -346,6 +346,62 @@ int alpha_dconv3D_deltaW_GemmSK_deltaB(const int64_t *streams, int length, int G
                                        int FH, int FW, int N, int IC, int OC,
                                        int sh, int sw, int ph, int pw);
 
+/* ---- this build's fused epilogues: batch normalisation and leaky ReLU around the convolution ------------------------
+ * The reference runs them as separate passes over the convolution's output: conv3D, then batchNorm2D_row /
+ * batchNorm_affined2D_row (Cuda_function.java:3829, 3862; in inference, statistics given), then leakyRelu2D (:1607) -
+ * after every convolution of its ResNets (experiments/alpha_code/src/cifar10/resnet18/Net.java:42-58) - and, going back,
+ * leakyRelu2D_deltaX_v1 (:1640) before dconv3D_deltaX. Here they ride in the convolution kernels' epilogues where a
+ * kernel has the fused form (the LDS-halo kernels, the stem kernel, the generic kernel, the non-persistent Winograd
+ * kernel) and are one more pass over the output otherwise (1x1 streaming kernel, persistent Winograd kernel). */
+typedef struct alpha_conv_epilogue {
+    const float *Bias;     /* NULL or [OC]: added first */
+    const float *X_mean;   /* NULL or [OC], with X_var: y = (y - X_mean) * rsqrt(X_var + eps) */
+    const float *X_var;
+    float eps;
+    const float *A;        /* NULL or [OC], with B: y = A * y + B */
+    const float *B;
+    float k;               /* leaky ReLU: y = y > 0 ? y : k * y; k = 1 leaves y alone */
+} alpha_conv_epilogue;
+
+/* Y = leakyRelu(batchNorm(conv3D(X, W) + Bias)), filter read as W[OC,FH,FW,IC] (conv/A.cu:14 + the row functions) */
+int alpha_conv3D_fused(const int64_t *streams, int length,
+                       const float *X, int IH, int IW,
+                       const float *W, int FH, int FW,
+                       const alpha_conv_epilogue *epilogue,
+                       float *Y, int OH, int OW,
+                       int N, int IC, int OC, int sh, int sw, int ph, int pw);
+/* the same from the re-laid-out filter CW (conv/A.cu:149) */
+int alpha_conv3D_GemmR_fused(const int64_t *streams, int length,
+                             const float *X, int IH, int IW,
+                             const float *W, const float *CW, int FH, int FW,
+                             const alpha_conv_epilogue *epilogue,
+                             float *Y, int OH, int OW,
+                             int N, int IC, int OC, int sh, int sw, int ph, int pw);
+/* the same through Winograd F(2x2,3x3) from the transformed filter U */
+int alpha_conv3D_winograd_fused(const int64_t *streams, int length,
+                                const float *X, int IH, int IW, const float *U,
+                                const alpha_conv_epilogue *epilogue,
+                                float *Y, int OH, int OW, int N, int IC, int OC, int ph, int pw);
+/* deltaX = dconv3D_deltaX_s1(deltaY, W) * (Xf > 0 ? 1 : k): stride-1 backward-data (dX/A.cu:14) fused with the backward of
+ * the leaky ReLU whose output Xf[N,IH,IW,IC] is this layer's input (leakyRelu2D_deltaX_v1 applied to the result). */
+int alpha_dconv3D_deltaX_s1_leakyRelu(const int64_t *streams, int length,
+                                      const float *deltaY, int OH, int OW,
+                                      const float *W, int FH, int FW,
+                                      const float *Xf, float k,
+                                      float *deltaX, int IH, int IW,
+                                      int N, int IC, int OC, int ph, int pw);
+/* The row functions themselves (one HBM-bound pass; X == Y allowed), argument order of the reference's natives:
+ * lengthv = height * mem_stride elements, mem_width data elements per row, the mem_stride - mem_width pad elements are
+ * written as zeros. row_lengthv (the length of X_mean / X_var) must equal mem_stride. */
+int alpha_leakyRelu2D(int64_t stream, const float *X, float k, float *Y, int lengthv, int mem_width, int mem_stride);
+int alpha_leakyRelu2D_deltaX_v1(int64_t stream, float *deltaX, const float *deltaY, const float *Y, float k,
+                                int lengthv, int mem_width, int mem_stride);
+int alpha_batchNorm2D_row(int64_t stream, const float *X, const float *X_mean, const float *X_var, float eps, int row_lengthv,
+                          float *Y, int lengthv, int mem_width, int mem_stride);
+int alpha_batchNorm_affined2D_row(int64_t stream, const float *X, const float *X_mean, const float *X_var, float eps,
+                                  const float *A, const float *B, int row_lengthv,
+                                  float *Y, int lengthv, int mem_width, int mem_stride);
+
 #ifdef __cplusplus
 }
 #endif

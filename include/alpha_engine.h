@@ -14,6 +14,8 @@
 
 #include <stdint.h>
 
+#include "alpha_conv.h"   /* alpha_conv_epilogue */
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -113,6 +115,12 @@ int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *
 int alpha_engine_conv3D_biased(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W,
                                int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                const float *Bias, int lengthv, int width, alpha_conv_plan *plan_out);
+/* conv3D, batch normalisation with given statistics and leaky ReLU as one operator (this build's addition; the reference
+ * composes eg.conv3D, eg.batchNorm and eg.leakyRelu: experiments/alpha_code/src/cifar10/resnet18/Net.java:42-58). The plan
+ * is conv3D's; the row functions run in the convolution kernel's epilogue where the kernel has the fused form. */
+int alpha_engine_conv3D_fused(alpha_engine *e, float *Y, int OH, int OW, const float *X, int IH, int IW, const float *W,
+                              int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                              const alpha_conv_epilogue *epilogue, alpha_conv_plan *plan_out);
 int alpha_engine_dconv3D_deltaW(alpha_engine *e, float *deltaW, int FH, int FW, const float *X, int IH, int IW,
                                 const float *deltaY, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                 alpha_conv_plan *plan_out);
@@ -124,6 +132,13 @@ int alpha_engine_dconv3D_deltaW_deltaB(alpha_engine *e, float *deltaW, float *de
 int alpha_engine_dconv3D_deltaX(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
                                 const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                 alpha_conv_plan *plan_out);
+
+/* dconv3D_deltaX followed by the backward of the leaky ReLU (slope k) whose output Xf[N,IH,IW,IC] is this layer's input
+ * (eg.leakyRelu_deltaX on the result), as one operator: the plan is dconv3D_deltaX's; the mask is applied in the kernel's
+ * epilogue for the stride-1 entries and by leakyRelu2D_deltaX_v1 in place after the others. */
+int alpha_engine_dconv3D_deltaX_leakyRelu(alpha_engine *e, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,
+                                          const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
+                                          const float *Xf, float k, alpha_conv_plan *plan_out);
 
 #ifdef __cplusplus
 }

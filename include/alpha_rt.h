@@ -39,6 +39,51 @@ int alpha_rt_getDeviceId(int *id);
 int alpha_rt_getDeviceCount(int *count);
 int alpha_rt_setDevice(int dev_id);
 int alpha_rt_resetDevice(void);
+
+/* The device description the reference's class CudaDevice holds (CudaDevice.java:31-215), filled by its one native
+ * `setProperty(int device_id)` (src/cu32_src/CudaDevice/CudaDevice/A.cu:7-330) from cudaGetDeviceProperties. Here it is
+ * filled from hipGetDeviceProperties: same field names and meanings; `major.minor` is the gfx target version (9.5 for
+ * gfx950), warpSize is 64, multiProcessorCount is the number of compute units. The JNI symbol
+ * Java_z_dragon_engine_cuda_impl_CudaDevice_setProperty copies every member into the Java field of the same name. */
+typedef struct alpha_device_properties {
+    char name[256];
+    unsigned char uuid[16];
+    unsigned char luid[8];
+    int luidDeviceNodeMask;
+    int major, minor;
+    int pciBusID, pciDeviceID, pciDomainID;
+    int multiGpuBoardGroupID;
+    int computeMode;
+    int deviceOverlap, integrated, kernelExecTimeoutEnabled, unifiedAddressing, canMapHostMemory;
+    int canUseHostPointerForRegisteredMem, directManagedMemAccessFromHost, concurrentKernels, ECCEnabled, tccDriver;
+    int streamPrioritiesSupported, globalL1CacheSupported, localL1CacheSupported, managedMemory, multiGpuBoard;
+    int hostNativeAtomicSupported, pageableMemoryAccess, cooperativeLaunch, concurrentManagedAccess, computePreemptionSupported;
+    int clockRate, memoryClockRate, memoryBusWidth;
+    int64_t totalGlobalMemory, totalConstMemory;
+    int l2CacheSize, persistingL2CacheMaxSize, multiProcessorCount, asyncEngineCount;
+    int maxGridSize[3];
+    int singleToDoublePrecisionPerfRatio, accessPolicyMaxWindowSize;
+    int64_t memoryPitch;
+    int maxThreadsPerMultiProcessor;
+    int64_t sharedMemPerMultiprocessor;
+    int regsPerMultiprocessor, maxBlocksPerMultiProcessor;
+    int64_t sharedMemPerBlock, reservedSharedMemPerBlock, sharedMemPerBlockOptin;
+    int regsPerBlock, maxThreadsPerBlock;
+    int maxThreadsDim[3];
+    int warpSize;
+    int64_t textureAlignment, texturePitchAlignment;
+    int maxTexture1D, maxTexture1DMipmap, maxTexture1DLinear;
+    int maxTexture2D[2], maxTexture2DMipmap[2], maxTexture2DLinear[3], maxTexture2DGather[2];
+    int maxTexture3D[3], maxTexture3DAlt[3], maxTexture1DLayered[2], maxTexture2DLayered[3], maxTextureCubemapLayered[2];
+    int64_t surfaceAlignment;
+    int maxSurface1D;
+    int maxSurface2D[2], maxSurface3D[3], maxSurface1DLayered[2], maxSurface2DLayered[3];
+    int maxSurfaceCubemap;
+    int maxSurfaceCubemapLayered[2];
+} alpha_device_properties;
+
+/* CudaDevice/A.cu:7-12 (cudaGetDeviceProperties) */
+int alpha_rt_getDeviceProperties(int device_id, alpha_device_properties *out);
 int alpha_rt_deviceSynchronize(void);
 int alpha_rt_isDeviceP2PAccessEnabled(int dev1_id, int dev2_id, int *enabled);
 int alpha_rt_enableDeviceP2PAccess(int dev2_id);

@@ -1,7 +1,10 @@
 """A fake JNIEnv for driving the JNI symbols without a JVM: a function table with the slots the shims use at the
-indices the JNI specification assigns them (6 FindClass, 14 ThrowNew, 17 ExceptionClear, 167 NewStringUTF,
-179 NewIntArray, 200/203/204/205 Get{Byte,Int,Long,Float}ArrayRegion, 208/211/213 Set{Byte,Int,Float}ArrayRegion).
-A Java array is modelled as an integer key into a dict of Python lists; a jstring as a key into a dict of strings."""
+indices the JNI specification assigns them (6 FindClass, 14 ThrowNew, 17 ExceptionClear, 31 GetObjectClass, 94 GetFieldID,
+104/105/109/110 Set{Object,Boolean,Int,Long}Field, 167 NewStringUTF, 176 NewByteArray, 179 NewIntArray,
+200/203/204/205 Get{Byte,Int,Long,Float}ArrayRegion, 208/211/213 Set{Byte,Int,Float}ArrayRegion).
+A Java array is modelled as an integer key into a dict of Python lists; a jstring as a key into a dict of strings; a Java
+object (new_object) as a key into a dict of {field name: value} whose class declares a given set of (name, signature)
+fields - GetFieldID returns NULL for a field the class does not declare, or declares with another signature."""
 import ctypes
 
 SLOT_COUNT = 235
@@ -68,7 +71,50 @@ class FakeEnv:
             self.arrays[key] = [0] * n
             return key
 
-        extra = {167: NEWSTR(newstr), 179: NEWINTS(newints),
+        # ---- objects and fields (CudaDevice.setProperty) ----
+        self.objects = {}         # object handle -> {field name: value}
+        self.declared = {}        # class handle -> {field name: signature}
+        self.class_of = {}        # object handle -> class handle
+        self.field_ids = {}       # field id -> (name, signature)
+        self.set_calls = []       # (setter kind, field name) in call order
+        V = ctypes.c_void_p
+        GETCLS = ctypes.CFUNCTYPE(V, V, V)
+        GETFID = ctypes.CFUNCTYPE(V, V, V, ctypes.c_char_p, ctypes.c_char_p)
+        SETOBJ = ctypes.CFUNCTYPE(None, V, V, V, V)
+        SETBOOL = ctypes.CFUNCTYPE(None, V, V, V, ctypes.c_uint8)
+        SETINT = ctypes.CFUNCTYPE(None, V, V, V, ctypes.c_int32)
+        SETLONG = ctypes.CFUNCTYPE(None, V, V, V, ctypes.c_int64)
+
+        def getcls(env, obj):
+            return self.class_of[obj]
+
+        def getfid(env, cls, name, sig):
+            name, sig = name.decode(), sig.decode()
+            if self.declared[cls].get(name) != sig:
+                return None
+            fid = 0x5000 + len(self.field_ids)
+            self.field_ids[fid] = (name, sig)
+            return fid
+
+        def setter(kind, expect):
+            def put(env, obj, fid, value):
+                name, sig = self.field_ids[fid]
+                assert sig in expect, "Set%sField on field %s of type %s" % (kind, name, sig)
+                self.set_calls.append((kind, name))
+                if kind == "Object":
+                    value = self.strings[value] if value in self.strings else self.arrays[value]
+                self.objects[obj][name] = bool(value) if kind == "Boolean" else value
+            return put
+
+        def newbytes(env, n):
+            key = 0x2000 + len(self.arrays)
+            self.arrays[key] = [0] * n
+            return key
+
+        extra = {31: GETCLS(getcls), 94: GETFID(getfid),
+                 104: SETOBJ(setter("Object", ("Ljava/lang/String;", "[B", "[I"))), 105: SETBOOL(setter("Boolean", ("Z",))),
+                 109: SETINT(setter("Int", ("I",))), 110: SETLONG(setter("Long", ("J",))), 176: NEWINTS(newbytes),
+                 167: NEWSTR(newstr), 179: NEWINTS(newints),
                  200: region_cb(ctypes.c_int8, False), 203: region_cb(ctypes.c_int32, False), 205: region_cb(ctypes.c_float, False),
                  208: region_cb(ctypes.c_int8, True), 211: region_cb(ctypes.c_int32, True), 213: region_cb(ctypes.c_float, True)}
         self._cbs = (FIND(find), THROWNEW(thrownew), CLEAR(clear), GETLONG(getlong)) + tuple(extra.values())
@@ -82,6 +128,15 @@ class FakeEnv:
         self._table = table
         self._env = ctypes.c_void_p(ctypes.addressof(table))   # JNIEnv_ { const JNINativeInterface_* functions; }
         self.ptr = ctypes.pointer(self._env)
+
+    def new_object(self, declared_fields):
+        """A Java object whose class declares {field name: JNI signature}; returns its handle."""
+        cls = 0x4000 + len(self.declared)
+        self.declared[cls] = dict(declared_fields)
+        obj = 0x6000 + len(self.objects)
+        self.objects[obj] = {}
+        self.class_of[obj] = cls
+        return obj
 
     def array(self, values):
         """A Java primitive array of any element type (byte[], int[], float[]); returns its handle."""

@@ -114,3 +114,117 @@ def test_runtime_class_stubs_that_need_no_device():
     jni("deleteStream__J", None, L)(0)                      # a zero handle is skipped without touching the device
     jni("deleteStream___3JI", None, P, I)(env.long_array([0, 0]), 2)
     assert len(env.thrown) == 1
+
+
+# ---- CudaDevice.setProperty -------------------------------------------------------------------------------------------
+# the fields of the reference's class z.dragon.engine.cuda.impl.CudaDevice that its native fills (CudaDevice.java:31-215),
+# with their JNI signatures
+DEVICE_FIELDS = dict(
+    [("name", "Ljava/lang/String;"), ("uuid", "[B"), ("luid", "[B")]
+    + [(n, "I") for n in ("luidDeviceNodeMask", "major", "minor", "pciBusID", "pciDeviceID", "pciDomainID", "multiGpuBoardGroupID",
+                          "computeMode", "clockRate", "memoryClockRate", "memoryBusWidth", "l2CacheSize", "persistingL2CacheMaxSize",
+                          "multiProcessorCount", "asyncEngineCount", "singleToDoublePrecisionPerfRatio", "accessPolicyMaxWindowSize",
+                          "maxThreadsPerMultiProcessor", "regsPerMultiprocessor", "maxBlocksPerMultiProcessor", "regsPerBlock",
+                          "maxThreadsPerBlock", "warpSize", "maxTexture1D", "maxTexture1DMipmap", "maxTexture1DLinear", "maxSurface1D",
+                          "maxSurfaceCubemap")]
+    + [(n, "Z") for n in ("deviceOverlap", "integrated", "kernelExecTimeoutEnabled", "unifiedAddressing", "canMapHostMemory",
+                          "canUseHostPointerForRegisteredMem", "directManagedMemAccessFromHost", "concurrentKernels", "ECCEnabled",
+                          "tccDriver", "streamPrioritiesSupported", "globalL1CacheSupported", "localL1CacheSupported", "managedMemory",
+                          "multiGpuBoard", "hostNativeAtomicSupported", "pageableMemoryAccess", "cooperativeLaunch",
+                          "concurrentManagedAccess", "computePreemptionSupported")]
+    + [(n, "J") for n in ("totalGlobalMemory", "totalConstMemory", "memoryPitch", "sharedMemPerMultiprocessor", "sharedMemPerBlock",
+                          "reservedSharedMemPerBlock", "sharedMemPerBlockOptin", "textureAlignment", "texturePitchAlignment",
+                          "surfaceAlignment")]
+    + [(n, "[I") for n in ("maxGridSize", "maxThreadsDim", "maxTexture2D", "maxTexture2DMipmap", "maxTexture2DLinear",
+                           "maxTexture2DGather", "maxTexture3D", "maxTexture3DAlt", "maxTexture1DLayered", "maxTexture2DLayered",
+                           "maxTextureCubemapLayered", "maxSurface2D", "maxSurface3D", "maxSurface1DLayered", "maxSurface2DLayered",
+                           "maxSurfaceCubemapLayered")])
+
+
+def _known_properties():
+    """A struct in which every member holds a different value."""
+    P = pkg.runtime.DeviceProperties
+    props, want = P(), {}
+    k = 100
+    for name, ctype in P._fields_:
+        if name == "name":
+            props.name = b"fake device gfx950"
+            want[name] = "fake device gfx950"
+        elif name in ("uuid", "luid"):
+            vals = [(k + 7 * i) % 127 for i in range(len(getattr(props, name)))]
+            for i, v in enumerate(vals):
+                getattr(props, name)[i] = v
+            want[name] = vals
+        elif hasattr(getattr(props, name), "__len__"):
+            vals = [k + i for i in range(len(getattr(props, name)))]
+            for i, v in enumerate(vals):
+                getattr(props, name)[i] = v
+            want[name] = vals
+        elif DEVICE_FIELDS[name] == "Z":
+            setattr(props, name, k % 2)
+            want[name] = bool(k % 2)
+        elif DEVICE_FIELDS[name] == "J":
+            setattr(props, name, (k << 33) + 5)     # needs all 64 bits
+            want[name] = (k << 33) + 5
+        else:
+            setattr(props, name, k)
+            want[name] = k
+        k += 3
+    return props, want
+
+
+def test_device_native_is_exported_and_the_struct_has_the_java_fields():
+    out = subprocess.check_output(["nm", "-D", "--defined-only", pkg.lib_path()], text=True)
+    assert "Java_z_dragon_engine_cuda_impl_CudaDevice_setProperty" in out
+    assert sorted(n for n, _ in pkg.runtime.DeviceProperties._fields_) == sorted(DEVICE_FIELDS)
+    assert len(DEVICE_FIELDS) == 77
+
+
+def test_device_properties_reach_every_java_field_with_its_type():
+    env = FakeEnv()
+    obj = env.new_object(DEVICE_FIELDS)
+    props, want = _known_properties()
+    fn = pkg.lib().alpha_rt_selfcheck_fillDeviceObject
+    fn.restype = None
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(pkg.runtime.DeviceProperties)]
+    fn(env.ptr, obj, ctypes.byref(props))
+    got = env.objects[obj]
+    assert sorted(got) == sorted(DEVICE_FIELDS)                      # every field set ...
+    assert len(env.set_calls) == len(DEVICE_FIELDS)                  # ... exactly once
+    for name in DEVICE_FIELDS:
+        assert got[name] == want[name], name
+    # a Java class that lacks a field (an older CudaDevice): the others are still filled
+    fewer = {k: v for k, v in DEVICE_FIELDS.items() if k != "maxTexture1DLinear"}
+    obj2 = env.new_object(fewer)
+    fn(env.ptr, obj2, ctypes.byref(props))
+    assert sorted(env.objects[obj2]) == sorted(fewer)
+
+
+@pytest.mark.gpu
+def test_device_properties_of_the_real_device_through_the_jni_symbol():
+    import torch
+    assert torch.cuda.is_available()
+    env = FakeEnv()
+    obj = env.new_object(DEVICE_FIELDS)
+    fn = _jni("Java_z_dragon_engine_cuda_impl_CudaDevice_setProperty")
+    fn.restype = None
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32]
+    fn(env.ptr, obj, 0)
+    assert not env.thrown
+    got = env.objects[obj]
+    assert sorted(got) == sorted(DEVICE_FIELDS)
+    tp = torch.cuda.get_device_properties(0)
+    assert got["name"] == tp.name
+    assert got["multiProcessorCount"] == tp.multi_processor_count == pkg.device_info()[0]
+    assert got["totalGlobalMemory"] == tp.total_memory
+    assert got["warpSize"] == 64 and (got["major"], got["minor"]) == (tp.major, tp.minor)
+    assert got["maxThreadsPerBlock"] == 1024 and got["maxThreadsDim"][0] == 1024
+    assert got["clockRate"] == pkg.device_info()[1]
+    # the ctypes mirror of the Java class reads the same struct
+    d = pkg.CudaDevice(0)
+    assert (d.name, d.multiProcessorCount, d.l2CacheSize) == (got["name"], got["multiProcessorCount"], got["l2CacheSize"])
+    assert len(pkg.CudaDevice.getDevices()) == pkg.Cuda.getDeviceCount()
+    # an invalid device id becomes a Java exception, not a crash
+    env2 = FakeEnv()
+    fn(env2.ptr, env2.new_object(DEVICE_FIELDS), 99)
+    assert env2.thrown and env2.thrown[0][0] == "z/dragon/engine/cuda/impl/CudaException"
