@@ -191,6 +191,12 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
                            int b_off, int b_sth, int b_stw, int b_sc, const float *bias = nullptr, int sh = 1, int sw = 1,
                            int b_sn = 1, const Epilogue *ep = nullptr);
 
+// Kernel-split backward-data for stride 2 x 2, all four phases in one launch of the LDS-halo kernel (tap_conv.hip).
+hipError_t launch_tap_conv_merged(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC, int CO,
+                                  int OHt, int OWt, const int *TH, const int *TW, const int *ph, const int *pw, const int *b_off,
+                                  const int *b_sth, int b_stw, int b_sc, const int *o_off, int o_sn, int o_sh, int o_sw,
+                                  const Epilogue *ep = nullptr);
+
 // 1x1 stride-1 convolution as a streaming GEMM with the filter resident in LDS (pointwise.hip):
 // O[(n,oh,ow)][co] = sum_k A[n, oh*sh, ow*sw, k] * B(k, co), B given as [K][N] (b_kmajor) or [N][K]. Returns
 // hipErrorNotSupported (nothing launched) when the shape does not fit.

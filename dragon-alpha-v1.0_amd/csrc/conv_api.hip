@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <vector>
 
 using namespace alpha;
 
@@ -181,7 +182,7 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
 // iw = iws (mod sw). from_CW: filter taken from the v2 kernel-split layout; otherwise from W in place.
 int deltaX_phases(const char *fn, const int64_t *streams, int length,
                   const float *dY, int OH, int OW, const float *F, bool from_CW, int FH, int FW,
-                  float *dX, int IH, int IW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+                  float *dX, int IH, int IW, int N, int IC, int OC, int sh, int sw, int ph, int pw, const Epilogue *ep = nullptr)
 {
     if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
     if (!dY || !F || !dX || !aligned16(dY) || !aligned16(F) || !aligned16(dX))
@@ -191,6 +192,10 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
     const int mCFH = (FH + sh - 1) / sh, mCFW = (FW + sw - 1) / sw;
     const int CWstride = mCFH * mCFW * OC * IC;
     hipStream_t s = stream0(streams);
+    if (sh * sw > 64) return fail(ALPHA_CONV_EINVAL, "%s: more than 64 phases (sh*sw)", fn);
+    // the phases as dense stride-1 problems
+    struct Phase { GatherConvArgs a; int th, tw, OHt, OWt; };
+    std::vector<Phase> phases;
     for (int y = 0; y < sh; y++)
         for (int x = 0; x < sw; x++) {
             const int CFH = (FH - y + sh - 1) / sh, CFW = (FW - x + sw - 1) / sw;
@@ -203,6 +208,7 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
 
             GatherConvArgs a{};
             a.A = dY; a.B = F; a.O = dX;
+            a.ep = ep ? *ep : bias_epilogue(nullptr);
             a.CO = IC;
             a.AH = OH; a.AW = OW; a.AC = OC;
             a.sh = 1; a.sw = 1;
@@ -218,8 +224,24 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
             }
             const int th = CFH > 0 && CFW > 0 ? CFH : 0, tw = CFH > 0 && CFW > 0 ? CFW : 0;
             if (th == 0) a.b_off = 0;
-            if (int e = hip_status(launch_gather_conv(s, a, th, tw, OHt, OWt, N), fn)) return e;
+            phases.push_back(Phase{a, th, tw, OHt, OWt});
         }
+    // Stride 2 x 2 with even sizes (the reference's Ims2 case): the four phases in ONE launch, sharing one LDS halo per
+    // unit (the reference runs its phases in one grid too: dconv3D_dX_kernelSplit_Ims2R_kernel.cuh:18, dim3(.., .., 4)).
+    // Everything else, and whatever that kernel refuses: one launch of the generic kernel per phase.
+    if (fwd_algo() != 3 && sh == 2 && sw == 2 && (IH & 1) == 0 && (IW & 1) == 0 && phases.size() == 4) {
+        int TH[4], TW[4], pph[4], ppw[4], boff[4], bsth[4], ooff[4];
+        for (int f = 0; f < 4; f++) {
+            const GatherConvArgs &a = phases[f].a;
+            TH[f] = phases[f].th; TW[f] = phases[f].tw; pph[f] = a.ph; ppw[f] = a.pw; boff[f] = a.b_off; bsth[f] = a.b_sth; ooff[f] = a.o_off;
+        }
+        const GatherConvArgs &a0 = phases[0].a;
+        hipError_t e = launch_tap_conv_merged(s, dY, F, dX, N, OH, OW, OC, IC, phases[0].OHt, phases[0].OWt, TH, TW, pph, ppw, boff, bsth,
+                                              a0.b_stw, a0.b_sc, ooff, a0.o_sn, a0.o_sh, a0.o_sw, ep);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
+    for (const Phase &f : phases)
+        if (int e = hip_status(launch_gather_conv(s, f.a, f.th, f.tw, f.OHt, f.OWt, N), fn)) return e;
     return 0;
 }
 

@@ -42,9 +42,22 @@ struct TapConvArgs {
     int pieces;       // the remaining units cut into piece_split pieces of piece_tiles tiles each, one piece per workgroup
     int piece_split, piece_tiles;
     FastDiv d_OW, d_OHW, d_PHt, d_PWt, d_sw;
+    // merged kernel-split backward-data only (tap_conv_merged_kernel): output pixel (n, i, j) of phase f goes to
+    // O + f_o_off[f] + n*o_sn + i*o_sh + j*o_sw; tap (th, tw) of phase f reads the halo at (row + th + f_row[f],
+    // column + tw + f_col[f]) and the filter at f_b_off[f] + th*f_b_sth[f] + tw*b_stw + c*b_sc + co
+    int o_sn, o_sh, o_sw;
+    int f_TH[4], f_TW[4], f_row[4], f_col[4], f_b_off[4], f_b_sth[4], f_o_off[4];
 };
 
 template <int V> struct TapInt { static constexpr int value = V; };
+template <int I, int N, class F>
+static __device__ __forceinline__ void pf_phase_loop(F &&f)
+{
+    if constexpr (I < N) {
+        f(TapInt<I>{});
+        pf_phase_loop<I + 1, N>(f);
+    }
+}
 constexpr int TC_ICC = 64;            // input channels per halo pass
 constexpr int TC_PS = TC_ICC + 8;     // LDS pixel stride (floats)
 constexpr int TC_OS = 64 + 4;         // output staging row stride (floats)
@@ -71,6 +84,68 @@ __host__ __device__ __forceinline__ unsigned tap_filter_lane_bytes(int b_sc, int
     return (unsigned)(((16 * g + 4 * q + s) * b_sc + co) * 4);
 }
 
+// Stages the zero-padded input rows pgr0 .. pgr0 + rows - 1 ("padded global rows" n*PHt + ih + ph), channels
+// ic0 .. ic0 + 63, into Hs[row][sw planes][PWp][TC_PS]: zero outside the image and beyond AC. A thread keeps its place in
+// the row: 16 lanes per pixel (64 channels), padded column 16*cg + t/16 of column group cg. What depends on the column is
+// computed once per 64 columns, what depends on the row is uniform (scalar registers); per element the vector unit is
+// left with two address operations and the zero-fill selects. (Computing pixel, row and column of every element from a
+// flat index cost ~60 vector instructions per element, and those take issue slots from the MFMAs of the workgroup that
+// shares the compute unit.) A step stages RS rows of CGS column groups (16 columns each), at most eight loads in flight
+// per thread; narrow images take more rows per step, wide ones more column groups (and several trips along the row).
+static __device__ __forceinline__ void tap_stage_halo(const TapConvArgs &p, float *Hs, const int ic0, const int pgr0, const int rows, const int t)
+{
+    const int PHt = p.PHt, PWt = p.PWt, RP = p.RP;
+    auto stage = [&](auto cgs_c, auto rs_c) {
+        constexpr int CGS = decltype(cgs_c)::value, RS = decltype(rs_c)::value;
+        const int cq4 = (t & 15) * 4;
+        const bool ch_ok = ic0 + cq4 < p.AC;
+        const int row_floats = RP * TC_PS, spare = p.lds_rows * row_floats;
+        for (int c0 = 0; c0 < PWt; c0 += 16 * CGS) {
+            int goff[CGS], loff[CGS];
+            bool cok[CGS];
+#pragma unroll
+            for (int cg = 0; cg < CGS; cg++) {
+                const int cp = c0 + 16 * cg + (t >> 4), iw = cp - p.pw;
+                cok[cg] = cp < PWt && (unsigned)iw < (unsigned)p.AW && ch_ok;
+                goff[cg] = cok[cg] ? iw * p.AC + ic0 + cq4 : 0;
+                const int cq = fdiv(cp, p.d_sw), cr = cp - cq * p.sw;
+                // threads past the end of the row write their zeros to a spare slot behind the halo
+                loff[cg] = cp < PWt ? (cr * p.PWp + cq) * TC_PS + cq4 : spare;
+            }
+            for (int r = 0; r < rows; r += RS) {
+                float4 v[RS][CGS];
+                bool rok[RS];
+#pragma unroll
+                for (int rr = 0; rr < RS; rr++) {
+                    const int pgr = pgr0 + min(r + rr, rows - 1);   // past the last row: the last row again
+                    const int n = fdiv(pgr, p.d_PHt), ih = pgr - n * PHt - p.ph;
+                    rok[rr] = (unsigned)ih < (unsigned)p.AH;
+                    const int rowbase = rok[rr] ? (n * p.AH + ih) * p.AW * p.AC : 0;
+                    const int rowmask = rok[rr] ? -1 : 0;
+#pragma unroll
+                    for (int cg = 0; cg < CGS; cg++)   // outside the image: element 0, zeroed below
+                        v[rr][cg] = *reinterpret_cast<const float4 *>(p.A + rowbase + (goff[cg] & rowmask));
+                }
+#pragma unroll
+                for (int rr = 0; rr < RS; rr++) {
+                    const int rowoff = min(r + rr, rows - 1) * row_floats;
+#pragma unroll
+                    for (int cg = 0; cg < CGS; cg++) {
+                        const bool ok = rok[rr] && cok[cg];   // per-component selects keep v[] in registers
+                        const int dst = loff[cg] == spare ? spare : rowoff + loff[cg];
+                        *reinterpret_cast<float4 *>(Hs + dst) = make_float4(ok ? v[rr][cg].x : 0.f, ok ? v[rr][cg].y : 0.f,
+                                                                            ok ? v[rr][cg].z : 0.f, ok ? v[rr][cg].w : 0.f);
+                    }
+                }
+            }
+        }
+    };
+    if (PWt <= 16) stage(TapInt<1>{}, TapInt<8>{});
+    else if (PWt <= 32) stage(TapInt<2>{}, TapInt<4>{});
+    else if (PWt <= 48) stage(TapInt<3>{}, TapInt<2>{});
+    else stage(TapInt<4>{}, TapInt<2>{});
+}
+
 // RAGGED: AC is not a multiple of 64, so the last pass has channels beyond AC whose filter fragments
 // must be zeroed (kept out of the common case: the extra selects would pull the wait for the
 // prefetched fragment in front of the MFMAs).
@@ -84,7 +159,7 @@ __device__ __forceinline__ void tap_conv_unit(const TapConvArgs &p, float *smem,
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
     const int l16 = lane & 15, q = lane >> 4;
-    const int OW = p.d_OW.d, OHW = p.d_OHW.d, PHt = p.PHt, PWt = p.PWt, RP = p.RP;
+    const int OW = p.d_OW.d, OHW = p.d_OHW.d, PHt = p.PHt, RP = p.RP;
 
     // first padded global row held in LDS, and how many rows this unit needs (<= p.lds_rows, host-checked)
     const int n_first = fdiv(m0, p.d_OHW);
@@ -193,63 +268,8 @@ __device__ __forceinline__ void tap_conv_unit(const TapConvArgs &p, float *smem,
         // wavefront of the other workgroup at the same priority hardly ever gets a turn: staging ended exactly
         // when the other workgroup's MFMA loop did. Staging and the epilogue therefore run at a raised priority.
         __builtin_amdgcn_s_setprio(2);
-        // ---- stage the halo row by row, zero outside the image / beyond AC. A thread keeps its place in the row:
-        // 16 lanes per pixel (64 channels), padded column 16*cg + t/16 of column group cg. What depends on the
-        // column is computed once per 64 columns, what depends on the row is uniform (scalar registers); per
-        // element the vector unit is left with two address operations and the zero-fill selects. (Computing
-        // pixel, row and column of every element from a flat index cost ~60 vector instructions per element, and
-        // those take issue slots from the MFMAs of the workgroup that shares the compute unit.)
-        // A step stages RS rows of CGS column groups (16 columns each), at most eight loads in flight per thread;
-        // narrow images take more rows per step, wide ones more column groups (and several trips along the row).
-        auto stage = [&](auto cgs_c, auto rs_c) {
-            constexpr int CGS = decltype(cgs_c)::value, RS = decltype(rs_c)::value;
-            const int cq4 = (t & 15) * 4;
-            const bool ch_ok = ic0 + cq4 < p.AC;
-            const int row_floats = RP * TC_PS, spare = p.lds_rows * row_floats;
-            for (int c0 = 0; c0 < PWt; c0 += 16 * CGS) {
-                int goff[CGS], loff[CGS];
-                bool cok[CGS];
-#pragma unroll
-                for (int cg = 0; cg < CGS; cg++) {
-                    const int cp = c0 + 16 * cg + (t >> 4), iw = cp - p.pw;
-                    cok[cg] = cp < PWt && (unsigned)iw < (unsigned)p.AW && ch_ok;
-                    goff[cg] = cok[cg] ? iw * p.AC + ic0 + cq4 : 0;
-                    const int cq = fdiv(cp, p.d_sw), cr = cp - cq * p.sw;
-                    // threads past the end of the row write their zeros to a spare slot behind the halo
-                    loff[cg] = cp < PWt ? (cr * p.PWp + cq) * TC_PS + cq4 : spare;
-                }
-                for (int r = 0; r < rows; r += RS) {
-                    float4 v[RS][CGS];
-                    bool rok[RS];
-#pragma unroll
-                    for (int rr = 0; rr < RS; rr++) {
-                        const int pgr = pgr0 + min(r + rr, rows - 1);   // past the last row: the last row again
-                        const int n = fdiv(pgr, p.d_PHt), ih = pgr - n * PHt - p.ph;
-                        rok[rr] = (unsigned)ih < (unsigned)p.AH;
-                        const int rowbase = rok[rr] ? (n * p.AH + ih) * p.AW * p.AC : 0;
-                        const int rowmask = rok[rr] ? -1 : 0;
-#pragma unroll
-                        for (int cg = 0; cg < CGS; cg++)   // outside the image: element 0, zeroed below
-                            v[rr][cg] = *reinterpret_cast<const float4 *>(p.A + rowbase + (goff[cg] & rowmask));
-                    }
-#pragma unroll
-                    for (int rr = 0; rr < RS; rr++) {
-                        const int rowoff = min(r + rr, rows - 1) * row_floats;
-#pragma unroll
-                        for (int cg = 0; cg < CGS; cg++) {
-                            const bool ok = rok[rr] && cok[cg];   // per-component selects keep v[] in registers
-                            const int dst = loff[cg] == spare ? spare : rowoff + loff[cg];
-                            *reinterpret_cast<float4 *>(Hs + dst) = make_float4(ok ? v[rr][cg].x : 0.f, ok ? v[rr][cg].y : 0.f,
-                                                                                ok ? v[rr][cg].z : 0.f, ok ? v[rr][cg].w : 0.f);
-                        }
-                    }
-                }
-            }
-        };
-        if (PWt <= 16) stage(TapInt<1>{}, TapInt<8>{});
-        else if (PWt <= 32) stage(TapInt<2>{}, TapInt<4>{});
-        else if (PWt <= 48) stage(TapInt<3>{}, TapInt<2>{});
-        else stage(TapInt<4>{}, TapInt<2>{});
+        // ---- stage the halo (at raised priority, see above) ----
+        tap_stage_halo(p, Hs, ic0, pgr0, rows, t);
         __syncthreads();
 
         // ---- main loop: one tap (four 16-channel chunks) per iteration ------------------------------------
@@ -316,6 +336,231 @@ __device__ __forceinline__ void tap_conv_unit(const TapConvArgs &p, float *smem,
         if (m < m_lim && oc0 + cq < p.CO)
             *reinterpret_cast<float4 *>(p.O + (size_t)m * p.CO + oc0 + cq) =
                 epilogue4(*reinterpret_cast<const float4 *>(Os + pix * TC_OS + cq), p.ep, oc0 + cq, (size_t)m * p.CO + oc0 + cq);
+    }
+}
+
+// Kernel-split backward-data for stride 2 x 2 with all four phases in ONE unit. The four output pixels of a 2 x 2 block
+// (one per phase) read the same small window of deltaY, each through its own subset of the filter taps, so a unit of
+// P "coarse" pixels stages the halo once per 64 channels and runs every tap of every phase on it - as many MFMAs per
+// staged byte as a dense convolution with the whole filter, where a phase on its own has a quarter of them (one to four
+// taps of a 3x3 filter). Accumulators exist per phase (compile-time index); the sequence of taps runs through the phases,
+// filter fragments and input fragments prefetched across phase and pass boundaries exactly as in tap_conv_unit.
+// A phase without taps (filter smaller than the stride) keeps its zeros and writes them.
+template <int TILES, bool RAGGED>
+__device__ __forceinline__ void tap_conv_merged_unit(const TapConvArgs &p, float *smem, const int m0, const int m_lim, const int oc0)
+{
+    constexpr int P = TILES * 16, NPH = 4;
+    float *Hs = smem;
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, w = t >> 6;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int OW = p.d_OW.d, OHW = p.d_OHW.d, PHt = p.PHt, RP = p.RP;
+
+    const int n_first = fdiv(m0, p.d_OHW);
+    const int oh_first = fdiv(m0 - n_first * OHW, p.d_OW);
+    const int pgr0 = n_first * PHt + oh_first;
+    const int m_last = min(m0 + P, m_lim) - 1;
+    const int n_last = fdiv(m_last, p.d_OHW);
+    const int oh_last = fdiv(m_last - n_last * OHW, p.d_OW);
+    const int rows = n_last * PHt + oh_last + p.TH - 1 - pgr0 + 1;   // p.TH, p.TW: the window all phases read together
+
+    int abase[TILES];
+#pragma unroll
+    for (int i = 0; i < TILES; i++) {
+        const int m = min(m0 + 16 * i + l16, m_lim - 1);
+        const int n = fdiv(m, p.d_OHW), rem = m - n * OHW;
+        const int oh = fdiv(rem, p.d_OW), ow = rem - oh * OW;
+        abase[i] = ((n * PHt + oh - pgr0) * RP + ow) * TC_PS + 4 * q;
+    }
+
+    floatx4 acc[NPH][TILES];
+#pragma unroll
+    for (int f = 0; f < NPH; f++)
+#pragma unroll
+        for (int i = 0; i < TILES; i++) acc[f][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int b_co = oc0 + 16 * w + l16;
+    const bool b_cov = b_co < p.CO;
+    unsigned b_lane[2][4];
+#pragma unroll
+    for (int g = 0; g < 2; g++)
+#pragma unroll
+        for (int s = 0; s < 4; s++) b_lane[g][s] = tap_filter_lane_bytes(p.b_sc, g, q, s, b_cov ? b_co : 0);
+    auto load_b = [&](float (&b)[2][4], int icbase, int f, int th, int tw) {   // f, th, tw uniform
+        const int sbase = __builtin_amdgcn_readfirstlane(
+            tap_filter_half_tap_base<RAGGED>(p.f_b_off[f], p.f_b_sth[f], p.b_stw, p.b_sc, p.AC, icbase, th, tw));
+        const char *sb = reinterpret_cast<const char *>(p.B + sbase);
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const unsigned ok = tap_filter_lane_mask<RAGGED>(p.AC, icbase, g, q);
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                if (!RAGGED) asm volatile("" : "+v"(b_lane[g][s]));
+                b[g][s] = *reinterpret_cast<const float *>(sb + (b_lane[g][s] & ok));
+            }
+        }
+    };
+    auto mask_b = [&](float (&b)[2][4], int icbase) {
+        if (!RAGGED) return;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const bool ok = icbase + 16 * g + 4 * q < p.AC;
+#pragma unroll
+            for (int s = 0; s < 4; s++) b[g][s] = ok ? b[g][s] : 0.f;
+        }
+    };
+    // the first phase that has taps, from phase f on (NPH when there is none); uniform
+    auto next_phase = [&](int f) {
+        while (f < NPH && p.f_TH[f] * p.f_TW[f] == 0) f++;
+        return f;
+    };
+    auto tap_offset = [&](int f, int th, int tw) { return ((th + p.f_row[f]) * RP + tw + p.f_col[f]) * TC_PS; };
+
+    int cur[TILES];
+    auto read_a = [&](floatx4 (&a)[TILES], int ck) {
+#pragma unroll
+        for (int i = 0; i < TILES; i++) a[i] = *reinterpret_cast<const floatx4 *>(Hs + cur[i] + 16 * ck);
+    };
+    auto spread_reads = [&]() {
+#pragma unroll
+        for (int i = 0; i < TILES; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+
+    const int f0 = next_phase(0);
+    if (f0 < NPH) {
+        float bA[2][4], bB[2][4];
+        floatx4 aP[TILES], aQ[TILES];
+        load_b(bA, 0, f0, 0, 0);
+        for (int ic0 = 0; ic0 < p.AC; ic0 += TC_ICC) {
+            if (ic0 > 0) __syncthreads();
+            __builtin_amdgcn_s_setprio(2);
+            tap_stage_halo(p, Hs, ic0, pgr0, rows, t);
+            __syncthreads();
+            __builtin_amdgcn_s_setprio(0);
+            int coff = tap_offset(f0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < TILES; i++) cur[i] = abase[i] + coff;
+            read_a(aP, 0);
+            pf_phase_loop<0, NPH>([&](auto fc) {
+                constexpr int F = decltype(fc)::value;
+                auto mfma_chunk = [&](const floatx4 (&a)[TILES], const float (&b)[4]) {
+#pragma unroll
+                    for (int s = 0; s < 4; s++)
+#pragma unroll
+                        for (int i = 0; i < TILES; i++)
+                            acc[F][i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i][s], b[s], acc[F][i], 0, 0, 0);
+                };
+                const int TWf = p.f_TW[F], taps = p.f_TH[F] * TWf;
+                int th = 0, tw = 0;
+                for (int tap = 0; tap < taps; tap++) {
+                    // what comes next: the phase's next tap, the first tap of the next phase that has any, or - after
+                    // the last phase - the first tap of the next pass (of this pass again at the very end: unused)
+                    int nf = F, nth = th, ntw = tw + 1, nic = ic0;
+                    if (ntw == TWf) { ntw = 0; nth = th + 1; }
+                    if (tap + 1 == taps) {
+                        nth = 0; ntw = 0;
+                        nf = next_phase(F + 1);
+                        if (nf == NPH) { nf = f0; nic = ic0 + TC_ICC < p.AC ? ic0 + TC_ICC : ic0; }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_b(bB, ic0 + 32, F, th, tw);
+                    __builtin_amdgcn_sched_barrier(0);
+                    mask_b(bA, ic0);
+                    read_a(aQ, 1);
+                    mfma_chunk(aP, bA[0]);
+                    spread_reads();
+                    __builtin_amdgcn_sched_barrier(0);
+                    read_a(aP, 2);
+                    mfma_chunk(aQ, bA[1]);
+                    spread_reads();
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_b(bA, nic, nf, nth, ntw);
+                    __builtin_amdgcn_sched_barrier(0);
+                    mask_b(bB, ic0 + 32);
+                    read_a(aQ, 3);
+                    mfma_chunk(aP, bB[0]);
+                    spread_reads();
+                    __builtin_amdgcn_sched_barrier(0);
+                    {
+                        const int noff = tap_offset(nf, nth, ntw), d = noff - coff;
+                        coff = noff;
+#pragma unroll
+                        for (int i = 0; i < TILES; i++) cur[i] += d;
+                    }
+                    read_a(aP, 0);   // after the last tap of a pass: re-read once the next halo is staged
+                    mfma_chunk(aQ, bB[1]);
+                    spread_reads();
+                    __builtin_amdgcn_sched_barrier(0);
+                    th = nth;
+                    tw = ntw;
+                }
+            });
+        }
+        (void)bA;
+        (void)aP;
+    }
+    __builtin_amdgcn_s_setprio(2);
+
+    // ---- epilogue: phase by phase through LDS, every pixel's channels leave as whole 256-byte lines ----------------------
+    float *Os = Hs;    // [P][TC_OS]
+#pragma unroll
+    for (int f = 0; f < NPH; f++) {
+        __syncthreads();   // the halo (or the previous phase's staging) has been read by everyone
+#pragma unroll
+        for (int i = 0; i < TILES; i++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) Os[(16 * i + 4 * q + r) * TC_OS + 16 * w + l16] = acc[f][i][r];
+        __syncthreads();
+        for (int idx = t; idx < P * 16; idx += 256) {
+            const int pix = idx >> 4, cq = (idx & 15) * 4;
+            const int m = m0 + pix;
+            if (m < m_lim && oc0 + cq < p.CO) {
+                const int n = fdiv(m, p.d_OHW), rem = m - n * OHW;
+                const int i = fdiv(rem, p.d_OW), j = rem - i * OW;
+                const size_t elem = (size_t)(p.f_o_off[f] + n * p.o_sn + i * p.o_sh + j * p.o_sw + oc0 + cq);
+                *reinterpret_cast<float4 *>(p.O + elem) = epilogue4(*reinterpret_cast<const float4 *>(Os + pix * TC_OS + cq), p.ep, oc0 + cq, elem);
+            }
+        }
+    }
+}
+
+// Persistent grid over 16-pixel tiles: each XCD (workgroups are dealt round-robin to the 8 XCDs) works on a contiguous
+// run of tiles, each of its workgroups on a contiguous share of that run, equal to within one tile; a share is processed
+// in units of 4, 3 or 2 tiles so that no MFMA is spent on tiles that do not exist (whole units of one size left some
+// compute units a quarter more work than others: 3136 tiles on 256 compute units).
+template <bool RAGGED>
+__global__ __launch_bounds__(256, 2) void tap_conv_merged_kernel(const TapConvArgs p)
+{
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    const int oc0 = blockIdx.y * 64;
+    const int G = gridDim.x;
+    const int X = G < 8 ? G : 8;                           // groups of workgroups: the XCDs (fewer workgroups than XCDs: one each)
+    const int xcd = blockIdx.x % X, xi = blockIdx.x / X;
+    const int wgs = G / X + (xcd < G % X ? 1 : 0);         // workgroups of this group
+    const int T = p.full_units;                            // tiles in all
+    const int x_lo = xcd * (T / X) + min(xcd, T % X), x_n = T / X + (xcd < T % X ? 1 : 0);   // this group's run
+    const int q = x_n / wgs, r = x_n - q * wgs;
+    int tile = x_lo + xi * q + min(xi, r);
+    int left = q + (xi < r ? 1 : 0);
+    bool first = true;
+    while (left > 0) {
+        if (!first) __syncthreads();   // the previous unit's output staging has been read
+        first = false;
+        const int m0 = tile * 16;
+        if (left >= 6 || left == 4) {
+            tap_conv_merged_unit<4, RAGGED>(p, smem, m0, p.M, oc0);
+            tile += 4; left -= 4;
+        } else if (left == 5 || left == 3) {
+            tap_conv_merged_unit<3, RAGGED>(p, smem, m0, min(p.M, m0 + 48), oc0);
+            tile += 3; left -= 3;
+        } else {   // 2, or a single tile (a share of one tile: the second tile is computed and not stored)
+            tap_conv_merged_unit<2, RAGGED>(p, smem, m0, min(p.M, m0 + 16 * left), oc0);
+            tile += 2; left -= 2;
+        }
     }
 }
 
@@ -476,6 +721,96 @@ hipError_t launch_tap_conv(hipStream_t stream, const float *A, const float *B, f
         tiles = (tiles == 8) ? 7 : 8;
     }
     return hipErrorNotSupported;
+}
+
+// Kernel-split backward-data for stride 2 x 2 with even output sizes: all four phases in one launch, one halo per unit
+// (see tap_conv_merged_unit). Phase f is the dense stride-1 problem
+//   O[o_off[f] + n*o_sn + i*o_sh + j*o_sw + co] = sum_{th < TH[f], tw < TW[f], c < AC} A[n, i - ph[f] + th, j - pw[f] + tw, c]
+//                                                 * B[b_off[f] + th*b_sth[f] + tw*b_stw + c*b_sc + co]
+// for i < OHt, j < OWt (the same for every phase); TH[f] = 0 marks a phase without taps, which is written as zeros.
+// Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
+hipError_t launch_tap_conv_merged(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC, int CO,
+                                  int OHt, int OWt, const int *TH, const int *TW, const int *ph, const int *pw, const int *b_off,
+                                  const int *b_sth, int b_stw, int b_sc, const int *o_off, int o_sn, int o_sh, int o_sw, const Epilogue *ep)
+{
+    if (AC < 32 || (CO & 3) || OHt < 1 || OWt < 1) return hipErrorNotSupported;
+    const int cus = device_cu_count();
+    if (cus < 1) return hipErrorNotSupported;
+    int PH = 0, PW = 0;
+    for (int f = 0; f < 4; f++) {
+        if (TH[f] == 0 || TW[f] == 0) continue;
+        if (TH[f] < 0 || TW[f] < 0 || ph[f] < 0 || pw[f] < 0) return hipErrorNotSupported;
+        if (ph[f] > PH) PH = ph[f];
+        if (pw[f] > PW) PW = pw[f];
+    }
+    TapConvArgs a{};
+    int WH = 1, WW = 1;
+    for (int f = 0; f < 4; f++) {
+        const bool any = TH[f] > 0 && TW[f] > 0;
+        a.f_TH[f] = any ? TH[f] : 0; a.f_TW[f] = any ? TW[f] : 0;
+        a.f_row[f] = any ? PH - ph[f] : 0; a.f_col[f] = any ? PW - pw[f] : 0;
+        a.f_b_off[f] = any ? b_off[f] : 0; a.f_b_sth[f] = any ? b_sth[f] : 0;
+        a.f_o_off[f] = o_off[f];
+        if (any && a.f_row[f] + TH[f] > WH) WH = a.f_row[f] + TH[f];
+        if (any && a.f_col[f] + TW[f] > WW) WW = a.f_col[f] + TW[f];
+    }
+    if (WH > 7 || WW > 7) return hipErrorNotSupported;
+    a.A = A; a.B = B; a.O = O; a.ep = ep ? *ep : bias_epilogue(nullptr);
+    a.CO = CO;
+    a.AH = AH; a.AW = AW; a.AC = AC;
+    a.TH = WH; a.TW = WW; a.ph = PH; a.pw = PW;
+    a.PHt = AH + PH > OHt + WH - 1 ? AH + PH : OHt + WH - 1;
+    a.PWt = AW + PW > OWt + WW - 1 ? AW + PW : OWt + WW - 1;
+    a.sh = 1; a.sw = 1;
+    a.PWp = a.PWt; a.RP = a.PWt;
+    a.d_sw = make_fastdiv(1);
+    a.b_stw = b_stw; a.b_sc = b_sc;
+    a.o_sn = o_sn; a.o_sh = o_sh; a.o_sw = o_sw;
+    const long M = (long)N * OHt * OWt;
+    if (M >= (1L << 30) || (long)N * a.PHt >= (1L << 24)) return hipErrorNotSupported;
+    a.M = (int)M;
+    a.d_OW = make_fastdiv(OWt);
+    a.d_OHW = make_fastdiv(OHt * OWt);
+    a.d_PHt = make_fastdiv(a.PHt);
+    a.d_PWt = make_fastdiv(a.PWt);
+    // LDS rows of the worst unit: up to 64 pixels from any tile boundary on
+    constexpr int P = 64;
+    {
+        const int OHW = OHt * OWt, tiles = (a.M + 15) / 16;
+        int worst = 0;
+        const int scan = tiles < 65536 ? tiles : 65536;
+        for (int u = 0; u < scan; u++) {
+            const long m0 = (long)u * 16, m1 = (m0 + P < a.M ? m0 + P : a.M) - 1;
+            const int n0 = (int)(m0 / OHW), oh0 = (int)(m0 % OHW) / OWt;
+            const int n1 = (int)(m1 / OHW), oh1 = (int)(m1 % OHW) / OWt;
+            const int rows = (n1 * a.PHt + oh1 + WH - 1) - (n0 * a.PHt + oh0) + 1;
+            if (rows > worst) worst = rows;
+        }
+        if (tiles > scan) {   // analytic bound for what was not scanned
+            const int span = (P + OWt - 2) / OWt + 1, cross = (P + OHW - 2) / OHW + 1;
+            const int bound = (span - 1) + WH + cross * (a.PHt - OHt > 0 ? a.PHt - OHt : 0);
+            if (bound > worst) worst = bound;
+        }
+        a.lds_rows = worst;
+    }
+    size_t halo = (size_t)a.lds_rows * a.RP * TC_PS + 4;
+    const size_t stage = (size_t)P * TC_OS;
+    if (halo < stage) halo = stage;
+    const size_t lds = halo * sizeof(float);
+    if (lds > 80 * 1024) return hipErrorNotSupported;
+    const int tiles = (a.M + 15) / 16, ocb = (CO + 63) / 64;
+    a.full_units = tiles;
+    int G = 2 * cus / ocb;
+    if (G < 1) G = 1;
+    if (G > (tiles + 1) / 2) G = (tiles + 1) / 2;   // at least two tiles per workgroup
+    if ((AC % TC_ICC) != 0) {
+        if (hipError_t e = ensure_dynamic_lds<tap_conv_merged_kernel<true>>(lds); e != hipSuccess) return e;
+        hipLaunchKernelGGL(tap_conv_merged_kernel<true>, dim3(G, ocb, 1), dim3(256), lds, stream, a);
+    } else {
+        if (hipError_t e = ensure_dynamic_lds<tap_conv_merged_kernel<false>>(lds); e != hipSuccess) return e;
+        hipLaunchKernelGGL(tap_conv_merged_kernel<false>, dim3(G, ocb, 1), dim3(256), lds, stream, a);
+    }
+    return hipGetLastError();
 }
 
 }  // namespace alpha

@@ -458,6 +458,14 @@ KS_SHAPES = [
     (4, 12, 9, 16, 16, 3, 3, 3, 3, 1, 1),     # Ims: IH % sh == 0
     (4, 13, 11, 16, 16, 5, 4, 3, 2, 2, 1),    # general kernel split (IH % sh != 0)
     (4, 9, 9, 12, 8, 2, 2, 2, 2, 0, 0),       # odd IH with stride 2
+    # deltaY channel counts the LDS-halo kernel takes (>= 32): every phase in one launch
+    (4, 28, 28, 64, 128, 3, 3, 2, 2, 1, 1),   # c4b geometry
+    (4, 15, 13, 20, 96, 5, 5, 2, 2, 2, 2),    # odd sizes: the phases have different numbers of pixels; 96 = 64 + 32 channels
+    (4, 12, 12, 36, 68, 7, 7, 2, 2, 3, 3),    # ragged channel counts on both sides
+    (4, 12, 9, 64, 32, 3, 3, 3, 3, 1, 1),     # nine phases of one tap each
+    (4, 13, 11, 32, 64, 5, 4, 3, 2, 2, 1),    # six phases, rectangular filter
+    (4, 20, 20, 64, 64, 2, 2, 2, 2, 0, 0),    # one tap per phase, no padding
+    (4, 11, 11, 64, 48, 3, 3, 2, 2, 0, 0),    # no padding, odd size
 ]
 
 
@@ -491,6 +499,19 @@ def test_deltaX_kernel_split_family(dev, shape):
         else:
             getattr(DX, entry)(*base, sh, sw, ph, pw)
         check(dev.get(dXo), want, "%s %s" % (entry, shape))
+    # the other path (one launch of the generic kernel per phase), and the tiny-IC entry, which reads W in place
+    L = pkg.lib()
+    try:
+        L.alpha_conv_set_fwd_algo(3)
+        dXo = dev.guarded(N, IH, IW, IC)
+        DX.dconv3D_deltaX_kernelSplit(dev.streams, 1, dy.data_ptr(), OH, OW, CW.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC,
+                                      sh, sw, ph, pw)
+        check(dev.get(dXo), want, "kernelSplit through the generic kernel %s" % (shape,))
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+    dXo = dev.guarded(N, IH, IW, IC)
+    DX.dconv3D_deltaX_crossAdd(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC, sh, sw, ph, pw)
+    check(dev.get(dXo), want, "crossAdd (filter in place) %s" % (shape,))
 
 
 @pytest.mark.parametrize("shape", [
