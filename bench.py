@@ -47,7 +47,7 @@ LAYERS = {
     "c5b": (32, 56, 56, 64, 64, 3, 1, 1, 64, ("dx", "dw")),
     "c5c": (32, 56, 56, 64, 256, 1, 1, 0, 64, ("dx", "dw")),
 }
-HBM_BOUND = {"c1", "c4c", "c5a", "c5c"}   # arithmetic intensity below the ridge
+RIDGE = PEAK_MFMA_F32_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9)   # FLOP per byte at which the two published peaks meet (19.7)
 UNIFORM_INPUT = {"c1", "c4a", "c4b", "c4c", "c4d"}   # BASELINE.json: inputs uniform[-1,1] (the others N(0,1)); filters He-normal
 REL_TOL, ABS_TOL = 1e-4, 1e-5
 
@@ -96,6 +96,13 @@ class Workload:
         self.CW = torch.empty(F * F * IC * OC, device=dev)
         self.Bias = torch.randn((OC,), generator=g)
         self.Biash, self.Bias = self.Bias, self.Bias.to(dev)
+        # batch-norm statistics and affine parameters of the fused-epilogue row
+        self.bn_h = {"mean": torch.randn((OC,), generator=g), "var": torch.rand((OC,), generator=g) * 1.5 + 0.5,
+                     "A": torch.rand((OC,), generator=g) + 0.5, "B": torch.randn((OC,), generator=g)}
+        self.bn_d = {k: v.to(dev) for k, v in self.bn_h.items()}
+        self.bn_eps, self.leaky_k = 1e-5, 0.1
+        self.epilogue = pkg.Epilogue(X_mean=self.bn_d["mean"].data_ptr(), X_var=self.bn_d["var"].data_ptr(), eps=self.bn_eps,
+                                     A=self.bn_d["A"].data_ptr(), B=self.bn_d["B"].data_ptr(), k=self.leaky_k)
         self.stream = int(torch.cuda.current_stream().cuda_stream)
         self.streams = [self.stream]
         self.engine = pkg.engine.Engine(self.stream)
@@ -151,6 +158,17 @@ class Workload:
         N, IH, IW, IC, OC, F, s, p = self.dims
         self.engine.conv3D_biased(self.Y.data_ptr(), self.OH, self.OW, self.X.data_ptr(), IH, IW, self.W.data_ptr(), F, F,
                                   N, IC, OC, s, s, p, p, self.Bias.data_ptr(), N * self.OH * self.OW * OC, OC)
+
+    def fwd_fused(self):
+        # conv3D + batch normalisation (given statistics, affine) + leaky ReLU as one operator through the host layer
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.engine.conv3D_fused(self.Y.data_ptr(), self.OH, self.OW, self.X.data_ptr(), IH, IW, self.W.data_ptr(), F, F,
+                                 N, IC, OC, s, s, p, p, self.epilogue)
+
+    def fwd_fused_conv(self):
+        N, IH, IW, IC, OC, F, s, p = self.dims
+        self.pkg.Cuda_conv3D.conv3D_GemmR_fused(self.streams, 1, self.X.data_ptr(), IH, IW, self.W.data_ptr(), self.CW.data_ptr(), F, F,
+                                                self.epilogue, self.Y.data_ptr(), self.OH, self.OW, N, IC, OC, s, s, p, p)
 
     def fwd(self):
         # whole operator through the C++ host layer: entry selection, CW scratch, kernel_remode, conv entry
@@ -314,6 +332,10 @@ def parity(wl, op, step):
             want = O.conv3D_f64(np.ascontiguousarray(wl.Xh.numpy()[imgs]), wl.Wh.numpy(), s, s, p, p)
             if op == "fwd_bias":
                 want = want + wl.Biash.numpy().astype(np.float64)
+            if op == "fwd_fused":   # closed form of the row functions in fp64
+                b = {k: v.numpy().astype(np.float64) for k, v in wl.bn_h.items()}
+                want = (want - b["mean"]) / np.sqrt(b["var"] + wl.bn_eps) * b["A"] + b["B"]
+                want = np.where(want > 0, want, wl.leaky_k * want)
         else:
             want = O.deltaX_f64(np.ascontiguousarray(wl.dYh.numpy()[imgs]), wl.Wh.numpy(), IH, IW, s, s, p, p)
         got = out[imgs].cpu().numpy()
@@ -331,18 +353,18 @@ def parity(wl, op, step):
 
 
 def kind_of(op):
-    return "fwd" if op in ("fwd", "fwd_bias", "fwd_cached", "wino") else "dx" if op in ("dx", "dx_wino") else "dw"
+    return "fwd" if op in ("fwd", "fwd_bias", "fwd_cached", "fwd_fused", "wino") else "dx" if op in ("dx", "dx_wino") else "dw"
 
 
 def measure(wl, op, steps, warmup, with_parity=True):
     pkg, torch, layer = wl.pkg, wl.torch, wl.layer
     wl.set_op(op)
-    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd, "fwd_bias": wl.fwd_bias, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.fwd,
+    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd, "fwd_bias": wl.fwd_bias, "fwd_fused": wl.fwd_fused, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.fwd,
             "dx_wino": wl.dx_op, "dw_wino": wl.dw}[op]
-    kernel = {"fwd": wl.fwd_conv, "fwd_cached": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
+    kernel = {"fwd": wl.fwd_conv, "fwd_cached": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "fwd_fused": wl.fwd_fused_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
               "wino": wl.wino_conv, "dx_wino": wl.dx_wino_conv, "dw_wino": wl.dw_wino_gemm}[op]
     N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
-    if op in ("fwd", "fwd_bias", "fwd_cached"):
+    if op in ("fwd", "fwd_bias", "fwd_cached", "fwd_fused"):
         wl.fwd_remode()
     if op == "wino":
         pkg.Cuda_conv3D.winograd_filter_transform(wl.stream, wl.W.data_ptr(), wl.U.data_ptr(), IC_, OC_)
@@ -354,7 +376,8 @@ def measure(wl, op, steps, warmup, with_parity=True):
     wl.engine.sync()
     _, k_ms = time_loop(torch, kernel, steps, max(1, warmup // 2))   # dominant kernel alone, HIP events on its stream
     fl, by = flops(layer), algorithmic_bytes(layer)
-    hbm = layer in HBM_BOUND
+    hbm = fl / by < RIDGE   # below the ridge the HBM roofline binds (c1, c4c), above it the matrix pipes (the 1x1 layers of
+    #                         config 5 sit just above: 25.6 FLOP/B against a ridge of 19.7)
     roof = {
         "bound": "hbm" if hbm else "mfma",
         "achieved": round(by / (k_ms * 1e-3) / 1e9, 2) if hbm else round(fl / (k_ms * 1e-3) / 1e12, 3),
@@ -364,6 +387,10 @@ def measure(wl, op, steps, warmup, with_parity=True):
         "traffic": load_traffic(layer, op),
     }
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
+    roof["flop_per_byte"] = round(fl / by, 2)
+    if not hbm and fl / by < 2 * RIDGE:   # near the ridge: the other roofline as well
+        roof["hbm_GBps"] = round(by / (k_ms * 1e-3) / 1e9, 1)
+        roof["hbm_frac"] = round(roof["hbm_GBps"] / PEAK_HBM_GBPS, 4)
     if op in ("wino", "dx_wino", "dw_wino"):
         roof["note"] = "Winograd: FLOPs credited are the direct convolution's (2.25x the multiplies executed); frac is not a roofline fraction"
     row = {"layer": layer, "op": op, "ms_per_step": round(wall_ms, 5), "event_ms_per_step": round(ev_ms, 5),
@@ -387,7 +414,7 @@ def layer_ops(layer):
     if "dw" in ops and F == 3 and s == 1:
         ops.append("dw_wino")
     if layer == "c3a":
-        ops += ["fwd_bias", "fwd_cached"]
+        ops += ["fwd_bias", "fwd_cached", "fwd_fused"]
     return ops
 
 
@@ -397,7 +424,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
-    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "dx", "dw", "dw_fill", "wino", "dx_wino", "dw_wino"],
+    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "fwd_fused", "dx", "dw", "dw_fill", "wino", "dx_wino", "dw_wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="accepted for compatibility: the layers array is part of the default line")
     ap.add_argument("--no-layers", action="store_true", help="leave out the array with every layer/op of BASELINE.json's configs")

@@ -740,6 +740,15 @@ int alpha_dconv3D_deltaX_s1_leakyRelu(const int64_t *streams, int length, const 
     ep.gate = Xf; ep.slope = k; ep.fused = 1;
     return deltaX_s1(__func__, streams, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw, &ep);
 }
+int alpha_dconv3D_deltaX_kernelSplit_leakyRelu(const int64_t *streams, int length, const float *deltaY, int OH, int OW,
+                                               const float *CW, int FH, int FW, const float *Xf, float k, float *deltaX,
+                                               int IH, int IW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
+{
+    CHECK_PTR(Xf);
+    Epilogue ep{};
+    ep.gate = Xf; ep.slope = k; ep.fused = 1;
+    return deltaX_phases(__func__, streams, length, deltaY, OH, OW, CW, true, FH, FW, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw, &ep);
+}
 int alpha_leakyRelu2D(int64_t stream, const float *X, float k, float *Y, int lengthv, int mem_width, int mem_stride)
 {
     Epilogue ep{};

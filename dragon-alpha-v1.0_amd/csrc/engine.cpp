@@ -678,6 +678,12 @@ static int deltaX_impl(alpha_engine *e, const char *what, float *deltaX, int IH,
         float *CW = filter_block(e, 2, W, FH, FW, IC, OC, sh, sw, (size_t)p.scratch_floats * sizeof(float), &fresh);
         if (!CW) return fail(e, -1, what);
         if (fresh && (rc = alpha_ks_remodev2(streams[0], W, FH, FW, CW, CFH, CFW, OC, IC, sh, sw))) { forget_filter_block(e, CW); return fail(e, rc, "ks_remodev2"); }
+        if (Xf != nullptr) {   // every kernel-split entry runs the same kernels: the mask rides in their epilogue
+            rc = alpha_dconv3D_deltaX_kernelSplit_leakyRelu(streams, p.streams, deltaY, OH, OW, CW, FH, FW, Xf, k, deltaX, IH, IW, N, IC, OC,
+                                                            sh, sw, ph, pw);
+            gated = true;
+            break;
+        }
         switch (p.entry) {
         case ALPHA_E_dconv3D_deltaX_ksV2_Ims2R:
             rc = alpha_dconv3D_deltaX_ksV2_Ims2R(p.useTexture, streams, p.streams, deltaY, OH, OW, CW, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw);

@@ -66,6 +66,7 @@ _SIGS = {
     "alpha_conv3D_GemmR_fused": "sipiippiiepiiiiiiiii",
     "alpha_conv3D_winograd_fused": "sipiipepiiiiiii",
     "alpha_dconv3D_deltaX_s1_leakyRelu": "sipiipiipfpiiiiiii",
+    "alpha_dconv3D_deltaX_kernelSplit_leakyRelu": "sipiipiipfpiiiiiiiii",
     "alpha_leakyRelu2D": "lpfpiii",
     "alpha_leakyRelu2D_deltaX_v1": "lpppfiii",
     "alpha_batchNorm2D_row": "lpppfipiii",
@@ -286,6 +287,11 @@ class Cuda_dconv3D_deltaX:
     def dconv3D_deltaX_s1_leakyRelu(streamArray, length, deltaY, OH, OW, W, FH, FW, Xf, k, deltaX, IH, IW, N, IC, OC, ph, pw):
         """Backward-data times the derivative of the leaky ReLU whose output Xf is this layer's input (fused epilogue)."""
         _call("alpha_dconv3D_deltaX_s1_leakyRelu", streamArray, length, deltaY, OH, OW, W, FH, FW, Xf, k, deltaX, IH, IW, N, IC, OC, ph, pw)
+
+    @staticmethod
+    def dconv3D_deltaX_kernelSplit_leakyRelu(streamArray, length, deltaY, OH, OW, CW, FH, FW, Xf, k, deltaX, IH, IW, N, IC, OC, sh, sw, ph, pw):
+        _call("alpha_dconv3D_deltaX_kernelSplit_leakyRelu", streamArray, length, deltaY, OH, OW, CW, FH, FW, Xf, k, deltaX, IH, IW,
+              N, IC, OC, sh, sw, ph, pw)
 
     @staticmethod
     def dconv3D_deltaX_s1_texture(streamArray, length, deltaY, OH, OW, W, FH, FW, deltaX, IH, IW, N, IC, OC, ph, pw):

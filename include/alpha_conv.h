@@ -390,6 +390,13 @@ int alpha_dconv3D_deltaX_s1_leakyRelu(const int64_t *streams, int length,
                                       const float *Xf, float k,
                                       float *deltaX, int IH, int IW,
                                       int N, int IC, int OC, int ph, int pw);
+/* the same for any stride, from the kernel-split filter layout of alpha_ks_remodev2 (dX/A.cu:141) */
+int alpha_dconv3D_deltaX_kernelSplit_leakyRelu(const int64_t *streams, int length,
+                                               const float *deltaY, int OH, int OW,
+                                               const float *CW, int FH, int FW,
+                                               const float *Xf, float k,
+                                               float *deltaX, int IH, int IW,
+                                               int N, int IC, int OC, int sh, int sw, int ph, int pw);
 /* The row functions themselves (one HBM-bound pass; X == Y allowed), argument order of the reference's natives:
  * lengthv = height * mem_stride elements, mem_width data elements per row, the mem_stride - mem_width pad elements are
  * written as zeros. row_lengthv (the length of X_mean / X_var) must equal mem_stride. */

@@ -140,6 +140,25 @@ def test_backward_data_with_the_leaky_relu_derivative_in_the_epilogue(dev, shape
     check(dev.get(dx), want, "deltaX_s1_leakyRelu %s" % (shape,))
 
 
+@pytest.mark.parametrize("shape", [(4, 16, 16, 64, 128, 3, 3, 2, 2, 1, 1),     # four phases in one launch of the LDS-halo kernel
+                                   (4, 13, 11, 16, 16, 5, 4, 3, 2, 2, 1)])     # one launch of the generic kernel per phase
+def test_strided_backward_data_with_the_leaky_relu_derivative_in_the_epilogue(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    dY, W = normal((N, OH, OW, OC), 8311), he_normal(OC, FH, FW, IC, 8312)
+    k = 0.2
+    Xf = leaky(normal((N, IH, IW, IC), 8313).astype(np.float64), k).astype(np.float32)
+    want = O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw) * np.where(Xf > 0, 1.0, k)
+    CFH, CFW = O.ks_dims(FH, FW, sh, sw)
+    dy, w, xf = dev.put(dY), dev.put(W), dev.put(Xf)
+    cw = dev.empty(sh * sw * OC * CFH * CFW * IC, fill=0.0)
+    DX.ks_remodev2(dev.stream, w.data_ptr(), FH, FW, cw.data_ptr(), CFH, CFW, OC, IC, sh, sw)
+    dx = dev.guarded(N, IH, IW, IC)
+    DX.dconv3D_deltaX_kernelSplit_leakyRelu(dev.streams, 1, dy.data_ptr(), OH, OW, cw.data_ptr(), FH, FW, xf.data_ptr(), k, dx.data_ptr(),
+                                            IH, IW, N, IC, OC, sh, sw, ph, pw)
+    check(dev.get(dx), want, "deltaX_kernelSplit_leakyRelu %s" % (shape,))
+
+
 def test_row_functions_keep_pad_columns_zero_and_match_their_definitions(dev):
     height, width, stride = 37, 10, 12     # two pad columns per row
     X = normal((height, stride), 8401)
