@@ -203,6 +203,12 @@ hipError_t launch_tap_conv_merged(hipStream_t stream, const float *A, const floa
 hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, float *O, int Nimg, int AH, int AW,
                             int OH, int OW, int sh, int sw, int K, int N, int b_kmajor, const float *bias = nullptr);
 
+// The same GEMM with both operands straight from memory and no LDS (pointwise_direct.hip): O[m][n] = sum_k A[m][k] * B[k][n]
+// for dense rows (stride 1) and B given as [K][N]; K a multiple of 32. Applies the whole epilogue `ep` when given (else
+// `bias`). Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
+hipError_t launch_pointwise_direct(hipStream_t stream, const float *A, const float *B, float *O, long M, int K, int N,
+                                   const float *bias = nullptr, const Epilogue *ep = nullptr);
+
 // Backward-filter implicit GEMM with split-K over k = (n, oh, ow):
 //   dst_z[oc, fh, fw, ic] = sum_{k in slice z} deltaY[k, oc] * X[n, oh*sh - ph + fh, ow*sw - pw + fw, ic]
 // slice z = [z*GK_slice, (z+1)*GK_slice), the last one running to GK; dst_0 = deltaW,

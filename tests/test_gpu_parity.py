@@ -335,6 +335,12 @@ POINTWISE_SHAPES = [
     (3, 5, 5, 128, 128),      # 75 pixels: fewer tiles than wavefronts
     (2, 33, 31, 64, 64),      # 2046 pixels
     (1, 1, 3, 192, 64),       # 3 pixels: a single ragged tile; K = 192 = 3 blocks forward (backward falls to another kernel)
+    # the kernel without LDS (both operands from memory): any K that is a multiple of 32, N in blocks of 64
+    (8, 56, 56, 64, 64),      # 25088 pixels = 1568 tiles: shares of 0 or 1 tile
+    (37, 28, 28, 96, 36),     # 29008 pixels = 1813 tiles; K = 96 forward, a ragged block of 36 produced channels (K = 36 backward: other kernel)
+    (64, 28, 30, 32, 200),    # 53760 pixels = 3360 tiles over 2048 wavefronts: shares of 1 and 2 tiles; 200 = 3 blocks + 8 channels
+    (32, 56, 56, 64, 32),     # 100352 pixels = 6272 tiles: shares of 3 and 4 tiles (c5 geometry with fewer channels)
+    (64, 60, 64, 32, 32),     # 245760 pixels = 15360 tiles: shares of 7 and 8 tiles (4 + 3 and 4 + 4)
 ]
 
 
@@ -345,20 +351,27 @@ def test_pointwise_kernel_forward_and_deltaX(dev, shape):
     want_y, want_dx = O.conv3D_f64(X, W, 1, 1, 0, 0), O.deltaX_f64(dY, W, IH, IW, 1, 1, 0, 0)
     L = pkg.lib()
     outs = {}
+    import os
+    VARIANTS = (0, 3, "resident", "direct")
     try:
-        for algo in (0, 3):   # 0: streaming GEMM kernel, 3: generic kernel
-            L.alpha_conv_set_fwd_algo(algo)
+        # 0: the 1x1 kernels as the library chooses between them, 3: generic kernel, "resident" / "direct": algo 0 with
+        # the kernel without LDS switched off / on wherever it applies, so that both stay tested on every shape
+        for algo in VARIANTS:
+            L.alpha_conv_set_fwd_algo(algo if isinstance(algo, int) else 0)
+            if not isinstance(algo, int):
+                os.environ["ALPHA_PW_DIRECT"] = "0" if algo == "resident" else "1"
             outs[algo] = (_run_fwd(dev, "conv3D_W1", X, W, 1, 1, 0, 0), _run_fwd(dev, "conv3D_GemmR_W1", X, W, 1, 1, 0, 0))
             dXo = dev.guarded(N, IH, IW, IC)
             dy, w = dev.put(dY), dev.put(W)
             DX.dconv3D_deltaX_W1(dev.streams, 1, dy.data_ptr(), w.data_ptr(), dXo.data_ptr(), IH, IW, N, IC, OC)
             outs[algo] += (dev.get(dXo),)
     finally:
+        os.environ.pop("ALPHA_PW_DIRECT", None)
         L.alpha_conv_set_fwd_algo(0)
-    for algo in (0, 3):
-        check(outs[algo][0], want_y, "conv3D_W1 algo %d %s" % (algo, shape))
-        check(outs[algo][1], want_y, "conv3D_GemmR_W1 algo %d %s" % (algo, shape))
-        check(outs[algo][2], want_dx, "deltaX_W1 algo %d %s" % (algo, shape))
+    for algo in VARIANTS:
+        check(outs[algo][0], want_y, "conv3D_W1 algo %s %s" % (algo, shape))
+        check(outs[algo][1], want_y, "conv3D_GemmR_W1 algo %s %s" % (algo, shape))
+        check(outs[algo][2], want_dx, "deltaX_W1 algo %s %s" % (algo, shape))
 
 
 @pytest.mark.parametrize("shape", [
