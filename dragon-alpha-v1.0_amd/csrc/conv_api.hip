@@ -216,6 +216,12 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
     const int CWstride = mCFH * mCFW * OC * IC;
     hipStream_t s = stream0(streams);
     if (sh * sw > 64) return fail(ALPHA_CONV_EINVAL, "%s: more than 64 phases (sh*sw)", fn);
+    if (!from_CW && fwd_algo() != 3) {
+        // 4 stored input channels (the gradient of a stem's input): one stride-1 convolution of deltaY into the
+        // sh*sw*4 values of each sh x sw block of deltaX
+        hipError_t e = launch_delta_x_stem(s, dY, F, dX, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, ep);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     // the phases as dense stride-1 problems
     struct Phase { GatherConvArgs a; int th, tw, OHt, OWt; };
     std::vector<Phase> phases;

@@ -548,6 +548,51 @@ def test_deltaX_crossAdd_is_deterministic_gather(dev, shape):
     assert np.array_equal(outs[0], outs[1])
 
 
+DX_STEM_SHAPES = [
+    # N, IH, IW, OC, FH, FW, sh, sw, ph, pw: 4 stored input channels, strides 1 or 2 -> the stem backward-data kernel
+    (4, 32, 32, 64, 7, 7, 2, 2, 3, 3),      # c4a geometry: window 4 x 4, one block of 16 x 16 coarse pixels per image... and a row of blocks
+    (2, 46, 70, 64, 7, 7, 2, 2, 3, 3),      # several blocks per image, ragged in both directions (23 x 35 coarse pixels)
+    (3, 21, 19, 64, 7, 7, 2, 2, 3, 3),      # odd sizes: the last coarse row and column have one phase only
+    (5, 16, 16, 32, 7, 7, 2, 2, 3, 3),      # 32 output channels: two wavefronts' share of the reduction is empty
+    (2, 18, 18, 20, 5, 5, 2, 2, 2, 2),      # window 3 x 3 inside the 4 x 4 kernel, ragged channel count
+    (4, 16, 20, 64, 3, 3, 2, 2, 1, 1),      # window 2 x 2 (the small instantiation)
+    (4, 17, 15, 48, 4, 4, 2, 2, 1, 1),      # 4 x 4 stride 2 padding 1: window 3 x 3
+    (4, 14, 14, 64, 2, 2, 2, 2, 0, 0),      # one tap per phase
+    (3, 12, 18, 64, 3, 3, 1, 1, 1, 1),      # stride 1: one phase, window 3 x 3
+    (3, 12, 18, 16, 3, 5, 1, 2, 1, 2),      # mixed strides: two phases
+    (3, 19, 12, 64, 6, 3, 2, 1, 2, 1),      # stride along the height only, no padding symmetry
+    (2, 20, 20, 64, 7, 7, 2, 2, 0, 0),      # no padding: window 4 x 4 from offset -3
+    (140, 16, 16, 64, 7, 7, 2, 2, 3, 3),    # 140 blocks over 512 workgroups: most get none
+    (9, 64, 64, 64, 7, 7, 2, 2, 3, 3),      # 72 blocks per... 9 x 4 x 2 blocks: every XCD's range holds several
+]
+
+
+@pytest.mark.parametrize("shape", DX_STEM_SHAPES)
+def test_deltaX_stem_kernel(dev, shape):
+    N, IH, IW, OC, FH, FW, sh, sw, ph, pw = shape
+    IC = 4
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    dY, W = normal((N, OH, OW, OC), 2301), he_normal(OC, FH, FW, IC, 2302)
+    W[..., 3] = 0      # three logical channels stored as four
+    want = O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw)
+    dy, w = dev.put(dY), dev.put(W)
+    L = pkg.lib()
+    outs = {}
+    try:
+        for algo in (0, 0, 3):          # twice through the stem kernel (bit-identical), once through the generic one
+            L.alpha_conv_set_fwd_algo(algo)
+            dXo = dev.guarded(N, IH, IW, IC)
+            DX.dconv3D_deltaX_crossAdd(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW,
+                                       N, IC, OC, sh, sw, ph, pw)
+            outs.setdefault(algo, []).append(dev.get(dXo))
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+    check(outs[0][0], want, "stem deltaX %s" % (shape,))
+    check(outs[3][0], want, "generic deltaX %s" % (shape,))
+    assert np.array_equal(outs[0][0], outs[0][1])
+    assert not np.any(outs[0][0][..., 3])     # the pad channel's gradient is exactly zero
+
+
 # ----------------------------------------------------------------------------------------------
 # backward-filter
 # ----------------------------------------------------------------------------------------------
