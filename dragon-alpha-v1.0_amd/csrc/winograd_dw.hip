@@ -13,18 +13,26 @@
 // gives bit-identical results. (The partition is over tiles, not over the reference's pixel ranges: the partial results
 // differ from the direct kernels', their sum does not, up to rounding.)
 //
-// A workgroup owns one slice, 64 output channels and 32 input channels, and has six wavefronts. Four multiply: wavefront w
-// accumulates output channels [16w, 16w+16) x 32 input channels x 16 xi = 128 registers. Tiles advance in chunks of 8.
-// Two wavefronts stage the patches: a thread loads the 4x4 patch of one (tile, pair of input channels) two chunks before
-// it is transformed and writes Xh[tile][32][16 xi] into the LDS buffer that is multiplied in the chunk after; one barrier
-// per chunk joins the two kinds (wavefronts of one kind doing both jobs needed scheduling directives, spilled, or moved
-// the accumulators through AGPRs). deltaY does not pass through LDS: a multiplying wavefront is the only user of its 16
-// output channels, so its lanes load their own 2x2 tiles and transform them in registers into MFMA operands.
+// A workgroup owns one slice, 64 output channels and 32 input channels, and has eight wavefronts, two per SIMD: one that
+// multiplies and one that stages. Multiplying wavefront w accumulates output channels [16w, 16w+16) x 32 input channels x
+// 16 xi = 128 registers; tiles advance in chunks of 8. A staging thread loads the 4x4 patch of one (tile, input channel)
+// two chunks before it is transformed and writes Xh[tile][channel][16 xi] into the LDS buffer that is multiplied in the
+// chunk after; one barrier per chunk joins the two kinds (wavefronts of one kind doing both jobs needed scheduling
+// directives, spilled, or moved the accumulators through AGPRs). deltaY does not pass through LDS: a multiplying wavefront
+// is the only user of its 16 output channels, so its lanes load their own 2x2 tiles and transform them in registers into
+// MFMA operands.
+// What a chunk costs beyond its 64 MFMAs per SIMD is the number of vector instructions the SIMD issues beside them (each
+// takes 5-9 cycles out of the MFMA stream, whichever wavefront issues it). The transforms need 56 per SIMD and chunk;
+// where tiles are and which of their pixels exist must not add to that. One wavefront therefore computes, once per 64
+// tiles, a table in LDS with each tile's load offsets - four row terms and four column terms of its patch, the four
+// pixels of its deltaY tile, "outside" encoded as an offset beyond the descriptor - and every other thread gets the
+// offsets of its tile with two or three 128-bit LDS reads and adds its channel (tile cursors kept per thread and advanced by
+// additions cost 24-67 vector instructions per wavefront and chunk; the staging work on two of the four SIMDs made
+// those two 3.7 k cycles per chunk against 2.05 k of MFMAs).
 // In LDS the 16 xi of a (tile, channel) are contiguous, so a lane's patch operand for four xi is one 128-bit read (an
 // operand per xi as a 32-bit read - three LDS instructions per two MFMAs - cost 30 cycles per pair of MFMAs). A (tile,
-// channel) takes 80 bytes, its four 16-byte groups of xi stored permuted (group g at position g ^ (channel / 16 % 4)): the
-// 16 lanes of a read (16 consecutive channels) and the 16 lanes of a staging write (channels 2 apart) then both touch 16
-// different 16-byte bank groups.
+// channel) takes 80 bytes and a tile 32 x 80 + 256: the 32 lanes of a staging write (32 channels of a tile) and the 32
+// lanes of a half wavefront's read (16 channels of two tiles) then touch 32 different 16-byte bank groups.
 #include "common.hpp"
 #include <type_traits>
 
@@ -38,25 +46,27 @@ struct WinoDwArgs {
     int IH, IW, IC, OH, OW, OC, ph, pw;
     int TC, TR, TRC;     // tile columns, tile rows, tiles per image
     int ntiles, S, GZ;   // N*TRC; tiles per slice (a multiple of 8); slices
-    int x_bytes, y_bytes;   // X at most 1 GB, deltaY below 2 GB
-    // a thread's tile moves on by 8 per chunk: (ty, tx) += (adv_ty, adv_tx), then at most one wrap of tx and one of ty;
-    // its patch origin in X and its tile origin in deltaY (element offsets) move by dx0 / dy0 plus wx1 / wy1 when tx
-    // wraps and wx2 / wy2 when ty wraps (into the next image)
-    int adv_ty, adv_tx, dx0, dy0, wx1, wy1, wx2, wy2;
+    int x_bytes, y_bytes;   // X below 1 GB (512 MB when IC % 32 != 0), deltaY below 2 GB (1 GB when OC % 64 != 0)
     FastDiv d_TC, d_TRC;
 };
 
 constexpr int WD_TK = 8;                        // tiles per chunk
-constexpr int WD_CS = 20;                       // floats per (tile, channel): 16 xi + 4 (see the layout note above)
-constexpr int WD_XBUF = WD_TK * 32 * WD_CS;     // Xh[tile][32 input channels][16 xi + 4]: one LDS buffer
-constexpr int WD_BUF = WD_XBUF;
-constexpr unsigned WD_OOR = 0x80000000u;        // beyond both descriptors: the load returns 0
-constexpr unsigned WD_OOR_COL = 0x40000000u;    // added to a valid offset of X (at most 1 GB) or to WD_OOR: beyond too
+constexpr int WD_CS = 20;                       // floats per (tile, channel): 16 xi + 4
+constexpr int WD_TS = 32 * WD_CS + 64;          // floats per tile: 176 16-byte groups = 16 (mod 32), see the layout note above
+constexpr int WD_BUF = WD_TK * WD_TS;           // Xh[tile][32 input channels][16 xi + 4]: one LDS buffer
+constexpr int WD_TG = 64;                       // tiles per group of the offset table (8 chunks)
+constexpr unsigned WD_OOR = 0x80000000u;        // row term / deltaY pixel outside: beyond both descriptors, the load returns 0
+constexpr unsigned WD_OOR_COL = 0x40000000u;    // column term outside (X ends below 1 GB)
+constexpr unsigned WD_OOR_XCH = 0x20000000u;    // input channel past the end (X ends below 512 MB when IC % 32 != 0)
+constexpr unsigned WD_OOR_YCH = 0x40000000u;    // output channel past the end (deltaY ends below 1 GB when OC % 64 != 0)
+// no sum of these with valid terms wraps around 2^32: 0x80000000 + 0x40000000 + 0x20000000 + (valid terms < 0x20000000)
 
-__global__ __launch_bounds__(384) void winograd_dw_kernel(const WinoDwArgs p)
+__global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
 {
-    extern __shared__ __attribute__((aligned(16))) float wd_smem[];   // Xh[2][WD_BUF]
+    extern __shared__ __attribute__((aligned(16))) float wd_smem[];   // Xh[2][WD_BUF], XT[2][64][8], YT[2][64][4]
     float *smem = wd_smem;
+    unsigned *XT = reinterpret_cast<unsigned *>(wd_smem + 2 * WD_BUF);
+    unsigned *YT = XT + 2 * WD_TG * 8;
 
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
@@ -73,146 +83,122 @@ __global__ __launch_bounds__(384) void winograd_dw_kernel(const WinoDwArgs p)
         acc[x][1] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // Tile positions are kept per thread from chunk to chunk and moved on by additions only (no division, no multiplication:
-    // recomputing a chunk's offsets from tile indices cost more issue slots than the chunk's MFMAs).
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.dY), 0, p.y_bytes, 0x00020000);
-    const int row_elems = p.IW * p.IC;
-    struct TileCur {
-        int tile, ty, tx, x00, y00;   // x00 / y00: element offsets of X[n, 2ty-ph, 2tx-pw, channel] (may be negative) / deltaY[n, 2ty, 2tx, channel]
-    };
-    auto cur_init = [&](TileCur &c, int tile, int x_channel, int y_channel) {
-        c.tile = tile;
-        const int n = fdiv(tile, p.d_TRC), rem = tile - n * p.TRC;
-        c.ty = fdiv(rem, p.d_TC);
-        c.tx = rem - c.ty * p.TC;
-        c.x00 = (n * p.IH + 2 * c.ty - p.ph) * row_elems + (2 * c.tx - p.pw) * p.IC + x_channel;
-        c.y00 = ((n * p.OH + 2 * c.ty) * p.OW + 2 * c.tx) * p.OC + y_channel;
-    };
-    auto cur_advance = [&](TileCur &c) {   // 8 tiles on
-        c.tile += WD_TK;
-        c.tx += p.adv_tx;
-        c.ty += p.adv_ty;
-        c.x00 += p.dx0;
-        c.y00 += p.dy0;
-        const bool w1 = c.tx >= p.TC;
-        c.tx -= w1 ? p.TC : 0;
-        c.ty += w1 ? 1 : 0;
-        c.x00 += w1 ? p.wx1 : 0;
-        c.y00 += w1 ? p.wy1 : 0;
-        const bool w2 = c.ty >= p.TR;
-        c.ty -= w2 ? p.TR : 0;
-        c.x00 += w2 ? p.wx2 : 0;
-        c.y00 += w2 ? p.wy2 : 0;
-    };
     typedef std::integral_constant<int, 0> Set0;
     typedef std::integral_constant<int, 1> Set1;
+    typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
-    // ---- wavefronts 4 and 5 stage the patches: a thread takes (tile, pair of input channels) - 16 64-bit loads two chunks
-    //      ahead, B^T x B, eight 128-bit LDS writes into the buffer that is multiplied in the next chunk. Offsets outside the
-    //      tensor (padding, tiles past the slice, channels past the end) are beyond the descriptor and read as zeros. -------
-    if (t >= 256) {
-        if (nchunks == 0) return;
-        __builtin_amdgcn_s_setprio(3);   // few instructions, and the multiplying wavefronts wait for them at the barrier
-        const int item = t - 256, st = item >> 4, x_ch = 2 * (item & 15);
-        const bool xc_ok = ic0 + x_ch < p.IC;          // IC % 4 == 0: a pair is valid as a whole
-        const int swz_wx = (x_ch >> 4) & 3;            // (channel / 16) % 4 of the channels this thread writes
-        TileCur cur;
-        cur_init(cur, tile_begin + st, ic0 + x_ch, 0);
-        float2 xr[2][4][4];   // raw patches: set s holds a chunk of parity s, requested two chunks before it is transformed
-        auto request = [&](auto set_c) {   // the 16 loads of the chunk the tile cursor stands on
-            constexpr int SET = decltype(set_c)::value;
-            const bool ok = cur.tile < tile_end && xc_ok;
-            const int ih0 = 2 * cur.ty - p.ph, iw0 = 2 * cur.tx - p.pw;
-            unsigned rowterm[4], colterm[4];
+    // Offsets of the 64 tiles of group g of the slice (lane = tile), into table slot g & 1. Patch of tile (n, ty, tx): rows
+    // 2ty - ph + i, columns 2tx - pw + j; a load's byte offset is row term i + column term j + 4 * channel.
+    auto table = [&](int g) {
+        const int tile = tile_begin + g * WD_TG + lane;
+        const bool ok = tile < tile_end;
+        const int tl = ok ? tile : tile_begin;
+        const int n = fdiv(tl, p.d_TRC), rem = tl - n * p.TRC;
+        const int ty = fdiv(rem, p.d_TC), tx = rem - ty * p.TC;
+        const int ih0 = 2 * ty - p.ph, iw0 = 2 * tx - p.pw;
+        const int row_elems = p.IW * p.IC;
+        const unsigned x00 = (unsigned)(((n * p.IH + ih0) * p.IW + iw0) * p.IC) * 4u;   // may stand before the tensor
+        uintx4 rt, ct, yo;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const unsigned rv = (unsigned)cur.x00 * 4u + (unsigned)(i * row_elems) * 4u, cv = (unsigned)(i * p.IC) * 4u;
-                rowterm[i] = (ok && (unsigned)(ih0 + i) < (unsigned)p.IH) ? rv : WD_OOR;
-                colterm[i] = ((unsigned)(iw0 + i) < (unsigned)p.IW) ? cv : WD_OOR_COL;
-            }
+        for (int i = 0; i < 4; i++) {
+            rt[i] = (ok && (unsigned)(ih0 + i) < (unsigned)p.IH) ? x00 + (unsigned)(i * row_elems) * 4u : WD_OOR;
+            ct[i] = ((unsigned)(iw0 + i) < (unsigned)p.IW) ? (unsigned)(i * p.IC) * 4u : WD_OOR_COL;
+        }
+        const unsigned y00 = (unsigned)(((n * p.OH + 2 * ty) * p.OW + 2 * tx) * p.OC) * 4u;
+        const bool right = 2 * tx + 1 < p.OW, below = 2 * ty + 1 < p.OH;
+        yo[0] = ok ? y00 : WD_OOR;
+        yo[1] = (ok && right) ? y00 + (unsigned)p.OC * 4u : WD_OOR;
+        yo[2] = (ok && below) ? y00 + (unsigned)(p.OW * p.OC) * 4u : WD_OOR;
+        yo[3] = (ok && right && below) ? y00 + (unsigned)((p.OW + 1) * p.OC) * 4u : WD_OOR;
+        const int e = (g & 1) * WD_TG + lane;
+        *reinterpret_cast<uintx4 *>(XT + e * 8) = rt;
+        *reinterpret_cast<uintx4 *>(XT + e * 8 + 4) = ct;
+        *reinterpret_cast<uintx4 *>(YT + e * 4) = yo;
+    };
+    if (t >= 256) {
+        if (nchunks == 0) return;   // an empty slice: the multiplying wavefronts write its zeros
+        // ---- wavefronts 4-7 stage the patches: a thread takes (tile, input channel) - 16 loads two chunks ahead, B^T x B,
+        //      four 128-bit LDS writes into the buffer that is multiplied in the next chunk --------------------------------
+        if (w == 4) table(0);
+        __syncthreads();
+        const int item = t - 256, st = item >> 5, x_ch = item & 31;
+        const unsigned ch4 = ic0 + x_ch < p.IC ? (unsigned)(ic0 + x_ch) * 4u : WD_OOR_XCH;
+        float xr[2][4][4];   // raw patches: set s holds a chunk of parity s, requested two chunks before it is transformed
+        auto request = [&](auto set_c, int chunk) {
+            constexpr int SET = decltype(set_c)::value;
+            const int tt = chunk * WD_TK + st;
+            const unsigned *e = XT + (((tt >> 6) & 1) * WD_TG + (tt & 63)) * 8;
+            const uintx4 rt = *reinterpret_cast<const uintx4 *>(e);
+            uintx4 ct = *reinterpret_cast<const uintx4 *>(e + 4);
+            ct += ch4;
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    xr[SET][i][j] = __builtin_bit_cast(float2, __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, rowterm[i] + colterm[j], 0, 0));
+                    xr[SET][i][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, rt[i] + ct[j], 0, 0));
         };
-        // Xh = B^T x B per channel; the 4 xi of a row are one 128-bit element of the (tile, channel)
+        // Xh = B^T x B; the 4 xi of a row are one 128-bit element of the (tile, channel)
         auto transform = [&](auto set_c, int buf, bool store) {
             constexpr int SET = decltype(set_c)::value;
-            float *Xh = smem + buf * WD_BUF + (st * 32 + x_ch) * WD_CS;
+            float *Xh = smem + buf * WD_BUF + st * WD_TS + x_ch * WD_CS;
+            float r[4][4];
 #pragma unroll
-            for (int k = 0; k < 2; k++) {
-                float r[4][4];
+            for (int j = 0; j < 4; j++) {
+                const float x0 = xr[SET][0][j], x1 = xr[SET][1][j], x2 = xr[SET][2][j], x3 = xr[SET][3][j];
+                r[0][j] = x0 - x2;
+                r[1][j] = x1 + x2;
+                r[2][j] = x2 - x1;
+                r[3][j] = x3 - x1;
+            }
+            if (store) {
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const float x0 = k ? xr[SET][0][j].y : xr[SET][0][j].x, x1 = k ? xr[SET][1][j].y : xr[SET][1][j].x;
-                    const float x2 = k ? xr[SET][2][j].y : xr[SET][2][j].x, x3 = k ? xr[SET][3][j].y : xr[SET][3][j].x;
-                    r[0][j] = x0 - x2;
-                    r[1][j] = x1 + x2;
-                    r[2][j] = x2 - x1;
-                    r[3][j] = x3 - x1;
-                }
-                if (store) {
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        *reinterpret_cast<floatx4 *>(Xh + k * WD_CS + ((i ^ swz_wx) << 2)) =
-                            floatx4{r[i][0] - r[i][2], r[i][1] + r[i][2], r[i][2] - r[i][1], r[i][3] - r[i][1]};
-                }
+                for (int i = 0; i < 4; i++)
+                    *reinterpret_cast<floatx4 *>(Xh + (i << 2)) =
+                        floatx4{r[i][0] - r[i][2], r[i][1] + r[i][2], r[i][2] - r[i][1], r[i][3] - r[i][1]};
             }
         };
-        request(Set0{});
+        request(Set0{}, 0);
         transform(Set0{}, 0, true);   // chunk 0, waited for
-        cur_advance(cur);
-        request(Set1{});              // chunk 1
-        cur_advance(cur);
-        request(Set0{});              // chunk 2
+        request(Set1{}, 1);
+        request(Set0{}, 2);
         __syncthreads();
         // chunk c: chunk c+1 (requested two chunks ago) is transformed into the other buffer, chunk c+3 requested into the
         // set it leaves. Two chunks per round so that the sets are fixed registers; the loads of the second half are issued
-        // even when that chunk does not exist (only its LDS writes and its barrier are skipped).
+        // even when that chunk does not exist (only its LDS writes and its barrier are skipped). Every eighth chunk the
+        // first staging wavefront writes the table of the next 64 tiles.
         for (int c = 0; c < nchunks; c += 2) {
+            if ((c & 7) == 0 && w == 4) table((c >> 3) + 1);
             transform(Set1{}, 1, true);
-            cur_advance(cur);
-            request(Set1{});
+            request(Set1{}, c + 3);
             __syncthreads();
             const bool more = c + 1 < nchunks;
             transform(Set0{}, 0, more);
-            cur_advance(cur);
-            request(Set0{});
+            request(Set0{}, c + 4);
             if (more) __syncthreads();
         }
         return;
-    }
-
-    // ---- wavefronts 0-3 multiply. deltaY does not go through LDS: wavefront w is the only one that needs output channels
-    //      [16w, 16w+16), so lane (l16, q) loads the 2x2 tiles of channel 16w + l16 for its two tiles of a chunk (q and
-    //      4 + q) itself, two chunks ahead, and transforms them in registers into the 32 MFMA operands of the chunk. The
-    //      patches come from LDS. ------------------------------------------------------------------------------------------
-    if (nchunks > 0) {
+    } else if (nchunks > 0) {
+        // ---- wavefronts 0-3 multiply. Wavefront w is the only one that needs output channels [16w, 16w+16), so lane
+        //      (l16, q) loads the 2x2 tiles of channel 16w + l16 for its two tiles of a chunk (q and 4 + q) itself, two
+        //      chunks ahead, and transforms them in registers into the 32 MFMA operands of the chunk. The patches come
+        //      from LDS. -------------------------------------------------------------------------------------------------
+        __syncthreads();
         const int y_ch = oc0 + 16 * w + l16;
-        const bool yc_ok = y_ch < p.OC;
-        const int y_px = p.OC, y_row = p.OW * p.OC;
-        TileCur ca, cb;
-        cur_init(ca, tile_begin + q, 0, y_ch);
-        cur_init(cb, tile_begin + 4 + q, 0, y_ch);
+        const unsigned ych4 = y_ch < p.OC ? (unsigned)y_ch * 4u : WD_OOR_YCH;
         float yraw[2][2][4];   // [set][kk][pixel]
-        auto request_one = [&](const TileCur &c, float (&y)[4]) {
-            const bool ok = c.tile < tile_end && yc_ok;
-            const bool right = 2 * c.tx + 1 < p.OW, below = 2 * c.ty + 1 < p.OH;
-            const unsigned o = (unsigned)c.y00 * 4u;
-            const unsigned o00 = ok ? o : WD_OOR, o01 = (ok && right) ? o + (unsigned)y_px * 4u : WD_OOR;
-            const unsigned o10 = (ok && below) ? o + (unsigned)y_row * 4u : WD_OOR;
-            const unsigned o11 = (ok && right && below) ? o + (unsigned)(y_row + y_px) * 4u : WD_OOR;
-            y[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o00, 0, 0));
-            y[1] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o01, 0, 0));
-            y[2] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o10, 0, 0));
-            y[3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o11, 0, 0));
-        };
-        auto request = [&](auto set_c) {
+        auto request = [&](auto set_c, int chunk) {
             constexpr int SET = decltype(set_c)::value;
-            request_one(ca, yraw[SET][0]);
-            request_one(cb, yraw[SET][1]);
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                const int tt = chunk * WD_TK + 4 * kk + q;
+                uintx4 o = *reinterpret_cast<const uintx4 *>(YT + (((tt >> 6) & 1) * WD_TG + (tt & 63)) * 4);
+                o += ych4;
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    yraw[SET][kk][k] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(y_rsrc, o[k], 0, 0));
+            }
         };
         // Yh' = G' y G'^T with G' = [[1,0],[1,1],[1,-1],[0,1]] = G without its factors 1/2, which are applied to the
         // accumulators once, at the end
@@ -236,20 +222,16 @@ __global__ __launch_bounds__(384) void winograd_dw_kernel(const WinoDwArgs p)
                 }
             }
         };
-        int rdx0[4], rdx1[4];   // float offsets of this lane's patch operands for xi group gx (tile q; channels l16, 16 + l16)
-#pragma unroll
-        for (int gx = 0; gx < 4; gx++) {
-            rdx0[gx] = (q * 32 + l16) * WD_CS + (gx << 2);
-            rdx1[gx] = (q * 32 + 16 + l16) * WD_CS + ((gx ^ 1) << 2);
-        }
+        // this lane's patch operands: tile q (and 4 + q), channels l16 and 16 + l16, xi group gx
+        const float *rd = smem + q * WD_TS + l16 * WD_CS;
         // One chunk = 8 groups of 8 MFMAs: (4 tiles kk, 4 xi) x (two blocks of input channels); two 128-bit LDS reads per
         // group, one group ahead. The two MFMAs into one accumulator (kk = 0, 1) are 4 groups apart.
         auto multiply = [&](int buf) {
-            const float *B = smem + buf * WD_BUF;
+            const float *B = rd + buf * WD_BUF;
             auto frag = [&](int g, floatx4 &fb0, floatx4 &fb1) {
                 const int kk = g >> 2, gx = g & 3;
-                fb0 = *reinterpret_cast<const floatx4 *>(B + rdx0[gx] + kk * 4 * 32 * WD_CS);
-                fb1 = *reinterpret_cast<const floatx4 *>(B + rdx1[gx] + kk * 4 * 32 * WD_CS);
+                fb0 = *reinterpret_cast<const floatx4 *>(B + kk * 4 * WD_TS + (gx << 2));
+                fb1 = *reinterpret_cast<const floatx4 *>(B + kk * 4 * WD_TS + 16 * WD_CS + (gx << 2));
             };
             floatx4 b0[2], b1[2];
             frag(0, b0[0], b1[0]);
@@ -265,23 +247,17 @@ __global__ __launch_bounds__(384) void winograd_dw_kernel(const WinoDwArgs p)
                 }
             }
         };
-        request(Set0{});       // chunk 0
-        cur_advance(ca);
-        cur_advance(cb);
-        request(Set1{});       // chunk 1
+        request(Set0{}, 0);
+        request(Set1{}, 1);
         __syncthreads();
         for (int c = 0; c < nchunks; c += 2) {
             transform(Set0{});
-            cur_advance(ca);
-            cur_advance(cb);
-            request(Set0{});   // chunk c + 2
+            request(Set0{}, c + 2);
             multiply(0);
             __syncthreads();
             const bool more = c + 1 < nchunks;
             transform(Set1{});
-            cur_advance(ca);
-            cur_advance(cb);
-            request(Set1{});   // chunk c + 3
+            request(Set1{}, c + 3);
             if (more) {
                 multiply(1);
                 __syncthreads();
@@ -331,8 +307,10 @@ hipError_t launch_deltaW_winograd(hipStream_t stream, const float *X, const floa
     if (IC < 4 || OC < 4 || (OC & 3) || N < 1 || OH < 1 || OW < 1 || GZ < 1) return hipErrorNotSupported;
     if (!winograd_deltaW_fits(N, IH, IW, IC, OH, OW, OC)) return hipErrorNotSupported;
     const long x_bytes = (long)N * IH * IW * IC * 4, y_bytes = (long)N * OH * OW * OC * 4;
-    // the patch offsets are sums of a row term and a column term that mark "outside" by 2 GB and 1 GB: X must end below 1 GB
-    if (x_bytes + 8L * IC > (1L << 30) || y_bytes >= (1L << 31)) return hipErrorNotSupported;
+    // the load offsets are sums of terms that mark "outside" by 2 GB (row, deltaY pixel), 1 GB (column, output channel) and
+    // 512 MB (input channel): the tensors must end below the smallest mark that can meet a valid offset
+    if (x_bytes + 16L * IC > ((IC & 31) ? (1L << 29) : (1L << 30))) return hipErrorNotSupported;
+    if (y_bytes >= ((OC & 63) ? (1L << 30) : (1L << 31))) return hipErrorNotSupported;
     WinoDwArgs a{};
     a.X = X; a.dY = dY; a.dW = dW; a.dW_buf = dW_buf;
     a.IH = IH; a.IW = IW; a.IC = IC; a.OH = OH; a.OW = OW; a.OC = OC; a.ph = ph; a.pw = pw;
@@ -343,27 +321,14 @@ hipError_t launch_deltaW_winograd(hipStream_t stream, const float *X, const floa
     if (nt >= (1L << 30)) return hipErrorNotSupported;
     a.ntiles = (int)nt;
     a.GZ = GZ;
-    {   // 8 tiles on: whole images, whole tile rows, tile columns; then at most one wrap of the column and one of the row
-        const int adv_n = WD_TK / a.TRC, rest = WD_TK % a.TRC;
-        a.adv_ty = rest / a.TC;
-        a.adv_tx = rest % a.TC;
-        const long imgX = (long)IH * IW * IC, imgY = (long)OH * OW * OC;
-        const long rowX = 2L * IW * IC, rowY = 2L * OW * OC, colX = 2L * IC, colY = 2L * OC;
-        a.dx0 = (int)(adv_n * imgX + a.adv_ty * rowX + a.adv_tx * colX);
-        a.dy0 = (int)(adv_n * imgY + a.adv_ty * rowY + a.adv_tx * colY);
-        a.wx1 = (int)(rowX - a.TC * colX);
-        a.wy1 = (int)(rowY - a.TC * colY);
-        a.wx2 = (int)(imgX - a.TR * rowX);
-        a.wy2 = (int)(imgY - a.TR * rowY);
-    }
     a.S = (int)(((nt + GZ - 1) / GZ + WD_TK - 1) / WD_TK * WD_TK);
     a.x_bytes = (int)x_bytes; a.y_bytes = (int)y_bytes;
     a.d_TC = make_fastdiv(a.TC);
     a.d_TRC = make_fastdiv(a.TRC);
     constexpr auto kern = winograd_dw_kernel;
-    const size_t lds = (size_t)2 * WD_BUF * sizeof(float);
+    const size_t lds = (size_t)2 * WD_BUF * sizeof(float) + (size_t)2 * WD_TG * (8 + 4) * sizeof(unsigned);
     if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((IC + 31) / 32, (OC + 63) / 64, GZ), dim3(384), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3((IC + 31) / 32, (OC + 63) / 64, GZ), dim3(512), lds, stream, a);
     return hipGetLastError();
 }
 
