@@ -28,7 +28,10 @@
 // pixels of its deltaY tile, "outside" encoded as an offset beyond the descriptor - and every other thread gets the
 // offsets of its tile with two or three 128-bit LDS reads and adds its channel (tile cursors kept per thread and advanced by
 // additions cost 24-67 vector instructions per wavefront and chunk; the staging work on two of the four SIMDs made
-// those two 3.7 k cycles per chunk against 2.05 k of MFMAs).
+// those two 3.7 k cycles per chunk against 2.05 k of MFMAs). Measured and not kept: a staging thread per (tile, four
+// channels) with 128-bit loads, one wavefront per chunk, each chunk spread over four chunk periods so that every SIMD
+// has a quarter of one chunk's staging per period (fewer instructions in total, but 10 % slower: a request then has one
+// period to arrive instead of two).
 // In LDS the 16 xi of a (tile, channel) are contiguous, so a lane's patch operand for four xi is one 128-bit read (an
 // operand per xi as a 32-bit read - three LDS instructions per two MFMAs - cost 30 cycles per pair of MFMAs). A (tile,
 // channel) takes 80 bytes and a tile 32 x 80 + 256: the 32 lanes of a staging write (32 channels of a tile) and the 32
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(512) void winograd_dw_kernel(const WinoDwArgs p)
     unsigned *YT = XT + 2 * WD_TG * 8;
 
     const int t = threadIdx.x;
-    const int lane = t & 63, w = t >> 6;
+    const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l16 = lane & 15, q = lane >> 4;
     const int ic0 = blockIdx.x * 32, oc0 = blockIdx.y * 64, z = blockIdx.z;
     const int tile_begin = z * p.S;
