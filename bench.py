@@ -432,6 +432,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--probe-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy a few times (calibrates FETCH_SIZE/WRITE_SIZE counters)")
+    ap.add_argument("--probe-lds", type=int, default=None, metavar="STRIDE_BYTES",
+                    help="only run a kernel of 128-bit LDS reads whose lanes are STRIDE_BYTES apart (puts the LDS counters of a "
+                         "known access pattern beside those of the real kernels); prints the time per read")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -447,6 +450,28 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"probe": "copy", "bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}))
+        return
+    if args.probe_lds is not None:
+        import ctypes
+        here = os.path.dirname(os.path.abspath(__file__))
+        from __graft_entry__ import package
+        package().lib()   # maps the HIP runtime PyTorch ships before the probe library asks for one
+        probe = ctypes.CDLL(os.path.join(here, "dragon-alpha-v1.0_amd", "libalpha_probe.so"))
+        probe.alpha_probe_lds_read128.argtypes = [ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        blocks, iters = 256, 4096          # one workgroup of four wavefronts per compute unit, 32768 reads per wavefront
+        out = torch.empty(blocks * 256, dtype=torch.float32, device="cuda:0")
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        times = []
+        for _ in range(5):
+            ev[0].record()
+            rc = probe.alpha_probe_lds_read128(torch.cuda.current_stream().cuda_stream, out.data_ptr(), args.probe_lds, iters, blocks)
+            assert rc == 0, rc
+            ev[1].record()
+            torch.cuda.synchronize()
+            times.append(ev[0].elapsed_time(ev[1]))
+        ms = min(times)
+        print(json.dumps({"probe": "lds_read128", "stride_bytes": args.probe_lds, "reads_per_wavefront": 8 * iters,
+                          "wavefronts_per_cu": 4, "ms": round(ms, 4), "ns_per_read_per_cu": round(ms * 1e6 / (8 * iters * 4), 3)}))
         return
     from __graft_entry__ import package
     pkg = package()
