@@ -388,11 +388,12 @@ def measure(wl, op, steps, warmup, with_parity=True):
     }
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     roof["flop_per_byte"] = round(fl / by, 2)
-    if not hbm and fl / by < 2 * RIDGE:   # near the ridge: the other roofline as well
-        roof["hbm_GBps"] = round(by / (k_ms * 1e-3) / 1e9, 1)
-        roof["hbm_frac"] = round(roof["hbm_GBps"] / PEAK_HBM_GBPS, 4)
+    # both fractions for every row, whichever roofline binds
+    roof["mfma_frac"] = round(fl / (k_ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4)
+    roof["hbm_frac"] = round(by / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
     if op in ("wino", "dx_wino", "dw_wino"):
         roof["note"] = "Winograd: FLOPs credited are the direct convolution's (2.25x the multiplies executed); frac is not a roofline fraction"
+        roof["executed_mfma_frac"] = round(roof["mfma_frac"] / 2.25, 4)
     row = {"layer": layer, "op": op, "ms_per_step": round(wall_ms, 5), "event_ms_per_step": round(ev_ms, 5),
            "tflops": round(fl / (wall_ms * 1e-3) / 1e12, 3), "gflop": round(fl / 1e9, 3),
            "algorithmic_MB": round(by / 1e6, 2), "GridZ": wl.GridZ if kind_of(op) == "dw" else None, "roofline": roof}
