@@ -43,10 +43,18 @@ __global__ __launch_bounds__(512, 1) void delta_w_pointwise_kernel(const DwPoint
     const int l16 = lane & 15, q = lane >> 4;
     const int TPW = p.TPW, KSPLIT = 8 / TPW;
     const int tw = w % TPW, kpart = w / TPW;
-    const int tile = blockIdx.x * TPW + tw;
+    // The workgroups of a slice read the same pixels (deltaY or X, whichever their blocks share). Workgroups are dealt
+    // round-robin to the 8 XCDs, each with its own L2: when the slices divide among the XCDs, slice z runs on XCD z % 8,
+    // its workgroups next to each other in time, and the second reader of a row finds it in that L2.
+    int bx = blockIdx.x, z = blockIdx.y;
+    if ((p.GZ & 7) == 0) {
+        const int lin = blockIdx.x + gridDim.x * blockIdx.y, xcd = lin & 7, idx = lin >> 3;
+        bx = idx % (int)gridDim.x;
+        z = xcd + 8 * (idx / (int)gridDim.x);
+    }
+    const int tile = bx * TPW + tw;
     const bool live = tile < p.tiles;
     const int ocb = live ? tile / p.icb_count : 0, icb = live ? tile - ocb * p.icb_count : 0;
-    const int z = blockIdx.y;
 
     const int k_start = p.GK_slice * z;
     const int k_end = (z != p.GZ - 1) ? k_start + p.GK_slice : p.GK;
