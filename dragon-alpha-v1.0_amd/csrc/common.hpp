@@ -208,6 +208,10 @@ hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, 
 // `bias`). Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
 hipError_t launch_pointwise_direct(hipStream_t stream, const float *A, const float *B, float *O, long M, int K, int N,
                                    const float *bias = nullptr, const Epilogue *ep = nullptr);
+// Forward from CW[FH,FW,IC,OC] with both operands straight from memory (any filter, stride, padding): direct_conv.hip.
+// hipErrorNotSupported (nothing launched) when the layer does not fit.
+hipError_t launch_direct_conv(hipStream_t stream, const float *X, const float *CW, float *Y, int N, int IH, int IW, int IC,
+                              int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw, const float *bias, const Epilogue *ep);
 // Backward-data for 4 stored input channels and strides of 1 or 2 (network stems), filter W[OC,FH,FW,4] in place:
 // delta_x_stem.hip. hipErrorNotSupported (nothing launched) when the layer does not fit.
 hipError_t launch_delta_x_stem(hipStream_t stream, const float *dY, const float *W, float *dX, int N, int IH, int IW, int IC,

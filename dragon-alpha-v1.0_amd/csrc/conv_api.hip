@@ -78,6 +78,7 @@ int fwd_algo()
         else if (e && !strcmp(e, "generic")) v = 3;
         else if (e && !strcmp(e, "taps")) v = 4;
         else if (e && !strcmp(e, "rows")) v = 5;
+        else if (e && !strcmp(e, "direct")) v = 6;
         int expected = -1;
         if (!g_fwd_algo.compare_exchange_strong(expected, v)) v = expected;   // a setter was quicker
     }
@@ -95,6 +96,12 @@ bool pointwise_direct_preferred(int K, int N)
     const char *e = getenv("ALPHA_PW_DIRECT");
     if (e) return atoi(e) != 0 && (K % 32) == 0;
     return (K % 32) == 0 && K >= 128 && N <= 64;
+}
+
+// Forward through direct_conv.hip (no LDS): filters of more than one tap on strided layers.
+bool direct_conv_preferred(int FH, int FW, int sh, int sw)
+{
+    return FH * FW > 1 && (sh > 1 || sw > 1);
 }
 
 // The rest of a fused epilogue as a pass of its own over a dense [pixels, C] output (kernels that add a bias only).
@@ -130,6 +137,11 @@ int forward(const char *fn, const int64_t *streams, int length,
         // W[OC][IC] is [N][K]; CW[IC][OC] is [K][N]; a stride only thins the input pixels that are read
         hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW, ep ? nullptr : bias);
         if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), Y, *ep, (long)N * OH * OW, OC);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
+    if (layout == FILTER_CW && (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, sh, sw)))) {
+        // both operands straight from memory: strided layers, whose halo in LDS costs more than it saves
+        hipError_t e = launch_direct_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, bias, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (algo != 3) {
@@ -391,7 +403,7 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz)
 int alpha_conv_get_fwd_algo(void) { return fwd_algo(); }
 int alpha_conv_set_fwd_algo(int algo)
 {
-    if (algo < 0 || algo > 5) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..5");
+    if (algo < 0 || algo > 6) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..6");
     g_fwd_algo.store(algo);
     return 0;
 }

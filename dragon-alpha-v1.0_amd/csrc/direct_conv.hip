@@ -1,0 +1,255 @@
+// Convolution with both operands straight from memory - no LDS, no barrier -, fp32 MFMA v_mfma_f32_16x16x4_f32, gfx950.
+// Any filter size, stride and padding; filter with the produced channel contiguous (CW[FH, FW, IC, OC]).
+//
+//   O[m, co] = sum over taps (th, tw) and channels c of A[n, oh*sh - ph + th, ow*sw - pw + tw, c] * B[(th, tw), c, co]
+//
+// For whom: strided layers. A stride-2 3x3 layer touches every input pixel 2.25 times, so a halo in LDS buys little
+// and costs a lot (four input pixels per output pixel: the LDS-halo kernel's unit of 112 output pixels needs 150 KB,
+// one workgroup per compute unit, nothing overlaps its staging). Here an input pixel's re-reads come out of L1 / L2.
+//
+// The pointwise_direct.hip scheme with a tap loop around it: a wavefront owns T <= 4 tiles of 16 output pixels and one
+// block of 64 produced channels; per step (one tap, 16 reduced channels)
+//   a_t = A[pixel l16 of tile t at this tap][16c + 4q .. +3]       one 128-bit load per tile
+//   b_s = B[tap][16c + 4q + s][n0 + 4*l16 .. +3], s = 0..3           four 128-bit loads, shared by the T tiles
+// and MFMA (t, s, j) multiplies component s of a_t with component j of b_s: 16 T MFMAs per T + 4 loads. A lane's
+// accumulators are 4 consecutive produced channels of a pixel: results leave as 128-bit stores without a transpose.
+// Where a tile's pixels are (they may straddle image rows and images) is worked out per lane once per group of tiles;
+// per tap a lane's load offset is that origin plus the tap's (uniform) term, or an offset beyond the buffer descriptor
+// where the tap falls into the padding (the load then returns zeros): five vector instructions per tile and tap, none
+// per load. Loads run one step ahead of the multiplications through a cursor over (group, tap, channels), so the
+// pipeline does not drain between tiles.
+//
+// Work items are (block of produced channels, tile); a wavefront's share is a contiguous range of them, equal to within
+// one item, processed as groups of 4, 3, 2 or 1 tiles with one loop per group size (every load and store unconditional,
+// every wait an exact count).
+#include "common.hpp"
+
+namespace alpha {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+struct DirectConvArgs {
+    const float *A;   // [N, AH, AW, AC]
+    const float *B;   // element (tap, c, co) at tap * b_tap + c * b_k + co (floats)
+    float *O;         // [M, CO] dense
+    int M, AH, AW, AC, CO;
+    int TH, TW, sh, sw, ph, pw;
+    int b_tap, b_k;
+    int a_bytes, b_bytes, o_bytes;
+    int tiles, nblocks, items, waves;
+    FastDiv d_OW, d_OHW, d_TW;
+    Epilogue ep;
+};
+
+template <int V> struct DcInt { static constexpr int value = V; };
+constexpr unsigned DC_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
+
+template <bool EPI>
+__global__ __launch_bounds__(256, 2) void direct_conv_kernel(const DirectConvArgs p)
+{
+    const int t = threadIdx.x, lane = t & 63;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (t >> 6));
+    const int i_lo = (int)((long)p.items * wave / p.waves), i_hi = (int)((long)p.items * (wave + 1) / p.waves);
+    const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group: even (host-checked)
+
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.B), 0, p.b_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.O, 0, p.o_bytes, 0x00020000);
+
+    // `count` groups of T tiles each, from tile0 on, block nb of the produced channels
+    auto run = [&](auto tc, const int nb, const int tile0, const int count) {
+        constexpr int T = decltype(tc)::value;
+        if (count <= 0) return;
+        const int n_l = nb * 64 + 4 * l16;
+        const unsigned b_lane = n_l < p.CO ? (unsigned)((4 * q * p.b_k + n_l) * 4) : DC_NEVER;
+        const unsigned o_lane = n_l < p.CO ? (unsigned)((4 * q * p.CO + n_l) * 4) : DC_NEVER;
+        floatx4 a[2][T], b[2][4];
+        // ---- load cursor: one step ahead of the multiplications, through (group, tap, 16 channels) ----------------------
+        int c_tile = tile0, c_tap = 0, c_ch = 0, c_left = count * KS;
+        int org[T];          // byte offset of (this lane's pixel's window origin, channel 4q); may lie before the tensor
+        unsigned rc[T];      // bit th: window row th is inside the image; bit 16 + tw: window column tw is
+        unsigned voff[T];    // this tap's load offset, or DC_NEVER in the padding
+        auto locate = [&]() {
+#pragma unroll
+            for (int i = 0; i < T; i++) {
+                const int m = (c_tile + i) * 16 + l16;
+                const bool live = m < p.M;
+                const int mm = live ? m : 0;
+                const int n = fdiv(mm, p.d_OHW), rem = mm - n * (int)p.d_OHW.d;
+                const int oh = fdiv(rem, p.d_OW), ow = rem - oh * (int)p.d_OW.d;
+                const int ih0 = oh * p.sh - p.ph, iw0 = ow * p.sw - p.pw;
+                org[i] = (((n * p.AH + ih0) * p.AW + iw0) * p.AC + 4 * q) * 4;
+                unsigned m_ = 0;
+                for (int th = 0; th < p.TH; th++) m_ |= (unsigned)(live && (unsigned)(ih0 + th) < (unsigned)p.AH) << th;
+                for (int tw = 0; tw < p.TW; tw++) m_ |= (unsigned)((unsigned)(iw0 + tw) < (unsigned)p.AW) << (16 + tw);
+                rc[i] = m_;
+            }
+        };
+        auto aim = [&]() {   // offsets of tap c_tap
+            const int th = fdiv(c_tap, p.d_TW), tw = c_tap - th * p.TW;
+            const int term = (th * p.AW + tw) * p.AC * 4;
+            const unsigned need = (1u << th) | (1u << (16 + tw));
+#pragma unroll
+            for (int i = 0; i < T; i++) voff[i] = (rc[i] & need) == need ? (unsigned)(org[i] + term) : DC_NEVER;
+        };
+        auto request = [&](int slot) {
+            // past the last step the loads repeat the last step's (unused)
+            const int a_off = c_ch * 64;
+            const int b_off = __builtin_amdgcn_readfirstlane((c_tap * p.b_tap + c_ch * 16 * p.b_k) * 4);
+#pragma unroll
+            for (int i = 0; i < T; i++)
+                a[slot][i] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, voff[i], a_off, 0));
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+                b[slot][s] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_lane + (unsigned)(s * p.b_k * 4), b_off, 0));
+            if (c_left > 1) {   // bookkeeping: scalar, and vector arithmetic without memory operations
+                c_left--;
+                c_ch++;
+                if (c_ch == CH) {
+                    c_ch = 0;
+                    c_tap++;
+                    if (c_tap == taps) {
+                        c_tap = 0;
+                        c_tile += T;
+                        locate();
+                    }
+                    aim();
+                }
+            }
+        };
+        locate();
+        aim();
+        request(0);
+        for (int g = 0; g < count; g++) {
+            const int tile = tile0 + g * T;
+            floatx4 acc[T][4];
+#pragma unroll
+            for (int i = 0; i < T; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+            auto multiply = [&](int slot) {
+#pragma unroll
+                for (int s = 0; s < 4; s++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int i = 0; i < T; i++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[slot][i][s], b[slot][s][j], acc[i][j], 0, 0, 0);
+            };
+            for (int ks = 0; ks < KS; ks += 2) {
+                request(1);
+                multiply(0);
+                __builtin_amdgcn_sched_barrier(0);
+                request(0);
+                multiply(1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // ---- results: lane holds pixels 16(tile + i) + 4q + r, produced channels 64 nb + 4 l16 + j -----------------
+            float sub[4], mul[4], add[4];
+            floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
+            if (EPI) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    sub[j] = 0.f; mul[j] = 1.f; add[j] = 0.f;
+                    if (n_l < p.CO && !p.ep.gate) ep_channel(p.ep, n_l + j, sub[j], mul[j], add[j]);
+                }
+            } else if (p.ep.bias != nullptr && n_l < p.CO) {
+                bias = *reinterpret_cast<const floatx4 *>(p.ep.bias + n_l);
+            }
+#pragma unroll
+            for (int i = 0; i < T; i++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int o_off = __builtin_amdgcn_readfirstlane(((tile + i) * 16 + r) * p.CO * 4);   // rows past M: beyond the descriptor
+                    floatx4 v = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+                    if (EPI) {
+                        if (p.ep.gate) {   // uniform
+                            const floatx4 gt = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                                __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.ep.gate), 0, p.o_bytes, 0x00020000), o_lane, o_off, 0));
+#pragma unroll
+                            for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) v[j] = ep_finish(v[j], sub[j], mul[j], add[j], p.ep.slope);
+                        }
+                    } else {
+                        v += bias;
+                    }
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v),
+                                                           o_rsrc, o_lane, o_off, 0);
+                }
+        }
+    };
+
+    // the share as runs of tiles of one block of produced channels each (item = nb * tiles + tile), every run as groups
+    // of 4, 3, 2 and 1 tiles: 4a + 3b for six tiles or more, 3 + 2 for five
+    int i = i_lo;
+    while (i < i_hi) {
+        const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
+        const int cnt = min(i_hi - i, p.tiles - tile0);
+        int n4 = 0, n3 = 0, n2 = 0, n1 = 0;
+        if (cnt >= 6) {
+            n3 = (4 - (cnt & 3)) & 3;
+            n4 = (cnt - 3 * n3) >> 2;
+        } else if (cnt == 5) {
+            n3 = 1; n2 = 1;
+        } else if (cnt == 4) {
+            n4 = 1;
+        } else if (cnt == 3) {
+            n3 = 1;
+        } else if (cnt == 2) {
+            n2 = 1;
+        } else {
+            n1 = 1;
+        }
+        run(DcInt<4>{}, nb, tile0, n4);
+        run(DcInt<3>{}, nb, tile0 + 4 * n4, n3);
+        run(DcInt<2>{}, nb, tile0 + 4 * n4 + 3 * n3, n2);
+        run(DcInt<1>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1);
+        i += cnt;
+    }
+}
+
+// Forward convolution from CW[FH, FW, IC, OC]. Returns hipErrorNotSupported (nothing launched) when the layer does not
+// fit: IC not a multiple of 16, an odd number of steps (FH * FW * IC / 16), a filter beyond 16 x 16, tensors of 2 GB.
+hipError_t launch_direct_conv(hipStream_t stream, const float *X, const float *CW, float *Y, int N, int IH, int IW, int IC,
+                              int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw, const float *bias, const Epilogue *ep)
+{
+    if (IC < 16 || (IC & 15) || OC < 4 || (OC & 3) || FH < 1 || FW < 1 || FH > 16 || FW > 16) return hipErrorNotSupported;
+    if (((FH * FW * (IC >> 4)) & 1) != 0) return hipErrorNotSupported;
+    const long M = (long)N * OH * OW;
+    const long a_bytes = (long)N * IH * IW * IC * 4, b_bytes = (long)FH * FW * IC * OC * 4, o_bytes = M * OC * 4;
+    // a lane's window origin may lie up to ph rows and pw columns before the tensor: its offset must not wrap into range
+    if (M < 1 || a_bytes + ((long)ph * IW + pw + 1) * IC * 4 >= (1L << 31) || o_bytes >= (1L << 31) || b_bytes >= (1L << 30)) return hipErrorNotSupported;
+    const int cus = device_cu_count();
+    if (cus < 1) return hipErrorNotSupported;
+    DirectConvArgs a{};
+    a.A = X; a.B = CW; a.O = Y;
+    a.M = (int)M; a.AH = IH; a.AW = IW; a.AC = IC; a.CO = OC;
+    a.TH = FH; a.TW = FW; a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
+    a.b_tap = IC * OC; a.b_k = OC;
+    a.a_bytes = (int)a_bytes; a.b_bytes = (int)b_bytes; a.o_bytes = (int)o_bytes;
+    a.tiles = (int)((M + 15) / 16);
+    a.nblocks = (OC + 63) / 64;
+    if ((long)a.tiles * a.nblocks >= (1L << 30)) return hipErrorNotSupported;
+    a.items = a.tiles * a.nblocks;
+    a.d_OW = make_fastdiv(OW);
+    a.d_OHW = make_fastdiv(OH * OW);
+    a.d_TW = make_fastdiv(FW);
+    a.ep = ep ? *ep : bias_epilogue(bias);
+    // one or two wavefronts per SIMD, whichever leaves the shares more even (the largest share sets the time)
+    int wgs = 2 * cus;
+    {
+        const long w1 = 4L * cus, w2 = 8L * cus;
+        const long s1 = (a.items + w1 - 1) / w1, s2 = (a.items + w2 - 1) / w2;
+        if (s1 * w1 < s2 * w2) wgs = cus;   // items / (waves * largest share) is higher with one wavefront per SIMD
+    }
+    if (wgs * 4 > a.items) wgs = (a.items + 3) / 4;
+    a.waves = wgs * 4;
+    if (a.ep.fused) hipLaunchKernelGGL(direct_conv_kernel<true>, dim3(wgs), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(direct_conv_kernel<false>, dim3(wgs), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace alpha

@@ -53,8 +53,8 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz);
  * 0 = auto, 1 = implicit GEMM only (LDS-halo kernel where eligible, else the generic one),
  * 2 = Winograd F(2x2,3x3) where eligible, 3 = the generic kernels only,
  * 4 = backward-filter through the tap-per-workgroup kernel wherever it fits, 5 = through the row-streaming kernel
- * wherever it fits (forward and backward-data as 0).
- * Also read once from the environment variable ALPHA_HIP_CONV_ALGO = auto|igemm|winograd|generic|taps|rows.
+ * wherever it fits (forward and backward-data as 0), 6 = forward from CW through the kernel without LDS wherever it fits.
+ * Also read once from the environment variable ALPHA_HIP_CONV_ALGO = auto|igemm|winograd|generic|taps|rows|direct.
  * No counterpart in the reference (its Winograd experiments are compiled out, conv/conv3D.cuh:39-44). */
 int alpha_conv_set_fwd_algo(int algo);
 int alpha_conv_get_fwd_algo(void);

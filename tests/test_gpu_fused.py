@@ -60,7 +60,7 @@ FUSED_SHAPES = [
     (4, 14, 14, 64, 64, 3, 3, 1, 1, 1, 1, "3x3 stride-1 kernel with the prefetched halo"),
     (4, 8, 8, 128, 132, 3, 3, 1, 1, 1, 1, "the same, narrow rows, ragged block of output channels"),
     (4, 13, 13, 20, 36, 3, 3, 1, 1, 1, 1, "ragged channel counts: generic kernel"),
-    (4, 14, 14, 64, 128, 3, 3, 2, 2, 1, 1, "strided LDS-halo kernel"),
+    (4, 14, 14, 64, 128, 3, 3, 2, 2, 1, 1, "strided: the kernel without LDS from CW, the LDS-halo kernel from W"),
     (4, 12, 12, 96, 64, 5, 5, 1, 1, 2, 2, "LDS-halo kernel, 5x5"),
     (4, 30, 30, 4, 64, 7, 7, 2, 2, 3, 3, "stem kernel"),
     (4, 14, 14, 64, 128, 1, 1, 1, 1, 0, 0, "1x1 streaming kernel + a separate pass"),

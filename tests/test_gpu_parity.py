@@ -388,6 +388,51 @@ def test_pointwise_kernel_strided(dev, shape):
         check(_run_fwd(dev, entry, X, W, sh, sw, 0, 0), want, "%s strided 1x1 %s" % (entry, shape))
 
 
+def _run_fwd_biased(dev, X, W, B, sh, sw, ph, pw):
+    N, IH, IW, IC = X.shape
+    OC, FH, FW, _ = W.shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    x, w, b = dev.put(X), dev.put(W), dev.put(B)
+    cw = dev.empty(FH * FW * IC * OC, fill=float("nan"))
+    C3.kernel_remode(dev.stream, w.data_ptr(), cw.data_ptr(), FH, FW, OC, IC)
+    y = dev.guarded(N, OH, OW, OC)
+    C3.conv3D_GemmR_biased(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), cw.data_ptr(), FH, FW, b.data_ptr(), y.data_ptr(),
+                           OH, OW, N, IC, OC, sh, sw, ph, pw)
+    return dev.get(y)
+
+
+DIRECT_CONV_SHAPES = [
+    # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw: the kernel without LDS (both operands from memory), forward from CW
+    (4, 28, 28, 64, 128, 3, 3, 2, 2, 1, 1),     # c4b geometry (56 -> 28 there): two blocks of produced channels
+    (16, 56, 56, 64, 128, 3, 3, 2, 2, 1, 1),    # 12544 pixels = 784 tiles x 2 blocks: shares of 1 and 2 items
+    (4, 15, 13, 64, 64, 3, 3, 2, 2, 1, 1),      # odd sizes: tiles straddle rows and images, last tile ragged
+    (4, 17, 19, 32, 96, 5, 3, 2, 3, 2, 1),      # mixed strides, non-square filter, 96 = one and a half blocks
+    (2, 16, 16, 96, 64, 2, 2, 2, 2, 0, 0),      # no overlap, no padding
+    (3, 9, 30, 64, 36, 3, 3, 1, 2, 1, 1),       # stride only along the width; a ragged block of 36 produced channels
+    (2, 12, 12, 32, 64, 3, 3, 1, 1, 1, 1),      # stride 1 (forced): every tap of a border pixel's window in the padding
+    (1, 5, 5, 16, 8, 7, 6, 1, 1, 3, 3),         # window larger than the image, 16 channels (42 steps), 8 produced channels
+    (40, 20, 20, 32, 64, 3, 3, 2, 2, 1, 1),     # 4000 pixels = 250 tiles: fewer items than wavefronts
+    (64, 30, 34, 48, 64, 3, 3, 2, 2, 1, 1),     # 16320 pixels = 1020 tiles, 48 channels (27 steps are odd: refused -> other kernel)
+]
+
+
+@pytest.mark.parametrize("shape", DIRECT_CONV_SHAPES)
+def test_forward_direct_conv_kernel(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
+    X, W = normal((N, IH, IW, IC), 2401), he_normal(OC, FH, FW, IC, 2402)
+    bias = normal((OC,), 2403)
+    want = O.conv3D_f64(X, W, sh, sw, ph, pw)
+    L = pkg.lib()
+    try:
+        for algo in (6, 1, 3):      # the kernel without LDS, the LDS-halo kernel, the generic kernel
+            L.alpha_conv_set_fwd_algo(algo)
+            for entry in ("conv3D_GemmR", "conv3D_GemmR_texture", "conv3D_GemmV2R"):
+                check(_run_fwd(dev, entry, X, W, sh, sw, ph, pw), want, "%s algo %d %s" % (entry, algo, shape))
+            check(_run_fwd_biased(dev, X, W, bias, sh, sw, ph, pw), want + bias.astype(np.float64), "GemmR_biased algo %d %s" % (algo, shape))
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+
+
 STRIDED_TAP_SHAPES = [
     # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw: strided layers with >= 32 input channels through the LDS-halo kernel
     # (columns of the halo de-interleaved by ow parity class), remode entries
@@ -406,7 +451,7 @@ def test_strided_forward_through_the_halo_kernel(dev, shape):
     want = O.conv3D_f64(X, W, sh, sw, ph, pw)
     L = pkg.lib()
     try:
-        for algo in (0, 3):   # 0: halo kernel, 3: generic kernel
+        for algo in (0, 1, 3):   # 0: the library's choice, 1: LDS-halo kernel, 3: generic kernel
             L.alpha_conv_set_fwd_algo(algo)
             for entry in ("conv3D_GemmR", "conv3D_GemmV2R"):
                 check(_run_fwd(dev, entry, X, W, sh, sw, ph, pw), want, "%s algo %d %s" % (entry, algo, shape))
