@@ -208,10 +208,14 @@ hipError_t launch_pointwise(hipStream_t stream, const float *A, const float *B, 
 // `bias`). Returns hipErrorNotSupported (nothing launched) when the layer does not fit.
 hipError_t launch_pointwise_direct(hipStream_t stream, const float *A, const float *B, float *O, long M, int K, int N,
                                    const float *bias = nullptr, const Epilogue *ep = nullptr);
-// Forward from CW[FH,FW,IC,OC] with both operands straight from memory (any filter, stride, padding): direct_conv.hip.
-// hipErrorNotSupported (nothing launched) when the layer does not fit.
-hipError_t launch_direct_conv(hipStream_t stream, const float *X, const float *CW, float *Y, int N, int IH, int IW, int IC,
-                              int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw, const float *bias, const Epilogue *ep);
+// Convolution with both operands straight from memory (any filter, stride, padding): direct_conv.hip. Filter element
+// (tap = th*TW + tw, c, co) at b_off + tap*b_tap + c*b_k + co, `b_elems` floats in all. hipErrorNotSupported (nothing
+// launched) when the layer does not fit. direct_conv_balanced: whether its work divides evenly enough among the
+// wavefronts to beat the LDS-halo kernels on a stride-1 layer.
+hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC,
+                              int OHt, int OWt, int CO, int TH, int TW, int sh, int sw, int ph, int pw,
+                              int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep);
+bool direct_conv_balanced(long M, int CO);
 // Backward-data for 4 stored input channels and strides of 1 or 2 (network stems), filter W[OC,FH,FW,4] in place:
 // delta_x_stem.hip. hipErrorNotSupported (nothing launched) when the layer does not fit.
 hipError_t launch_delta_x_stem(hipStream_t stream, const float *dY, const float *W, float *dX, int N, int IH, int IW, int IC,

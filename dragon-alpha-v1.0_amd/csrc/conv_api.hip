@@ -98,10 +98,12 @@ bool pointwise_direct_preferred(int K, int N)
     return (K % 32) == 0 && K >= 128 && N <= 64;
 }
 
-// Forward through direct_conv.hip (no LDS): filters of more than one tap on strided layers.
-bool direct_conv_preferred(int FH, int FW, int sh, int sw)
+// Through direct_conv.hip (no LDS): filters of more than one tap on strided layers (the halo kernel's LDS footprint is
+// four input pixels per output pixel there), and stride-1 layers whose work items divide evenly among the wavefronts.
+bool direct_conv_preferred(int FH, int FW, int sh, int sw, long M, int CO)
 {
-    return FH * FW > 1 && (sh > 1 || sw > 1);
+    if (FH * FW <= 1) return false;
+    return sh > 1 || sw > 1 || direct_conv_balanced(M, CO);
 }
 
 // The rest of a fused epilogue as a pass of its own over a dense [pixels, C] output (kernels that add a bias only).
@@ -139,9 +141,10 @@ int forward(const char *fn, const int64_t *streams, int length,
         if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), Y, *ep, (long)N * OH * OW, OC);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (layout == FILTER_CW && (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, sh, sw)))) {
-        // both operands straight from memory: strided layers, whose halo in LDS costs more than it saves
-        hipError_t e = launch_direct_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, bias, ep);
+    if (layout == FILTER_CW && (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, sh, sw, (long)N * OH * OW, OC)))) {
+        // both operands straight from memory
+        hipError_t e = launch_direct_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
+                                          0, IC * OC, OC, (long)FH * FW * IC * OC, bias, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (algo != 3) {
@@ -193,6 +196,12 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
         // deltaX[m][ic] = sum_oc deltaY[m][oc] * W[oc][ic]: W is [K][N]
         hipError_t e = launch_pointwise(stream0(streams), dY, W, dX, N, IH, IW, IH, IW, 1, 1, OC, IC, 1);
         if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), dX, *ep, (long)N * IH * IW, IC);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
+    if (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, 1, 1, (long)N * IH * IW, IC))) {
+        // both operands straight from memory; W rotated by 180 degrees is read in place (input channel contiguous)
+        hipError_t e = launch_direct_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, 1, 1, FH - 1 - ph, FW - 1 - pw,
+                                          (FH * FW - 1) * IC, -IC, FH * FW * IC, (long)OC * FH * FW * IC, nullptr, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (algo != 3) {

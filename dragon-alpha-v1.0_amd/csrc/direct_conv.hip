@@ -1,5 +1,6 @@
 // Convolution with both operands straight from memory - no LDS, no barrier -, fp32 MFMA v_mfma_f32_16x16x4_f32, gfx950.
-// Any filter size, stride and padding; filter with the produced channel contiguous (CW[FH, FW, IC, OC]).
+// Any filter size, stride and padding; filter with the produced channel contiguous (CW[FH, FW, IC, OC] forward,
+// W[OC, FH, FW, IC] rotated by 180 degrees for stride-1 backward-data).
 //
 //   O[m, co] = sum over taps (th, tw) and channels c of A[n, oh*sh - ph + th, ow*sw - pw + tw, c] * B[(th, tw), c, co]
 //
@@ -30,11 +31,11 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 struct DirectConvArgs {
     const float *A;   // [N, AH, AW, AC]
-    const float *B;   // element (tap, c, co) at tap * b_tap + c * b_k + co (floats)
+    const float *B;   // element (tap, c, co) at b_off + tap * b_tap + c * b_k + co (floats); b_tap may be negative
     float *O;         // [M, CO] dense
     int M, AH, AW, AC, CO;
     int TH, TW, sh, sw, ph, pw;
-    int b_tap, b_k;
+    int b_off, b_tap, b_k;
     int a_bytes, b_bytes, o_bytes;
     int tiles, nblocks, items, waves;
     FastDiv d_OW, d_OHW, d_TW;
@@ -96,7 +97,7 @@ __global__ __launch_bounds__(256, 2) void direct_conv_kernel(const DirectConvArg
         auto request = [&](int slot) {
             // past the last step the loads repeat the last step's (unused)
             const int a_off = c_ch * 64;
-            const int b_off = __builtin_amdgcn_readfirstlane((c_tap * p.b_tap + c_ch * 16 * p.b_k) * 4);
+            const int b_off = __builtin_amdgcn_readfirstlane((p.b_off + c_tap * p.b_tap + c_ch * 16 * p.b_k) * 4);
 #pragma unroll
             for (int i = 0; i < T; i++)
                 a[slot][i] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, voff[i], a_off, 0));
@@ -211,40 +212,60 @@ __global__ __launch_bounds__(256, 2) void direct_conv_kernel(const DirectConvArg
     }
 }
 
-// Forward convolution from CW[FH, FW, IC, OC]. Returns hipErrorNotSupported (nothing launched) when the layer does not
-// fit: IC not a multiple of 16, an odd number of steps (FH * FW * IC / 16), a filter beyond 16 x 16, tensors of 2 GB.
-hipError_t launch_direct_conv(hipStream_t stream, const float *X, const float *CW, float *Y, int N, int IH, int IW, int IC,
-                              int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw, const float *bias, const Epilogue *ep)
+// Share of the wavefronts' time that is work when `items` equal items are dealt to one or two wavefronts per SIMD
+// (whichever is better): the largest share sets the time.
+static double direct_conv_balance(long items, int cus, int *wgs_out)
 {
-    if (IC < 16 || (IC & 15) || OC < 4 || (OC & 3) || FH < 1 || FW < 1 || FH > 16 || FW > 16) return hipErrorNotSupported;
-    if (((FH * FW * (IC >> 4)) & 1) != 0) return hipErrorNotSupported;
-    const long M = (long)N * OH * OW;
-    const long a_bytes = (long)N * IH * IW * IC * 4, b_bytes = (long)FH * FW * IC * OC * 4, o_bytes = M * OC * 4;
-    // a lane's window origin may lie up to ph rows and pw columns before the tensor: its offset must not wrap into range
-    if (M < 1 || a_bytes + ((long)ph * IW + pw + 1) * IC * 4 >= (1L << 31) || o_bytes >= (1L << 31) || b_bytes >= (1L << 30)) return hipErrorNotSupported;
+    const long w1 = 4L * cus, w2 = 8L * cus;
+    const long s1 = (items + w1 - 1) / w1, s2 = (items + w2 - 1) / w2;
+    const bool one = s1 * w1 < s2 * w2;
+    if (wgs_out) *wgs_out = one ? cus : 2 * cus;
+    return (double)items / (double)(one ? s1 * w1 : s2 * w2);
+}
+
+// Whether the kernel's work items (16 pixels x 64 produced channels) divide evenly enough among the wavefronts for it
+// to beat the LDS-halo kernels on a stride-1 layer. Measured (forward, 3x3): 8x8x256 and 16x16x128 at N = 128 (shares
+// exactly equal) 9-12 % and 5 % faster; 56x56x64, 28x28x128 at N = 64 (seven items where the mean is 6.1) within 2.5 %
+// either way; 14x14x256 (two items where the mean is 1.5) 7 % slower.
+bool direct_conv_balanced(long M, int CO)
+{
+    const int cus = device_cu_count();
+    if (cus < 1 || M < 1) return false;
+    return direct_conv_balance(((M + 15) / 16) * ((CO + 63) / 64), cus, nullptr) >= 0.95;
+}
+
+// O[N, OHt, OWt, CO] = convolution of A[N, AH, AW, AC] (stride sh x sw, padding ph x pw, TH x TW taps) with the filter B
+// whose element (tap = th * TW + tw, c, co) is at b_off + tap * b_tap + c * b_k + co: CW[FH, FW, IC, OC] forward
+// (0, IC * OC, OC), W[OC, FH, FW, IC] rotated by 180 degrees for stride-1 backward-data ((FH*FW - 1) * IC, -IC, FH*FW*IC).
+// Returns hipErrorNotSupported (nothing launched) when the layer does not fit: AC not a multiple of 16, an odd number
+// of steps (TH * TW * AC / 16), a filter beyond 16 x 16, tensors of 2 GB.
+hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC,
+                              int OHt, int OWt, int CO, int TH, int TW, int sh, int sw, int ph, int pw,
+                              int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep)
+{
+    if (AC < 16 || (AC & 15) || CO < 4 || (CO & 3) || TH < 1 || TW < 1 || TH > 16 || TW > 16) return hipErrorNotSupported;
+    if (((TH * TW * (AC >> 4)) & 1) != 0) return hipErrorNotSupported;
+    const long M = (long)N * OHt * OWt;
+    const long a_bytes = (long)N * AH * AW * AC * 4, b_bytes = b_elems * 4, o_bytes = M * CO * 4;
+    if (M < 1 || a_bytes >= (1L << 31) || o_bytes >= (1L << 31) || b_bytes >= (1L << 30)) return hipErrorNotSupported;
     const int cus = device_cu_count();
     if (cus < 1) return hipErrorNotSupported;
     DirectConvArgs a{};
-    a.A = X; a.B = CW; a.O = Y;
-    a.M = (int)M; a.AH = IH; a.AW = IW; a.AC = IC; a.CO = OC;
-    a.TH = FH; a.TW = FW; a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
-    a.b_tap = IC * OC; a.b_k = OC;
+    a.A = A; a.B = B; a.O = O;
+    a.M = (int)M; a.AH = AH; a.AW = AW; a.AC = AC; a.CO = CO;
+    a.TH = TH; a.TW = TW; a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
+    a.b_off = b_off; a.b_tap = b_tap; a.b_k = b_k;
     a.a_bytes = (int)a_bytes; a.b_bytes = (int)b_bytes; a.o_bytes = (int)o_bytes;
     a.tiles = (int)((M + 15) / 16);
-    a.nblocks = (OC + 63) / 64;
+    a.nblocks = (CO + 63) / 64;
     if ((long)a.tiles * a.nblocks >= (1L << 30)) return hipErrorNotSupported;
     a.items = a.tiles * a.nblocks;
-    a.d_OW = make_fastdiv(OW);
-    a.d_OHW = make_fastdiv(OH * OW);
-    a.d_TW = make_fastdiv(FW);
+    a.d_OW = make_fastdiv(OWt);
+    a.d_OHW = make_fastdiv(OHt * OWt);
+    a.d_TW = make_fastdiv(TW);
     a.ep = ep ? *ep : bias_epilogue(bias);
-    // one or two wavefronts per SIMD, whichever leaves the shares more even (the largest share sets the time)
     int wgs = 2 * cus;
-    {
-        const long w1 = 4L * cus, w2 = 8L * cus;
-        const long s1 = (a.items + w1 - 1) / w1, s2 = (a.items + w2 - 1) / w2;
-        if (s1 * w1 < s2 * w2) wgs = cus;   // items / (waves * largest share) is higher with one wavefront per SIMD
-    }
+    direct_conv_balance(a.items, cus, &wgs);   // one or two wavefronts per SIMD, whichever leaves the shares more even
     if (wgs * 4 > a.items) wgs = (a.items + 3) / 4;
     a.waves = wgs * 4;
     if (a.ep.fused) hipLaunchKernelGGL(direct_conv_kernel<true>, dim3(wgs), dim3(256), 0, stream, a);

@@ -176,8 +176,14 @@ def test_forward_lds_halo_kernel_vs_oracle_and_generic(dev, shape):
         fast_w = _run_fwd(dev, "conv3D", X, W, 1, 1, ph, pw)   # W[OC,FH,FW,IC] as it is (3x3: 128-bit filter fragment loads)
         L.alpha_conv_set_fwd_algo(3)
         generic = _run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, ph, pw)
+        L.alpha_conv_set_fwd_algo(1)
+        halo = _run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, ph, pw)
+        L.alpha_conv_set_fwd_algo(6)
+        direct = _run_fwd(dev, "conv3D_GemmR", X, W, 1, 1, ph, pw)
     finally:
         L.alpha_conv_set_fwd_algo(0)
+    check(halo, want, "lds-halo fwd (forced) %s" % (shape,))
+    check(direct, want, "fwd without LDS (forced) %s" % (shape,))
     check(fast, want, "lds-halo fwd %s" % (shape,))
     check(fast_w, want, "lds-halo fwd from W %s" % (shape,))
     check(generic, want, "generic fwd %s" % (shape,))
@@ -191,9 +197,16 @@ def test_deltaX_lds_halo_kernel_vs_oracle(dev, shape):
     OH, OW = out_dim(IH, IW, FH, FW, 1, 1, ph, pw)
     dY, W = normal((N, OH, OW, OC), 1103), he_normal(OC, FH, FW, IC, 1104)
     dy, w = dev.put(dY), dev.put(W)
-    dXo = dev.guarded(N, IH, IW, IC)
-    DX.dconv3D_deltaX_s1(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC, ph, pw)
-    check(dev.get(dXo), O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw), "lds-halo dX %s" % (shape,))
+    want = O.deltaX_f64(dY, W, IH, IW, 1, 1, ph, pw)
+    L = pkg.lib()
+    try:
+        for algo in (0, 1, 6, 3):   # the library's choice, the LDS-halo kernels, the kernel without LDS, the generic kernel
+            L.alpha_conv_set_fwd_algo(algo)
+            dXo = dev.guarded(N, IH, IW, IC)
+            DX.dconv3D_deltaX_s1(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC, ph, pw)
+            check(dev.get(dXo), want, "dX algo %d %s" % (algo, shape))
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
 
 
 WINO_SHAPES = [
