@@ -276,10 +276,30 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
             if (th == 0) a.b_off = 0;
             phases.push_back(Phase{a, th, tw, OHt, OWt});
         }
+    // Up to four phases of the same size (IH % sh == 0, IW % sw == 0: the reference's Ims case): ONE launch of the kernel
+    // without LDS, every wavefront running all phases on its tiles of coarse pixels.
+    const int algo = fwd_algo();
+    if ((algo == 0 || algo == 6) && sh * sw <= 4 && IH % sh == 0 && IW % sw == 0 && (int)phases.size() == sh * sw) {
+        int TH[4], TW[4], pph[4], ppw[4], boff[4], bsth[4], ooff[4];
+        bool same = true;
+        for (int f = 0; f < sh * sw; f++) {
+            const GatherConvArgs &a = phases[f].a;
+            TH[f] = phases[f].th; TW[f] = phases[f].tw; pph[f] = a.ph; ppw[f] = a.pw; boff[f] = a.b_off; bsth[f] = a.b_sth; ooff[f] = a.o_off;
+            same = same && phases[f].OHt == phases[0].OHt && phases[f].OWt == phases[0].OWt;
+        }
+        if (same) {
+            const GatherConvArgs &a0 = phases[0].a;
+            const long b_elems = from_CW ? (long)sh * sw * CWstride : (long)OC * FH * FW * IC;
+            hipError_t e = launch_direct_conv_phased(s, dY, F, dX, N, OH, OW, OC, IC, phases[0].OHt, phases[0].OWt, sh * sw, TH, TW, pph, ppw,
+                                                     boff, bsth, a0.b_stw, a0.b_sc, b_elems, ooff, a0.o_sn, a0.o_sh, a0.o_sw,
+                                                     (long)N * IH * IW * IC, ep);
+            if (e != hipErrorNotSupported) return hip_status(e, fn);
+        }
+    }
     // Stride 2 x 2 with even sizes (the reference's Ims2 case): the four phases in ONE launch, sharing one LDS halo per
     // unit (the reference runs its phases in one grid too: dconv3D_dX_kernelSplit_Ims2R_kernel.cuh:18, dim3(.., .., 4)).
     // Everything else, and whatever that kernel refuses: one launch of the generic kernel per phase.
-    if (fwd_algo() != 3 && sh == 2 && sw == 2 && (IH & 1) == 0 && (IW & 1) == 0 && phases.size() == 4) {
+    if (algo != 3 && sh == 2 && sw == 2 && (IH & 1) == 0 && (IW & 1) == 0 && phases.size() == 4) {
         int TH[4], TW[4], pph[4], ppw[4], boff[4], bsth[4], ooff[4];
         for (int f = 0; f < 4; f++) {
             const GatherConvArgs &a = phases[f].a;

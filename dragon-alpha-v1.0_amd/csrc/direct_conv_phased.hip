@@ -1,0 +1,284 @@
+// Kernel-split backward-data (stride > 1) with both operands straight from memory - the phased form of
+// direct_conv.hip -, fp32 MFMA v_mfma_f32_16x16x4_f32, gfx950. No LDS, no barrier.
+//
+// deltaX of a strided layer is sh*sw dense stride-1 problems ("phases"), one per sub-lattice of deltaX, each with its
+// own subset of the filter taps. Phase f:
+//   O[o_off[f] + n*o_sn + i*o_sh + j*o_sw + co] = sum over th < TH[f], tw < TW[f], c < AC of
+//       A[n, i - ph[f] + th, j - pw[f] + tw, c] * B[b_off[f] + th*b_sth[f] + tw*b_stw + c*b_k + co]
+// for the "coarse" pixels (n, i, j), i < OHt, j < OWt - the same set for every phase. A work item is (phase, block of
+// 64 produced channels, tile of 16 coarse pixels) and costs its phase's number of taps; a wavefront owns T <= 4 tiles of
+// one phase at a time and the scheme is direct_conv.hip's: per step (one tap, 16 reduced channels) one 128-bit load per
+// tile and four for the filter feed 16 T MFMAs, loads run one step ahead through a cursor over (group, tap, channels),
+// results leave as 128-bit stores. A phase without taps (filter smaller than the stride) writes zeros.
+//
+// Shares: the items in the order (phase, block, tile) form a line of cost - 4 per tap plus 1 for the item's stores -; the
+// wavefronts' shares are equal stretches of it, cut between items. A share then differs from the mean by at most one item - a quarter of the cost of a tile with
+// all its phases - and still consists of runs of tiles of one phase, so that a filter fragment serves up to four tiles.
+// (Whole tiles with all phases: shares of 3 and 4 on 56x56 -> 28x28, 64 channels - 3136 tiles on 1024 SIMDs; shares cut
+// inside tiles with the cut tiles run alone: the filter is then read per tile, 0.6 GB from L2, and nothing is gained.)
+#include "common.hpp"
+
+namespace alpha {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+struct DirectPhasedArgs {
+    const float *A;   // [N, AH, AW, AC]
+    const float *B;
+    float *O;
+    int M, AH, AW, AC, CO;   // M = N * OHt * OWt coarse pixels
+    int nph;
+    int f_TH[4], f_TW[4], f_ph[4], f_pw[4], f_b_off[4], f_b_sth[4], f_o_off[4];
+    int b_stw, b_k;
+    int o_sn, o_sh, o_sw;
+    int a_bytes, b_bytes, o_bytes;
+    int tiles, nblocks, items, waves;
+    long total_cost;         // items * sum over the phases of (4 * TH * TW + 1)
+    FastDiv d_OW, d_OHW;
+    Epilogue ep;
+};
+
+template <int V> struct DcpInt { static constexpr int value = V; };
+constexpr unsigned DCP_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
+
+template <bool EPI>
+__global__ __launch_bounds__(256, 2) void direct_conv_phased_kernel(const DirectPhasedArgs p)
+{
+    const int t = threadIdx.x, lane = t & 63;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (t >> 6));
+    const int CH = p.AC >> 4;   // even (host-checked): every phase has an even number of steps
+
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.B), 0, p.b_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.O, 0, p.o_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t g_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(EPI ? p.ep.gate : p.A), 0, EPI ? p.o_bytes : 0, 0x00020000);
+
+    // phase data by (uniform) index
+    auto TH = [&](int f) { return f == 0 ? p.f_TH[0] : f == 1 ? p.f_TH[1] : f == 2 ? p.f_TH[2] : p.f_TH[3]; };
+    auto TW = [&](int f) { return f == 0 ? p.f_TW[0] : f == 1 ? p.f_TW[1] : f == 2 ? p.f_TW[2] : p.f_TW[3]; };
+    auto PH = [&](int f) { return f == 0 ? p.f_ph[0] : f == 1 ? p.f_ph[1] : f == 2 ? p.f_ph[2] : p.f_ph[3]; };
+    auto PW = [&](int f) { return f == 0 ? p.f_pw[0] : f == 1 ? p.f_pw[1] : f == 2 ? p.f_pw[2] : p.f_pw[3]; };
+    auto BOFF = [&](int f) { return f == 0 ? p.f_b_off[0] : f == 1 ? p.f_b_off[1] : f == 2 ? p.f_b_off[2] : p.f_b_off[3]; };
+    auto BSTH = [&](int f) { return f == 0 ? p.f_b_sth[0] : f == 1 ? p.f_b_sth[1] : f == 2 ? p.f_b_sth[2] : p.f_b_sth[3]; };
+    auto OOFF = [&](int f) { return f == 0 ? p.f_o_off[0] : f == 1 ? p.f_o_off[1] : f == 2 ? p.f_o_off[2] : p.f_o_off[3]; };
+
+    // `count` groups of T tiles each, from tile0 on, block nb of the produced channels, phase f
+    auto run = [&](auto tc, const int f, const int nb, const int tile0, const int count) {
+        constexpr int T = decltype(tc)::value;
+        if (count <= 0) return;
+        const int fTH = TH(f), fTW = TW(f), fPH = PH(f), fPW = PW(f), fBOFF = BOFF(f), fBSTH = BSTH(f);
+        const int steps = fTH * fTW * CH;
+        const int n_l = nb * 64 + 4 * l16;
+        const bool n_ok = n_l < p.CO;
+        const unsigned b_lane = n_ok ? (unsigned)((4 * q * p.b_k + n_l) * 4) : DCP_NEVER;
+        floatx4 a[2][T], b[2][4];
+        // ---- load cursor: one step ahead of the multiplications, through (group, phase, tap, 16 channels) ----------------
+        int c_tile = tile0, c_th = 0, c_tw = 0, c_ch = 0, c_left = count * steps;
+        int org[T], pi[T], pj[T];   // lane l16's coarse pixel of tile i: byte offset of A[n, i, j, 4q], and (i, j)
+        unsigned voff[T];           // this tap's load offset, or DCP_NEVER in the padding
+        unsigned opix[T][4];        // byte offset of the lane's result pixels 4q + r in O (phase offset apart), or DCP_NEVER
+        auto locate = [&]() {
+#pragma unroll
+            for (int i = 0; i < T; i++) {
+                const int m = (c_tile + i) * 16 + l16;
+                const bool live = m < p.M;
+                const int mm = live ? m : 0;
+                const int n = fdiv(mm, p.d_OHW), rem = mm - n * (int)p.d_OHW.d;
+                const int ii = fdiv(rem, p.d_OW), jj = rem - ii * (int)p.d_OW.d;
+                org[i] = (((n * p.AH + ii) * p.AW + jj) * p.AC + 4 * q) * 4;
+                pi[i] = live ? ii : -0x1000000;   // every window row of a dead pixel is outside
+                pj[i] = jj;
+            }
+        };
+        auto aim = [&]() {   // offsets of tap (c_th, c_tw)
+            const int dy = c_th - fPH, dx = c_tw - fPW;
+            const int term = (dy * p.AW + dx) * p.AC * 4;
+#pragma unroll
+            for (int i = 0; i < T; i++) {
+                const bool ok = (unsigned)(pi[i] + dy) < (unsigned)p.AH && (unsigned)(pj[i] + dx) < (unsigned)p.AW;
+                voff[i] = ok ? (unsigned)(org[i] + term) : DCP_NEVER;
+            }
+        };
+        auto request = [&](int slot) {
+            // past the last step the loads repeat the last step's (unused)
+            const int a_off = c_ch * 64;
+            const int b_off = __builtin_amdgcn_readfirstlane((fBOFF + c_th * fBSTH + c_tw * p.b_stw + c_ch * 16 * p.b_k) * 4);
+#pragma unroll
+            for (int i = 0; i < T; i++)
+                a[slot][i] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, voff[i], a_off, 0));
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+                b[slot][s] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_lane + (unsigned)(s * p.b_k * 4), b_off, 0));
+            if (c_left > 1) {   // bookkeeping: scalar, and vector arithmetic without memory operations
+                c_left--;
+                c_ch++;
+                if (c_ch == CH) {
+                    c_ch = 0;
+                    c_tw++;
+                    if (c_tw == fTW) {
+                        c_tw = 0;
+                        c_th++;
+                        if (c_th == fTH) {   // the next group
+                            c_th = 0;
+                            c_tile += T;
+                            locate();
+                        }
+                    }
+                    aim();
+                }
+            }
+        };
+        if (steps > 0) {
+            locate();
+            aim();
+            request(0);
+        }
+        for (int g = 0; g < count; g++) {
+            const int tile = tile0 + g * T;
+            // where this lane's results go: pixels 16(tile + i) + 4q + r, produced channels 64 nb + 4 l16 + j
+#pragma unroll
+            for (int i = 0; i < T; i++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int m = (tile + i) * 16 + 4 * q + r;
+                    const bool live = m < p.M && n_ok;
+                    const int mm = m < p.M ? m : 0;
+                    const int n = fdiv(mm, p.d_OHW), rem = mm - n * (int)p.d_OHW.d;
+                    const int ii = fdiv(rem, p.d_OW), jj = rem - ii * (int)p.d_OW.d;
+                    opix[i][r] = live ? (unsigned)((n * p.o_sn + ii * p.o_sh + jj * p.o_sw + n_l) * 4) : DCP_NEVER;
+                }
+            {
+                floatx4 acc[T][4];
+#pragma unroll
+                for (int i = 0; i < T; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+                auto multiply = [&](int slot) {
+#pragma unroll
+                    for (int s = 0; s < 4; s++)
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+#pragma unroll
+                            for (int i = 0; i < T; i++)
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[slot][i][s], b[slot][s][j], acc[i][j], 0, 0, 0);
+                };
+                for (int ks = 0; ks < steps; ks += 2) {
+                    request(1);
+                    multiply(0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    request(0);
+                    multiply(1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                const int o_off = OOFF(f) * 4;
+#pragma unroll
+                for (int i = 0; i < T; i++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        floatx4 v = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+                        if (EPI) {   // the derivative of the leaky ReLU whose output is this layer's input
+                            const floatx4 gt = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, opix[i][r], o_off, 0));
+#pragma unroll
+                            for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
+                        }
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v),
+                                                               o_rsrc, opix[i][r], o_off, 0);
+                    }
+            }
+        }
+    };
+
+    // ---- this wavefront's share: an equal stretch of the line of items (phase, block, tile), each as long as its cost
+    //      (4 per tap of its phase + 1 for its stores), cut between items --------------------------------------------------
+    const long pos_lo = p.total_cost * wave / p.waves, pos_hi = p.total_cost * (wave + 1) / p.waves;
+    long start = 0;   // where phase f begins on the line
+    for (int f = 0; f < p.nph; f++) {
+        const int cost = 4 * TH(f) * TW(f) + 1;
+        const long len = (long)p.items * cost;
+        // items of this phase whose beginning lies in [pos_lo, pos_hi)
+        const long lo = pos_lo > start ? pos_lo - start : 0, hi = pos_hi > start ? min(pos_hi - start, len) : 0;
+        int it = (int)((lo + cost - 1) / cost);
+        const int it_end = (int)((hi + cost - 1) / cost);
+        // runs of one block of produced channels each (item = nb * tiles + tile), every run as groups of 4, 3, 2 and 1
+        // tiles - 4a + 3b for six tiles or more, 3 + 2 for five
+        while (it < it_end) {
+            const int nb = it / p.tiles, tile0 = it - nb * p.tiles;
+            const int cnt = min(it_end - it, p.tiles - tile0);
+            int n4 = 0, n3 = 0, n2 = 0, n1 = 0;
+            if (cnt >= 6) {
+                n3 = (4 - (cnt & 3)) & 3;
+                n4 = (cnt - 3 * n3) >> 2;
+            } else if (cnt == 5) {
+                n3 = 1; n2 = 1;
+            } else if (cnt == 4) {
+                n4 = 1;
+            } else if (cnt == 3) {
+                n3 = 1;
+            } else if (cnt == 2) {
+                n2 = 1;
+            } else {
+                n1 = 1;
+            }
+            run(DcpInt<4>{}, f, nb, tile0, n4);
+            run(DcpInt<3>{}, f, nb, tile0 + 4 * n4, n3);
+            run(DcpInt<2>{}, f, nb, tile0 + 4 * n4 + 3 * n3, n2);
+            run(DcpInt<1>{}, f, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1);
+            it += cnt;
+        }
+        start += len;
+    }
+}
+
+// Up to four phases over the coarse pixels (n, i < OHt, j < OWt); see the formula at the top. TH[f] = 0 marks a phase
+// without taps (written as zeros). `ep`: NULL, or a gate epilogue (nothing else is applied to backward-data). Returns
+// hipErrorNotSupported (nothing launched) when the layer does not fit: more than four phases, AC not a multiple of 32,
+// CO not a multiple of 4, tensors of 2 GB.
+hipError_t launch_direct_conv_phased(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC, int CO,
+                                     int OHt, int OWt, int nph, const int *TH, const int *TW, const int *ph, const int *pw,
+                                     const int *b_off, const int *b_sth, int b_stw, int b_k, long b_elems,
+                                     const int *o_off, int o_sn, int o_sh, int o_sw, long o_elems, const Epilogue *ep)
+{
+    if (nph < 1 || nph > 4 || AC < 32 || (AC & 31) || CO < 4 || (CO & 3) || OHt < 1 || OWt < 1) return hipErrorNotSupported;
+    if (ep && ep->fused && !ep->gate) return hipErrorNotSupported;
+    const long M = (long)N * OHt * OWt;
+    const long a_bytes = (long)N * AH * AW * AC * 4, b_bytes = b_elems * 4, o_bytes = o_elems * 4;
+    if (M < 1 || M >= (1L << 30) || a_bytes >= (1L << 31) || o_bytes >= (1L << 31) || b_bytes >= (1L << 30)) return hipErrorNotSupported;
+    const int cus = device_cu_count();
+    if (cus < 1) return hipErrorNotSupported;
+    DirectPhasedArgs a{};
+    a.A = A; a.B = B; a.O = O;
+    a.M = (int)M; a.AH = AH; a.AW = AW; a.AC = AC; a.CO = CO;
+    a.nph = nph;
+    long cost = 0, taps = 0;
+    for (int f = 0; f < nph; f++) {
+        const bool any = TH[f] > 0 && TW[f] > 0;
+        if (TH[f] < 0 || TW[f] < 0 || TH[f] > 64 || TW[f] > 64) return hipErrorNotSupported;
+        a.f_TH[f] = any ? TH[f] : 0; a.f_TW[f] = any ? TW[f] : 0;
+        a.f_ph[f] = ph[f]; a.f_pw[f] = pw[f];
+        a.f_b_off[f] = any ? b_off[f] : 0; a.f_b_sth[f] = any ? b_sth[f] : 0;
+        a.f_o_off[f] = o_off[f];
+        taps += a.f_TH[f] * a.f_TW[f];
+        cost += 4 * a.f_TH[f] * a.f_TW[f] + 1;
+    }
+    if (taps == 0) return hipErrorNotSupported;
+    a.b_stw = b_stw; a.b_k = b_k;
+    a.o_sn = o_sn; a.o_sh = o_sh; a.o_sw = o_sw;
+    a.a_bytes = (int)a_bytes; a.b_bytes = (int)b_bytes; a.o_bytes = (int)o_bytes;
+    a.tiles = (int)((M + 15) / 16);
+    a.nblocks = (CO + 63) / 64;
+    if ((long)a.tiles * a.nblocks >= (1L << 30) || (long)a.tiles * taps * (AC >> 4) >= (1L << 30)) return hipErrorNotSupported;
+    a.items = a.tiles * a.nblocks;
+    a.total_cost = (long)a.items * cost;
+    a.d_OW = make_fastdiv(OWt);
+    a.d_OHW = make_fastdiv(OHt * OWt);
+    a.ep = ep ? *ep : bias_epilogue(nullptr);
+    int wgs = 2 * cus;   // two wavefronts per SIMD
+    if (wgs * 4 > a.items) wgs = (a.items + 3) / 4;
+    a.waves = wgs * 4;
+    if (a.ep.fused) hipLaunchKernelGGL(direct_conv_phased_kernel<true>, dim3(wgs), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(direct_conv_phased_kernel<false>, dim3(wgs), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace alpha

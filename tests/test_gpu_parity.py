@@ -537,6 +537,13 @@ KS_SHAPES = [
     (4, 13, 11, 32, 64, 5, 4, 3, 2, 2, 1),    # six phases, rectangular filter
     (4, 20, 20, 64, 64, 2, 2, 2, 2, 0, 0),    # one tap per phase, no padding
     (4, 11, 11, 64, 48, 3, 3, 2, 2, 0, 0),    # no padding, odd size
+    # the kernel without LDS: phases of one size (IH % sh == 0, IW % sw == 0), deltaY channels a multiple of 32
+    (16, 56, 56, 64, 128, 3, 3, 2, 2, 1, 1),  # 12544 coarse pixels = 784 tiles: shares of 0 and 1 item
+    (6, 30, 34, 36, 64, 3, 3, 2, 2, 1, 1),    # 1530 coarse pixels (last tile ragged), a ragged block of 36 produced channels
+    (4, 12, 16, 64, 32, 3, 3, 1, 2, 1, 1),    # two phases (stride along the width only)
+    (4, 16, 12, 68, 96, 3, 5, 2, 1, 1, 2),    # two phases (stride along the height only), two blocks of produced channels
+    (4, 14, 14, 64, 64, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2: three phases without taps write zeros
+    (4, 16, 16, 32, 32, 2, 3, 2, 2, 0, 1),    # filter rows = stride: every phase one tap row
 ]
 
 
@@ -570,14 +577,21 @@ def test_deltaX_kernel_split_family(dev, shape):
         else:
             getattr(DX, entry)(*base, sh, sw, ph, pw)
         check(dev.get(dXo), want, "%s %s" % (entry, shape))
-    # the other path (one launch of the generic kernel per phase), and the tiny-IC entry, which reads W in place
+    # the other paths - 1: all phases in one launch of the LDS-halo kernel (stride 2 x 2, even sizes) else as 3; 3: one
+    # launch of the generic kernel per phase; 6: as 0 (the kernel without LDS where the phases have one size) - and the
+    # tiny-IC entry, which reads W in place
     L = pkg.lib()
     try:
-        L.alpha_conv_set_fwd_algo(3)
-        dXo = dev.guarded(N, IH, IW, IC)
-        DX.dconv3D_deltaX_kernelSplit(dev.streams, 1, dy.data_ptr(), OH, OW, CW.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC,
-                                      sh, sw, ph, pw)
-        check(dev.get(dXo), want, "kernelSplit through the generic kernel %s" % (shape,))
+        for algo in (1, 3, 6):
+            L.alpha_conv_set_fwd_algo(algo)
+            dXo = dev.guarded(N, IH, IW, IC)
+            DX.dconv3D_deltaX_kernelSplit(dev.streams, 1, dy.data_ptr(), OH, OW, CW.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC,
+                                          sh, sw, ph, pw)
+            check(dev.get(dXo), want, "kernelSplit algo %d %s" % (algo, shape))
+            dXo = dev.guarded(N, IH, IW, IC)
+            DX.dconv3D_deltaX_crossAdd(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC,
+                                       sh, sw, ph, pw)
+            check(dev.get(dXo), want, "crossAdd (filter in place) algo %d %s" % (algo, shape))
     finally:
         L.alpha_conv_set_fwd_algo(0)
     dXo = dev.guarded(N, IH, IW, IC)
