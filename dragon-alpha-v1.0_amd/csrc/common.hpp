@@ -34,6 +34,18 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
     return (__umulhi(n, f.mul) + n) >> f.shift;
 }
 
+// 128-bit buffer store whose data registers may be reused at once. Measured on gfx950: a `buffer_store_dwordx4 ... offen`
+// with its soffset in a scalar register, followed within two instructions by a vector instruction that writes one of its
+// data registers, now and then stores the NEW value in lanes 12-15 of each group of 16 (one element in a thousand on a
+// 51 MB output, different ones from run to run). The compiler guards this hazard with wait states only for stores
+// WITHOUT a scalar soffset; here the two wait states follow the store explicitly, tied to the data registers so that no
+// write to them can be scheduled in between.
+static __device__ __forceinline__ void buffer_store_b128_guarded(floatx4 v, __amdgpu_buffer_rsrc_t rsrc, unsigned voffset, int soffset)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v), rsrc, voffset, soffset, 0);
+    asm volatile("s_nop 1" : "+v"(v));
+}
+
 // Bumped by alpha_rt_resetDevice: a device reset drops function attributes and symbol addresses, so whatever this
 // library remembers per device is only valid for the generation it was recorded in.
 inline std::atomic<unsigned> &device_generation()

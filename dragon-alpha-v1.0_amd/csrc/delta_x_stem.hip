@@ -203,8 +203,7 @@ __global__ __launch_bounds__(256, 2) void delta_x_stem_kernel(const DxStemArgs p
         deposit();             // next block's halo (requested before the MFMA loop) -> LDS
 #pragma unroll
         for (int j = 0; j < NJ; j++)
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, out[j]),
-                                                   x_rsrc, out_off[j], 0, 0);
+            buffer_store_b128_guarded(out[j], x_rsrc, out_off[j], 0);
         request(blk + 2 * G8);
         __syncthreads();
     }

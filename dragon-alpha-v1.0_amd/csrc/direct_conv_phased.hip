@@ -182,8 +182,7 @@ __global__ __launch_bounds__(256, 2) void direct_conv_phased_kernel(const Direct
 #pragma unroll
                             for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
                         }
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v),
-                                                               o_rsrc, opix[i][r], o_off, 0);
+                        buffer_store_b128_guarded(v, o_rsrc, opix[i][r], o_off);
                     }
             }
         }

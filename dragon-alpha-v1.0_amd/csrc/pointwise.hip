@@ -211,8 +211,7 @@ __global__ __launch_bounds__(512, 1) void pointwise_kernel(const PointwiseArgs p
         auto store = [&](int g) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v[i] + bsel[g]),
-                                                       o_rsrc, o_lane, o_tile + (4 * i * ldn + 64 * g) * 4, 0);
+                buffer_store_b128_guarded(v[i] + bsel[g], o_rsrc, o_lane, o_tile + (4 * i * ldn + 64 * g) * 4);
         };
         b[0] = read_b(0);
         b[1] = read_b(1);

@@ -144,8 +144,7 @@ __global__ __launch_bounds__(256, 2) void pointwise_direct_kernel(const PwDirect
                         } else {
                             v += bias;
                         }
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v),
-                                                               o_rsrc, o_lane, o_off, 0);
+                        buffer_store_b128_guarded(v, o_rsrc, o_lane, o_off);
                     }
             }
         }
