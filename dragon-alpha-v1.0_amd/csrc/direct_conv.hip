@@ -20,9 +20,8 @@
 // per load. Loads run one step ahead of the multiplications through a cursor over (group, tap, channels), so the
 // pipeline does not drain between tiles.
 //
-// Work items are (block of produced channels, tile); a wavefront's share is a contiguous range of them, equal to within
-// one item, processed as groups of 4, 3, 2 or 1 tiles with one loop per group size (every load and store unconditional,
-// every wait an exact count).
+// Work items are (block of produced channels, tile); a wavefront's share is a contiguous range of them, processed as groups
+// of 4, 3, 2 or 1 tiles with one loop per group size (every load and store unconditional, every wait an exact count).
 #include "common.hpp"
 
 namespace alpha {
@@ -37,7 +36,7 @@ struct DirectConvArgs {
     int TH, TW, sh, sw, ph, pw;
     int b_off, b_tap, b_k;
     int a_bytes, b_bytes, o_bytes;
-    int tiles, nblocks, items, waves;
+    int tiles, nblocks, items, waves;   // waves: the SIMDs the items are dealt to (4 per workgroup)
     FastDiv d_OW, d_OHW, d_TW;
     Epilogue ep;
 };
@@ -45,13 +44,20 @@ struct DirectConvArgs {
 template <int V> struct DcInt { static constexpr int value = V; };
 constexpr unsigned DC_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
+// A workgroup has eight wavefronts, two per SIMD (wavefronts w and w + 4 of a workgroup run on SIMD w % 4). The items are
+// dealt to the SIMDs - `slots` = 4 per workgroup - as contiguous shares equal to within one item, and a SIMD's two
+// wavefronts split its share in halves: what must be even is the work per SIMD, not per wavefront (12544 items on 1024
+// SIMDs: 13 = 7 + 6 or 12 = 6 + 6 per SIMD; dealt to 2048 wavefronts they would be 7 + 7 on some SIMDs).
 template <bool EPI>
-__global__ __launch_bounds__(256, 2) void direct_conv_kernel(const DirectConvArgs p)
+__global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArgs p)
 {
     const int t = threadIdx.x, lane = t & 63;
     const int l16 = lane & 15, q = lane >> 4;
-    const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (t >> 6));
-    const int i_lo = (int)((long)p.items * wave / p.waves), i_hi = (int)((long)p.items * (wave + 1) / p.waves);
+    const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int slot = blockIdx.x * 4 + (w & 3);
+    const int s_lo = (int)((long)p.items * slot / p.waves), s_hi = (int)((long)p.items * (slot + 1) / p.waves);
+    const int s_mid = s_lo + (s_hi - s_lo + 1) / 2;
+    const int i_lo = w < 4 ? s_lo : s_mid, i_hi = w < 4 ? s_mid : s_hi;
     const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group: even (host-checked)
 
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
@@ -211,26 +217,23 @@ __global__ __launch_bounds__(256, 2) void direct_conv_kernel(const DirectConvArg
     }
 }
 
-// Share of the wavefronts' time that is work when `items` equal items are dealt to one or two wavefronts per SIMD
-// (whichever is better): the largest share sets the time.
-static double direct_conv_balance(long items, int cus, int *wgs_out)
+// Share of the SIMDs' time that is work when `items` equal items are dealt to them: the largest share sets the time.
+static double direct_conv_balance(long items, int cus)
 {
-    const long w1 = 4L * cus, w2 = 8L * cus;
-    const long s1 = (items + w1 - 1) / w1, s2 = (items + w2 - 1) / w2;
-    const bool one = s1 * w1 < s2 * w2;
-    if (wgs_out) *wgs_out = one ? cus : 2 * cus;
-    return (double)items / (double)(one ? s1 * w1 : s2 * w2);
+    const long slots = 4L * cus, share = (items + slots - 1) / slots;
+    return (double)items / (double)(share * slots);
 }
 
-// Whether the kernel's work items (16 pixels x 64 produced channels) divide evenly enough among the wavefronts for it
-// to beat the LDS-halo kernels on a stride-1 layer. Measured (forward, 3x3): 8x8x256 and 16x16x128 at N = 128 (shares
-// exactly equal) 9-12 % and 5 % faster; 56x56x64, 28x28x128 at N = 64 (seven items where the mean is 6.1) within 2.5 %
-// either way; 14x14x256 (two items where the mean is 1.5) 7 % slower.
+// Whether the kernel's work items (16 pixels x 64 produced channels) divide evenly enough among the SIMDs for it to
+// beat the LDS-halo kernels on a stride-1 layer. Measured (forward, 3x3, against the kernel with the prefetched halo):
+// 8x8x256 and 16x16x128 and 32x32x64 at N = 128 (shares exactly equal) 12 %, 5 % and 6 % faster; 56x56x64 at N = 64 (13
+// items where the mean is 12.25) 3-5 %, 28x28x128 (7 where the mean is 6.1) 4-6 % faster; 7x7x512 (2 where the mean is
+// 1.5) 1-2 % faster, 14x14x256 (4 where the mean is 3.1) 8 % slower.
 bool direct_conv_balanced(long M, int CO)
 {
     const int cus = device_cu_count();
     if (cus < 1 || M < 1) return false;
-    return direct_conv_balance(((M + 15) / 16) * ((CO + 63) / 64), cus, nullptr) >= 0.95;
+    return direct_conv_balance(((M + 15) / 16) * ((CO + 63) / 64), cus) >= 0.87;
 }
 
 // O[N, OHt, OWt, CO] = convolution of A[N, AH, AW, AC] (stride sh x sw, padding ph x pw, TH x TW taps) with the filter B
@@ -263,12 +266,11 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
     a.d_OHW = make_fastdiv(OHt * OWt);
     a.d_TW = make_fastdiv(TW);
     a.ep = ep ? *ep : bias_epilogue(bias);
-    int wgs = 2 * cus;
-    direct_conv_balance(a.items, cus, &wgs);   // one or two wavefronts per SIMD, whichever leaves the shares more even
+    int wgs = cus;   // one workgroup of eight wavefronts per compute unit
     if (wgs * 4 > a.items) wgs = (a.items + 3) / 4;
     a.waves = wgs * 4;
-    if (a.ep.fused) hipLaunchKernelGGL(direct_conv_kernel<true>, dim3(wgs), dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL(direct_conv_kernel<false>, dim3(wgs), dim3(256), 0, stream, a);
+    if (a.ep.fused) hipLaunchKernelGGL(direct_conv_kernel<true>, dim3(wgs), dim3(512), 0, stream, a);
+    else hipLaunchKernelGGL(direct_conv_kernel<false>, dim3(wgs), dim3(512), 0, stream, a);
     return hipGetLastError();
 }
 
