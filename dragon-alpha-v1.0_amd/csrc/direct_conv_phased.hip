@@ -11,9 +11,11 @@
 // tile and four for the filter feed 16 T MFMAs, loads run one step ahead through a cursor over (group, tap, channels),
 // results leave as 128-bit stores. A phase without taps (filter smaller than the stride) writes zeros.
 //
-// Shares: the items in the order (phase, block, tile) form a line of cost - 4 per tap plus 1 for the item's stores -; the
-// wavefronts' shares are equal stretches of it, cut between items. A share then differs from the mean by at most one item - a quarter of the cost of a tile with
-// all its phases - and still consists of runs of tiles of one phase, so that a filter fragment serves up to four tiles.
+// Shares: the items in the order (block, chunk of 32 tiles, phase, tile) form a line of cost - 4 per tap plus 1 for the
+// item's stores -; the wavefronts' shares are equal stretches of it, cut between items. A share then differs from the
+// mean by at most one item - a quarter of the cost of a tile with all its phases - and still consists of runs of tiles
+// of one phase, so that a filter fragment serves up to four tiles; the line is dealt out XCD by XCD, so the phases of a
+// chunk of tiles, which read the same pixels, share an L2 (phase-major order: deltaY fetched 7 times).
 // (Whole tiles with all phases: shares of 3 and 4 on 56x56 -> 28x28, 64 channels - 3136 tiles on 1024 SIMDs; shares cut
 // inside tiles with the cut tiles run alone: the filter is then read per tile, 0.6 GB from L2, and nothing is gained.)
 #include "common.hpp"
@@ -39,6 +41,7 @@ struct DirectPhasedArgs {
 };
 
 template <int V> struct DcpInt { static constexpr int value = V; };
+constexpr int DCP_TB = 32;                    // tiles per chunk of the line of items
 constexpr unsigned DCP_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
 template <bool EPI>
@@ -188,44 +191,58 @@ __global__ __launch_bounds__(256, 2) void direct_conv_phased_kernel(const Direct
         }
     };
 
-    // ---- this wavefront's share: an equal stretch of the line of items (phase, block, tile), each as long as its cost
-    //      (4 per tap of its phase + 1 for its stores), cut between items --------------------------------------------------
-    const long pos_lo = p.total_cost * wave / p.waves, pos_hi = p.total_cost * (wave + 1) / p.waves;
-    long start = 0;   // where phase f begins on the line
-    for (int f = 0; f < p.nph; f++) {
-        const int cost = 4 * TH(f) * TW(f) + 1;
-        const long len = (long)p.items * cost;
-        // items of this phase whose beginning lies in [pos_lo, pos_hi)
-        const long lo = pos_lo > start ? pos_lo - start : 0, hi = pos_hi > start ? min(pos_hi - start, len) : 0;
+    // ---- this wavefront's share: an equal stretch of the line of items, each as long as its cost (4 per tap of its phase
+    //      + 1 for its stores), cut between items. The line runs through (block of produced channels, chunk of DCP_TB
+    //      tiles, phase, tile): the phases of a chunk of tiles - which read the same pixels of deltaY - lie next to each
+    //      other, and the line is dealt to the wavefronts XCD by XCD (workgroups go round-robin to the 8 XCDs, each with
+    //      its own L2), so the second to fourth reader of a pixel finds it in L2 ------------------------------------------
+    const int G = gridDim.x;
+    const int order = (G & 7) == 0 ? ((int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3)) * 4 + (wave & 3) : wave;
+    const long pos_lo = p.total_cost * order / p.waves, pos_hi = p.total_cost * (order + 1) / p.waves;
+    int csum = 0;   // cost of a tile with all its phases
+    for (int f = 0; f < p.nph; f++) csum += 4 * TH(f) * TW(f) + 1;
+    const long per_nb = (long)p.tiles * csum;
+    long pos = pos_lo;
+    while (pos < pos_hi) {
+        // the (block, chunk, phase) segment that holds position pos
+        const int nb = (int)(pos / per_nb);
+        const long r = pos - (long)nb * per_nb;
+        const int chunk = (int)(r / ((long)DCP_TB * csum));
+        const int tile_c = chunk * DCP_TB, tb = min(DCP_TB, p.tiles - tile_c);
+        long seg = (long)nb * per_nb + (long)tile_c * csum;   // where the chunk begins
+        int f = 0, cost = 4 * TH(0) * TW(0) + 1;
+        while (f + 1 < p.nph && pos >= seg + (long)tb * cost) {
+            seg += (long)tb * cost;
+            f++;
+            cost = 4 * TH(f) * TW(f) + 1;
+        }
+        const long seg_end = seg + (long)tb * cost;
+        // items of this segment whose beginning lies in [pos_lo, pos_hi)
+        const long lo = pos_lo > seg ? pos_lo - seg : 0, hi = min(pos_hi, seg_end) - seg;
         int it = (int)((lo + cost - 1) / cost);
         const int it_end = (int)((hi + cost - 1) / cost);
-        // runs of one block of produced channels each (item = nb * tiles + tile), every run as groups of 4, 3, 2 and 1
-        // tiles - 4a + 3b for six tiles or more, 3 + 2 for five
-        while (it < it_end) {
-            const int nb = it / p.tiles, tile0 = it - nb * p.tiles;
-            const int cnt = min(it_end - it, p.tiles - tile0);
-            int n4 = 0, n3 = 0, n2 = 0, n1 = 0;
-            if (cnt >= 6) {
-                n3 = (4 - (cnt & 3)) & 3;
-                n4 = (cnt - 3 * n3) >> 2;
-            } else if (cnt == 5) {
-                n3 = 1; n2 = 1;
-            } else if (cnt == 4) {
-                n4 = 1;
-            } else if (cnt == 3) {
-                n3 = 1;
-            } else if (cnt == 2) {
-                n2 = 1;
-            } else {
-                n1 = 1;
-            }
-            run(DcpInt<4>{}, f, nb, tile0, n4);
-            run(DcpInt<3>{}, f, nb, tile0 + 4 * n4, n3);
-            run(DcpInt<2>{}, f, nb, tile0 + 4 * n4 + 3 * n3, n2);
-            run(DcpInt<1>{}, f, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1);
-            it += cnt;
+        // groups of 4, 3, 2 and 1 tiles - 4a + 3b for six tiles or more, 3 + 2 for five
+        const int cnt = it_end - it, tile0 = tile_c + it;
+        int n4 = 0, n3 = 0, n2 = 0, n1 = 0;
+        if (cnt >= 6) {
+            n3 = (4 - (cnt & 3)) & 3;
+            n4 = (cnt - 3 * n3) >> 2;
+        } else if (cnt == 5) {
+            n3 = 1; n2 = 1;
+        } else if (cnt == 4) {
+            n4 = 1;
+        } else if (cnt == 3) {
+            n3 = 1;
+        } else if (cnt == 2) {
+            n2 = 1;
+        } else if (cnt == 1) {
+            n1 = 1;
         }
-        start += len;
+        run(DcpInt<4>{}, f, nb, tile0, n4);
+        run(DcpInt<3>{}, f, nb, tile0 + 4 * n4, n3);
+        run(DcpInt<2>{}, f, nb, tile0 + 4 * n4 + 3 * n3, n2);
+        run(DcpInt<1>{}, f, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1);
+        pos = seg_end;
     }
 }
 
