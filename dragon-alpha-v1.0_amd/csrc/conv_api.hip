@@ -99,13 +99,15 @@ bool pointwise_direct_preferred(int K, int N)
 }
 
 // Through direct_conv.hip (no LDS): strided layers (the halo kernel's LDS footprint is four input pixels per output pixel
-// there; a strided 1x1 layer 4 % faster than through the filter-resident kernel), stride-1 layers with more than one tap
-// whose work items divide evenly among the SIMDs, and 1x1 layers with many blocks of produced channels (256 -> 1024 on
-// 64x14x14 pixels: 0.059 against 0.068 ms; 64 -> 256 and 256 -> 64 on 32x56x56 pixels: the same as the 1x1 kernels).
-bool direct_conv_preferred(int FH, int FW, int sh, int sw, long M, int CO)
+// there; a strided 1x1 layer 3 % faster than through the filter-resident kernel), layers with more than one tap whose work
+// items divide evenly enough among the compute units (every 3x3 layer of the benchmark configurations: 3-14 % faster than
+// the LDS-halo kernel), and 1x1 layers with a long reduction (256 -> 1024 channels on 64x14x14 pixels: 0.053 against 0.060 ms
+// through the filter-resident kernel; 256 -> 64 on 32x56x56 pixels: 0.030 against 0.032 ms through pointwise_direct.hip;
+// 64 -> 256 there: 0.036 against 0.031 ms through the filter-resident kernel, which keeps that shape).
+bool direct_conv_preferred(int FH, int FW, int sh, int sw, long M, int AC, int CO)
 {
     if (sh > 1 || sw > 1) return true;
-    if (FH * FW <= 1) return CO >= 512 && direct_conv_balanced(M, CO);
+    if (FH * FW <= 1) return AC >= 256 && direct_conv_balanced(M, CO);
     return direct_conv_balanced(M, CO);
 }
 
@@ -133,7 +135,7 @@ int forward(const char *fn, const int64_t *streams, int length,
         hipError_t e = launch_stem_conv(stream0(streams), X, F, layout == FILTER_CW, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, bias, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (layout == FILTER_CW && (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, sh, sw, (long)N * OH * OW, OC)))) {
+    if (layout == FILTER_CW && (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, sh, sw, (long)N * OH * OW, IC, OC)))) {
         // both operands straight from memory
         hipError_t e = launch_direct_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
                                           0, IC * OC, OC, (long)FH * FW * IC * OC, bias, ep);
@@ -190,7 +192,7 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
     if (FH - 1 - ph < 0 || FW - 1 - pw < 0) return fail(ALPHA_CONV_EINVAL, "%s: padding larger than FH-1", fn);
     const int algo = fwd_algo();
 
-    if (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, 1, 1, (long)N * IH * IW, IC))) {
+    if (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, 1, 1, (long)N * IH * IW, OC, IC))) {
         // both operands straight from memory; W rotated by 180 degrees is read in place (input channel contiguous)
         hipError_t e = launch_direct_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, 1, 1, FH - 1 - ph, FW - 1 - pw,
                                           (FH * FW - 1) * IC, -IC, FH * FW * IC, (long)OC * FH * FW * IC, nullptr, ep);

@@ -20,8 +20,10 @@
 // per load. Loads run one step ahead of the multiplications through a cursor over (group, tap, channels), so the
 // pipeline does not drain between tiles.
 //
-// Work items are (block of produced channels, tile); a wavefront's share is a contiguous range of them, processed as groups
-// of 4, 3, 2 or 1 tiles with one loop per group size (every load and store unconditional, every wait an exact count).
+// Work items are (block of produced channels, tile). A workgroup's share is a contiguous range of them: an even number
+// per SIMD is processed whole (a wavefront's part as groups of 4, 3, 2 or 1 tiles with one loop per group size, every
+// load and store unconditional, every wait an exact count), and the up to seven items left over are processed by the
+// whole workgroup together, the reduction (taps x channels) cut into eight parts, the partial sums added through LDS.
 #include "common.hpp"
 
 namespace alpha {
@@ -36,44 +38,53 @@ struct DirectConvArgs {
     int TH, TW, sh, sw, ph, pw;
     int b_off, b_tap, b_k;
     int a_bytes, b_bytes, o_bytes;
-    int tiles, nblocks, items, waves;   // waves: the SIMDs the items are dealt to (4 per workgroup)
+    int tiles, nblocks, items, wgs;
     FastDiv d_OW, d_OHW, d_TW;
     Epilogue ep;
 };
 
 template <int V> struct DcInt { static constexpr int value = V; };
+template <bool V> struct DcBool { static constexpr bool value = V; };
 constexpr unsigned DC_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
-// A workgroup has eight wavefronts, two per SIMD (wavefronts w and w + 4 of a workgroup run on SIMD w % 4). The items are
-// dealt to the SIMDs - `slots` = 4 per workgroup - as contiguous shares equal to within one item, and a SIMD's two
-// wavefronts split its share in halves: what must be even is the work per SIMD, not per wavefront (12544 items on 1024
-// SIMDs: 13 = 7 + 6 or 12 = 6 + 6 per SIMD; dealt to 2048 wavefronts they would be 7 + 7 on some SIMDs).
+constexpr int DC_SPLIT_T = 2;   // tiles per group where the workgroup shares the reduction (LDS: 8 x 4 DC_SPLIT_T x 1 KB)
+
+// A workgroup has eight wavefronts, two per SIMD (wavefronts w and w + 4 of a workgroup run on SIMD w % 4). What must be
+// even is the work per SIMD. A workgroup's n items: f = the largest even number with 4 f <= n go whole to each SIMD, half
+// to each of its two wavefronts (both stay busy to the end: a wavefront alone on a SIMD fills the MFMA pipe less well);
+// the n - 4 f < 8 items left are processed by all eight wavefronts together, wavefront w on part 2 (w % 4) + w / 4 of
+// eight parts of the reduction steps - a SIMD's two parts together are a quarter of the steps -, and the eight partial
+// results are added through LDS in a fixed order. 12544 items on 256 workgroups: 49 = 4 x 12 + 1 per workgroup, 12.25
+// per SIMD, where whole items alone would make it 13 on some SIMDs.
 template <bool EPI>
 __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArgs p)
 {
+    __shared__ floatx4 part[8 * 4 * DC_SPLIT_T * 64];
     const int t = threadIdx.x, lane = t & 63;
     const int l16 = lane & 15, q = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int slot = blockIdx.x * 4 + (w & 3);
-    const int s_lo = (int)((long)p.items * slot / p.waves), s_hi = (int)((long)p.items * (slot + 1) / p.waves);
-    const int s_mid = s_lo + (s_hi - s_lo + 1) / 2;
-    const int i_lo = w < 4 ? s_lo : s_mid, i_hi = w < 4 ? s_mid : s_hi;
+    const int g_lo = (int)((long)p.items * blockIdx.x / p.wgs), g_hi = (int)((long)p.items * (blockIdx.x + 1) / p.wgs);
+    const int f = ((g_hi - g_lo) >> 2) & ~1;
+    const int i_lo = g_lo + (w & 3) * f + (w >> 2) * (f >> 1), i_hi = i_lo + (f >> 1);
     const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group: even (host-checked)
 
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.B), 0, p.b_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.O, 0, p.o_bytes, 0x00020000);
 
-    // `count` groups of T tiles each, from tile0 on, block nb of the produced channels
-    auto run = [&](auto tc, const int nb, const int tile0, const int count) {
+    // `count` groups of T tiles each, from tile0 on, block nb of the produced channels, reduction steps [k_lo, k_lo + k_n)
+    // of every group. SPLIT (count 1, every wavefront of the workgroup calls it with its own steps, k_n >= 0 of either
+    // parity): the wavefronts' partial results are added through LDS. Otherwise k_n is even and at least 2.
+    auto run = [&](auto tc, auto sp, const int nb, const int tile0, const int count, const int k_lo, const int k_n) {
         constexpr int T = decltype(tc)::value;
+        constexpr bool SPLIT = decltype(sp)::value;
         if (count <= 0) return;
         const int n_l = nb * 64 + 4 * l16;
         const unsigned b_lane = n_l < p.CO ? (unsigned)((4 * q * p.b_k + n_l) * 4) : DC_NEVER;
         const unsigned o_lane = n_l < p.CO ? (unsigned)((4 * q * p.CO + n_l) * 4) : DC_NEVER;
         floatx4 a[2][T], b[2][4];
         // ---- load cursor: one step ahead of the multiplications, through (group, tap, 16 channels) ----------------------
-        int c_tile = tile0, c_tap = 0, c_ch = 0, c_left = count * KS;
+        int c_tile = tile0, c_tap = k_lo / CH, c_ch = k_lo - (k_lo / CH) * CH, c_left = count * k_n;
         int org[T];          // byte offset of (this lane's pixel's window origin, channel 4q); may lie before the tensor
         unsigned rc[T];      // bit th: window row th is inside the image; bit 16 + tw: window column tw is
         unsigned voff[T];    // this tap's load offset, or DC_NEVER in the padding
@@ -125,9 +136,11 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                 }
             }
         };
-        locate();
-        aim();
-        request(0);
+        if (!SPLIT || k_n > 0) {
+            locate();
+            aim();
+            request(0);
+        }
         for (int g = 0; g < count; g++) {
             const int tile = tile0 + g * T;
             floatx4 acc[T][4];
@@ -144,7 +157,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                         for (int i = 0; i < T; i++)
                             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[slot][i][s], b[slot][s][j], acc[i][j], 0, 0, 0);
             };
-            for (int ks = 0; ks < KS; ks += 2) {
+            for (int ks = 0; ks + 1 < k_n; ks += 2) {
                 request(1);
                 multiply(0);
                 __builtin_amdgcn_sched_barrier(0);
@@ -152,6 +165,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                 multiply(1);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if (SPLIT && (k_n & 1)) multiply(0);
             // ---- results: lane holds pixels 16(tile + i) + 4q + r, produced channels 64 nb + 4 l16 + j -----------------
             float sub[4], mul[4], add[4];
             floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -164,32 +178,50 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
             } else if (p.ep.bias != nullptr && n_l < p.CO) {
                 bias = *reinterpret_cast<const floatx4 *>(p.ep.bias + n_l);
             }
+            auto emit = [&](const int i, const int r, floatx4 v) {   // pixel 16 (tile + i) + 4 q + r, channels n_l .. n_l + 3
+                const int o_off = __builtin_amdgcn_readfirstlane(((tile + i) * 16 + r) * p.CO * 4);   // rows past M: beyond the descriptor
+                if (EPI) {
+                    if (p.ep.gate) {   // uniform
+                        const floatx4 gt = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                            __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.ep.gate), 0, p.o_bytes, 0x00020000), o_lane, o_off, 0));
 #pragma unroll
-            for (int i = 0; i < T; i++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int o_off = __builtin_amdgcn_readfirstlane(((tile + i) * 16 + r) * p.CO * 4);   // rows past M: beyond the descriptor
-                    floatx4 v = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
-                    if (EPI) {
-                        if (p.ep.gate) {   // uniform
-                            const floatx4 gt = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
-                                __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.ep.gate), 0, p.o_bytes, 0x00020000), o_lane, o_off, 0));
-#pragma unroll
-                            for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
-                        } else {
-#pragma unroll
-                            for (int j = 0; j < 4; j++) v[j] = ep_finish(v[j], sub[j], mul[j], add[j], p.ep.slope);
-                        }
+                        for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
                     } else {
-                        v += bias;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) v[j] = ep_finish(v[j], sub[j], mul[j], add[j], p.ep.slope);
                     }
-                    buffer_store_b128_guarded(v, o_rsrc, o_lane, o_off);
+                } else {
+                    v += bias;
                 }
+                buffer_store_b128_guarded(v, o_rsrc, o_lane, o_off);
+            };
+            if constexpr (!SPLIT) {
+#pragma unroll
+                for (int i = 0; i < T; i++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) emit(i, r, floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]});
+            } else {
+                // unit u = 4 i + r (one 128-bit store per lane); partial results [wavefront][unit][lane]
+                static_assert(T <= DC_SPLIT_T, "LDS holds 4 DC_SPLIT_T units per wavefront");
+#pragma unroll
+                for (int i = 0; i < T; i++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        part[(w * 4 * DC_SPLIT_T + 4 * i + r) * 64 + lane] = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+                __syncthreads();
+                for (int u = w; u < 4 * T; u += 8) {   // uniform
+                    floatx4 v = part[u * 64 + lane];
+#pragma unroll
+                    for (int x = 1; x < 8; x++) v += part[(x * 4 * DC_SPLIT_T + u) * 64 + lane];
+                    emit(u >> 2, u & 3, v);
+                }
+                __syncthreads();   // the next group writes `part` again
+            }
         }
     };
 
-    // the share as runs of tiles of one block of produced channels each (item = nb * tiles + tile), every run as groups
-    // of 4, 3, 2 and 1 tiles: 4a + 3b for six tiles or more, 3 + 2 for five
+    // the wavefront's whole items as runs of tiles of one block of produced channels each (item = nb * tiles + tile),
+    // every run as groups of 4, 3, 2 and 1 tiles: 4a + 3b for six tiles or more, 3 + 2 for five
     int i = i_lo;
     while (i < i_hi) {
         const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
@@ -209,31 +241,46 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         } else {
             n1 = 1;
         }
-        run(DcInt<4>{}, nb, tile0, n4);
-        run(DcInt<3>{}, nb, tile0 + 4 * n4, n3);
-        run(DcInt<2>{}, nb, tile0 + 4 * n4 + 3 * n3, n2);
-        run(DcInt<1>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1);
+        run(DcInt<4>{}, DcBool<false>{}, nb, tile0, n4, 0, KS);
+        run(DcInt<3>{}, DcBool<false>{}, nb, tile0 + 4 * n4, n3, 0, KS);
+        run(DcInt<2>{}, DcBool<false>{}, nb, tile0 + 4 * n4 + 3 * n3, n2, 0, KS);
+        run(DcInt<1>{}, DcBool<false>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1, 0, KS);
+        i += cnt;
+    }
+    // the workgroup's items left over (uniform over the workgroup: every wavefront meets the same barriers)
+    const int part_idx = 2 * (w & 3) + (w >> 2);
+    const int k_lo = KS * part_idx / 8, k_n = KS * (part_idx + 1) / 8 - k_lo;
+    i = g_lo + 4 * f;
+    while (i < g_hi) {
+        const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
+        const int cnt = min(min(g_hi - i, p.tiles - tile0), DC_SPLIT_T);
+        if (cnt == 2) run(DcInt<2>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
+        else run(DcInt<1>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
         i += cnt;
     }
 }
 
-// Share of the SIMDs' time that is work when `items` equal items are dealt to them: the largest share sets the time.
+// Share of the SIMDs' time that is work when `items` equal items are dealt to `cus` workgroups as the kernel does: a
+// workgroup with n items spends f(n) whole items per SIMD and a quarter of each item left over (counted 10 % dearer:
+// the partial sums' way through LDS, shorter loops).
 static double direct_conv_balance(long items, int cus)
 {
-    const long slots = 4L * cus, share = (items + slots - 1) / slots;
-    return (double)items / (double)(share * slots);
+    const long wgs = items < cus ? items : cus;
+    auto cost = [](long n) { const long f = (n >> 2) & ~1L; return (double)f + 1.1 * 0.25 * (double)(n - 4 * f); };
+    const long n_hi = (items + wgs - 1) / wgs, n_lo = items / wgs;
+    const double worst = cost(n_hi) > cost(n_lo) ? cost(n_hi) : cost(n_lo);
+    return (double)items / (4.0 * (double)cus) / worst;
 }
 
-// Whether the kernel's work items (16 pixels x 64 produced channels) divide evenly enough among the SIMDs for it to
-// beat the LDS-halo kernels on a stride-1 layer. Measured (forward, 3x3, against the kernel with the prefetched halo):
-// 8x8x256 and 16x16x128 and 32x32x64 at N = 128 (shares exactly equal) 12 %, 5 % and 6 % faster; 56x56x64 at N = 64 (13
-// items where the mean is 12.25) 3-5 %, 28x28x128 (7 where the mean is 6.1) 4-6 % faster; 7x7x512 (2 where the mean is
-// 1.5) 1-2 % faster, 14x14x256 (4 where the mean is 3.1) 8 % slower.
+// Whether the kernel's work items (16 pixels x 64 produced channels) divide evenly enough among the compute units for it
+// to beat the LDS-halo kernels on a stride-1 layer. Measured (forward, 3x3, N = 64, against the kernel with the prefetched
+// halo): 56x56x64 (49 items per workgroup) 0.111 against 0.115 ms, 28x28x128 (24 or 25) 0.110 against 0.123 ms, 14x14x256
+// (12 or 13: balance 0.91) 0.121 against 0.124 ms, 7x7x512 (6 or 7: 0.80) 0.126 against 0.141 ms.
 bool direct_conv_balanced(long M, int CO)
 {
     const int cus = device_cu_count();
     if (cus < 1 || M < 1) return false;
-    return direct_conv_balance(((M + 15) / 16) * ((CO + 63) / 64), cus) >= 0.87;
+    return direct_conv_balance(((M + 15) / 16) * ((CO + 63) / 64), cus) >= 0.75;
 }
 
 // O[N, OHt, OWt, CO] = convolution of A[N, AH, AW, AC] (stride sh x sw, padding ph x pw, TH x TW taps) with the filter B
@@ -266,9 +313,8 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
     a.d_OHW = make_fastdiv(OHt * OWt);
     a.d_TW = make_fastdiv(TW);
     a.ep = ep ? *ep : bias_epilogue(bias);
-    int wgs = cus;   // one workgroup of eight wavefronts per compute unit
-    if (wgs * 4 > a.items) wgs = (a.items + 3) / 4;
-    a.waves = wgs * 4;
+    const int wgs = cus < a.items ? cus : a.items;   // one workgroup of eight wavefronts per compute unit
+    a.wgs = wgs;
     if (a.ep.fused) hipLaunchKernelGGL(direct_conv_kernel<true>, dim3(wgs), dim3(512), 0, stream, a);
     else hipLaunchKernelGGL(direct_conv_kernel<false>, dim3(wgs), dim3(512), 0, stream, a);
     return hipGetLastError();

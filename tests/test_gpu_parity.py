@@ -426,6 +426,11 @@ DIRECT_CONV_SHAPES = [
     (1, 5, 5, 16, 8, 7, 6, 1, 1, 3, 3),         # window larger than the image, 16 channels (42 steps), 8 produced channels
     (40, 20, 20, 32, 64, 3, 3, 2, 2, 1, 1),     # 4000 pixels = 250 tiles: fewer items than wavefronts
     (64, 30, 34, 48, 64, 3, 3, 2, 2, 1, 1),     # 16320 pixels = 1020 tiles, 48 channels (27 steps are odd: refused -> other kernel)
+    # items left over in a workgroup are shared by its eight wavefronts (reduction cut in eight, partial sums through LDS):
+    (8, 24, 24, 32, 192, 3, 3, 1, 1, 1, 1),     # 864 items on 256 workgroups: 3 or 4 each, all shared, 18 steps in parts of 2 and 3; a pair meets the end of a block
+    (4, 10, 10, 32, 64, 1, 1, 1, 1, 0, 0),      # 2 steps: six of the eight wavefronts have none
+    (32, 40, 40, 32, 64, 3, 3, 1, 1, 1, 1),     # 3200 items: 12 or 13 per workgroup = 2 whole per SIMD + 4 or 5 shared
+    (2, 56, 56, 64, 64, 3, 3, 1, 1, 1, 1),      # 392 items: 1 or 2 per workgroup, 36 steps in parts of 4 and 5
 ]
 
 
