@@ -47,24 +47,35 @@ template <int V> struct DcInt { static constexpr int value = V; };
 template <bool V> struct DcBool { static constexpr bool value = V; };
 constexpr unsigned DC_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
-constexpr int DC_SPLIT_T = 2;   // tiles per group where the workgroup shares the reduction (LDS: 8 x 4 DC_SPLIT_T x 1 KB)
+constexpr int DC_SPLIT_T = 4;   // tiles per group where the workgroup shares the reduction (LDS: 8 x 4 DC_SPLIT_T x 1 KB)
+constexpr size_t DC_LDS_BYTES = 8 * 4 * DC_SPLIT_T * 64 * sizeof(floatx4);
 
 // A workgroup has eight wavefronts, two per SIMD (wavefronts w and w + 4 of a workgroup run on SIMD w % 4). What must be
 // even is the work per SIMD. A workgroup's n items: f = the largest even number with 4 f <= n go whole to each SIMD, half
-// to each of its two wavefronts (both stay busy to the end: a wavefront alone on a SIMD fills the MFMA pipe less well);
-// the n - 4 f < 8 items left are processed by all eight wavefronts together, wavefront w on part 2 (w % 4) + w / 4 of
+// to each of its two wavefronts (both stay busy to the end: a wavefront alone on a SIMD fills the MFMA pipe less well),
+// but none where that would be a single item per wavefront (groups of one tile: five loads per 16 MFMAs, where a group of
+// four tiles has eight per 64); the items left - fewer than 8, or all n < 16 - are processed by all eight wavefronts together
+// in groups of up to four tiles, wavefront w on part 2 (w % 4) + w / 4 of
 // eight parts of the reduction steps - a SIMD's two parts together are a quarter of the steps -, and the eight partial
 // results are added through LDS in a fixed order. 12544 items on 256 workgroups: 49 = 4 x 12 + 1 per workgroup, 12.25
 // per SIMD, where whole items alone would make it 13 on some SIMDs.
+// whole items per SIMD of a workgroup with n items
+__host__ __device__ inline int dc_whole_items(int n)
+{
+    const int f = (n >> 2) & ~1;
+    return f < 4 ? 0 : f;
+}
+
 template <bool EPI>
 __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArgs p)
 {
-    __shared__ floatx4 part[8 * 4 * DC_SPLIT_T * 64];
+    extern __shared__ __attribute__((aligned(16))) float dc_smem[];
+    floatx4 *part = reinterpret_cast<floatx4 *>(dc_smem);   // [8 wavefronts][4 DC_SPLIT_T units][64 lanes]
     const int t = threadIdx.x, lane = t & 63;
     const int l16 = lane & 15, q = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int g_lo = (int)((long)p.items * blockIdx.x / p.wgs), g_hi = (int)((long)p.items * (blockIdx.x + 1) / p.wgs);
-    const int f = ((g_hi - g_lo) >> 2) & ~1;
+    const int f = dc_whole_items(g_hi - g_lo);
     const int i_lo = g_lo + (w & 3) * f + (w >> 2) * (f >> 1), i_hi = i_lo + (f >> 1);
     const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group: even (host-checked)
 
@@ -254,7 +265,9 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     while (i < g_hi) {
         const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
         const int cnt = min(min(g_hi - i, p.tiles - tile0), DC_SPLIT_T);
-        if (cnt == 2) run(DcInt<2>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
+        if (cnt == 4) run(DcInt<4>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
+        else if (cnt == 3) run(DcInt<3>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
+        else if (cnt == 2) run(DcInt<2>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
         else run(DcInt<1>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
         i += cnt;
     }
@@ -266,7 +279,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
 static double direct_conv_balance(long items, int cus)
 {
     const long wgs = items < cus ? items : cus;
-    auto cost = [](long n) { const long f = (n >> 2) & ~1L; return (double)f + 1.1 * 0.25 * (double)(n - 4 * f); };
+    auto cost = [](long n) { const long f = dc_whole_items((int)(n < (1 << 30) ? n : (1 << 30))); return (double)f + 1.1 * 0.25 * (double)(n - 4 * f); };
     const long n_hi = (items + wgs - 1) / wgs, n_lo = items / wgs;
     const double worst = cost(n_hi) > cost(n_lo) ? cost(n_hi) : cost(n_lo);
     return (double)items / (4.0 * (double)cus) / worst;
@@ -315,8 +328,13 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
     a.ep = ep ? *ep : bias_epilogue(bias);
     const int wgs = cus < a.items ? cus : a.items;   // one workgroup of eight wavefronts per compute unit
     a.wgs = wgs;
-    if (a.ep.fused) hipLaunchKernelGGL(direct_conv_kernel<true>, dim3(wgs), dim3(512), 0, stream, a);
-    else hipLaunchKernelGGL(direct_conv_kernel<false>, dim3(wgs), dim3(512), 0, stream, a);
+    if (a.ep.fused) {
+        if (hipError_t e = ensure_dynamic_lds<direct_conv_kernel<true>>(DC_LDS_BYTES); e != hipSuccess) return e;
+        hipLaunchKernelGGL(direct_conv_kernel<true>, dim3(wgs), dim3(512), DC_LDS_BYTES, stream, a);
+    } else {
+        if (hipError_t e = ensure_dynamic_lds<direct_conv_kernel<false>>(DC_LDS_BYTES); e != hipSuccess) return e;
+        hipLaunchKernelGGL(direct_conv_kernel<false>, dim3(wgs), dim3(512), DC_LDS_BYTES, stream, a);
+    }
     return hipGetLastError();
 }
 

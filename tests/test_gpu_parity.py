@@ -429,7 +429,8 @@ DIRECT_CONV_SHAPES = [
     # items left over in a workgroup are shared by its eight wavefronts (reduction cut in eight, partial sums through LDS):
     (8, 24, 24, 32, 192, 3, 3, 1, 1, 1, 1),     # 864 items on 256 workgroups: 3 or 4 each, all shared, 18 steps in parts of 2 and 3; a pair meets the end of a block
     (4, 10, 10, 32, 64, 1, 1, 1, 1, 0, 0),      # 2 steps: six of the eight wavefronts have none
-    (32, 40, 40, 32, 64, 3, 3, 1, 1, 1, 1),     # 3200 items: 12 or 13 per workgroup = 2 whole per SIMD + 4 or 5 shared
+    (32, 40, 40, 32, 64, 3, 3, 1, 1, 1, 1),     # 3200 items: 12 or 13 per workgroup, all shared in groups of 4, 4, 4 (, 1)
+    (44, 40, 40, 32, 64, 3, 3, 1, 1, 1, 1),     # 4400 items: 17 or 18 per workgroup = 4 whole per SIMD + 1 or 2 shared
     (2, 56, 56, 64, 64, 3, 3, 1, 1, 1, 1),      # 392 items: 1 or 2 per workgroup, 36 steps in parts of 4 and 5
 ]
 
