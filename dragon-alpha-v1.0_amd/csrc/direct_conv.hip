@@ -93,6 +93,19 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         const int n_l = nb * 64 + 4 * l16;
         const unsigned b_lane = n_l < p.CO ? (unsigned)((4 * q * p.b_k + n_l) * 4) : DC_NEVER;
         const unsigned o_lane = n_l < p.CO ? (unsigned)((4 * q * p.CO + n_l) * 4) : DC_NEVER;
+        // the epilogue's per-channel terms: once per run, so that the loop below carries twelve registers, not the
+        // epilogue's pointers
+        float sub[4], mul[4], add[4];
+        floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (EPI) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                sub[j] = 0.f; mul[j] = 1.f; add[j] = 0.f;
+                if (n_l < p.CO && !p.ep.gate) ep_channel(p.ep, n_l + j, sub[j], mul[j], add[j]);
+            }
+        } else if (p.ep.bias != nullptr && n_l < p.CO) {
+            bias = *reinterpret_cast<const floatx4 *>(p.ep.bias + n_l);
+        }
         floatx4 a[2][T], b[2][4];
         // ---- load cursor: one step ahead of the multiplications, through (group, tap, 16 channels) ----------------------
         int c_tile = tile0, c_tap = k_lo / CH, c_ch = k_lo - (k_lo / CH) * CH, c_left = count * k_n;
@@ -178,17 +191,6 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
             }
             if (SPLIT && (k_n & 1)) multiply(0);
             // ---- results: lane holds pixels 16(tile + i) + 4q + r, produced channels 64 nb + 4 l16 + j -----------------
-            float sub[4], mul[4], add[4];
-            floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
-            if (EPI) {
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    sub[j] = 0.f; mul[j] = 1.f; add[j] = 0.f;
-                    if (n_l < p.CO && !p.ep.gate) ep_channel(p.ep, n_l + j, sub[j], mul[j], add[j]);
-                }
-            } else if (p.ep.bias != nullptr && n_l < p.CO) {
-                bias = *reinterpret_cast<const floatx4 *>(p.ep.bias + n_l);
-            }
             auto emit = [&](const int i, const int r, floatx4 v) {   // pixel 16 (tile + i) + 4 q + r, channels n_l .. n_l + 3
                 const int o_off = __builtin_amdgcn_readfirstlane(((tile + i) * 16 + r) * p.CO * 4);   // rows past M: beyond the descriptor
                 if (EPI) {
