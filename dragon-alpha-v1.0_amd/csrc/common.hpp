@@ -277,6 +277,11 @@ hipError_t launch_stem_conv(hipStream_t stream, const float *X, const float *F, 
                             int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw,
                             const float *bias = nullptr, const Epilogue *ep = nullptr);
 
+// The same layers with both operands straight from memory (stem_direct.hip): W[OC,FH,FW,4] in place. Returns
+// hipErrorNotSupported (nothing launched) for filters other than 3x3 and 7x7.
+hipError_t launch_stem_direct(hipStream_t stream, const float *X, const float *W, float *Y, int N, int IH, int IW, int OH, int OW,
+                              int OC, int FH, int FW, int sh, int sw, int ph, int pw, const float *bias, const Epilogue *ep);
+
 // Backward-filter of 1x1 stride-1 layers from registers (delta_w_pointwise.hip); same slice partition and outputs.
 // Returns hipErrorNotSupported (nothing launched) unless IC and OC are multiples of 64.
 hipError_t launch_deltaW_pointwise(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,

@@ -122,8 +122,11 @@ int epilogue_pass(const char *fn, hipStream_t s, float *Y, const Epilogue &ep, l
 int forward(const char *fn, const int64_t *streams, int length,
             const float *X, int IH, int IW, const float *F, FilterLayout layout, int FH, int FW,
             float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
-            const float *bias = nullptr, const Epilogue *ep = nullptr)
+            const float *bias = nullptr, const Epilogue *ep = nullptr, const float *W_too = nullptr)
 {
+    // W_too: the entries that take CW also receive W[OC,FH,FW,IC], the filter CW was made from (the reference's
+    // conv3D_GemmR hands both on, conv/A.cu:165-170); the kernel for 4 stored channels reads its 16-byte taps in place
+    const float *W_inplace = layout == FILTER_W ? F : (aligned16(W_too) ? W_too : nullptr);
     if (streams == nullptr || length < 1) return fail(ALPHA_CONV_EINVAL, "%s: empty stream array", fn);
     if (!X || !F || !Y || !aligned16(X) || !aligned16(F) || !aligned16(Y) || !aligned16(bias))
         return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
@@ -131,6 +134,11 @@ int forward(const char *fn, const int64_t *streams, int length,
     if (ep && !ep->fused) { bias = ep->bias; ep = nullptr; }
     const int algo = fwd_algo();
 
+    if (IC == 4 && W_inplace && (algo == 0 || algo == 6)) {
+        // both operands straight from memory
+        hipError_t e = launch_stem_direct(stream0(streams), X, W_inplace, Y, N, IH, IW, OH, OW, OC, FH, FW, sh, sw, ph, pw, bias, ep);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     if (IC == 4 && algo != 3) {
         hipError_t e = launch_stem_conv(stream0(streams), X, F, layout == FILTER_CW, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, bias, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
@@ -480,28 +488,24 @@ int alpha_kernel_remode(int64_t stream, const float *W, float *CW, int FH, int F
 int alpha_conv3D_GemmR(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, const float *CW,
                        int FH, int FW, float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
 {
-    (void)W;
-    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, nullptr, nullptr, W);
 }
 int alpha_conv3D_GemmR_texture(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, const float *CW,
                                int FH, int FW, float *Y, int OH, int OW, int N, int IC, int OC, int sh, int sw, int ph, int pw)
 {
-    (void)W;
-    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, nullptr, nullptr, W);
 }
 int alpha_conv3D_GemmV2R(int useTexture, const int64_t *streams, int length, const float *X, int IH, int IW, const float *W,
                          const float *CW, int FH, int FW, float *Y, int OH, int OW, int N, int IC, int OC,
                          int sh, int sw, int ph, int pw)
 {
     (void)useTexture;
-    (void)W;
-    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw);
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, nullptr, nullptr, W);
 }
 int alpha_conv3D_GemmR_W1(const int64_t *streams, int length, const float *X, int IH, int IW, const float *W, const float *CW,
                           float *Y, int N, int IC, int OC)
 {
-    (void)W;
-    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, 1, 1, Y, IH, IW, N, IC, OC, 1, 1, 0, 0);
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, 1, 1, Y, IH, IW, N, IC, OC, 1, 1, 0, 0, nullptr, nullptr, W);
 }
 
 // ---- backward-data ---------------------------------------------------------------------------
@@ -731,9 +735,8 @@ int alpha_conv3D_GemmR_biased(const int64_t *streams, int length, const float *X
                               int FH, int FW, const float *Bias, float *Y, int OH, int OW, int N, int IC, int OC,
                               int sh, int sw, int ph, int pw)
 {
-    (void)W;
     CHECK_PTR(Bias);
-    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, Bias);
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, Bias, nullptr, W);
 }
 int alpha_conv3D_winograd_biased(const int64_t *streams, int length, const float *X, int IH, int IW, const float *U,
                                  const float *Bias, float *Y, int OH, int OW, int N, int IC, int OC, int ph, int pw)
@@ -787,10 +790,9 @@ int alpha_conv3D_GemmR_fused(const int64_t *streams, int length, const float *X,
                              int FH, int FW, const alpha_conv_epilogue *epilogue, float *Y, int OH, int OW, int N, int IC, int OC,
                              int sh, int sw, int ph, int pw)
 {
-    (void)W;
     Epilogue ep;
     if (int e = make_epilogue(__func__, epilogue, &ep)) return e;
-    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, nullptr, &ep);
+    return forward(__func__, streams, length, X, IH, IW, CW, FILTER_CW, FH, FW, Y, OH, OW, N, IC, OC, sh, sw, ph, pw, nullptr, &ep, W);
 }
 int alpha_conv3D_winograd_fused(const int64_t *streams, int length, const float *X, int IH, int IW, const float *U,
                                 const alpha_conv_epilogue *epilogue, float *Y, int OH, int OW, int N, int IC, int OC, int ph, int pw)

@@ -1,0 +1,279 @@
+// Forward convolution of layers with 4 stored input channels - network stems such as 7x7 stride 2 on RGB - with both
+// operands straight from memory: no LDS, no barrier in the main loop, fp32 MFMA v_mfma_f32_16x16x4_f32, gfx950.
+//
+//   Y[m, oc] = sum over taps (fh, fw) and channels c < 4 of X[n, oh*sh - ph + fh, ow*sw - pw + fw, c] * W[oc, fh, fw, c]
+//
+// The reduction index of one MFMA is FOUR TAPS of one channel (stem_conv.hip's scheme): lane (l16, q) loads the float4 -
+// all four channels - of the input pixel that tap 4g + q touches for output pixel l16 of a tile, and the float4 of filter
+// tap 4g + q for output channel 4*l16 + j, j = 0..3; component s (the channel) of both feeds MFMA (s, j). A step is one
+// group g of four taps: one 128-bit load per tile and four for the filter, shared by the T <= 4 tiles a wavefront
+// owns, feed 16 T MFMAs (12 T when the fourth stored channel has zero weights everywhere: layers with three logical
+// channels). A lane's accumulators are 4 consecutive output channels of a pixel: results leave as 128-bit stores.
+// The filter is read as W[OC, FH, FW, 4] in place - its 4-channel taps are exactly the 16-byte units the lanes need - and
+// stays in L1 / L2 (64 channels of a 7x7 filter: 50 KB).
+//
+// Where a tile's pixels are is worked out per lane once per group of tiles (window origin, masks of the window rows and
+// columns inside the image); a lane's tap offsets and the mask bits its taps need are registers computed once (the
+// step loop is unrolled over the tap groups, so they are indexed statically). Per step and tile: and, compare, add,
+// select. Loads run one step ahead through a cursor over (group of tiles, tap group); with an odd number of steps per
+// group of tiles the two register sets swap roles from one group to the next (template parameter P).
+//
+// Against stem_conv.hip (window staged in LDS per block of 16 x 16 output pixels, results through an LDS patch): no
+// staging phase, no barriers, no output transpose; the window's re-reads go to L1 / L2 instead.
+#include "common.hpp"
+#include <type_traits>
+
+namespace alpha {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx3 __attribute__((ext_vector_type(3)));
+
+struct StemDirectArgs {
+    const float *X;   // [N, IH, IW, 4]
+    const float *W;   // [OC, FH, FW, 4]
+    float *Y;         // [M, OC] dense
+    int M, IH, IW, OC;
+    int FH, FW, taps, sh, sw, ph, pw;
+    int x_bytes, w_bytes, y_bytes;
+    int tiles, nblocks, items, slots;   // slots: the SIMDs the items are dealt to (4 per workgroup)
+    FastDiv d_OW, d_OHW, d_FW;
+    Epilogue ep;
+};
+
+template <int V> struct SdInt { static constexpr int value = V; };
+constexpr unsigned SD_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
+
+// Bits f < F (F <= 15) with 0 <= x0 + f < L: the window positions inside the image along one axis.
+__device__ inline unsigned sd_range_mask(int x0, int F, int L)
+{
+    const int lo = max(0, -x0), hi = min(F, L - x0);
+    return hi > lo ? ((1u << hi) - 1u) & ~((1u << lo) - 1u) : 0u;
+}
+
+// G: tap groups (ceil(taps / 4)). Eight wavefronts per workgroup, two per SIMD; the items (block of 64 output channels,
+// tile of 16 pixels) are dealt to the SIMDs as contiguous shares equal to within one, a SIMD's two wavefronts take half
+// a share each.
+template <int G, bool EPI>
+__global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArgs p)
+{
+    __shared__ int any_ch3;
+    const int t = threadIdx.x, lane = t & 63;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int slot = blockIdx.x * 4 + (w & 3);
+    const int s_lo = (int)((long)p.items * slot / p.slots), s_hi = (int)((long)p.items * (slot + 1) / p.slots);
+    const int s_mid = s_lo + (s_hi - s_lo + 1) / 2;
+    const int i_lo = w < 4 ? s_lo : s_mid, i_hi = w < 4 ? s_mid : s_hi;
+
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.W), 0, p.w_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.Y, 0, p.y_bytes, 0x00020000);
+
+    // ---- does any weight of the fourth stored channel differ from zero? (layers with three logical channels arrive with
+    // it zero-filled in X and W: its MFMA step, a quarter of all, is then left out) ---------------------------------------
+    if (t == 0) any_ch3 = 0;
+    __syncthreads();
+    {
+        int nz = 0;
+        const int n_taps_all = p.OC * p.taps;
+        for (int idx = t; idx < n_taps_all; idx += 512) nz |= p.W[(size_t)idx * 4 + 3] != 0.f;
+        if (nz) any_ch3 = 1;   // every writer writes the same value
+    }
+    __syncthreads();
+    const bool use_ch3 = any_ch3 != 0;
+
+    // ---- per-lane tap data: byte offset of tap 4g + q from a window's origin, and the window row / column it needs --------
+    int toff[G];
+    unsigned need[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const int tap = 4 * g + q;
+        const int fh = fdiv(tap, p.d_FW), fw = tap - fh * p.FW;
+        toff[g] = (fh * p.IW + fw) * 16;
+        need[g] = tap < p.taps ? (1u << fh) | (1u << (16 + fw)) : 0x80000000u;   // taps past the last: never inside
+    }
+
+    auto run = [&](auto tc, auto scc, const int nb, const int tile0, const int count) {
+        constexpr int T = decltype(tc)::value;
+        constexpr int SC = decltype(scc)::value;
+        if (count <= 0) return;
+        const int n_l = nb * 64 + 4 * l16;
+        const bool n_ok = n_l < p.OC;   // OC % 4 == 0: a lane's four channels are valid together
+        unsigned b_voff[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) b_voff[j] = n_ok ? (unsigned)(((n_l + j) * p.taps + q) * 16) : SD_NEVER;
+        const bool last_tap_ok = 4 * (G - 1) + q < p.taps;
+        const unsigned o_lane = n_ok ? (unsigned)((4 * q * p.OC + n_l) * 4) : SD_NEVER;
+        float sub[4], mul[4], add[4];
+        floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (EPI) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                sub[j] = 0.f; mul[j] = 1.f; add[j] = 0.f;
+                if (n_ok && !p.ep.gate) ep_channel(p.ep, n_l + j, sub[j], mul[j], add[j]);
+            }
+        } else if (p.ep.bias != nullptr && n_ok) {
+            bias = *reinterpret_cast<const floatx4 *>(p.ep.bias + n_l);
+        }
+
+        // three channels: 96-bit loads, so that the unused fourth component takes no registers
+        using frag = std::conditional_t<SC == 3, floatx3, floatx4>;
+        frag a[2][T], b[2][4];
+        // ---- load cursor: one step ahead of the multiplications ------------------------------------------------------------
+        int c_tile = tile0, c_groups_left = count;
+        int org[T];       // byte offset of this lane's pixel's window origin; may lie before the tensor
+        unsigned rc[T];   // bit fh: window row fh is inside the image; bit 16 + fw: window column fw is
+        auto locate = [&]() {
+#pragma unroll
+            for (int i = 0; i < T; i++) {
+                const int m = (c_tile + i) * 16 + l16;
+                const bool live = m < p.M;
+                const int mm = live ? m : 0;
+                const int n = fdiv(mm, p.d_OHW), rem = mm - n * (int)p.d_OHW.d;
+                const int oh = fdiv(rem, p.d_OW), ow = rem - oh * (int)p.d_OW.d;
+                const int ih0 = oh * p.sh - p.ph, iw0 = ow * p.sw - p.pw;
+                org[i] = ((n * p.IH + ih0) * p.IW + iw0) * 16;
+                rc[i] = (live ? sd_range_mask(ih0, p.FH, p.IH) : 0u) | (sd_range_mask(iw0, p.FW, p.IW) << 16);
+            }
+        };
+        auto request = [&](int slot, auto gc) {   // the loads of tap group g of the cursor's tiles
+            constexpr int g = decltype(gc)::value;
+#pragma unroll
+            for (int i = 0; i < T; i++) {
+                const unsigned voff = (rc[i] & need[g]) == need[g] ? (unsigned)(org[i] + toff[g]) : SD_NEVER;
+                if constexpr (SC == 3) a[slot][i] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(x_rsrc, voff, 0, 0));
+                else a[slot][i] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, voff, 0, 0));
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const unsigned voff = (g == G - 1 && !last_tap_ok) ? SD_NEVER : b_voff[j];
+                if constexpr (SC == 3) b[slot][j] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(w_rsrc, voff, g * 64, 0));
+                else b[slot][j] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, voff, g * 64, 0));
+            }
+        };
+        floatx4 acc[T][4];
+        auto multiply = [&](int slot) {
+#pragma unroll
+            for (int s = 0; s < SC; s++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int i = 0; i < T; i++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[slot][i][s], b[slot][j][s], acc[i][j], 0, 0, 0);
+        };
+        // one group of tiles; P: the register set that holds its first step
+        auto group = [&](auto pc, const int tile) {
+            constexpr int P = decltype(pc)::value;
+#pragma unroll
+            for (int i = 0; i < T; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+            auto step = [&](auto kc, auto self) {
+                constexpr int k = decltype(kc)::value;
+                if constexpr (k < G) {
+                    if constexpr (k + 1 < G) {
+                        request((P + k + 1) & 1, SdInt<k + 1>{});
+                    } else {
+                        // the first step of the next group of tiles (past the last group: this group's again, unused)
+                        if (c_groups_left > 1) {
+                            c_groups_left--;
+                            c_tile += T;
+                            locate();
+                        }
+                        request((P + k + 1) & 1, SdInt<0>{});
+                    }
+                    multiply((P + k) & 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    self(SdInt<k + 1>{}, self);
+                }
+            };
+            step(SdInt<0>{}, step);
+            // ---- results: lane holds pixels 16 (tile + i) + 4q + r, output channels 64 nb + 4 l16 + j ------------------------
+#pragma unroll
+            for (int i = 0; i < T; i++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int o_off = __builtin_amdgcn_readfirstlane(((tile + i) * 16 + r) * p.OC * 4);   // rows past M: beyond the descriptor
+                    floatx4 v = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+                    if (EPI) {
+                        if (p.ep.gate) {   // uniform
+                            const floatx4 gt = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                                __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.ep.gate), 0, p.y_bytes, 0x00020000), o_lane, o_off, 0));
+#pragma unroll
+                            for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) v[j] = ep_finish(v[j], sub[j], mul[j], add[j], p.ep.slope);
+                        }
+                    } else if (p.ep.bias != nullptr) {   // uniform
+                        v += bias;
+                    }
+                    buffer_store_b128_guarded(v, y_rsrc, o_lane, o_off);
+                }
+        };
+        locate();
+        request(0, SdInt<0>{});
+        for (int g2 = 0; g2 < count; g2++) {
+            const int tile = tile0 + g2 * T;
+            if ((G & 1) && (g2 & 1)) group(SdInt<1>{}, tile);
+            else group(SdInt<0>{}, tile);
+        }
+    };
+
+    // the share as runs of tiles of one block of output channels each (item = nb * tiles + tile): groups of four tiles,
+    // then single tiles
+    int i = i_lo;
+    while (i < i_hi) {
+        const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
+        const int cnt = min(i_hi - i, p.tiles - tile0);
+        const int n4 = cnt >> 2, n1 = cnt & 3;
+        if (use_ch3) {
+            run(SdInt<4>{}, SdInt<4>{}, nb, tile0, n4);
+            run(SdInt<1>{}, SdInt<4>{}, nb, tile0 + 4 * n4, n1);
+        } else {
+            run(SdInt<4>{}, SdInt<3>{}, nb, tile0, n4);
+            run(SdInt<1>{}, SdInt<3>{}, nb, tile0 + 4 * n4, n1);
+        }
+        i += cnt;
+    }
+}
+
+// Y[N, OH, OW, OC] = convolution of X[N, IH, IW, 4] with W[OC, FH, FW, 4] (stride sh x sw, padding ph x pw). Returns
+// hipErrorNotSupported (nothing launched) when the layer does not fit: a filter other than 3x3 or 7x7, tensors of 2 GB.
+hipError_t launch_stem_direct(hipStream_t stream, const float *X, const float *W, float *Y, int N, int IH, int IW, int OH, int OW,
+                              int OC, int FH, int FW, int sh, int sw, int ph, int pw, const float *bias, const Epilogue *ep)
+{
+    const int taps = FH * FW, G = (taps + 3) / 4;
+    if ((G != 13 && G != 3) || FH > 15 || FW > 15 || OC < 4 || (OC & 3)) return hipErrorNotSupported;
+    const long M = (long)N * OH * OW;
+    const long x_bytes = (long)N * IH * IW * 16, w_bytes = (long)OC * taps * 16, y_bytes = M * OC * 4;
+    if (M < 1 || x_bytes >= (1L << 31) || y_bytes >= (1L << 31) || w_bytes >= (1L << 30)) return hipErrorNotSupported;
+    const int cus = device_cu_count();
+    if (cus < 1) return hipErrorNotSupported;
+    StemDirectArgs a{};
+    a.X = X; a.W = W; a.Y = Y;
+    a.M = (int)M; a.IH = IH; a.IW = IW; a.OC = OC;
+    a.FH = FH; a.FW = FW; a.taps = taps; a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw;
+    a.x_bytes = (int)x_bytes; a.w_bytes = (int)w_bytes; a.y_bytes = (int)y_bytes;
+    a.tiles = (int)((M + 15) / 16);
+    a.nblocks = (OC + 63) / 64;
+    if ((long)a.tiles * a.nblocks >= (1L << 30)) return hipErrorNotSupported;
+    a.items = a.tiles * a.nblocks;
+    a.d_OW = make_fastdiv(OW);
+    a.d_OHW = make_fastdiv(OH * OW);
+    a.d_FW = make_fastdiv(FW);
+    a.ep = ep ? *ep : bias_epilogue(bias);
+    int wgs = cus;   // one workgroup of eight wavefronts per compute unit
+    if (wgs * 8 > a.items) wgs = (a.items + 7) / 8;
+    a.slots = wgs * 4;
+    if (G == 13) {
+        if (a.ep.fused) hipLaunchKernelGGL((stem_direct_kernel<13, true>), dim3(wgs), dim3(512), 0, stream, a);
+        else hipLaunchKernelGGL((stem_direct_kernel<13, false>), dim3(wgs), dim3(512), 0, stream, a);
+    } else {
+        if (a.ep.fused) hipLaunchKernelGGL((stem_direct_kernel<3, true>), dim3(wgs), dim3(512), 0, stream, a);
+        else hipLaunchKernelGGL((stem_direct_kernel<3, false>), dim3(wgs), dim3(512), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace alpha

@@ -452,6 +452,43 @@ def test_forward_direct_conv_kernel(dev, shape):
         L.alpha_conv_set_fwd_algo(0)
 
 
+STEM_FWD_SHAPES = [
+    # N, IH, IW, OC, F, s, p: 4 stored input channels, 7x7 or 3x3 -> the stem kernels (without LDS, with LDS), forward
+    (4, 30, 30, 64, 7, 2, 3),       # 900 pixels: ragged last tile, tiles straddle rows and images
+    (16, 64, 64, 64, 7, 2, 3),      # 16384 pixels = 1024 tiles: shares of one tile, single-tile groups only
+    (64, 64, 64, 64, 7, 2, 3),      # 4096 tiles: 4 per SIMD = 2 per wavefront
+    (40, 96, 96, 64, 7, 2, 3),      # 92160 pixels = 5760 tiles: 5 or 6 per SIMD, groups of four tiles
+    (150, 96, 96, 64, 7, 2, 3),     # 21600 tiles: 21 or 22 per SIMD, two or three groups of four in a row (the register sets swap)
+    (8, 33, 29, 36, 7, 1, 3),       # stride 1, 36 output channels (a ragged block)
+    (8, 21, 23, 136, 7, 2, 0),      # no padding, three blocks of output channels (the last with 8)
+    (4, 32, 32, 64, 3, 1, 1),       # c1 geometry: 3x3 = three tap groups (taps 9..11 are padding)
+    (32, 17, 19, 20, 3, 2, 1),      # 3x3 stride 2, 20 output channels
+    (3, 9, 9, 64, 5, 1, 2),         # 5x5: not taken by the kernel without LDS -> the LDS one
+]
+
+
+@pytest.mark.parametrize("shape", STEM_FWD_SHAPES)
+@pytest.mark.parametrize("rgb", [True, False])
+def test_forward_stem_kernels(dev, shape, rgb):
+    """rgb: the fourth stored channel is zero in X and W (three logical channels; its MFMA step is left out)."""
+    N, IH, IW, OC, F_, s_, p_ = shape
+    X, W = normal((N, IH, IW, 4), 2501), he_normal(OC, F_, F_, 4, 2502)
+    bias = normal((OC,), 2503)
+    if rgb:
+        X[..., 3] = 0.0
+        W[..., 3] = 0.0
+    want = O.conv3D_f64(X, W, s_, s_, p_, p_)
+    L = pkg.lib()
+    try:
+        for algo in (0, 1, 3):      # the kernel without LDS, the kernel with the window in LDS, the generic kernel
+            L.alpha_conv_set_fwd_algo(algo)
+            for entry in ("conv3D", "conv3D_GemmR", "conv3D_GemmV2R"):
+                check(_run_fwd(dev, entry, X, W, s_, s_, p_, p_), want, "%s algo %d %s" % (entry, algo, shape))
+            check(_run_fwd_biased(dev, X, W, bias, s_, s_, p_, p_), want + bias.astype(np.float64), "GemmR_biased algo %d %s" % (algo, shape))
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+
+
 STRIDED_TAP_SHAPES = [
     # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw: strided layers with >= 32 input channels through the LDS-halo kernel
     # (columns of the halo de-interleaved by ow parity class), remode entries
