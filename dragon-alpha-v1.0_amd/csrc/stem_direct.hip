@@ -35,7 +35,7 @@ struct StemDirectArgs {
     int M, IH, IW, OC;
     int FH, FW, taps, sh, sw, ph, pw;
     int x_bytes, w_bytes, y_bytes;
-    int tiles, nblocks, items, slots;   // slots: the SIMDs the items are dealt to (4 per workgroup)
+    int tiles, nblocks, items, wgs;
     FastDiv d_OW, d_OHW, d_FW;
     Epilogue ep;
 };
@@ -51,8 +51,7 @@ __device__ inline unsigned sd_range_mask(int x0, int F, int L)
 }
 
 // G: tap groups (ceil(taps / 4)). Eight wavefronts per workgroup, two per SIMD; the items (block of 64 output channels,
-// tile of 16 pixels) are dealt to the SIMDs as contiguous shares equal to within one, a SIMD's two wavefronts take half
-// a share each.
+// tile of 16 pixels) are dealt to the workgroups as contiguous shares equal to within one.
 template <int G, bool EPI>
 __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArgs p)
 {
@@ -60,10 +59,7 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
     const int t = threadIdx.x, lane = t & 63;
     const int l16 = lane & 15, q = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int slot = blockIdx.x * 4 + (w & 3);
-    const int s_lo = (int)((long)p.items * slot / p.slots), s_hi = (int)((long)p.items * (slot + 1) / p.slots);
-    const int s_mid = s_lo + (s_hi - s_lo + 1) / 2;
-    const int i_lo = w < 4 ? s_lo : s_mid, i_hi = w < 4 ? s_mid : s_hi;
+    const int i_lo = (int)((long)p.items * blockIdx.x / p.wgs), i_hi = (int)((long)p.items * (blockIdx.x + 1) / p.wgs);
 
     const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.X), 0, p.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.W), 0, p.w_bytes, 0x00020000);
@@ -93,7 +89,8 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
         need[g] = tap < p.taps ? (1u << fh) | (1u << (16 + fw)) : 0x80000000u;   // taps past the last: never inside
     }
 
-    auto run = [&](auto tc, auto scc, const int nb, const int tile0, const int count) {
+    // `count` groups of T tiles: the first from tile0 on, the next `stride` tiles further on, ...
+    auto run = [&](auto tc, auto scc, const int nb, const int tile0, const int count, const int stride) {
         constexpr int T = decltype(tc)::value;
         constexpr int SC = decltype(scc)::value;
         if (count <= 0) return;
@@ -177,7 +174,7 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
                         // the first step of the next group of tiles (past the last group: this group's again, unused)
                         if (c_groups_left > 1) {
                             c_groups_left--;
-                            c_tile += T;
+                            c_tile += stride;
                             locate();
                         }
                         request((P + k + 1) & 1, SdInt<0>{});
@@ -214,25 +211,30 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
         locate();
         request(0, SdInt<0>{});
         for (int g2 = 0; g2 < count; g2++) {
-            const int tile = tile0 + g2 * T;
+            const int tile = tile0 + g2 * stride;
             if ((G & 1) && (g2 & 1)) group(SdInt<1>{}, tile);
             else group(SdInt<0>{}, tile);
         }
     };
 
-    // the share as runs of tiles of one block of output channels each (item = nb * tiles + tile): groups of four tiles,
-    // then single tiles
+    // The workgroup's share as runs of tiles of one block of output channels each (item = nb * tiles + tile). A run's
+    // groups of four tiles are dealt to the eight wavefronts round-robin, so that at any time the workgroup works on some
+    // 32 neighbouring tiles, whose windows overlap (rows oh and oh + 1 of a 7x7 stride-2 layer share five of seven input
+    // rows): the re-reads then hit the L2 of the workgroup's XCD. Their number is a multiple of four, so that every SIMD
+    // (wavefronts w and w + 4) gets the same number; the tiles left - fewer than 16 - go out one by one.
     int i = i_lo;
     while (i < i_hi) {
         const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
         const int cnt = min(i_hi - i, p.tiles - tile0);
-        const int n4 = cnt >> 2, n1 = cnt & 3;
+        const int n4 = (cnt >> 2) & ~3;
+        const int mine4 = n4 > w ? (n4 - w + 7) >> 3 : 0;
+        const int rest = cnt - 4 * n4, mine1 = rest > w ? (rest - w + 7) >> 3 : 0;
         if (use_ch3) {
-            run(SdInt<4>{}, SdInt<4>{}, nb, tile0, n4);
-            run(SdInt<1>{}, SdInt<4>{}, nb, tile0 + 4 * n4, n1);
+            run(SdInt<4>{}, SdInt<4>{}, nb, tile0 + 4 * w, mine4, 32);
+            run(SdInt<1>{}, SdInt<4>{}, nb, tile0 + 4 * n4 + w, mine1, 8);
         } else {
-            run(SdInt<4>{}, SdInt<3>{}, nb, tile0, n4);
-            run(SdInt<1>{}, SdInt<3>{}, nb, tile0 + 4 * n4, n1);
+            run(SdInt<4>{}, SdInt<3>{}, nb, tile0 + 4 * w, mine4, 32);
+            run(SdInt<1>{}, SdInt<3>{}, nb, tile0 + 4 * n4 + w, mine1, 8);
         }
         i += cnt;
     }
@@ -265,7 +267,7 @@ hipError_t launch_stem_direct(hipStream_t stream, const float *X, const float *W
     a.ep = ep ? *ep : bias_epilogue(bias);
     int wgs = cus;   // one workgroup of eight wavefronts per compute unit
     if (wgs * 8 > a.items) wgs = (a.items + 7) / 8;
-    a.slots = wgs * 4;
+    a.wgs = wgs;
     if (G == 13) {
         if (a.ep.fused) hipLaunchKernelGGL((stem_direct_kernel<13, true>), dim3(wgs), dim3(512), 0, stream, a);
         else hipLaunchKernelGGL((stem_direct_kernel<13, false>), dim3(wgs), dim3(512), 0, stream, a);
