@@ -264,6 +264,14 @@ hipError_t launch_deltaW_rows(hipStream_t stream, const float *X, const float *d
                               int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,
                               int sh, int sw, int ph, int pw, int GK_slice, int GZ, float *dB = nullptr, float *dB_buf = nullptr);
 
+// Backward-filter with the reduction dealt out evenly to one persistent workgroup per compute unit (delta_w_stream.hip):
+// deltaW and the GZ - 1 buffers add up to the result, but which pixels go into which buffer is the kernel's choice (an
+// item's pieces in order; buffers beyond them are zero-filled). Returns hipErrorNotSupported (nothing launched) when GZ
+// is 1 or too small for the pieces of an item.
+hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
+                                int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,
+                                int sh, int sw, int ph, int pw, int GZ);
+
 // Backward-filter with the filter tap in the grid and both operands straight from memory (delta_w_taps.hip): any filter,
 // stride and padding; same slice partition and outputs. Returns hipErrorNotSupported (nothing launched) when it does not fit.
 hipError_t launch_deltaW_taps(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,

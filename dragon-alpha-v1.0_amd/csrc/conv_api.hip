@@ -350,7 +350,10 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     a.GZ = GridZ;
     a.GK_slice = (a.GK / GridZ) >> 3 << 3;
     const int algo = fwd_algo();
-    // Which kernel (all share the slice partition and the outputs):
+    // Which kernel (all but the first share the slice partition and the outputs):
+    //  - layers whose channel counts fill 64 x 64 blocks to 75 % or more, GridZ of 2 or more: the persistent kernel of
+    //    delta_w_stream.hip (its own partition of the pixels among deltaW and the buffers; a bias gradient takes a pass of
+    //    its own over deltaY then, so layers where another kernel produces it on the way stay with that kernel);
     //  - 1x1 stride 1 with channel counts in multiples of 64: the register kernel of delta_w_pointwise.hip;
     //  - layers whose channel counts fill the 64 x 64 blocks of the tap-per-workgroup kernel to 75 % or more: that kernel
     //    (any filter, stride and padding); the bias gradient, when asked for, then takes a pass of its own over deltaY -
@@ -359,13 +362,19 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     // algo 3 forces the generic kernel, 4 the tap-per-workgroup kernel wherever it fits, 5 the row-streaming kernel
     // wherever it fits (comparisons and tests).
     const bool w1 = FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
+    const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
+    const bool blocks_filled = 4L * IC * OC >= 3L * icb * 64 * ocb * 64;
+    const bool rows_fill = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1)) && icb * ((OC + 31) / 32) * GridZ >= 2L * device_cu_count();
+    if (algo == 0 && blocks_filled && !(dB && (rows_fill || w1))) {
+        // the same arithmetic with the reduction dealt out evenly (its own partition of the pixels among the buffers)
+        hipError_t e = launch_deltaW_stream(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, GridZ);
+        if (e == hipSuccess && dB) e = launch_col_sum(stream0(streams), dY, dB, dB_buf, OC, a.GK, a.GK_slice, GridZ);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     if (algo != 3 && algo != 4 && algo != 5 && w1) {
         hipError_t e = launch_deltaW_pointwise(stream0(streams), X, dY, dW, dW_buf, a.GK, IC, OC, a.GK_slice, GridZ, dB, dB_buf);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
-    const bool blocks_filled = 4L * IC * OC >= 3L * icb * 64 * ocb * 64;
-    const bool rows_fill = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1)) && icb * ((OC + 31) / 32) * GridZ >= 2L * device_cu_count();
     if (algo == 4 || (algo != 3 && algo != 5 && blocks_filled && !(dB && rows_fill))) {
         hipError_t e = launch_deltaW_taps(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, a.GK_slice, GridZ);
         if (e == hipSuccess && dB) e = launch_col_sum(stream0(streams), dY, dB, dB_buf, OC, a.GK, a.GK_slice, GridZ);

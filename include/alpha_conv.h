@@ -98,7 +98,10 @@ int alpha_conv3D_W1(const int64_t *streams, int length,
 /* conv/A.cu:137  Java: Cuda_conv3D.kernel_remode   W[OC,FH,FW,IC] -> CW[FH,FW,IC,OC] */
 int alpha_kernel_remode(int64_t stream, const float *W, float *CW, int FH, int FW, int OC, int IC);
 
-/* conv/A.cu:149  Java: Cuda_conv3D.conv3D_GemmR   (CW = remoded filter; W kept for signature parity) */
+/* conv/A.cu:149  Java: Cuda_conv3D.conv3D_GemmR   (CW = remoded filter). W is the filter CW was made from, as the
+ * Java engine passes it (the reference hands both to its kernels, conv/A.cu:165-170): layers with 4 stored input
+ * channels read its 16-byte taps in place; NULL is accepted and keeps every layer on CW. The same holds for the other
+ * entries that take W and CW. */
 int alpha_conv3D_GemmR(const int64_t *streams, int length,
                        const float *X, int IH, int IW,
                        const float *W, const float *CW, int FH, int FW,

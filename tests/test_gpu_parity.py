@@ -763,6 +763,54 @@ def test_deltaW_split_k_slices_follow_the_reference_partition(dev):
         check(parts[z], O.deltaW_slice_f64(X, dY, F_, F_, s, s, p, p, GridZ, z), "slice %d" % z)
 
 
+DW_STREAM_SHAPES = [
+    # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw, GridZ, R: the persistent backward-filter kernel (one workgroup per compute
+    # unit; its own partition of the pixels among deltaW and the buffers, so only the sum is compared). On 256 compute units
+    # (R: pieces per item where every item is cut into equal pieces - partial sums R .. GridZ - 1 are then zeros - else None):
+    (128, 8, 8, 256, 256, 3, 3, 1, 1, 1, 1, 3, None),      # c2c: 144 items in a line cut into 256 shares, 2 or 3 pieces per item
+    (32, 56, 56, 64, 64, 3, 3, 1, 1, 1, 1, 128, 28),     # c5b: 9 items x 28 pieces, buffers 28 .. 127 filled with zeros
+    (40, 30, 30, 64, 128, 3, 3, 2, 2, 1, 1, 16, 14),     # stride 2, rows of 15 pixels (ragged last group): 18 items x 14 pieces
+    (24, 21, 23, 64, 176, 3, 3, 1, 1, 1, 1, 12, None),     # 27 items (third block of output channels 48 of 64) in a line, rows of 23 pixels
+    (8, 32, 32, 256, 64, 1, 1, 1, 1, 0, 0, 128, 64),     # 1x1: 4 items x 64 pieces
+    (128, 9, 9, 256, 256, 4, 4, 1, 1, 1, 1, 2, 1),      # 256 items, one piece each; the one buffer is all zeros
+    (16, 40, 36, 128, 64, 5, 3, 1, 2, 2, 1, 64, None),  # 5x3 filter, stride 1 x 2: 30 items in a line (8 equal pieces each would use 240 workgroups)
+]
+
+
+@pytest.mark.parametrize("shape", DW_STREAM_SHAPES)
+def test_deltaW_persistent_kernel_sum_and_reproducibility(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw, GridZ, R = shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    X, dY = normal((N, IH, IW, IC), 3401), normal((N, OH, OW, OC), 3402)
+    want = O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw)
+    x, dy = dev.put(X), dev.put(dY)
+    sizeW = OC * FH * FW * IC
+    runs = []
+    for _ in range(2):
+        dWo = dev.guarded(OC, FH, FW, IC)
+        buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+        DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
+                                 FH, FW, N, IC, OC, sh, sw, ph, pw)
+        parts = np.concatenate([dev.get(dWo).reshape(1, -1), dev.get(buf)])
+        runs.append(parts)
+        check(_sum_partials(dev, dWo, buf, GridZ), want, "persistent dW GridZ=%d %s" % (GridZ, shape))
+    assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32)), "partial sums differ between two runs %s" % (shape,)
+    if R is not None and pkg.device_info()[0] == 256:
+        # this kernel, not another one, served the call: the partial sums beyond an item's pieces are zeros, the last piece is not
+        assert not runs[0][R:].any() and runs[0][R - 1].any(), "partial sums %d .. %d are not all zeros %s" % (R, GridZ - 1, shape)
+    # the same layer through the tap-per-workgroup kernel (the reference's partition): the totals agree within tolerance
+    L = pkg.lib()
+    try:
+        L.alpha_conv_set_fwd_algo(4)
+        dWo = dev.guarded(OC, FH, FW, IC)
+        buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+        DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
+                                 FH, FW, N, IC, OC, sh, sw, ph, pw)
+        check(_sum_partials(dev, dWo, buf, GridZ), want, "tap kernel GridZ=%d %s" % (GridZ, shape))
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+
+
 DW_ROWS_SHAPES = [
     # stride-1 layers served by the row-streaming kernel: N, IH, IW, IC, OC, F, p, GridZ
     (4, 56, 56, 64, 64, 3, 1, 16),     # c5b geometry
