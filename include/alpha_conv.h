@@ -235,9 +235,12 @@ int alpha_dconv3D_deltaW_W1(const int64_t *streams, int length,
 /* dW/A.cu:66   Java: buf_summary   deltaW += sum_{p<part} deltaW_buf[p], fixed order, fp32 Kahan */
 int alpha_buf_summary(int64_t stream, const float *deltaW_buf, float *deltaW, int part, int sizeW);
 
-/* dW/A.cu:79   Java: dconv3D_deltaW_GemmSK.  Split-K: GK_slice = (GK/GridZ) >> 3 << 3; slice 0 is
- * written to deltaW, slice z >= 1 to deltaW_buf[z-1] (sizeW floats each); the last slice takes the
- * remainder. The caller sums with alpha_buf_summary(part = GridZ-1). No atomics: bit-reproducible. */
+/* dW/A.cu:79   Java: dconv3D_deltaW_GemmSK.  Split-K: deltaW and the GridZ-1 buffers of deltaW_buf (sizeW floats
+ * each) receive partial sums that add up to the result; the caller sums them with alpha_buf_summary(part = GridZ-1).
+ * Every element of all of them is written (zeros where a buffer is not needed). No atomics: bit-reproducible.
+ * Which pixels a buffer holds: the reference's partition (buffer z the pixels [z*GK_slice, (z+1)*GK_slice), GK_slice =
+ * (GK/GridZ) >> 3 << 3, the last slice the remainder) in the kernels behind alpha_conv_set_fwd_algo(4) and for layers
+ * the default kernel does not take; the default kernel deals the pixels out evenly over the compute units instead. */
 int alpha_dconv3D_deltaW_GemmSK(const int64_t *streams, int length, int GridZ,
                                 const float *X, int IH, int IW,
                                 const float *deltaY, int OH, int OW,
