@@ -45,11 +45,11 @@ constexpr int DCP_TB = 32;                    // tiles per chunk of the line of 
 constexpr unsigned DCP_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
 template <bool EPI>
-__global__ __launch_bounds__(256, 2) void direct_conv_phased_kernel(const DirectPhasedArgs p)
+__global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const DirectPhasedArgs p)
 {
     const int t = threadIdx.x, lane = t & 63;
     const int l16 = lane & 15, q = lane >> 4;
-    const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (t >> 6));
+    const int w = __builtin_amdgcn_readfirstlane(t >> 6);   // wavefronts w and w + 4 of a workgroup share SIMD w % 4
     const int CH = p.AC >> 4;   // even (host-checked): every phase has an even number of steps
 
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
@@ -197,8 +197,13 @@ __global__ __launch_bounds__(256, 2) void direct_conv_phased_kernel(const Direct
     //      other, and the line is dealt to the wavefronts XCD by XCD (workgroups go round-robin to the 8 XCDs, each with
     //      its own L2), so the second to fourth reader of a pixel finds it in L2 ------------------------------------------
     const int G = gridDim.x;
-    const int order = (G & 7) == 0 ? ((int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3)) * 4 + (wave & 3) : wave;
-    const long pos_lo = p.total_cost * order / p.waves, pos_hi = p.total_cost * (order + 1) / p.waves;
+    // A share belongs to a SIMD (what has to be even is the work per SIMD, whose two wavefronts halve it): the items that
+    // begin in it differ from the mean by at most one item per SIMD, not per wavefront.
+    const int wg_order = (G & 7) == 0 ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    const int order = wg_order * 4 + (w & 3);
+    const long s_lo = p.total_cost * order / p.waves, s_hi = p.total_cost * (order + 1) / p.waves;
+    const long s_mid = s_lo + (s_hi - s_lo) / 2;
+    const long pos_lo = w < 4 ? s_lo : s_mid, pos_hi = w < 4 ? s_mid : s_hi;
     int csum = 0;   // cost of a tile with all its phases
     for (int f = 0; f < p.nph; f++) csum += 4 * TH(f) * TW(f) + 1;
     const long per_nb = (long)p.tiles * csum;
@@ -289,11 +294,11 @@ hipError_t launch_direct_conv_phased(hipStream_t stream, const float *A, const f
     a.d_OW = make_fastdiv(OWt);
     a.d_OHW = make_fastdiv(OHt * OWt);
     a.ep = ep ? *ep : bias_epilogue(nullptr);
-    int wgs = 2 * cus;   // two wavefronts per SIMD
-    if (wgs * 4 > a.items) wgs = (a.items + 3) / 4;
-    a.waves = wgs * 4;
-    if (a.ep.fused) hipLaunchKernelGGL(direct_conv_phased_kernel<true>, dim3(wgs), dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL(direct_conv_phased_kernel<false>, dim3(wgs), dim3(256), 0, stream, a);
+    int wgs = cus;   // one workgroup of eight wavefronts per compute unit
+    if (wgs * 8 > a.items) wgs = (a.items + 7) / 8;
+    a.waves = wgs * 4;   // the SIMDs the line of items is dealt to
+    if (a.ep.fused) hipLaunchKernelGGL(direct_conv_phased_kernel<true>, dim3(wgs), dim3(512), 0, stream, a);
+    else hipLaunchKernelGGL(direct_conv_phased_kernel<false>, dim3(wgs), dim3(512), 0, stream, a);
     return hipGetLastError();
 }
 
