@@ -59,6 +59,13 @@ constexpr size_t DC_LDS_BYTES = 8 * 4 * DC_SPLIT_T * 64 * sizeof(floatx4);
 // eight parts of the reduction steps - a SIMD's two parts together are a quarter of the steps -, and the eight partial
 // results are added through LDS in a fixed order. 12544 items on 256 workgroups: 49 = 4 x 12 + 1 per workgroup, 12.25
 // per SIMD, where whole items alone would make it 13 on some SIMDs.
+// Bits f < F (F <= 16) with 0 <= x0 + f < L: the window positions inside the image along one axis.
+__device__ inline unsigned dc_range_mask(int x0, int F, int L)
+{
+    const int lo = max(0, -x0), hi = min(F, L - x0);
+    return hi > lo ? ((1u << hi) - 1u) & ~((1u << lo) - 1u) : 0u;
+}
+
 // whole items per SIMD of a workgroup with n items
 __host__ __device__ inline int dc_whole_items(int n)
 {
@@ -78,6 +85,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     const int f = dc_whole_items(g_hi - g_lo);
     const int i_lo = g_lo + (w & 3) * f + (w >> 2) * (f >> 1), i_hi = i_lo + (f >> 1);
     const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group: even (host-checked)
+    const bool pointwise = taps == 1 && p.sh == 1 && p.sw == 1 && p.ph == 0 && p.pw == 0;
 
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.B), 0, p.b_bytes, 0x00020000);
@@ -113,6 +121,15 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         unsigned rc[T];      // bit th: window row th is inside the image; bit 16 + tw: window column tw is
         unsigned voff[T];    // this tap's load offset, or DC_NEVER in the padding
         auto locate = [&]() {
+            if (pointwise) {   // uniform: a 1x1 stride-1 layer without padding reads pixel m itself
+#pragma unroll
+                for (int i = 0; i < T; i++) {
+                    const int m = (c_tile + i) * 16 + l16;
+                    org[i] = (m * p.AC + 4 * q) * 4;
+                    rc[i] = m < p.M ? 0x00010001u : 0u;
+                }
+                return;
+            }
 #pragma unroll
             for (int i = 0; i < T; i++) {
                 const int m = (c_tile + i) * 16 + l16;
@@ -122,10 +139,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                 const int oh = fdiv(rem, p.d_OW), ow = rem - oh * (int)p.d_OW.d;
                 const int ih0 = oh * p.sh - p.ph, iw0 = ow * p.sw - p.pw;
                 org[i] = (((n * p.AH + ih0) * p.AW + iw0) * p.AC + 4 * q) * 4;
-                unsigned m_ = 0;
-                for (int th = 0; th < p.TH; th++) m_ |= (unsigned)(live && (unsigned)(ih0 + th) < (unsigned)p.AH) << th;
-                for (int tw = 0; tw < p.TW; tw++) m_ |= (unsigned)((unsigned)(iw0 + tw) < (unsigned)p.AW) << (16 + tw);
-                rc[i] = m_;
+                rc[i] = (live ? dc_range_mask(ih0, p.TH, p.AH) : 0u) | (dc_range_mask(iw0, p.TW, p.AW) << 16);
             }
         };
         auto aim = [&]() {   // offsets of tap c_tap
