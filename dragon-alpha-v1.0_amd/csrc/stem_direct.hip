@@ -35,8 +35,10 @@ struct StemDirectArgs {
     int M, IH, IW, OC;
     int FH, FW, taps, sh, sw, ph, pw;
     int x_bytes, w_bytes, y_bytes;
-    int tiles, nblocks, items, wgs;
-    FastDiv d_OW, d_OHW, d_FW;
+    int tiles, nblocks, groups, items, wgs;   // items = nblocks * groups
+    int TPR, rows;    // OW % 16 == 0: tiles per output row and output rows N * OH; else TPR = 0
+    FastDiv d_TPR;
+    FastDiv d_OW, d_OHW, d_FW, d_OH;
     Epilogue ep;
 };
 
@@ -44,7 +46,7 @@ template <int V> struct SdInt { static constexpr int value = V; };
 constexpr unsigned SD_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
 // Bits f < F (F <= 15) with 0 <= x0 + f < L: the window positions inside the image along one axis.
-__device__ inline unsigned sd_range_mask(int x0, int F, int L)
+__device__ inline unsigned sd_range_mask(int x0, int F, int L)   // works on uniform and on per-lane values
 {
     const int lo = max(0, -x0), hi = min(F, L - x0);
     return hi > lo ? ((1u << hi) - 1u) & ~((1u << lo) - 1u) : 0u;
@@ -89,8 +91,21 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
         need[g] = tap < p.taps ? (1u << fh) | (1u << (16 + fw)) : 0x80000000u;   // taps past the last: never inside
     }
 
-    // `count` groups of T tiles: the first from tile0 on, the next `stride` tiles further on, ...
-    auto run = [&](auto tc, auto scc, const int nb, const int tile0, const int count, const int stride) {
+    // The tiles of group gidx. Where the rows are whole tiles (OW % 16 == 0) a group is the same 16 columns of four
+    // consecutive output rows - their windows overlap most, and whether every tap of every pixel lies inside the image is
+    // then the same question for all four: true for most groups, which take the short way in `request` below -; else
+    // four consecutive tiles. Tiles past the end get the index p.tiles: no live pixel, nothing stored.
+    auto tile_of = [&](const int gidx, const int i) {   // uniform
+        if (p.TPR > 0) {
+            const int sb = fdiv(gidx, p.d_TPR), tx = gidx - sb * p.TPR, row = 4 * sb + i;
+            return row < p.rows ? row * p.TPR + tx : p.tiles;
+        }
+        const int tl = 4 * gidx + i;
+        return tl < p.tiles ? tl : p.tiles;
+    };
+    // `count` groups of T tiles. T = 4: groups g0 + first, g0 + first + 8, ...; T = 1: the single tiles number first,
+    // first + 8, ... of the groups from g0 on (tile k belongs to group g0 + k / 4).
+    auto run = [&](auto tc, auto scc, const int nb, const int g0, const int first, const int count) {
         constexpr int T = decltype(tc)::value;
         constexpr int SC = decltype(scc)::value;
         if (count <= 0) return;
@@ -117,13 +132,36 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
         using frag = std::conditional_t<SC == 3, floatx3, floatx4>;
         frag a[2][T], b[2][4];
         // ---- load cursor: one step ahead of the multiplications ------------------------------------------------------------
-        int c_tile = tile0, c_groups_left = count;
+        int c_idx = first, c_groups_left = count;
+        bool c_inside = false;   // every tap of every pixel of the cursor's tiles lies inside the image (uniform)
+        auto tile_at = [&](const int idx, const int i) { return T == 4 ? tile_of(g0 + idx, i) : tile_of(g0 + (idx >> 2), idx & 3); };
         int org[T];       // byte offset of this lane's pixel's window origin; may lie before the tensor
         unsigned rc[T];   // bit fh: window row fh is inside the image; bit 16 + fw: window column fw is
+        const unsigned full = ((1u << p.FH) - 1u) | (((1u << p.FW) - 1u) << 16);
         auto locate = [&]() {
+            bool all_full = true;
+            if (p.TPR > 0) {
+                // rows are whole tiles: the image, the output row and with them the window rows are the same for the 16
+                // pixels of a tile (scalar arithmetic); only the columns differ from lane to lane
+#pragma unroll
+                for (int i = 0; i < T; i++) {
+                    const int tile = tile_at(c_idx, i);
+                    const bool live = tile < p.tiles;
+                    const int row = fdiv(live ? tile : 0, p.d_TPR), tx = (live ? tile : 0) - row * p.TPR;
+                    const int n = fdiv(row, p.d_OH), oh = row - n * (int)p.d_OH.d;
+                    const int ih0 = oh * p.sh - p.ph;
+                    const unsigned rows_in = live ? sd_range_mask(ih0, p.FH, p.IH) : 0u;
+                    const int iw0 = (tx * 16 + l16) * p.sw - p.pw;
+                    org[i] = ((n * p.IH + ih0) * p.IW + iw0) * 16;
+                    rc[i] = rows_in | (sd_range_mask(iw0, p.FW, p.IW) << 16);
+                    all_full = all_full && rc[i] == full;
+                }
+                c_inside = __all(all_full) != 0;
+                return;
+            }
 #pragma unroll
             for (int i = 0; i < T; i++) {
-                const int m = (c_tile + i) * 16 + l16;
+                const int m = tile_at(c_idx, i) * 16 + l16;
                 const bool live = m < p.M;
                 const int mm = live ? m : 0;
                 const int n = fdiv(mm, p.d_OHW), rem = mm - n * (int)p.d_OHW.d;
@@ -131,21 +169,31 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
                 const int ih0 = oh * p.sh - p.ph, iw0 = ow * p.sw - p.pw;
                 org[i] = ((n * p.IH + ih0) * p.IW + iw0) * 16;
                 rc[i] = (live ? sd_range_mask(ih0, p.FH, p.IH) : 0u) | (sd_range_mask(iw0, p.FW, p.IW) << 16);
+                all_full = all_full && rc[i] == full;
             }
+            c_inside = __all(all_full) != 0;
         };
         auto request = [&](int slot, auto gc) {   // the loads of tap group g of the cursor's tiles
             constexpr int g = decltype(gc)::value;
+            unsigned voff[T];
+            if (c_inside) {   // uniform: one addition per tile (taps past the last, in the last group, stay out of range)
+#pragma unroll
+                for (int i = 0; i < T; i++)
+                    voff[i] = (g == G - 1 && !last_tap_ok) ? SD_NEVER : (unsigned)(org[i] + toff[g]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < T; i++) voff[i] = (rc[i] & need[g]) == need[g] ? (unsigned)(org[i] + toff[g]) : SD_NEVER;
+            }
 #pragma unroll
             for (int i = 0; i < T; i++) {
-                const unsigned voff = (rc[i] & need[g]) == need[g] ? (unsigned)(org[i] + toff[g]) : SD_NEVER;
-                if constexpr (SC == 3) a[slot][i] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(x_rsrc, voff, 0, 0));
-                else a[slot][i] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, voff, 0, 0));
+                if constexpr (SC == 3) a[slot][i] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(x_rsrc, voff[i], 0, 0));
+                else a[slot][i] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, voff[i], 0, 0));
             }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const unsigned voff = (g == G - 1 && !last_tap_ok) ? SD_NEVER : b_voff[j];
-                if constexpr (SC == 3) b[slot][j] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(w_rsrc, voff, g * 64, 0));
-                else b[slot][j] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, voff, g * 64, 0));
+                const unsigned bv = (g == G - 1 && !last_tap_ok) ? SD_NEVER : b_voff[j];
+                if constexpr (SC == 3) b[slot][j] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(w_rsrc, bv, g * 64, 0));
+                else b[slot][j] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, bv, g * 64, 0));
             }
         };
         floatx4 acc[T][4];
@@ -159,7 +207,7 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
                         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[slot][i][s], b[slot][j][s], acc[i][j], 0, 0, 0);
         };
         // one group of tiles; P: the register set that holds its first step
-        auto group = [&](auto pc, const int tile) {
+        auto group = [&](auto pc, const int idx) {
             constexpr int P = decltype(pc)::value;
 #pragma unroll
             for (int i = 0; i < T; i++)
@@ -174,7 +222,7 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
                         // the first step of the next group of tiles (past the last group: this group's again, unused)
                         if (c_groups_left > 1) {
                             c_groups_left--;
-                            c_tile += stride;
+                            c_idx += 8;
                             locate();
                         }
                         request((P + k + 1) & 1, SdInt<0>{});
@@ -187,10 +235,12 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
             step(SdInt<0>{}, step);
             // ---- results: lane holds pixels 16 (tile + i) + 4q + r, output channels 64 nb + 4 l16 + j ------------------------
 #pragma unroll
-            for (int i = 0; i < T; i++)
+            for (int i = 0; i < T; i++) {
+                const int tile = tile_at(idx, i);
+                if (tile >= p.tiles) continue;   // uniform
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const int o_off = __builtin_amdgcn_readfirstlane(((tile + i) * 16 + r) * p.OC * 4);   // rows past M: beyond the descriptor
+                    const int o_off = __builtin_amdgcn_readfirstlane((tile * 16 + r) * p.OC * 4);   // rows past M: beyond the descriptor
                     floatx4 v = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
                     if (EPI) {
                         if (p.ep.gate) {   // uniform
@@ -207,34 +257,34 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
                     }
                     buffer_store_b128_guarded(v, y_rsrc, o_lane, o_off);
                 }
+            }
         };
         locate();
         request(0, SdInt<0>{});
         for (int g2 = 0; g2 < count; g2++) {
-            const int tile = tile0 + g2 * stride;
-            if ((G & 1) && (g2 & 1)) group(SdInt<1>{}, tile);
-            else group(SdInt<0>{}, tile);
+            if ((G & 1) && (g2 & 1)) group(SdInt<1>{}, first + 8 * g2);
+            else group(SdInt<0>{}, first + 8 * g2);
         }
     };
 
-    // The workgroup's share as runs of tiles of one block of output channels each (item = nb * tiles + tile). A run's
-    // groups of four tiles are dealt to the eight wavefronts round-robin, so that at any time the workgroup works on some
-    // 32 neighbouring tiles, whose windows overlap (rows oh and oh + 1 of a 7x7 stride-2 layer share five of seven input
-    // rows): the re-reads then hit the L2 of the workgroup's XCD. Their number is a multiple of four, so that every SIMD
-    // (wavefronts w and w + 4) gets the same number; the tiles left - fewer than 16 - go out one by one.
+    // The workgroup's share as runs of groups of one block of output channels each (item = nb * groups + group). A run's
+    // groups are dealt to the eight wavefronts round-robin, so that at any time the workgroup works on neighbouring
+    // tiles, whose windows overlap (rows oh and oh + 1 of a 7x7 stride-2 layer share five of seven input rows): the
+    // re-reads then hit the L2 of the workgroup's XCD. The groups dealt out whole are a multiple of four, so that every
+    // SIMD (wavefronts w and w + 4) gets the same number; the tiles of the up to three groups left go out one by one.
     int i = i_lo;
     while (i < i_hi) {
-        const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
-        const int cnt = min(i_hi - i, p.tiles - tile0);
-        const int n4 = (cnt >> 2) & ~3;
+        const int nb = i / p.groups, g0 = i - nb * p.groups;
+        const int cnt = min(i_hi - i, p.groups - g0);
+        const int n4 = cnt & ~3;
         const int mine4 = n4 > w ? (n4 - w + 7) >> 3 : 0;
-        const int rest = cnt - 4 * n4, mine1 = rest > w ? (rest - w + 7) >> 3 : 0;
+        const int rest = 4 * (cnt - n4), mine1 = rest > w ? (rest - w + 7) >> 3 : 0;
         if (use_ch3) {
-            run(SdInt<4>{}, SdInt<4>{}, nb, tile0 + 4 * w, mine4, 32);
-            run(SdInt<1>{}, SdInt<4>{}, nb, tile0 + 4 * n4 + w, mine1, 8);
+            run(SdInt<4>{}, SdInt<4>{}, nb, g0, w, mine4);
+            run(SdInt<1>{}, SdInt<4>{}, nb, g0 + n4, w, mine1);
         } else {
-            run(SdInt<4>{}, SdInt<3>{}, nb, tile0 + 4 * w, mine4, 32);
-            run(SdInt<1>{}, SdInt<3>{}, nb, tile0 + 4 * n4 + w, mine1, 8);
+            run(SdInt<4>{}, SdInt<3>{}, nb, g0, w, mine4);
+            run(SdInt<1>{}, SdInt<3>{}, nb, g0 + n4, w, mine1);
         }
         i += cnt;
     }
@@ -260,13 +310,24 @@ hipError_t launch_stem_direct(hipStream_t stream, const float *X, const float *W
     a.tiles = (int)((M + 15) / 16);
     a.nblocks = (OC + 63) / 64;
     if ((long)a.tiles * a.nblocks >= (1L << 30)) return hipErrorNotSupported;
-    a.items = a.tiles * a.nblocks;
+    if ((OW & 15) == 0) {   // rows are whole tiles: a group is the same 16 columns of four consecutive output rows
+        a.TPR = OW / 16;
+        a.rows = N * OH;
+        a.groups = ((a.rows + 3) / 4) * a.TPR;
+    } else {
+        a.TPR = 0;
+        a.rows = 0;
+        a.groups = (a.tiles + 3) / 4;
+    }
+    a.d_TPR = make_fastdiv(a.TPR > 0 ? a.TPR : 1);
+    a.items = a.groups * a.nblocks;
     a.d_OW = make_fastdiv(OW);
     a.d_OHW = make_fastdiv(OH * OW);
     a.d_FW = make_fastdiv(FW);
+    a.d_OH = make_fastdiv(OH);
     a.ep = ep ? *ep : bias_epilogue(bias);
     int wgs = cus;   // one workgroup of eight wavefronts per compute unit
-    if (wgs * 8 > a.items) wgs = (a.items + 7) / 8;
+    if (wgs * 2 > a.items) wgs = (a.items + 1) / 2;
     a.wgs = wgs;
     if (G == 13) {
         if (a.ep.fused) hipLaunchKernelGGL((stem_direct_kernel<13, true>), dim3(wgs), dim3(512), 0, stream, a);
