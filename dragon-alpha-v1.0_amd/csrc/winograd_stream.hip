@@ -15,7 +15,7 @@
 // So the only thing outside the MFMA stream is an item's output transform (A^T m A per lane, which holds all 16 xi of
 // its (tile, channel) pairs) and its stores, which leave the registers directly: 16 lanes write 64 consecutive bytes.
 // Items that do not divide evenly among the workgroups are cut into halves of 16 tiles (the second MFMA row block is
-// left out), so the longest workgroup is half an item above the shortest.
+// left out) as far as the workgroups reach, so the longest workgroup is half an item above most of the others.
 #include "common.hpp"
 #include <type_traits>
 
@@ -32,7 +32,7 @@ struct WinoStreamArgs {
     int x_bytes, u_bytes, y_bytes;   // X and U below 2 GB, Y at most 1 GB
     int whole;           // items every workgroup takes: workgroup b owns [b*whole, (b+1)*whole)
     int extra;           // workgroups below this take item gridDim.x*whole + b as well
-    int halves;          // or: workgroups below this take half (b & 1) of item gridDim.x*whole + b/2
+    int halves;          // the next so many workgroups, b' = b - extra, take half (b' & 1) of item gridDim.x*whole + extra + b'/2
     FastDiv d_TC, d_TRC, d_groups;
 };
 
@@ -50,7 +50,8 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
     const int l16 = lane & 15, q = lane >> 4;
     const int xt = t >> 3, xq = (t & 7) * 2;   // input transform: thread -> (tile xt, channel pair xq of the chunk)
     const int b = blockIdx.x, G = gridDim.x;
-    const int nitems = p.whole + (b < p.extra ? 1 : 0) + (b < p.halves ? 1 : 0);
+    const bool has_half = b >= p.extra && b < p.extra + p.halves;
+    const int nitems = p.whole + (b < p.extra ? 1 : 0) + (has_half ? 1 : 0);
     const int nchunks = p.IC >> 4;
     const unsigned xi_stride4 = (unsigned)p.IC * p.OC * 4;   // bytes between two transform positions of U
     const unsigned chunk_stride4 = 16u * p.OC * 4;           // bytes between two 16-channel chunks of U
@@ -63,11 +64,12 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
         int id, hoff = 0;
         it.half = 0;
         if (k < p.whole) id = b * p.whole + k;
-        else if (p.extra) id = G * p.whole + b;
+        else if (b < p.extra) id = G * p.whole + b;
         else {
-            id = G * p.whole + (b >> 1);
+            const int hb = b - p.extra;
+            id = G * p.whole + p.extra + (hb >> 1);
             it.half = 1;
-            hoff = (b & 1) * 16;
+            hoff = (hb & 1) * 16;
         }
         const int ocb = fdiv(id, p.d_groups), g = id - ocb * p.groups;
         it.oc0 = ocb * 64;
@@ -312,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void winograd_stream_kernel(const WinoStrea
         store_item(half_c, k & 1);
         cur = nxt;
     };
-    const int nfull = b < p.halves ? nitems - 1 : nitems;
+    const int nfull = has_half ? nitems - 1 : nitems;
     for (int k = 0; k < nfull; k++) run_item(std::false_type{}, k);
     if (nfull < nitems) run_item(std::true_type{}, nfull);
 }
@@ -343,12 +345,22 @@ hipError_t launch_winograd_stream(hipStream_t stream, const float *X, const floa
     a.d_groups = make_fastdiv(a.groups);
     const long items = (long)a.groups * ((OC + 63) / 64);
     if (items >= (1L << 30)) return hipErrorNotSupported;
+    // The items beyond a whole number per workgroup go out as halves as far as the workgroups reach - a workgroup takes one
+    // more item or one half -: `left` items on `grid` workgroups are 2 left - grid whole ones and 2 (grid - left) halves when
+    // left > grid / 2, else 2 left halves (28x28x128 at N = 64, 784 items on 512 workgroups: 32 + 480 instead of 272 whole
+    // ones, 0.068 -> 0.062 ms). Fewer items than workgroups: one each - as halves on twice the workgroups every half streams
+    // the item's filter again, and the layers with few items are the ones with large filters (7x7x512 at N = 64, 256 items:
+    // 0.069 ms whole, 0.078 ms in halves).
     const int slots = 2 * cus;
     const int grid = items < slots ? (int)items : slots;
     a.whole = (int)(items / grid);
     const int left = (int)(items - (long)a.whole * grid);   // < grid
-    if (2 * left <= grid) a.halves = 2 * left;
-    else a.extra = left;
+    if (2 * left <= grid) {
+        a.halves = 2 * left;
+    } else {
+        a.extra = 2 * left - grid;
+        a.halves = 2 * (grid - left);
+    }
 
     constexpr auto kern = winograd_stream_kernel;
     const size_t lds = (size_t)2 * WS_VBUF * sizeof(float) + 2 * WS_TILES * 4 * sizeof(unsigned);   // V[2], otab[2]
