@@ -311,6 +311,8 @@ DX_S1_SHAPES = [
     (4, 9, 9, 8, 8, 3, 3, 0, 0),
     (4, 7, 9, 4, 36, 3, 2, 2, 1),
     (4, 12, 12, 132, 44, 3, 3, 1, 1),
+    (16, 14, 14, 128, 256, 3, 3, 1, 1),  # 392 items of 144 steps on 256 workgroups: one or two each, all shared by the wavefronts
+    (40, 7, 7, 192, 512, 3, 3, 1, 1),    # 369 items (the last tile ragged), three blocks of produced channels, 288 steps
 ]
 
 
@@ -432,6 +434,10 @@ DIRECT_CONV_SHAPES = [
     (32, 40, 40, 32, 64, 3, 3, 1, 1, 1, 1),     # 3200 items: 12 or 13 per workgroup, all shared in groups of 4, 4, 4 (, 1)
     (44, 40, 40, 32, 64, 3, 3, 1, 1, 1, 1),     # 4400 items: 17 or 18 per workgroup = 4 whole per SIMD + 1 or 2 shared
     (2, 56, 56, 64, 64, 3, 3, 1, 1, 1, 1),      # 392 items: 1 or 2 per workgroup, 36 steps in parts of 4 and 5
+    # long reductions
+    (16, 14, 14, 256, 128, 3, 3, 1, 1, 1, 1),   # 392 items of 144 steps on 256 workgroups: one or two each
+    (36, 7, 7, 512, 192, 3, 3, 1, 1, 1, 1),     # 333 items of 288 steps (ragged last tile), three blocks of produced channels
+    (4, 9, 9, 256, 64, 5, 5, 2, 2, 2, 2),       # strided 5x5: 7 items of 400 steps on 7 workgroups
 ]
 
 
