@@ -469,6 +469,8 @@ STEM_FWD_SHAPES = [
     (8, 21, 23, 136, 7, 2, 0),      # no padding, three blocks of output channels (the last with 8)
     (4, 32, 32, 64, 3, 1, 1),       # c1 geometry: 3x3 = three tap groups (taps 9..11 are padding)
     (32, 17, 19, 20, 3, 2, 1),      # 3x3 stride 2, 20 output channels
+    (3, 34, 32, 64, 3, 1, 1),       # rows are whole tiles (groups = 16 columns x 4 rows), 102 rows: the last group has two
+    (5, 38, 64, 64, 7, 2, 3),       # 7x7 stride 2, rows of 32 pixels, 19 rows per image: groups straddle images, 95 rows in all
     (3, 9, 9, 64, 5, 1, 2),         # 5x5: not taken by the kernel without LDS -> the LDS one
 ]
 
