@@ -280,7 +280,10 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     i = g_lo + 4 * f;
     while (i < g_hi) {
         const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
-        const int cnt = min(min(g_hi - i, p.tiles - tile0), DC_SPLIT_T);
+        // groups of sizes equal to within one tile (13 tiles: 4 + 3 + 3 + 3, not 4 + 4 + 4 + 1: a group of one tile pays the
+        // first loads and the two barriers for a quarter of the work, with five loads per 16 MFMAs)
+        const int run_len = min(g_hi - i, p.tiles - tile0), ngroups = (run_len + DC_SPLIT_T - 1) / DC_SPLIT_T;
+        const int cnt = (run_len + ngroups - 1) / ngroups;
         if (cnt == 4) run(DcInt<4>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
         else if (cnt == 3) run(DcInt<3>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
         else if (cnt == 2) run(DcInt<2>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
