@@ -94,7 +94,8 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     // `count` groups of T tiles each, from tile0 on, block nb of the produced channels, reduction steps [k_lo, k_lo + k_n)
     // of every group. SPLIT (count 1, every wavefront of the workgroup calls it with its own steps, k_n >= 0 of either
     // parity): the wavefronts' partial results are added through LDS. Otherwise k_n is even and at least 2.
-    auto run = [&](auto tc, auto sp, const int nb, const int tile0, const int count, const int k_lo, const int k_n) {
+    // The groups of a run begin `stride` tiles apart (T: one after the other).
+    auto run = [&](auto tc, auto sp, const int nb, const int tile0, const int count, const int k_lo, const int k_n, const int stride) {
         constexpr int T = decltype(tc)::value;
         constexpr bool SPLIT = decltype(sp)::value;
         if (count <= 0) return;
@@ -167,7 +168,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                     c_tap++;
                     if (c_tap == taps) {
                         c_tap = 0;
-                        c_tile += T;
+                        c_tile += stride;
                         locate();
                     }
                     aim();
@@ -180,7 +181,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
             request(0);
         }
         for (int g = 0; g < count; g++) {
-            const int tile = tile0 + g * T;
+            const int tile = tile0 + g * stride;
             floatx4 acc[T][4];
 #pragma unroll
             for (int i = 0; i < T; i++)
@@ -247,13 +248,12 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         }
     };
 
-    // the wavefront's whole items as runs of tiles of one block of produced channels each (item = nb * tiles + tile),
-    // every run as groups of 4, 3, 2 and 1 tiles: 4a + 3b for six tiles or more, 3 + 2 for five
-    int i = i_lo;
-    while (i < i_hi) {
-        const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
-        const int cnt = min(i_hi - i, p.tiles - tile0);
-        int n4 = 0, n3 = 0, n2 = 0, n1 = 0;
+    // The whole items, f / 2 tiles per wavefront as groups of 4, 3, 2 and 1 tiles (4a + 3b for six tiles or more, 3 + 2 for
+    // five). Where the workgroup's 4 f tiles lie in one block of produced channels the groups are dealt to the eight
+    // wavefronts round-robin - all wavefronts run groups of the same size at the same time, on neighbouring tiles, so the
+    // rows their windows share are fetched into L2 once -; else every wavefront takes its f / 2 tiles as one contiguous run.
+    auto groups_of = [&](const int cnt, int &n4, int &n3, int &n2, int &n1) {
+        n4 = n3 = n2 = n1 = 0;
         if (cnt >= 6) {
             n3 = (4 - (cnt & 3)) & 3;
             n4 = (cnt - 3 * n3) >> 2;
@@ -265,29 +265,51 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
             n3 = 1;
         } else if (cnt == 2) {
             n2 = 1;
-        } else {
+        } else if (cnt == 1) {
             n1 = 1;
         }
-        run(DcInt<4>{}, DcBool<false>{}, nb, tile0, n4, 0, KS);
-        run(DcInt<3>{}, DcBool<false>{}, nb, tile0 + 4 * n4, n3, 0, KS);
-        run(DcInt<2>{}, DcBool<false>{}, nb, tile0 + 4 * n4 + 3 * n3, n2, 0, KS);
-        run(DcInt<1>{}, DcBool<false>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1, 0, KS);
-        i += cnt;
+    };
+    const int nb_first = g_lo / p.tiles;
+    if (f > 0 && g_lo + 4 * f <= (nb_first + 1) * p.tiles) {   // uniform
+        const int t0 = g_lo - nb_first * p.tiles;
+        int n4, n3, n2, n1;
+        groups_of(f >> 1, n4, n3, n2, n1);
+        int base = t0;
+        run(DcInt<4>{}, DcBool<false>{}, nb_first, base + 4 * w, n4, 0, KS, 32);
+        base += 32 * n4;
+        run(DcInt<3>{}, DcBool<false>{}, nb_first, base + 3 * w, n3, 0, KS, 24);
+        base += 24 * n3;
+        run(DcInt<2>{}, DcBool<false>{}, nb_first, base + 2 * w, n2, 0, KS, 16);
+        base += 16 * n2;
+        run(DcInt<1>{}, DcBool<false>{}, nb_first, base + w, n1, 0, KS, 8);
+    } else {
+        int i = i_lo;
+        while (i < i_hi) {
+            const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
+            const int cnt = min(i_hi - i, p.tiles - tile0);
+            int n4, n3, n2, n1;
+            groups_of(cnt, n4, n3, n2, n1);
+            run(DcInt<4>{}, DcBool<false>{}, nb, tile0, n4, 0, KS, 4);
+            run(DcInt<3>{}, DcBool<false>{}, nb, tile0 + 4 * n4, n3, 0, KS, 3);
+            run(DcInt<2>{}, DcBool<false>{}, nb, tile0 + 4 * n4 + 3 * n3, n2, 0, KS, 2);
+            run(DcInt<1>{}, DcBool<false>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1, 0, KS, 1);
+            i += cnt;
+        }
     }
     // the workgroup's items left over (uniform over the workgroup: every wavefront meets the same barriers)
     const int part_idx = 2 * (w & 3) + (w >> 2);
     const int k_lo = KS * part_idx / 8, k_n = KS * (part_idx + 1) / 8 - k_lo;
-    i = g_lo + 4 * f;
+    int i = g_lo + 4 * f;
     while (i < g_hi) {
         const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
         // groups of sizes equal to within one tile (13 tiles: 4 + 3 + 3 + 3, not 4 + 4 + 4 + 1: a group of one tile pays the
         // first loads and the two barriers for a quarter of the work, with five loads per 16 MFMAs)
         const int run_len = min(g_hi - i, p.tiles - tile0), ngroups = (run_len + DC_SPLIT_T - 1) / DC_SPLIT_T;
         const int cnt = (run_len + ngroups - 1) / ngroups;
-        if (cnt == 4) run(DcInt<4>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
-        else if (cnt == 3) run(DcInt<3>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
-        else if (cnt == 2) run(DcInt<2>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
-        else run(DcInt<1>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n);
+        if (cnt == 4) run(DcInt<4>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n, 4);
+        else if (cnt == 3) run(DcInt<3>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n, 3);
+        else if (cnt == 2) run(DcInt<2>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n, 2);
+        else run(DcInt<1>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n, 1);
         i += cnt;
     }
 }
