@@ -94,6 +94,9 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     // `count` groups of T tiles each, from tile0 on, block nb of the produced channels, reduction steps [k_lo, k_lo + k_n)
     // of every group. SPLIT (count 1, every wavefront of the workgroup calls it with its own steps, k_n >= 0 of either
     // parity): the wavefronts' partial results are added through LDS. Otherwise k_n is even and at least 2.
+    int ep_nb = -1;   // the block of produced channels the epilogue terms below belong to
+    float sub[4], mul[4], add[4];
+    floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
     // The groups of a run begin `stride` tiles apart (T: one after the other).
     auto run = [&](auto tc, auto sp, const int nb, const int tile0, const int count, const int k_lo, const int k_n, const int stride) {
         constexpr int T = decltype(tc)::value;
@@ -102,18 +105,20 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         const int n_l = nb * 64 + 4 * l16;
         const unsigned b_lane = n_l < p.CO ? (unsigned)((4 * q * p.b_k + n_l) * 4) : DC_NEVER;
         const unsigned o_lane = n_l < p.CO ? (unsigned)((4 * q * p.CO + n_l) * 4) : DC_NEVER;
-        // the epilogue's per-channel terms: once per run, so that the loop below carries twelve registers, not the
-        // epilogue's pointers
-        float sub[4], mul[4], add[4];
-        floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
-        if (EPI) {
+        // the epilogue's per-channel terms: once per block of produced channels (they are loaded from memory and the loads
+        // are waited for), so that the loop below carries twelve registers, not the epilogue's pointers
+        if (nb != ep_nb) {
+            ep_nb = nb;
+            bias = floatx4{0.f, 0.f, 0.f, 0.f};
+            if (EPI) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                sub[j] = 0.f; mul[j] = 1.f; add[j] = 0.f;
-                if (n_l < p.CO && !p.ep.gate) ep_channel(p.ep, n_l + j, sub[j], mul[j], add[j]);
+                for (int j = 0; j < 4; j++) {
+                    sub[j] = 0.f; mul[j] = 1.f; add[j] = 0.f;
+                    if (n_l < p.CO && !p.ep.gate) ep_channel(p.ep, n_l + j, sub[j], mul[j], add[j]);
+                }
+            } else if (p.ep.bias != nullptr && n_l < p.CO) {
+                bias = *reinterpret_cast<const floatx4 *>(p.ep.bias + n_l);
             }
-        } else if (p.ep.bias != nullptr && n_l < p.CO) {
-            bias = *reinterpret_cast<const floatx4 *>(p.ep.bias + n_l);
         }
         floatx4 a[2][T], b[2][4];
         // ---- load cursor: one step ahead of the multiplications, through (group, tap, 16 channels) ----------------------
