@@ -8,7 +8,10 @@
 // tap 4g + q for output channel 4*l16 + j, j = 0..3; component s (the channel) of both feeds MFMA (s, j). A step is one
 // group g of four taps: one 128-bit load per tile and four for the filter, shared by the T <= 4 tiles a wavefront
 // owns, feed 16 T MFMAs (12 T when the fourth stored channel has zero weights everywhere: layers with three logical
-// channels). A lane's accumulators are 4 consecutive output channels of a pixel: results leave as 128-bit stores.
+// channels). The last tap (7x7 and 3x3 have 4 k + 1 taps) would fill a group on its own, three quarters of it padding:
+// in that step the reduction index is the CHANNEL instead - lane (l16, q) loads channel q of the last tap's pixel and of
+// the filter's last tap with 32-bit loads -, one MFMA per tile and j instead of three or four.
+// A lane's accumulators are 4 consecutive output channels of a pixel: results leave as 128-bit stores.
 // The filter is read as W[OC, FH, FW, 4] in place - its 4-channel taps are exactly the 16-byte units the lanes need - and
 // stays in L1 / L2 (64 channels of a 7x7 filter: 50 KB).
 //
@@ -85,10 +88,12 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
     unsigned need[G];
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        const int tap = 4 * g + q;
+        // the last group is the last tap alone (taps = 4 (G - 1) + 1, host-checked): there the reduction index of the MFMA
+        // is the CHANNEL, lane (l16, q) loads channel q of that tap's pixel - one MFMA per tile and j, not one per channel
+        const int tap = g < G - 1 ? 4 * g + q : 4 * g;
         const int fh = fdiv(tap, p.d_FW), fw = tap - fh * p.FW;
-        toff[g] = (fh * p.IW + fw) * 16;
-        need[g] = tap < p.taps ? (1u << fh) | (1u << (16 + fw)) : 0x80000000u;   // taps past the last: never inside
+        toff[g] = (fh * p.IW + fw) * 16 + (g < G - 1 ? 0 : 4 * q);
+        need[g] = (1u << fh) | (1u << (16 + fw));
     }
 
     // The tiles of group gidx. Where the rows are whole tiles (OW % 16 == 0) a group is the same 16 columns of four
@@ -114,7 +119,7 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
         unsigned b_voff[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) b_voff[j] = n_ok ? (unsigned)(((n_l + j) * p.taps + q) * 16) : SD_NEVER;
-        const bool last_tap_ok = 4 * (G - 1) + q < p.taps;
+        const bool last_ok = q < SC;   // the last step's channel q exists (with three channels the fourth is never read)
         const unsigned o_lane = n_ok ? (unsigned)((4 * q * p.OC + n_l) * 4) : SD_NEVER;
         float sub[4], mul[4], add[4];
         floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -179,10 +184,21 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
             if (c_inside) {   // uniform: one addition per tile (taps past the last, in the last group, stay out of range)
 #pragma unroll
                 for (int i = 0; i < T; i++)
-                    voff[i] = (g == G - 1 && !last_tap_ok) ? SD_NEVER : (unsigned)(org[i] + toff[g]);
+                    voff[i] = (g == G - 1 && !last_ok) ? SD_NEVER : (unsigned)(org[i] + toff[g]);
             } else {
 #pragma unroll
-                for (int i = 0; i < T; i++) voff[i] = (rc[i] & need[g]) == need[g] ? (unsigned)(org[i] + toff[g]) : SD_NEVER;
+                for (int i = 0; i < T; i++)
+                    voff[i] = ((rc[i] & need[g]) == need[g] && (g < G - 1 || last_ok)) ? (unsigned)(org[i] + toff[g]) : SD_NEVER;
+            }
+            if constexpr (g == G - 1) {   // one channel of the last tap per lane, into component 0
+#pragma unroll
+                for (int i = 0; i < T; i++) a[slot][i][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, voff[i], 0, 0));
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const unsigned bv = last_ok ? b_voff[j] - (unsigned)(12 * q) : SD_NEVER;   // tap 4 (G - 1) of the lane's channel, its component q
+                    b[slot][j][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, bv, g * 64, 0));
+                }
+                return;
             }
 #pragma unroll
             for (int i = 0; i < T; i++) {
@@ -191,15 +207,14 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
             }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const unsigned bv = (g == G - 1 && !last_tap_ok) ? SD_NEVER : b_voff[j];
-                if constexpr (SC == 3) b[slot][j] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(w_rsrc, bv, g * 64, 0));
-                else b[slot][j] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, bv, g * 64, 0));
+                if constexpr (SC == 3) b[slot][j] = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(w_rsrc, b_voff[j], g * 64, 0));
+                else b[slot][j] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, b_voff[j], g * 64, 0));
             }
         };
         floatx4 acc[T][4];
-        auto multiply = [&](int slot) {
+        auto multiply = [&](int slot, const int channels) {   // channels: SC, or 1 in the last step (component 0 = the lane's channel)
 #pragma unroll
-            for (int s = 0; s < SC; s++)
+            for (int s = 0; s < channels; s++)
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -227,7 +242,7 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
                         }
                         request((P + k + 1) & 1, SdInt<0>{});
                     }
-                    multiply((P + k) & 1);
+                    multiply((P + k) & 1, k < G - 1 ? SC : 1);
                     __builtin_amdgcn_sched_barrier(0);
                     self(SdInt<k + 1>{}, self);
                 }
@@ -291,12 +306,12 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
 }
 
 // Y[N, OH, OW, OC] = convolution of X[N, IH, IW, 4] with W[OC, FH, FW, 4] (stride sh x sw, padding ph x pw). Returns
-// hipErrorNotSupported (nothing launched) when the layer does not fit: a filter other than 3x3 or 7x7, tensors of 2 GB.
+// hipErrorNotSupported (nothing launched) when the layer does not fit: a filter of other than 49 or 9 taps, tensors of 2 GB.
 hipError_t launch_stem_direct(hipStream_t stream, const float *X, const float *W, float *Y, int N, int IH, int IW, int OH, int OW,
                               int OC, int FH, int FW, int sh, int sw, int ph, int pw, const float *bias, const Epilogue *ep)
 {
     const int taps = FH * FW, G = (taps + 3) / 4;
-    if ((G != 13 && G != 3) || FH > 15 || FW > 15 || OC < 4 || (OC & 3)) return hipErrorNotSupported;
+    if ((taps != 49 && taps != 9) || FH > 15 || FW > 15 || OC < 4 || (OC & 3)) return hipErrorNotSupported;   // 4 (G - 1) + 1 taps
     const long M = (long)N * OH * OW;
     const long x_bytes = (long)N * IH * IW * 16, w_bytes = (long)OC * taps * 16, y_bytes = M * OC * 4;
     if (M < 1 || x_bytes >= (1L << 31) || y_bytes >= (1L << 31) || w_bytes >= (1L << 30)) return hipErrorNotSupported;
