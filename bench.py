@@ -68,6 +68,16 @@ def algorithmic_bytes(layer):
     return 4.0 * (N * IH * IW * IC + OC * F * F * IC + N * OH * OW * OC)
 
 
+def touched_bytes(layer):
+    """As algorithmic_bytes, but of the input only the pixels a strided 1x1 filter reads (c4c: every second pixel of every
+    second row, a quarter of X); None where every input pixel is read."""
+    N, IH, IW, IC, OC, F, s, p, _, _ = LAYERS[layer]
+    if s <= F:
+        return None
+    OH, OW = out_dim(IH, F, s, p), out_dim(IW, F, s, p)
+    return 4.0 * (N * OH * OW * F * F * IC + OC * F * F * IC + N * OH * OW * OC)
+
+
 class Workload:
     """Device tensors of one layer plus closures that enqueue each operator the way the Java engine does."""
 
@@ -404,6 +414,10 @@ def measure(wl, op, steps, warmup, with_parity=True):
     # both fractions for every row, whichever roofline binds
     roof["mfma_frac"] = round(fl / (k_ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4)
     roof["hbm_frac"] = round(by / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+    if touched_bytes(layer) is not None and kind_of(op) == "fwd":
+        # a stride beyond the filter: forward reads only the pixels under the filter; both figures are stated
+        roof["touched_MB"] = round(touched_bytes(layer) / 1e6, 2)
+        roof["hbm_frac_touched"] = round(touched_bytes(layer) / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
     if op in ("wino", "dx_wino", "dw_wino"):
         roof["note"] = "Winograd: FLOPs credited are the direct convolution's (2.25x the multiplies executed); frac is not a roofline fraction"
         roof["executed_mfma_frac"] = round(roof["mfma_frac"] / 2.25, 4)
