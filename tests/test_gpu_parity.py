@@ -438,6 +438,10 @@ DIRECT_CONV_SHAPES = [
     (16, 14, 14, 256, 128, 3, 3, 1, 1, 1, 1),   # 392 items of 144 steps on 256 workgroups: one or two each
     (36, 7, 7, 512, 192, 3, 3, 1, 1, 1, 1),     # 333 items of 288 steps (ragged last tile), three blocks of produced channels
     (4, 9, 9, 256, 64, 5, 5, 2, 2, 2, 2),       # strided 5x5: 7 items of 400 steps on 7 workgroups
+    # short reductions (4 or 8 steps)
+    (48, 56, 56, 64, 128, 1, 1, 2, 2, 0, 0),    # c4c geometry: 4704 items of 4 steps = 18 or 19 per workgroup: 4 whole per SIMD + 2 or 3 shared
+    (24, 56, 56, 128, 64, 1, 1, 1, 1, 0, 0),    # 1x1 stride 1, 8 steps, 4704 items
+    (64, 64, 64, 16, 64, 2, 2, 2, 2, 0, 0),     # 2x2 taps x 16 channels = 4 steps, 4096 items = 16 per workgroup, all whole
 ]
 
 
