@@ -130,7 +130,7 @@ class Workload:
         N, IH, IW, IC, OC, F, s, p = self.dims
         cfg = self.engine.config
         cus = self.pkg.device_info()[0]
-        cfg.deltaW_SK_fillUnits = cus if op == "dw_fill" else 0
+        cfg.deltaW_SK_leastUnits = cus if op == "dw_least" else 0
         cfg.deltaW_winograd = cus if op == "dw_wino" else 0
         cfg.conv3D_winograd = 1 if op == "wino" else 0
         cfg.deltaX_winograd = 1 if op == "dx_wino" else 0
@@ -382,9 +382,9 @@ def kind_of(op):
 def measure(wl, op, steps, warmup, with_parity=True):
     pkg, torch, layer = wl.pkg, wl.torch, wl.layer
     wl.set_op(op)
-    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd, "fwd_bias": wl.fwd_bias, "fwd_fused": wl.fwd_fused, "dx": wl.dx_op, "dw": wl.dw, "dw_fill": wl.dw, "wino": wl.fwd,
+    step = {"fwd": wl.fwd, "fwd_cached": wl.fwd, "fwd_bias": wl.fwd_bias, "fwd_fused": wl.fwd_fused, "dx": wl.dx_op, "dw": wl.dw, "dw_least": wl.dw, "wino": wl.fwd,
             "dx_wino": wl.dx_op, "dw_wino": wl.dw}[op]
-    kernel = {"fwd": wl.fwd_conv, "fwd_cached": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "fwd_fused": wl.fwd_fused_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_fill": wl.dw_gemm,
+    kernel = {"fwd": wl.fwd_conv, "fwd_cached": wl.fwd_conv, "fwd_bias": wl.fwd_conv, "fwd_fused": wl.fwd_fused_conv, "dx": wl.dx, "dw": wl.dw_gemm, "dw_least": wl.dw_gemm,
               "wino": wl.wino_conv, "dx_wino": wl.dx_wino_conv, "dw_wino": wl.dw_wino_gemm}[op]
     N_, IH_, IW_, IC_, OC_, F_, s_, p_ = wl.dims
     if op in ("fwd", "fwd_bias", "fwd_cached", "fwd_fused"):
@@ -438,7 +438,7 @@ def layer_ops(layer):
     if "dx" in ops and F == 3 and s == 1:
         ops.append("dx_wino")
     if "dw" in ops:
-        ops.append("dw_fill")
+        ops.append("dw_least")
     if "dw" in ops and F == 3 and s == 1:
         ops.append("dw_wino")
     if layer == "c3a":
@@ -452,7 +452,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
-    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "fwd_fused", "dx", "dw", "dw_fill", "wino", "dx_wino", "dw_wino"],
+    ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "fwd_fused", "dx", "dw", "dw_least", "wino", "dx_wino", "dw_wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="accepted for compatibility: the layers array is part of the default line")
     ap.add_argument("--no-layers", action="store_true", help="leave out the array with every layer/op of BASELINE.json's configs")

@@ -9,6 +9,11 @@
 #include "../../include/alpha_engine.h"
 #include "winograd_limits.hpp"
 
+namespace alpha {
+// delta_w_stream.hip (host code): the least split-K factor with which the persistent backward-filter kernel cuts a layer as it does with GZ
+int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ);
+}
+
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -68,6 +73,7 @@ void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
     c->deltaX_winograd = 0;
     c->deltaW_winograd = 0;
     c->deltaW_SK_fillUnits = 0;
+    c->deltaW_SK_leastUnits = 0;
     c->cache_filter_transforms = 0;
 }
 
@@ -166,6 +172,8 @@ void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int
         if (want < 1) want = 1;
         GridZ = want;
     }
+    if (c->deltaW_SK_leastUnits > 0 && !winograd)
+        GridZ = alpha::deltaW_stream_least_GridZ(c->deltaW_SK_leastUnits, N, OH, OW, IC, OC, FH, FW, GridZ);
     out->GridZ = GridZ;
     out->scratch_floats = (long)OC * FH * FW * IC * (GridZ - 1);
     if (winograd) {

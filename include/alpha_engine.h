@@ -46,6 +46,10 @@ typedef struct alpha_engine_config {
     int deltaW_winograd;          /* this build only: > 0 = backward-filter of 3x3 stride-1 layers (split-K case) through Winograd
                                      F(3x3,2x2). 1: with the reference's GridZ; > 1: the number of compute units to fill - GridZ becomes
                                      that many workgroups' worth of slices (at least 64 tiles each). Default 0 */
+    int deltaW_SK_leastUnits;     /* this build only: > 0 = the number of compute units of the device; the split-K factor is then lowered
+                                     (never raised) to the least value with which the persistent backward-filter kernel cuts the layer
+                                     the same way - it deals the pixels evenly among the compute units whatever GridZ is, so a larger
+                                     GridZ only adds buffers of zeros for buf_summary to add. Default 0 = the reference's GridZ exactly */
 } alpha_engine_config;
 
 /* Native entry chosen by a plan; names are the Java native method names. */

@@ -105,6 +105,35 @@ def test_deltaW_fill_option_only_raises_the_split_k_factor():
     assert big == E.plan_deltaW(cfg, 14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1).GridZ
 
 
+def test_deltaW_least_option_only_lowers_the_split_k_factor():
+    """deltaW_SK_leastUnits is this build's option (no reference flag): the persistent backward-filter kernel cuts every
+    (tap, 64 x 64 block) item into R = floor(units / items) pieces whatever GridZ is (or the line of items into one share per
+    unit), so GridZ can come down to R (or to the most shares an item meets) without changing what the kernel does."""
+    cfg = E.default_config(256)
+    assert cfg.deltaW_SK_leastUnits == 0
+    cfg.deltaW_SK_leastUnits = 256
+    # c5b, c2a: 9 items -> 28 pieces each (reference: 128)
+    p = E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1)
+    assert p.GridZ == 28 and p.scratch_floats == 27 * 64 * 9 * 64 and p.entry_name == "dconv3D_deltaW_GemmSK"
+    assert E.plan_deltaW(cfg, 32, 32, 32, 32, 3, 3, 128, 64, 64, 1, 1).GridZ == 28
+    # c2b: 36 items -> 7 pieces (reference: 28); c5a / c5c: 4 items -> 64 (reference: 128)
+    assert E.plan_deltaW(cfg, 16, 16, 16, 16, 3, 3, 128, 128, 128, 1, 1).GridZ == 7
+    assert E.plan_deltaW(cfg, 56, 56, 56, 56, 1, 1, 32, 256, 64, 1, 1).GridZ == 64
+    assert E.plan_deltaW(cfg, 56, 56, 56, 56, 1, 1, 32, 64, 256, 1, 1).GridZ == 64
+    # c2c: 144 items form a line cut into 256 shares, an item meets 2 or 3 of them: the reference's 3 stays
+    assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 128, 256, 256, 1, 1).GridZ == 3
+    # never raised: 9 items on 256 units want 28, the reference gives 2 (GK = 512)
+    assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 8, 64, 64, 1, 1).GridZ == 2
+    # channel counts that fill the 64 x 64 blocks to less than 75 % go to other kernels: unchanged
+    cfg0 = E.default_config(256)
+    for shape in [(28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1), (14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1)]:
+        assert E.plan_deltaW(cfg, *shape).GridZ <= E.plan_deltaW(cfg0, *shape).GridZ
+    assert E.plan_deltaW(cfg, 28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1).GridZ == E.plan_deltaW(cfg0, 28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1).GridZ
+    # the Winograd option sets its own GridZ
+    cfg.deltaW_winograd = 256
+    assert E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).GridZ == 128
+
+
 def test_deltaX_plans():
     cfg = E.default_config(256)
     assert E.plan_deltaX(cfg, 224, 224, 112, 112, 7, 7, 64, 4, 64, 2, 2).entry_name == "dconv3D_deltaX_crossAdd"   # IC <= 8

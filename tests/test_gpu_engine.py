@@ -270,6 +270,37 @@ def test_engine_deltaW_with_fill_option(dev):
         e.close()
 
 
+@pytest.mark.parametrize("shape,least", [((32, 28, 64, 64, 3), 28),      # 9 items of (tap, 64 x 64 block): 28 pieces each on 256 units (reference: 39)
+                                         ((32, 28, 256, 64, 1), 64),     # 1x1: 4 items -> 64 pieces (reference: 98)
+                                         ((32, 16, 128, 128, 3), 7)])    # 36 items -> 7 pieces (reference: 28)
+def test_engine_deltaW_with_least_option(dev, shape, least):
+    """The least split-K factor the persistent kernel needs: the same result to the parity bar from fewer partial sums,
+    and bit-identical from run to run."""
+    N, IH, IC, OC, F_ = shape
+    p_ = F_ // 2
+    X, dY = normal((N, IH, IH, IC), 6111), normal((N, IH, IH, OC), 6112)
+    x, dy = dev.put(X), dev.put(dY)
+    want = O.deltaW_f64(X, dY, F_, F_, 1, 1, p_, p_)
+    units = pkg.device_info()[0]
+    e = pkg.engine.Engine(dev.stream)
+    try:
+        gz, got = [], []
+        for on in (0, units, units):
+            e.config.deltaW_SK_leastUnits = on
+            dw = dev.empty(OC, F_, F_, IC, fill=float("nan"))
+            p = e.dconv3D_deltaW(dw.data_ptr(), F_, F_, x.data_ptr(), IH, IH, dy.data_ptr(), IH, IH, N, IC, OC, 1, 1, p_, p_)
+            e.sync()
+            gz.append(p.GridZ)
+            got.append(dev.get(dw))
+            check(got[-1], want, "engine deltaW leastUnits=%d (GridZ %d) %s" % (on, p.GridZ, shape))
+        assert gz[1] <= gz[0] and gz[1] == gz[2]
+        if units == 256:
+            assert gz[1] == least, gz
+        assert np.array_equal(got[1], got[2])
+    finally:
+        e.close()
+
+
 def test_engine_scratch_is_recycled_after_sync(dev, eng):
     N, IH, IC, OC = 8, 16, 32, 64
     X, W = normal((N, IH, IH, IC), 6004), he_normal(OC, 3, 3, IC, 6005)
