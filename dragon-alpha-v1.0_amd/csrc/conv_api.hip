@@ -640,6 +640,11 @@ int alpha_dconv3D_deltaW_GemmSK_W1(const int64_t *streams, int length, int GridZ
 // alpha_dconv3D_deltaW_GemmSK followed by alpha_buf_summary: the results are bit-identical to that pair.
 // Every slice's kernel overwrites its whole partial tensor (empty slices write zeros), so nothing of an earlier call
 // is read. All calls on one device share the array: two calls whose work overlaps in time on one device race.
+int alpha_dconv3D_deltaW_least_GridZ(int units, int GridZ, int OH, int OW, int FH, int FW, int N, int IC, int OC)
+{
+    return deltaW_stream_least_GridZ(units, N, OH, OW, IC, OC, FH, FW, GridZ);
+}
+
 int alpha_dconv3D_deltaW_GemmSK_static(const int64_t *streams, int length, int GridZ, const float *X, int IH, int IW,
                                        const float *deltaY, int OH, int OW, float *deltaW, int FH, int FW,
                                        int N, int IC, int OC, int sh, int sw, int ph, int pw)

@@ -260,6 +260,16 @@ int alpha_dconv3D_deltaW_GemmSK_W1(const int64_t *streams, int length, int GridZ
                                    const float *deltaY, float *deltaW, float *deltaW_buf,
                                    int N, int IC, int OC);
 
+/* No counterpart in the reference (its split-K factor is the Java engine's choice,
+ * CudaFloat32EngineBase.java:1707-1715, sized for devices of at most 128 multiprocessors). The
+ * least GridZ' <= GridZ with which alpha_dconv3D_deltaW_GemmSK / _GemmV2SK / _GemmSK_W1 on a device
+ * of `units` compute units cut this layer exactly as they do with GridZ - their persistent kernel
+ * deals the pixels evenly among the compute units whatever GridZ is, and buffers beyond what it needs
+ * are only filled with zeros -, or GridZ itself for layers that kernel does not serve. A caller that
+ * passes the result instead of GridZ allocates and sums fewer partial results. Pure host arithmetic:
+ * no device is touched. */
+int alpha_dconv3D_deltaW_least_GridZ(int units, int GridZ, int OH, int OW, int FH, int FW, int N, int IC, int OC);
+
 /* No counterpart in the reference. For callers that cannot allocate device memory or hand over a
  * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * Same computation as alpha_dconv3D_deltaW_GemmSK followed by alpha_buf_summary(deltaW_buf, deltaW,

@@ -129,6 +129,12 @@ def test_deltaW_least_option_only_lowers_the_split_k_factor():
     for shape in [(28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1), (14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1)]:
         assert E.plan_deltaW(cfg, *shape).GridZ <= E.plan_deltaW(cfg0, *shape).GridZ
     assert E.plan_deltaW(cfg, 28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1).GridZ == E.plan_deltaW(cfg0, 28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1).GridZ
+    # the same arithmetic behind the C ABI, for a caller that chooses GridZ itself (units, GridZ, OH, OW, FH, FW, N, IC, OC)
+    L = pkg.lib()
+    assert L.alpha_dconv3D_deltaW_least_GridZ(256, 128, 56, 56, 3, 3, 32, 64, 64) == 28
+    assert L.alpha_dconv3D_deltaW_least_GridZ(256, 16, 56, 56, 3, 3, 32, 64, 64) == 16      # never raised
+    assert L.alpha_dconv3D_deltaW_least_GridZ(304, 128, 56, 56, 3, 3, 32, 64, 64) == 33     # another device width
+    assert L.alpha_dconv3D_deltaW_least_GridZ(256, 1, 56, 56, 3, 3, 32, 64, 64) == 1        # no split-K: nothing to lower
     # the Winograd option sets its own GridZ
     cfg.deltaW_winograd = 256
     assert E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).GridZ == 128
