@@ -4,16 +4,20 @@
 Default run: the headline workload of BASELINE.json's north_star — fp32 NHWC 3x3 stride-1 pad-1
 forward, N=64, 56x56x64 -> 64 (config "c3a") — called the way the reference's Java engine calls it
 (kernel_remode then the GemmR entry, both per step; CudaFloat32EngineBase.java:1363-1420), inputs
-resident in HBM. One "step" = one forward pass over that batch. Prints ONE JSON line.
+resident in HBM. One "step" = one forward pass over that batch.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--layer c3a] [--op fwd|dx|dw] [--no-layers] [--no-parity]
 
-The line also carries a "layers" array: every layer and operator of BASELINE.json's five configs (fewer iterations
-each), each row with its time, its roofline fraction and its parity against the fp64 CPU oracle on a subset of the
-same seeded tensors (images for forward / backward-data, output channels over the full batch for backward-filter),
-with the tolerance it is held to stated in the row. --no-layers leaves the array out.
-The cpu_baseline leg times the CPU oracle's float-accumulate direct convolution on a bounded batch
-subset of the same workload on the host cores (baseline only, never a target).
+Output: the LAST line of stdout is the result, one JSON object kept under 4 KB (headline figures, `roofline`, the
+headline's parity, `winograd`, `parity_summary`, `cpu_baseline` and `layers_min`: one short entry per layer and operator).
+Before it, every layer and operator of BASELINE.json's five configs is printed as a JSON line of its own, as soon as it
+is measured (same step count as the headline): its time, its roofline fractions and its parity against the fp64 CPU
+oracle on a subset of the same seeded tensors (images for forward / backward-data, output channels over the full batch
+for backward-filter), with the tolerance it is held to. The same rows go to gpurun_out/bench_layers.json as one array.
+--no-layers leaves them out.
+The cpu_baseline leg times the CPU oracle's float-accumulate direct loops on a bounded sample on the host cores
+(baseline only, never a target): the headline operator on all cores, backward-data and backward-filter of c5b on all
+cores, and config 1 forward on one core.
 """
 import argparse
 import json
@@ -270,13 +274,16 @@ def time_loop(torch, fn, steps, warmup):
     return wall_ms, e0.elapsed_time(e1) / steps
 
 
-def cpu_baseline(layer, op, budget_s=12.0):
-    """Times the oracle's float-accumulate direct convolution on a batch subset sized for ~budget_s."""
+def cpu_baseline(layer, op, budget_s=12.0, threads=None):
+    """Times the oracle's float-accumulate direct loops (forward: conv3D_f32acc, backward-data: deltaX_img2col,
+    backward-filter: deltaW_f32acc) on a batch subset sized for ~budget_s, on `threads` host threads (default: all)."""
     from oracle import oracle as O
     N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[layer]
     OH, OW = out_dim(IH, F, s, p), out_dim(IW, F, s, p)
     r = np.random.Generator(np.random.PCG64(7))
-    cores = O.num_threads()
+    all_cores = O.num_threads()
+    cores = all_cores if threads is None else threads
+    O.set_num_threads(cores)
 
     def run(n):
         X = r.standard_normal((n, IH, IW, IC)).astype(np.float32)
@@ -291,18 +298,20 @@ def cpu_baseline(layer, op, budget_s=12.0):
             O.deltaW_f32acc(X, dY, F, F, s, s, p, p)
         return time.perf_counter() - t0
 
-    per_image = flops(layer) / N
-    n0 = min(N, max(1, cores // 4))
-    t_probe = run(n0)
-    n = int(max(n0, min(N, n0 * budget_s / max(t_probe, 1e-6))))
-    t1 = run(n) if n > n0 else t_probe
-    n_used = n if n > n0 else n0
-    reps = int(max(1, min(5000, budget_s / max(t1, 1e-6))))   # repeat the subset until ~budget_s of CPU work is timed
-    t = sum(run(n_used) for _ in range(reps))
+    try:
+        per_image = flops(layer) / N
+        n0 = min(N, max(1, cores // 4))
+        t_probe = run(n0)
+        n = int(max(n0, min(N, n0 * budget_s / max(t_probe, 1e-6))))
+        t1 = run(n) if n > n0 else t_probe
+        n_used = n if n > n0 else n0
+        reps = int(max(1, min(5000, budget_s / max(t1, 1e-6))))   # repeat the subset until ~budget_s of CPU work is timed
+        t = sum(run(n_used) for _ in range(reps))
+    finally:
+        O.set_num_threads(all_cores)
     return {
         "value": round(per_image * n_used * reps / t / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-        "sample": "%s %s on %d of %d images x %d repeats (%.1f s total, OpenMP over n,oh; float accumulate, direct loops)"
-                  % (layer, op, n_used, N, reps, t),
+        "sample": "%s %s, %d of %d images x %d repeats, %.1f s; direct loops, fp32 accumulate, OpenMP" % (layer, op, n_used, N, reps, t),
     }
 
 
@@ -369,7 +378,8 @@ def parity(wl, op, step):
          "max_err_ratio": round(O.max_err_ratio(got, want, REL_TOL, tol_abs), 4),
          "max_err_ratio_at_abs_1e-5": round(O.max_err_ratio(got, want, REL_TOL, ABS_TOL), 4),
          "max_abs_err": float("%.3g" % float(np.max(np.abs(got.astype(np.float64) - want)))), "rms_expected": float("%.4g" % rms),
-         "samePercentRelative_1e-4": round(O.samePercentRelative(want.astype(np.float32), got, 1e-4), 6)}
+         "samePercentRelative_1e-4": round(O.samePercentRelative(want.astype(np.float32), got, 1e-4), 6),
+         "samePercentRelative_1e-5": round(O.samePercentRelative(want.astype(np.float32), got, 1e-5), 6)}
     r["ok"] = bool(r["max_err_ratio"] <= 1.0 and np.isfinite(got).all())
     r.update(extra)
     return r
@@ -446,6 +456,40 @@ def layer_ops(layer):
     return ops
 
 
+FINAL_LINE_LIMIT = 4096   # bytes; a harness that keeps only the tail of stdout must still see the whole result line
+
+
+def compact_parity(par):
+    """The few parity figures the result line keeps of a row's full parity record."""
+    if not par:
+        return None
+    keys = ("ok", "max_err_ratio", "max_err_ratio_at_abs_1e-5", "max_abs_err", "tol_rel", "tol_abs", "checked",
+            "samePercentRelative_1e-4", "samePercentRelative_1e-5", "bit_reproducible_run_to_run")
+    return {k: par[k] for k in keys if k in par}
+
+
+def layers_min(rows):
+    """One short entry per measured row: "layer/op": [kernel fraction of its binding roofline, operator ms, parity ok]."""
+    return {"%s/%s" % (r["layer"], r["op"]): [round(r["roofline"]["frac"], 3), round(r["ms_per_step"], 4),
+                                              (1 if r["parity"]["ok"] else 0) if "parity" in r else None] for r in rows}
+
+
+def result_line(out, rows):
+    """Serialises the result object with its per-row summary; sheds the optional parts, least important first, should the
+    line ever exceed FINAL_LINE_LIMIT."""
+    out = dict(out)
+    if rows:
+        out["layers_min"] = layers_min(rows)
+        out["layers_min_key"] = "layer/op: [kernel frac of its roofline, operator ms, parity ok]"
+    line = json.dumps(out, separators=(",", ":"))
+    for drop in ("layers_min_key", "winograd", "layers_min", "parity"):
+        if len(line) <= FINAL_LINE_LIMIT:
+            break
+        out.pop(drop, None)
+        line = json.dumps(out, separators=(",", ":"))
+    return line
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -460,9 +504,6 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--probe-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy a few times (calibrates FETCH_SIZE/WRITE_SIZE counters)")
-    ap.add_argument("--probe-lds", type=int, default=None, metavar="STRIDE_BYTES",
-                    help="only run a kernel of 128-bit LDS reads whose lanes are STRIDE_BYTES apart (puts the LDS counters of a "
-                         "known access pattern beside those of the real kernels); prints the time per read")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -478,28 +519,6 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"probe": "copy", "bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4}))
-        return
-    if args.probe_lds is not None:
-        import ctypes
-        here = os.path.dirname(os.path.abspath(__file__))
-        from __graft_entry__ import package
-        package().lib()   # maps the HIP runtime PyTorch ships before the probe library asks for one
-        probe = ctypes.CDLL(os.path.join(here, "dragon-alpha-v1.0_amd", "libalpha_probe.so"))
-        probe.alpha_probe_lds_read128.argtypes = [ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
-        blocks, iters = 256, 4096          # one workgroup of four wavefronts per compute unit, 32768 reads per wavefront
-        out = torch.empty(blocks * 256, dtype=torch.float32, device="cuda:0")
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-        times = []
-        for _ in range(5):
-            ev[0].record()
-            rc = probe.alpha_probe_lds_read128(torch.cuda.current_stream().cuda_stream, out.data_ptr(), args.probe_lds, iters, blocks)
-            assert rc == 0, rc
-            ev[1].record()
-            torch.cuda.synchronize()
-            times.append(ev[0].elapsed_time(ev[1]))
-        ms = min(times)
-        print(json.dumps({"probe": "lds_read128", "stride_bytes": args.probe_lds, "reads_per_wavefront": 8 * iters,
-                          "wavefronts_per_cu": 4, "ms": round(ms, 4), "ns_per_read_per_cu": round(ms * 1e6 / (8 * iters * 4), 3)}))
         return
     from __graft_entry__ import package
     pkg = package()
@@ -527,44 +546,58 @@ def main():
                    "layer": args.layer, "op": op, "gflop_per_step": head["gflop"],
                    "algorithmic_MB_per_step": head["algorithmic_MB"],
                    "frac_of_fp32_mfma_peak": round(head["tflops"] / PEAK_MFMA_F32_TFLOPS, 4),
-                   "tolerance": "rel 1e-4, abs 1e-5*max(1, rms(expected)) against the fp64 CPU oracle; each row's parity states its own "
-                                "figures, also against the literal abs 1e-5",
+                   "tolerance": "rel 1e-4, abs 1e-5*max(1, rms(expected)) vs the fp64 CPU oracle",
                    "clock_ramp_ms": CLOCK_RAMP_MS,   # untimed run-in of the same calls before the warmup steps of every measurement
                    "device": {"name": props.name, "cus": cus, "clock_ghz": round(clk_ghz, 3),
                               "fp32_mfma_peak_from_device_tflops": round(cus * 256 * clk_ghz / 1e3, 1)}},
         "roofline": head["roofline"],
     }
     if "parity" in head:
-        out["parity"] = head["parity"]
+        out["parity"] = compact_parity(head["parity"])
     if op == "fwd" and F == 3 and s == 1 and IC >= 16:
-        # the same layer through this build's second forward algorithm, in direct-convolution-equivalent FLOPs
+        # the same layer through this build's second forward algorithm, in direct-convolution-equivalent FLOPs (2.25x the
+        # multiplies executed; the executed-FLOP figure counts the 16 GEMMs only, not the transforms)
         wn = measure(wl, "wino", args.steps, args.warmup, with_parity=not args.no_parity)
         out["winograd"] = {"value": wn["tflops"], "unit": "TFLOP/s (direct-conv-equivalent)", "ms_per_step": wn["ms_per_step"],
                            "kernel_ms": wn["roofline"]["kernel_ms"], "kernel_tflops": wn["roofline"]["achieved"],
                            "direct_equivalent_over_fp32_mfma_peak": wn["roofline"]["frac"],
                            "executed_flop_frac_of_fp32_mfma_peak": round(wn["roofline"]["frac"] / 2.25, 4),
-                           "note": "Winograd F(2x2,3x3): 2.25x fewer multiplies than the FLOP count credited; the executed-FLOP figure "
-                                   "counts the 16 GEMMs only, not the transforms",
-                           "parity": wn.get("parity")}
+                           "parity": {k: v for k, v in (compact_parity(wn.get("parity")) or {}).items()
+                                      if k in ("ok", "max_err_ratio", "max_abs_err", "samePercentRelative_1e-4")} or None}
     wl.close()
     del wl
+    rows = []
     if not args.no_layers:
-        out["layers"] = []
-        lsteps, lwarm = max(5, args.steps // 5), max(2, args.warmup // 3)
         for layer in sorted(LAYERS):
             wl = Workload(pkg, torch, layer, seed_of(layer))
             for o in layer_ops(layer):
-                out["layers"].append(measure(wl, o, lsteps, lwarm, with_parity=not args.no_parity))
+                row = measure(wl, o, args.steps, args.warmup, with_parity=not args.no_parity)
+                rows.append(row)
+                print(json.dumps(row, separators=(",", ":")), flush=True)   # full row: a line of its own, before the result line
             wl.close()
             del wl
             torch.cuda.empty_cache()
-        rows = [r for r in out["layers"] if "parity" in r]
-        if rows:
-            out["parity_summary"] = {"rows": len(rows), "rows_ok": sum(1 for r in rows if r["parity"]["ok"]),
-                                     "worst_max_err_ratio": max(r["parity"]["max_err_ratio"] for r in rows),
-                                     "worst_max_err_ratio_at_abs_1e-5": max(r["parity"]["max_err_ratio_at_abs_1e-5"] for r in rows)}
-    out["cpu_baseline"] = None if args.no_cpu else cpu_baseline(args.layer, op)
-    print(json.dumps(out))
+        try:
+            os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+            with open(os.path.join(ROOT, "gpurun_out", "bench_layers.json"), "w") as f:
+                json.dump(rows, f, indent=1)
+        except OSError as e:
+            print("bench.py: could not write gpurun_out/bench_layers.json: %s" % e, file=sys.stderr)
+        checked = [r for r in rows if "parity" in r]
+        if checked:
+            out["parity_summary"] = {"rows": len(checked), "rows_ok": sum(1 for r in checked if r["parity"]["ok"]),
+                                     "worst_max_err_ratio": max(r["parity"]["max_err_ratio"] for r in checked),
+                                     "worst_max_err_ratio_at_abs_1e-5": max(r["parity"]["max_err_ratio_at_abs_1e-5"] for r in checked),
+                                     "least_samePercentRelative_1e-4": min(r["parity"]["samePercentRelative_1e-4"] for r in checked)}
+    if args.no_cpu:
+        out["cpu_baseline"] = None
+    else:
+        out["cpu_baseline"] = cpu_baseline(args.layer, op)
+        if args.layer == "c3a" and op == "fwd":   # the default run: a CPU figure beside the backward rows and config 1 on one core
+            out["cpu_baseline_dx"] = cpu_baseline("c5b", "dx", budget_s=5.0)
+            out["cpu_baseline_dw"] = cpu_baseline("c5b", "dw", budget_s=5.0)
+            out["cpu_baseline_c1_1core"] = cpu_baseline("c1", "fwd", budget_s=2.0, threads=1)
+    print(result_line(out, rows), flush=True)
 
 
 if __name__ == "__main__":

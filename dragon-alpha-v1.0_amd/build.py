@@ -11,8 +11,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libalpha_conv_hip.so")
-PROBE_SRC = os.path.join(HERE, "probe", "lds_probe.hip")      # measurement helper of bench.py --probe-lds, its own library
-PROBE_LIB = os.path.join(HERE, "libalpha_probe.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 FLAGS = [
@@ -49,7 +47,6 @@ def build(jobs=8, verbose=False):
     objs = [o for o, _ in results]
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     subprocess.check_call(cmd)
-    subprocess.check_call([HIPCC] + FLAGS + ["-shared", "-o", PROBE_LIB, PROBE_SRC], stderr=subprocess.DEVNULL)
     return LIB
 
 
