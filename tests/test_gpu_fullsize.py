@@ -151,3 +151,92 @@ def test_full_size_layer(dev, layer):
     # (3) run-to-run bit reproducibility of backward-filter (config 5)
     if dw2 is not None:
         assert torch.equal(dw, dw2), "%s: deltaW differs between two runs" % layer
+
+
+# ----------------------------------------------------------------------------------------------
+# The reference's own acceptance criterion on the kernels that serve the BASELINE layers, at full size and on the
+# reference's own data distribution: uniform [0,1) operands, Vector.samePercentRelative (|a-b| / |a+b| below the
+# threshold) against the CPU loops that add float products into a double (Tense.conv3D_naive,
+# deconv3D_deltaX_img2col, deconv3d_deltaW_naive):
+#   forward         threshold 1e-5, at least 99.9 % of the elements   (experiments/test_cuda/Cuda_conv3D_test.java:86-97)
+#   backward-data   threshold 1e-4, at least 99.9 %                   (Cuda_dconv3D_dX_test.java:93-100)
+#   backward-filter threshold 1e-5, 100 %                             (Cuda_dconv3D_dW_test.java:98-105)
+# The CPU side runs on whole images of the batch (forward, backward-data) and on the whole batch for a few output
+# channels (backward-filter: deltaW[oc] depends on deltaY[..., oc] only).
+# ----------------------------------------------------------------------------------------------
+def _uniform01(dev, shape, seed):
+    g = dev.torch.Generator(device="cpu").manual_seed(seed)
+    return dev.torch.rand(shape, generator=g)
+
+
+def _same_percent(got, want, thr, need, what):
+    pct = O.samePercentRelative(np.ascontiguousarray(want, dtype=np.float32), np.ascontiguousarray(got, dtype=np.float32), thr)
+    assert np.isfinite(got).all(), what
+    assert pct >= need, "%s: samePercentRelative(%g) = %.6f, the reference's test asks for %.4f" % (what, thr, pct, need)
+    return pct
+
+
+@pytest.mark.parametrize("layer,winograd", [("c3a", False), ("c3a", True), ("c3d", False)])
+def test_reference_criterion_forward_full_size(dev, layer, winograd):
+    torch = dev.torch
+    N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[layer]
+    OH, OW = out_dim(IH, IW, F, F, s, s, p, p)
+    X, W = _uniform01(dev, (N, IH, IW, IC), 8101), _uniform01(dev, (OC, F, F, IC), 8102)
+    x, w = X.to(dev.dev), W.to(dev.dev)
+    y = torch.full((N, OH, OW, OC), float("nan"), device=dev.dev)
+    eng = pkg.engine.Engine(dev.stream)
+    try:
+        eng.config.conv3D_winograd = 1 if winograd else 0
+        plan = eng.conv3D(y.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), F, F, N, IC, OC, s, s, p, p)
+        eng.sync()
+    finally:
+        eng.close()
+    assert (plan.entry_name == "conv3D_winograd") == winograd
+    imgs = sorted({0, N // 2, N - 1})
+    want = O.conv3D_naive(np.ascontiguousarray(X.numpy()[imgs]), W.numpy(), s, s, p, p)
+    _same_percent(y[imgs].cpu().numpy(), want, 1e-5, 0.999, "%s forward%s" % (layer, " (Winograd)" if winograd else ""))
+
+
+@pytest.mark.parametrize("layer,winograd", [("c5b", False), ("c5b", True), ("c5a", False), ("c5c", False)])
+def test_reference_criterion_deltaX_full_size(dev, layer, winograd):
+    torch = dev.torch
+    N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[layer]
+    OH, OW = out_dim(IH, IW, F, F, s, s, p, p)
+    dY, W = _uniform01(dev, (N, OH, OW, OC), 8103), _uniform01(dev, (OC, F, F, IC), 8104)
+    dy, w = dY.to(dev.dev), W.to(dev.dev)
+    dx = torch.full((N, IH, IW, IC), float("nan"), device=dev.dev)
+    eng = pkg.engine.Engine(dev.stream)
+    try:
+        eng.config.deltaX_winograd = 1 if winograd else 0
+        plan = eng.dconv3D_deltaX(dx.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), F, F, N, IC, OC, s, s, p, p)
+        eng.sync()
+    finally:
+        eng.close()
+    assert (plan.entry_name == "dconv3D_deltaX_winograd") == winograd
+    imgs = sorted({0, N - 1})
+    want = O.deltaX_img2col(np.ascontiguousarray(dY.numpy()[imgs]), W.numpy(), IH, IW, s, s, p, p)
+    _same_percent(dx[imgs].cpu().numpy(), want, 1e-4, 0.999, "%s deltaX%s" % (layer, " (Winograd)" if winograd else ""))
+
+
+@pytest.mark.parametrize("layer,mode", [("c5a", "direct"), ("c5b", "direct"), ("c5c", "direct"), ("c2c", "direct"), ("c2a", "direct"),
+                                        ("c5b", "least"), ("c5a", "least"), ("c5b", "winograd"), ("c2c", "winograd")])
+def test_reference_criterion_deltaW_full_size(dev, layer, mode):
+    torch = dev.torch
+    N, IH, IW, IC, OC, F, s, p, ICl, _ = LAYERS[layer]
+    OH, OW = out_dim(IH, IW, F, F, s, s, p, p)
+    X, dY = _uniform01(dev, (N, IH, IW, IC), 8105), _uniform01(dev, (N, OH, OW, OC), 8106)
+    x, dy = X.to(dev.dev), dY.to(dev.dev)
+    dw = torch.full((OC, F, F, IC), float("nan"), device=dev.dev)
+    eng = pkg.engine.Engine(dev.stream)
+    try:
+        cus = pkg.device_info()[0]
+        eng.config.deltaW_winograd = cus if mode == "winograd" else 0
+        eng.config.deltaW_SK_leastUnits = cus if mode == "least" else 0
+        plan = eng.dconv3D_deltaW(dw.data_ptr(), F, F, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, s, s, p, p)
+        eng.sync()
+    finally:
+        eng.close()
+    assert (plan.entry_name == "dconv3D_deltaW_GemmSK_winograd") == (mode == "winograd")
+    ocs = sorted({0, 1, OC // 2 + 1, OC - 1})
+    want = O.deltaW_naive(X.numpy(), np.ascontiguousarray(dY.numpy()[..., ocs]), F, F, s, s, p, p)
+    _same_percent(dw[ocs].cpu().numpy(), want, 1e-5, 1.0, "%s deltaW (%s, GridZ %d)" % (layer, mode, plan.GridZ))
