@@ -55,25 +55,23 @@ inline std::atomic<unsigned> &device_generation()
 }
 
 // The dynamic LDS limit is a property of (kernel, device): raise it the first time a device needs more than it has.
-// One instantiation, and so one table, per kernel. A racing first call sets the same value twice.
+// One instantiation, and so one table, per kernel. Each device's entry is one atomic word holding the generation it was
+// recorded in together with the bytes configured, so an entry recorded before a device reset never matches afterwards,
+// whichever thread looks first. A racing first call sets the same attribute twice.
 template <auto KERNEL>
 inline hipError_t ensure_dynamic_lds(size_t bytes)
 {
-    static size_t configured[64] = {0};
-    static unsigned seen_generation = 0;
-    const unsigned gen = device_generation().load(std::memory_order_acquire);
-    if (gen != seen_generation) {   // a device was reset since: every device's attribute is asked for again
-        for (size_t &c : configured) c = 0;
-        seen_generation = gen;
-    }
+    static std::atomic<uint64_t> configured[64];   // (generation << 32) | bytes; zero-initialised
+    const uint64_t gen = device_generation().load(std::memory_order_acquire);
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
-    if (bytes > configured[dev]) {
+    if (dev < 0 || dev >= 64 || bytes >= (1ull << 32)) return hipErrorInvalidDevice;
+    const uint64_t have = configured[dev].load(std::memory_order_acquire);
+    if ((have >> 32) != gen || bytes > (have & 0xffffffffull)) {
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (e != hipSuccess) return e;
-        configured[dev] = bytes;
+        configured[dev].store((gen << 32) | (uint64_t)bytes, std::memory_order_release);
     }
     return hipSuccess;
 }

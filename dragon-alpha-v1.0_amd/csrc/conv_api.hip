@@ -87,14 +87,29 @@ int fwd_algo()
 
 // Which 1x1 stride-1 kernel: the one without LDS (pointwise_direct.hip) re-reads the filter per group of tiles and per
 // block of 64 produced channels, the filter-resident one (pointwise.hip) stages it once per compute unit.
+// Measured on 32x56x56 pixels: 256 -> 64 channels 0.036 ms direct against 0.043 ms filter-resident; 64 -> 256 channels
+// 0.042 against 0.035 ms, and 256 -> 1024 on 64x14x14 pixels 0.089 against 0.068 ms: the direct kernel wins where one
+// block of 64 produced channels covers the output and the reduction is long. A debugging switch forces the choice
+// (alpha_conv_set_pointwise_algo, or ALPHA_PW_DIRECT=0/1 in the environment, read once per process): the parity tests
+// run both kernels on every shape.
+std::atomic<int> g_pw_algo{-2};   // -2: not yet read from the environment, -1: by shape, 0: filter-resident, 1: without LDS
+
+int pointwise_algo()
+{
+    int v = g_pw_algo.load(std::memory_order_relaxed);
+    if (v == -2) {
+        const char *e = getenv("ALPHA_PW_DIRECT");
+        v = e ? (atoi(e) != 0 ? 1 : 0) : -1;
+        int expected = -2;
+        if (!g_pw_algo.compare_exchange_strong(expected, v)) v = expected;   // a setter was quicker
+    }
+    return v;
+}
+
 bool pointwise_direct_preferred(int K, int N)
 {
-    // Measured on 32x56x56 pixels: 256 -> 64 channels 0.036 ms direct against 0.043 ms filter-resident; 64 -> 256 channels
-    // 0.042 against 0.035 ms, and 256 -> 1024 on 64x14x14 pixels 0.089 against 0.068 ms: the direct kernel wins where one
-    // block of 64 produced channels covers the output and the reduction is long. ALPHA_PW_DIRECT=0/1 forces the choice
-    // (the parity tests run both kernels on every shape).
-    const char *e = getenv("ALPHA_PW_DIRECT");
-    if (e) return atoi(e) != 0 && (K % 32) == 0;
+    const int forced = pointwise_algo();
+    if (forced >= 0) return forced != 0 && (K % 32) == 0;
     return (K % 32) == 0 && K >= 128 && N <= 64;
 }
 
@@ -452,6 +467,12 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz)
 }
 
 int alpha_conv_get_fwd_algo(void) { return fwd_algo(); }
+int alpha_conv_set_pointwise_algo(int algo)
+{
+    if (algo < -1 || algo > 1) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_pointwise_algo: algo must be -1, 0 or 1");
+    g_pw_algo.store(algo);
+    return 0;
+}
 int alpha_conv_set_fwd_algo(int algo)
 {
     if (algo < 0 || algo > 6) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..6");

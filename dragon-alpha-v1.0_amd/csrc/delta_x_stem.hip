@@ -41,7 +41,7 @@ struct DxStemArgs {
     Epilogue ep;
 };
 
-constexpr int DXS_RB = 8;          // coarse rows per block
+constexpr int DXS_RB_MAX = 8;      // coarse rows per block: 8, or 7 or 6 where that deals the blocks out more evenly
 constexpr int DXS_PS = 72;         // floats per halo pixel: 64 channels + 8 (conflict-free 128-bit reads at 288 bytes)
 constexpr int DXS_RS = 20;         // floats per pixel in the reduction buffer: 16 columns + 4
 constexpr unsigned DXS_NEVER = 0x80000000u;   // beyond any descriptor of this kernel (tensors are below 2 GB)
@@ -56,10 +56,10 @@ __device__ __forceinline__ void dxs_static_for(F &&f)
     }
 }
 
-template <int DH, int DW>
+template <int DH, int DW, int RB>
 __global__ __launch_bounds__(256, 2) void delta_x_stem_kernel(const DxStemArgs p)
 {
-    constexpr int RB = DXS_RB, HR = RB + DH - 1, HC = 16 + DW - 1, PS = DXS_PS, RS = DXS_RS;
+    constexpr int HR = RB + DH - 1, HC = 16 + DW - 1, PS = DXS_PS, RS = DXS_RS;
     constexpr int NE = HR * HC * 16;              // float4 elements of a halo
     constexpr int NI = (NE + 255) / 256;          // per thread
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -209,6 +209,8 @@ __global__ __launch_bounds__(256, 2) void delta_x_stem_kernel(const DxStemArgs p
     }
 }
 
+template <auto K> struct DxsKernel { static constexpr auto value = K; };
+
 // deltaX[N, IH, IW, 4] from deltaY[N, OH, OW, OC] and W[OC, FH, FW, 4]. Returns hipErrorNotSupported (nothing launched)
 // when the layer does not fit: IC != 4, a stride above 2, OC above 64 or not a multiple of 4, a window above 4 x 4.
 hipError_t launch_delta_x_stem(hipStream_t stream, const float *dY, const float *W, float *dX, int N, int IH, int IW, int IC,
@@ -241,30 +243,46 @@ hipError_t launch_delta_x_stem(hipStream_t stream, const float *dY, const float 
     if (DH > 4 || DW > 4) return hipErrorNotSupported;
     a.dmin_h = hmin; a.dmin_w = wmin;
     const int U = (IH + sh - 1) / sh, V = (IW + sw - 1) / sw;
-    const int nb_u = (U + DXS_RB - 1) / DXS_RB;
+    const int cus = device_cu_count();
+    if (cus < 1) return hipErrorNotSupported;
+    int grid = 2 * cus;
+    grid = (grid + 7) / 8 * 8;               // whole groups of 8: workgroup g runs on XCD g % 8
     a.nb_v = (V + 15) / 16;
+    // Rows per block: a workgroup's blocks cost whole rounds, so the block height that wastes the least of the last round
+    // wins (a block of RB rows costs about RB + 1: its halo has DH - 1 more rows to stage and its hand-over is fixed).
+    // 112 x 112 coarse pixels at N = 64 on 512 workgroups: 6272 blocks of 8 rows are 12.25 rounds (13 x 9 = 117), 7168
+    // blocks of 7 rows are 14 (14 x 8 = 112).
+    int RB = DXS_RB_MAX;
+    long best = -1;
+    for (int rb = DXS_RB_MAX; rb >= 6; rb--) {
+        const long blocks = (long)N * ((U + rb - 1) / rb) * a.nb_v;
+        const long cost = ((blocks + grid - 1) / grid) * (rb + 1);
+        if (best < 0 || cost < best) { best = cost; RB = rb; }
+    }
+    const int nb_u = (U + RB - 1) / RB;
     a.nb_uv = nb_u * a.nb_v;
     if ((long)N * a.nb_uv >= (1l << 30)) return hipErrorNotSupported;
     a.blocks = N * a.nb_uv;
     a.d_nbv = make_fastdiv(a.nb_v);
     a.d_nbuv = make_fastdiv(a.nb_uv);
-    const int cus = device_cu_count();
-    if (cus < 1) return hipErrorNotSupported;
-    int grid = 2 * cus;
-    grid = (grid + 7) / 8 * 8;               // whole groups of 8: workgroup g runs on XCD g % 8
     const bool small = DH <= 2 && DW <= 2;
-    const int HR = DXS_RB + (small ? 2 : 4) - 1, HC = 16 + (small ? 2 : 4) - 1;
+    const int HR = RB + (small ? 2 : 4) - 1, HC = 16 + (small ? 2 : 4) - 1;
     size_t lds = (size_t)HR * HC * DXS_PS * sizeof(float);
-    const size_t red = (size_t)4 * DXS_RB * 16 * DXS_RS * sizeof(float);
+    const size_t red = (size_t)4 * RB * 16 * DXS_RS * sizeof(float);
     if (lds < red) lds = red;
+    auto go = [&](auto kern) -> hipError_t {
+        if (hipError_t e = ensure_dynamic_lds<decltype(kern)::value>(lds); e != hipSuccess) return e;
+        hipLaunchKernelGGL(decltype(kern)::value, dim3(grid), dim3(256), lds, stream, a);
+        return hipGetLastError();
+    };
     if (small) {
-        if (hipError_t e = ensure_dynamic_lds<delta_x_stem_kernel<2, 2>>(lds); e != hipSuccess) return e;
-        hipLaunchKernelGGL((delta_x_stem_kernel<2, 2>), dim3(grid), dim3(256), lds, stream, a);
-    } else {
-        if (hipError_t e = ensure_dynamic_lds<delta_x_stem_kernel<4, 4>>(lds); e != hipSuccess) return e;
-        hipLaunchKernelGGL((delta_x_stem_kernel<4, 4>), dim3(grid), dim3(256), lds, stream, a);
+        if (RB == 8) return go(DxsKernel<delta_x_stem_kernel<2, 2, 8>>{});
+        if (RB == 7) return go(DxsKernel<delta_x_stem_kernel<2, 2, 7>>{});
+        return go(DxsKernel<delta_x_stem_kernel<2, 2, 6>>{});
     }
-    return hipGetLastError();
+    if (RB == 8) return go(DxsKernel<delta_x_stem_kernel<4, 4, 8>>{});
+    if (RB == 7) return go(DxsKernel<delta_x_stem_kernel<4, 4, 7>>{});
+    return go(DxsKernel<delta_x_stem_kernel<4, 4, 6>>{});
 }
 
 }  // namespace alpha

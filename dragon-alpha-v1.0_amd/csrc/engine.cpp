@@ -598,12 +598,17 @@ int alpha_engine_dconv3D_deltaW_deltaB(alpha_engine *e, float *deltaW, float *de
     }
     BlockScope scope{e};
     alpha_conv_plan p;
-    alpha_plan_deltaW(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+    // deltaW_SK_leastUnits lowers GridZ to what the persistent backward-filter kernel needs; with a bias gradient the
+    // library may serve the layer through a kernel that produces the column sums on the way and keeps the slice
+    // partition (1x1 layers, layers whose slices fill the device), which the lowered GridZ would leave under-filled:
+    // this operator always plans with the Java engine's GridZ.
+    alpha_engine_config cfg = e->cfg;
+    cfg.deltaW_SK_leastUnits = 0;
+    alpha_plan_deltaW(&cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
     if (p.entry == ALPHA_E_dconv3D_deltaW_GemmSK_winograd && (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2)) {
         // an output smaller than the formula's is legal for the engine but not for the Winograd kernel: the default plan
-        alpha_engine_config plain = e->cfg;
-        plain.deltaW_winograd = 0;
-        alpha_plan_deltaW(&plain, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
+        cfg.deltaW_winograd = 0;
+        alpha_plan_deltaW(&cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
     }
     if (plan_out) *plan_out = p;
     int64_t streams[16];

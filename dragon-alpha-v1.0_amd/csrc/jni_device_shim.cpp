@@ -180,7 +180,10 @@ static void fill_java_object(JNIEnv *env, jobject device, const alpha_device_pro
     const char *base = reinterpret_cast<const char *>(&props);
     for (const Field &f : FIELDS) {
         jfieldID id = env->GetFieldID(cls, f.name, f.sig);
-        if (id == nullptr) continue;   // a Java class without this field: the pending NoSuchFieldError is the JVM's to report
+        if (id == nullptr) {   // a Java class without this field (an older CudaDevice): the other fields are still filled
+            env->ExceptionClear();   // no JNI call may follow while the NoSuchFieldError is pending
+            continue;
+        }
         const char *src = base + f.offset;
         switch (f.kind) {
         case K_STRING: env->SetObjectField(device, id, env->NewStringUTF(src)); break;

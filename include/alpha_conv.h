@@ -58,6 +58,10 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz);
  * No counterpart in the reference (its Winograd experiments are compiled out, conv/conv3D.cuh:39-44). */
 int alpha_conv_set_fwd_algo(int algo);
 int alpha_conv_get_fwd_algo(void);
+/* Debugging switch of the same kind for 1x1 stride-1 forward / backward-data where the kernel of direct_conv.hip does not
+ * take the layer: -1 = chosen by shape, 0 = the filter-resident kernel, 1 = the kernel without LDS wherever it fits.
+ * Also read once from the environment variable ALPHA_PW_DIRECT = 0|1. No counterpart in the reference. */
+int alpha_conv_set_pointwise_algo(int algo);
 
 /* ---- Cuda_conv3D: forward ------------------------------------------------------------------ */
 

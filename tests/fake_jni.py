@@ -4,7 +4,10 @@ indices the JNI specification assigns them (6 FindClass, 14 ThrowNew, 17 Excepti
 200/203/204/205 Get{Byte,Int,Long,Float}ArrayRegion, 208/211/213 Set{Byte,Int,Float}ArrayRegion).
 A Java array is modelled as an integer key into a dict of Python lists; a jstring as a key into a dict of strings; a Java
 object (new_object) as a key into a dict of {field name: value} whose class declares a given set of (name, signature)
-fields - GetFieldID returns NULL for a field the class does not declare, or declares with another signature."""
+fields - GetFieldID returns NULL for a field the class does not declare, or declares with another signature, and
+leaves an exception pending as a JVM does (so does FindClass for an unknown class). The JNI specification allows only
+a handful of calls while an exception is pending (ExceptionClear among them): every other call made in that state is
+recorded in `calls_while_pending`, which a correct shim leaves empty."""
 import ctypes
 
 SLOT_COUNT = 235
@@ -16,6 +19,8 @@ class FakeEnv:
         self.thrown = []          # (class name, message)
         self.find_calls = []
         self.cleared = 0
+        self.pending = False              # an exception raised by a JNI call itself and not yet cleared
+        self.calls_while_pending = []     # names of JNI calls the specification forbids in that state
         self.known = {name: 0x1000 + i for i, name in enumerate(known_classes)}
         self._rev = {v: k for k, v in self.known.items()}
 
@@ -25,18 +30,29 @@ class FakeEnv:
         GETLONG = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32,
                                    ctypes.POINTER(ctypes.c_int64))
 
+        def guard(what):
+            if self.pending:
+                self.calls_while_pending.append(what)
+
         def find(env, name):
+            guard("FindClass")
             self.find_calls.append(name.decode())
-            return self.known.get(name.decode(), None)
+            got = self.known.get(name.decode(), None)
+            if got is None:
+                self.pending = True       # NoClassDefFoundError
+            return got
 
         def thrownew(env, cls, msg):
+            guard("ThrowNew")
             self.thrown.append((self._rev.get(cls, "?"), msg.decode()))
             return 0
 
         def clear(env):
             self.cleared += 1
+            self.pending = False
 
         def getlong(env, arr, start, n, buf):
+            guard("GetLongArrayRegion")
             src = self.arrays[arr]
             for i in range(n):
                 buf[i] = src[start + i]
@@ -47,11 +63,13 @@ class FakeEnv:
             proto = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctype))
 
             def get(env, arr, start, n, buf):      # Java array -> native buffer
+                guard("GetArrayRegion")
                 src = self.arrays[arr]
                 for i in range(n):
                     buf[i] = src[start + i]
 
             def put(env, arr, start, n, buf):      # native buffer -> Java array
+                guard("SetArrayRegion")
                 dst = self.arrays[arr]
                 for i in range(n):
                     dst[start + i] = buf[i]
@@ -62,11 +80,13 @@ class FakeEnv:
         NEWINTS = ctypes.CFUNCTYPE(ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32)
 
         def newstr(env, utf):
+            guard("NewStringUTF")
             key = 0x3000 + len(self.strings)
             self.strings[key] = utf.decode()
             return key
 
         def newints(env, n):
+            guard("NewIntArray")
             key = 0x2000 + len(self.arrays)
             self.arrays[key] = [0] * n
             return key
@@ -86,11 +106,14 @@ class FakeEnv:
         SETLONG = ctypes.CFUNCTYPE(None, V, V, V, ctypes.c_int64)
 
         def getcls(env, obj):
+            guard("GetObjectClass")
             return self.class_of[obj]
 
         def getfid(env, cls, name, sig):
+            guard("GetFieldID")
             name, sig = name.decode(), sig.decode()
             if self.declared[cls].get(name) != sig:
+                self.pending = True       # NoSuchFieldError
                 return None
             fid = 0x5000 + len(self.field_ids)
             self.field_ids[fid] = (name, sig)
@@ -98,6 +121,7 @@ class FakeEnv:
 
         def setter(kind, expect):
             def put(env, obj, fid, value):
+                guard("Set%sField" % kind)
                 name, sig = self.field_ids[fid]
                 assert sig in expect, "Set%sField on field %s of type %s" % (kind, name, sig)
                 self.set_calls.append((kind, name))
@@ -107,6 +131,7 @@ class FakeEnv:
             return put
 
         def newbytes(env, n):
+            guard("NewByteArray")
             key = 0x2000 + len(self.arrays)
             self.arrays[key] = [0] * n
             return key

@@ -1,5 +1,6 @@
 """GPU: the natives of one training step of a layer - kernel_remode, conv3D_GemmR, dconv3D_deltaX_s1,
-dconv3D_deltaW_GemmSK, buf_summary - recorded into a HIP graph and replayed. The natives only enqueue kernels on the
+dconv3D_deltaW_GemmSK, buf_summary, and the backward-filter entry that takes no workspace - recorded into a HIP graph and
+replayed. The natives only enqueue kernels on the
 stream they are given (conv/A.cu:149-171 and twins take the stream handles from Java and launch on them), allocate nothing
 and clear nothing with memset calls, so a caller may capture them; every replay, with fresh inputs copied into the same
 buffers and eager work of the program between the replays, is compared with the fp64 oracle.
@@ -48,6 +49,7 @@ def test_natives_replayed_from_a_graph(dev, shape):
     y = dev.empty(N, OH, OW, OC, fill=float("nan"))
     dx = dev.empty(N, IH, IW, IC, fill=float("nan"))
     dw = dev.empty(OC, F_, F_, IC, fill=float("nan"))
+    dw_static = dev.empty(OC, F_, F_, IC, fill=float("nan"))
     buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
 
     def step(stream):
@@ -59,6 +61,10 @@ def test_natives_replayed_from_a_graph(dev, shape):
         DW.dconv3D_deltaW_GemmSK(S, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dw.data_ptr(), buf.data_ptr(),
                                  F_, F_, N, IC, OC, s_, s_, p_, p_)
         DW.buf_summary(stream, buf.data_ptr(), dw.data_ptr(), GridZ - 1, sizeW)
+        # the entry that takes no workspace (partial sums in the library's static device array): capture refuses any
+        # allocation, so recording it here tests that it makes none
+        DW.dconv3D_deltaW_GemmSK_static(S, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dw_static.data_ptr(),
+                                        F_, F_, N, IC, OC, s_, s_, p_, p_)
 
     def fresh(seed):
         X, W, dY = normal((N, IH, IW, IC), seed), he_normal(OC, F_, F_, IC, seed + 1), normal((N, OH, OW, OC), seed + 2)
@@ -66,7 +72,7 @@ def test_natives_replayed_from_a_graph(dev, shape):
             X[..., 3] = 0.0
             W[..., 3] = 0.0
         x.copy_(dev.put(X)); w.copy_(dev.put(W)); dy.copy_(dev.put(dY))
-        for t in (cw, y, dx, dw, buf):
+        for t in (cw, y, dx, dw, dw_static, buf):
             t.fill_(float("nan"))
         return X, W, dY
 
@@ -76,6 +82,7 @@ def test_natives_replayed_from_a_graph(dev, shape):
         if with_dx:
             check(dx.cpu().numpy(), O.deltaX_f64(dY, W, IH, IW, s_, s_, p_, p_), "backward-data, %s %s" % (what, shape))
         check(dw.cpu().numpy(), O.deltaW_f64(X, dY, F_, F_, s_, s_, p_, p_), "backward-filter, %s %s" % (what, shape))
+        assert torch.equal(dw.view(torch.int32), dw_static.view(torch.int32)), "static-scratch backward-filter, %s %s" % (what, shape)
 
     side = torch.cuda.Stream()
     # eager first, on the stream that will capture: per-kernel attributes (dynamic LDS limits) are set on a kernel's first launch

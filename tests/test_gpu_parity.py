@@ -374,14 +374,14 @@ def test_pointwise_kernel_forward_and_deltaX(dev, shape):
         for algo in VARIANTS:
             L.alpha_conv_set_fwd_algo(algo if isinstance(algo, int) else 0)
             if not isinstance(algo, int):
-                os.environ["ALPHA_PW_DIRECT"] = "0" if algo == "resident" else "1"
+                L.alpha_conv_set_pointwise_algo(0 if algo == "resident" else 1)
             outs[algo] = (_run_fwd(dev, "conv3D_W1", X, W, 1, 1, 0, 0), _run_fwd(dev, "conv3D_GemmR_W1", X, W, 1, 1, 0, 0))
             dXo = dev.guarded(N, IH, IW, IC)
             dy, w = dev.put(dY), dev.put(W)
             DX.dconv3D_deltaX_W1(dev.streams, 1, dy.data_ptr(), w.data_ptr(), dXo.data_ptr(), IH, IW, N, IC, OC)
             outs[algo] += (dev.get(dXo),)
     finally:
-        os.environ.pop("ALPHA_PW_DIRECT", None)
+        L.alpha_conv_set_pointwise_algo(-1)
         L.alpha_conv_set_fwd_algo(0)
     for algo in VARIANTS:
         check(outs[algo][0], want_y, "conv3D_W1 algo %s %s" % (algo, shape))

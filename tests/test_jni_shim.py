@@ -61,6 +61,7 @@ def test_error_becomes_java_exception_and_streams_are_copied():
     assert env2.find_calls == ["z/dragon/engine/cuda/impl/CudaException", "z/jcuda/exception/CudaException",
                                "java/lang/RuntimeException"]
     assert env2.cleared == 2 and env2.thrown[0][0] == "java/lang/RuntimeException"
+    assert env2.calls_while_pending == []   # each failed FindClass is cleared before the next JNI call
     # an empty stream array is refused, not dereferenced
     env3 = FakeEnv()
     fn(env3.ptr, None, env3.long_array([]), 0, 256, 8, 8, 256, 3, 3, 256, 8, 8, 4, 4, 8, 1, 1, 1, 1)
@@ -198,6 +199,8 @@ def test_device_properties_reach_every_java_field_with_its_type():
     obj2 = env.new_object(fewer)
     fn(env.ptr, obj2, ctypes.byref(props))
     assert sorted(env.objects[obj2]) == sorted(fewer)
+    # the NoSuchFieldError that GetFieldID leaves pending is cleared before the next JNI call
+    assert env.calls_while_pending == [] and not env.pending
 
 
 @pytest.mark.gpu

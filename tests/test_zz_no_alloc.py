@@ -38,12 +38,22 @@ def test_static_scratch_entry_equals_the_workspace_entry_on_consecutive_calls():
                                  FH, FW, N, IC, OC, sh, sw, ph, pw)
         DW.buf_summary(dev.stream, buf.data_ptr(), ref.data_ptr(), GridZ - 1, sizeW)
         want = dev.get(ref)
-        # the entry under test, with allocation made impossible to miss: the caching allocator's counters must not move
+        # the entry under test. Device memory as the driver counts it (hipMemGetInfo: it sees an allocation made by any
+        # library of the process, which the counters of PyTorch's caching allocator do not) must not move across the
+        # call; the first call of the process resolves the static array's address and may load code, so it is made once
+        # before the one that is measured.
         got_t = dev.guarded(OC, FH, FW, IC)
+        if i == 0:
+            DW.dconv3D_deltaW_GemmSK_static(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, got_t.data_ptr(),
+                                            FH, FW, N, IC, OC, sh, sw, ph, pw)
+            got_t.fill_(float("nan"))
         dev.sync()
+        free_before = torch.cuda.mem_get_info()[0]
         before = torch.cuda.memory_stats()["allocation.all.allocated"]
         DW.dconv3D_deltaW_GemmSK_static(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, got_t.data_ptr(),
                                         FH, FW, N, IC, OC, sh, sw, ph, pw)
+        dev.sync()
+        assert torch.cuda.mem_get_info()[0] == free_before, "device memory in use changed across the call"
         assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
         got = dev.get(got_t)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "call %d differs from GemmSK + buf_summary" % i
