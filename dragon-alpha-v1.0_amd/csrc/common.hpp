@@ -319,4 +319,13 @@ hipError_t launch_buf_summary(hipStream_t s, const float *buf, float *dW, int pa
 // Column sums of deltaY[GK][OC] per K slice (bias gradient), same slice partition and destinations as backward-filter.
 hipError_t launch_col_sum(hipStream_t s, const float *dY, float *dB, float *dB_buf, int OC, int GK, int GK_slice, int GZ);
 
+// Backward of batch normalisation (batchnorm_backward.hip). form: 0 = X_norm given in S, 1 = X_norm = (S - B) / A,
+// 2 = X_norm = (S - mean) * rsqrt(var + eps). Field sums: deltaA = sum_n deltaY * X_norm, deltaB = sum_n deltaY per column.
+int bn_field_nextN(int N, int M);
+hipError_t launch_bn_field_sums(hipStream_t s, int form, const float *dY, const float *S, const float *mean, const float *var, float eps,
+                                const float *A, const float *B, int N, int M, float *bufA, float *outA, float *bufB, float *outB, int width);
+hipError_t launch_bn_delta_x(hipStream_t s, int form, bool affine, const float *dY, const float *S, const float *mean, const float *var,
+                             float eps, const float *A, const float *B, const float *p1, const float *p2, int row_lengthv, float *dX,
+                             long lengthv, int width);
+
 }  // namespace alpha

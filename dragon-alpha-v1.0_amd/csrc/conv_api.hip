@@ -898,5 +898,104 @@ int alpha_batchNorm_affined2D_row(int64_t stream, const float *X, const float *X
     return row_function(__func__, stream, X, Y, ep, lengthv, mem_width, mem_stride);
 }
 
+// ---- backward of batch normalisation: the field sums and the row functions ------------------------------------------
+namespace {
+int bn_sums(const char *fn, int64_t stream1, int form, const float *deltaY, const float *S, const float *mean, const float *var, float eps,
+            const float *A, const float *B, int N, int M, float *deltaA_buf, float *deltaA, float *deltaB_buf, float *deltaB,
+            int mem_width, int mem_stride, int partNum, int *nextN)
+{
+    if (!deltaY || !S || !deltaA || !deltaB || !aligned16(deltaY) || !aligned16(S) || !aligned16(deltaA) || !aligned16(deltaB) ||
+        !aligned16(deltaA_buf) || !aligned16(deltaB_buf) || !aligned16(mean) || !aligned16(var) || !aligned16(A) || !aligned16(B))
+        return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
+    if (N < 1 || M < 4 || (M & 3) || mem_stride < 4 || (mem_stride & 3) || mem_width < 1 || mem_width > mem_stride || M % mem_stride != 0)
+        return fail(ALPHA_CONV_EINVAL, "%s: need N >= 1, M a multiple of mem_stride, mem_stride a multiple of 4, 1 <= mem_width <= mem_stride", fn);
+    if (M != mem_stride) return fail(ALPHA_CONV_EINVAL, "%s: rows of more than one mem_stride are not supported", fn);
+    if ((long)N * M >= (1L << 31)) return fail(ALPHA_CONV_EINVAL, "%s: tensor exceeds 2^31 elements", fn);
+    if (partNum < 1) partNum = 1;
+    int n = bn_field_nextN(N, M);
+    if (n > partNum && (!deltaA_buf || !deltaB_buf)) return fail(ALPHA_CONV_EINVAL, "%s: buffers are null", fn);
+    if (int e = hip_status(launch_bn_field_sums(reinterpret_cast<hipStream_t>((intptr_t)stream1), form, deltaY, S, mean, var, eps, A, B, N, M,
+                                                n > partNum ? deltaA_buf : nullptr, deltaA, n > partNum ? deltaB_buf : nullptr, deltaB, mem_width), fn))
+        return e;
+    // the value the reference returns: rows left after its last stage (Cuda_reduce field_*_deltaAB: "return nextN")
+    while (n > partNum) {
+        const int next = bn_field_nextN(n, M);
+        if (next >= n) break;
+        n = next;
+    }
+    if (nextN) *nextN = n;
+    return 0;
+}
+
+int bn_dx(const char *fn, int64_t stream, int form, bool affine, const float *deltaY, const float *S, const float *mean, const float *var,
+          float eps, const float *A, const float *B, const float *p1, const float *p2, int row_lengthv, float *deltaX, int lengthv,
+          int mem_width, int mem_stride)
+{
+    if (!deltaY || !S || !var || !p1 || !p2 || !deltaX || !aligned16(deltaY) || !aligned16(S) || !aligned16(var) || !aligned16(p1) ||
+        !aligned16(p2) || !aligned16(deltaX) || !aligned16(mean) || !aligned16(A) || !aligned16(B))
+        return fail(ALPHA_CONV_EINVAL, "%s: null or misaligned pointer", fn);
+    if (lengthv < 0 || mem_stride < 4 || (mem_stride & 3) || mem_width < 1 || mem_width > mem_stride || lengthv % mem_stride != 0)
+        return fail(ALPHA_CONV_EINVAL, "%s: need lengthv = height * mem_stride, mem_stride a multiple of 4, 1 <= mem_width <= mem_stride", fn);
+    if (row_lengthv != mem_stride) return fail(ALPHA_CONV_EINVAL, "%s: row_lengthv must equal mem_stride", fn);
+    return hip_status(launch_bn_delta_x(reinterpret_cast<hipStream_t>((intptr_t)stream), form, affine, deltaY, S, mean, var, eps, A, B, p1, p2,
+                                        row_lengthv, deltaX, lengthv, mem_width), fn);
+}
+}  // namespace
+
+int alpha_field_affine_deltaAB_v1(int64_t stream1, int64_t stream2, const float *deltaY, const float *Y, const float *A, const float *B,
+                                  int N, int M, float *deltaA_buf, float *deltaA, float *deltaB_buf, float *deltaB,
+                                  int mem_width, int mem_stride, int partNum, int *nextN)
+{
+    (void)stream2;   // everything is ordered on stream1; the caller records its event on both streams
+    CHECK_PTR(A);
+    CHECK_PTR(B);
+    return bn_sums(__func__, stream1, 1, deltaY, Y, nullptr, nullptr, 0.f, A, B, N, M, deltaA_buf, deltaA, deltaB_buf, deltaB, mem_width, mem_stride, partNum, nextN);
+}
+int alpha_field_affine_deltaAB_v2(int64_t stream1, int64_t stream2, const float *deltaY, const float *X_norm,
+                                  int N, int M, float *deltaA_buf, float *deltaA, float *deltaB_buf, float *deltaB,
+                                  int mem_width, int mem_stride, int partNum, int *nextN)
+{
+    (void)stream2;
+    return bn_sums(__func__, stream1, 0, deltaY, X_norm, nullptr, nullptr, 0.f, nullptr, nullptr, N, M, deltaA_buf, deltaA, deltaB_buf, deltaB, mem_width, mem_stride, partNum, nextN);
+}
+int alpha_field_batchNorm_deltaAB_v2(int64_t stream1, int64_t stream2, const float *deltaY, const float *X, const float *X_mean,
+                                     const float *X_var, float eps, int N, int M, float *deltaA_buf, float *deltaA,
+                                     float *deltaB_buf, float *deltaB, int mem_width, int mem_stride, int partNum, int *nextN)
+{
+    (void)stream2;
+    CHECK_PTR(X_mean);
+    CHECK_PTR(X_var);
+    return bn_sums(__func__, stream1, 2, deltaY, X, X_mean, X_var, eps, nullptr, nullptr, N, M, deltaA_buf, deltaA, deltaB_buf, deltaB, mem_width, mem_stride, partNum, nextN);
+}
+int alpha_batchNorm2D_row_deltaX_v1(int64_t stream, const float *deltaY, const float *Y, const float *X_var, float eps,
+                                    const float *deltaXp1, const float *deltaXp2, int row_lengthv, float *deltaX,
+                                    int lengthv, int mem_width, int mem_stride)
+{
+    return bn_dx(__func__, stream, 0, false, deltaY, Y, nullptr, X_var, eps, nullptr, nullptr, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv, mem_width, mem_stride);
+}
+int alpha_batchNorm2D_row_deltaX_v2(int64_t stream, const float *deltaY, const float *X, const float *X_mean, const float *X_var, float eps,
+                                    const float *deltaXp1, const float *deltaXp2, int row_lengthv, float *deltaX,
+                                    int lengthv, int mem_width, int mem_stride)
+{
+    CHECK_PTR(X_mean);
+    return bn_dx(__func__, stream, 2, false, deltaY, X, X_mean, X_var, eps, nullptr, nullptr, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv, mem_width, mem_stride);
+}
+int alpha_batchNorm_affined2D_row_deltaX_v1(int64_t stream, const float *deltaY, const float *Y, const float *X_var, float eps,
+                                            const float *A, const float *B, const float *deltaXp1, const float *deltaXp2,
+                                            int row_lengthv, float *deltaX, int lengthv, int mem_width, int mem_stride)
+{
+    CHECK_PTR(A);
+    CHECK_PTR(B);
+    return bn_dx(__func__, stream, 1, true, deltaY, Y, nullptr, X_var, eps, A, B, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv, mem_width, mem_stride);
+}
+int alpha_batchNorm_affined2D_row_deltaX_v2(int64_t stream, const float *deltaY, const float *X, const float *X_mean, const float *X_var,
+                                            float eps, const float *A, const float *deltaXp1, const float *deltaXp2,
+                                            int row_lengthv, float *deltaX, int lengthv, int mem_width, int mem_stride)
+{
+    CHECK_PTR(X_mean);
+    CHECK_PTR(A);
+    return bn_dx(__func__, stream, 2, true, deltaY, X, X_mean, X_var, eps, A, nullptr, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv, mem_width, mem_stride);
+}
+
 }  // extern "C"
 #pragma GCC visibility pop

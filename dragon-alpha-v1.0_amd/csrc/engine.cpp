@@ -630,6 +630,68 @@ int alpha_engine_dconv3D_deltaW_deltaB(alpha_engine *e, float *deltaW, float *de
     return 0;
 }
 
+// Backward of batch normalisation: CudaFloat32EngineBase.batchNorm2D_deltaX_v1 / _v2 (:4385-4475, affine :4478-4576) and
+// batchNorm2D_gradients_v1 / _v2 (:4648-4760). Stage 1: the field sums deltaXp1 = sum deltaY, deltaXp2 = sum deltaY * X_norm
+// (into deltaB / deltaA when the caller wants them - the gradients forms -, else into scratch); stage 2: the row function.
+// The Java engine runs stage 1 on two streams and joins them with an event; here one stream orders everything.
+static int bn_backward(alpha_engine *e, const char *what, bool from_x, float *deltaX, const float *deltaY, const float *S,
+                       const float *X_mean, const float *X_var, float eps, const float *A, const float *B, float *deltaA, float *deltaB,
+                       int field_length, int row_lengthv, int lengthv, int width, int stride)
+{
+    if (field_length < 1 || row_lengthv < 4 || (long)field_length * row_lengthv != lengthv) {
+        snprintf(e->err, sizeof(e->err), "%s: need lengthv = field_length * row_lengthv", what);
+        return ALPHA_CONV_EINVAL;
+    }
+    BlockScope scope{e};
+    const int M = row_lengthv;
+    // buffers as the Java engine sizes them: nextN x M floats each (Cuda_reduce.field_nextN), with the sums at their heads
+    // when the caller does not ask for them
+    int nextN = (M > 15 && field_length > 63) ? field_length >> 6 : (M > 15 && field_length > 15) ? 1
+              : (M > 7 && field_length > 127) ? field_length >> 7 : (M > 7 && field_length > 31) ? 1 : (field_length + 63) >> 6;
+    if (nextN < 1) nextN = 1;
+    float *buf = static_cast<float *>(take_block(e, (size_t)2 * nextN * M * sizeof(float)));
+    if (!buf) return fail(e, -1, what);
+    float *bufB = buf, *bufA = buf + (size_t)nextN * M;
+    float *p1 = deltaB ? deltaB : bufB, *p2 = deltaA ? deltaA : bufA;
+    int rc;
+    if (from_x) rc = alpha_field_batchNorm_deltaAB_v2(e->stream, e->stream, deltaY, S, X_mean, X_var, eps, field_length, M, bufA, p2, bufB, p1, width, stride, 1, nullptr);
+    else if (A) rc = alpha_field_affine_deltaAB_v1(e->stream, e->stream, deltaY, S, A, B, field_length, M, bufA, p2, bufB, p1, width, stride, 1, nullptr);
+    else rc = alpha_field_affine_deltaAB_v2(e->stream, e->stream, deltaY, S, field_length, M, bufA, p2, bufB, p1, width, stride, 1, nullptr);
+    if (rc) return fail(e, rc, what);
+    if (from_x) {
+        rc = A ? alpha_batchNorm_affined2D_row_deltaX_v2(e->stream, deltaY, S, X_mean, X_var, eps, A, p1, p2, M, deltaX, lengthv, width, stride)
+               : alpha_batchNorm2D_row_deltaX_v2(e->stream, deltaY, S, X_mean, X_var, eps, p1, p2, M, deltaX, lengthv, width, stride);
+    } else {
+        rc = A ? alpha_batchNorm_affined2D_row_deltaX_v1(e->stream, deltaY, S, X_var, eps, A, B, p1, p2, M, deltaX, lengthv, width, stride)
+               : alpha_batchNorm2D_row_deltaX_v1(e->stream, deltaY, S, X_var, eps, p1, p2, M, deltaX, lengthv, width, stride);
+    }
+    return rc ? fail(e, rc, what) : 0;
+}
+
+int alpha_engine_batchNorm2D_deltaX_v1(alpha_engine *e, float *deltaX, const float *deltaY, const float *Y, const float *X_var, float eps,
+                                       const float *A, const float *B, float *deltaA, float *deltaB,
+                                       int field_length, int row_lengthv, int lengthv, int width, int stride)
+{
+    if ((A == nullptr) != (B == nullptr) || (!A && (deltaA || deltaB)) || (deltaA == nullptr) != (deltaB == nullptr)) {
+        snprintf(e->err, sizeof(e->err), "alpha_engine_batchNorm2D_deltaX_v1: A and B go together, deltaA and deltaB go together and need A");
+        return ALPHA_CONV_EINVAL;
+    }
+    return bn_backward(e, "batchNorm2D_deltaX_v1", false, deltaX, deltaY, Y, nullptr, X_var, eps, A, B, deltaA, deltaB,
+                       field_length, row_lengthv, lengthv, width, stride);
+}
+
+int alpha_engine_batchNorm2D_deltaX_v2(alpha_engine *e, float *deltaX, const float *deltaY, const float *X, const float *X_mean,
+                                       const float *X_var, float eps, const float *A, float *deltaA, float *deltaB,
+                                       int field_length, int row_lengthv, int lengthv, int width, int stride)
+{
+    if ((!A && (deltaA || deltaB)) || (deltaA == nullptr) != (deltaB == nullptr)) {
+        snprintf(e->err, sizeof(e->err), "alpha_engine_batchNorm2D_deltaX_v2: deltaA and deltaB go together and need A");
+        return ALPHA_CONV_EINVAL;
+    }
+    return bn_backward(e, "batchNorm2D_deltaX_v2", true, deltaX, deltaY, X, X_mean, X_var, eps, A, nullptr, deltaA, deltaB,
+                       field_length, row_lengthv, lengthv, width, stride);
+}
+
 // Xf != NULL: deltaX is multiplied by the derivative of the leaky ReLU (slope k) whose output Xf is this layer's input - in
 // the kernel's epilogue for the stride-1 entries, by leakyRelu2D_deltaX_v1 in place after the others.
 static int deltaX_impl(alpha_engine *e, const char *what, float *deltaX, int IH, int IW, const float *deltaY, int OH, int OW,

@@ -82,6 +82,9 @@ def _lib():
                                                 + [ctypes.POINTER(native.Epilogue), ctypes.POINTER(Plan)])
         L.alpha_engine_dconv3D_deltaX_leakyRelu.argtypes = ([_P, _P, _I, _I, _P, _I, _I, _P, _I, _I] + [_I] * 7
                                                             + [_P, ctypes.c_float, ctypes.POINTER(Plan)])
+        F = ctypes.c_float
+        L.alpha_engine_batchNorm2D_deltaX_v1.argtypes = [_P, _P, _P, _P, _P, F, _P, _P, _P, _P] + [_I] * 5
+        L.alpha_engine_batchNorm2D_deltaX_v2.argtypes = [_P, _P, _P, _P, _P, _P, F, _P, _P, _P] + [_I] * 5
         _bound = True
     return L
 
@@ -171,6 +174,18 @@ class Engine:
         self._check(self._L.alpha_engine_dconv3D_deltaX_leakyRelu(self._h, deltaX, IH, IW, deltaY, OH, OW, W, FH, FW, N, IC, OC,
                                                                   sh, sw, ph, pw, Xf, k, ctypes.byref(p)))
         return p
+
+    def batchNorm2D_deltaX_v1(self, deltaX, deltaY, Y, X_var, eps, field_length, row_lengthv, lengthv, width, stride,
+                              A=None, B=None, deltaA=None, deltaB=None):
+        """EngineBase.batchNorm2D_deltaX_v1 (A is None: not affine); with deltaA / deltaB: batchNorm2D_gradients_v1."""
+        self._check(self._L.alpha_engine_batchNorm2D_deltaX_v1(self._h, deltaX, deltaY, Y, X_var, eps, A, B, deltaA, deltaB,
+                                                               field_length, row_lengthv, lengthv, width, stride))
+
+    def batchNorm2D_deltaX_v2(self, deltaX, deltaY, X, X_mean, X_var, eps, field_length, row_lengthv, lengthv, width, stride,
+                              A=None, deltaA=None, deltaB=None):
+        """EngineBase.batchNorm2D_deltaX_v2 (A is None: not affine); with deltaA / deltaB: batchNorm2D_gradients_v2."""
+        self._check(self._L.alpha_engine_batchNorm2D_deltaX_v2(self._h, deltaX, deltaY, X, X_mean, X_var, eps, A, deltaA, deltaB,
+                                                               field_length, row_lengthv, lengthv, width, stride))
 
     def dconv3D_deltaW(self, deltaW, FH, FW, X, IH, IW, deltaY, OH, OW, N, IC, OC, sh, sw, ph, pw):
         p = Plan()

@@ -71,6 +71,13 @@ _SIGS = {
     "alpha_leakyRelu2D_deltaX_v1": "lpppfiii",
     "alpha_batchNorm2D_row": "lpppfipiii",
     "alpha_batchNorm_affined2D_row": "lpppfppipiii",
+    "alpha_field_affine_deltaAB_v1": "llppppiippppiiin",
+    "alpha_field_affine_deltaAB_v2": "llppiippppiiin",
+    "alpha_field_batchNorm_deltaAB_v2": "llppppfiippppiiin",
+    "alpha_batchNorm2D_row_deltaX_v1": "lpppfppipiii",
+    "alpha_batchNorm2D_row_deltaX_v2": "lppppfppipiii",
+    "alpha_batchNorm_affined2D_row_deltaX_v1": "lpppfppppipiii",
+    "alpha_batchNorm_affined2D_row_deltaX_v2": "lppppfpppipiii",
 }
 
 
@@ -82,7 +89,7 @@ class Epilogue(ctypes.Structure):
         super().__init__(Bias or None, X_mean or None, X_var or None, eps, A or None, B or None, k)
 
 
-_CT = {"s": _S, "i": _I, "p": _P, "l": _L, "f": ctypes.c_float, "e": ctypes.POINTER(Epilogue)}
+_CT = {"s": _S, "i": _I, "p": _P, "l": _L, "f": ctypes.c_float, "e": ctypes.POINTER(Epilogue), "n": ctypes.POINTER(ctypes.c_int)}
 
 
 class AlphaConvError(RuntimeError):
@@ -166,6 +173,8 @@ def _call(name, *args):
         elif c == "e":
             keep.append(a)
             conv.append(ctypes.byref(a))
+        elif c == "n":
+            conv.append(a)   # a ctypes.byref(c_int), or None
         else:
             conv.append(int(a))
     rc = getattr(L, name)(*conv)
@@ -391,9 +400,72 @@ class Cuda_dconv3D_deltaW:
               deltaB, deltaB_buf, FH, FW, N, IC, OC, sh, sw, ph, pw)
 
 
+class Cuda_reduce:
+    """The field sums of batch normalisation's backward (Cuda_reduce.java:697, 746, 939), same argument order; they return
+    the number of rows left after the last stage, as the reference's natives do. Only these three of the class."""
+
+    @staticmethod
+    def _run(name, *args):
+        n = ctypes.c_int(0)
+        _call(name, *args, ctypes.byref(n))
+        return n.value
+
+    @staticmethod
+    def field_affine_deltaAB_v1(stream1, stream2, deltaY, Y, A, B, N, M, deltaA_buf, deltaA, deltaB_buf, deltaB, mem_width, mem_stride, partNum):
+        return Cuda_reduce._run("alpha_field_affine_deltaAB_v1", stream1, stream2, deltaY, Y, A, B, N, M, deltaA_buf, deltaA, deltaB_buf, deltaB,
+                                mem_width, mem_stride, partNum)
+
+    @staticmethod
+    def field_affine_deltaAB_v2(stream1, stream2, deltaY, X_norm, N, M, deltaA_buf, deltaA, deltaB_buf, deltaB, mem_width, mem_stride, partNum):
+        return Cuda_reduce._run("alpha_field_affine_deltaAB_v2", stream1, stream2, deltaY, X_norm, N, M, deltaA_buf, deltaA, deltaB_buf, deltaB,
+                                mem_width, mem_stride, partNum)
+
+    @staticmethod
+    def field_batchNorm_deltaAB_v2(stream1, stream2, deltaY, X, X_mean, X_var, eps, N, M, deltaA_buf, deltaA, deltaB_buf, deltaB,
+                                   mem_width, mem_stride, partNum):
+        return Cuda_reduce._run("alpha_field_batchNorm_deltaAB_v2", stream1, stream2, deltaY, X, X_mean, X_var, eps, N, M, deltaA_buf, deltaA,
+                                deltaB_buf, deltaB, mem_width, mem_stride, partNum)
+
+    @staticmethod
+    def field_nextN(N, M):
+        """Cuda_reduce.field_nextN (Cuda_reduce.java:35-45): rows of the buffers the Java engine allocates for these sums."""
+        if M > 15:
+            if N > 63:
+                return N >> 6
+            if N > 15:
+                return 1
+        if M > 7:
+            if N > 127:
+                return N >> 7
+            if N > 31:
+                return 1
+        return (N + 63) >> 6
+
+
 class Cuda_function:
-    """The row functions the reference applies to convolution outputs (Cuda_function.java:1607, 1640, 3829, 3862), same
-    argument order; one HBM-bound pass each. Only these four: the class's other natives are outside this library."""
+    """The row functions the reference applies around a convolution (Cuda_function.java:1607, 1640, 3829, 3862 forward;
+    3890, 3923, 3958, 3992 backward of batch normalisation), same argument order; one HBM-bound pass each. Only these:
+    the class's other natives are outside this library."""
+
+    @staticmethod
+    def batchNorm2D_row_deltaX_v1(stream, deltaY, Y, X_var, eps, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv, mem_width, mem_stride):
+        _call("alpha_batchNorm2D_row_deltaX_v1", stream, deltaY, Y, X_var, eps, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv, mem_width, mem_stride)
+
+    @staticmethod
+    def batchNorm2D_row_deltaX_v2(stream, deltaY, X, X_mean, X_var, eps, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv, mem_width, mem_stride):
+        _call("alpha_batchNorm2D_row_deltaX_v2", stream, deltaY, X, X_mean, X_var, eps, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv,
+              mem_width, mem_stride)
+
+    @staticmethod
+    def batchNorm_affined2D_row_deltaX_v1(stream, deltaY, Y, X_var, eps, A, B, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv, mem_width, mem_stride):
+        _call("alpha_batchNorm_affined2D_row_deltaX_v1", stream, deltaY, Y, X_var, eps, A, B, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv,
+              mem_width, mem_stride)
+
+    @staticmethod
+    def batchNorm_affined2D_row_deltaX_v2(stream, deltaY, X, X_mean, X_var, eps, A, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv,
+                                          mem_width, mem_stride):
+        _call("alpha_batchNorm_affined2D_row_deltaX_v2", stream, deltaY, X, X_mean, X_var, eps, A, deltaXp1, deltaXp2, row_lengthv, deltaX, lengthv,
+              mem_width, mem_stride)
 
     @staticmethod
     def leakyRelu2D(stream, X, k, Y, lengthv, mem_width, mem_stride):

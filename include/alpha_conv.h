@@ -429,6 +429,46 @@ int alpha_batchNorm_affined2D_row(int64_t stream, const float *X, const float *X
                                   const float *A, const float *B, int row_lengthv,
                                   float *Y, int lengthv, int mem_width, int mem_stride);
 
+/* ---- backward of batch normalisation around the convolution ---------------------------------------------------------
+ * The reference's training step runs these between leakyRelu2D_deltaX and dconv3D_deltaX
+ * (CudaFloat32EngineBase.java:4385-4760: batchNorm2D_deltaX_v1 / _v2, batchNorm2D_gradients_v1 / _v2). The tensor is
+ * [N = field_length rows, M = row_lengthv columns] (rows = pixels of the batch, columns = channels, M == mem_stride).
+ *
+ * Field sums (Cuda_reduce.java:697, 746, 939; reduce/A.cu:486 and twins): per column m
+ *     deltaB[m] = deltaXp1[m] = sum_n deltaY[n, m]            deltaA[m] = deltaXp2[m] = sum_n deltaY[n, m] * X_norm[n, m]
+ * with X_norm = (Y - B) / A (affine_v1), = the second tensor itself (affine_v2), = (X - X_mean) * rsqrt(X_var + eps)
+ * (batchNorm_v2). deltaA_buf / deltaB_buf hold field_nextN(N, M) * M floats each (may be NULL when that is 1) and a
+ * result may be the head of its own buffer, as the Java engine passes them. Everything is enqueued on stream1 (stream2 is
+ * accepted and left idle). Deterministic: fixed summation order, bit-identical from run to run. The reference's natives
+ * return the number of rows left after their last stage; here that value goes to *nextN (may be NULL) and the return
+ * value is the status, as for every entry of this header. */
+int alpha_field_affine_deltaAB_v1(int64_t stream1, int64_t stream2, const float *deltaY, const float *Y, const float *A, const float *B,
+                                  int N, int M, float *deltaA_buf, float *deltaA, float *deltaB_buf, float *deltaB,
+                                  int mem_width, int mem_stride, int partNum, int *nextN);
+int alpha_field_affine_deltaAB_v2(int64_t stream1, int64_t stream2, const float *deltaY, const float *X_norm,
+                                  int N, int M, float *deltaA_buf, float *deltaA, float *deltaB_buf, float *deltaB,
+                                  int mem_width, int mem_stride, int partNum, int *nextN);
+int alpha_field_batchNorm_deltaAB_v2(int64_t stream1, int64_t stream2, const float *deltaY, const float *X, const float *X_mean,
+                                     const float *X_var, float eps, int N, int M, float *deltaA_buf, float *deltaA,
+                                     float *deltaB_buf, float *deltaB, int mem_width, int mem_stride, int partNum, int *nextN);
+/* Row functions (Cuda_function.java:3890, 3923, 3958, 3992; function/extra_batchNorm*_row_deltaX_v*.cuh):
+ *     deltaX = scale * (deltaY - (deltaXp1 + deltaXp2 * X_norm) / N),   N = lengthv / row_lengthv,
+ * scale = rsqrt(X_var + eps) (times A for the affine forms); v1 takes X_norm from the layer's output Y (Y itself, or
+ * (Y - B) / A), v2 from its input X. Pad elements (mem_width <= column < mem_stride) are written as zeros, and so are NaN
+ * results of the affine v1 form (A == 0), as in the reference. deltaX may be deltaY. */
+int alpha_batchNorm2D_row_deltaX_v1(int64_t stream, const float *deltaY, const float *Y, const float *X_var, float eps,
+                                    const float *deltaXp1, const float *deltaXp2, int row_lengthv, float *deltaX,
+                                    int lengthv, int mem_width, int mem_stride);
+int alpha_batchNorm2D_row_deltaX_v2(int64_t stream, const float *deltaY, const float *X, const float *X_mean, const float *X_var, float eps,
+                                    const float *deltaXp1, const float *deltaXp2, int row_lengthv, float *deltaX,
+                                    int lengthv, int mem_width, int mem_stride);
+int alpha_batchNorm_affined2D_row_deltaX_v1(int64_t stream, const float *deltaY, const float *Y, const float *X_var, float eps,
+                                            const float *A, const float *B, const float *deltaXp1, const float *deltaXp2,
+                                            int row_lengthv, float *deltaX, int lengthv, int mem_width, int mem_stride);
+int alpha_batchNorm_affined2D_row_deltaX_v2(int64_t stream, const float *deltaY, const float *X, const float *X_mean, const float *X_var,
+                                            float eps, const float *A, const float *deltaXp1, const float *deltaXp2,
+                                            int row_lengthv, float *deltaX, int lengthv, int mem_width, int mem_stride);
+
 #ifdef __cplusplus
 }
 #endif

@@ -144,6 +144,18 @@ int alpha_engine_dconv3D_deltaX_leakyRelu(alpha_engine *e, float *deltaX, int IH
                                           const float *W, int FH, int FW, int N, int IC, int OC, int sh, int sw, int ph, int pw,
                                           const float *Xf, float k, alpha_conv_plan *plan_out);
 
+/* Backward of the batch normalisation that follows a convolution, as one operator each (field sums, then the row function):
+ * EngineBase.batchNorm2D_deltaX_v1 / _v2 without A (CudaFloat32EngineBase.java:4385-4475), with A (:4478-4576), and with
+ * deltaA / deltaB as further results batchNorm2D_gradients_v1 / _v2 (:4648-4760). v1 reads the layer's output Y (and B
+ * when affine), v2 its input X and X_mean. A == NULL: not affine (B, deltaA, deltaB must be NULL too); deltaA and deltaB
+ * go together. field_length rows of row_lengthv == stride elements, lengthv = field_length * row_lengthv. */
+int alpha_engine_batchNorm2D_deltaX_v1(alpha_engine *e, float *deltaX, const float *deltaY, const float *Y, const float *X_var, float eps,
+                                       const float *A, const float *B, float *deltaA, float *deltaB,
+                                       int field_length, int row_lengthv, int lengthv, int width, int stride);
+int alpha_engine_batchNorm2D_deltaX_v2(alpha_engine *e, float *deltaX, const float *deltaY, const float *X, const float *X_mean,
+                                       const float *X_var, float eps, const float *A, float *deltaA, float *deltaB,
+                                       int field_length, int row_lengthv, int lengthv, int width, int stride);
+
 #ifdef __cplusplus
 }
 #endif

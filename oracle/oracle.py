@@ -193,3 +193,38 @@ def max_err_ratio(got, want, rel=1e-4, floor_abs=1e-5):
     assert got.size == want.size
     return float(lib().oracle_max_err_ratio(_p32(got), _p64(want), ctypes.c_long(got.size),
                                             ctypes.c_double(rel), ctypes.c_double(floor_abs)))
+
+
+# ---- backward of batch normalisation (numpy, fp64): restates the reference's kernels operation by operation -------------
+def batchNorm_xnorm(form, S, X_mean=None, X_var=None, eps=0.0, A=None, B=None):
+    """X_norm as the reference's backward kernels recover it. form "given": S itself (batchNorm2D_row_deltaX_v1,
+    function/extra_batchNorm2D_row_deltaX_v1.cuh:57, 76); "from_y_affine": (S - B) / A
+    (extra_batchNorm_affined2D_row_deltaX_v1.cuh:56, 91-95); "from_x": (S - X_mean) * rsqrt(X_var + eps)
+    (extra_batchNorm2D_row_deltaX_v2.cuh:53-54, 86-90). S is [N, M]; the per-column vectors are [M]."""
+    S = np.asarray(S, dtype=np.float64)
+    if form == "given":
+        return S
+    if form == "from_y_affine":
+        return (S - np.asarray(B, dtype=np.float64)) / np.asarray(A, dtype=np.float64)
+    if form == "from_x":
+        return (S - np.asarray(X_mean, dtype=np.float64)) / np.sqrt(np.asarray(X_var, dtype=np.float64) + float(eps))
+    raise ValueError(form)
+
+
+def batchNorm_deltaAB(deltaY, X_norm):
+    """(deltaA, deltaB) = (sum over rows of deltaY * X_norm, sum over rows of deltaY) per column
+    (reduce/field_batchNorm_deltaAB_v2.cuh:13-14, 40-45; deltaA is the row function's deltaXp2, deltaB its deltaXp1)."""
+    dY = np.asarray(deltaY, dtype=np.float64)
+    return (dY * np.asarray(X_norm, dtype=np.float64)).sum(axis=0), dY.sum(axis=0)
+
+
+def batchNorm_deltaX(deltaY, X_norm, X_var, eps, deltaXp1, deltaXp2, A=None):
+    """deltaX = scale * (deltaY - (deltaXp1 + deltaXp2 * X_norm) / N), scale = rsqrt(X_var + eps), times A when affine
+    (function/extra_batchNorm2D_row_deltaX_v1.cuh:50-58, 86-90; extra_batchNorm_affined2D_row_deltaX_v2.cuh:52-60, 99-103).
+    N is the number of rows."""
+    dY = np.asarray(deltaY, dtype=np.float64)
+    N = dY.shape[0]
+    scale = 1.0 / np.sqrt(np.asarray(X_var, dtype=np.float64) + float(eps))
+    if A is not None:
+        scale = scale * np.asarray(A, dtype=np.float64)
+    return scale * (dY - (np.asarray(deltaXp1, dtype=np.float64) + np.asarray(deltaXp2, dtype=np.float64) * np.asarray(X_norm, dtype=np.float64)) / N)

@@ -301,3 +301,33 @@ def test_max_err_ratio():
     got = np.array([1.00005, 5e-6, -2.0], np.float32)
     r = O.max_err_ratio(got, want, 1e-4, 1e-5)
     assert 0.49 < r < 0.52
+
+
+# ---- backward of batch normalisation: the oracle's closed forms against automatic differentiation ----------------------
+@pytest.mark.parametrize("N,M,affine", [(37, 8, True), (64, 12, False), (200, 4, True)])
+def test_batchNorm_backward_oracle_equals_autograd(N, M, affine):
+    """The reference's formulas are the gradient of Y = A * (X - mean(X)) / sqrt(var(X) + eps) + B when mean / var are the
+    batch statistics of X (biased variance): torch's automatic differentiation of exactly that expression, in fp64, pins
+    deltaA, deltaB and deltaX of all four forms (X_norm taken from Y, from (Y - B) / A and from X); a dropped 1/N, a sign
+    or a swapped deltaXp1 / deltaXp2 changes deltaX by orders of magnitude more than the 1e-10 allowed."""
+    import torch
+    g = torch.Generator().manual_seed(77 + N)
+    X = torch.randn((N, M), generator=g, dtype=torch.float64) * 1.7 + 0.3
+    dY = torch.randn((N, M), generator=g, dtype=torch.float64)
+    A = (torch.rand((M,), generator=g, dtype=torch.float64) + 0.5) if affine else torch.ones(M, dtype=torch.float64)
+    B = torch.randn((M,), generator=g, dtype=torch.float64) if affine else torch.zeros(M, dtype=torch.float64)
+    eps = 1e-5
+    Xr, Ar, Br = X.clone().requires_grad_(True), A.clone().requires_grad_(True), B.clone().requires_grad_(True)
+    mean, var = Xr.mean(0), Xr.var(0, unbiased=False)
+    Y = Ar * (Xr - mean) / torch.sqrt(var + eps) + Br
+    (Y * dY).sum().backward()
+    mean_n, var_n, Yn = mean.detach().numpy(), var.detach().numpy(), Y.detach().numpy()
+    forms = [("from_x", X.numpy())]
+    forms.append(("from_y_affine", Yn) if affine else ("given", Yn))
+    for form, S in forms:
+        xn = O.batchNorm_xnorm(form, S, X_mean=mean_n, X_var=var_n, eps=eps, A=A.numpy(), B=B.numpy())
+        dA, dB = O.batchNorm_deltaAB(dY.numpy(), xn)
+        dX = O.batchNorm_deltaX(dY.numpy(), xn, var_n, eps, dB, dA, A=A.numpy() if affine else None)
+        assert np.allclose(dA, Ar.grad.numpy(), rtol=1e-10, atol=1e-10), form
+        assert np.allclose(dB, Br.grad.numpy(), rtol=1e-10, atol=1e-10), form
+        assert np.allclose(dX, Xr.grad.numpy(), rtol=1e-9, atol=1e-10), form
