@@ -440,6 +440,66 @@ def measure(wl, op, steps, warmup, with_parity=True):
     return row
 
 
+def measure_bn_backward(wl, steps, warmup, with_parity=True):
+    """Backward of the batch normalisation that follows the layer's convolution (batchNorm2D_gradients_v2 through the host
+    layer: field sums of deltaY and deltaY * X_norm over the layer's output, then the row function), an HBM-bound operator:
+    algorithmic bytes = one read of deltaY and of the normalisation's input, one write of deltaX (the two passes read both
+    inputs twice). `kernel_ms` is the row function alone, with the sums given."""
+    from oracle import oracle as O
+    pkg, torch = wl.pkg, wl.torch
+    N, IH, IW, IC, OC, F, s, p = wl.dims
+    rows, M = N * wl.OH * wl.OW, OC
+    dev = wl.X.device
+    g = torch.Generator(device="cpu").manual_seed(4242)
+    Xb = torch.randn((rows, M), generator=g) * 1.3 + 0.4          # the convolution's output that was normalised
+    mean, var = Xb.double().mean(0).float(), Xb.double().var(0, unbiased=False).float()
+    A = torch.rand((M,), generator=g) + 0.5
+    dYv = wl.dYh.reshape(rows, M)
+    d = {k: v.to(dev) for k, v in dict(X=Xb, mean=mean, var=var, A=A).items()}
+    dX = torch.empty((rows, M), device=dev)
+    dA, dB = torch.empty(M, device=dev), torch.empty(M, device=dev)
+    eps = 1e-5
+
+    def step():
+        wl.engine.batchNorm2D_deltaX_v2(dX.data_ptr(), wl.dY.data_ptr(), d["X"].data_ptr(), d["mean"].data_ptr(), d["var"].data_ptr(), eps,
+                                        rows, M, rows * M, M, M, A=d["A"].data_ptr(), deltaA=dA.data_ptr(), deltaB=dB.data_ptr())
+
+    def kernel():
+        pkg.Cuda_function.batchNorm_affined2D_row_deltaX_v2(wl.stream, wl.dY.data_ptr(), d["X"].data_ptr(), d["mean"].data_ptr(), d["var"].data_ptr(),
+                                                            eps, d["A"].data_ptr(), dB.data_ptr(), dA.data_ptr(), M, dX.data_ptr(), rows * M, M, M)
+
+    wall_ms, ev_ms = time_loop(torch, step, steps, warmup)
+    wl.engine.sync()
+    _, k_ms = time_loop(torch, kernel, steps, max(1, warmup // 2))
+    by = 4.0 * 3 * rows * M
+    roof = {"bound": "hbm", "achieved": round(by / (k_ms * 1e-3) / 1e9, 2), "peak": PEAK_HBM_GBPS, "unit": "GB/s", "kernel_ms": round(k_ms, 5),
+            "traffic": None, "operator_GBps_on_two_passes": round((by + 4.0 * 2 * rows * M) / (wall_ms * 1e-3) / 1e9, 2)}
+    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
+    row = {"layer": wl.layer, "op": "bn_bwd", "ms_per_step": round(wall_ms, 5), "event_ms_per_step": round(ev_ms, 5), "tflops": None, "gflop": None,
+           "algorithmic_MB": round(by / 1e6, 2), "GridZ": None, "roofline": roof}
+    if with_parity:
+        dX.fill_(float("nan"))
+        step()
+        wl.engine.sync()
+        torch.cuda.synchronize()
+        xn = O.batchNorm_xnorm("from_x", Xb.numpy(), X_mean=mean.numpy(), X_var=var.numpy(), eps=eps)
+        wA, wB = O.batchNorm_deltaAB(dYv.numpy(), xn)
+        want = O.batchNorm_deltaX(dYv.numpy(), xn, var.numpy(), eps, wB, wA, A=A.numpy())
+        got = dX.cpu().numpy()
+        rms = float(np.sqrt(np.mean(want * want)))
+        tol_abs = ABS_TOL * max(1.0, rms)
+        worst = max(O.max_err_ratio(got, want, REL_TOL, tol_abs), O.max_err_ratio(dA.cpu().numpy(), wA, REL_TOL, ABS_TOL * max(1.0, float(np.sqrt(np.mean(wA * wA))))),
+                    O.max_err_ratio(dB.cpu().numpy(), wB, REL_TOL, ABS_TOL * max(1.0, float(np.sqrt(np.mean(wB * wB))))))
+        row["parity"] = {"vs": "fp64 closed form (oracle)", "subset": "deltaX, deltaA, deltaB: every element", "checked": int(want.size + 2 * M),
+                         "tol_rel": REL_TOL, "tol_abs": float("%.3g" % tol_abs), "max_err_ratio": round(worst, 4),
+                         "max_err_ratio_at_abs_1e-5": round(O.max_err_ratio(got, want, REL_TOL, ABS_TOL), 4),
+                         "max_abs_err": float("%.3g" % float(np.max(np.abs(got.astype(np.float64) - want)))), "rms_expected": float("%.4g" % rms),
+                         "samePercentRelative_1e-4": round(O.samePercentRelative(want.astype(np.float32), got, 1e-4), 6),
+                         "samePercentRelative_1e-5": round(O.samePercentRelative(want.astype(np.float32), got, 1e-5), 6),
+                         "ok": bool(worst <= 1.0 and np.isfinite(got).all())}
+    return row
+
+
 def layer_ops(layer):
     N, IH, IW, IC, OC, F, s, p, ICl, ops = LAYERS[layer]
     ops = list(ops)
@@ -452,7 +512,7 @@ def layer_ops(layer):
     if "dw" in ops and F == 3 and s == 1:
         ops.append("dw_wino")
     if layer == "c3a":
-        ops += ["fwd_bias", "fwd_cached", "fwd_fused"]
+        ops += ["fwd_bias", "fwd_cached", "fwd_fused", "bn_bwd"]
     return ops
 
 
@@ -571,7 +631,10 @@ def main():
         for layer in sorted(LAYERS):
             wl = Workload(pkg, torch, layer, seed_of(layer))
             for o in layer_ops(layer):
-                row = measure(wl, o, args.steps, args.warmup, with_parity=not args.no_parity)
+                if o == "bn_bwd":
+                    row = measure_bn_backward(wl, args.steps, args.warmup, with_parity=not args.no_parity)
+                else:
+                    row = measure(wl, o, args.steps, args.warmup, with_parity=not args.no_parity)
                 rows.append(row)
                 print(json.dumps(row, separators=(",", ":")), flush=True)   # full row: a line of its own, before the result line
             wl.close()

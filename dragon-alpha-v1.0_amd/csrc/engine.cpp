@@ -360,6 +360,10 @@ alpha_engine *alpha_engine_create(int64_t stream)
     int cu = 0, clk = 0;
     if (alpha_conv_device_info(&cu, &clk) != 0) cu = 0;
     alpha_engine_config_default(&e->cfg, cu);
+    // The one setting in which an engine object departs from the Java engine's defaults: the split-K factor is lowered to
+    // what the persistent backward-filter kernel needs on this device (the same cut of the layer, no buffers of zeros for
+    // buf_summary to add). Set it to 0 for the Java engine's GridZ exactly.
+    e->cfg.deltaW_SK_leastUnits = cu;
     e->stream = stream;
     e->err[0] = 0;
     return e;

@@ -97,43 +97,42 @@ hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, 
 // deltaW += sum_{p < part} deltaW_buf[p], summed in the fixed order p = 0, 1, ... with fp32 Kahan
 // compensation (the reference's recurrence, operation for operation). The adds of one element form a serial
 // chain, but the loads do not depend on it: one thread owns ONE element (so even a 16 K-element filter gives
-// hundreds of wavefronts) and fetches 24 partials at a time, the next batch while the current one runs through the chain.
+// hundreds of wavefronts) and requests U partials at a time, the next U before the current ones run through the chain.
+// Every load is unconditional - a batch that reaches past the last partial reads the last one again - and a partial
+// that is not there is left out of the chain by a select (adding a zero would still apply the compensation), so no
+// partial is ever waited for on its own: with U = 64 the 127 partials of the Java engine's largest split-K factor are in
+// flight at once and the kernel waits for memory once.
+template <int U>
 __global__ __launch_bounds__(256) void buf_summary_kernel(const float *__restrict__ buf, float *__restrict__ dW,
                                                           int part, int sizeW)
 {
-    constexpr int U = 24;   // partials per batch; two batches in flight (the next one is requested before this one is added)
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= sizeW) return;
     float dw = dW[i], c = 0.f;
-    int p = 0;
     float b[U], nb[U];
-    if (U <= part) {
+    const float *src = buf + i;
+    const int last = part - 1;
 #pragma unroll
-        for (int u = 0; u < U; u++) b[u] = buf[(size_t)u * sizeW + i];
-    }
-    for (; p + U <= part; p += U) {
-        const bool more = p + 2 * U <= part;
+    for (int u = 0; u < U; u++) b[u] = src[(size_t)(u < last ? u : last) * sizeW];
+    for (int p = 0; p < part; p += U) {
+        const bool more = p + U < part;   // uniform
         if (more) {
 #pragma unroll
-            for (int u = 0; u < U; u++) nb[u] = buf[(size_t)(p + U + u) * sizeW + i];
+            for (int u = 0; u < U; u++) nb[u] = src[(size_t)(p + U + u < last ? p + U + u : last) * sizeW];
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
+            const bool live = p + u < part;   // uniform
             const float y = b[u] - c;
             const float s = dw + y;
-            c = (s - dw) - y;
-            dw = s;
+            const float cn = (s - dw) - y;
+            c = live ? cn : c;
+            dw = live ? s : dw;
         }
         if (more) {
 #pragma unroll
             for (int u = 0; u < U; u++) b[u] = nb[u];
         }
-    }
-    for (; p < part; p++) {
-        const float y = buf[(size_t)p * sizeW + i] - c;
-        const float s = dw + y;
-        c = (s - dw) - y;
-        dw = s;
     }
     dW[i] = dw;
 }
@@ -141,7 +140,13 @@ __global__ __launch_bounds__(256) void buf_summary_kernel(const float *__restric
 hipError_t launch_buf_summary(hipStream_t s, const float *buf, float *dW, int part, int sizeW)
 {
     if (sizeW <= 0 || part <= 0) return hipSuccess;
-    hipLaunchKernelGGL(buf_summary_kernel, dim3((sizeW + 255) / 256), dim3(256), 0, s, buf, dW, part, sizeW);
+    // One element per thread: a filter of 16 K elements is 256 wavefronts. Workgroups of one or two wavefronts spread them
+    // over all compute units (each wavefront waits for its own partials; four on one unit share that unit's load path).
+    const int block = sizeW >= 256 * 256 ? 256 : sizeW >= 128 * 256 ? 128 : 64;
+    const dim3 grid((sizeW + block - 1) / block);
+    if (part <= 4) hipLaunchKernelGGL(buf_summary_kernel<4>, grid, dim3(block), 0, s, buf, dW, part, sizeW);
+    else if (part <= 32) hipLaunchKernelGGL(buf_summary_kernel<16>, grid, dim3(block), 0, s, buf, dW, part, sizeW);
+    else hipLaunchKernelGGL(buf_summary_kernel<64>, grid, dim3(block), 0, s, buf, dW, part, sizeW);
     return hipGetLastError();
 }
 

@@ -49,7 +49,8 @@ typedef struct alpha_engine_config {
     int deltaW_SK_leastUnits;     /* this build only: > 0 = the number of compute units of the device; the split-K factor is then lowered
                                      (never raised) to the least value with which the persistent backward-filter kernel cuts the layer
                                      the same way - it deals the pixels evenly among the compute units whatever GridZ is, so a larger
-                                     GridZ only adds buffers of zeros for buf_summary to add. Default 0 = the reference's GridZ exactly */
+                                     GridZ only adds buffers of zeros for buf_summary to add. alpha_engine_config_default: 0 = the reference's GridZ
+                                     exactly; alpha_engine_create sets it to the device's compute units */
 } alpha_engine_config;
 
 /* Native entry chosen by a plan; names are the Java native method names. */
