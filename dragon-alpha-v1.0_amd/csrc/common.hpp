@@ -224,8 +224,9 @@ hipError_t launch_pointwise_direct(hipStream_t stream, const float *A, const flo
 // wavefronts to beat the LDS-halo kernels on a stride-1 layer.
 hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC,
                               int OHt, int OWt, int CO, int TH, int TW, int sh, int sw, int ph, int pw,
-                              int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep);
-bool direct_conv_balanced(long M, int CO);
+                              int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep,
+                              float *ws = nullptr, size_t ws_bytes = 0);
+bool direct_conv_balanced(long M, int CO, bool workspace = false);
 // Kernel-split backward-data, up to four phases over the same coarse pixels in one launch, both operands straight from
 // memory: direct_conv_phased.hip. Phase f: O[o_off[f] + n*o_sn + i*o_sh + j*o_sw + co] = sum A[n, i - ph[f] + th,
 // j - pw[f] + tw, c] * B[b_off[f] + th*b_sth[f] + tw*b_stw + c*b_k + co]. hipErrorNotSupported: nothing launched.

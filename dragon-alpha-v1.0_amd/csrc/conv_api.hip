@@ -63,6 +63,11 @@ int check_dims(const char *fn, int N, int IC, int OC, int IH, int IW, int OH, in
 
 enum FilterLayout { FILTER_W, FILTER_CW };
 
+// Scratch a caller lends to the calls it makes on this thread (alpha_conv_bind_workspace): per thread, so concurrent
+// callers never see each other's.
+thread_local float *t_workspace = nullptr;
+thread_local size_t t_workspace_bytes = 0;
+
 // Debugging switch (tests and comparisons force the generic kernels with it); not part of the drop-in contract. The only
 // mutable process-wide setting of the library: atomic, read once per call, so a call sees one value throughout.
 std::atomic<int> g_fwd_algo{-1};   // -1: not yet read from the environment
@@ -122,8 +127,9 @@ bool pointwise_direct_preferred(int K, int N)
 bool direct_conv_preferred(int FH, int FW, int sh, int sw, long M, int AC, int CO)
 {
     if (sh > 1 || sw > 1) return true;
-    if (FH * FW <= 1) return AC >= 256 && direct_conv_balanced(M, CO);
-    return direct_conv_balanced(M, CO);
+    const bool ws = t_workspace != nullptr && t_workspace_bytes >= (1u << 20);
+    if (FH * FW <= 1) return AC >= 256 && direct_conv_balanced(M, CO, ws);
+    return direct_conv_balanced(M, CO, ws);
 }
 
 // The rest of a fused epilogue as a pass of its own over a dense [pixels, C] output (kernels that add a bias only).
@@ -161,7 +167,7 @@ int forward(const char *fn, const int64_t *streams, int length,
     if (layout == FILTER_CW && (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, sh, sw, (long)N * OH * OW, IC, OC)))) {
         // both operands straight from memory
         hipError_t e = launch_direct_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
-                                          0, IC * OC, OC, (long)FH * FW * IC * OC, bias, ep);
+                                          0, IC * OC, OC, (long)FH * FW * IC * OC, bias, ep, t_workspace, t_workspace_bytes);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && sh == 1 && sw == 1 && OH == IH && OW == IW && layout == FILTER_CW && algo != 3 &&
@@ -218,7 +224,8 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
     if (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, 1, 1, (long)N * IH * IW, OC, IC))) {
         // both operands straight from memory; W rotated by 180 degrees is read in place (input channel contiguous)
         hipError_t e = launch_direct_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, 1, 1, FH - 1 - ph, FW - 1 - pw,
-                                          (FH * FW - 1) * IC, -IC, FH * FW * IC, (long)OC * FH * FW * IC, nullptr, ep);
+                                          (FH * FW - 1) * IC, -IC, FH * FW * IC, (long)OC * FH * FW * IC, nullptr, ep,
+                                          t_workspace, t_workspace_bytes);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && OH == IH && OW == IW && algo != 3 && pointwise_direct_preferred(OC, IC)) {
@@ -466,6 +473,14 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz)
     return 0;
 }
 
+int alpha_conv_bind_workspace(float *workspace, long bytes)
+{
+    if (workspace != nullptr && (!aligned16(workspace) || bytes < 0))
+        return fail(ALPHA_CONV_EINVAL, "alpha_conv_bind_workspace: misaligned workspace or negative size");
+    t_workspace = workspace;
+    t_workspace_bytes = workspace ? (size_t)bytes : 0;
+    return 0;
+}
 int alpha_conv_get_fwd_algo(void) { return fwd_algo(); }
 int alpha_conv_set_pointwise_algo(int algo)
 {

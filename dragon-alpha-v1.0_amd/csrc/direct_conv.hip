@@ -39,6 +39,11 @@ struct DirectConvArgs {
     int b_off, b_tap, b_k;
     int a_bytes, b_bytes, o_bytes;
     int tiles, nblocks, items, wgs;
+    // Shares equal to the item: with a workspace every workgroup takes `base` items and the items_left = items - wgs * base
+    // left over are cut `split` ways along the reduction, one piece each for the first items_left * split workgroups; piece
+    // (item e, part z) leaves its partial sums in ws[(e * split + z) * 1024 ..] and direct_conv_fixup_kernel adds them.
+    float *ws;
+    int base, items_left, split;
     FastDiv d_OW, d_OHW, d_TW;
     Epilogue ep;
 };
@@ -73,7 +78,7 @@ __host__ __device__ inline int dc_whole_items(int n)
     return f < 4 ? 0 : f;
 }
 
-template <bool EPI>
+template <bool EPI, bool WS = false>
 __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float dc_smem[];
@@ -81,7 +86,8 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     const int t = threadIdx.x, lane = t & 63;
     const int l16 = lane & 15, q = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int g_lo = (int)((long)p.items * blockIdx.x / p.wgs), g_hi = (int)((long)p.items * (blockIdx.x + 1) / p.wgs);
+    const int g_lo = WS ? (int)blockIdx.x * p.base : (int)((long)p.items * blockIdx.x / p.wgs);
+    const int g_hi = WS ? g_lo + p.base : (int)((long)p.items * (blockIdx.x + 1) / p.wgs);
     const int f = dc_whole_items(g_hi - g_lo);
     const int i_lo = g_lo + (w & 3) * f + (w >> 2) * (f >> 1), i_hi = i_lo + (f >> 1);
     const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group: even (host-checked)
@@ -100,7 +106,8 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     // The groups of a run begin `stride` tiles apart (T: one after the other).
     auto run = [&](auto tc, auto sp, const int nb, const int tile0, const int count, const int k_lo, const int k_n, const int stride) {
         constexpr int T = decltype(tc)::value;
-        constexpr bool SPLIT = decltype(sp)::value;
+        constexpr int MODE = decltype(sp)::value;   // 0: whole items; 1: shared by the workgroup; 2: the same, sums to the workspace
+        constexpr bool SPLIT = MODE != 0;
         if (count <= 0) return;
         const int n_l = nb * 64 + 4 * l16;
         const unsigned b_lane = n_l < p.CO ? (unsigned)((4 * q * p.b_k + n_l) * 4) : DC_NEVER;
@@ -246,7 +253,13 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                     floatx4 v = part[u * 64 + lane];
 #pragma unroll
                     for (int x = 1; x < 8; x++) v += part[(x * 4 * DC_SPLIT_T + u) * 64 + lane];
-                    emit(u >> 2, u & 3, v);
+                    if constexpr (MODE == 2) {
+                        // row 4 q + (u & 3) of the piece's 16 x 64 block (T == 1), channels 4 l16 .. + 3; `stride` carries the piece
+                        float *dst = p.ws + ((size_t)stride * 16 + 4 * q + (u & 3)) * 64 + 4 * l16;
+                        *reinterpret_cast<floatx4 *>(dst) = v;
+                    } else {
+                        emit(u >> 2, u & 3, v);
+                    }
                 }
                 __syncthreads();   // the next group writes `part` again
             }
@@ -280,13 +293,13 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         int n4, n3, n2, n1;
         groups_of(f >> 1, n4, n3, n2, n1);
         int base = t0;
-        run(DcInt<4>{}, DcBool<false>{}, nb_first, base + 4 * w, n4, 0, KS, 32);
+        run(DcInt<4>{}, DcInt<0>{}, nb_first, base + 4 * w, n4, 0, KS, 32);
         base += 32 * n4;
-        run(DcInt<3>{}, DcBool<false>{}, nb_first, base + 3 * w, n3, 0, KS, 24);
+        run(DcInt<3>{}, DcInt<0>{}, nb_first, base + 3 * w, n3, 0, KS, 24);
         base += 24 * n3;
-        run(DcInt<2>{}, DcBool<false>{}, nb_first, base + 2 * w, n2, 0, KS, 16);
+        run(DcInt<2>{}, DcInt<0>{}, nb_first, base + 2 * w, n2, 0, KS, 16);
         base += 16 * n2;
-        run(DcInt<1>{}, DcBool<false>{}, nb_first, base + w, n1, 0, KS, 8);
+        run(DcInt<1>{}, DcInt<0>{}, nb_first, base + w, n1, 0, KS, 8);
     } else {
         int i = i_lo;
         while (i < i_hi) {
@@ -294,10 +307,10 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
             const int cnt = min(i_hi - i, p.tiles - tile0);
             int n4, n3, n2, n1;
             groups_of(cnt, n4, n3, n2, n1);
-            run(DcInt<4>{}, DcBool<false>{}, nb, tile0, n4, 0, KS, 4);
-            run(DcInt<3>{}, DcBool<false>{}, nb, tile0 + 4 * n4, n3, 0, KS, 3);
-            run(DcInt<2>{}, DcBool<false>{}, nb, tile0 + 4 * n4 + 3 * n3, n2, 0, KS, 2);
-            run(DcInt<1>{}, DcBool<false>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1, 0, KS, 1);
+            run(DcInt<4>{}, DcInt<0>{}, nb, tile0, n4, 0, KS, 4);
+            run(DcInt<3>{}, DcInt<0>{}, nb, tile0 + 4 * n4, n3, 0, KS, 3);
+            run(DcInt<2>{}, DcInt<0>{}, nb, tile0 + 4 * n4 + 3 * n3, n2, 0, KS, 2);
+            run(DcInt<1>{}, DcInt<0>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1, 0, KS, 1);
             i += cnt;
         }
     }
@@ -311,23 +324,59 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         // first loads and the two barriers for a quarter of the work, with five loads per 16 MFMAs)
         const int run_len = min(g_hi - i, p.tiles - tile0), ngroups = (run_len + DC_SPLIT_T - 1) / DC_SPLIT_T;
         const int cnt = (run_len + ngroups - 1) / ngroups;
-        if (cnt == 4) run(DcInt<4>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n, 4);
-        else if (cnt == 3) run(DcInt<3>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n, 3);
-        else if (cnt == 2) run(DcInt<2>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n, 2);
-        else run(DcInt<1>{}, DcBool<true>{}, nb, tile0, 1, k_lo, k_n, 1);
+        if (cnt == 4) run(DcInt<4>{}, DcInt<1>{}, nb, tile0, 1, k_lo, k_n, 4);
+        else if (cnt == 3) run(DcInt<3>{}, DcInt<1>{}, nb, tile0, 1, k_lo, k_n, 3);
+        else if (cnt == 2) run(DcInt<2>{}, DcInt<1>{}, nb, tile0, 1, k_lo, k_n, 2);
+        else run(DcInt<1>{}, DcInt<1>{}, nb, tile0, 1, k_lo, k_n, 1);
         i += cnt;
+    }
+    if constexpr (WS) {
+        // this workgroup's piece of an item left over after the equal shares: part z of `split` of the reduction, cut in
+        // eight again among the wavefronts; the sums of the eight go to the workspace, not to O
+        if ((int)blockIdx.x < p.items_left * p.split) {   // uniform
+            const int e = (int)blockIdx.x / p.split, z = (int)blockIdx.x - e * p.split;
+            const int item = p.wgs * p.base + e;
+            const int nb = item / p.tiles, tile0 = item - nb * p.tiles;
+            const int parts = 8 * p.split, idx = 8 * z + part_idx;
+            const int z_lo = (int)((long)KS * idx / parts), z_n = (int)((long)KS * (idx + 1) / parts) - z_lo;
+            run(DcInt<1>{}, DcInt<2>{}, nb, tile0, 1, z_lo, z_n, e * p.split + z);
+        }
+    }
+}
+
+// O[item's 16 pixels][its 64 channels] = epilogue(sum over z < split of ws[(e * split + z)][16][64]), the pieces added in
+// the order z = 0, 1, ...: one workgroup of 256 threads per item left over, a thread per 128-bit store.
+__global__ __launch_bounds__(256) void direct_conv_fixup_kernel(const DirectConvArgs p)
+{
+    const int e = blockIdx.x, row = threadIdx.x >> 4, c4 = threadIdx.x & 15;
+    const int item = p.wgs * p.base + e;
+    const int nb = item / p.tiles, tile = item - nb * p.tiles;
+    const float *src = p.ws + ((size_t)e * p.split * 16 + row) * 64 + 4 * c4;
+    floatx4 v = *reinterpret_cast<const floatx4 *>(src);
+    for (int z = 1; z < p.split; z++) v += *reinterpret_cast<const floatx4 *>(src + (size_t)z * 1024);
+    const int m = tile * 16 + row, col = nb * 64 + 4 * c4;
+    if (m < p.M && col < p.CO) {
+        const size_t elem = (size_t)m * p.CO + col;
+        const float4 r = epilogue4(make_float4(v[0], v[1], v[2], v[3]), p.ep, col, elem);
+        *reinterpret_cast<float4 *>(p.O + elem) = r;
     }
 }
 
 // Share of the SIMDs' time that is work when `items` equal items are dealt to `cus` workgroups as the kernel does: a
 // workgroup with n items spends f(n) whole items per SIMD and a quarter of each item left over (counted 10 % dearer:
-// the partial sums' way through LDS, shorter loops).
-static double direct_conv_balance(long items, int cus)
+// the partial sums' way through LDS, shorter loops). With a workspace (and all items shared) the items that do not
+// divide by the workgroups are cut into pieces, so the largest share is base items and one piece.
+static double direct_conv_balance(long items, int cus, bool workspace)
 {
     const long wgs = items < cus ? items : cus;
     auto cost = [](long n) { const long f = dc_whole_items((int)(n < (1 << 30) ? n : (1 << 30))); return (double)f + 1.1 * 0.25 * (double)(n - 4 * f); };
     const long n_hi = (items + wgs - 1) / wgs, n_lo = items / wgs;
-    const double worst = cost(n_hi) > cost(n_lo) ? cost(n_hi) : cost(n_lo);
+    double worst = cost(n_hi) > cost(n_lo) ? cost(n_hi) : cost(n_lo);
+    const long left = items - n_lo * wgs;
+    if (workspace && left > 0 && wgs / left >= 2 && n_lo >= 1 && dc_whole_items((int)n_lo + 1) == 0) {
+        const long split = wgs / left < 8 ? wgs / left : 8;
+        worst = cost(n_lo) + 1.1 * 0.25 / (double)split;
+    }
     return (double)items / (4.0 * (double)cus) / worst;
 }
 
@@ -335,11 +384,11 @@ static double direct_conv_balance(long items, int cus)
 // to beat the LDS-halo kernels on a stride-1 layer. Measured (forward, 3x3, N = 64, against the kernel with the prefetched
 // halo): 56x56x64 (49 items per workgroup) 0.111 against 0.115 ms, 28x28x128 (24 or 25) 0.110 against 0.123 ms, 14x14x256
 // (12 or 13: balance 0.91) 0.121 against 0.124 ms, 7x7x512 (6 or 7: 0.80) 0.126 against 0.141 ms.
-bool direct_conv_balanced(long M, int CO)
+bool direct_conv_balanced(long M, int CO, bool workspace)
 {
     const int cus = device_cu_count();
     if (cus < 1 || M < 1) return false;
-    return direct_conv_balance(((M + 15) / 16) * ((CO + 63) / 64), cus) >= 0.75;
+    return direct_conv_balance(((M + 15) / 16) * ((CO + 63) / 64), cus, workspace) >= 0.75;
 }
 
 // O[N, OHt, OWt, CO] = convolution of A[N, AH, AW, AC] (stride sh x sw, padding ph x pw, TH x TW taps) with the filter B
@@ -347,9 +396,14 @@ bool direct_conv_balanced(long M, int CO)
 // (0, IC * OC, OC), W[OC, FH, FW, IC] rotated by 180 degrees for stride-1 backward-data ((FH*FW - 1) * IC, -IC, FH*FW*IC).
 // Returns hipErrorNotSupported (nothing launched) when the layer does not fit: AC not a multiple of 16, an odd number
 // of steps (TH * TW * AC / 16), a filter beyond 16 x 16, tensors of 2 GB.
+// `ws` (may be NULL), ws_bytes: scratch for the duration of the launch. With it, a layer whose items do not divide by the
+// workgroups and are few per workgroup (fewer than 16: all of them shared by the workgroup's wavefronts) is dealt out in
+// equal shares of whole items, the items left over are cut along the reduction into one piece per workgroup, and a second
+// short launch adds the pieces: 1568 items on 256 workgroups are 6 each + an eighth of one, not 6 or 7.
 hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC,
                               int OHt, int OWt, int CO, int TH, int TW, int sh, int sw, int ph, int pw,
-                              int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep)
+                              int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep,
+                              float *ws, size_t ws_bytes)
 {
     if (AC < 16 || (AC & 15) || CO < 4 || (CO & 3) || TH < 1 || TW < 1 || TH > 16 || TW > 16) return hipErrorNotSupported;
     if (((TH * TW * (AC >> 4)) & 1) != 0) return hipErrorNotSupported;
@@ -374,6 +428,33 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
     a.ep = ep ? *ep : bias_epilogue(bias);
     const int wgs = cus < a.items ? cus : a.items;   // one workgroup of eight wavefronts per compute unit
     a.wgs = wgs;
+    a.ws = nullptr;
+    a.base = a.items / wgs;
+    a.items_left = a.items - a.base * wgs;
+    a.split = a.items_left > 0 ? wgs / a.items_left : 0;
+    if (a.split > 8) a.split = 8;   // pieces of an eighth of the steps, cut in eight again among the wavefronts, are short enough
+    {
+        // Worth it where the workgroups that would hold base + 1 items set the time (all items shared: fewer than 16 per
+        // workgroup) and what a workgroup saves - an item less the piece it gets, at 128 cycles per step of an item shared
+        // by four SIMDs - outweighs the second launch (some 8 k cycles).
+        const long KS = (long)TH * TW * (AC >> 4);
+        const bool shared_only = a.base >= 1 && dc_whole_items(a.base + 1) == 0;
+        if (ws != nullptr && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 && a.items_left > 0 && a.split >= 2 && shared_only &&
+            ws_bytes >= (size_t)a.items_left * a.split * 1024 * sizeof(float) && KS * 128 * (a.split - 1) / a.split > 8192 && KS >= 8L * a.split)
+            a.ws = ws;
+    }
+    if (a.ws != nullptr) {
+        if (a.ep.fused) {
+            if (hipError_t e = ensure_dynamic_lds<direct_conv_kernel<true, true>>(DC_LDS_BYTES); e != hipSuccess) return e;
+            hipLaunchKernelGGL((direct_conv_kernel<true, true>), dim3(wgs), dim3(512), DC_LDS_BYTES, stream, a);
+        } else {
+            if (hipError_t e = ensure_dynamic_lds<direct_conv_kernel<false, true>>(DC_LDS_BYTES); e != hipSuccess) return e;
+            hipLaunchKernelGGL((direct_conv_kernel<false, true>), dim3(wgs), dim3(512), DC_LDS_BYTES, stream, a);
+        }
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        hipLaunchKernelGGL(direct_conv_fixup_kernel, dim3(a.items_left), dim3(256), 0, stream, a);
+        return hipGetLastError();
+    }
     if (a.ep.fused) {
         if (hipError_t e = ensure_dynamic_lds<direct_conv_kernel<true>>(DC_LDS_BYTES); e != hipSuccess) return e;
         hipLaunchKernelGGL(direct_conv_kernel<true>, dim3(wgs), dim3(512), DC_LDS_BYTES, stream, a);

@@ -74,6 +74,7 @@ void alpha_engine_config_default(alpha_engine_config *c, int compute_units)
     c->deltaW_winograd = 0;
     c->deltaW_SK_fillUnits = 0;
     c->deltaW_SK_leastUnits = 0;
+    c->conv_workspace = 0;
     c->cache_filter_transforms = 0;
 }
 
@@ -279,6 +280,24 @@ struct BlockScope {   // returns the operator's scratch to the pool when the ope
     ~BlockScope() { release_blocks(e); }
 };
 
+static void *take_block(alpha_engine *e, size_t bytes);
+
+// Lends the library scratch for the calls the operator makes on this thread (alpha_conv_bind_workspace): taken from the
+// engine's pool like every other block of the operator, so it is recycled in stream order after the operator's kernels.
+struct WorkspaceScope {
+    bool bound = false;
+    explicit WorkspaceScope(alpha_engine *e)
+    {
+        if (!e->cfg.conv_workspace) return;
+        constexpr size_t bytes = 1u << 20;
+        if (void *p = take_block(e, bytes)) bound = alpha_conv_bind_workspace(static_cast<float *>(p), (long)bytes) == 0;
+    }
+    ~WorkspaceScope()
+    {
+        if (bound) alpha_conv_bind_workspace(nullptr, 0);
+    }
+};
+
 static void *take_block(alpha_engine *e, size_t bytes)
 {
     std::lock_guard<std::mutex> g(e->mu);
@@ -364,6 +383,7 @@ alpha_engine *alpha_engine_create(int64_t stream)
     // what the persistent backward-filter kernel needs on this device (the same cut of the layer, no buffers of zeros for
     // buf_summary to add). Set it to 0 for the Java engine's GridZ exactly.
     e->cfg.deltaW_SK_leastUnits = cu;
+    e->cfg.conv_workspace = 1;   // and forward / backward-data calls may use a piece of the engine's scratch (see the header)
     e->stream = stream;
     e->err[0] = 0;
     return e;
@@ -423,6 +443,7 @@ int alpha_engine_conv3D(alpha_engine *e, float *Y, int OH, int OW, const float *
         return ALPHA_CONV_EINVAL;
     }
     BlockScope scope{e};
+    WorkspaceScope workspace(e);
     alpha_conv_plan p;
     alpha_plan_conv3D(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, ph, pw, &p);
     if (plan_out) *plan_out = p;
@@ -474,6 +495,7 @@ static int conv3D_with_epilogue(alpha_engine *e, const char *what, float *Y, int
                                 const alpha_conv_epilogue *ep, alpha_conv_plan *plan_out)
 {
     BlockScope scope{e};
+    WorkspaceScope workspace(e);
     alpha_conv_plan p;
     alpha_plan_conv3D(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, ph, pw, &p);
     if (plan_out) *plan_out = p;
@@ -707,6 +729,7 @@ static int deltaX_impl(alpha_engine *e, const char *what, float *deltaX, int IH,
         return ALPHA_CONV_EINVAL;
     }
     BlockScope scope{e};
+    WorkspaceScope workspace(e);
     alpha_conv_plan p;
     alpha_plan_deltaX(&e->cfg, IH, IW, OH, OW, FH, FW, N, IC, OC, sh, sw, &p);
     if (p.entry == ALPHA_E_dconv3D_deltaX_winograd && (OH != IH + 2 * ph - 2 || OW != IW + 2 * pw - 2)) {

@@ -26,7 +26,7 @@ class Config(ctypes.Structure):
                 ("deltaX_s1_V2_Q", ctypes.c_float), ("deltaX_ks_V2_Q", ctypes.c_float),
                 ("conv3D_winograd", ctypes.c_int), ("deltaW_SK_fillUnits", ctypes.c_int),
                 ("cache_filter_transforms", ctypes.c_int), ("deltaX_winograd", ctypes.c_int), ("deltaW_winograd", ctypes.c_int),
-                ("deltaW_SK_leastUnits", ctypes.c_int)]
+                ("deltaW_SK_leastUnits", ctypes.c_int), ("conv_workspace", ctypes.c_int)]
 
 
 class Plan(ctypes.Structure):

@@ -58,6 +58,14 @@ int alpha_conv_device_info(int *compute_units, int *clock_khz);
  * No counterpart in the reference (its Winograd experiments are compiled out, conv/conv3D.cuh:39-44). */
 int alpha_conv_set_fwd_algo(int algo);
 int alpha_conv_get_fwd_algo(void);
+/* Scratch for the calling thread's next calls (no counterpart in the reference, whose natives get no scratch beyond CW and
+ * deltaW_buf): device memory the caller lends until it binds NULL again; kernels enqueued by this thread's calls in
+ * between may write it, so it must stay untouched until they have finished (stream order). With at least 1 MiB the
+ * forward and stride-1 backward-data entries deal layers of few work items per compute unit out in equal shares (the
+ * items left over are cut along the reduction, their pieces added by a short second kernel in a fixed order: results are
+ * bit-identical from run to run, and differ from the unbound path's in the last bits of those items only). Per thread:
+ * concurrent callers do not see each other's binding. */
+int alpha_conv_bind_workspace(float *workspace, long bytes);
 /* Debugging switch of the same kind for 1x1 stride-1 forward / backward-data where the kernel of direct_conv.hip does not
  * take the layer: -1 = chosen by shape, 0 = the filter-resident kernel, 1 = the kernel without LDS wherever it fits.
  * Also read once from the environment variable ALPHA_PW_DIRECT = 0|1. No counterpart in the reference. */

@@ -51,6 +51,11 @@ typedef struct alpha_engine_config {
                                      the same way - it deals the pixels evenly among the compute units whatever GridZ is, so a larger
                                      GridZ only adds buffers of zeros for buf_summary to add. alpha_engine_config_default: 0 = the reference's GridZ
                                      exactly; alpha_engine_create sets it to the device's compute units */
+    int conv_workspace;           /* this build only: 1 = forward and stride-1 backward-data calls lend the library 1 MiB of the engine's
+                                     scratch for the duration of the call (alpha_conv_bind_workspace), with which the kernel without
+                                     LDS deals a layer of few items per compute unit out in equal shares (7x7x512 and 14x14x256 maps at
+                                     N = 64: 6 and 12 items each plus a piece of one, instead of 6 or 7 and 12 or 13).
+                                     alpha_engine_config_default: 0; alpha_engine_create: 1 */
 } alpha_engine_config;
 
 /* Native entry chosen by a plan; names are the Java native method names. */

@@ -1054,3 +1054,73 @@ def test_reference_style_criterion_deltaW(dev):
     DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
                              F_, F_, N, IC, OC, s, s, p, p)
     check_reference_style(_sum_partials(dev, dWo, buf, GridZ), cpu, "deltaW_GemmSK", 1e-5, 1.0)
+
+
+# ----------------------------------------------------------------------------------------------
+# the kernel without LDS with scratch lent by the caller (alpha_conv_bind_workspace): equal shares of whole items, the items
+# left over cut along the reduction and added by a second kernel
+# ----------------------------------------------------------------------------------------------
+WORKSPACE_SHAPES = [
+    # N, IH, IW, IC, OC, F, p, (items left over, pieces per item) on 256 compute units
+    (24, 7, 7, 256, 512, 3, 1, (80, 3)),     # 1176 pixels = 74 tiles (the last one half empty) x 8 blocks = 592 = 2 x 256 + 80
+    (16, 14, 14, 256, 256, 3, 1, (16, 8)),   # 196 tiles x 4 blocks = 784 = 3 x 256 + 16: 16 pieces possible, 8 used
+    (64, 8, 8, 128, 320, 3, 1, (0, 0)),      # 256 tiles x 5 blocks = 5 x 256: nothing left over, the workspace stays untouched
+]
+
+
+@pytest.mark.parametrize("shape", WORKSPACE_SHAPES)
+def test_forward_and_deltaX_with_bound_workspace(dev, shape):
+    N, IH, IW, IC, OC, F_, p_, (left, split) = shape
+    torch = dev.torch
+    L = pkg.lib()
+    X, W, dY = normal((N, IH, IW, IC), 5301), he_normal(OC, F_, F_, IC, 5302), normal((N, IH, IW, OC), 5303)
+    B = normal((OC,), 5304)
+    want_y = O.conv3D_f64(X, W, 1, 1, p_, p_)
+    want_dx = O.deltaX_f64(dY, W, IH, IW, 1, 1, p_, p_)
+    x, w, dy, b = dev.put(X), dev.put(W), dev.put(dY), dev.put(B)
+    cw = dev.empty(F_ * F_ * IC * OC, fill=float("nan"))
+    C3.kernel_remode(dev.stream, w.data_ptr(), cw.data_ptr(), F_, F_, OC, IC)
+    ws_floats = 1 << 18
+    ws = dev.guarded(ws_floats)
+
+    def forward(bias):
+        y = dev.guarded(N, IH, IW, OC)
+        if bias:
+            C3.conv3D_GemmR_biased(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), cw.data_ptr(), F_, F_, b.data_ptr(), y.data_ptr(),
+                                   IH, IW, N, IC, OC, 1, 1, p_, p_)
+        else:
+            C3.conv3D_GemmR(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), cw.data_ptr(), F_, F_, y.data_ptr(), IH, IW, N, IC, OC, 1, 1, p_, p_)
+        return dev.get(y)
+
+    def backward():
+        dx = dev.guarded(N, IH, IW, IC)
+        DX.dconv3D_deltaX_s1(dev.streams, 1, dy.data_ptr(), IH, IW, w.data_ptr(), F_, F_, dx.data_ptr(), IH, IW, N, IC, OC, p_, p_)
+        return dev.get(dx)
+
+    plain_y, plain_dx = forward(False), backward()
+    try:
+        assert L.alpha_conv_bind_workspace(ws.data_ptr(), ws_floats * 4) == 0
+        ws.fill_(float("nan"))
+        got_y = forward(False)
+        used = ws[:max(1, left * split * 1024)].clone()
+        got_y2 = forward(False)
+        got_yb = forward(True)
+        ws.fill_(float("nan"))
+        got_dx = backward()
+    finally:
+        L.alpha_conv_bind_workspace(None, 0)
+    dev.check_guards(ws)
+    check(got_y, want_y, "forward with workspace %s" % (shape,))
+    check(got_yb, want_y + B.astype(np.float64), "forward with workspace and bias %s" % (shape,))
+    check(got_dx, want_dx, "backward-data with workspace %s" % (shape,))
+    assert np.array_equal(got_y.view(np.uint32), got_y2.view(np.uint32)), "two runs differ"
+    if pkg.device_info()[0] == 256:
+        if left:
+            # the path ran: every partial sum was written (without the workspace such a layer may go to another kernel
+            # altogether, so the two results are only compared through the oracle)
+            assert not bool(torch.isnan(used).any()), "partial sums missing in the workspace"
+        else:
+            assert bool(torch.isnan(used).all()) and np.array_equal(got_y.view(np.uint32), plain_y.view(np.uint32))
+    # after unbinding the plain path is back
+    assert np.array_equal(forward(False).view(np.uint32), plain_y.view(np.uint32))
+    assert np.array_equal(backward().view(np.uint32), plain_dx.view(np.uint32))
