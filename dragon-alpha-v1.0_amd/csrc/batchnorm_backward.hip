@@ -13,7 +13,7 @@
 //
 // The field sums run in two launches, both deterministic: workgroups of 16 x 16 threads sum a chunk of rows for 64
 // columns (each thread its rows in order, the 16 partial sums added through LDS in the order 0..15) into parts[chunk][M],
-// then the chunks are added the same way. The caller's buffers (deltaA_buf, deltaB_buf: nextN x M floats each, nextN as
+// then the chunks are added by a second, small kernel (64 lanes per column, fixed order). The caller's buffers (deltaA_buf, deltaB_buf: nextN x M floats each, nextN as
 // the reference's field_nextN) hold the chunk sums; a result may alias the head of its buffer, as the Java engine passes
 // them (CudaFloat32EngineBase.java:4396-4409).
 #include "common.hpp"
@@ -86,18 +86,19 @@ __global__ __launch_bounds__(256) void bn_field_sums_kernel(const BnArgs p, floa
     }
 }
 
-// out[m] = sum over chunks of parts[chunk][m], chunk lanes 0..15 each in order, then the sixteen in order. `out` may
-// alias parts[0]: a workgroup reads all of its columns' parts before it writes, and no other workgroup touches them.
-__global__ __launch_bounds__(256) void bn_sum_parts_kernel(const float *partsA, const float *partsB, float *outA, float *outB, int chunks, int M)
+// out[m] = sum over chunks of parts[chunk][m]: 64 lanes per column take chunks k, k + 64, ... in order (their loads are all
+// in flight at once), then the 64 sums are added in the order 0..63. `out` may alias parts[0]: a workgroup reads all of
+// its columns' parts before it writes, and no other workgroup touches them.
+__global__ __launch_bounds__(1024) void bn_sum_parts_kernel(const float *partsA, const float *partsB, float *outA, float *outB, int chunks, int M)
 {
-    __shared__ float4 red[16][17];
+    __shared__ float4 red[64][17];
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int c = (blockIdx.x * 16 + tx) * 4;
     const float *parts = blockIdx.y == 0 ? partsA : partsB;
     float *out = blockIdx.y == 0 ? outA : outB;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     if (c < M)
-        for (int k = ty; k < chunks; k += 16) {
+        for (int k = ty; k < chunks; k += 64) {
             const float4 v = *reinterpret_cast<const float4 *>(parts + (size_t)k * M + c);
             s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
         }
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(256) void bn_sum_parts_kernel(const float *partsA, 
     __syncthreads();
     if (ty == 0 && c < M) {
         float4 v = red[0][tx];
-        for (int k = 1; k < 16; k++) { v.x += red[k][tx].x; v.y += red[k][tx].y; v.z += red[k][tx].z; v.w += red[k][tx].w; }
+        for (int k = 1; k < 64; k++) { v.x += red[k][tx].x; v.y += red[k][tx].y; v.z += red[k][tx].z; v.w += red[k][tx].w; }
         *reinterpret_cast<float4 *>(out + c) = v;
     }
 }
@@ -182,7 +183,7 @@ hipError_t launch_bn_field_sums(hipStream_t s, int form, const float *dY, const 
     else hipLaunchKernelGGL(bn_field_sums_kernel<BN_FROM_X>, grid, dim3(256), 0, s, p, pa, pb, rows_per_chunk);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (chunks > 1) {
-        hipLaunchKernelGGL(bn_sum_parts_kernel, dim3(col_tiles, 2), dim3(256), 0, s, bufA, bufB, outA, outB, chunks, M);
+        hipLaunchKernelGGL(bn_sum_parts_kernel, dim3(col_tiles, 2), dim3(1024), 0, s, bufA, bufB, outA, outB, chunks, M);
         return hipGetLastError();
     }
     return hipSuccess;
