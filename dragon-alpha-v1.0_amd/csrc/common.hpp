@@ -227,6 +227,10 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
                               int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep,
                               float *ws = nullptr, size_t ws_bytes = 0);
 bool direct_conv_balanced(long M, int CO, bool workspace = false);
+// Backward-data of a 1x1 layer whose stride exceeds the filter (no padding, IH = sh*OH, IW = sw*OW): the product into every
+// sh x sw block's first pixel, zeros elsewhere (pointwise_scatter.hip). W is [K = OC][N = IC]. hipErrorNotSupported: nothing launched.
+hipError_t launch_pointwise_scatter(hipStream_t stream, const float *dY, const float *W, float *dX, int Nimg, int OH, int OW,
+                                    int K, int N, int sh, int sw);
 // Kernel-split backward-data, up to four phases over the same coarse pixels in one launch, both operands straight from
 // memory: direct_conv_phased.hip. Phase f: O[o_off[f] + n*o_sn + i*o_sh + j*o_sw + co] = sum A[n, i - ph[f] + th,
 // j - pw[f] + tw, c] * B[b_off[f] + th*b_sth[f] + tw*b_stw + c*b_k + co]. hipErrorNotSupported: nothing launched.

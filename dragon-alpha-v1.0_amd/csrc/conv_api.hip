@@ -278,6 +278,13 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
         hipError_t e = launch_delta_x_stem(s, dY, F, dX, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
+    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && sh * sw > 1 && IH == sh * OH && IW == sw * OW && !(ep && ep->fused) &&
+        (fwd_algo() == 0 || fwd_algo() == 6)) {
+        // a 1x1 filter under a larger stride: one matrix product scattered over deltaX, zeros in between. The filter is
+        // [OC][IC] in both layouts (W as it is; phase 0 of the kernel-split layout, the only one with a tap).
+        hipError_t e = launch_pointwise_scatter(s, dY, F, dX, N, OH, OW, OC, IC, sh, sw);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     // the phases as dense stride-1 problems
     struct Phase { GatherConvArgs a; int th, tw, OHt, OWt; };
     std::vector<Phase> phases;

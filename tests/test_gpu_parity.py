@@ -599,6 +599,11 @@ KS_SHAPES = [
     (4, 16, 12, 68, 96, 3, 5, 2, 1, 1, 2),    # two phases (stride along the height only), two blocks of produced channels
     (4, 14, 14, 64, 64, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2: three phases without taps write zeros
     (4, 16, 16, 32, 32, 2, 3, 2, 2, 0, 1),    # filter rows = stride: every phase one tap row
+    # 1x1 filters under a larger stride: one scattered matrix product with zeros in between (its own kernel where IH = sh * OH)
+    (8, 28, 28, 64, 128, 1, 1, 2, 2, 0, 0),   # c4c geometry (56 -> 28 there) at N = 8
+    (3, 9, 12, 132, 96, 1, 1, 3, 2, 0, 0),    # blocks of 3 x 2 pixels, 54 pixels of deltaY (ragged tile), 132 produced channels (ragged block)
+    (2, 6, 20, 8, 32, 1, 1, 1, 4, 0, 0),      # stride along the width only, 8 produced channels
+    (2, 15, 15, 64, 64, 1, 1, 2, 2, 0, 0),    # odd size: the last row and column of deltaX belong to no block -> the phase kernels
 ]
 
 
