@@ -79,6 +79,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
         // ---- load cursor: one step ahead of the multiplications, through (group, phase, tap, 16 channels) ----------------
         int c_tile = tile0, c_th = 0, c_tw = 0, c_ch = 0, c_left = count * steps;
         int org[T], pi[T], pj[T];   // lane l16's coarse pixel of tile i: byte offset of A[n, i, j, 4q], and (i, j)
+        int obase[T];               // where that pixel's results go in O (elements, phase offset and channel apart); dead pixels: beyond O
         unsigned voff[T];           // this tap's load offset, or DCP_NEVER in the padding
         unsigned opix[T][4];        // byte offset of the lane's result pixels 4q + r in O (phase offset apart), or DCP_NEVER
         auto locate = [&]() {
@@ -92,6 +93,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
                 org[i] = (((n * p.AH + ii) * p.AW + jj) * p.AC + 4 * q) * 4;
                 pi[i] = live ? ii : -0x1000000;   // every window row of a dead pixel is outside
                 pj[i] = jj;
+                obase[i] = live ? n * p.o_sn + ii * p.o_sh + jj * p.o_sw : 0x20000000;
             }
         };
         auto aim = [&]() {   // offsets of tap (c_th, c_tw)
@@ -139,17 +141,20 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
         }
         for (int g = 0; g < count; g++) {
             const int tile = tile0 + g * T;
-            // where this lane's results go: pixels 16(tile + i) + 4q + r, produced channels 64 nb + 4 l16 + j
+            if (steps == 0) {   // a phase without taps has no cursor: place the group's pixels here (uniform)
+                c_tile = tile;
+                locate();
+            }
+            // where this lane's results go: pixels 16(tile + i) + 4q + r, produced channels 64 nb + 4 l16 + j. The cursor
+            // worked out every pixel's place in O when it reached this group (lane l16 holds pixel l16's; it moves on to the
+            // next group's only after this group's first request): pixel 4q + r's comes from lane 4q + r, one cross-lane
+            // read instead of two divisions per pixel.
 #pragma unroll
             for (int i = 0; i < T; i++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const int m = (tile + i) * 16 + 4 * q + r;
-                    const bool live = m < p.M && n_ok;
-                    const int mm = m < p.M ? m : 0;
-                    const int n = fdiv(mm, p.d_OHW), rem = mm - n * (int)p.d_OHW.d;
-                    const int ii = fdiv(rem, p.d_OW), jj = rem - ii * (int)p.d_OW.d;
-                    opix[i][r] = live ? (unsigned)((n * p.o_sn + ii * p.o_sh + jj * p.o_sw + n_l) * 4) : DCP_NEVER;
+                    const int ob = __builtin_amdgcn_ds_bpermute((4 * q + r) * 4, obase[i]);
+                    opix[i][r] = n_ok ? (unsigned)((ob + n_l) * 4) : DCP_NEVER;
                 }
             {
                 floatx4 acc[T][4];
