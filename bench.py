@@ -120,6 +120,8 @@ class Workload:
         self.stream = int(torch.cuda.current_stream().cuda_stream)
         self.streams = [self.stream]
         self.engine = pkg.engine.Engine(self.stream)
+        if NO_WORKSPACE:
+            self.engine.config.conv_workspace = 0
         self.dx_plan = pkg.engine.plan_deltaX(self.engine.config, IH, IW, OH, OW, F, F, N, IC, OC, s, s)
         if s > 1:
             cf = (F + s - 1) // s
@@ -245,6 +247,7 @@ class Workload:
                                    N, IC, OC, s, s, p, p)
 
 
+NO_WORKSPACE = False   # --no-workspace: the conv entries as an unmodified Java engine calls them (no scratch lent)
 CLOCK_RAMP_MS = 40.0   # untimed run-in before every measurement; reported in the JSON line
 
 
@@ -410,7 +413,8 @@ def measure(wl, op, steps, warmup, with_parity=True):
     # the conv entry alone (its dominant kernel; HIP events on its stream), with the scratch the host layer lends it
     if getattr(wl, "ws", None) is None:
         wl.ws = torch.empty(1 << 18, device=wl.X.device)
-    pkg.lib().alpha_conv_bind_workspace(wl.ws.data_ptr(), wl.ws.numel() * 4)
+    if wl.engine.config.conv_workspace:
+        pkg.lib().alpha_conv_bind_workspace(wl.ws.data_ptr(), wl.ws.numel() * 4)
     try:
         _, k_ms = time_loop(torch, kernel, steps, max(1, warmup // 2))
     finally:
@@ -569,6 +573,9 @@ def main():
     ap.add_argument("--no-layers", action="store_true", help="leave out the array with every layer/op of BASELINE.json's configs")
     ap.add_argument("--no-parity", action="store_true", help="leave out the per-row comparison with the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-workspace", action="store_true",
+                    help="do not lend the forward / backward-data entries scratch (the host layer's conv_workspace option off): "
+                         "the natives as an unmodified Java engine calls them")
     ap.add_argument("--probe-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy a few times (calibrates FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -578,6 +585,8 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    global NO_WORKSPACE
+    NO_WORKSPACE = args.no_workspace
     import torch
     if args.probe_copy:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0").normal_()
