@@ -46,6 +46,15 @@ static __device__ __forceinline__ void buffer_store_b128_guarded(floatx4 v, __am
     asm volatile("s_nop 1" : "+v"(v));
 }
 
+// Workgroup barrier that orders LDS accesses only: __syncthreads() also waits for every global load and store of the
+// wavefront (its fences cover all address spaces), which stalls a kernel that keeps loads for later in flight.
+static __device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // Bumped by alpha_rt_resetDevice: a device reset drops function attributes and symbol addresses, so whatever this
 // library remembers per device is only valid for the generation it was recorded in.
 inline std::atomic<unsigned> &device_generation()

@@ -98,8 +98,9 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.O, 0, p.o_bytes, 0x00020000);
 
     // `count` groups of T tiles each, from tile0 on, block nb of the produced channels, reduction steps [k_lo, k_lo + k_n)
-    // of every group. SPLIT (count 1, every wavefront of the workgroup calls it with its own steps, k_n >= 0 of either
-    // parity): the wavefronts' partial results are added through LDS. Otherwise k_n is even and at least 2.
+    // of every group. SPLIT (every wavefront of the workgroup calls it with its own steps; count 1 and k_n >= 0 of either
+    // parity, or several groups and k_n even and at least 2): the wavefronts' partial results are added through LDS, and
+    // the first loads of the next group are in flight meanwhile. Otherwise k_n is even and at least 2.
     int ep_nb = -1;   // the block of produced channels the epilogue terms below belong to
     float sub[4], mul[4], add[4];
     floatx4 bias = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -129,7 +130,10 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         }
         floatx4 a[2][T], b[2][4];
         // ---- load cursor: one step ahead of the multiplications, through (group, tap, 16 channels) ----------------------
-        int c_tile = tile0, c_tap = k_lo / CH, c_ch = k_lo - (k_lo / CH) * CH, c_left = count * k_n;
+        // (the division runs on the vector unit; without the explicit move to a scalar register the compiler keeps the whole
+        // cursor, which restarts from these values at every group, in vector registers)
+        const int tap_lo = __builtin_amdgcn_readfirstlane(k_lo / CH), ch_lo = __builtin_amdgcn_readfirstlane(k_lo - tap_lo * CH);
+        int c_tile = tile0, c_tap = tap_lo, c_ch = ch_lo, c_left = count * k_n;
         int org[T];          // byte offset of (this lane's pixel's window origin, channel 4q); may lie before the tensor
         unsigned rc[T];      // bit th: window row th is inside the image; bit 16 + tw: window column tw is
         unsigned voff[T];    // this tap's load offset, or DC_NEVER in the padding
@@ -162,7 +166,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
 #pragma unroll
             for (int i = 0; i < T; i++) voff[i] = (rc[i] & need) == need ? (unsigned)(org[i] + term) : DC_NEVER;
         };
-        auto request = [&](int slot) {
+        auto request = [&](int slot, const bool wrap = false) {   // wrap (SPLIT): these are the loads of a group's last step
             // past the last step the loads repeat the last step's (unused)
             const int a_off = c_ch * 64;
             const int b_off = __builtin_amdgcn_readfirstlane((p.b_off + c_tap * p.b_tap + c_ch * 16 * p.b_k) * 4);
@@ -174,16 +178,24 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                 b[slot][s] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_lane + (unsigned)(s * p.b_k * 4), b_off, 0));
             if (c_left > 1) {   // bookkeeping: scalar, and vector arithmetic without memory operations
                 c_left--;
-                c_ch++;
-                if (c_ch == CH) {
-                    c_ch = 0;
-                    c_tap++;
-                    if (c_tap == taps) {
-                        c_tap = 0;
-                        c_tile += stride;
-                        locate();
-                    }
+                if (SPLIT && wrap) {   // the next group's steps begin at k_lo again
+                    c_tap = tap_lo;
+                    c_ch = ch_lo;
+                    c_tile += stride;
+                    locate();
                     aim();
+                } else {
+                    c_ch++;
+                    if (c_ch == CH) {
+                        c_ch = 0;
+                        c_tap++;
+                        if (!SPLIT && c_tap == taps) {
+                            c_tap = 0;
+                            c_tile += stride;
+                            locate();
+                        }
+                        aim();
+                    }
                 }
             }
         };
@@ -209,7 +221,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[slot][i][s], b[slot][s][j], acc[i][j], 0, 0, 0);
             };
             for (int ks = 0; ks + 1 < k_n; ks += 2) {
-                request(1);
+                request(1, ks + 2 >= k_n);
                 multiply(0);
                 __builtin_amdgcn_sched_barrier(0);
                 request(0);
@@ -248,7 +260,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
 #pragma unroll
                     for (int r = 0; r < 4; r++)
                         part[(w * 4 * DC_SPLIT_T + 4 * i + r) * 64 + lane] = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
-                __syncthreads();
+                lds_barrier();   // orders LDS only: the next group's loads and this group's stores stay in flight across it
                 for (int u = w; u < 4 * T; u += 8) {   // uniform
                     floatx4 v = part[u * 64 + lane];
 #pragma unroll
@@ -261,7 +273,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                         emit(u >> 2, u & 3, v);
                     }
                 }
-                __syncthreads();   // the next group writes `part` again
+                lds_barrier();   // the next group writes `part` again
             }
         }
     };
@@ -324,11 +336,21 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         // first loads and the two barriers for a quarter of the work, with five loads per 16 MFMAs)
         const int run_len = min(g_hi - i, p.tiles - tile0), ngroups = (run_len + DC_SPLIT_T - 1) / DC_SPLIT_T;
         const int cnt = (run_len + ngroups - 1) / ngroups;
-        if (cnt == 4) run(DcInt<4>{}, DcInt<1>{}, nb, tile0, 1, k_lo, k_n, 4);
-        else if (cnt == 3) run(DcInt<3>{}, DcInt<1>{}, nb, tile0, 1, k_lo, k_n, 3);
-        else if (cnt == 2) run(DcInt<2>{}, DcInt<1>{}, nb, tile0, 1, k_lo, k_n, 2);
-        else run(DcInt<1>{}, DcInt<1>{}, nb, tile0, 1, k_lo, k_n, 1);
-        i += cnt;
+        auto groups = [&](const int T, const int first, const int count) {
+            if (T == 4) run(DcInt<4>{}, DcInt<1>{}, nb, first, count, k_lo, k_n, 4);
+            else if (T == 3) run(DcInt<3>{}, DcInt<1>{}, nb, first, count, k_lo, k_n, 3);
+            else if (T == 2) run(DcInt<2>{}, DcInt<1>{}, nb, first, count, k_lo, k_n, 2);
+            else if (T == 1) run(DcInt<1>{}, DcInt<1>{}, nb, first, count, k_lo, k_n, 1);
+        };
+        if ((KS & 15) == 0) {   // every wavefront's part is an even number of steps: groups of one size are one run
+            const int n_big = run_len - ngroups * (cnt - 1);   // groups of cnt tiles, the others have cnt - 1
+            groups(cnt, tile0, n_big);
+            groups(cnt - 1, tile0 + n_big * cnt, ngroups - n_big);
+            i += run_len;
+        } else {
+            groups(cnt, tile0, 1);
+            i += cnt;
+        }
     }
     if constexpr (WS) {
         // this workgroup's piece of an item left over after the equal shares: part z of `split` of the reduction, cut in

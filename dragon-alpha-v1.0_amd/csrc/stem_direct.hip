@@ -146,22 +146,27 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
         auto locate = [&]() {
             bool all_full = true;
             if (p.TPR > 0) {
-                // rows are whole tiles: the image, the output row and with them the window rows are the same for the 16
-                // pixels of a tile (scalar arithmetic); only the columns differ from lane to lane
+                // rows are whole tiles and a group is the same 16 columns of consecutive output rows: the columns - the only
+                // per-lane part - are worked out once per group, the image and the window rows of each tile in scalar
+                // arithmetic
+                const int gidx = __builtin_amdgcn_readfirstlane(T == 4 ? g0 + c_idx : g0 + (c_idx >> 2));
+                const int sb = fdiv(gidx, p.d_TPR), tx = gidx - sb * p.TPR;
+                const int iw0 = (tx * 16 + l16) * p.sw - p.pw;
+                const unsigned cols_in = sd_range_mask(iw0, p.FW, p.IW) << 16;
+                const int col_off = iw0 * 16;
+                bool rows_full = true;
 #pragma unroll
                 for (int i = 0; i < T; i++) {
-                    const int tile = tile_at(c_idx, i);
-                    const bool live = tile < p.tiles;
-                    const int row = fdiv(live ? tile : 0, p.d_TPR), tx = (live ? tile : 0) - row * p.TPR;
-                    const int n = fdiv(row, p.d_OH), oh = row - n * (int)p.d_OH.d;
+                    const int row = 4 * sb + (T == 4 ? i : (c_idx & 3));
+                    const bool live = row < p.rows;
+                    const int n = fdiv(live ? row : 0, p.d_OH), oh = (live ? row : 0) - n * (int)p.d_OH.d;
                     const int ih0 = oh * p.sh - p.ph;
                     const unsigned rows_in = live ? sd_range_mask(ih0, p.FH, p.IH) : 0u;
-                    const int iw0 = (tx * 16 + l16) * p.sw - p.pw;
-                    org[i] = ((n * p.IH + ih0) * p.IW + iw0) * 16;
-                    rc[i] = rows_in | (sd_range_mask(iw0, p.FW, p.IW) << 16);
-                    all_full = all_full && rc[i] == full;
+                    org[i] = __builtin_amdgcn_readfirstlane((n * p.IH + ih0) * p.IW * 16) + col_off;
+                    rc[i] = (unsigned)__builtin_amdgcn_readfirstlane((int)rows_in) | cols_in;
+                    rows_full = rows_full && rows_in == (full & 0xffffu);
                 }
-                c_inside = __all(all_full) != 0;
+                c_inside = rows_full && __all(cols_in == (full & 0xffff0000u)) != 0;
                 return;
             }
 #pragma unroll
