@@ -122,6 +122,8 @@ class Workload:
         self.engine = pkg.engine.Engine(self.stream)
         if NO_WORKSPACE:
             self.engine.config.conv_workspace = 0
+        elif NO_TICKETS:
+            self.engine.config.conv_workspace = 2
         self.dx_plan = pkg.engine.plan_deltaX(self.engine.config, IH, IW, OH, OW, F, F, N, IC, OC, s, s)
         if s > 1:
             cf = (F + s - 1) // s
@@ -247,6 +249,7 @@ class Workload:
                                    N, IC, OC, s, s, p, p)
 
 
+NO_TICKETS = False     # --no-tickets: scratch lent, but the pieces of the items left over are added by a second kernel
 NO_WORKSPACE = False   # --no-workspace: the conv entries as an unmodified Java engine calls them (no scratch lent)
 CLOCK_RAMP_MS = 40.0   # untimed run-in before every measurement; reported in the JSON line
 
@@ -413,11 +416,16 @@ def measure(wl, op, steps, warmup, with_parity=True):
     # the conv entry alone (its dominant kernel; HIP events on its stream), with the scratch the host layer lends it
     if getattr(wl, "ws", None) is None:
         wl.ws = torch.empty(1 << 18, device=wl.X.device)
+        wl.tickets = torch.zeros(128, dtype=torch.int32, device=wl.X.device)   # zero when bound; the kernels leave them zero
+        torch.cuda.synchronize()
     if wl.engine.config.conv_workspace:
         pkg.lib().alpha_conv_bind_workspace(wl.ws.data_ptr(), wl.ws.numel() * 4)
+        if not NO_TICKETS:
+            pkg.lib().alpha_conv_bind_tickets(wl.tickets.data_ptr(), wl.tickets.numel())
     try:
         _, k_ms = time_loop(torch, kernel, steps, max(1, warmup // 2))
     finally:
+        pkg.lib().alpha_conv_bind_tickets(None, 0)
         pkg.lib().alpha_conv_bind_workspace(None, 0)
     fl, by = flops(layer), algorithmic_bytes(layer)
     hbm = fl / by < RIDGE   # below the ridge the HBM roofline binds (c1, c4c), above it the matrix pipes (the 1x1 layers of
@@ -576,6 +584,8 @@ def main():
     ap.add_argument("--no-workspace", action="store_true",
                     help="do not lend the forward / backward-data entries scratch (the host layer's conv_workspace option off): "
                          "the natives as an unmodified Java engine calls them")
+    ap.add_argument("--no-tickets", action="store_true",
+                    help="lend the scratch but no ticket words: the pieces of the items left over are added by a second kernel")
     ap.add_argument("--probe-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy a few times (calibrates FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -585,8 +595,9 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
-    global NO_WORKSPACE
+    global NO_WORKSPACE, NO_TICKETS
     NO_WORKSPACE = args.no_workspace
+    NO_TICKETS = args.no_tickets
     import torch
     if args.probe_copy:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0").normal_()

@@ -40,9 +40,11 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
 // 51 MB output, different ones from run to run). The compiler guards this hazard with wait states only for stores
 // WITHOUT a scalar soffset; here the two wait states follow the store explicitly, tied to the data registers so that no
 // write to them can be scheduled in between.
+// AUX: the instruction's cache-policy bits (16 = sc1: written through to device scope).
+template <int AUX = 0>
 static __device__ __forceinline__ void buffer_store_b128_guarded(floatx4 v, __amdgpu_buffer_rsrc_t rsrc, unsigned voffset, int soffset)
 {
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v), rsrc, voffset, soffset, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v), rsrc, voffset, soffset, AUX);
     asm volatile("s_nop 1" : "+v"(v));
 }
 
@@ -234,7 +236,7 @@ hipError_t launch_pointwise_direct(hipStream_t stream, const float *A, const flo
 hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC,
                               int OHt, int OWt, int CO, int TH, int TW, int sh, int sw, int ph, int pw,
                               int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep,
-                              float *ws = nullptr, size_t ws_bytes = 0);
+                              float *ws = nullptr, size_t ws_bytes = 0, unsigned *tickets = nullptr, int n_tickets = 0);
 bool direct_conv_balanced(long M, int CO, bool workspace = false);
 // Backward-data of a 1x1 layer whose stride exceeds the filter (no padding, IH = sh*OH, IW = sw*OW): the product into every
 // sh x sw block's first pixel, zeros elsewhere (pointwise_scatter.hip). W is [K = OC][N = IC]. hipErrorNotSupported: nothing launched.

@@ -67,6 +67,9 @@ enum FilterLayout { FILTER_W, FILTER_CW };
 // callers never see each other's.
 thread_local float *t_workspace = nullptr;
 thread_local size_t t_workspace_bytes = 0;
+// Ticket words lent with it (alpha_conv_bind_tickets): zero between launches.
+thread_local unsigned *t_tickets = nullptr;
+thread_local int t_tickets_count = 0;
 
 // Debugging switch (tests and comparisons force the generic kernels with it); not part of the drop-in contract. The only
 // mutable process-wide setting of the library: atomic, read once per call, so a call sees one value throughout.
@@ -167,7 +170,7 @@ int forward(const char *fn, const int64_t *streams, int length,
     if (layout == FILTER_CW && (algo == 6 || (algo == 0 && direct_conv_preferred(FH, FW, sh, sw, (long)N * OH * OW, IC, OC)))) {
         // both operands straight from memory
         hipError_t e = launch_direct_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
-                                          0, IC * OC, OC, (long)FH * FW * IC * OC, bias, ep, t_workspace, t_workspace_bytes);
+                                          0, IC * OC, OC, (long)FH * FW * IC * OC, bias, ep, t_workspace, t_workspace_bytes, t_tickets, t_tickets_count);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && sh == 1 && sw == 1 && OH == IH && OW == IW && layout == FILTER_CW && algo != 3 &&
@@ -225,7 +228,7 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
         // both operands straight from memory; W rotated by 180 degrees is read in place (input channel contiguous)
         hipError_t e = launch_direct_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, 1, 1, FH - 1 - ph, FW - 1 - pw,
                                           (FH * FW - 1) * IC, -IC, FH * FW * IC, (long)OC * FH * FW * IC, nullptr, ep,
-                                          t_workspace, t_workspace_bytes);
+                                          t_workspace, t_workspace_bytes, t_tickets, t_tickets_count);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && OH == IH && OW == IW && algo != 3 && pointwise_direct_preferred(OC, IC)) {
@@ -486,6 +489,15 @@ int alpha_conv_bind_workspace(float *workspace, long bytes)
         return fail(ALPHA_CONV_EINVAL, "alpha_conv_bind_workspace: misaligned workspace or negative size");
     t_workspace = workspace;
     t_workspace_bytes = workspace ? (size_t)bytes : 0;
+    return 0;
+}
+
+int alpha_conv_bind_tickets(unsigned *tickets, int count)
+{
+    if (count < 0 || (tickets != nullptr && (reinterpret_cast<uintptr_t>(tickets) & 3) != 0))
+        return fail(ALPHA_CONV_EINVAL, "alpha_conv_bind_tickets: misaligned words or negative count");
+    t_tickets = tickets;
+    t_tickets_count = tickets ? count : 0;
     return 0;
 }
 int alpha_conv_get_fwd_algo(void) { return fwd_algo(); }

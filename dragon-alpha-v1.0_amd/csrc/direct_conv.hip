@@ -41,8 +41,11 @@ struct DirectConvArgs {
     int tiles, nblocks, items, wgs;
     // Shares equal to the item: with a workspace every workgroup takes `base` items and the items_left = items - wgs * base
     // left over are cut `split` ways along the reduction, one piece each for the first items_left * split workgroups; piece
-    // (item e, part z) leaves its partial sums in ws[(e * split + z) * 1024 ..] and direct_conv_fixup_kernel adds them.
+    // (item e, part z) leaves its partial sums in ws[(e * split + z) * 1024 ..]. Who adds them: with `tickets` (one word per
+    // item left over, zero before the launch and after it) the workgroup that delivers an item's last piece; without,
+    // direct_conv_fixup_kernel in a second launch. The order of the addition is z = 0, 1, ... either way.
     float *ws;
+    unsigned *tickets;
     int base, items_left, split;
     FastDiv d_OW, d_OHW, d_TW;
     Epilogue ep;
@@ -52,6 +55,7 @@ template <int V> struct DcInt { static constexpr int value = V; };
 template <bool V> struct DcBool { static constexpr bool value = V; };
 constexpr unsigned DC_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
+constexpr int DC_AUX_SC1 = 16;   // cache-policy bit of the buffer instructions: coherent at device scope (across the XCDs' L2s)
 constexpr int DC_SPLIT_T = 4;   // tiles per group where the workgroup shares the reduction (LDS: 8 x 4 DC_SPLIT_T x 1 KB)
 constexpr size_t DC_LDS_BYTES = 8 * 4 * DC_SPLIT_T * 64 * sizeof(floatx4);
 
@@ -78,6 +82,35 @@ __host__ __device__ inline int dc_whole_items(int n)
     return f < 4 ? 0 : f;
 }
 
+// O[item's 16 pixels][its 64 channels] = epilogue(sum over z < split of ws[(e * split + z)][16][64]), the pieces added in
+// the order z = 0, 1, ...: 256 threads per item left over, a thread per 128-bit store. COHERENT: the pieces were written
+// during this launch, possibly through another XCD's L2 - read them at device scope.
+template <bool COHERENT>
+__device__ __forceinline__ void dc_add_pieces(const DirectConvArgs &p, const int e, const int t)
+{
+    const int row = t >> 4, c4 = t & 15;
+    const int item = p.wgs * p.base + e;
+    const int nb = item / p.tiles, tile = item - nb * p.tiles;
+    const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.ws, 0, p.items_left * p.split * 4096, 0x00020000);
+    const unsigned src = (unsigned)(((e * p.split * 16 + row) * 64 + 4 * c4) * 4);
+    // all pieces requested before the first addition (split <= 8; the loads past the last piece repeat it, unused)
+    floatx4 piece[8];
+#pragma unroll
+    for (int z = 0; z < 8; z++)
+        piece[z] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, src, (z < p.split ? z : p.split - 1) * 4096,
+                                                                                      COHERENT ? DC_AUX_SC1 : 0));
+    floatx4 v = piece[0];
+#pragma unroll
+    for (int z = 1; z < 8; z++)
+        if (z < p.split) v += piece[z];   // uniform
+    const int m = tile * 16 + row, col = nb * 64 + 4 * c4;
+    if (m < p.M && col < p.CO) {
+        const size_t elem = (size_t)m * p.CO + col;
+        const float4 r = epilogue4(make_float4(v[0], v[1], v[2], v[3]), p.ep, col, elem);
+        *reinterpret_cast<float4 *>(p.O + elem) = r;
+    }
+}
+
 template <bool EPI, bool WS = false>
 __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArgs p)
 {
@@ -96,6 +129,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.B), 0, p.b_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.O, 0, p.o_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.ws, 0, WS ? p.items_left * p.split * 4096 : 0, 0x00020000);
 
     // `count` groups of T tiles each, from tile0 on, block nb of the produced channels, reduction steps [k_lo, k_lo + k_n)
     // of every group. SPLIT (every wavefront of the workgroup calls it with its own steps; count 1 and k_n >= 0 of either
@@ -266,9 +300,10 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
 #pragma unroll
                     for (int x = 1; x < 8; x++) v += part[(x * 4 * DC_SPLIT_T + u) * 64 + lane];
                     if constexpr (MODE == 2) {
-                        // row 4 q + (u & 3) of the piece's 16 x 64 block (T == 1), channels 4 l16 .. + 3; `stride` carries the piece
-                        float *dst = p.ws + ((size_t)stride * 16 + 4 * q + (u & 3)) * 64 + 4 * l16;
-                        *reinterpret_cast<floatx4 *>(dst) = v;
+                        // row 4 q + (u & 3) of the piece's 16 x 64 block (T == 1), channels 4 l16 .. + 3; `stride` carries the
+                        // piece. Stored through to device scope (sc1): the workgroup that adds the pieces may sit on another XCD
+                        const unsigned dst = (unsigned)(((stride * 16 + 4 * q + (u & 3)) * 64 + 4 * l16) * 4);
+                        buffer_store_b128_guarded<DC_AUX_SC1>(v, ws_rsrc, dst, 0);
                     } else {
                         emit(u >> 2, u & 3, v);
                     }
@@ -362,26 +397,29 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
             const int parts = 8 * p.split, idx = 8 * z + part_idx;
             const int z_lo = (int)((long)KS * idx / parts), z_n = (int)((long)KS * (idx + 1) / parts) - z_lo;
             run(DcInt<1>{}, DcInt<2>{}, nb, tile0, 1, z_lo, z_n, e * p.split + z);
+            if (p.tickets != nullptr) {   // uniform over the launch
+                // The piece is in memory at device scope once its stores have been acknowledged; then the ticket: the
+                // workgroup that draws the last one of an item adds the pieces, in index order whoever it is. Nobody waits
+                // for anybody. The ticket word is left zero for the next launch.
+                __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+                __builtin_amdgcn_s_barrier();
+                int *last = reinterpret_cast<int *>(dc_smem);   // `part` is free: the group ended with a barrier
+                if (t == 0)
+                    *last = __hip_atomic_fetch_add(p.tickets + e, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(p.split - 1);
+                lds_barrier();
+                if (*last) {   // uniform
+                    if (t < 256) dc_add_pieces<true>(p, e, t);
+                    if (t == 0) __hip_atomic_store(p.tickets + e, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
         }
     }
 }
 
-// O[item's 16 pixels][its 64 channels] = epilogue(sum over z < split of ws[(e * split + z)][16][64]), the pieces added in
-// the order z = 0, 1, ...: one workgroup of 256 threads per item left over, a thread per 128-bit store.
+// The second launch of the form without tickets: one workgroup of 256 threads per item left over.
 __global__ __launch_bounds__(256) void direct_conv_fixup_kernel(const DirectConvArgs p)
 {
-    const int e = blockIdx.x, row = threadIdx.x >> 4, c4 = threadIdx.x & 15;
-    const int item = p.wgs * p.base + e;
-    const int nb = item / p.tiles, tile = item - nb * p.tiles;
-    const float *src = p.ws + ((size_t)e * p.split * 16 + row) * 64 + 4 * c4;
-    floatx4 v = *reinterpret_cast<const floatx4 *>(src);
-    for (int z = 1; z < p.split; z++) v += *reinterpret_cast<const floatx4 *>(src + (size_t)z * 1024);
-    const int m = tile * 16 + row, col = nb * 64 + 4 * c4;
-    if (m < p.M && col < p.CO) {
-        const size_t elem = (size_t)m * p.CO + col;
-        const float4 r = epilogue4(make_float4(v[0], v[1], v[2], v[3]), p.ep, col, elem);
-        *reinterpret_cast<float4 *>(p.O + elem) = r;
-    }
+    dc_add_pieces<false>(p, blockIdx.x, threadIdx.x);
 }
 
 // Share of the SIMDs' time that is work when `items` equal items are dealt to `cus` workgroups as the kernel does: a
@@ -422,10 +460,13 @@ bool direct_conv_balanced(long M, int CO, bool workspace)
 // workgroups and are few per workgroup (fewer than 16: all of them shared by the workgroup's wavefronts) is dealt out in
 // equal shares of whole items, the items left over are cut along the reduction into one piece per workgroup, and a second
 // short launch adds the pieces: 1568 items on 256 workgroups are 6 each + an eighth of one, not 6 or 7.
+// `tickets` (may be NULL), n_tickets: 32-bit words that are zero before the launch, one per item left over (fewer than half
+// the compute units); with them the workgroup that delivers an item's last piece adds the pieces and there is no second
+// launch. The kernel leaves them zero. Launches that share them, like launches that share `ws`, must not overlap.
 hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC,
                               int OHt, int OWt, int CO, int TH, int TW, int sh, int sw, int ph, int pw,
                               int b_off, int b_tap, int b_k, long b_elems, const float *bias, const Epilogue *ep,
-                              float *ws, size_t ws_bytes)
+                              float *ws, size_t ws_bytes, unsigned *tickets, int n_tickets)
 {
     if (AC < 16 || (AC & 15) || CO < 4 || (CO & 3) || TH < 1 || TW < 1 || TH > 16 || TW > 16) return hipErrorNotSupported;
     if (((TH * TW * (AC >> 4)) & 1) != 0) return hipErrorNotSupported;
@@ -464,6 +505,7 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
         if (ws != nullptr && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 && a.items_left > 0 && a.split >= 2 && shared_only &&
             ws_bytes >= (size_t)a.items_left * a.split * 1024 * sizeof(float) && KS * 128 * (a.split - 1) / a.split > 8192 && KS >= 8L * a.split)
             a.ws = ws;
+        a.tickets = a.ws != nullptr && tickets != nullptr && n_tickets >= a.items_left ? tickets : nullptr;
     }
     if (a.ws != nullptr) {
         if (a.ep.fused) {
@@ -473,7 +515,7 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
             if (hipError_t e = ensure_dynamic_lds<direct_conv_kernel<false, true>>(DC_LDS_BYTES); e != hipSuccess) return e;
             hipLaunchKernelGGL((direct_conv_kernel<false, true>), dim3(wgs), dim3(512), DC_LDS_BYTES, stream, a);
         }
-        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+        if (hipError_t e = hipGetLastError(); e != hipSuccess || a.tickets != nullptr) return e;
         hipLaunchKernelGGL(direct_conv_fixup_kernel, dim3(a.items_left), dim3(256), 0, stream, a);
         return hipGetLastError();
     }

@@ -265,6 +265,10 @@ struct alpha_engine {
         }
     };
     std::map<FilterKey, std::pair<size_t, void *>> filter_cache;
+    // Ticket words lent to the library beside the workspace (alpha_conv_bind_tickets): zeroed once here, left zero by
+    // every kernel; all of this engine's kernels run on its one stream, so no two of them use the words at a time.
+    unsigned *tickets = nullptr;
+    static constexpr int n_tickets = 128;
     char err[256];
 };
 
@@ -291,10 +295,14 @@ struct WorkspaceScope {
         if (!e->cfg.conv_workspace) return;
         constexpr size_t bytes = 1u << 20;
         if (void *p = take_block(e, bytes)) bound = alpha_conv_bind_workspace(static_cast<float *>(p), (long)bytes) == 0;
+        if (bound && e->tickets && e->cfg.conv_workspace == 1) alpha_conv_bind_tickets(e->tickets, alpha_engine::n_tickets);
     }
     ~WorkspaceScope()
     {
-        if (bound) alpha_conv_bind_workspace(nullptr, 0);
+        if (bound) {
+            alpha_conv_bind_tickets(nullptr, 0);
+            alpha_conv_bind_workspace(nullptr, 0);
+        }
     }
 };
 
@@ -386,6 +394,11 @@ alpha_engine *alpha_engine_create(int64_t stream)
     e->cfg.conv_workspace = 1;   // and forward / backward-data calls may use a piece of the engine's scratch (see the header)
     e->stream = stream;
     e->err[0] = 0;
+    void *words = nullptr;
+    if (cu > 0 && hipMalloc(&words, alpha_engine::n_tickets * sizeof(unsigned)) == hipSuccess) {
+        if (hipMemset(words, 0, alpha_engine::n_tickets * sizeof(unsigned)) == hipSuccess) e->tickets = static_cast<unsigned *>(words);
+        else (void)hipFree(words);
+    }
     return e;
 }
 
@@ -405,6 +418,7 @@ void alpha_engine_destroy(alpha_engine *e)
     alpha_engine_sync(e);
     for (auto &b : e->free_blocks) (void)hipFree(b.second);
     for (auto &b : e->filter_cache) (void)hipFree(b.second.second);
+    if (e->tickets) (void)hipFree(e->tickets);
     delete e;
 }
 

@@ -66,6 +66,12 @@ int alpha_conv_get_fwd_algo(void);
  * bit-identical from run to run, and differ from the unbound path's in the last bits of those items only). Per thread:
  * concurrent callers do not see each other's binding. */
 int alpha_conv_bind_workspace(float *workspace, long bytes);
+/* No counterpart in the reference. Beside a bound workspace: `count` 32-bit words of device memory (128 cover every layer)
+ * that are ZERO when bound and that only this library's kernels write until NULL is bound again; every kernel leaves them
+ * zero. With them the pieces of the items left over are added by the workgroup that delivers an item's last piece - a
+ * ticket per item decides WHO adds, never the order, so the bits are those of the second kernel - and the second launch
+ * is saved. Kernels that share the words must not overlap on the device (the rule of the workspace). Per thread. */
+int alpha_conv_bind_tickets(unsigned *tickets, int count);
 /* Debugging switch of the same kind for 1x1 stride-1 forward / backward-data where the kernel of direct_conv.hip does not
  * take the layer: -1 = chosen by shape, 0 = the filter-resident kernel, 1 = the kernel without LDS wherever it fits.
  * Also read once from the environment variable ALPHA_PW_DIRECT = 0|1. No counterpart in the reference. */

@@ -54,7 +54,9 @@ typedef struct alpha_engine_config {
     int conv_workspace;           /* this build only: 1 = forward and stride-1 backward-data calls lend the library 1 MiB of the engine's
                                      scratch for the duration of the call (alpha_conv_bind_workspace), with which the kernel without
                                      LDS deals a layer of few items per compute unit out in equal shares (7x7x512 and 14x14x256 maps at
-                                     N = 64: 6 and 12 items each plus a piece of one, instead of 6 or 7 and 12 or 13).
+                                     N = 64: 6 and 12 items each plus a piece of one, instead of 6 or 7 and 12 or 13), and the engine's
+                                     ticket words (alpha_conv_bind_tickets), with which the pieces are added inside that kernel;
+                                     2 = the scratch without the ticket words (a second short kernel adds the pieces).
                                      alpha_engine_config_default: 0; alpha_engine_create: 1 */
 } alpha_engine_config;
 

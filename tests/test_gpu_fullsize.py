@@ -240,3 +240,47 @@ def test_reference_criterion_deltaW_full_size(dev, layer, mode):
     ocs = sorted({0, 1, OC // 2 + 1, OC - 1})
     want = O.deltaW_naive(X.numpy(), np.ascontiguousarray(dY.numpy()[..., ocs]), F, F, s, s, p, p)
     _same_percent(dw[ocs].cpu().numpy(), want, 1e-5, 1.0, "%s deltaW (%s, GridZ %d)" % (layer, mode, plan.GridZ))
+
+
+# ----------------------------------------------------------------------------------------------
+# The items left over after equal shares (c3c: 64 items in 4 pieces, c3d: 32 in 8): added by a second kernel, or - with
+# ticket words, what an engine object lends - by whichever workgroup delivers an item's last piece. Who adds must not
+# show in the bits: the whole output is compared bit for bit, over several launches (the workgroup that comes last
+# changes from launch to launch), and the ticket words are zero afterwards.
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("layer", ["c3c", "c3d"])
+def test_pieces_added_by_last_workgroup_equal_second_kernel_full_size(dev, layer):
+    torch = dev.torch
+    L = pkg.lib()
+    C3 = pkg.Cuda_conv3D
+    N, IH, IW, IC, OC, F, s, p, _, _ = LAYERS[layer]
+    X, W, _, OH, OW = _tensors(dev, layer, 8301)
+    x, w = X.to(dev.dev), W.to(dev.dev)
+    cw = torch.empty(F * F * IC * OC, device=dev.dev)
+    C3.kernel_remode(dev.stream, w.data_ptr(), cw.data_ptr(), F, F, OC, IC)
+    ws = torch.full((1 << 18,), float("nan"), device=dev.dev)
+    tickets = torch.zeros(128, dtype=torch.int32, device=dev.dev)
+
+    def forward():
+        y = torch.full((N, OH, OW, OC), float("nan"), device=dev.dev)
+        C3.conv3D_GemmR(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), cw.data_ptr(), F, F, y.data_ptr(), OH, OW, N, IC, OC, s, s, p, p)
+        dev.sync()
+        return y
+
+    try:
+        assert L.alpha_conv_bind_workspace(ws.data_ptr(), ws.numel() * 4) == 0
+        second_kernel = forward()
+        assert L.alpha_conv_bind_tickets(tickets.data_ptr(), tickets.numel()) == 0
+        for k in range(6):
+            ws.fill_(float("nan"))
+            got = forward()
+            assert torch.equal(got.view(torch.int32), second_kernel.view(torch.int32)), "%s launch %d: bits differ" % (layer, k)
+            assert int(tickets.abs().sum().item()) == 0, "%s launch %d: ticket words not left zero" % (layer, k)
+    finally:
+        L.alpha_conv_bind_tickets(None, 0)
+        L.alpha_conv_bind_workspace(None, 0)
+    if pkg.device_info()[0] == 256:
+        assert not bool(torch.isnan(ws[:32 * 8 * 1024]).any()), "the pieces were not written: the path did not run"
+    imgs = [0, N - 1]
+    want = O.conv3D_f64(np.ascontiguousarray(X.numpy()[imgs]), W.numpy(), s, s, p, p)
+    _check(second_kernel[imgs].cpu().numpy(), want, "%s forward, equal shares" % layer)

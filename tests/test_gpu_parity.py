@@ -1112,9 +1112,28 @@ def test_forward_and_deltaX_with_bound_workspace(dev, shape):
         got_yb = forward(True)
         ws.fill_(float("nan"))
         got_dx = backward()
+        # with ticket words the workgroup that delivers an item's last piece adds the pieces (no second kernel): the
+        # same order of addition, so the same bits; the words are zero again after every launch
+        tickets = torch.zeros(128, dtype=torch.int32, device=ws.device)
+        assert L.alpha_conv_bind_tickets(tickets.data_ptr(), 128) == 0
+        ws.fill_(float("nan"))
+        ticket_y = [forward(False) for _ in range(3)]
+        ticket_used = ws[:max(1, left * split * 1024)].clone()
+        ticket_yb = forward(True)
+        ticket_dx = [backward() for _ in range(2)]
+        dev.sync()
+        assert int(tickets.abs().sum().item()) == 0, "ticket words not left zero"
     finally:
+        L.alpha_conv_bind_tickets(None, 0)
         L.alpha_conv_bind_workspace(None, 0)
     dev.check_guards(ws)
+    for k, ty in enumerate(ticket_y):
+        assert np.array_equal(ty.view(np.uint32), got_y.view(np.uint32)), "forward with tickets, run %d: bits differ from the second kernel's" % k
+    assert np.array_equal(ticket_yb.view(np.uint32), got_yb.view(np.uint32)), "forward with tickets and bias"
+    for k, tdx in enumerate(ticket_dx):
+        assert np.array_equal(tdx.view(np.uint32), got_dx.view(np.uint32)), "backward-data with tickets, run %d" % k
+    if pkg.device_info()[0] == 256 and left:
+        assert not bool(torch.isnan(ticket_used).any())
     check(got_y, want_y, "forward with workspace %s" % (shape,))
     check(got_yb, want_y + B.astype(np.float64), "forward with workspace and bias %s" % (shape,))
     check(got_dx, want_dx, "backward-data with workspace %s" % (shape,))
