@@ -272,8 +272,8 @@ __global__ __launch_bounds__(512, 1) void stem_direct_kernel(const StemDirectArg
 #pragma unroll
                             for (int j = 0; j < 4; j++) v[j] = ep_finish(v[j], sub[j], mul[j], add[j], p.ep.slope);
                         }
-                    } else if (p.ep.bias != nullptr) {   // uniform
-                        v += bias;
+                    } else {
+                        v += bias;   // zeros without a bias: the additions gather the lane's four channels into the store's registers anyway
                     }
                     buffer_store_b128_guarded(v, y_rsrc, o_lane, o_off);
                 }
