@@ -595,6 +595,8 @@ KS_SHAPES = [
     # the kernel without LDS: phases of one size (IH % sh == 0, IW % sw == 0), deltaY channels a multiple of 32
     (16, 56, 56, 64, 128, 3, 3, 2, 2, 1, 1),  # 12544 coarse pixels = 784 tiles: shares of 0 and 1 item
     (6, 30, 34, 36, 64, 3, 3, 2, 2, 1, 1),    # 1530 coarse pixels (last tile ragged), a ragged block of 36 produced channels
+    (40, 56, 56, 32, 64, 3, 3, 2, 2, 1, 1),   # 1960 tiles: shares of several items per SIMD
+    (24, 60, 52, 36, 32, 5, 5, 2, 2, 2, 2),   # the same with phases of 9, 6, 6 and 4 taps, ragged channels and a ragged last tile
     (4, 12, 16, 64, 32, 3, 3, 1, 2, 1, 1),    # two phases (stride along the width only)
     (4, 16, 12, 68, 96, 3, 5, 2, 1, 1, 2),    # two phases (stride along the height only), two blocks of produced channels
     (4, 14, 14, 64, 64, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2: three phases without taps write zeros
