@@ -170,7 +170,10 @@ hipError_t launch_bn_field_sums(hipStream_t s, int form, const float *dY, const 
     const int capacity = bn_field_nextN(N, M);   // chunks the buffers can hold
     int chunks = 1;
     if (capacity > 1 && bufA && bufB) {
-        chunks = (2048 + col_tiles - 1) / col_tiles;           // enough workgroups for the device, whatever the channel count
+        // two workgroups per compute unit, whatever the channel count: more chunks only lengthen the second kernel's sums
+        // (200704 x 64: operator 0.0623 ms with 2048 chunks, 0.0572 with 1024, 0.0544 with 512, 0.0556 with 256)
+        const int cus = device_cu_count();
+        chunks = (2 * (cus > 0 ? cus : 256) + col_tiles - 1) / col_tiles;
         if (chunks > capacity) chunks = capacity;
         if (chunks > (N + 15) / 16) chunks = (N + 15) / 16;     // sixteen rows per chunk at least
     }
