@@ -30,16 +30,19 @@ def check(got, want, what):
 
 
 GRAPH_SHAPES = [
-    # N, IH, IW, IC, OC, F, s, p, GridZ, backward-data?
-    (32, 28, 28, 64, 64, 3, 1, 1, 32, True),
-    (8, 64, 64, 4, 64, 7, 2, 3, 8, False),
+    # N, IH, IW, IC, OC, F, s, p, GridZ, backward-data?, scratch and ticket words lent?
+    (32, 28, 28, 64, 64, 3, 1, 1, 32, True, False),
+    (8, 64, 64, 4, 64, 7, 2, 3, 8, False, False),
+    # 784 work items on 256 compute units: with the scratch three each and 16 left over, whose pieces the workgroup that
+    # delivers the last one adds - the ticket words must be zero again after every replay for the next one to be right
+    (16, 14, 14, 256, 256, 3, 1, 1, 8, True, True),
 ]
 
 
 @pytest.mark.parametrize("shape", GRAPH_SHAPES)
 def test_natives_replayed_from_a_graph(dev, shape):
     torch = dev.torch
-    N, IH, IW, IC, OC, F_, s_, p_, GridZ, with_dx = shape
+    N, IH, IW, IC, OC, F_, s_, p_, GridZ, with_dx, lend = shape
     OH, OW = out_dim(IH, IW, F_, F_, s_, s_, p_, p_)
     sizeW = OC * F_ * F_ * IC
     x = dev.empty(N, IH, IW, IC, fill=0.0)
@@ -84,6 +87,26 @@ def test_natives_replayed_from_a_graph(dev, shape):
         check(dw.cpu().numpy(), O.deltaW_f64(X, dY, F_, F_, s_, s_, p_, p_), "backward-filter, %s %s" % (what, shape))
         assert torch.equal(dw.view(torch.int32), dw_static.view(torch.int32)), "static-scratch backward-filter, %s %s" % (what, shape)
 
+    ws = dev.empty(1 << 18, fill=float("nan"))
+    tickets = torch.zeros(128, dtype=torch.int32, device=ws.device)
+    torch.cuda.synchronize()
+    L = pkg.lib()
+    if lend:
+        assert L.alpha_conv_bind_workspace(ws.data_ptr(), ws.numel() * 4) == 0
+        assert L.alpha_conv_bind_tickets(tickets.data_ptr(), tickets.numel()) == 0
+    try:
+        _capture_and_replay(dev, torch, step, fresh, verify)
+        if lend:
+            torch.cuda.synchronize()
+            assert int(tickets.abs().sum().item()) == 0, "ticket words not left zero"
+            if pkg.device_info()[0] == 256:
+                assert not bool(torch.isnan(ws[:16 * 8 * 1024]).any()), "the pieces were not written: the path did not run"
+    finally:
+        L.alpha_conv_bind_tickets(None, 0)
+        L.alpha_conv_bind_workspace(None, 0)
+
+
+def _capture_and_replay(dev, torch, step, fresh, verify):
     side = torch.cuda.Stream()
     # eager first, on the stream that will capture: per-kernel attributes (dynamic LDS limits) are set on a kernel's first launch
     data = fresh(4100)
