@@ -413,3 +413,39 @@ def test_engine_random_3x3_stride1_layers(dev, eng, case):
         assert p3.entry_name == "dconv3D_deltaW_GemmSK_winograd"
     check(dev.get(dw2), O.deltaW_f64(X, dY, 3, 3, 1, 1, ph, pw), "Winograd deltaW %s" % (case,))
 
+
+
+DECONV_CASES = [
+    # N, input H, W, input channels (= OC of the filter W[OC, FH, FW, IC]), produced channels (= IC), FH, FW, sh, sw, ph, pw
+    (8, 14, 14, 64, 32, 4, 4, 2, 2, 1, 1),    # the usual 2x up-sampling: 14x14 -> 28x28
+    (4, 16, 16, 32, 64, 3, 3, 1, 1, 1, 1),    # stride 1: a 3x3 convolution with the rotated, transposed filter
+    (4, 9, 7, 32, 16, 3, 3, 2, 2, 0, 0),      # no padding, odd sizes: 9x7 -> 19x15
+]
+
+
+@pytest.mark.parametrize("case", DECONV_CASES)
+def test_engine_transposed_convolution_unit(dev, eng, case):
+    """The reference's Deconv3D unit is the same three operators with the roles swapped (nn/unit/simple/Deconv3D.java:141-176,
+    Engine.java:1819-1852): forward = dconv3D_deltaX of its input, gradient of W = dconv3D_deltaW with the unit's deltaY as
+    X and its input as deltaY, gradient of the input = conv3D of deltaY. Each against the oracle, and the pair
+    (forward, input gradient) against each other: <forward(X), dY> = <X, backward(dY)> for any X, dY."""
+    N, H, Wd, C_in, C_out, FH, FW, sh, sw, ph, pw = case
+    OH, OW = (H - 1) * sh + FH - 2 * ph, (Wd - 1) * sw + FW - 2 * pw     # Deconv3D.java:144-145
+    X, Wt, dYu = normal((N, H, Wd, C_in), 6101), he_normal(C_in, FH, FW, C_out, 6102), normal((N, OH, OW, C_out), 6103)
+    x, w, dyu = dev.put(X), dev.put(Wt), dev.put(dYu)
+    y = dev.empty(N, OH, OW, C_out, fill=float("nan"))
+    dw = dev.empty(C_in, FH, FW, C_out, fill=float("nan"))
+    dx = dev.empty(N, H, Wd, C_in, fill=float("nan"))
+    # in the operators' own terms the convolution is [N, OH, OW, IC = C_out] -> [N, H, Wd, OC = C_in]
+    eng.dconv3D_deltaX(y.data_ptr(), OH, OW, x.data_ptr(), H, Wd, w.data_ptr(), FH, FW, N, C_out, C_in, sh, sw, ph, pw)
+    eng.dconv3D_deltaW(dw.data_ptr(), FH, FW, dyu.data_ptr(), OH, OW, x.data_ptr(), H, Wd, N, C_out, C_in, sh, sw, ph, pw)
+    eng.conv3D(dx.data_ptr(), H, Wd, dyu.data_ptr(), OH, OW, w.data_ptr(), FH, FW, N, C_out, C_in, sh, sw, ph, pw)
+    eng.sync()
+    got_y, got_dw, got_dx = dev.get(y), dev.get(dw), dev.get(dx)
+    check(got_y, O.deltaX_f64(X, Wt, OH, OW, sh, sw, ph, pw), "transposed convolution forward %s" % (case,))
+    check(got_dw, O.deltaW_f64(dYu, X, FH, FW, sh, sw, ph, pw), "transposed convolution, gradient of W %s" % (case,))
+    check(got_dx, O.conv3D_f64(dYu, Wt, sh, sw, ph, pw), "transposed convolution, gradient of the input %s" % (case,))
+    lhs = float(np.sum(got_y.astype(np.float64) * dYu))
+    rhs = float(np.sum(X.astype(np.float64) * got_dx))
+    scale = float(np.sqrt(np.sum(got_y.astype(np.float64) ** 2) * np.sum(dYu.astype(np.float64) ** 2)))
+    assert abs(lhs - rhs) <= 1e-5 * scale, "adjointness: %.9g against %.9g" % (lhs, rhs)
