@@ -40,7 +40,7 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
 // 51 MB output, different ones from run to run). The compiler guards this hazard with wait states only for stores
 // WITHOUT a scalar soffset; here the two wait states follow the store explicitly, tied to the data registers so that no
 // write to them can be scheduled in between.
-// AUX: the instruction's cache-policy bits (16 = sc1: written through to device scope).
+// AUX: the instruction's cache-policy bits (16 = sc1: written through to device scope; 2 = nt: non-temporal, streamed).
 template <int AUX = 0>
 static __device__ __forceinline__ void buffer_store_b128_guarded(floatx4 v, __amdgpu_buffer_rsrc_t rsrc, unsigned voffset, int soffset)
 {

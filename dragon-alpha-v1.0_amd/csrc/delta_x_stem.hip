@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256, 2) void delta_x_stem_kernel(const DxStemArgs p
         deposit();             // next block's halo (requested before the MFMA loop) -> LDS
 #pragma unroll
         for (int j = 0; j < NJ; j++)
-            buffer_store_b128_guarded(out[j], x_rsrc, out_off[j], 0);
+            buffer_store_b128_guarded<2>(out[j], x_rsrc, out_off[j], 0);   // non-temporal: streamed out
         request(blk + 2 * G8);
         __syncthreads();
     }

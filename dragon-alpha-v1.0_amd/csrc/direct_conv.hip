@@ -279,7 +279,9 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                 } else {
                     v += bias;
                 }
-                buffer_store_b128_guarded(v, o_rsrc, o_lane, o_off);
+                // non-temporal: the output is streamed out, nothing of it is read again here, and it does not displace the
+                // input's and the filter's lines from L2 (1x1, 256 -> 1024 channels: 0.0523 -> 0.0508 ms; 56x56x64 3x3: 0.1097 -> 0.1087)
+                buffer_store_b128_guarded<2>(v, o_rsrc, o_lane, o_off);
             };
             if constexpr (!SPLIT) {
 #pragma unroll

@@ -190,7 +190,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
 #pragma unroll
                             for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
                         }
-                        buffer_store_b128_guarded(v, o_rsrc, opix[i][r], o_off);
+                        buffer_store_b128_guarded<2>(v, o_rsrc, opix[i][r], o_off);   // non-temporal, as in direct_conv.hip
                     }
             }
         }
