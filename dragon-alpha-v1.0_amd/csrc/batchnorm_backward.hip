@@ -140,7 +140,8 @@ __global__ __launch_bounds__(256) void bn_delta_x_kernel(const BnArgs p, const f
             if (c + j >= p.width || v != v) v = 0.f;
             r[j] = v;
         }
-        *reinterpret_cast<float4 *>(dX + 4 * i) = make_float4(r[0], r[1], r[2], r[3]);
+        // streamed out (non-temporal store: 0.0328 -> 0.0321 ms on 200704 x 64; non-temporal loads of the two inputs cost 6 %)
+        __builtin_nontemporal_store(floatx4{r[0], r[1], r[2], r[3]}, reinterpret_cast<floatx4 *>(dX + 4 * i));
     }
 }
 
