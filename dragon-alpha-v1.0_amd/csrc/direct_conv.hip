@@ -141,7 +141,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     // The groups of a run begin `stride` tiles apart (T: one after the other).
     auto run = [&](auto tc, auto sp, const int nb, const int tile0, const int count, const int k_lo, const int k_n, const int stride) {
         constexpr int T = decltype(tc)::value;
-        constexpr int MODE = decltype(sp)::value;   // 0: whole items; 1: shared by the workgroup; 2: the same, sums to the workspace
+        constexpr int MODE = decltype(sp)::value;   // 0: whole items; 1: shared by the workgroup; 2: the same, sums to the workspace; 3: shared by a SIMD's two wavefronts
         constexpr bool SPLIT = MODE != 0;
         if (count <= 0) return;
         const int n_l = nb * 64 + 4 * l16;
@@ -288,6 +288,27 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                 for (int i = 0; i < T; i++)
 #pragma unroll
                     for (int r = 0; r < 4; r++) emit(i, r, floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]});
+            } else if constexpr (MODE == 3) {
+                // The SIMD's two wavefronts (w and w ^ 4) hold the sums over the first and the second half of the steps:
+                // each keeps every other unit u = 4 i + r (w < 4 the even ones), hands the rest to its partner through
+                // LDS, adds what it receives and stores its units. One barrier pair per workgroup.
+                static_assert(T <= DC_SPLIT_T, "LDS holds 4 DC_SPLIT_T units per wavefront");
+                const int keep = w >> 2;
+#pragma unroll
+                for (int i = 0; i < T; i++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (((4 * i + r) & 1) != keep)   // uniform
+                            part[(w * 4 * DC_SPLIT_T + 4 * i + r) * 64 + lane] = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+                lds_barrier();
+#pragma unroll
+                for (int i = 0; i < T; i++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (((4 * i + r) & 1) == keep)   // uniform
+                            emit(i, r, floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]} +
+                                           part[((w ^ 4) * 4 * DC_SPLIT_T + 4 * i + r) * 64 + lane]);
+                lds_barrier();   // whoever writes `part` next
             } else {
                 // unit u = 4 i + r (one 128-bit store per lane); partial results [wavefront][unit][lane]
                 static_assert(T <= DC_SPLIT_T, "LDS holds 4 DC_SPLIT_T units per wavefront");
@@ -337,7 +358,17 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         }
     };
     const int nb_first = g_lo / p.tiles;
-    if (f > 0 && g_lo + 4 * f <= (nb_first + 1) * p.tiles) {   // uniform
+    // 8 to 15 items (no whole items: one or two per wavefront would be groups of a single tile): every SIMD takes a group
+    // of two or three tiles of its own, the steps halved between its two wavefronts - an eighth of the steps per
+    // wavefront, as where all eight share a group, costs each of them the group's pixel arithmetic for an eighth of its
+    // MFMAs (14x14x256 at N = 64, 12 items per workgroup: 0.50 vector instructions per MFMA).
+    const int pc = (f == 0 && g_hi - g_lo >= 8 && g_lo + 4 * ((g_hi - g_lo) >> 2) <= (nb_first + 1) * p.tiles) ? (g_hi - g_lo) >> 2 : 0;
+    if (pc > 0) {   // uniform
+        const int tile0 = g_lo - nb_first * p.tiles + (w & 3) * pc;
+        const int h_lo = (w >> 2) ? KS / 2 : 0, h_n = (w >> 2) ? KS - KS / 2 : KS / 2;
+        if (pc == 3) run(DcInt<3>{}, DcInt<3>{}, nb_first, tile0, 1, h_lo, h_n, 3);
+        else run(DcInt<2>{}, DcInt<3>{}, nb_first, tile0, 1, h_lo, h_n, 2);
+    } else if (f > 0 && g_lo + 4 * f <= (nb_first + 1) * p.tiles) {   // uniform
         const int t0 = g_lo - nb_first * p.tiles;
         int n4, n3, n2, n1;
         groups_of(f >> 1, n4, n3, n2, n1);
@@ -366,7 +397,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     // the workgroup's items left over (uniform over the workgroup: every wavefront meets the same barriers)
     const int part_idx = 2 * (w & 3) + (w >> 2);
     const int k_lo = KS * part_idx / 8, k_n = KS * (part_idx + 1) / 8 - k_lo;
-    int i = g_lo + 4 * f;
+    int i = g_lo + 4 * (pc > 0 ? pc : f);
     while (i < g_hi) {
         const int nb = i / p.tiles, tile0 = i - nb * p.tiles;
         // groups of sizes equal to within one tile (13 tiles: 4 + 3 + 3 + 3, not 4 + 4 + 4 + 1: a group of one tile pays the
