@@ -47,6 +47,7 @@ struct DirectConvArgs {
     float *ws;
     unsigned *tickets;
     int base, items_left, split;
+    int xcd_major;   // shares dealt XCD by XCD (see the kernel)
     FastDiv d_OW, d_OHW, d_TW;
     Epilogue ep;
 };
@@ -119,8 +120,12 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     const int t = threadIdx.x, lane = t & 63;
     const int l16 = lane & 15, q = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int g_lo = WS ? (int)blockIdx.x * p.base : (int)((long)p.items * blockIdx.x / p.wgs);
-    const int g_hi = WS ? g_lo + p.base : (int)((long)p.items * (blockIdx.x + 1) / p.wgs);
+    // Workgroups go round-robin to the eight XCDs, each with its own L2. Where a workgroup holds few items and the filter
+    // is larger than an L2 (xcd_major) share sb of the line of items goes to workgroup (sb % (wgs / 8)) * 8 +
+    // sb / (wgs / 8): an XCD's workgroups then hold neighbouring shares, one or two blocks' filters per L2 instead of all.
+    const int sb = p.xcd_major ? (int)(blockIdx.x & 7) * (p.wgs >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    const int g_lo = WS ? sb * p.base : (int)((long)p.items * sb / p.wgs);
+    const int g_hi = WS ? g_lo + p.base : (int)((long)p.items * (sb + 1) / p.wgs);
     const int f = dc_whole_items(g_hi - g_lo);
     const int i_lo = g_lo + (w & 3) * f + (w >> 2) * (f >> 1), i_hi = i_lo + (f >> 1);
     const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group: even (host-checked)
@@ -524,6 +529,10 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
     a.ep = ep ? *ep : bias_epilogue(bias);
     const int wgs = cus < a.items ? cus : a.items;   // one workgroup of eight wavefronts per compute unit
     a.wgs = wgs;
+    // few items per workgroup and a filter beyond an XCD's 4 MB of L2: every workgroup streams its blocks' filter slices, and
+    // an XCD whose workgroups hold all blocks at once fetches them again and again (7x7x512 -> 512 at N = 64, 9.4 MB of
+    // filter: 313 MB of L2 fills; 124 MB with an XCD's workgroups on neighbouring shares, at the same speed or 0.5 % better)
+    a.xcd_major = (wgs & 7) == 0 && a.nblocks > 1 && a.items / wgs < 16 && b_bytes > (4L << 20) ? 1 : 0;
     a.ws = nullptr;
     a.base = a.items / wgs;
     a.items_left = a.items - a.base * wgs;
