@@ -13,7 +13,7 @@ headline's parity, `winograd`, `parity_summary`, `cpu_baseline` and `layers_min`
 Before it, every layer and operator of BASELINE.json's five configs is printed as a JSON line of its own, as soon as it
 is measured (same step count as the headline): its time, its roofline fractions and its parity against the fp64 CPU
 oracle on a subset of the same seeded tensors (images for forward / backward-data, output channels over the full batch
-for backward-filter), with the tolerance it is held to. The same rows go to gpurun_out/bench_layers.json as one array.
+for backward-filter), with the tolerance it is held to. The same rows are also written to a file, as one array.
 --no-layers leaves them out.
 The cpu_baseline leg times the CPU oracle's float-accumulate direct loops on a bounded sample on the host cores
 (baseline only, never a target): the headline operator on all cores, backward-data and backward-filter of c5b on all
