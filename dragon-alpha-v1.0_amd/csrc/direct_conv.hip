@@ -126,9 +126,12 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     const int sb = p.xcd_major ? (int)(blockIdx.x & 7) * (p.wgs >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
     const int g_lo = WS ? sb * p.base : (int)((long)p.items * sb / p.wgs);
     const int g_hi = WS ? g_lo + p.base : (int)((long)p.items * (sb + 1) / p.wgs);
-    const int f = dc_whole_items(g_hi - g_lo);
+    // An odd number of steps per item (48 channels under a 3x3 filter: 27): the loop over whole items multiplies two steps
+    // per turn, so such a layer has no whole items - all of them are shared, in runs of a single group, whose parts
+    // may be odd.
+    const int f = (((p.AC >> 4) * p.TH * p.TW) & 1) ? 0 : dc_whole_items(g_hi - g_lo);
     const int i_lo = g_lo + (w & 3) * f + (w >> 2) * (f >> 1), i_hi = i_lo + (f >> 1);
-    const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group: even (host-checked)
+    const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group
     const bool pointwise = taps == 1 && p.sh == 1 && p.sw == 1 && p.ph == 0 && p.pw == 0;
 
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
@@ -367,11 +370,12 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     // of two or three tiles of its own, the steps halved between its two wavefronts - an eighth of the steps per
     // wavefront, as where all eight share a group, costs each of them the group's pixel arithmetic for an eighth of its
     // MFMAs (14x14x256 at N = 64, 12 items per workgroup: 0.50 vector instructions per MFMA).
-    const int pc = (f == 0 && g_hi - g_lo >= 8 && g_lo + 4 * ((g_hi - g_lo) >> 2) <= (nb_first + 1) * p.tiles) ? (g_hi - g_lo) >> 2 : 0;
+    const int pc = (f == 0 && g_hi - g_lo >= 8 && g_hi - g_lo < 20 && g_lo + 4 * ((g_hi - g_lo) >> 2) <= (nb_first + 1) * p.tiles) ? (g_hi - g_lo) >> 2 : 0;
     if (pc > 0) {   // uniform
         const int tile0 = g_lo - nb_first * p.tiles + (w & 3) * pc;
         const int h_lo = (w >> 2) ? KS / 2 : 0, h_n = (w >> 2) ? KS - KS / 2 : KS / 2;
-        if (pc == 3) run(DcInt<3>{}, DcInt<3>{}, nb_first, tile0, 1, h_lo, h_n, 3);
+        if (pc == 4) run(DcInt<4>{}, DcInt<3>{}, nb_first, tile0, 1, h_lo, h_n, 4);
+        else if (pc == 3) run(DcInt<3>{}, DcInt<3>{}, nb_first, tile0, 1, h_lo, h_n, 3);
         else run(DcInt<2>{}, DcInt<3>{}, nb_first, tile0, 1, h_lo, h_n, 2);
     } else if (f > 0 && g_lo + 4 * f <= (nb_first + 1) * p.tiles) {   // uniform
         const int t0 = g_lo - nb_first * p.tiles;
@@ -492,8 +496,8 @@ bool direct_conv_balanced(long M, int CO, bool workspace)
 // O[N, OHt, OWt, CO] = convolution of A[N, AH, AW, AC] (stride sh x sw, padding ph x pw, TH x TW taps) with the filter B
 // whose element (tap = th * TW + tw, c, co) is at b_off + tap * b_tap + c * b_k + co: CW[FH, FW, IC, OC] forward
 // (0, IC * OC, OC), W[OC, FH, FW, IC] rotated by 180 degrees for stride-1 backward-data ((FH*FW - 1) * IC, -IC, FH*FW*IC).
-// Returns hipErrorNotSupported (nothing launched) when the layer does not fit: AC not a multiple of 16, an odd number
-// of steps (TH * TW * AC / 16), a filter beyond 16 x 16, tensors of 2 GB.
+// Returns hipErrorNotSupported (nothing launched) when the layer does not fit: AC not a multiple of 16, a filter beyond
+// 16 x 16, tensors of 2 GB. (An odd number of steps TH * TW * AC / 16 is taken, without whole items: see the kernel.)
 // `ws` (may be NULL), ws_bytes: scratch for the duration of the launch. With it, a layer whose items do not divide by the
 // workgroups and are few per workgroup (fewer than 16: all of them shared by the workgroup's wavefronts) is dealt out in
 // equal shares of whole items, the items left over are cut along the reduction into one piece per workgroup, and a second
@@ -507,7 +511,6 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
                               float *ws, size_t ws_bytes, unsigned *tickets, int n_tickets)
 {
     if (AC < 16 || (AC & 15) || CO < 4 || (CO & 3) || TH < 1 || TW < 1 || TH > 16 || TW > 16) return hipErrorNotSupported;
-    if (((TH * TW * (AC >> 4)) & 1) != 0) return hipErrorNotSupported;
     const long M = (long)N * OHt * OWt;
     const long a_bytes = (long)N * AH * AW * AC * 4, b_bytes = b_elems * 4, o_bytes = M * CO * 4;
     if (M < 1 || a_bytes >= (1L << 31) || o_bytes >= (1L << 31) || b_bytes >= (1L << 30)) return hipErrorNotSupported;

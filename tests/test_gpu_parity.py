@@ -313,6 +313,8 @@ DX_S1_SHAPES = [
     (4, 12, 12, 132, 44, 3, 3, 1, 1),
     (16, 14, 14, 128, 256, 3, 3, 1, 1),  # 392 items of 144 steps on 256 workgroups: one or two each, all shared by the wavefronts
     (40, 7, 7, 192, 512, 3, 3, 1, 1),    # 369 items (the last tile ragged), three blocks of produced channels, 288 steps
+    (48, 20, 20, 64, 48, 3, 3, 1, 1),    # 48 reduced channels: 27 steps, an odd number (the filter, rotated in place, is read with a negative tap stride)
+    (32, 12, 12, 96, 80, 5, 5, 2, 2),    # 125 steps
 ]
 
 
@@ -427,7 +429,7 @@ DIRECT_CONV_SHAPES = [
     (2, 12, 12, 32, 64, 3, 3, 1, 1, 1, 1),      # stride 1 (forced): every tap of a border pixel's window in the padding
     (1, 5, 5, 16, 8, 7, 6, 1, 1, 3, 3),         # window larger than the image, 16 channels (42 steps), 8 produced channels
     (40, 20, 20, 32, 64, 3, 3, 2, 2, 1, 1),     # 4000 pixels = 250 tiles: fewer items than wavefronts
-    (64, 30, 34, 48, 64, 3, 3, 2, 2, 1, 1),     # 16320 pixels = 1020 tiles, 48 channels (27 steps are odd: refused -> other kernel)
+    (64, 30, 34, 48, 64, 3, 3, 2, 2, 1, 1),     # 16320 pixels = 1020 tiles, 48 channels: 27 steps, an odd number -> one empty step is added
     # items left over in a workgroup are shared by its eight wavefronts (reduction cut in eight, partial sums through LDS):
     (8, 24, 24, 32, 192, 3, 3, 1, 1, 1, 1),     # 864 items on 256 workgroups: 3 or 4 each, all shared, 18 steps in parts of 2 and 3; a pair meets the end of a block
     (4, 10, 10, 32, 64, 1, 1, 1, 1, 0, 0),      # 2 steps: six of the eight wavefronts have none
@@ -442,6 +444,12 @@ DIRECT_CONV_SHAPES = [
     (48, 56, 56, 64, 128, 1, 1, 2, 2, 0, 0),    # c4c geometry: 4704 items of 4 steps = 18 or 19 per workgroup: 4 whole per SIMD + 2 or 3 shared
     (24, 56, 56, 128, 64, 1, 1, 1, 1, 0, 0),    # 1x1 stride 1, 8 steps, 4704 items
     (64, 64, 64, 16, 64, 2, 2, 2, 2, 0, 0),     # 2x2 taps x 16 channels = 4 steps, 4096 items = 16 per workgroup, all whole
+    # an odd number of steps (tap, 16 channels): an empty step is added to every group
+    (64, 28, 28, 48, 96, 3, 3, 1, 1, 1, 1),     # 27 steps; 6272 items = 24 or 25 per workgroup: whole items and a shared one
+    (24, 14, 14, 80, 128, 5, 5, 1, 1, 2, 2),    # 125 steps; 588 items: 2 or 3 per workgroup, all shared (parts of 15 and 16 steps)
+    (40, 20, 20, 16, 64, 3, 3, 1, 1, 1, 1),     # 9 steps; 1000 items: 3 or 4 per workgroup, the eighth part of 10 steps is 1 or 2
+    (96, 24, 24, 16, 64, 1, 1, 1, 1, 0, 0),     # a single step per item (1x1, 16 channels)
+    (50, 14, 14, 48, 256, 3, 3, 1, 1, 1, 1),    # 27 steps, 2452 items: 9 or 10 per workgroup - a group of two tiles per SIMD, steps 14 + 14
 ]
 
 
