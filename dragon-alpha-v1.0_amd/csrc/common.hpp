@@ -245,10 +245,11 @@ hipError_t launch_pointwise_scatter(hipStream_t stream, const float *dY, const f
 // Kernel-split backward-data, up to four phases over the same coarse pixels in one launch, both operands straight from
 // memory: direct_conv_phased.hip. Phase f: O[o_off[f] + n*o_sn + i*o_sh + j*o_sw + co] = sum A[n, i - ph[f] + th,
 // j - pw[f] + tw, c] * B[b_off[f] + th*b_sth[f] + tw*b_stw + c*b_k + co]. hipErrorNotSupported: nothing launched.
+// `sharing`: -1 = by shape, 0 = every wavefront its own items, 1 = a workgroup's wavefronts share every group of items.
 hipError_t launch_direct_conv_phased(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC, int CO,
                                      int OHt, int OWt, int nph, const int *TH, const int *TW, const int *ph, const int *pw,
                                      const int *b_off, const int *b_sth, int b_stw, int b_k, long b_elems,
-                                     const int *o_off, int o_sn, int o_sh, int o_sw, long o_elems, const Epilogue *ep);
+                                     const int *o_off, int o_sn, int o_sh, int o_sw, long o_elems, const Epilogue *ep, int sharing = -1);
 // Backward-data for 4 stored input channels and strides of 1 or 2 (network stems), filter W[OC,FH,FW,4] in place:
 // delta_x_stem.hip. hipErrorNotSupported (nothing launched) when the layer does not fit.
 hipError_t launch_delta_x_stem(hipStream_t stream, const float *dY, const float *W, float *dX, int N, int IH, int IW, int IC,

@@ -102,6 +102,23 @@ int fwd_algo()
 // run both kernels on every shape.
 std::atomic<int> g_pw_algo{-2};   // -2: not yet read from the environment, -1: by shape, 0: filter-resident, 1: without LDS
 
+// The same kind of switch for the kernel-split kernel without LDS (direct_conv_phased.hip): whether a workgroup's
+// wavefronts share every group of work items (-1: by shape; alpha_conv_set_kernel_split_sharing, or ALPHA_KS_SHARED=0/1
+// in the environment, read once per process).
+std::atomic<int> g_ks_sharing{-2};
+
+int ks_sharing()
+{
+    int v = g_ks_sharing.load(std::memory_order_relaxed);
+    if (v == -2) {
+        const char *e = getenv("ALPHA_KS_SHARED");
+        v = e ? (atoi(e) != 0 ? 1 : 0) : -1;
+        int expected = -2;
+        if (!g_ks_sharing.compare_exchange_strong(expected, v)) v = expected;   // a setter was quicker
+    }
+    return v;
+}
+
 int pointwise_algo()
 {
     int v = g_pw_algo.load(std::memory_order_relaxed);
@@ -337,7 +354,7 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
             const long b_elems = from_CW ? (long)sh * sw * CWstride : (long)OC * FH * FW * IC;
             hipError_t e = launch_direct_conv_phased(s, dY, F, dX, N, OH, OW, OC, IC, phases[0].OHt, phases[0].OWt, sh * sw, TH, TW, pph, ppw,
                                                      boff, bsth, a0.b_stw, a0.b_sc, b_elems, ooff, a0.o_sn, a0.o_sh, a0.o_sw,
-                                                     (long)N * IH * IW * IC, ep);
+                                                     (long)N * IH * IW * IC, ep, ks_sharing());
             if (e != hipErrorNotSupported) return hip_status(e, fn);
         }
     }
@@ -505,6 +522,12 @@ int alpha_conv_set_pointwise_algo(int algo)
 {
     if (algo < -1 || algo > 1) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_pointwise_algo: algo must be -1, 0 or 1");
     g_pw_algo.store(algo);
+    return 0;
+}
+int alpha_conv_set_kernel_split_sharing(int sharing)
+{
+    if (sharing < -1 || sharing > 1) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_kernel_split_sharing: sharing must be -1, 0 or 1");
+    g_ks_sharing.store(sharing);
     return 0;
 }
 int alpha_conv_set_fwd_algo(int algo)

@@ -18,6 +18,10 @@
 // chunk of tiles, which read the same pixels, share an L2 (phase-major order: deltaY fetched 7 times).
 // (Whole tiles with all phases: shares of 3 and 4 on 56x56 -> 28x28, 64 channels - 3136 tiles on 1024 SIMDs; shares cut
 // inside tiles with the cut tiles run alone: the filter is then read per tile, 0.6 GB from L2, and nothing is gained.)
+// Small maps with many channels (14x14x512 <- 7x7 at N = 64: 784 items of up to 128 steps for 1024 SIMDs) have fewer than
+// four of their costliest items per SIMD, and shares cut between items are then far from equal. There the line is dealt
+// to the workgroups instead, and a workgroup's eight wavefronts work on every group of its items together: the steps
+// (tap, 16 channels) of a group cut into eight parts, the partial sums added through LDS in a fixed order.
 #include "common.hpp"
 
 namespace alpha {
@@ -36,15 +40,17 @@ struct DirectPhasedArgs {
     int a_bytes, b_bytes, o_bytes;
     int tiles, nblocks, items, waves;
     long total_cost;         // items * sum over the phases of (4 * TH * TW + 1)
+    int shared;              // the line of items is dealt to the workgroups, whose wavefronts share every group (few items per SIMD)
     FastDiv d_OW, d_OHW;
     Epilogue ep;
 };
 
 template <int V> struct DcpInt { static constexpr int value = V; };
 constexpr int DCP_TB = 32;                    // tiles per chunk of the line of items
+constexpr size_t DCP_LDS_BYTES = 8 * 16 * 64 * sizeof(floatx4);   // shared groups: [wavefront][unit = 4 tile + r][lane]
 constexpr unsigned DCP_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
-template <bool EPI>
+template <bool EPI, bool SHARED = false>
 __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const DirectPhasedArgs p)
 {
     const int t = threadIdx.x, lane = t & 63;
@@ -66,18 +72,33 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
     auto BSTH = [&](int f) { return f == 0 ? p.f_b_sth[0] : f == 1 ? p.f_b_sth[1] : f == 2 ? p.f_b_sth[2] : p.f_b_sth[3]; };
     auto OOFF = [&](int f) { return f == 0 ? p.f_o_off[0] : f == 1 ? p.f_o_off[1] : f == 2 ? p.f_o_off[2] : p.f_o_off[3]; };
 
-    // `count` groups of T tiles each, from tile0 on, block nb of the produced channels, phase f
+    // `count` groups of T tiles each, from tile0 on, block nb of the produced channels, phase f. SHARED (called by
+    // all eight wavefronts of the workgroup): this wavefront multiplies one of eight parts of the group's steps - an even
+    // number of them, possibly none - and the eight partial results are added through LDS.
+    extern __shared__ __attribute__((aligned(16))) float dcp_smem[];
+    floatx4 *part = reinterpret_cast<floatx4 *>(dcp_smem);
     auto run = [&](auto tc, const int f, const int nb, const int tile0, const int count) {
         constexpr int T = decltype(tc)::value;
         if (count <= 0) return;
         const int fTH = TH(f), fTW = TW(f), fPH = PH(f), fPW = PW(f), fBOFF = BOFF(f), fBSTH = BSTH(f);
-        const int steps = fTH * fTW * CH;
+        // SHARED: part x of the group's pairs of steps, x = 2 (w % 4) + w / 4 - a SIMD's two wavefronts hold neighbouring parts
+        const int pairs = (fTH * fTW * CH) >> 1, x = 2 * (w & 3) + (w >> 2);
+        const int k_lo = SHARED ? 2 * (pairs * x >> 3) : 0;
+        const int steps = SHARED ? 2 * (pairs * (x + 1) >> 3) - k_lo : 2 * pairs;   // steps of a group that this wavefront multiplies
         const int n_l = nb * 64 + 4 * l16;
         const bool n_ok = n_l < p.CO;
         const unsigned b_lane = n_ok ? (unsigned)((4 * q * p.b_k + n_l) * 4) : DCP_NEVER;
         floatx4 a[2][T], b[2][4];
         // ---- load cursor: one step ahead of the multiplications, through (group, phase, tap, 16 channels) ----------------
         int c_tile = tile0, c_th = 0, c_tw = 0, c_ch = 0, c_left = count * steps;
+        int th_lo = 0, tw_lo = 0, ch_lo = 0;   // SHARED: step k_lo = ((th_lo * fTW) + tw_lo) * CH + ch_lo, where the cursor begins every group
+        if (SHARED && steps > 0) {
+            const int tap_lo = __builtin_amdgcn_readfirstlane(k_lo / CH);
+            ch_lo = __builtin_amdgcn_readfirstlane(k_lo - tap_lo * CH);
+            th_lo = __builtin_amdgcn_readfirstlane(tap_lo / fTW);
+            tw_lo = __builtin_amdgcn_readfirstlane(tap_lo - th_lo * fTW);
+            c_th = th_lo; c_tw = tw_lo; c_ch = ch_lo;
+        }
         int org[T], pi[T], pj[T];   // lane l16's coarse pixel of tile i: byte offset of A[n, i, j, 4q], and (i, j)
         int obase[T];               // where that pixel's results go in O (elements, phase offset and channel apart); dead pixels: beyond O
         unsigned voff[T];           // this tap's load offset, or DCP_NEVER in the padding
@@ -105,7 +126,8 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
                 voff[i] = ok ? (unsigned)(org[i] + term) : DCP_NEVER;
             }
         };
-        auto request = [&](int slot) {
+        // `last` (SHARED): the step loaded is the last of this wavefront's part of the group
+        auto request = [&](int slot, const bool last = false) {
             // past the last step the loads repeat the last step's (unused)
             const int a_off = c_ch * 64;
             const int b_off = __builtin_amdgcn_readfirstlane((fBOFF + c_th * fBSTH + c_tw * p.b_stw + c_ch * 16 * p.b_k) * 4);
@@ -117,20 +139,27 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
                 b[slot][s] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_lane + (unsigned)(s * p.b_k * 4), b_off, 0));
             if (c_left > 1) {   // bookkeeping: scalar, and vector arithmetic without memory operations
                 c_left--;
-                c_ch++;
-                if (c_ch == CH) {
-                    c_ch = 0;
-                    c_tw++;
-                    if (c_tw == fTW) {
-                        c_tw = 0;
-                        c_th++;
-                        if (c_th == fTH) {   // the next group
-                            c_th = 0;
-                            c_tile += T;
-                            locate();
-                        }
-                    }
+                if (SHARED && last) {   // the next group, from this wavefront's first step
+                    c_th = th_lo; c_tw = tw_lo; c_ch = ch_lo;
+                    c_tile += T;
+                    locate();
                     aim();
+                } else {
+                    c_ch++;
+                    if (c_ch == CH) {
+                        c_ch = 0;
+                        c_tw++;
+                        if (c_tw == fTW) {
+                            c_tw = 0;
+                            c_th++;
+                            if (!SHARED && c_th == fTH) {   // the next group
+                                c_th = 0;
+                                c_tile += T;
+                                locate();
+                            }
+                        }
+                        aim();
+                    }
                 }
             }
         };
@@ -149,13 +178,26 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
             // worked out every pixel's place in O when it reached this group (lane l16 holds pixel l16's; it moves on to the
             // next group's only after this group's first request): pixel 4q + r's comes from lane 4q + r, one cross-lane
             // read instead of two divisions per pixel.
+            unsigned mine[2];   // SHARED: this wavefront finishes the units u = 4 i + r = w and w + 8 of the group
+            if constexpr (!SHARED) {
 #pragma unroll
-            for (int i = 0; i < T; i++)
+                for (int i = 0; i < T; i++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int ob = __builtin_amdgcn_ds_bpermute((4 * q + r) * 4, obase[i]);
-                    opix[i][r] = n_ok ? (unsigned)((ob + n_l) * 4) : DCP_NEVER;
+                    for (int r = 0; r < 4; r++) {
+                        const int ob = __builtin_amdgcn_ds_bpermute((4 * q + r) * 4, obase[i]);
+                        opix[i][r] = n_ok ? (unsigned)((ob + n_l) * 4) : DCP_NEVER;
+                    }
+            } else {
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int i = (w >> 2) + 2 * h;   // uniform
+                    int from = obase[0];
+#pragma unroll
+                    for (int y = 1; y < T; y++) from = i == y ? obase[y] : from;
+                    const int ob = __builtin_amdgcn_ds_bpermute((4 * q + (w & 3)) * 4, from);
+                    mine[h] = n_ok && i < T ? (unsigned)((ob + n_l) * 4) : DCP_NEVER;
                 }
+            }
             {
                 floatx4 acc[T][4];
 #pragma unroll
@@ -172,7 +214,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
                                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[slot][i][s], b[slot][s][j], acc[i][j], 0, 0, 0);
                 };
                 for (int ks = 0; ks < steps; ks += 2) {
-                    request(1);
+                    request(1, ks + 2 >= steps);
                     multiply(0);
                     __builtin_amdgcn_sched_barrier(0);
                     request(0);
@@ -180,18 +222,40 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 const int o_off = OOFF(f) * 4;
+                auto emit = [&](floatx4 v, const unsigned at) __attribute__((always_inline)) {
+                    if (EPI) {   // the derivative of the leaky ReLU whose output is this layer's input
+                        const floatx4 gt = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, at, o_off, 0));
 #pragma unroll
-                for (int i = 0; i < T; i++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        floatx4 v = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
-                        if (EPI) {   // the derivative of the leaky ReLU whose output is this layer's input
-                            const floatx4 gt = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, opix[i][r], o_off, 0));
-#pragma unroll
-                            for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
-                        }
-                        buffer_store_b128_guarded<2>(v, o_rsrc, opix[i][r], o_off);   // non-temporal, as in direct_conv.hip
+                        for (int j = 0; j < 4; j++) v[j] = ep_gate(v[j], gt[j], p.ep.slope);
                     }
+                    buffer_store_b128_guarded<2>(v, o_rsrc, at, o_off);   // non-temporal, as in direct_conv.hip
+                };
+                if constexpr (!SHARED) {
+#pragma unroll
+                    for (int i = 0; i < T; i++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) emit(floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]}, opix[i][r]);
+                } else {
+                    // unit u = 4 i + r (one 128-bit store per lane); partial results [wavefront][unit][lane], added in the
+                    // order of the wavefronts' numbers; wavefront w finishes the units u = w and w + 8
+#pragma unroll
+                    for (int i = 0; i < T; i++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            part[(w * 16 + 4 * i + r) * 64 + lane] = floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+                    lds_barrier();   // orders LDS only: the next group's loads and this group's stores stay in flight across it
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const int u = w + 8 * h;
+                        if (u < 4 * T) {   // uniform
+                            floatx4 v = part[u * 64 + lane];
+#pragma unroll
+                            for (int y = 1; y < 8; y++) v += part[(y * 16 + u) * 64 + lane];
+                            emit(v, mine[h]);
+                        }
+                    }
+                    lds_barrier();   // the next group writes `part` again
+                }
             }
         }
     };
@@ -205,10 +269,11 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
     // A share belongs to a SIMD (what has to be even is the work per SIMD, whose two wavefronts halve it): the items that
     // begin in it differ from the mean by at most one item per SIMD, not per wavefront.
     const int wg_order = (G & 7) == 0 ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
-    const int order = wg_order * 4 + (w & 3);
-    const long s_lo = p.total_cost * order / p.waves, s_hi = p.total_cost * (order + 1) / p.waves;
+    const int order = SHARED ? wg_order : wg_order * 4 + (w & 3), shares = SHARED ? G : p.waves;
+    const long s_lo = p.total_cost * order / shares, s_hi = p.total_cost * (order + 1) / shares;
     const long s_mid = s_lo + (s_hi - s_lo) / 2;
-    const long pos_lo = w < 4 ? s_lo : s_mid, pos_hi = w < 4 ? s_mid : s_hi;
+    // SHARED: the share is the workgroup's, and its wavefronts go through it together
+    const long pos_lo = SHARED || w < 4 ? s_lo : s_mid, pos_hi = SHARED || w >= 4 ? s_hi : s_mid;
     int csum = 0;   // cost of a tile with all its phases
     for (int f = 0; f < p.nph; f++) csum += 4 * TH(f) * TW(f) + 1;
     const long per_nb = (long)p.tiles * csum;
@@ -263,7 +328,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
 hipError_t launch_direct_conv_phased(hipStream_t stream, const float *A, const float *B, float *O, int N, int AH, int AW, int AC, int CO,
                                      int OHt, int OWt, int nph, const int *TH, const int *TW, const int *ph, const int *pw,
                                      const int *b_off, const int *b_sth, int b_stw, int b_k, long b_elems,
-                                     const int *o_off, int o_sn, int o_sh, int o_sw, long o_elems, const Epilogue *ep)
+                                     const int *o_off, int o_sn, int o_sh, int o_sw, long o_elems, const Epilogue *ep, int sharing)
 {
     if (nph < 1 || nph > 4 || AC < 32 || (AC & 31) || CO < 4 || (CO & 3) || OHt < 1 || OWt < 1) return hipErrorNotSupported;
     if (ep && ep->fused && !ep->gate) return hipErrorNotSupported;
@@ -300,8 +365,25 @@ hipError_t launch_direct_conv_phased(hipStream_t stream, const float *A, const f
     a.d_OHW = make_fastdiv(OHt * OWt);
     a.ep = ep ? *ep : bias_epilogue(nullptr);
     int wgs = cus;   // one workgroup of eight wavefronts per compute unit
-    if (wgs * 8 > a.items) wgs = (a.items + 7) / 8;
+    if ((long)wgs * 8 > (long)a.items * nph) wgs = (int)(((long)a.items * nph + 7) / 8);   // an item per phase
     a.waves = wgs * 4;   // the SIMDs the line of items is dealt to
+    // Fewer than two and a half of the costliest items per SIMD: shares cut between items would be uneven, the
+    // workgroups' wavefronts share every group instead. 3x3 stride 2 backward-data, deltaY -> deltaX, shared against own
+    // items: 64x7x7x512 -> 14x14x256 (1.8 per SIMD) 0.0709 against 0.0790 ms, 128x4x4x512 -> 8x8x256 (1.2) 0.0450 against
+    // 0.0659, 128x8x8x256 -> 16x16x128 (2.4) 0.0493 against 0.0496, 64x14x14x256 -> 28x28x128 (3.6) 0.0772 against 0.0678.
+    long cost_max = 0;
+    for (int f = 0; f < nph; f++) cost_max = std::max(cost_max, 4L * a.f_TH[f] * a.f_TW[f] + 1);
+    a.shared = sharing < 0 ? 2 * a.total_cost < 5 * cost_max * a.waves : sharing != 0;
+    if (a.shared) {
+        if (a.ep.fused) {
+            if (hipError_t e = ensure_dynamic_lds<direct_conv_phased_kernel<true, true>>(DCP_LDS_BYTES); e != hipSuccess) return e;
+            hipLaunchKernelGGL((direct_conv_phased_kernel<true, true>), dim3(wgs), dim3(512), DCP_LDS_BYTES, stream, a);
+        } else {
+            if (hipError_t e = ensure_dynamic_lds<direct_conv_phased_kernel<false, true>>(DCP_LDS_BYTES); e != hipSuccess) return e;
+            hipLaunchKernelGGL((direct_conv_phased_kernel<false, true>), dim3(wgs), dim3(512), DCP_LDS_BYTES, stream, a);
+        }
+        return hipGetLastError();
+    }
     if (a.ep.fused) hipLaunchKernelGGL(direct_conv_phased_kernel<true>, dim3(wgs), dim3(512), 0, stream, a);
     else hipLaunchKernelGGL(direct_conv_phased_kernel<false>, dim3(wgs), dim3(512), 0, stream, a);
     return hipGetLastError();

@@ -76,6 +76,11 @@ int alpha_conv_bind_tickets(unsigned *tickets, int count);
  * take the layer: -1 = chosen by shape, 0 = the filter-resident kernel, 1 = the kernel without LDS wherever it fits.
  * Also read once from the environment variable ALPHA_PW_DIRECT = 0|1. No counterpart in the reference. */
 int alpha_conv_set_pointwise_algo(int algo);
+/* And for kernel-split backward-data through the kernel without LDS (all phases of one size, deltaY channels a multiple
+ * of 32): -1 = by shape, 0 = every wavefront works on items of its own, 1 = the eight wavefronts of a workgroup share
+ * every group of items, each taking an eighth of the reduction (what layers with few items per compute unit get by
+ * shape). Also read once from the environment variable ALPHA_KS_SHARED = 0|1. No counterpart in the reference. */
+int alpha_conv_set_kernel_split_sharing(int sharing);
 
 /* ---- Cuda_conv3D: forward ------------------------------------------------------------------ */
 

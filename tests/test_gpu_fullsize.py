@@ -284,3 +284,60 @@ def test_pieces_added_by_last_workgroup_equal_second_kernel_full_size(dev, layer
     imgs = [0, N - 1]
     want = O.conv3D_f64(np.ascontiguousarray(X.numpy()[imgs]), W.numpy(), s, s, p, p)
     _check(second_kernel[imgs].cpu().numpy(), want, "%s forward, equal shares" % layer)
+
+
+# Kernel-split backward-data of a workgroup's wavefronts sharing every group of items (what small maps with many
+# channels get by shape), at full size: the stride-2 3x3 layers that open the third and fourth stage of a ResNet
+# (N = 64; the first has items enough for every wavefront and shares only when forced), the second stage's on 16x16
+# maps at N = 128, and c4b. Whole images against the oracle, <X, deltaX> = <Y, deltaY> in fp64 over the
+# full batch, and the two distributions of the work against each other.
+@pytest.mark.parametrize("case", [(64, 28, 28, 128, 256, False), (64, 14, 14, 256, 512, True), (128, 16, 16, 128, 256, True),
+                                  (64, 56, 56, 64, 128, False)])
+def test_kernel_split_shared_groups_full_size(dev, case):
+    torch = dev.torch
+    L = pkg.lib()
+    DX = pkg.Cuda_dconv3D_deltaX
+    N, IH, IW, IC, OC, shares_by_shape = case
+    F, s, p = 3, 2, 1
+    OH, OW = out_dim(IH, IW, F, F, s, s, p, p)
+    g = torch.Generator(device="cpu").manual_seed(8400 + IH)
+    X = torch.randn((N, IH, IW, IC), generator=g)
+    W = torch.randn((OC, F, F, IC), generator=g) * float(np.sqrt(2.0 / (F * F * IC)))
+    dY = torch.randn((N, OH, OW, OC), generator=g)
+    x, w, dy = X.to(dev.dev), W.to(dev.dev), dY.to(dev.dev)
+
+    def backward(sharing):
+        assert L.alpha_conv_set_kernel_split_sharing(sharing) == 0
+        dx = torch.full((N, IH, IW, IC), float("nan"), device=dev.dev)
+        DX.dconv3D_deltaX_crossAdd(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), F, F, dx.data_ptr(), IH, IW, N, IC, OC, s, s, p, p)
+        dev.sync()
+        return dx
+
+    try:
+        own = backward(0)
+        shared = backward(1)
+        by_shape = backward(-1)
+    finally:
+        L.alpha_conv_set_kernel_split_sharing(-1)
+    expect = shared if shares_by_shape else own
+    assert torch.equal(by_shape.view(torch.int32), expect.view(torch.int32)), "the choice by shape is not the expected one"
+    imgs = [0, N // 2, N - 1]
+    want = O.deltaX_f64(np.ascontiguousarray(dY.numpy()[imgs]), W.numpy(), IH, IW, s, s, p, p)
+    _check(own[imgs].cpu().numpy(), want, "deltaX, items of their own %s" % (case,))
+    _check(shared[imgs].cpu().numpy(), want, "deltaX, shared groups %s" % (case,))
+    y = torch.full((N, OH, OW, OC), float("nan"), device=dev.dev)
+    eng = pkg.engine.Engine(dev.stream)
+    try:
+        eng.conv3D(y.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), F, F, N, IC, OC, s, s, p, p)
+        eng.sync()
+    finally:
+        eng.close()
+    a = float((y.double() * dy.double()).sum())
+    scale = float((y.double().abs() * dy.double().abs()).sum())
+    for name, dx in (("own", own), ("shared", shared)):
+        b = float((x.double() * dx.double()).sum())
+        assert abs(a - b) <= 2e-5 * scale, "%s %s: <Y,dY> = %r vs <X,dX> = %r" % (case, name, a, b)
+    ref = own.double()
+    floor = 1e-5 * max(1.0, float(ref.pow(2).mean().sqrt()))
+    err = (shared.double() - ref).abs() - 2 * torch.clamp(1e-4 * ref.abs(), min=floor)
+    assert float(err.max()) <= 0.0, "%s: the two distributions differ beyond twice the bar" % (case,)

@@ -140,7 +140,8 @@ def test_backward_data_with_the_leaky_relu_derivative_in_the_epilogue(dev, shape
     check(dev.get(dx), want, "deltaX_s1_leakyRelu %s" % (shape,))
 
 
-@pytest.mark.parametrize("shape", [(4, 16, 16, 64, 128, 3, 3, 2, 2, 1, 1),     # four phases in one launch of the LDS-halo kernel
+@pytest.mark.parametrize("shape", [(4, 16, 16, 64, 128, 3, 3, 2, 2, 1, 1),     # four phases in one launch of the kernel without LDS
+                                   (6, 14, 18, 132, 96, 3, 3, 2, 2, 1, 1),     # the same, three blocks of produced channels (the last ragged), ragged last tile
                                    (4, 13, 11, 16, 16, 5, 4, 3, 2, 2, 1)])     # one launch of the generic kernel per phase
 def test_strided_backward_data_with_the_leaky_relu_derivative_in_the_epilogue(dev, shape):
     N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
@@ -153,10 +154,16 @@ def test_strided_backward_data_with_the_leaky_relu_derivative_in_the_epilogue(de
     dy, w, xf = dev.put(dY), dev.put(W), dev.put(Xf)
     cw = dev.empty(sh * sw * OC * CFH * CFW * IC, fill=0.0)
     DX.ks_remodev2(dev.stream, w.data_ptr(), FH, FW, cw.data_ptr(), CFH, CFW, OC, IC, sh, sw)
-    dx = dev.guarded(N, IH, IW, IC)
-    DX.dconv3D_deltaX_kernelSplit_leakyRelu(dev.streams, 1, dy.data_ptr(), OH, OW, cw.data_ptr(), FH, FW, xf.data_ptr(), k, dx.data_ptr(),
-                                            IH, IW, N, IC, OC, sh, sw, ph, pw)
-    check(dev.get(dx), want, "deltaX_kernelSplit_leakyRelu %s" % (shape,))
+    L = pkg.lib()
+    try:
+        for sharing in (0, 1, -1):   # the kernel without LDS: wavefronts with items of their own / sharing every group / by shape
+            L.alpha_conv_set_kernel_split_sharing(sharing)
+            dx = dev.guarded(N, IH, IW, IC)
+            DX.dconv3D_deltaX_kernelSplit_leakyRelu(dev.streams, 1, dy.data_ptr(), OH, OW, cw.data_ptr(), FH, FW, xf.data_ptr(), k, dx.data_ptr(),
+                                                    IH, IW, N, IC, OC, sh, sw, ph, pw)
+            check(dev.get(dx), want, "deltaX_kernelSplit_leakyRelu sharing %d %s" % (sharing, shape))
+    finally:
+        L.alpha_conv_set_kernel_split_sharing(-1)
 
 
 def test_row_functions_keep_pad_columns_zero_and_match_their_definitions(dev):

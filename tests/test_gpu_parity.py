@@ -605,6 +605,8 @@ KS_SHAPES = [
     (6, 30, 34, 36, 64, 3, 3, 2, 2, 1, 1),    # 1530 coarse pixels (last tile ragged), a ragged block of 36 produced channels
     (40, 56, 56, 32, 64, 3, 3, 2, 2, 1, 1),   # 1960 tiles: shares of several items per SIMD
     (24, 60, 52, 36, 32, 5, 5, 2, 2, 2, 2),   # the same with phases of 9, 6, 6 and 4 taps, ragged channels and a ragged last tile
+    (6, 14, 18, 132, 96, 3, 3, 2, 2, 1, 1),   # small map, 96 channels of deltaY (6 steps per tap: parts of 0 and 2 steps), three blocks of produced channels
+    (10, 8, 8, 64, 256, 3, 3, 2, 2, 1, 1),    # 4x4 coarse pixels per image, 256 channels of deltaY
     (4, 12, 16, 64, 32, 3, 3, 1, 2, 1, 1),    # two phases (stride along the width only)
     (4, 16, 12, 68, 96, 3, 5, 2, 1, 1, 2),    # two phases (stride along the height only), two blocks of produced channels
     (4, 14, 14, 64, 64, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2: three phases without taps write zeros
@@ -651,6 +653,21 @@ def test_deltaX_kernel_split_family(dev, shape):
     # launch of the generic kernel per phase; 6: as 0 (the kernel without LDS where the phases have one size) - and the
     # tiny-IC entry, which reads W in place
     L = pkg.lib()
+    try:
+        # the kernel without LDS with every wavefront on items of its own, and with the workgroup's wavefronts sharing
+        # every group (by shape above: the small layers share)
+        for sharing in (0, 1):
+            L.alpha_conv_set_kernel_split_sharing(sharing)
+            dXo = dev.guarded(N, IH, IW, IC)
+            DX.dconv3D_deltaX_kernelSplit(dev.streams, 1, dy.data_ptr(), OH, OW, CW.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC,
+                                          sh, sw, ph, pw)
+            check(dev.get(dXo), want, "kernelSplit sharing %d %s" % (sharing, shape))
+            dXo = dev.guarded(N, IH, IW, IC)
+            DX.dconv3D_deltaX_crossAdd(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dXo.data_ptr(), IH, IW, N, IC, OC,
+                                       sh, sw, ph, pw)
+            check(dev.get(dXo), want, "crossAdd (filter in place) sharing %d %s" % (sharing, shape))
+    finally:
+        L.alpha_conv_set_kernel_split_sharing(-1)
     try:
         for algo in (1, 3, 6):
             L.alpha_conv_set_fwd_algo(algo)
