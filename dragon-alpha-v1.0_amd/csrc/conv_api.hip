@@ -299,9 +299,12 @@ int deltaX_phases(const char *fn, const int64_t *streams, int length,
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && sh * sw > 1 && IH == sh * OH && IW == sw * OW && !(ep && ep->fused) &&
-        (fwd_algo() == 0 || fwd_algo() == 6)) {
+        (fwd_algo() == 0 || fwd_algo() == 6) && (long)OC * IC < 40L * (OC + sh * sw * IC)) {
         // a 1x1 filter under a larger stride: one matrix product scattered over deltaX, zeros in between. The filter is
-        // [OC][IC] in both layouts (W as it is; phase 0 of the kernel-split layout, the only one with a tap).
+        // [OC][IC] in both layouts (W as it is; phase 0 of the kernel-split layout, the only one with a tap). For the layers
+        // that memory bounds - fewer than 20 FLOP per byte of deltaY read and deltaX written -: its wavefronts own tiles
+        // of pixels with all their channels, which is how the bytes move best and the matrix pipes work worst (14x14x1024
+        // <- 7x7x2048 at N = 64: 196 tiles, 0.65 ms); with more channels the phases below take the layer.
         hipError_t e = launch_pointwise_scatter(s, dY, F, dX, N, OH, OW, OC, IC, sh, sw);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }

@@ -11,8 +11,8 @@
 // tile and four for the filter feed 16 T MFMAs, loads run one step ahead through a cursor over (group, tap, channels),
 // results leave as 128-bit stores. A phase without taps (filter smaller than the stride) writes zeros.
 //
-// Shares: the items in the order (block, chunk of 32 tiles, phase, tile) form a line of cost - 4 per tap plus 1 for the
-// item's stores -; the wavefronts' shares are equal stretches of it, cut between items. A share then differs from the
+// Shares: the items in the order (block, chunk of 32 tiles, phase, tile) form a line of cost - an item's steps (taps x
+// chunks of 16 reduced channels) plus 2 for its stores -; the wavefronts' shares are equal stretches of it, cut between items. A share then differs from the
 // mean by at most one item - a quarter of the cost of a tile with all its phases - and still consists of runs of tiles
 // of one phase, so that a filter fragment serves up to four tiles; the line is dealt out XCD by XCD, so the phases of a
 // chunk of tiles, which read the same pixels, share an L2 (phase-major order: deltaY fetched 7 times).
@@ -39,7 +39,7 @@ struct DirectPhasedArgs {
     int o_sn, o_sh, o_sw;
     int a_bytes, b_bytes, o_bytes;
     int tiles, nblocks, items, waves;
-    long total_cost;         // items * sum over the phases of (4 * TH * TW + 1)
+    long total_cost;         // items * sum over the phases of (TH * TW * AC / 16 + DCP_STORE_COST)
     int shared;              // the line of items is dealt to the workgroups, whose wavefronts share every group (few items per SIMD)
     FastDiv d_OW, d_OHW;
     Epilogue ep;
@@ -47,6 +47,9 @@ struct DirectPhasedArgs {
 
 template <int V> struct DcpInt { static constexpr int value = V; };
 constexpr int DCP_TB = 32;                    // tiles per chunk of the line of items
+// An item's cost on the line of items: its steps, plus this for its stores (in steps; 1 to 4 measure the same, 6 and 8
+// slower, on 56x56x64 <- 28x28x128 3x3 stride 2 and on 1x1 stride 2 layers of 512 to 2048 channels)
+constexpr int DCP_STORE_COST = 2;
 constexpr size_t DCP_LDS_BYTES = 8 * 16 * 64 * sizeof(floatx4);   // shared groups: [wavefront][unit = 4 tile + r][lane]
 constexpr unsigned DCP_NEVER = 0x80000000u;   // beyond every descriptor (tensors below 2 GB, host-checked)
 
@@ -260,8 +263,8 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
         }
     };
 
-    // ---- this wavefront's share: an equal stretch of the line of items, each as long as its cost (4 per tap of its phase
-    //      + 1 for its stores), cut between items. The line runs through (block of produced channels, chunk of DCP_TB
+    // ---- this wavefront's share: an equal stretch of the line of items, each as long as its cost (its steps
+    //      + 2 for its stores), cut between items. The line runs through (block of produced channels, chunk of DCP_TB
     //      tiles, phase, tile): the phases of a chunk of tiles - which read the same pixels of deltaY - lie next to each
     //      other, and the line is dealt to the wavefronts XCD by XCD (workgroups go round-robin to the 8 XCDs, each with
     //      its own L2), so the second to fourth reader of a pixel finds it in L2 ------------------------------------------
@@ -275,7 +278,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
     // SHARED: the share is the workgroup's, and its wavefronts go through it together
     const long pos_lo = SHARED || w < 4 ? s_lo : s_mid, pos_hi = SHARED || w >= 4 ? s_hi : s_mid;
     int csum = 0;   // cost of a tile with all its phases
-    for (int f = 0; f < p.nph; f++) csum += 4 * TH(f) * TW(f) + 1;
+    for (int f = 0; f < p.nph; f++) csum += TH(f) * TW(f) * CH + DCP_STORE_COST;
     const long per_nb = (long)p.tiles * csum;
     long pos = pos_lo;
     while (pos < pos_hi) {
@@ -285,11 +288,11 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
         const int chunk = (int)(r / ((long)DCP_TB * csum));
         const int tile_c = chunk * DCP_TB, tb = min(DCP_TB, p.tiles - tile_c);
         long seg = (long)nb * per_nb + (long)tile_c * csum;   // where the chunk begins
-        int f = 0, cost = 4 * TH(0) * TW(0) + 1;
+        int f = 0, cost = TH(0) * TW(0) * CH + DCP_STORE_COST;
         while (f + 1 < p.nph && pos >= seg + (long)tb * cost) {
             seg += (long)tb * cost;
             f++;
-            cost = 4 * TH(f) * TW(f) + 1;
+            cost = TH(f) * TW(f) * CH + DCP_STORE_COST;
         }
         const long seg_end = seg + (long)tb * cost;
         // items of this segment whose beginning lies in [pos_lo, pos_hi)
@@ -350,7 +353,7 @@ hipError_t launch_direct_conv_phased(hipStream_t stream, const float *A, const f
         a.f_b_off[f] = any ? b_off[f] : 0; a.f_b_sth[f] = any ? b_sth[f] : 0;
         a.f_o_off[f] = o_off[f];
         taps += a.f_TH[f] * a.f_TW[f];
-        cost += 4 * a.f_TH[f] * a.f_TW[f] + 1;
+        cost += (long)a.f_TH[f] * a.f_TW[f] * (AC >> 4) + DCP_STORE_COST;
     }
     if (taps == 0) return hipErrorNotSupported;
     a.b_stw = b_stw; a.b_k = b_k;
@@ -372,7 +375,7 @@ hipError_t launch_direct_conv_phased(hipStream_t stream, const float *A, const f
     // items: 64x7x7x512 -> 14x14x256 (1.8 per SIMD) 0.0709 against 0.0790 ms, 128x4x4x512 -> 8x8x256 (1.2) 0.0450 against
     // 0.0659, 128x8x8x256 -> 16x16x128 (2.4) 0.0493 against 0.0496, 64x14x14x256 -> 28x28x128 (3.6) 0.0772 against 0.0678.
     long cost_max = 0;
-    for (int f = 0; f < nph; f++) cost_max = std::max(cost_max, 4L * a.f_TH[f] * a.f_TW[f] + 1);
+    for (int f = 0; f < nph; f++) cost_max = std::max(cost_max, (long)a.f_TH[f] * a.f_TW[f] * (AC >> 4) + DCP_STORE_COST);
     a.shared = sharing < 0 ? 2 * a.total_cost < 5 * cost_max * a.waves : sharing != 0;
     if (a.shared) {
         if (a.ep.fused) {

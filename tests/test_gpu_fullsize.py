@@ -289,16 +289,18 @@ def test_pieces_added_by_last_workgroup_equal_second_kernel_full_size(dev, layer
 # Kernel-split backward-data of a workgroup's wavefronts sharing every group of items (what small maps with many
 # channels get by shape), at full size: the stride-2 3x3 layers that open the third and fourth stage of a ResNet
 # (N = 64; the first has items enough for every wavefront and shares only when forced), the second stage's on 16x16
-# maps at N = 128, and c4b. Whole images against the oracle, <X, deltaX> = <Y, deltaY> in fp64 over the
+# maps at N = 128, c4b, and a 1x1 stride-2 layer with too many channels for the scattered product. Whole images against the oracle, <X, deltaX> = <Y, deltaY> in fp64 over the
 # full batch, and the two distributions of the work against each other.
-@pytest.mark.parametrize("case", [(64, 28, 28, 128, 256, False), (64, 14, 14, 256, 512, True), (128, 16, 16, 128, 256, True),
-                                  (64, 56, 56, 64, 128, False)])
+@pytest.mark.parametrize("case", [(64, 28, 28, 128, 256, 3, 1, False), (64, 14, 14, 256, 512, 3, 1, True), (128, 16, 16, 128, 256, 3, 1, True),
+                                  (64, 56, 56, 64, 128, 3, 1, False),
+                                  # a 1x1 shortcut of a ResNet-50 under stride 2: one phase with the tap (128 steps an item), three that write zeros
+                                  (64, 14, 14, 1024, 2048, 1, 0, False)])
 def test_kernel_split_shared_groups_full_size(dev, case):
     torch = dev.torch
     L = pkg.lib()
     DX = pkg.Cuda_dconv3D_deltaX
-    N, IH, IW, IC, OC, shares_by_shape = case
-    F, s, p = 3, 2, 1
+    N, IH, IW, IC, OC, F, p, shares_by_shape = case
+    s = 2
     OH, OW = out_dim(IH, IW, F, F, s, s, p, p)
     g = torch.Generator(device="cpu").manual_seed(8400 + IH)
     X = torch.randn((N, IH, IW, IC), generator=g)

@@ -616,6 +616,7 @@ KS_SHAPES = [
     (3, 9, 12, 132, 96, 1, 1, 3, 2, 0, 0),    # blocks of 3 x 2 pixels, 54 pixels of deltaY (ragged tile), 132 produced channels (ragged block)
     (2, 6, 20, 8, 32, 1, 1, 1, 4, 0, 0),      # stride along the width only, 8 produced channels
     (2, 15, 15, 64, 64, 1, 1, 2, 2, 0, 0),    # odd size: the last row and column of deltaX belong to no block -> the phase kernels
+    (4, 14, 14, 128, 256, 1, 1, 2, 2, 0, 0),  # more than 20 FLOP per byte moved: the phases (one with the tap, three of zeros) instead of the scattered product
 ]
 
 
