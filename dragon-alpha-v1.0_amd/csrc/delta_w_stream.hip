@@ -232,7 +232,7 @@ int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, 
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
     if (4L * IC * OC < 3L * icb * 64 * ocb * 64) return GZ;
     const long items = icb * ocb * FH * FW, TG = (long)N * OH * ((OW + 3) / 4);
-    if (items >= (1L << 20) || TG >= (1L << 30) || items * TG < units || items > 4096 || TG < 8L * units) return GZ;
+    if (items >= (1L << 20) || TG >= (1L << 30) || items * TG < 8L * units || items > 4096) return GZ;
     long R = units / items;
     if (R > GZ) R = GZ;
     if (R >= 1 && 20 * R * items >= 19L * units) return R < 2 ? 2 : (int)R;
@@ -271,7 +271,8 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
     a.TG = (int)TG;
     a.L = items * TG;
     a.wgs = cus;   // one workgroup of eight wavefronts per compute unit
-    if (a.L < a.wgs || items > 4096 || TG < 8L * cus) return hipErrorNotSupported;
+    // at least eight pixel groups per workgroup (one per wavefront); smaller layers go to the kernels with one workgroup per slice
+    if (a.L < 8L * a.wgs || items > 4096) return hipErrorNotSupported;
     // Every item in R equal pieces where R * items workgroups are (nearly) all of them; else the line of items in equal
     // shares. Either way the pieces of an item go to deltaW and the GridZ - 1 buffers.
     long R = cus / items;

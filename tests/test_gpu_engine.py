@@ -258,6 +258,7 @@ def test_engine_deltaW_with_fill_option(dev):
     e = pkg.engine.Engine(dev.stream)
     try:
         gz = []
+        e.config.deltaW_SK_leastUnits = 0     # engine objects lower GridZ to what the persistent kernel needs (7 here): not the subject
         for units in (0, 256):
             e.config.deltaW_SK_fillUnits = units
             dw = dev.empty(OC, 3, 3, IC, fill=float("nan"))

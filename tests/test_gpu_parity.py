@@ -819,6 +819,8 @@ DW_STREAM_SHAPES = [
     (8, 32, 32, 256, 64, 1, 1, 1, 1, 0, 0, 128, 64),     # 1x1: 4 items x 64 pieces
     (128, 9, 9, 256, 256, 4, 4, 1, 1, 1, 1, 2, 1),      # 256 items, one piece each; the one buffer is all zeros
     (16, 40, 36, 128, 64, 5, 3, 1, 2, 2, 1, 64, None),  # 5x3 filter, stride 1 x 2: 30 items in a line (8 equal pieces each would use 240 workgroups)
+    (16, 7, 7, 128, 192, 3, 3, 1, 1, 1, 1, 8, None),    # 7x7 maps: rows of two pixel groups (the second ragged), 54 items of 224 groups in a line, 47 groups per workgroup
+    (32, 14, 14, 128, 128, 3, 3, 2, 2, 1, 1, 8, 7),     # stride 2 onto 7x7 maps: 36 items x 7 pieces of 64 groups
 ]
 
 
