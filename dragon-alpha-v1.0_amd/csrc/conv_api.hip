@@ -138,18 +138,19 @@ bool pointwise_direct_preferred(int K, int N)
     return (K % 32) == 0 && K >= 128 && N <= 64;
 }
 
-// Through direct_conv.hip (no LDS): strided layers (the halo kernel's LDS footprint is four input pixels per output pixel
-// there; a strided 1x1 layer 3 % faster than through the filter-resident kernel), layers with more than one tap whose work
-// items divide evenly enough among the compute units (every 3x3 layer of the benchmark configurations: 3-14 % faster than
-// the LDS-halo kernel), and 1x1 layers with a long reduction (256 -> 1024 channels on 64x14x14 pixels: 0.053 against 0.060 ms
-// through the filter-resident kernel; 256 -> 64 on 32x56x56 pixels: 0.030 against 0.032 ms through pointwise_direct.hip;
-// 64 -> 256 there: 0.036 against 0.031 ms through the filter-resident kernel, which keeps that shape).
+// Through direct_conv.hip (no LDS): every layer with more than one tap or a stride (every 3x3 layer of the benchmark
+// configurations: 3-14 % faster than the LDS-halo kernel; small layers - a few work items per compute unit, which the
+// workgroup's wavefronts share - several times: 3x3 256 -> 256 on 8x14x14 pixels 0.021 against 0.068 ms, 5x5 48 -> 128 on
+// 64x7x7 0.014 against 0.103 ms, 3x3 64 -> 64 on one 56x56 image 0.007 against 0.019 ms; a strided 1x1 layer 3 % faster than
+// through the filter-resident kernel), and 1x1 layers with a long reduction whose work items divide evenly enough among
+// the compute units (256 -> 1024 channels on 64x14x14 pixels: 0.053 against 0.060 ms through the filter-resident kernel;
+// 256 -> 64 on 32x56x56 pixels: 0.030 against 0.032 ms through pointwise_direct.hip; 64 -> 256 there: 0.036 against
+// 0.031 ms through the filter-resident kernel, which keeps that shape).
 bool direct_conv_preferred(int FH, int FW, int sh, int sw, long M, int AC, int CO)
 {
-    if (sh > 1 || sw > 1) return true;
+    if (sh > 1 || sw > 1 || FH * FW > 1) return true;
     const bool ws = t_workspace != nullptr && t_workspace_bytes >= (1u << 20);
-    if (FH * FW <= 1) return AC >= 256 && direct_conv_balanced(M, CO, ws);
-    return direct_conv_balanced(M, CO, ws);
+    return AC >= 256 && direct_conv_balanced(M, CO, ws);
 }
 
 // The rest of a fused epilogue as a pass of its own over a dense [pixels, C] output (kernels that add a bias only).
