@@ -404,7 +404,7 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     a.GK_slice = (a.GK / GridZ) >> 3 << 3;
     const int algo = fwd_algo();
     // Which kernel (all but the first share the slice partition and the outputs):
-    //  - layers whose channel counts fill 64 x 64 blocks to 75 % or more, GridZ of 2 or more: the persistent kernel of
+    //  - layers whose channel counts fill 64 x 64 blocks well enough (below), GridZ of 2 or more: the persistent kernel of
     //    delta_w_stream.hip (its own partition of the pixels among deltaW and the buffers; a bias gradient takes a pass of
     //    its own over deltaY then, so layers where another kernel produces it on the way stay with that kernel);
     //  - 1x1 stride 1 with channel counts in multiples of 64: the register kernel of delta_w_pointwise.hip;
@@ -417,8 +417,13 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     const bool w1 = FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
     const bool blocks_filled = 4L * IC * OC >= 3L * icb * 64 * ocb * 64;
+    // what the persistent kernel needs of its 64 x 64 blocks to win: 40 % where the row-streaming kernel is the alternative
+    // (96 -> 208 channels 3x3: 0.066 against 0.103 ms; 32 -> 32: 0.107 against 0.074), 15 % where the generic kernel is
+    // (5x5, 16 -> 48: 0.026 against 0.043 ms; 16 -> 32: 0.078 against 0.047)
+    const bool rows_shape = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1));
+    const bool stream_filled = 100L * IC * OC >= (rows_shape ? 40L : 15L) * icb * 64 * ocb * 64;
     const bool rows_fill = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1)) && icb * ((OC + 31) / 32) * GridZ >= 2L * device_cu_count();
-    if (algo == 0 && blocks_filled && !(dB && (rows_fill || w1))) {
+    if (algo == 0 && stream_filled && !(dB && (rows_fill || w1))) {
         // the same arithmetic with the reduction dealt out evenly (its own partition of the pixels among the buffers)
         hipError_t e = launch_deltaW_stream(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, GridZ);
         if (e == hipSuccess && dB) e = launch_col_sum(stream0(streams), dY, dB, dB_buf, OC, a.GK, a.GK_slice, GridZ);

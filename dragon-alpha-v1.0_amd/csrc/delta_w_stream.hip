@@ -224,13 +224,13 @@ static int dws_max_pieces(long items, long TG, int G)
 
 // The least split-K factor <= GZ with which launch_deltaW_stream on a device of `units` compute units cuts the layer
 // exactly as it does with GZ (the same R pieces per item, or the same line of shares), or GZ itself where the kernel
-// does not take the layer or the split-K entries do not choose it (channel counts that fill 64 x 64 blocks to less than
-// 75 %). With it the kernel has no buffers to fill with zeros and the caller's buf_summary none to add for nothing.
+// does not take the layer or the split-K entries may not choose it (channel counts that fill 64 x 64 blocks to less than
+// 40 %). With it the kernel has no buffers to fill with zeros and the caller's buf_summary none to add for nothing.
 int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ)
 {
     if ((IC & 3) || (OC & 3) || IC < 4 || OC < 4 || FH < 1 || FW < 1 || GZ < 2 || units < 1 || N < 1 || OH < 1 || OW < 1) return GZ;
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
-    if (4L * IC * OC < 3L * icb * 64 * ocb * 64) return GZ;
+    if (100L * IC * OC < 40L * icb * 64 * ocb * 64) return GZ;   // the stricter of the split-K entries' two thresholds (the stride is not known here)
     const long items = icb * ocb * FH * FW, TG = (long)N * OH * ((OW + 3) / 4);
     if (items >= (1L << 20) || TG >= (1L << 30) || items * TG < 8L * units || items > 4096) return GZ;
     long R = units / items;

@@ -821,6 +821,8 @@ DW_STREAM_SHAPES = [
     (16, 40, 36, 128, 64, 5, 3, 1, 2, 2, 1, 64, None),  # 5x3 filter, stride 1 x 2: 30 items in a line (8 equal pieces each would use 240 workgroups)
     (16, 7, 7, 128, 192, 3, 3, 1, 1, 1, 1, 8, None),    # 7x7 maps: rows of two pixel groups (the second ragged), 54 items of 224 groups in a line, 47 groups per workgroup
     (32, 14, 14, 128, 128, 3, 3, 2, 2, 1, 1, 8, 7),     # stride 2 onto 7x7 maps: 36 items x 7 pieces of 64 groups
+    (8, 14, 14, 96, 208, 3, 3, 1, 1, 1, 1, 8, None),    # blocks filled to 61 % (96 of 128 input, 208 of 256 output channels): 72 items in a line
+    (16, 14, 14, 16, 48, 5, 5, 1, 1, 2, 2, 16, 10),     # 5x5, one block filled to 19 %: 25 items x 10 pieces
 ]
 
 
