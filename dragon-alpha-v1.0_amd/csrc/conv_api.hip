@@ -131,11 +131,13 @@ int pointwise_algo()
     return v;
 }
 
-bool pointwise_direct_preferred(int K, int N)
+bool pointwise_direct_preferred(int K, int N, long M)
 {
     const int forced = pointwise_algo();
     if (forced >= 0) return forced != 0 && (K % 32) == 0;
-    return (K % 32) == 0 && K >= 128 && N <= 64;
+    // its wavefronts own tiles of 16 pixels: with fewer tiles than SIMDs the kernel of direct_conv.hip, which cuts the
+    // reduction among a workgroup's wavefronts, is the faster (832 -> 48 channels on 64x7x7 pixels: 0.007 against 0.019 ms)
+    return (K % 32) == 0 && K >= 128 && N <= 64 && M >= 64L * device_cu_count();
 }
 
 // Through direct_conv.hip (no LDS): every layer with more than one tap or a stride (every 3x3 layer of the benchmark
@@ -192,7 +194,7 @@ int forward(const char *fn, const int64_t *streams, int length,
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && sh == 1 && sw == 1 && OH == IH && OW == IW && layout == FILTER_CW && algo != 3 &&
-        pointwise_direct_preferred(IC, OC)) {
+        pointwise_direct_preferred(IC, OC, (long)N * OH * OW)) {
         hipError_t e = launch_pointwise_direct(stream0(streams), X, F, Y, (long)N * OH * OW, IC, OC, bias, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
@@ -200,6 +202,15 @@ int forward(const char *fn, const int64_t *streams, int length,
         // W[OC][IC] is [N][K]; CW[IC][OC] is [K][N]; a stride only thins the input pixels that are read
         hipError_t e = launch_pointwise(stream0(streams), X, F, Y, N, IH, IW, OH, OW, sh, sw, IC, OC, layout == FILTER_CW, ep ? nullptr : bias);
         if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), Y, *ep, (long)N * OH * OW, OC);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
+    if (algo == 0 && layout == FILTER_CW && FH == 1 && FW == 1 && IC >= 32) {
+        // a 1x1 layer that none of the kernels above took (produced channels not a multiple of 64, more than 256 reduced
+        // ones ...): the kernel without LDS before the LDS-halo and the generic ones (192 -> 96 channels on 64x28x28 pixels:
+        // 0.023 against 0.035 ms; 832 -> 48 on 64x7x7: 0.007 against 0.019 ms; with 16 reduced channels the generic kernel
+        // is the faster: 16 -> 480 backward-data 0.012 against 0.019 ms)
+        hipError_t e = launch_direct_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
+                                          0, IC * OC, OC, (long)FH * FW * IC * OC, bias, ep, t_workspace, t_workspace_bytes, t_tickets, t_tickets_count);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (algo != 3) {
@@ -249,7 +260,7 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
                                           t_workspace, t_workspace_bytes, t_tickets, t_tickets_count);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && OH == IH && OW == IW && algo != 3 && pointwise_direct_preferred(OC, IC)) {
+    if (FH == 1 && FW == 1 && ph == 0 && pw == 0 && OH == IH && OW == IW && algo != 3 && pointwise_direct_preferred(OC, IC, (long)N * IH * IW)) {
         // deltaX[m][ic] = sum_oc deltaY[m][oc] * W[oc][ic]: W is [K][N]
         hipError_t e = launch_pointwise_direct(stream0(streams), dY, W, dX, (long)N * IH * IW, OC, IC, nullptr, ep);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
@@ -258,6 +269,13 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
         // deltaX[m][ic] = sum_oc deltaY[m][oc] * W[oc][ic]: W is [K][N]
         hipError_t e = launch_pointwise(stream0(streams), dY, W, dX, N, IH, IW, IH, IW, 1, 1, OC, IC, 1);
         if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), dX, *ep, (long)N * IH * IW, IC);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
+    if (algo == 0 && FH == 1 && FW == 1 && OC >= 32) {
+        // a 1x1 layer that none of the kernels above took: as in forward()
+        hipError_t e = launch_direct_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, 1, 1, FH - 1 - ph, FW - 1 - pw,
+                                          (FH * FW - 1) * IC, -IC, FH * FW * IC, (long)OC * FH * FW * IC, nullptr, ep,
+                                          t_workspace, t_workspace_bytes, t_tickets, t_tickets_count);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
     if (algo != 3) {
