@@ -51,6 +51,45 @@ LAYERS = {
     "c5b": (32, 56, 56, 64, 64, 3, 1, 1, 64, ("dx", "dw")),
     "c5c": (32, 56, 56, 64, 256, 1, 1, 0, 64, ("dx", "dw")),
 }
+# Layers outside BASELINE.json's five configs, for `--sweep`: the other layers of the networks the configs are taken from
+# (ResNet-18/34/50 stages, VGG, AlexNet) and of the reference's own example networks (GoogLeNet modules, its AlexNet and
+# CIFAR stems), small batches and ragged channel counts. Not part of the default line.
+OTHER_LAYERS = {
+    "vgg_112":    (32, 112, 112, 64, 128, 3, 1, 1, 64, ("fwd", "dx", "dw")),
+    "r18_s2_28":  (64, 56, 56, 64, 128, 3, 2, 1, 64, ("fwd", "dx", "dw")),
+    "r18_s2_14":  (64, 28, 28, 128, 256, 3, 2, 1, 128, ("fwd", "dx", "dw")),
+    "r18_s2_7":   (64, 14, 14, 256, 512, 3, 2, 1, 256, ("fwd", "dx", "dw")),
+    "r18_14":     (64, 14, 14, 256, 256, 3, 1, 1, 256, ("dx", "dw")),
+    "r18_7":      (64, 7, 7, 512, 512, 3, 1, 1, 512, ("dx", "dw")),
+    "r50_28_in":  (64, 28, 28, 512, 128, 1, 1, 0, 512, ("fwd", "dx", "dw")),
+    "r50_28_out": (64, 28, 28, 128, 512, 1, 1, 0, 128, ("fwd", "dx", "dw")),
+    "r50_14_in":  (64, 14, 14, 1024, 256, 1, 1, 0, 1024, ("fwd", "dx", "dw")),
+    "r50_7_in":   (64, 7, 7, 2048, 512, 1, 1, 0, 2048, ("fwd", "dx", "dw")),
+    "r50_7_out":  (64, 7, 7, 512, 2048, 1, 1, 0, 512, ("fwd", "dx", "dw")),
+    "r50_sc_28":  (64, 56, 56, 256, 512, 1, 2, 0, 256, ("fwd", "dx", "dw")),
+    "r50_sc_14":  (64, 28, 28, 512, 1024, 1, 2, 0, 512, ("fwd", "dx", "dw")),
+    "r50_sc_7":   (64, 14, 14, 1024, 2048, 1, 2, 0, 1024, ("fwd", "dx", "dw")),
+    "alex_c2":    (64, 27, 27, 96, 256, 5, 1, 2, 96, ("fwd", "dx", "dw")),
+    "alex_c3":    (64, 13, 13, 256, 384, 3, 1, 1, 256, ("fwd", "dx", "dw")),
+    "alex_c4":    (64, 13, 13, 384, 384, 3, 1, 1, 384, ("fwd", "dx", "dw")),
+    "alex_stem":  (64, 224, 224, 4, 64, 11, 4, 2, 3, ("fwd", "dw")),
+    "cifar_stem": (64, 32, 32, 4, 64, 5, 1, 2, 3, ("fwd", "dw")),
+    "g3a_1x1":    (64, 28, 28, 192, 64, 1, 1, 0, 192, ("fwd", "dx", "dw")),
+    "g3a_3x3r":   (64, 28, 28, 192, 96, 1, 1, 0, 192, ("fwd", "dx", "dw")),
+    "g3a_3x3":    (64, 28, 28, 96, 128, 3, 1, 1, 96, ("fwd", "dx", "dw")),
+    "g3a_5x5r":   (64, 28, 28, 192, 16, 1, 1, 0, 192, ("fwd", "dx", "dw")),
+    "g3a_5x5":    (64, 28, 28, 16, 32, 5, 1, 2, 16, ("fwd", "dx", "dw")),
+    "g4a_3x3":    (64, 14, 14, 96, 208, 3, 1, 1, 96, ("fwd", "dx", "dw")),
+    "g4a_5x5":    (64, 14, 14, 16, 48, 5, 1, 2, 16, ("fwd", "dx", "dw")),
+    "g5b_1x1":    (64, 7, 7, 832, 384, 1, 1, 0, 832, ("fwd", "dx", "dw")),
+    "g5b_5x5":    (64, 7, 7, 48, 128, 5, 1, 2, 48, ("fwd", "dx", "dw")),
+    "gan_4x4":    (64, 32, 32, 64, 128, 4, 2, 1, 64, ("fwd", "dx", "dw")),
+    "patch_2x2":  (64, 56, 56, 64, 128, 2, 2, 0, 64, ("fwd", "dx", "dw")),
+    "n8_14":      (8, 14, 14, 256, 256, 3, 1, 1, 256, ("fwd", "dx", "dw")),
+    "n1_56":      (1, 56, 56, 64, 64, 3, 1, 1, 64, ("fwd", "dx", "dw")),
+    "ic48_28":    (64, 28, 28, 48, 96, 3, 1, 1, 48, ("fwd", "dx", "dw")),
+    "ic32_56":    (64, 56, 56, 32, 32, 3, 1, 1, 32, ("fwd", "dx", "dw")),
+}
 RIDGE = PEAK_MFMA_F32_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9)   # FLOP per byte at which the two published peaks meet (19.7)
 UNIFORM_INPUT = {"c1", "c4a", "c4b", "c4c", "c4d"}   # BASELINE.json: inputs uniform[-1,1] (the others N(0,1)); filters He-normal
 REL_TOL, ABS_TOL = 1e-4, 1e-5
@@ -596,6 +635,9 @@ def main():
                          "the natives as an unmodified Java engine calls them")
     ap.add_argument("--no-tickets", action="store_true",
                     help="lend the scratch but no ticket words: the pieces of the items left over are added by a second kernel")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the default line: kernel / operator time and parity of OTHER_LAYERS (layers outside the five "
+                         "configs), one JSON line per row and a summary line")
     ap.add_argument("--probe-copy", action="store_true",
                     help="only run a plain 256 MiB device-to-device copy a few times (calibrates FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -621,6 +663,30 @@ def main():
     pkg = package()
     pkg.lib()   # raises if the HIP library is not built; there is no fallback
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.sweep:
+        LAYERS.update(OTHER_LAYERS)
+        worst, bad = None, []
+        for i, layer in enumerate(OTHER_LAYERS):
+            wl = Workload(pkg, torch, layer, 5000 + i)
+            for o in OTHER_LAYERS[layer][9]:
+                r = measure(wl, o, args.steps, args.warmup, with_parity=not args.no_parity)
+                rf = r["roofline"]
+                row = {"layer": layer, "op": o, "shape": list(OTHER_LAYERS[layer][:9]), "kernel_ms": rf["kernel_ms"], "ms_per_step": r["ms_per_step"],
+                       "mfma_frac": rf["mfma_frac"], "hbm_frac": rf["hbm_frac"]}
+                if "parity" in r:
+                    row["parity_ok"] = r["parity"]["ok"]
+                    row["max_err_ratio"] = r["parity"]["max_err_ratio"]
+                    if not r["parity"]["ok"]:
+                        bad.append(layer + "/" + o)
+                    if worst is None or r["parity"]["max_err_ratio"] > worst:
+                        worst = r["parity"]["max_err_ratio"]
+                print(json.dumps(row, separators=(",", ":")), flush=True)
+            wl.close()
+            del wl
+            torch.cuda.empty_cache()
+        print(json.dumps({"sweep": "layers outside the five configs", "layers": len(OTHER_LAYERS), "steps": args.steps,
+                          "parity_failed": bad, "worst_max_err_ratio": worst}, separators=(",", ":")), flush=True)
+        return
     op = args.op or LAYERS[args.layer][9][0]
 
     def seed_of(layer):
