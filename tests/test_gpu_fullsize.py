@@ -343,3 +343,54 @@ def test_kernel_split_shared_groups_full_size(dev, case):
     floor = 1e-5 * max(1.0, float(ref.pow(2).mean().sqrt()))
     err = (shared.double() - ref).abs() - 2 * torch.clamp(1e-4 * ref.abs(), min=floor)
     assert float(err.max()) <= 0.0, "%s: the two distributions differ beyond twice the bar" % (case,)
+
+
+# Tensors between 2 GB and the 2^31 elements the entries accept: the kernels that address through 2 GB buffer
+# descriptors refuse them (nothing launched) and the layer goes to the kernels that index elements. X and deltaX are
+# 2.2 GB here (44 x 512 x 512 x 48); first and last image against the oracle; backward-filter with deltaY zero outside
+# those two images, so the two images are the whole sum.
+# N = 38, 16 output channels: 1.9 GB, the largest the descriptor kernels take (byte offsets up to 2^31).
+@pytest.mark.parametrize("N,OC", [(44, 8), (38, 16)])
+def test_tensors_beyond_2GB(dev, N, OC):
+    torch = dev.torch
+    C3, DX, DW = pkg.Cuda_conv3D, pkg.Cuda_dconv3D_deltaX, pkg.Cuda_dconv3D_deltaW
+    IH, IW, IC, F, s, p = 512, 512, 48, 3, 1, 1
+    OH, OW = out_dim(IH, IW, F, F, s, s, p, p)
+    assert N * IH * IW * IC < (1 << 31) and (N * IH * IW * IC * 4 > (1 << 31)) == (N == 44)
+    g = torch.Generator(device=dev.dev).manual_seed(9100)
+    x = torch.randn((N, IH, IW, IC), generator=g, device=dev.dev)
+    w = torch.randn((OC, F, F, IC), generator=g, device=dev.dev) * float(np.sqrt(2.0 / (F * F * IC)))
+    dy = torch.randn((N, OH, OW, OC), generator=g, device=dev.dev)
+    imgs = [0, N - 1]
+    Xs, Ws, dYs = x[imgs].cpu().numpy(), w.cpu().numpy(), dy[imgs].cpu().numpy()
+
+    cw = torch.empty(F * F * IC * OC, device=dev.dev)
+    C3.kernel_remode(dev.stream, w.data_ptr(), cw.data_ptr(), F, F, OC, IC)
+    y = torch.full((N, OH, OW, OC), float("nan"), device=dev.dev)
+    C3.conv3D_GemmR(dev.streams, 1, x.data_ptr(), IH, IW, w.data_ptr(), cw.data_ptr(), F, F, y.data_ptr(), OH, OW, N, IC, OC, s, s, p, p)
+    dev.sync()
+    assert bool(torch.isfinite(y).all())
+    _check(y[imgs].cpu().numpy(), O.conv3D_f64(Xs, Ws, s, s, p, p), "forward, X of %.1f GB" % (x.numel() * 4 / 1e9))
+    del y
+
+    dx = torch.full((N, IH, IW, IC), float("nan"), device=dev.dev)
+    DX.dconv3D_deltaX_s1(dev.streams, 1, dy.data_ptr(), OH, OW, w.data_ptr(), F, F, dx.data_ptr(), IH, IW, N, IC, OC, p, p)
+    dev.sync()
+    assert bool(torch.isfinite(dx[N // 2]).all())
+    _check(dx[imgs].cpu().numpy(), O.deltaX_f64(dYs, Ws, IH, IW, s, s, p, p), "deltaX of %.1f GB" % (x.numel() * 4 / 1e9))
+    del dx
+
+    dy[1:N - 1].zero_()
+    GridZ, sizeW = 64, OC * F * F * IC    # the generic kernel: 7 x 1 blocks of the filter x GridZ workgroups
+    dw = torch.full((OC, F, F, IC), float("nan"), device=dev.dev)
+    buf = torch.full((GridZ - 1, sizeW), float("nan"), device=dev.dev)
+    DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dw.data_ptr(), buf.data_ptr(),
+                             F, F, N, IC, OC, s, s, p, p)
+    DW.buf_summary(dev.stream, buf.data_ptr(), dw.data_ptr(), GridZ - 1, sizeW)
+    dev.sync()
+    # 180 224 products per slice and element in one fp32 accumulator (an image spans a slice and a half): the floor that
+    # the other tests take for sums of a few thousand terms, 1e-5 rms, is below sqrt(180 224) rounding errors here - 4e-5
+    want = O.deltaW_f64(Xs, dYs, F, F, s, s, p, p)
+    floor = 4e-5 * float(np.sqrt(np.mean(want * want)))
+    r = O.max_err_ratio(np.ascontiguousarray(dw.cpu().numpy()), want, 1e-4, floor)
+    assert r <= 1.0, "deltaW, X of %.1f GB: err/allowed = %.3f (rel 1e-4, abs floor %.3g)" % (x.numel() * 4 / 1e9, r, floor)
