@@ -823,6 +823,7 @@ DW_STREAM_SHAPES = [
     (32, 14, 14, 128, 128, 3, 3, 2, 2, 1, 1, 8, 7),     # stride 2 onto 7x7 maps: 36 items x 7 pieces of 64 groups
     (8, 14, 14, 96, 208, 3, 3, 1, 1, 1, 1, 8, None),    # blocks filled to 61 % (96 of 128 input, 208 of 256 output channels): 72 items in a line
     (16, 14, 14, 16, 48, 5, 5, 1, 1, 2, 2, 16, 10),     # 5x5, one block filled to 19 %: 25 items x 10 pieces
+    (128, 4, 4, 96, 208, 3, 3, 1, 1, 1, 1, 2, 2),       # 72 items would meet up to 5 shares of a line, GridZ is 2: 2 pieces each on 144 workgroups
 ]
 
 
