@@ -18,6 +18,11 @@
 // and MFMA (i, j) multiplies component i of ya with component j of xa; the eight wavefronts take equal contiguous runs of
 // the piece's pixel groups (a ring of D groups in registers hides the latency, descriptors per output row return zeros for
 // padding) and their accumulators are added through LDS in the order 0, 1, 2, ...
+// FLAT: short output rows leave most of a row's last group empty - half of every group on 2x2 maps, three of eight pixels
+// on rows of 5. There a group is four consecutive pixels of the IMAGE (row-major), the descriptors cover an image, vertical
+// padding falls outside them, and every lane keeps its pixel's column and offset in X (a few vector instructions per
+// group) for the horizontal padding. That bookkeeping costs 5-13 % of the kernel's time, so rows that waste less than a
+// quarter of their groups' pixels (7, 13, 14 pixels: an eighth to a fifth) keep the groups by row.
 #include "common.hpp"
 
 namespace alpha {
@@ -30,12 +35,13 @@ struct DwStreamArgs {
     int IH, IW, IC, OH, OW, OC, FH, FW;
     int sh, sw, ph, pw;
     int GZ, icb_count, ocb_count, taps, items;
-    int GPR;      // pixel groups (4 pixels) per output row = ceil(OW / 4)
-    int TG;       // pixel groups per item = N * OH * GPR
+    int flat;     // groups of four consecutive pixels of an image instead of an output row
+    int GPR;      // pixel groups (4 pixels) per output row = ceil(OW / 4); flat: per image = ceil(OH * OW / 4)
+    int TG;       // pixel groups per item = N * OH * GPR; flat: N * GPR
     long L;       // items * TG
     int wgs;
     int R;        // > 0: every item is cut into R equal pieces, one workgroup each (see below); 0: the line of items
-    FastDiv d_OH, d_FW, d_GPR, d_taps, d_ocb;
+    FastDiv d_OH, d_OW, d_FW, d_GPR, d_taps, d_ocb;
 };
 
 // Shares [L*s/G, L*(s+1)/G): the share that holds position P is the largest s with L*s/G <= P.
@@ -44,7 +50,7 @@ __host__ __device__ inline int dws_share_of(long P, long L, int G)
     return (int)(((P + 1) * G - 1) / L);
 }
 
-template <int D>
+template <int D, bool FLAT = false>
 __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const DwStreamArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) float dws_smem[];   // [8 wavefronts][16 units][64 lanes] float4
@@ -113,16 +119,38 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const DwStreamAr
             for (int j = 0; j < 4; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
         // ---- load cursor: the row being requested (all scalar), its descriptors, the group within it -----------------------
+        //      (FLAT: the image being requested, its descriptors, the group within it; per lane the pixel's column and
+        //      its byte offset in the image of X)
         __amdgpu_buffer_rsrc_t y_rsrc, x_rsrc;
-        const int gr0 = fdiv(g_lo, p.d_GPR);   // global output row n * OH + oh
+        const int gr0 = fdiv(g_lo, p.d_GPR);   // global output row n * OH + oh; FLAT: image n
         int cur_g = g_lo - gr0 * GPR, left = total;
-        const int n0 = fdiv(gr0, p.d_OH);
-        int oh = gr0 - n0 * OH;
-        const char *y_row = reinterpret_cast<const char *>(p.dY) + (size_t)gr0 * y_row_bytes;
+        const int n0 = FLAT ? gr0 : fdiv(gr0, p.d_OH);
+        int oh = FLAT ? 0 : gr0 - n0 * OH;
+        const size_t y_img_bytes = (size_t)OH * y_row_bytes;
+        const char *y_row = reinterpret_cast<const char *>(p.dY) + (FLAT ? (size_t)n0 * y_img_bytes : (size_t)gr0 * y_row_bytes);
         const char *x_img = reinterpret_cast<const char *>(p.X) + (size_t)n0 * x_img_bytes;
         int y_goff = 0, x_goff = 0;
+        // FLAT, per lane: pixel 4 cur_g + q of the image is (oh_l, ow_l); its tap's element of X is x_off bytes into the image
+        // (negative or beyond the image above and below it: outside the descriptor). Four pixels on are `rows4` rows and
+        // `cols4` columns, and one row more where the column passes the end of its row.
+        int ow_l = 0, ow_first = 0;
+        unsigned x_off = 0, x_first = 0;
+        const int rows4 = fdiv(4, p.d_OW), cols4 = 4 - rows4 * OW;
+        const int x_row4 = p.sh * p.IW * p.IC * 4, x_col4 = p.sw * p.IC * 4;
+        const int x_step = rows4 * x_row4 + cols4 * x_col4, x_wrap = x_row4 - OW * x_col4;
+        auto place = [&](int pix, int &ow_out, unsigned &off_out) {   // FLAT: pixel `pix` of an image
+            const int oh_l = fdiv(pix, p.d_OW);
+            ow_out = pix - oh_l * OW;
+            off_out = (unsigned)((((oh_l * p.sh + fh - p.ph) * p.IW + ow_out * p.sw + fw - p.pw) * p.IC + ic_l) * 4);
+        };
         auto setup_row = [&]() {   // descriptors of row (n, oh); `left` <= 0: nothing more to read, empty descriptors
             const bool live = left > 0;
+            if (FLAT) {
+                y_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(y_row), 0, live ? (int)y_img_bytes : 0, 0x00020000);
+                x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(x_img), 0, live ? (int)x_img_bytes : 0, 0x00020000);
+                y_goff = cur_g * y_gstride;
+                return;
+            }
             y_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(y_row), 0, live ? (int)y_row_bytes : 0, 0x00020000);
             y_goff = cur_g * y_gstride;
             const int ih = oh * p.sh - p.ph + fh;
@@ -133,6 +161,27 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const DwStreamAr
         };
         floatx4 ya[D], xa[D];
         auto load = [&](int d) {
+            if (FLAT) {
+                const bool col_ok = ic_l < p.IC && (unsigned)(ow_l * p.sw + fw - p.pw) < (unsigned)p.IW;
+                ya[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, y_lane + (unsigned)y_goff, 0, 0));
+                xa[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, col_ok ? x_off : 0x80000000u, 0, 0));
+                cur_g++;
+                left--;
+                y_goff += y_gstride;
+                ow_l += cols4;
+                const int wrap = ow_l >= OW ? -1 : 0;   // per lane, without a branch
+                ow_l -= OW & wrap;
+                x_off += (unsigned)(x_step + (x_wrap & wrap));
+                if (cur_g == GPR) {   // the next image (uniform)
+                    cur_g = 0;
+                    y_row += y_img_bytes;
+                    x_img += x_img_bytes;
+                    ow_l = ow_first;
+                    x_off = x_first;
+                    setup_row();
+                }
+                return;
+            }
             ya[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, y_lane + (unsigned)y_goff, 0, 0));
             xa[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_lane + (unsigned)x_goff, 0, 0));
             // on to the next group; the next row when this one is done (scalar work only: no memory operation in a branch)
@@ -159,6 +208,10 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const DwStreamAr
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ya[d][i], xa[d][j], acc[i][j], 0, 0, 0);
         };
         if (total > 0) {
+            if (FLAT) {   // where this lane's pixel of an image's first group lies, and its pixel of this run's first group
+                place(q, ow_first, x_first);
+                place(4 * cur_g + q, ow_l, x_off);
+            }
             setup_row();
 #pragma unroll
             for (int d = 0; d < D; d++) load(d);   // groups past the end read through empty descriptors: zeros, never multiplied
@@ -222,6 +275,15 @@ static int dws_max_pieces(long items, long TG, int G)
     return most;
 }
 
+// Pixel groups as four consecutive pixels of an image (row-major) instead of an output row: where a row's groups are
+// empty to a quarter or more (rows of 1, 2, 3, 5, 6 or 9 pixels). Images beyond 512 MB do not fit the 32-bit offsets
+// within an image.
+static bool dws_flat_rows(int OH, int OW, int OC)
+{
+    const int slots = (OW + 3) / 4 * 4;
+    return 4 * (slots - OW) >= slots && (long)OH * OW * OC * 4 < (1L << 29);
+}
+
 // The least split-K factor <= GZ with which launch_deltaW_stream on a device of `units` compute units cuts the layer
 // exactly as it does with GZ (the same R pieces per item, or the same line of shares), or GZ itself where the kernel
 // does not take the layer or the split-K entries may not choose it (channel counts that fill 64 x 64 blocks to less than
@@ -231,7 +293,9 @@ int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, 
     if ((IC & 3) || (OC & 3) || IC < 4 || OC < 4 || FH < 1 || FW < 1 || GZ < 2 || units < 1 || N < 1 || OH < 1 || OW < 1) return GZ;
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
     if (100L * IC * OC < 40L * icb * 64 * ocb * 64) return GZ;   // the stricter of the split-K entries' two thresholds (the stride is not known here)
-    const long items = icb * ocb * FH * FW, TG = (long)N * OH * ((OW + 3) / 4);
+    // (the input's size is not known here: the launcher's other condition for groups by image, an image of X below 512 MB)
+    const bool flat = dws_flat_rows(OH, OW, OC);
+    const long items = icb * ocb * FH * FW, TG = flat ? (long)N * (((long)OH * OW + 3) / 4) : (long)N * OH * ((OW + 3) / 4);
     if (items >= (1L << 20) || TG >= (1L << 30) || items * TG < 8L * units || items > 4096) return GZ;
     long R = units / items;
     if (R > GZ) R = GZ;
@@ -264,8 +328,9 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
     a.ocb_count = (OC + 63) / 64;
     a.taps = FH * FW;
     const long items = (long)a.icb_count * a.ocb_count * a.taps;
-    a.GPR = (OW + 3) / 4;
-    const long TG = (long)N * OH * a.GPR;
+    a.flat = dws_flat_rows(OH, OW, OC) && (long)IH * IW * IC * 4 < (1L << 29);
+    a.GPR = a.flat ? (OH * OW + 3) / 4 : (OW + 3) / 4;
+    const long TG = a.flat ? (long)N * a.GPR : (long)N * OH * a.GPR;
     if (items >= (1L << 20) || TG >= (1L << 30)) return hipErrorNotSupported;
     a.items = (int)items;
     a.TG = (int)TG;
@@ -290,12 +355,19 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
         }
     }
     a.d_OH = make_fastdiv(OH);
+    a.d_OW = make_fastdiv(OW);
     a.d_FW = make_fastdiv(FW);
     a.d_GPR = make_fastdiv(a.GPR);
     a.d_taps = make_fastdiv(a.taps);
     a.d_ocb = make_fastdiv(a.ocb_count);
-    constexpr auto kern = delta_w_stream_kernel<6>;
     const size_t lds = (size_t)8 * 16 * 64 * sizeof(floatx4);
+    if (a.flat) {
+        constexpr auto kern = delta_w_stream_kernel<6, true>;
+        if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(a.wgs), dim3(512), lds, stream, a);
+        return hipGetLastError();
+    }
+    constexpr auto kern = delta_w_stream_kernel<6>;
     if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(a.wgs), dim3(512), lds, stream, a);
     return hipGetLastError();

@@ -824,6 +824,12 @@ DW_STREAM_SHAPES = [
     (8, 14, 14, 96, 208, 3, 3, 1, 1, 1, 1, 8, None),    # blocks filled to 61 % (96 of 128 input, 208 of 256 output channels): 72 items in a line
     (16, 14, 14, 16, 48, 5, 5, 1, 1, 2, 2, 16, 10),     # 5x5, one block filled to 19 %: 25 items x 10 pieces
     (128, 4, 4, 96, 208, 3, 3, 1, 1, 1, 1, 2, 2),       # 72 items would meet up to 5 shares of a line, GridZ is 2: 2 pieces each on 144 workgroups
+    # short rows: pixel groups of four consecutive pixels of the image
+    (64, 2, 2, 128, 128, 3, 3, 1, 1, 1, 1, 8, 7),       # 2x2 maps: a group is an image (two rows on per group)
+    (32, 5, 5, 128, 64, 3, 3, 1, 1, 1, 1, 16, 14),      # rows of 5: 7 groups per image, the last with one pixel
+    (48, 6, 6, 64, 128, 3, 3, 2, 2, 1, 1, 16, 14),      # stride 2 onto 3x3 maps: a row and a column on per group
+    (16, 9, 9, 64, 64, 5, 5, 1, 1, 2, 2, 12, 10),       # rows of 9, 5x5 filter
+    (2048, 1, 1, 128, 64, 1, 1, 1, 1, 0, 0, 128, 128),  # 1x1 maps: one pixel per group (a fully connected layer's shape)
 ]
 
 
