@@ -334,6 +334,10 @@ hipError_t launch_ks_remode(hipStream_t s, int version, const float *W, int FH, 
                             int mCFH, int mCFW, int OC, int IC, int sh, int sw);
 hipError_t launch_buf_summary(hipStream_t s, const float *buf, float *dW, int part, int sizeW);
 // Column sums of deltaY[GK][OC] per K slice (bias gradient), same slice partition and destinations as backward-filter.
+// Backward-filter for 4 stored input channels (delta_w_stem.hip): its own equal cut of the pixels into GridZ slices,
+// slice 0 to deltaW, slice z to deltaW_buf[z - 1]. hipErrorNotSupported: nothing launched.
+hipError_t launch_deltaW_stem(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
+                              int N, int IH, int IW, int OH, int OW, int OC, int FH, int FW, int sh, int sw, int ph, int pw, int GZ);
 hipError_t launch_col_sum(hipStream_t s, const float *dY, float *dB, float *dB_buf, int OC, int GK, int GK_slice, int GZ);
 
 // Backward of batch normalisation (batchnorm_backward.hip). form: 0 = X_norm given in S, 1 = X_norm = (S - B) / A,

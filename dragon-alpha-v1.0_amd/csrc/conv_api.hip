@@ -421,7 +421,8 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     a.GZ = GridZ;
     a.GK_slice = (a.GK / GridZ) >> 3 << 3;
     const int algo = fwd_algo();
-    // Which kernel (all but the first share the slice partition and the outputs):
+    // Which kernel (all but the first two share the slice partition and the outputs):
+    //  - 4 stored input channels, GridZ of 2 or more: the kernel of delta_w_stem.hip (its own equal cut of the pixels);
     //  - layers whose channel counts fill 64 x 64 blocks well enough (below), GridZ of 2 or more: the persistent kernel of
     //    delta_w_stream.hip (its own partition of the pixels among deltaW and the buffers; a bias gradient takes a pass of
     //    its own over deltaY then, so layers where another kernel produces it on the way stay with that kernel);
@@ -441,6 +442,12 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     const bool rows_shape = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1));
     const bool stream_filled = 100L * IC * OC >= (rows_shape ? 40L : 15L) * icb * 64 * ocb * 64;
     const bool rows_fill = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1)) && icb * ((OC + 31) / 32) * GridZ >= 2L * device_cu_count();
+    if (algo == 0 && IC == 4 && GridZ >= 2) {
+        // 4 stored input channels (a network's first layer): the 16 columns of an MFMA operand are 16 taps
+        hipError_t e = launch_deltaW_stem(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, OH, OW, OC, FH, FW, sh, sw, ph, pw, GridZ);
+        if (e == hipSuccess && dB) e = launch_col_sum(stream0(streams), dY, dB, dB_buf, OC, a.GK, a.GK_slice, GridZ);
+        if (e != hipErrorNotSupported) return hip_status(e, fn);
+    }
     if (algo == 0 && stream_filled && !(dB && (rows_fill || w1))) {
         // the same arithmetic with the reduction dealt out evenly (its own partition of the pixels among the buffers)
         hipError_t e = launch_deltaW_stream(stream0(streams), X, dY, dW, dW_buf, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw, GridZ);

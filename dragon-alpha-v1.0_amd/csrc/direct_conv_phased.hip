@@ -239,10 +239,12 @@ __global__ __launch_bounds__(512, 1) void direct_conv_phased_kernel(const Direct
 #pragma unroll
                         for (int r = 0; r < 4; r++) emit(floatx4{acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]}, opix[i][r]);
                 } else if (pairs == 0) {
-                    // a phase without taps (uniform): nothing to add, every wavefront writes the zeros of its units
+                    // a phase without taps (uniform): nothing to add, every wavefront writes the zeros of its units (from
+                    // registers of their own, not a constant the compiler may keep elsewhere: the guarded store holds its
+                    // data registers for two wait states)
 #pragma unroll
                     for (int h = 0; h < 2; h++)
-                        if (w + 8 * h < 4 * T) emit(floatx4{0.f, 0.f, 0.f, 0.f}, mine[h]);
+                        if (w + 8 * h < 4 * T) emit(acc[0][h], mine[h]);
                 } else {
                     // unit u = 4 i + r (one 128-bit store per lane); partial results [wavefront][unit][lane], added in the
                     // order of the wavefronts' numbers; wavefront w finishes the units u = w and w + 8

@@ -80,16 +80,25 @@ def test_hip_library_matches_the_golden_vectors(name):
     dx = dev.guarded(N, IH, IW, IC)
     DX.dconv3D_deltaX_crossAdd(S, 1, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, dx.data_ptr(), IH, IW, N, IC, OC, sh, sw, ph, pw)
     _ok(dev.get(dx), d["dX"], name + " deltaX crossAdd")
-    # backward-filter: slices one by one, then the Kahan sum of the golden partials bit for bit
-    dw = dev.guarded(OC, FH, FW, IC)
-    buf = dev.empty(GRIDZ - 1, OC * FH * FW * IC, fill=float("nan"))
-    DW.dconv3D_deltaW_GemmSK(S, 1, GRIDZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dw.data_ptr(), buf.data_ptr(), FH, FW,
-                             N, IC, OC, sh, sw, ph, pw)
-    parts = [dev.get(dw)] + [b.reshape(OC, FH, FW, IC) for b in dev.get(buf)]
-    for z in range(GRIDZ):
-        _ok(parts[z], d["dW_parts"][z].astype(np.float64), "%s deltaW slice %d" % (name, z))
-    DW.buf_summary(dev.stream, buf.data_ptr(), dw.data_ptr(), GRIDZ - 1, OC * FH * FW * IC)
-    _ok(dev.get(dw), d["dW"], name + " deltaW after buf_summary")
+    # backward-filter: slices one by one through the kernels that keep the reference's slices (the default kernels for
+    # 4 stored input channels and for large layers cut the pixels their own way: only their sum is the reference's), the
+    # sum through the default path, then the Kahan sum of the golden partials bit for bit
+    L = pkg.lib()
+    for algo in (3, 4, 0):
+        dw = dev.guarded(OC, FH, FW, IC)
+        buf = dev.empty(GRIDZ - 1, OC * FH * FW * IC, fill=float("nan"))
+        try:
+            L.alpha_conv_set_fwd_algo(algo)
+            DW.dconv3D_deltaW_GemmSK(S, 1, GRIDZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dw.data_ptr(), buf.data_ptr(), FH, FW,
+                                     N, IC, OC, sh, sw, ph, pw)
+        finally:
+            L.alpha_conv_set_fwd_algo(0)
+        parts = [dev.get(dw)] + [b.reshape(OC, FH, FW, IC) for b in dev.get(buf)]
+        if algo != 0:
+            for z in range(GRIDZ):
+                _ok(parts[z], d["dW_parts"][z].astype(np.float64), "%s deltaW slice %d (algo %d)" % (name, z, algo))
+        DW.buf_summary(dev.stream, buf.data_ptr(), dw.data_ptr(), GRIDZ - 1, OC * FH * FW * IC)
+        _ok(dev.get(dw), d["dW"], "%s deltaW after buf_summary (algo %d)" % (name, algo))
     gp = dev.put(d["dW_parts"])
     DW.buf_summary(dev.stream, gp[1:].data_ptr(), gp[0].data_ptr(), GRIDZ - 1, OC * FH * FW * IC)
     assert np.array_equal(dev.get(gp)[0], d["dW_kahan"])

@@ -867,6 +867,52 @@ def test_deltaW_persistent_kernel_sum_and_reproducibility(dev, shape):
         L.alpha_conv_set_fwd_algo(0)
 
 
+DW_STEM_SHAPES = [
+    # N, IH, IW, OC, FH, FW, sh, sw, ph, pw, GridZ: 4 stored input channels (all four carry data here), the kernel whose MFMA
+    # columns are 16 taps; its own equal cut of the pixels into GridZ slices, so the sum is compared
+    (8, 32, 32, 64, 3, 3, 1, 1, 1, 1, 16),      # a VGG's first layer: 9 of a tap group's 16 taps, eight parts of a slice per workgroup
+    (4, 40, 36, 64, 7, 7, 2, 2, 3, 3, 8),       # a ResNet's stem: four tap groups (the last with one tap), rows of 18 pixels (ragged last group)
+    (6, 32, 32, 96, 6, 6, 2, 2, 2, 2, 4),       # the reference's AlexNet on CIFAR: three tap groups, two blocks of output channels (the second half full)
+    (4, 32, 32, 64, 5, 5, 1, 1, 2, 2, 128),     # GridZ 128: eight pixel groups a slice, one tap group per workgroup
+    (2, 23, 29, 20, 11, 11, 4, 4, 2, 2, 3),     # 121 taps: eight tap groups in a workgroup, 20 output channels, odd sizes
+    (4, 9, 9, 8, 1, 1, 1, 1, 0, 0, 2),          # a single tap
+    (3, 12, 12, 32, 3, 5, 2, 1, 1, 2, 5),       # 3x5 filter, stride 2 x 1
+    (5, 10, 10, 16, 3, 3, 1, 1, 1, 1, 64),      # more slices than pixel groups a part: empty parts and empty slices
+]
+
+
+@pytest.mark.parametrize("shape", DW_STEM_SHAPES)
+def test_deltaW_stem_kernel_sum_and_reproducibility(dev, shape):
+    N, IH, IW, OC, FH, FW, sh, sw, ph, pw, GridZ = shape
+    IC = 4
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    X, dY = normal((N, IH, IW, IC), 3501), normal((N, OH, OW, OC), 3502)
+    want = O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw)
+    x, dy = dev.put(X), dev.put(dY)
+    sizeW = OC * FH * FW * IC
+    runs = []
+    for _ in range(2):
+        dWo = dev.guarded(OC, FH, FW, IC)
+        buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+        DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
+                                 FH, FW, N, IC, OC, sh, sw, ph, pw)
+        runs.append(np.concatenate([dev.get(dWo).reshape(1, -1), dev.get(buf)]))
+        assert np.isfinite(runs[-1]).all(), "an element of deltaW or of a buffer was not written %s" % (shape,)
+        check(_sum_partials(dev, dWo, buf, GridZ), want, "stem dW GridZ=%d %s" % (GridZ, shape))
+    assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32)), "partial sums differ between two runs %s" % (shape,)
+    # the same layer through the generic kernel (the reference's slices): the totals agree within tolerance
+    L = pkg.lib()
+    try:
+        L.alpha_conv_set_fwd_algo(3)
+        dWo = dev.guarded(OC, FH, FW, IC)
+        buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+        DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
+                                 FH, FW, N, IC, OC, sh, sw, ph, pw)
+        check(_sum_partials(dev, dWo, buf, GridZ), want, "generic kernel GridZ=%d %s" % (GridZ, shape))
+    finally:
+        L.alpha_conv_set_fwd_algo(0)
+
+
 DW_ROWS_SHAPES = [
     # stride-1 layers served by the row-streaming kernel: N, IH, IW, IC, OC, F, p, GridZ
     (4, 56, 56, 64, 64, 3, 1, 16),     # c5b geometry
