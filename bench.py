@@ -89,6 +89,23 @@ OTHER_LAYERS = {
     "n1_56":      (1, 56, 56, 64, 64, 3, 1, 1, 64, ("fwd", "dx", "dw")),
     "ic48_28":    (64, 28, 28, 48, 96, 3, 1, 1, 48, ("fwd", "dx", "dw")),
     "ic32_56":    (64, 56, 56, 32, 32, 3, 1, 1, 32, ("fwd", "dx", "dw")),
+    # the reference's CIFAR-10 experiments (experiments/alpha_code/src/cifar10: VGG, ResNet, GoogLeNet, AlexNet) at their
+    # training batch of 512, and first layers (3 channels stored as 4) in backward-filter
+    "cf_vgg_32":  (512, 32, 32, 64, 64, 3, 1, 1, 64, ("fwd", "dx", "dw")),
+    "cf_vgg_8":   (512, 8, 8, 256, 256, 3, 1, 1, 256, ("fwd", "dx", "dw")),
+    "cf_vgg_4":   (512, 4, 4, 512, 512, 3, 1, 1, 512, ("fwd", "dx", "dw")),
+    "cf_vgg_2":   (512, 2, 2, 512, 512, 3, 1, 1, 512, ("fwd", "dx", "dw")),
+    "cf_res_s2":  (512, 8, 8, 256, 512, 3, 2, 1, 256, ("fwd", "dx", "dw")),
+    "cf_res_sc":  (512, 8, 8, 256, 512, 1, 2, 0, 256, ("fwd", "dx", "dw")),
+    "cf_goo_c2":  (512, 16, 16, 64, 192, 3, 1, 1, 64, ("fwd", "dx", "dw")),
+    "cf_goo_4":   (512, 4, 4, 96, 208, 3, 1, 1, 96, ("fwd", "dx", "dw")),
+    "cf_goo_2":   (512, 2, 2, 192, 384, 3, 1, 1, 192, ("fwd", "dx", "dw")),
+    "cf_alex_c2": (512, 8, 8, 96, 256, 5, 1, 2, 96, ("fwd", "dx", "dw")),
+    "cf_alex_c3": (512, 4, 4, 256, 384, 3, 1, 1, 256, ("fwd", "dx", "dw")),
+    "cf_first":   (512, 32, 32, 4, 64, 3, 1, 1, 3, ("fwd", "dw")),
+    "cf_first_5": (512, 32, 32, 4, 64, 5, 1, 2, 3, ("fwd", "dw")),
+    "cf_first_a": (512, 32, 32, 4, 96, 6, 2, 2, 3, ("fwd", "dw")),
+    "stem_7x7":   (64, 224, 224, 4, 64, 7, 2, 3, 3, ("dw",)),
 }
 RIDGE = PEAK_MFMA_F32_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9)   # FLOP per byte at which the two published peaks meet (19.7)
 UNIFORM_INPUT = {"c1", "c4a", "c4b", "c4c", "c4d"}   # BASELINE.json: inputs uniform[-1,1] (the others N(0,1)); filters He-normal
