@@ -305,6 +305,23 @@ int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, 
     return most < 2 ? 2 : most;
 }
 
+// The split-K factor a host layer that owns GridZ should pass: deltaW_stream_least_GridZ where GZ is enough for the kernel's
+// own cut, and where it is not (the reference sizes GridZ for the slices of its kernels: 2 on 4x4 maps at N = 512, where 72
+// items on 256 compute units meet up to 5 shares each) the pieces per item that cut wants, up to GZ_cap.
+int deltaW_stream_fill_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ, int GZ_cap)
+{
+    const int least = deltaW_stream_least_GridZ(units, N, OH, OW, IC, OC, FH, FW, GZ);
+    if (least != GZ || GZ < 2 || GZ_cap <= GZ || (IC & 3) || (OC & 3) || IC < 4 || OC < 4 || FH < 1 || FW < 1 || units < 1 || N < 1 || OH < 1 || OW < 1) return least;
+    const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
+    if (100L * IC * OC < 40L * icb * 64 * ocb * 64) return least;
+    const bool flat = dws_flat_rows(OH, OW, OC);
+    const long items = icb * ocb * FH * FW, TG = flat ? (long)N * (((long)OH * OW + 3) / 4) : (long)N * OH * ((OW + 3) / 4);
+    if (items >= (1L << 20) || TG >= (1L << 30) || items * TG < 8L * units || items > 4096) return least;
+    const long R = units / items;
+    const long want = (R >= 1 && 20 * R * items >= 19L * units) ? R : dws_max_pieces(items, TG, units);
+    return want > GZ && want <= GZ_cap ? (int)want : least;
+}
+
 // Returns hipErrorNotSupported (nothing launched) when the layer does not fit; the caller then uses another kernel.
 hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float *dY, float *dW, float *dW_buf,
                                 int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,

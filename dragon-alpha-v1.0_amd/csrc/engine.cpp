@@ -12,6 +12,7 @@
 namespace alpha {
 // delta_w_stream.hip (host code): the least split-K factor with which the persistent backward-filter kernel cuts a layer as it does with GZ
 int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ);
+int deltaW_stream_fill_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ, int GZ_cap);
 }
 
 #include <hip/hip_runtime.h>
@@ -174,7 +175,7 @@ void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int
         GridZ = want;
     }
     if (c->deltaW_SK_leastUnits > 0 && !winograd)
-        GridZ = alpha::deltaW_stream_least_GridZ(c->deltaW_SK_leastUnits, N, OH, OW, IC, OC, FH, FW, GridZ);
+        GridZ = alpha::deltaW_stream_fill_GridZ(c->deltaW_SK_leastUnits, N, OH, OW, IC, OC, FH, FW, GridZ, GridZ2);
     out->GridZ = GridZ;
     out->scratch_floats = (long)OC * FH * FW * IC * (GridZ - 1);
     if (winograd) {

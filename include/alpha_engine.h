@@ -47,10 +47,12 @@ typedef struct alpha_engine_config {
                                      F(3x3,2x2). 1: with the reference's GridZ; > 1: the number of compute units to fill - GridZ becomes
                                      that many workgroups' worth of slices (at least 64 tiles each). Default 0 */
     int deltaW_SK_leastUnits;     /* this build only: > 0 = the number of compute units of the device; the split-K factor is then lowered
-                                     (never raised) to the least value with which the persistent backward-filter kernel cuts the layer
-                                     the same way - it deals the pixels evenly among the compute units whatever GridZ is, so a larger
-                                     GridZ only adds buffers of zeros for buf_summary to add. alpha_engine_config_default: 0 = the reference's GridZ
-                                     exactly; alpha_engine_create sets it to the device's compute units */
+                                     to the least value with which the persistent backward-filter kernel cuts the layer the same way -
+                                     it deals the pixels evenly among the compute units whatever GridZ is, so a larger GridZ only adds
+                                     buffers of zeros for buf_summary to add -, and raised, within the reference's own cap of GK / 256,
+                                     where the reference's value has fewer buffers than that kernel's cut needs pieces per item (2 on
+                                     4x4 maps at N = 512). alpha_engine_config_default: 0 = the reference's GridZ exactly;
+                                     alpha_engine_create sets it to the device's compute units */
     int conv_workspace;           /* this build only: 1 = forward and stride-1 backward-data calls lend the library 1 MiB of the engine's
                                      scratch for the duration of the call (alpha_conv_bind_workspace), with which the kernel without
                                      LDS deals a layer of few items per compute unit out in equal shares (7x7x512 and 14x14x256 maps at

@@ -105,7 +105,7 @@ def test_deltaW_fill_option_only_raises_the_split_k_factor():
     assert big == E.plan_deltaW(cfg, 14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1).GridZ
 
 
-def test_deltaW_least_option_only_lowers_the_split_k_factor():
+def test_deltaW_least_option_sets_the_split_k_factor_the_persistent_kernel_needs():
     """deltaW_SK_leastUnits is this build's option (no reference flag): the persistent backward-filter kernel cuts every
     (tap, 64 x 64 block) item into R = floor(units / items) pieces whatever GridZ is (or the line of items into one share per
     unit), so GridZ can come down to R (or to the most shares an item meets) without changing what the kernel does."""
@@ -122,8 +122,14 @@ def test_deltaW_least_option_only_lowers_the_split_k_factor():
     assert E.plan_deltaW(cfg, 56, 56, 56, 56, 1, 1, 32, 64, 256, 1, 1).GridZ == 64
     # c2c: 144 items form a line cut into 256 shares, an item meets 2 or 3 of them: the reference's 3 stays
     assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 128, 256, 256, 1, 1).GridZ == 3
-    # never raised: 9 items on 256 units want 28, the reference gives 2 (GK = 512)
+    # not raised beyond the reference's own cap GK >> 8: 9 items on 256 units want 28, the reference gives 2 (GK = 512)
     assert E.plan_deltaW(cfg, 8, 8, 8, 8, 3, 3, 8, 64, 64, 1, 1).GridZ == 2
+    # raised within that cap where the reference's value has fewer buffers than the kernel's cut needs pieces: 4x4 maps at
+    # N = 512 (GK = 8192, the reference gives 2), 96 -> 208 channels: 72 items in a line of 256 shares meet up to 5 of them;
+    # 256 -> 384: 216 items, up to 3
+    assert E.plan_deltaW(E.default_config(256), 4, 4, 4, 4, 3, 3, 512, 96, 208, 1, 1).GridZ == 2
+    assert E.plan_deltaW(cfg, 4, 4, 4, 4, 3, 3, 512, 96, 208, 1, 1).GridZ == 5
+    assert E.plan_deltaW(cfg, 4, 4, 4, 4, 3, 3, 512, 256, 384, 1, 1).GridZ == 3
     # channel counts that fill the 64 x 64 blocks to less than 75 % go to other kernels: unchanged
     cfg0 = E.default_config(256)
     for shape in [(28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1), (14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1)]:
