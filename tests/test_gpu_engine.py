@@ -159,6 +159,8 @@ def test_engine_conv3D_biased(dev, eng):
     (8, 12, 12, 36, 44, 1, 1, 0),
     (8, 20, 20, 32, 48, 3, 2, 1),
     (4, 9, 9, 16, 24, 3, 1, 1),
+    (16, 32, 32, 4, 64, 3, 1, 1),      # a first layer (4 stored input channels): its own kernel, the column sums as a pass
+    (8, 40, 40, 4, 96, 7, 2, 3),
 ])
 def test_engine_deltaW_with_bias_gradient(dev, eng, shape):
     """deltaB[oc] = sum over all pixels of deltaY (the reference: field_sum(deltaY, OC) after dconv3D_deltaW)."""

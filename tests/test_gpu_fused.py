@@ -142,6 +142,7 @@ def test_backward_data_with_the_leaky_relu_derivative_in_the_epilogue(dev, shape
 
 @pytest.mark.parametrize("shape", [(4, 16, 16, 64, 128, 3, 3, 2, 2, 1, 1),     # four phases in one launch of the kernel without LDS
                                    (6, 14, 18, 132, 96, 3, 3, 2, 2, 1, 1),     # the same, three blocks of produced channels (the last ragged), ragged last tile
+                                   (4, 14, 14, 128, 256, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2: three phases without taps, whose zeros pass the gate too
                                    (4, 13, 11, 16, 16, 5, 4, 3, 2, 2, 1)])     # one launch of the generic kernel per phase
 def test_strided_backward_data_with_the_leaky_relu_derivative_in_the_epilogue(dev, shape):
     N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = shape
