@@ -360,6 +360,56 @@ def test_engine_random_geometries(dev, eng, case):
     check(dev.get(dw), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "deltaW %s" % (case,))
 
 
+def _random_small_map_cases(count, seed):
+    """Seeded random layers on small maps (2 to 14 pixels a side) at larger batches, channel counts on both sides of the 64-wide
+    blocks and 4 stored input channels: the geometries of the reference's CIFAR-10 networks' later stages, where the work
+    items per compute unit are few and the persistent backward-filter kernel's rows are short."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    cases = []
+    while len(cases) < count:
+        F_ = int(rng.choice([1, 3, 3, 5]))
+        s_ = int(rng.choice([1, 1, 2]))
+        p_ = int(rng.choice([0, F_ // 2]))
+        IH, IW = int(rng.choice([2, 3, 4, 5, 6, 7, 8, 9, 13, 14])), int(rng.choice([2, 3, 4, 5, 6, 7, 8, 9, 13, 14]))
+        IC = int(rng.choice([4, 16, 32, 48, 64, 96, 128, 256]))
+        OC = int(rng.choice([8, 36, 64, 96, 128, 208, 256]))
+        N = int(rng.choice([32, 64, 128]))
+        if IH + 2 * p_ < F_ or IW + 2 * p_ < F_ or s_ > F_:
+            continue
+        OH, OW = out_dim(IH, IW, F_, F_, s_, s_, p_, p_)
+        if OH < 1 or OW < 1 or N * OH * OW * OC * IC * F_ * F_ > 300_000_000:
+            continue
+        cases.append((N, IH, IW, IC, OC, F_, F_, s_, s_, p_, p_))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_small_map_cases(30, 20250217))
+def test_engine_random_small_maps(dev, eng, case):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw = case
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    seed = 7500 + (hash(case) % 1000)
+    X, W, dY = normal((N, IH, IW, IC), seed), he_normal(OC, FH, FW, IC, seed + 1), normal((N, OH, OW, OC), seed + 2)
+    x, w, dy = dev.put(X), dev.put(W), dev.put(dY)
+    y = dev.empty(N, OH, OW, OC, fill=float("nan"))
+    dw = dev.empty(OC, FH, FW, IC, fill=float("nan"))
+    eng.conv3D(y.data_ptr(), OH, OW, x.data_ptr(), IH, IW, w.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
+    eng.dconv3D_deltaW(dw.data_ptr(), FH, FW, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, N, IC, OC, sh, sw, ph, pw)
+    eng.sync()
+    check(dev.get(y), O.conv3D_f64(X, W, sh, sw, ph, pw), "conv3D %s" % (case,))
+    check(dev.get(dw), O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw), "deltaW %s" % (case,))
+    want = O.deltaX_f64(dY, W, IH, IW, sh, sw, ph, pw)
+    L = pkg.lib()
+    try:
+        for sharing in ((-1,) if sh == 1 else (-1, 0, 1)):   # strided: both distributions of the kernel-split kernel's work
+            L.alpha_conv_set_kernel_split_sharing(sharing)
+            dx = dev.empty(N, IH, IW, IC, fill=float("nan"))
+            eng.dconv3D_deltaX(dx.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, w.data_ptr(), FH, FW, N, IC, OC, sh, sw, ph, pw)
+            eng.sync()
+            check(dev.get(dx), want, "deltaX sharing %d %s" % (sharing, case))
+    finally:
+        L.alpha_conv_set_kernel_split_sharing(-1)
+
+
 def _random_3x3_cases(count, seed):
     """Seeded random 3x3 stride-1 layers with channel counts the LDS-halo kernels take: row widths from 3 to 62 (both
     row-width classes of the halo-prefetching kernel and its limits), batch sizes that give anything from a fraction of
