@@ -176,6 +176,14 @@ void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int
     }
     if (c->deltaW_SK_leastUnits > 0 && !winograd)
         GridZ = alpha::deltaW_stream_fill_GridZ(c->deltaW_SK_leastUnits, N, OH, OW, IC, OC, FH, FW, GridZ, GridZ2);
+    if (c->deltaW_SK_leastUnits > 0 && IC == 4 && FH * FW <= 128) {
+        // 4 stored input channels: the kernel of delta_w_stem.hip runs GridZ x (groups of 16 taps) x (blocks of 64 output
+        // channels) workgroups at most; a 3x3 first layer at the reference's 128 fills half of 256 compute units
+        const int per_slice = ((FH * FW + 15) / 16) * ((OC + 63) / 64);
+        int want = (c->deltaW_SK_leastUnits + per_slice - 1) / per_slice;
+        if (want > GridZ2) want = GridZ2;
+        if (want > GridZ) GridZ = want;
+    }
     out->GridZ = GridZ;
     out->scratch_floats = (long)OC * FH * FW * IC * (GridZ - 1);
     if (winograd) {

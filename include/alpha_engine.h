@@ -51,7 +51,8 @@ typedef struct alpha_engine_config {
                                      it deals the pixels evenly among the compute units whatever GridZ is, so a larger GridZ only adds
                                      buffers of zeros for buf_summary to add -, and raised, within the reference's own cap of GK / 256,
                                      where the reference's value has fewer buffers than that kernel's cut needs pieces per item (2 on
-                                     4x4 maps at N = 512). alpha_engine_config_default: 0 = the reference's GridZ exactly;
+                                     4x4 maps at N = 512; first layers - 4 stored input channels -, whose kernel runs GridZ x groups of
+                                     16 taps x blocks of 64 output channels workgroups). alpha_engine_config_default: 0 = the reference's GridZ exactly;
                                      alpha_engine_create sets it to the device's compute units */
     int conv_workspace;           /* this build only: 1 = forward and stride-1 backward-data calls lend the library 1 MiB of the engine's
                                      scratch for the duration of the call (alpha_conv_bind_workspace), with which the kernel without

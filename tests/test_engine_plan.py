@@ -130,6 +130,11 @@ def test_deltaW_least_option_sets_the_split_k_factor_the_persistent_kernel_needs
     assert E.plan_deltaW(E.default_config(256), 4, 4, 4, 4, 3, 3, 512, 96, 208, 1, 1).GridZ == 2
     assert E.plan_deltaW(cfg, 4, 4, 4, 4, 3, 3, 512, 96, 208, 1, 1).GridZ == 5
     assert E.plan_deltaW(cfg, 4, 4, 4, 4, 3, 3, 512, 256, 384, 1, 1).GridZ == 3
+    # a first layer (4 stored input channels): one workgroup per slice, group of 16 taps and block of 64 output channels
+    assert E.plan_deltaW(E.default_config(256), 32, 32, 32, 32, 3, 3, 512, 4, 64, 1, 1).GridZ == 128
+    assert E.plan_deltaW(cfg, 32, 32, 32, 32, 3, 3, 512, 4, 64, 1, 1).GridZ == 256      # 9 taps, 64 channels: a workgroup per slice
+    assert E.plan_deltaW(cfg, 224, 224, 112, 112, 7, 7, 64, 4, 64, 2, 2).GridZ == 128   # 49 taps: four groups, 64 slices would do
+    assert E.plan_deltaW(cfg, 32, 32, 32, 32, 3, 3, 4, 4, 64, 1, 1).GridZ == 16         # c1: GK / 256 = 16 caps it
     # channel counts that fill the 64 x 64 blocks to less than 75 % go to other kernels: unchanged
     cfg0 = E.default_config(256)
     for shape in [(28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1), (14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1)]:
