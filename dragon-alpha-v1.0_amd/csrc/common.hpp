@@ -287,6 +287,7 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
                                 int N, int IH, int IW, int IC, int OH, int OW, int OC, int FH, int FW,
                                 int sh, int sw, int ph, int pw, int GZ);
 int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ);
+int deltaW_stream_block_fill(int IC, int OC);
 int deltaW_stream_fill_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ, int GZ_cap);
 
 // Backward-filter with the filter tap in the grid and both operands straight from memory (delta_w_taps.hip): any filter,

@@ -436,11 +436,12 @@ int deltaW_impl(const char *fn, const int64_t *streams, int length, int GridZ,
     const bool w1 = FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
     const bool blocks_filled = 4L * IC * OC >= 3L * icb * 64 * ocb * 64;
-    // what the persistent kernel needs of its 64 x 64 blocks to win: 40 % where the row-streaming kernel is the alternative
+    // what the persistent kernel needs of its blocks (64 x 64 channels, or 16 x 1 to 3 channels per lane on either side
+    // where that holds the channels in as many blocks: 96 = 2 x 48, 32 = 1 x 32) to win: 40 % where the row-streaming kernel is the alternative
     // (96 -> 208 channels 3x3: 0.066 against 0.103 ms; 32 -> 32: 0.107 against 0.074), 15 % where the generic kernel is
     // (5x5, 16 -> 48: 0.026 against 0.043 ms; 16 -> 32: 0.078 against 0.047)
     const bool rows_shape = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1));
-    const bool stream_filled = 100L * IC * OC >= (rows_shape ? 40L : 15L) * icb * 64 * ocb * 64;
+    const bool stream_filled = deltaW_stream_block_fill(IC, OC) >= (rows_shape ? 40 : 15);
     const bool rows_fill = sh == 1 && sw == 1 && ((FH == 3 && FW == 3) || (FH == 1 && FW == 1)) && icb * ((OC + 31) / 32) * GridZ >= 2L * device_cu_count();
     if (algo == 0 && IC == 4 && GridZ >= 2) {
         // 4 stored input channels (a network's first layer): the 16 columns of an MFMA operand are 16 taps

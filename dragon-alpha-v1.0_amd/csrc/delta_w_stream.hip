@@ -28,6 +28,20 @@ static bool dws_flat_rows(int OH, int OW, int OC)
     return 4 * (slots - OW) >= slots && (long)OH * OW * OC * 4 < (1L << 29);
 }
 
+static int dws_per_lane(int C)
+{
+    const int blocks = (C + 63) / 64, n = (C + 16 * blocks - 1) / (16 * blocks);
+    return (n < 4 && C % n == 0) ? n : 4;
+}
+
+// How full the kernel's blocks of the filter are, in per cent: channels / (blocks x 16 x channels per lane), both sides.
+int deltaW_stream_block_fill(int IC, int OC)
+{
+    if (IC < 1 || OC < 1) return 0;
+    const long ib = (IC + 63) / 64 * 16L * dws_per_lane(IC), ob = (OC + 63) / 64 * 16L * dws_per_lane(OC);
+    return (int)(100L * IC * OC / (ib * ob));
+}
+
 // The least split-K factor <= GZ with which launch_deltaW_stream on a device of `units` compute units cuts the layer
 // exactly as it does with GZ (the same R pieces per item, or the same line of shares), or GZ itself where the kernel
 // does not take the layer or the split-K entries may not choose it (channel counts that fill 64 x 64 blocks to less than
@@ -36,7 +50,7 @@ int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, 
 {
     if ((IC & 3) || (OC & 3) || IC < 4 || OC < 4 || FH < 1 || FW < 1 || GZ < 2 || units < 1 || N < 1 || OH < 1 || OW < 1) return GZ;
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
-    if (100L * IC * OC < 40L * icb * 64 * ocb * 64) return GZ;   // the stricter of the split-K entries' two thresholds (the stride is not known here)
+    if (deltaW_stream_block_fill(IC, OC) < 40) return GZ;   // the stricter of the split-K entries' two thresholds (the stride is not known here)
     // (the input's size is not known here: the launcher's other condition for groups by image, an image of X below 512 MB)
     const bool flat = dws_flat_rows(OH, OW, OC);
     const long items = icb * ocb * FH * FW, TG = flat ? (long)N * (((long)OH * OW + 3) / 4) : (long)N * OH * ((OW + 3) / 4);
@@ -57,7 +71,7 @@ int deltaW_stream_fill_GridZ(int units, int N, int OH, int OW, int IC, int OC, i
     const int least = deltaW_stream_least_GridZ(units, N, OH, OW, IC, OC, FH, FW, GZ);
     if (least != GZ || GZ < 2 || GZ_cap <= GZ || (IC & 3) || (OC & 3) || IC < 4 || OC < 4 || FH < 1 || FW < 1 || units < 1 || N < 1 || OH < 1 || OW < 1) return least;
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
-    if (100L * IC * OC < 40L * icb * 64 * ocb * 64) return least;
+    if (deltaW_stream_block_fill(IC, OC) < 40) return least;
     const bool flat = dws_flat_rows(OH, OW, OC);
     const long items = icb * ocb * FH * FW, TG = flat ? (long)N * (((long)OH * OW + 3) / 4) : (long)N * OH * ((OW + 3) / 4);
     if (items >= (1L << 20) || TG >= (1L << 30) || items * TG < 8L * units || items > 4096) return least;
@@ -87,6 +101,11 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
     a.GZ = GZ;
     a.icb_count = (IC + 63) / 64;
     a.ocb_count = (OC + 63) / 64;
+    // Channels per lane: the least with which the same number of blocks (of 16 per-lane groups) holds the channels - 96
+    // channels are two blocks of 48 (3 per lane) instead of one of 64 and one half-empty -, where the channel count is a
+    // multiple of it (a lane's group never straddles the end of a pixel's channels). With pixel groups by image: 4.
+    int ni = dws_per_lane(OC), nj = dws_per_lane(IC);
+    if (dws_flat_rows(OH, OW, OC) && (long)IH * IW * IC * 4 < (1L << 29)) ni = nj = 4;
     a.taps = FH * FW;
     const long items = (long)a.icb_count * a.ocb_count * a.taps;
     const bool flat = dws_flat_rows(OH, OW, OC) && (long)IH * IW * IC * 4 < (1L << 29);
@@ -123,6 +142,9 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
     a.d_ocb = make_fastdiv(a.ocb_count);
     const size_t lds = (size_t)8 * 16 * 64 * sizeof(floatx4);
     if (flat) return launch_deltaW_stream_flat(stream, a, lds);
+    if (ni < 4 && nj < 4) return launch_deltaW_stream_narrow_xy(stream, a, lds, ni, nj);
+    if (nj < 4) return launch_deltaW_stream_narrow_x(stream, a, lds, nj);
+    if (ni < 4) return launch_deltaW_stream_narrow_y(stream, a, lds, ni);
     constexpr auto kern = delta_w_stream_kernel<6>;
     if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(a.wgs), dim3(512), lds, stream, static_cast<const DwStreamArgs &>(a));

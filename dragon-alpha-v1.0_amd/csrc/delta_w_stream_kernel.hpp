@@ -58,7 +58,30 @@ __host__ __device__ inline int dws_share_of(long P, long L, int G)
     return (int)(((P + 1) * G - 1) / L);
 }
 
-template <int D, bool FLAT = false, class Args = DwStreamArgs>
+// A lane's NI (NJ) consecutive channels of deltaY (X) as the low components of a float4: one 128-, 96-, 64- or 32-bit load.
+template <int N>
+static __device__ __forceinline__ floatx4 dws_load(__amdgpu_buffer_rsrc_t rsrc, unsigned voffset)
+{
+    if constexpr (N == 4) {
+        return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voffset, 0, 0));
+    } else if constexpr (N == 3) {
+        // (the builtin's result converted as a whole: indexing it directly compiles to a load of the first word only)
+        typedef float floatx3 __attribute__((ext_vector_type(3)));
+        const floatx3 v = __builtin_bit_cast(floatx3, __builtin_amdgcn_raw_buffer_load_b96(rsrc, voffset, 0, 0));
+        return floatx4{v[0], v[1], v[2], 0.f};
+    } else if constexpr (N == 2) {
+        typedef float floatx2 __attribute__((ext_vector_type(2)));
+        const floatx2 v = __builtin_bit_cast(floatx2, __builtin_amdgcn_raw_buffer_load_b64(rsrc, voffset, 0, 0));
+        return floatx4{v[0], v[1], 0.f, 0.f};
+    } else {
+        return floatx4{__builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voffset, 0, 0)), 0.f, 0.f, 0.f};
+    }
+}
+
+// NI, NJ: output (input) channels per lane, 1 to 4: a block of the filter is 16 NI output x 16 NJ input channels, and a
+// group of four pixels costs NI x NJ MFMAs. 4 x 4 = the 64 x 64 blocks; 96 input channels are two blocks of 48 with NJ = 3
+// (12 MFMAs a group on full blocks instead of 16 on one full and one half-empty block).
+template <int D, bool FLAT = false, class Args = DwStreamArgs, int NI = 4, int NJ = 4>
 __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
 {
     extern __shared__ __attribute__((aligned(16))) float dws_smem[];   // [8 wavefronts][16 units][64 lanes] float4
@@ -110,7 +133,7 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
         const int blk = fdiv(item, p.d_taps), tap = item - blk * p.taps;
         const int icb = fdiv(blk, p.d_ocb), ocb = blk - icb * p.ocb_count;
         const int fh = fdiv(tap, p.d_FW), fw = tap - fh * p.FW;
-        const int oc_l = 64 * ocb + 4 * l16, ic_l = 64 * icb + 4 * l16;
+        const int oc_l = 16 * NI * ocb + NI * l16, ic_l = 16 * NJ * icb + NJ * l16;
         const unsigned y_lane = oc_l < p.OC ? (unsigned)((q * p.OC + oc_l) * 4) : NEVER;
         const unsigned x_lane = ic_l < p.IC ? (unsigned)(((q * p.sw + fw - p.pw) * p.IC + ic_l) * 4) : NEVER;   // may be "negative"
 
@@ -120,11 +143,11 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
         const int g_hi = __builtin_amdgcn_readfirstlane(ga + (int)((long)n_g * (w + 1) / 8));
         const int total = g_hi - g_lo;
 
-        floatx4 acc[4][4];
+        floatx4 acc[NI][NJ];
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < NI; i++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+            for (int j = 0; j < NJ; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
         // ---- load cursor: the row being requested (all scalar), its descriptors, the group within it -----------------------
         //      (FLAT: the image being requested, its descriptors, the group within it; per lane the pixel's column and
@@ -178,8 +201,8 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
         auto load = [&](int d) {
             if (FLAT) {
                 const bool col_ok = ic_l < p.IC && (unsigned)(ow_l * p.sw + fw - p.pw) < (unsigned)p.IW;
-                ya[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, y_lane + (unsigned)y_goff, 0, 0));
-                xa[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, col_ok ? x_off : 0x80000000u, 0, 0));
+                ya[d] = dws_load<NI>(y_rsrc, y_lane + (unsigned)y_goff);
+                xa[d] = dws_load<NJ>(x_rsrc, col_ok ? x_off : 0x80000000u);
                 cur_g++;
                 left--;
                 y_goff += y_gstride;
@@ -197,8 +220,8 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
                 }
                 return;
             }
-            ya[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(y_rsrc, y_lane + (unsigned)y_goff, 0, 0));
-            xa[d] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_lane + (unsigned)x_goff, 0, 0));
+            ya[d] = dws_load<NI>(y_rsrc, y_lane + (unsigned)y_goff);
+            xa[d] = dws_load<NJ>(x_rsrc, x_lane + (unsigned)x_goff);
             // on to the next group; the next row when this one is done (scalar work only: no memory operation in a branch)
             cur_g++;
             left--;
@@ -217,9 +240,9 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
         };
         auto multiply = [&](int d) {
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int i = 0; i < NI; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++)
+                for (int j = 0; j < NJ; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ya[d][i], xa[d][j], acc[i][j], 0, 0, 0);
         };
         if (total > 0) {
@@ -246,35 +269,87 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
         }
 
         // ---- the eight parts added in the order 0, 1, 2, ...; unit u = 4 i + rr is one 128-bit store per lane:
-        // acc[i][j][rr] = deltaW[oc = 64 ocb + 4 (4q + rr) + i][tap][ic = 64 icb + 4 l16 + j] --------------------------------
+        // acc[i][j][rr] = deltaW[oc = 16 NI ocb + NI (4q + rr) + i][tap][ic = 16 NJ icb + NJ l16 + j] ---------------------------
+        if constexpr (NI == 4 && NJ == 4) {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+            for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int rr = 0; rr < 4; rr++)
-                part[(w * 16 + 4 * i + rr) * 64 + lane] = floatx4{acc[i][0][rr], acc[i][1][rr], acc[i][2][rr], acc[i][3][rr]};
-        __syncthreads();
-        float *dst = ord == 0 ? p.dW : p.dW_buf + (size_t)(ord - 1) * sizeW;
+                for (int rr = 0; rr < 4; rr++)
+                    part[(w * 16 + 4 * i + rr) * 64 + lane] = floatx4{acc[i][0][rr], acc[i][1][rr], acc[i][2][rr], acc[i][3][rr]};
+            __syncthreads();
+            float *dst = ord == 0 ? p.dW : p.dW_buf + (size_t)(ord - 1) * sizeW;
 #pragma unroll
-        for (int k = 0; k < 2; k++) {
-            const int u = w + 8 * k, i = u >> 2, rr = u & 3;
-            floatx4 v = part[u * 64 + lane];
+            for (int k = 0; k < 2; k++) {
+                const int u = w + 8 * k, i = u >> 2, rr = u & 3;
+                floatx4 v = part[u * 64 + lane];
 #pragma unroll
-            for (int x = 1; x < 8; x++) v += part[(x * 16 + u) * 64 + lane];
-            const int oc = ocb * 64 + 4 * (4 * q + rr) + i;
-            if (ic_l < p.IC && oc < p.OC)
-                *reinterpret_cast<float4 *>(dst + ((size_t)oc * p.taps + tap) * p.IC + ic_l) = make_float4(v[0], v[1], v[2], v[3]);
-        }
-        // ---- zeros into the buffers none of the item's pieces writes: piece `ord` of `npieces` takes every npieces-th ----------
-        for (int z = npieces + ord; z < p.GZ; z += npieces) {
-            float *zd = p.dW_buf + (size_t)(z - 1) * sizeW;   // z >= npieces >= 1
-            for (int e = t; e < 64 * 16; e += 512) {            // 64 output channels x 16 float4 of input channels
-                const int oc = ocb * 64 + (e >> 4), ic = icb * 64 + 4 * (e & 15);
-                if (oc < p.OC && ic < p.IC)
-                    *reinterpret_cast<float4 *>(zd + ((size_t)oc * p.taps + tap) * p.IC + ic) = make_float4(0.f, 0.f, 0.f, 0.f);
+                for (int x = 1; x < 8; x++) v += part[(x * 16 + u) * 64 + lane];
+                const int oc = ocb * 64 + 4 * (4 * q + rr) + i;
+                if (ic_l < p.IC && oc < p.OC)
+                    *reinterpret_cast<float4 *>(dst + ((size_t)oc * p.taps + tap) * p.IC + ic_l) = make_float4(v[0], v[1], v[2], v[3]);
+            }
+            // ---- zeros into the buffers none of the item's pieces writes: piece `ord` of `npieces` takes every npieces-th ------
+            for (int z = npieces + ord; z < p.GZ; z += npieces) {
+                float *zd = p.dW_buf + (size_t)(z - 1) * sizeW;   // z >= npieces >= 1
+                for (int e = t; e < 64 * 16; e += 512) {            // 64 output channels x 16 float4 of input channels
+                    const int oc = ocb * 64 + (e >> 4), ic = icb * 64 + 4 * (e & 15);
+                    if (oc < p.OC && ic < p.IC)
+                        *reinterpret_cast<float4 *>(zd + ((size_t)oc * p.taps + tap) * p.IC + ic) = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NI; i++)
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++) {
+                    floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int j = 0; j < NJ; j++) v[j] = acc[i][j][rr];
+                    part[(w * 16 + 4 * i + rr) * 64 + lane] = v;
+                }
+            __syncthreads();
+            float *dst = ord == 0 ? p.dW : p.dW_buf + (size_t)(ord - 1) * sizeW;
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const int u = w + 8 * k, i = u >> 2, rr = u & 3;
+                if (u < 4 * NI) {   // uniform
+                    floatx4 v = part[u * 64 + lane];
+#pragma unroll
+                    for (int x = 1; x < 8; x++) v += part[(x * 16 + u) * 64 + lane];
+                    const int oc = ocb * 16 * NI + NI * (4 * q + rr) + i;
+                    if (ic_l < p.IC && oc < p.OC) {
+                        float *o = dst + ((size_t)oc * p.taps + tap) * p.IC + ic_l;
+#pragma unroll
+                        for (int j = 0; j < NJ; j++) o[j] = v[j];
+                    }
+                }
+            }
+            for (int z = npieces + ord; z < p.GZ; z += npieces) {
+                float *zd = p.dW_buf + (size_t)(z - 1) * sizeW;
+                for (int e = t; e < 16 * NI * 4 * NJ; e += 512) {   // 16 NI output channels x 4 NJ float4 of input channels
+                    const int oc = ocb * 16 * NI + e / (4 * NJ), ic = icb * 16 * NJ + 4 * (e % (4 * NJ));
+                    if (oc < p.OC && ic < p.IC)
+                        *reinterpret_cast<float4 *>(zd + ((size_t)oc * p.taps + tap) * p.IC + ic) = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
             }
         }
         __syncthreads();   // the next piece writes `part` again
     }
 }
+
+// Launch of the kernel with NI x NJ channels per lane (groups by row).
+template <int NI, int NJ>
+static hipError_t dws_launch(hipStream_t stream, const DwStreamArgs &a, size_t lds)
+{
+    constexpr auto kern = delta_w_stream_kernel<6, false, DwStreamArgs, NI, NJ>;
+    if (hipError_t e = ensure_dynamic_lds<kern>(lds); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(a.wgs), dim3(512), lds, stream, a);
+    return hipGetLastError();
+}
+
+// delta_w_stream_narrow_*.hip: the kernels with fewer than 4 x 4 channels per lane, NI (NJ) output (input) channels
+hipError_t launch_deltaW_stream_narrow_x(hipStream_t stream, const DwStreamArgs &a, size_t lds, int NJ);            // NI = 4
+hipError_t launch_deltaW_stream_narrow_y(hipStream_t stream, const DwStreamArgs &a, size_t lds, int NI);            // NJ = 4
+hipError_t launch_deltaW_stream_narrow_xy(hipStream_t stream, const DwStreamArgs &a, size_t lds, int NI, int NJ);   // both below 4
 
 }  // namespace alpha

@@ -135,11 +135,13 @@ def test_deltaW_least_option_sets_the_split_k_factor_the_persistent_kernel_needs
     assert E.plan_deltaW(cfg, 32, 32, 32, 32, 3, 3, 512, 4, 64, 1, 1).GridZ == 256      # 9 taps, 64 channels: a workgroup per slice
     assert E.plan_deltaW(cfg, 224, 224, 112, 112, 7, 7, 64, 4, 64, 2, 2).GridZ == 128   # 49 taps: four groups, 64 slices would do
     assert E.plan_deltaW(cfg, 32, 32, 32, 32, 3, 3, 4, 4, 64, 1, 1).GridZ == 16         # c1: GK / 256 = 16 caps it
-    # channel counts that fill the 64 x 64 blocks to less than 75 % go to other kernels: unchanged
+    # channel counts that fill the kernel's blocks (16 x 1 to 4 channels per lane a side) to less than 40 % go to other
+    # kernels: unchanged (8 of 16 and 12 of 16: 37.5 %); 36 x 44 channels are 36 of 48 and 44 of 64 (52 %): lowered
     cfg0 = E.default_config(256)
     for shape in [(28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1), (14, 14, 14, 14, 3, 3, 64, 1024, 1024, 1, 1)]:
         assert E.plan_deltaW(cfg, *shape).GridZ <= E.plan_deltaW(cfg0, *shape).GridZ
-    assert E.plan_deltaW(cfg, 28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1).GridZ == E.plan_deltaW(cfg0, 28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1).GridZ
+    assert E.plan_deltaW(cfg, 28, 28, 28, 28, 3, 3, 32, 8, 12, 1, 1).GridZ == E.plan_deltaW(cfg0, 28, 28, 28, 28, 3, 3, 32, 8, 12, 1, 1).GridZ
+    assert E.plan_deltaW(cfg, 28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1).GridZ == 28 < E.plan_deltaW(cfg0, 28, 28, 28, 28, 3, 3, 32, 36, 44, 1, 1).GridZ
     # the same arithmetic behind the C ABI, for a caller that chooses GridZ itself (units, GridZ, OH, OW, FH, FW, N, IC, OC)
     L = pkg.lib()
     assert L.alpha_dconv3D_deltaW_least_GridZ(256, 128, 56, 56, 3, 3, 32, 64, 64) == 28

@@ -867,6 +867,31 @@ def test_deltaW_persistent_kernel_sum_and_reproducibility(dev, shape):
         L.alpha_conv_set_fwd_algo(0)
 
 
+@pytest.mark.parametrize("IC,OC", [(16, 64), (32, 64), (48, 128), (64, 16), (64, 32), (128, 48), (16, 16), (16, 32), (32, 16), (32, 32),
+                                   (48, 16), (16, 48), (48, 32), (32, 48), (48, 48), (96, 96), (36, 44), (144, 96), (20, 208)])
+@pytest.mark.parametrize("geom", [(16, 12, 12, 3, 3, 1, 1, 1, 1, 8), (12, 15, 13, 5, 5, 2, 2, 2, 2, 5)])
+def test_deltaW_persistent_kernel_channels_per_lane(dev, IC, OC, geom):
+    """Channel counts that the persistent backward-filter kernel holds in blocks of 16 x (1, 2 or 3) channels per lane on
+    either side (16, 32, 48, 96 = 2 x 48, 144 = 3 x 48; 36 of 48; 20 = 20 of 32; 44 and 208 stay at 4 per lane): every
+    pair of per-lane counts, the sum of deltaW and the buffers against the oracle, bit-identical from run to run."""
+    N, IH, IW, FH, FW, sh, sw, ph, pw, GridZ = geom
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    X, dY = normal((N, IH, IW, IC), 3601), normal((N, OH, OW, OC), 3602)
+    want = O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw)
+    x, dy = dev.put(X), dev.put(dY)
+    sizeW = OC * FH * FW * IC
+    runs = []
+    for _ in range(2):
+        dWo = dev.guarded(OC, FH, FW, IC)
+        buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+        DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
+                                 FH, FW, N, IC, OC, sh, sw, ph, pw)
+        runs.append(np.concatenate([dev.get(dWo).reshape(1, -1), dev.get(buf)]))
+        assert np.isfinite(runs[-1]).all(), "an element of deltaW or of a buffer was not written (%d, %d) %s" % (IC, OC, geom)
+        check(_sum_partials(dev, dWo, buf, GridZ), want, "dW %d -> %d channels %s" % (IC, OC, geom))
+    assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32)), "partial sums differ between two runs (%d, %d) %s" % (IC, OC, geom)
+
+
 DW_STEM_SHAPES = [
     # N, IH, IW, OC, FH, FW, sh, sw, ph, pw, GridZ: 4 stored input channels (all four carry data here), the kernel whose MFMA
     # columns are 16 taps; its own equal cut of the pixels into GridZ slices, so the sum is compared
