@@ -48,6 +48,32 @@ static __device__ __forceinline__ void buffer_store_b128_guarded(floatx4 v, __am
     asm volatile("s_nop 1" : "+v"(v));
 }
 
+// The same for the N low components of `v` (N = 1 to 4): a 32-, 64-, 96- or 128-bit store, with the wait states of the
+// 128-bit one (the hazard was measured on the 128-bit store; the narrower ones with a scalar soffset are guarded alike).
+template <int N, int AUX = 0>
+static __device__ __forceinline__ void buffer_store_guarded(floatx4 v, __amdgpu_buffer_rsrc_t rsrc, unsigned voffset, int soffset)
+{
+    if constexpr (N == 4) {
+        buffer_store_b128_guarded<AUX>(v, rsrc, voffset, soffset);
+    } else if constexpr (N == 3) {
+        typedef float floatx3 __attribute__((ext_vector_type(3)));
+        typedef unsigned uintx3 __attribute__((ext_vector_type(3)));
+        floatx3 d = floatx3{v[0], v[1], v[2]};
+        __builtin_amdgcn_raw_buffer_store_b96(__builtin_bit_cast(uintx3, d), rsrc, voffset, soffset, AUX);
+        asm volatile("s_nop 1" : "+v"(d));
+    } else if constexpr (N == 2) {
+        typedef float floatx2 __attribute__((ext_vector_type(2)));
+        typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+        floatx2 d = floatx2{v[0], v[1]};
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uintx2, d), rsrc, voffset, soffset, AUX);
+        asm volatile("s_nop 1" : "+v"(d));
+    } else {
+        float d = v[0];
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, d), rsrc, voffset, soffset, AUX);
+        asm volatile("s_nop 1" : "+v"(d));
+    }
+}
+
 // Workgroup barrier that orders LDS accesses only: __syncthreads() also waits for every global load and store of the
 // wavefront (its fences cover all address spaces), which stalls a kernel that keeps loads for later in flight.
 static __device__ __forceinline__ void lds_barrier()

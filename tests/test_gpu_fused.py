@@ -65,6 +65,10 @@ FUSED_SHAPES = [
     (4, 30, 30, 4, 64, 7, 7, 2, 2, 3, 3, "stem kernel"),
     (4, 14, 14, 64, 128, 1, 1, 1, 1, 0, 0, "1x1 streaming kernel + a separate pass"),
     (4, 9, 11, 12, 20, 5, 4, 2, 3, 2, 1, "generic kernel"),
+    (4, 12, 12, 64, 96, 3, 3, 2, 2, 1, 1, "the kernel without LDS, two blocks of 48 output channels (3 per lane)"),
+    (4, 12, 12, 32, 32, 3, 3, 2, 2, 1, 1, "the same, 2 per lane"),
+    (4, 12, 12, 32, 16, 5, 5, 1, 1, 2, 2, "the same, 1 per lane"),
+    (4, 10, 10, 48, 36, 3, 3, 1, 1, 1, 1, "the same, 36 of a block of 48"),
 ]
 
 
@@ -121,6 +125,10 @@ DX_SHAPES = [
     (4, 13, 11, 36, 44, 3, 1),      # generic kernel (ragged channels)
     (4, 12, 12, 64, 96, 5, 2),      # LDS-halo kernel
     (4, 14, 14, 128, 64, 1, 0),     # 1x1 streaming kernel + a separate pass
+    (4, 12, 12, 96, 64, 3, 1),      # the kernel without LDS, two blocks of 48 produced channels (3 per lane)
+    (4, 12, 12, 32, 64, 5, 2),      # the same, 2 per lane
+    (4, 10, 10, 16, 32, 3, 1),      # the same, 1 per lane
+    (4, 10, 10, 36, 64, 3, 1),      # the same, 36 of a block of 48
 ]
 
 

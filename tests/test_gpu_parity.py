@@ -449,6 +449,15 @@ DIRECT_CONV_SHAPES = [
     (24, 14, 14, 80, 128, 5, 5, 1, 1, 2, 2),    # 125 steps; 588 items: 2 or 3 per workgroup, all shared (parts of 15 and 16 steps)
     (40, 20, 20, 16, 64, 3, 3, 1, 1, 1, 1),     # 9 steps; 1000 items: 3 or 4 per workgroup, the eighth part of 10 steps is 1 or 2
     (96, 24, 24, 16, 64, 1, 1, 1, 1, 0, 0),     # a single step per item (1x1, 16 channels)
+    # one to three produced channels per lane: blocks of 16, 32 or 48 produced channels instead of 64
+    (8, 20, 20, 32, 48, 3, 3, 1, 1, 1, 1),      # one block of 48
+    (8, 14, 14, 64, 144, 3, 3, 1, 1, 1, 1),     # three blocks of 48
+    (8, 20, 20, 64, 32, 3, 3, 2, 2, 1, 1),      # one block of 32, strided
+    (8, 17, 15, 32, 16, 5, 5, 1, 1, 2, 2),      # one block of 16, ragged last tile
+    (8, 14, 14, 48, 24, 3, 3, 1, 1, 1, 1),      # 24 of a block of 32 (12 lanes of 2), an odd number of steps
+    (8, 14, 14, 32, 20, 3, 3, 2, 2, 1, 1),      # 20 of a block of 32
+    (8, 14, 14, 32, 12, 1, 1, 1, 1, 0, 0),      # 12 of a block of 16, 1x1
+    (8, 14, 14, 32, 40, 3, 3, 1, 1, 1, 1),      # 40 = 3 per lane would split a lane's group at the end: four per lane
     (50, 14, 14, 48, 256, 3, 3, 1, 1, 1, 1),    # 27 steps, 2452 items: 9 or 10 per workgroup - a group of two tiles per SIMD, steps 14 + 14
 ]
 
