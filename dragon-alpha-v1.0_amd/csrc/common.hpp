@@ -314,6 +314,7 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
                                 int sh, int sw, int ph, int pw, int GZ);
 int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ);
 int deltaW_stream_block_fill(int IC, int OC);
+void deltaW_stream_set_units(int units);   // -1 by shape, 0 never, 1 wherever the buffers allow: whole units instead of the line of items
 int deltaW_stream_fill_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ, int GZ_cap);
 
 // Backward-filter with the filter tap in the grid and both operands straight from memory (delta_w_taps.hip): any filter,

@@ -565,6 +565,12 @@ int alpha_conv_set_kernel_split_sharing(int sharing)
     g_ks_sharing.store(sharing);
     return 0;
 }
+int alpha_conv_set_deltaW_units(int units)
+{
+    if (units < -1 || units > 1) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_deltaW_units: units must be -1, 0 or 1");
+    deltaW_stream_set_units(units);
+    return 0;
+}
 int alpha_conv_set_fwd_algo(int algo)
 {
     if (algo < 0 || algo > 6) return fail(ALPHA_CONV_EINVAL, "alpha_conv_set_fwd_algo: algo must be 0..6");

@@ -1,5 +1,7 @@
 // Launcher of the persistent backward-filter kernel (delta_w_stream_kernel.hpp) and the split-K factors it needs.
 #include "delta_w_stream_kernel.hpp"
+#include <atomic>
+#include <cstdlib>
 
 namespace alpha {
 
@@ -17,6 +19,68 @@ static int dws_max_pieces(long items, long TG, int G)
         if (n > most) most = n;
     }
     return most;
+}
+
+// Whether layers outside the first rule below are cut into whole units (pieces x items): -1 by shape, 0 never, 1 wherever
+// the buffers allow it. A debugging switch (deltaW_stream_set_units, or ALPHA_DW_UNITS=0/1 in the environment, read once
+// per process): the parity tests run both cuts on small shapes.
+static std::atomic<int> g_dws_units{-2};
+
+static int dws_units_switch()
+{
+    int v = g_dws_units.load(std::memory_order_relaxed);
+    if (v == -2) {
+        const char *e = getenv("ALPHA_DW_UNITS");
+        v = e ? (atoi(e) != 0 ? 1 : 0) : -1;
+        int expected = -2;
+        if (!g_dws_units.compare_exchange_strong(expected, v)) v = expected;   // a setter was quicker
+    }
+    return v;
+}
+
+void deltaW_stream_set_units(int units) { g_dws_units.store(units < 0 ? -1 : units != 0); }
+
+// How the kernel cuts a layer of `items` items of TG pixel groups on G workgroups with GZ - 1 buffers:
+//   pieces > 0, units: every item in `pieces` equal pieces, the pieces x items units dealt out whole, piece-major;
+//   pieces > 0, !units: the line of items in G equal shares, of which an item meets at most `pieces`;
+//   pieces == 0: the kernel does not take the layer.
+struct DwsCut {
+    int pieces;
+    bool units;
+};
+
+static DwsCut dws_cut(long items, long TG, int G, int GZ, long bytes)
+{
+    // at least eight pixel groups per workgroup (one per wavefront); smaller layers go to the kernels with one workgroup per slice
+    if (items * TG < 8L * G || items > 4096 || GZ < 2) return {0, false};
+    // (1) R x items workgroups are (nearly) all of them: one unit each
+    long R = G / items;
+    if (R > GZ) R = GZ;
+    if (R >= 1 && 20 * R * items >= 19L * G) return {(int)R, true};
+    const int most = dws_max_pieces(items, TG, G);
+    // (2) Tensors well beyond the L2s (56 MB: measured between 50 and 65) whose shares of the line start at 32 or more
+    // different places of the pixel range (G / gcd(items, G): 27, 72, 200 items on 256 workgroups; with 144 items pairs
+    // of shares run over the same pixels, with 576 eight at a time, and the line stays the faster cut): every workgroup
+    // then streams pixels of its own and the L2s serve nobody twice (5x5 96 -> 256 on 64x27x27: 1.8 GB fetched for 65 MB
+    // of tensors). Whole units instead, ceil(P items / G) per workgroup: the workgroups of an XCD go through the same
+    // piece of the pixels at the same time, each for an item of its own. P minimises the modelled time, a unit's
+    // end (partial sums through LDS, stores, the loads of the next from cold) counted as 64 pixel groups.
+    const int sw = dws_units_switch();
+    long g = items, h = G;
+    while (h) { const long r = g % h; g = h; h = r; }
+    const long line = (items * TG + G - 1) / G + 128;
+    long best = 0;
+    int best_P = 0;
+    for (int P = 1; P <= GZ && 8L * P <= TG; P++) {
+        const long t = (P * items + G - 1) / G * ((TG + P - 1) / P + 64);
+        if (best_P == 0 || t < best) best = t, best_P = P;
+    }
+    if (best_P > 0 && (sw == 1 || (sw < 0 && bytes > (56L << 20) && g * 32 <= G && 100 * best <= 108 * line))) return {best_P, true};
+    // (3) the line of items; with fewer buffers than the shares an item would meet (the Java engine passes GridZ = 2 for
+    // 4x4 maps at N = 512, where 72 items on 256 workgroups meet up to 5 shares each) whole units all the same, some
+    // workgroups idle - still several times faster than the kernels with one workgroup per slice (3x3 96 -> 208 there: 0.463 ms)
+    if (most > GZ) return best_P > 0 ? DwsCut{best_P, true} : DwsCut{0, false};
+    return {most, false};
 }
 
 // Pixel groups as four consecutive pixels of an image (row-major) instead of an output row: where a row's groups are
@@ -42,42 +106,41 @@ int deltaW_stream_block_fill(int IC, int OC)
     return (int)(100L * IC * OC / (ib * ob));
 }
 
-// The least split-K factor <= GZ with which launch_deltaW_stream on a device of `units` compute units cuts the layer
-// exactly as it does with GZ (the same R pieces per item, or the same line of shares), or GZ itself where the kernel
-// does not take the layer or the split-K entries may not choose it (channel counts that fill 64 x 64 blocks to less than
-// 40 %). With it the kernel has no buffers to fill with zeros and the caller's buf_summary none to add for nothing.
-int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ)
+// The cut of a layer as the split-K helpers below know it (no input size, no stride): `bytes` is counted on the output's
+// pixels for both tensors, here and in the launcher.
+static DwsCut dws_cut_of_layer(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ)
 {
-    if ((IC & 3) || (OC & 3) || IC < 4 || OC < 4 || FH < 1 || FW < 1 || GZ < 2 || units < 1 || N < 1 || OH < 1 || OW < 1) return GZ;
+    if ((IC & 3) || (OC & 3) || IC < 4 || OC < 4 || FH < 1 || FW < 1 || GZ < 2 || units < 1 || N < 1 || OH < 1 || OW < 1) return {0, false};
+    // the stricter of the split-K entries' two thresholds (the stride is not known here)
+    if (deltaW_stream_block_fill(IC, OC) < 40) return {0, false};
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
-    if (deltaW_stream_block_fill(IC, OC) < 40) return GZ;   // the stricter of the split-K entries' two thresholds (the stride is not known here)
     // (the input's size is not known here: the launcher's other condition for groups by image, an image of X below 512 MB)
     const bool flat = dws_flat_rows(OH, OW, OC);
     const long items = icb * ocb * FH * FW, TG = flat ? (long)N * (((long)OH * OW + 3) / 4) : (long)N * OH * ((OW + 3) / 4);
-    if (items >= (1L << 20) || TG >= (1L << 30) || items * TG < 8L * units || items > 4096) return GZ;
-    long R = units / items;
-    if (R > GZ) R = GZ;
-    if (R >= 1 && 20 * R * items >= 19L * units) return R < 2 ? 2 : (int)R;
-    const int most = dws_max_pieces(items, TG, units);
-    if (most > GZ) return R >= 1 ? (R < 2 ? 2 : (int)R) : GZ;   // R pieces per item on fewer workgroups (see the launcher)
-    return most < 2 ? 2 : most;
+    if (items >= (1L << 20) || TG >= (1L << 30)) return {0, false};
+    return dws_cut(items, TG, units, GZ, (long)N * OH * OW * ((long)IC + OC) * 4);
 }
 
-// The split-K factor a host layer that owns GridZ should pass: deltaW_stream_least_GridZ where GZ is enough for the kernel's
-// own cut, and where it is not (the reference sizes GridZ for the slices of its kernels: 2 on 4x4 maps at N = 512, where 72
-// items on 256 compute units meet up to 5 shares each) the pieces per item that cut wants, up to GZ_cap.
+// The least split-K factor <= GZ with which launch_deltaW_stream on a device of `units` compute units cuts the layer
+// exactly as it does with GZ (the same pieces per item, or the same line of shares), or GZ itself where the kernel
+// does not take the layer or the split-K entries may not choose it (channel counts that fill their blocks to less than
+// 40 %). With it the kernel has no buffers to fill with zeros and the caller's buf_summary none to add for nothing.
+int deltaW_stream_least_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ)
+{
+    const DwsCut c = dws_cut_of_layer(units, N, OH, OW, IC, OC, FH, FW, GZ);
+    if (c.pieces == 0) return GZ;
+    return c.pieces < 2 ? 2 : c.pieces;
+}
+
+// The split-K factor a host layer that owns GridZ should pass: deltaW_stream_least_GridZ where GZ is enough for the cut
+// the kernel would make with GZ_cap buffers, and where it is not (the reference sizes GridZ for the slices of its
+// kernels: 2 on 4x4 maps at N = 512, where 72 items on 256 compute units meet up to 5 shares each) the factor that cut needs.
 int deltaW_stream_fill_GridZ(int units, int N, int OH, int OW, int IC, int OC, int FH, int FW, int GZ, int GZ_cap)
 {
     const int least = deltaW_stream_least_GridZ(units, N, OH, OW, IC, OC, FH, FW, GZ);
-    if (least != GZ || GZ < 2 || GZ_cap <= GZ || (IC & 3) || (OC & 3) || IC < 4 || OC < 4 || FH < 1 || FW < 1 || units < 1 || N < 1 || OH < 1 || OW < 1) return least;
-    const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
-    if (deltaW_stream_block_fill(IC, OC) < 40) return least;
-    const bool flat = dws_flat_rows(OH, OW, OC);
-    const long items = icb * ocb * FH * FW, TG = flat ? (long)N * (((long)OH * OW + 3) / 4) : (long)N * OH * ((OW + 3) / 4);
-    if (items >= (1L << 20) || TG >= (1L << 30) || items * TG < 8L * units || items > 4096) return least;
-    const long R = units / items;
-    const long want = (R >= 1 && 20 * R * items >= 19L * units) ? R : dws_max_pieces(items, TG, units);
-    return want > GZ && want <= GZ_cap ? (int)want : least;
+    if (GZ < 2 || GZ_cap <= GZ) return least;
+    const DwsCut c = dws_cut_of_layer(units, N, OH, OW, IC, OC, FH, FW, GZ_cap);
+    return c.pieces > GZ ? c.pieces : least;
 }
 
 // Returns hipErrorNotSupported (nothing launched) when the layer does not fit; the caller then uses another kernel.
@@ -116,24 +179,11 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
     a.TG = (int)TG;
     a.L = items * TG;
     a.wgs = cus;   // one workgroup of eight wavefronts per compute unit
-    // at least eight pixel groups per workgroup (one per wavefront); smaller layers go to the kernels with one workgroup per slice
-    if (a.L < 8L * a.wgs || items > 4096) return hipErrorNotSupported;
-    // Every item in R equal pieces where R * items workgroups are (nearly) all of them; else the line of items in equal
-    // shares. Either way the pieces of an item go to deltaW and the GridZ - 1 buffers.
-    long R = cus / items;
-    if (R > GZ) R = GZ;
-    if (R >= 1 && 20 * R * items >= 19L * cus) {
-        a.R = (int)R;
-    } else {
-        a.R = 0;
-        if (dws_max_pieces(items, TG, a.wgs) > GZ) {
-            // fewer items than workgroups and fewer buffers than the shares an item would meet (the Java engine passes
-            // GridZ = 2 for 4x4 maps at N = 512): R = GridZ pieces per item on R x items workgroups, the rest idle - still
-            // several times faster than the kernels with one workgroup per slice (3x3 96 -> 208 there: 0.463 ms)
-            if (R < 1) return hipErrorNotSupported;
-            a.R = (int)R;
-        }
-    }
+    // whole units (every item in R equal pieces) or the line of items in equal shares; either way the pieces of an item go
+    // to deltaW and the GridZ - 1 buffers
+    const DwsCut cut = dws_cut(items, TG, a.wgs, GZ, (long)N * OH * OW * ((long)IC + OC) * 4);
+    if (cut.pieces == 0) return hipErrorNotSupported;
+    a.R = cut.units ? cut.pieces : 0;
     a.d_OH = make_fastdiv(OH);
     a.d_OW = make_fastdiv(OW);
     a.d_FW = make_fastdiv(FW);

@@ -11,8 +11,9 @@
 // (tap, 64 x 64 block) with ALL its pixels, as groups of four pixels of an output row; the items one after the other form
 // a line, the line is cut into one equal share per workgroup, and the pieces of an item - it meets at most
 // workgroups / items + 2 shares - go to deltaW, deltaW_buf[0], deltaW_buf[1], ... in order; (item, buffer) pairs beyond an
-// item's pieces are filled with zeros. The partition is a function of the shape, GridZ and the device's compute units:
-// no atomics, bit-identical results from run to run.
+// item's pieces are filled with zeros. (Or every item is cut into R equal pieces and the R x items units are dealt out
+// whole: see the kernel.) The partition is a function of the shape, GridZ and the device's compute units: no atomics,
+// bit-identical results from run to run.
 //
 // Inside a piece the arithmetic is delta_w_taps.hip's: lane (l16, q) loads
 //   ya = deltaY[n, oh, 4g + q][oc0 + 4*l16 .. +3]      xa = X[n, ih, (4g + q)*sw + fw - pw][ic0 + 4*l16 .. +3]
@@ -41,7 +42,7 @@ struct DwStreamArgs {
     int TG;       // pixel groups per item = N * OH * GPR; flat: N * GPR
     long L;       // items * TG
     int wgs;
-    int R;        // > 0: every item is cut into R equal pieces, one workgroup each (see below); 0: the line of items
+    int R;        // > 0: every item is cut into R equal pieces, whole (piece, item) units per workgroup (see below); 0: the line of items
     FastDiv d_OH, d_FW, d_GPR, d_taps, d_ocb;
 };
 
@@ -93,18 +94,18 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
     // consecutive shares run on one XCD (workgroups are dealt round-robin to the 8 XCDs): the taps of a block, which read
     // the same rows, then share an L2
     const int s = (G & 7) == 0 ? (b & 7) * (G >> 3) + (b >> 3) : b;
-    long lo, hi;
+    // R > 0: every item is cut into R equal pieces and unit u = r * items + i is piece r of item i; the shares are whole units,
+    // [U s / G, U (s + 1) / G) of the U = R * items. The items' pieces over the same pixels are neighbours - the same XCD,
+    // or two -, start together and are equally long, so the rows one of them fetches are in L2 for the others. (In the
+    // line of items, R = 0, the shares of different items over the same pixels drift apart in time: with tensors beyond
+    // the caches every item then fetches its rows again - 9 x 51 MB on 56x56x64 at N = 32.)
+    long pos, hi;
     if (p.R > 0) {
-        // Piece r of item i is share r * items + i: the items' pieces over the same pixels are neighbours - the same XCD, or
-        // two -, start together and are equally long, so the rows one of them fetches are in L2 for the others. (In the
-        // line of items the shares of different items over the same pixels drift apart in time: with tensors beyond the
-        // caches every item then fetches its rows again - 9 x 51 MB on 56x56x64 at N = 32.)
-        if (s >= p.R * p.items) return;
-        const int r = s / p.items, i = s - r * p.items;
-        lo = (long)i * p.TG + (long)p.TG * r / p.R;
-        hi = (long)i * p.TG + (long)p.TG * (r + 1) / p.R;
+        const long U = (long)p.R * p.items;
+        pos = U * s / G;
+        hi = U * (s + 1) / G;
     } else {
-        lo = p.L * s / G;
+        pos = p.L * s / G;
         hi = p.L * (s + 1) / G;
     }
     const int OW = p.OW, OH = p.OH, GPR = p.GPR;
@@ -114,21 +115,25 @@ __global__ __launch_bounds__(512, 1) void delta_w_stream_kernel(const Args p)
     const size_t y_row_bytes = (size_t)OW * p.OC * 4, x_img_bytes = (size_t)p.IH * p.IW * p.IC * 4;
     const int x_row_bytes = p.IW * p.IC * 4;
 
-    long pos = lo;
     while (pos < hi) {   // uniform over the workgroup
-        const int item = (int)(pos / p.TG);
-        const long P0 = (long)item * p.TG;
-        const int ga = (int)(pos - P0), gb = (int)((hi < P0 + p.TG ? hi : P0 + p.TG) - P0);
-        int ord, npieces;
+        int item, ga, gb, ord, npieces;
         if (p.R > 0) {
-            ord = s / p.items;
+            ord = (int)pos / p.items;
+            item = (int)pos - ord * p.items;
             npieces = p.R;
+            ga = (int)((long)p.TG * ord / p.R);
+            gb = (int)((long)p.TG * (ord + 1) / p.R);
+            pos++;
         } else {
+            item = (int)(pos / p.TG);
+            const long P0 = (long)item * p.TG;
+            ga = (int)(pos - P0);
+            gb = (int)((hi < P0 + p.TG ? hi : P0 + p.TG) - P0);
             const int s_first = dws_share_of(P0, p.L, G), s_last = dws_share_of(P0 + p.TG - 1, p.L, G);
             ord = s - s_first;
             npieces = s_last - s_first + 1;
+            pos = P0 + gb;
         }
-        pos = P0 + gb;
 
         const int blk = fdiv(item, p.d_taps), tap = item - blk * p.taps;
         const int icb = fdiv(blk, p.d_ocb), ocb = blk - icb * p.ocb_count;

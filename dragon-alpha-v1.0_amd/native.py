@@ -103,7 +103,7 @@ def lib_path():
 def exported_symbols():
     """Names the C ABI must export (every function include/alpha_conv.h declares)."""
     return sorted(list(_SIGS) + ["alpha_conv_version", "alpha_conv_last_error", "alpha_conv_device_info", "alpha_conv_set_fwd_algo",
-                                 "alpha_conv_get_fwd_algo", "alpha_conv_set_pointwise_algo", "alpha_conv_set_kernel_split_sharing", "alpha_conv_bind_workspace", "alpha_conv_bind_tickets", "alpha_winograd_filter_size", "alpha_dconv3D_deltaW_least_GridZ"])
+                                 "alpha_conv_get_fwd_algo", "alpha_conv_set_pointwise_algo", "alpha_conv_set_kernel_split_sharing", "alpha_conv_set_deltaW_units", "alpha_conv_bind_workspace", "alpha_conv_bind_tickets", "alpha_winograd_filter_size", "alpha_dconv3D_deltaW_least_GridZ"])
 
 
 def _preload_hip_runtime():
@@ -145,6 +145,7 @@ def lib():
         L.alpha_conv_get_fwd_algo.restype = _I
         L.alpha_conv_set_pointwise_algo.argtypes = [_I]
         L.alpha_conv_set_kernel_split_sharing.argtypes = [_I]
+        L.alpha_conv_set_deltaW_units.argtypes = [_I]
         L.alpha_conv_bind_workspace.argtypes = [_P, ctypes.c_long]
         L.alpha_conv_bind_tickets.argtypes = [_P, ctypes.c_int]
         L.alpha_winograd_filter_size.argtypes = [_I, _I]

@@ -81,6 +81,12 @@ int alpha_conv_set_pointwise_algo(int algo);
  * every group of items, each taking an eighth of the reduction (what layers with few items per compute unit get by
  * shape). Also read once from the environment variable ALPHA_KS_SHARED = 0|1. No counterpart in the reference. */
 int alpha_conv_set_kernel_split_sharing(int sharing);
+/* And for backward-filter through the persistent kernel (delta_w_stream.hip), where its workgroups are not one piece of
+ * an item each: -1 = by shape, 0 = the line of items in equal shares, 1 = every item in equal pieces and the (piece, item)
+ * units dealt out whole, wherever GridZ allows (what large tensors with few items get by shape). The split-K helpers
+ * (alpha_dconv3D_deltaW_least_GridZ, the engine's options) follow the switch. Also read once from the environment
+ * variable ALPHA_DW_UNITS = 0|1. No counterpart in the reference. */
+int alpha_conv_set_deltaW_units(int units);
 
 /* ---- Cuda_conv3D: forward ------------------------------------------------------------------ */
 

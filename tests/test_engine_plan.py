@@ -153,6 +153,40 @@ def test_deltaW_least_option_sets_the_split_k_factor_the_persistent_kernel_needs
     assert E.plan_deltaW(cfg, 56, 56, 56, 56, 3, 3, 32, 64, 64, 1, 1).GridZ == 128
 
 
+def test_deltaW_whole_units_for_large_tensors_with_few_items():
+    """Tensors beyond 56 MB whose line of items would start its 256 shares at 32 or more different places of the pixel range
+    (256 / gcd(items, 256)) are cut into whole units instead - every item in P equal pieces, P minimising
+    ceil(P items / 256) x (ceil(groups / P) + 64) - and the helpers report P. (units, GridZ, OH, OW, FH, FW, N, IC, OC)"""
+    L = pkg.lib()
+    f = L.alpha_dconv3D_deltaW_least_GridZ
+    # AlexNet's second layer at N = 64: 200 items (two blocks of 48 x four of 64 x 25 taps) of 12096 groups, 65 MB:
+    # P = 5 -> 1000 units, 4 x (2420 + 64) = 9936 (P = 14: 11 x (864 + 64) = 10208; the line: 9450 + 128)
+    assert f(256, 14, 27, 27, 5, 5, 64, 96, 256) == 5
+    # 3x3 64 -> 192 on 512x16x16: 27 items, 134 MB: P = 9 (243 units, one each; P = 28 ties and the smaller wins)
+    assert f(256, 85, 16, 16, 3, 3, 512, 64, 192) == 9
+    assert f(256, 128, 56, 56, 3, 3, 64, 64, 192) == 28     # 206 MB, 50176 groups: 756 units, three each
+    assert f(256, 42, 32, 32, 3, 3, 64, 128, 256) == 7      # 72 items, 101 MB: 504 units, two each
+    # 144 items (pairs of shares over the same pixels), tensors of 46 MB, and either with the switch at "line": the line of items
+    assert f(256, 43, 56, 56, 3, 3, 32, 256, 256) == 3
+    assert f(256, 5, 8, 8, 5, 5, 512, 96, 256) == 3
+    try:
+        assert L.alpha_conv_set_deltaW_units(0) == 0
+        assert f(256, 14, 27, 27, 5, 5, 64, 96, 256) == 3
+        assert L.alpha_conv_set_deltaW_units(1) == 0
+        assert f(256, 43, 56, 56, 3, 3, 32, 256, 256) == 7
+    finally:
+        L.alpha_conv_set_deltaW_units(-1)
+    # what the reduced factor is, the launcher cuts the same way: the least factor of the least factor is itself
+    for args in [(14, 27, 27, 5, 5, 64, 96, 256), (128, 56, 56, 3, 3, 64, 64, 192), (42, 32, 32, 3, 3, 64, 128, 256), (43, 56, 56, 3, 3, 32, 256, 256)]:
+        g = f(256, *args)
+        assert f(256, g, *args[1:]) == g
+    # the engine's option lowers (or, within GK / 256, raises) GridZ to it
+    cfg = E.default_config(256)
+    cfg.deltaW_SK_leastUnits = 256
+    assert E.plan_deltaW(cfg, 27, 27, 27, 27, 5, 5, 64, 96, 256, 1, 1).GridZ == 5
+    assert E.plan_deltaW(cfg, 32, 32, 32, 32, 3, 3, 64, 128, 256, 1, 1).GridZ == 7
+
+
 def test_deltaX_plans():
     cfg = E.default_config(256)
     assert E.plan_deltaX(cfg, 224, 224, 112, 112, 7, 7, 64, 4, 64, 2, 2).entry_name == "dconv3D_deltaX_crossAdd"   # IC <= 8

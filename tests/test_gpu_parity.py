@@ -901,6 +901,44 @@ def test_deltaW_persistent_kernel_channels_per_lane(dev, IC, OC, geom):
     assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32)), "partial sums differ between two runs (%d, %d) %s" % (IC, OC, geom)
 
 
+DW_UNITS_SHAPES = [
+    # N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw, GridZ: the persistent kernel's other cut - every item in P equal pieces, the
+    # P x items units dealt out whole - forced on small layers (by shape only tensors beyond 56 MB get it)
+    (16, 16, 16, 256, 512, 3, 3, 1, 1, 1, 1, 8),    # 288 items of 1024 groups on 256 workgroups: P = 4, 4 or 5 units per workgroup
+    (32, 16, 16, 96, 128, 5, 5, 1, 1, 2, 2, 6),     # 100 items (blocks of 48 x 64): P = 5, 1 or 2 units per workgroup
+    (512, 2, 2, 256, 512, 3, 3, 1, 1, 1, 1, 4),     # pixel groups by image, 288 items of 512 groups: P = 2, 2 or 3 units
+    (24, 19, 13, 64, 192, 3, 3, 2, 2, 1, 1, 12),    # 27 items, rows of 7 pixels: P = 9, 243 units on 256 workgroups (13 idle, spread out)
+    (8, 12, 12, 64, 64, 3, 3, 1, 1, 1, 1, 3),       # 9 items, 3 buffers: 27 units
+]
+
+
+@pytest.mark.parametrize("shape", DW_UNITS_SHAPES)
+def test_deltaW_persistent_kernel_whole_units_against_the_line_of_items(dev, shape):
+    N, IH, IW, IC, OC, FH, FW, sh, sw, ph, pw, GridZ = shape
+    OH, OW = out_dim(IH, IW, FH, FW, sh, sw, ph, pw)
+    X, dY = normal((N, IH, IW, IC), 3701), normal((N, OH, OW, OC), 3702)
+    want = O.deltaW_f64(X, dY, FH, FW, sh, sw, ph, pw)
+    x, dy = dev.put(X), dev.put(dY)
+    sizeW = OC * FH * FW * IC
+    L = pkg.lib()
+    try:
+        for units in (1, 0, -1):
+            assert L.alpha_conv_set_deltaW_units(units) == 0
+            runs = []
+            for _ in range(2):
+                dWo = dev.guarded(OC, FH, FW, IC)
+                buf = dev.empty(GridZ - 1, sizeW, fill=float("nan"))
+                DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dWo.data_ptr(), buf.data_ptr(),
+                                         FH, FW, N, IC, OC, sh, sw, ph, pw)
+                runs.append(np.concatenate([dev.get(dWo).reshape(1, -1), dev.get(buf)]))
+                assert np.isfinite(runs[-1]).all(), "an element of deltaW or of a buffer was not written, units %d %s" % (units, shape)
+                check(_sum_partials(dev, dWo, buf, GridZ), want, "dW units %d %s" % (units, shape))
+            assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32)), "partial sums differ between two runs, units %d %s" % (units, shape)
+    finally:
+        L.alpha_conv_set_deltaW_units(-1)
+    assert L.alpha_conv_set_deltaW_units(2) != 0
+
+
 DW_STEM_SHAPES = [
     # N, IH, IW, OC, FH, FW, sh, sw, ph, pw, GridZ: 4 stored input channels (all four carry data here), the kernel whose MFMA
     # columns are 16 taps; its own equal cut of the pixels into GridZ slices, so the sum is compared
