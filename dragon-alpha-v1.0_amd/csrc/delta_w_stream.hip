@@ -84,12 +84,12 @@ static DwsCut dws_cut(long items, long TG, int G, int GZ, long bytes)
 }
 
 // Pixel groups as four consecutive pixels of an image (row-major) instead of an output row: where a row's groups are
-// empty to a quarter or more (rows of 1, 2, 3, 5, 6 or 9 pixels). Images beyond 512 MB do not fit the 32-bit offsets
+// empty to three sixteenths or more (rows of 1, 2, 3, 5, 6, 9 or 13 pixels). Images beyond 512 MB do not fit the 32-bit offsets
 // within an image.
 static bool dws_flat_rows(int OH, int OW, int OC)
 {
     const int slots = (OW + 3) / 4 * 4;
-    return 4 * (slots - OW) >= slots && (long)OH * OW * OC * 4 < (1L << 29);
+    return 16 * (slots - OW) >= 3 * slots && (long)OH * OW * OC * 4 < (1L << 29);
 }
 
 static int dws_per_lane(int C)

@@ -23,8 +23,8 @@
 // FLAT: short output rows leave most of a row's last group empty - half of every group on 2x2 maps, three of eight pixels
 // on rows of 5. There a group is four consecutive pixels of the IMAGE (row-major), the descriptors cover an image, vertical
 // padding falls outside them, and every lane keeps its pixel's column and offset in X (a few vector instructions per
-// group) for the horizontal padding. That bookkeeping costs 5-13 % of the kernel's time, so rows that waste less than a
-// quarter of their groups' pixels (7, 13, 14 pixels: an eighth to a fifth) keep the groups by row.
+// group) for the horizontal padding. That bookkeeping costs 5-13 % of the kernel's time, so rows that waste less than
+// three sixteenths of their groups' pixels (7, 14 pixels: an eighth) keep the groups by row.
 #pragma once
 #include "common.hpp"
 

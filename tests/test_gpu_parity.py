@@ -839,6 +839,7 @@ DW_STREAM_SHAPES = [
     (48, 6, 6, 64, 128, 3, 3, 2, 2, 1, 1, 16, 14),      # stride 2 onto 3x3 maps: a row and a column on per group
     (16, 9, 9, 64, 64, 5, 5, 1, 1, 2, 2, 12, 10),       # rows of 9, 5x5 filter
     (2048, 1, 1, 128, 64, 1, 1, 1, 1, 0, 0, 128, 128),  # 1x1 maps: one pixel per group (a fully connected layer's shape)
+    (16, 13, 13, 128, 192, 3, 3, 1, 1, 1, 1, 6, None),   # rows of 13 (AlexNet's later layers): 43 groups per image, the last with one pixel; 54 items in a line
 ]
 
 
