@@ -180,7 +180,7 @@ void alpha_plan_deltaW(const alpha_engine_config *c, int IH, int IW, int OH, int
         // 4 stored input channels: the kernel of delta_w_stem.hip runs GridZ x (groups of 16 taps) x (blocks of 64 output
         // channels) workgroups at most; a 3x3 first layer at the reference's 128 fills half of 256 compute units
         const int per_slice = ((FH * FW + 15) / 16) * ((OC + 63) / 64);
-        int want = (c->deltaW_SK_leastUnits + per_slice - 1) / per_slice;
+        int want = c->deltaW_SK_leastUnits / per_slice;   // rounded down: one workgroup more than compute units is a second round
         if (want > GridZ2) want = GridZ2;
         if (want > GridZ) GridZ = want;
     }
