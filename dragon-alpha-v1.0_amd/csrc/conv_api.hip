@@ -137,7 +137,14 @@ bool pointwise_direct_preferred(int K, int N, long M)
     if (forced >= 0) return forced != 0 && (K % 32) == 0;
     // its wavefronts own tiles of 16 pixels: with fewer tiles than SIMDs the kernel of direct_conv.hip, which cuts the
     // reduction among a workgroup's wavefronts, is the faster (832 -> 48 channels on 64x7x7 pixels: 0.007 against 0.019 ms)
-    return (K % 32) == 0 && K >= 128 && N <= 64 && M >= 64L * device_cu_count();
+    if ((K % 32) != 0 || M < 64L * device_cu_count()) return false;
+    // long reductions into one block of 64 produced channels; 48 or fewer go to direct_conv.hip's blocks of 16, 32 or 48
+    // (192 -> 16 / 32 / 48 on 64x28x28 pixels: 0.011 / 0.013 / 0.014 against 0.015 ms, 128 -> 32 on 32x56x56: 0.015 against 0.019)
+    if (K >= 128) return N > 48 && N <= 64;
+    // short reductions into many channels, where the output's stores are the time (backward-data of the same layers:
+    // 32 -> 192 / 256 on 64x28x28 0.011 / 0.013 against 0.014 / 0.015 ms, 32 -> 512 on 256x14x14 0.023 against 0.027, 96 -> 192
+    // 0.022 against 0.024; with 64 reduced channels the filter-resident kernel keeps the layer: 64 -> 256 0.019 against 0.021)
+    return (K == 32 || K == 96) && N >= 128;
 }
 
 // Through direct_conv.hip (no LDS): every layer with more than one tap or a stride (every 3x3 layer of the benchmark
@@ -148,6 +155,14 @@ bool pointwise_direct_preferred(int K, int N, long M)
 // the compute units (256 -> 1024 channels on 64x14x14 pixels: 0.053 against 0.060 ms through the filter-resident kernel;
 // 256 -> 64 on 32x56x56 pixels: 0.030 against 0.032 ms through pointwise_direct.hip; 64 -> 256 there: 0.036 against
 // 0.031 ms through the filter-resident kernel, which keeps that shape).
+// Whether a workgroup of direct_conv.hip's kernel has 16 or more items (tile of 16 pixels, block of produced channels) -
+// from there on its wavefronts take whole items of their own.
+bool direct_conv_whole_items(long M, int CO)
+{
+    const long cus = device_cu_count();
+    return cus > 0 && ((M + 15) / 16 * ((CO + 63) / 64) + cus - 1) / cus >= 16;
+}
+
 bool direct_conv_preferred(int FH, int FW, int sh, int sw, long M, int AC, int CO)
 {
     if (sh > 1 || sw > 1 || FH * FW > 1) return true;
@@ -204,11 +219,12 @@ int forward(const char *fn, const int64_t *streams, int length,
         if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), Y, *ep, (long)N * OH * OW, OC);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (algo == 0 && layout == FILTER_CW && FH == 1 && FW == 1 && IC >= 32) {
+    if (algo == 0 && layout == FILTER_CW && FH == 1 && FW == 1 && (IC >= 32 || direct_conv_whole_items((long)N * OH * OW, OC))) {
         // a 1x1 layer that none of the kernels above took (produced channels not a multiple of 64, more than 256 reduced
         // ones ...): the kernel without LDS before the LDS-halo and the generic ones (192 -> 96 channels on 64x28x28 pixels:
-        // 0.023 against 0.035 ms; 832 -> 48 on 64x7x7: 0.007 against 0.019 ms; with 16 reduced channels the generic kernel
-        // is the faster: 16 -> 480 backward-data 0.012 against 0.019 ms)
+        // 0.023 against 0.035 ms; 832 -> 48 on 64x7x7: 0.007 against 0.019 ms; with 16 reduced channels - a single step per
+        // item - only where a workgroup has whole items: 16 -> 192 backward-data on 64x28x28 0.015 against 0.020 ms through
+        // the generic kernel; where all items are shared by the wavefronts the generic kernel is the faster)
         hipError_t e = launch_direct_conv(stream0(streams), X, F, Y, N, IH, IW, IC, OH, OW, OC, FH, FW, sh, sw, ph, pw,
                                           0, IC * OC, OC, (long)FH * FW * IC * OC, bias, ep, t_workspace, t_workspace_bytes, t_tickets, t_tickets_count);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
@@ -271,7 +287,7 @@ int deltaX_s1(const char *fn, const int64_t *streams, int length,
         if (e == hipSuccess && ep) return epilogue_pass(fn, stream0(streams), dX, *ep, (long)N * IH * IW, IC);
         if (e != hipErrorNotSupported) return hip_status(e, fn);
     }
-    if (algo == 0 && FH == 1 && FW == 1 && OC >= 32) {
+    if (algo == 0 && FH == 1 && FW == 1 && (OC >= 32 || direct_conv_whole_items((long)N * IH * IW, IC))) {
         // a 1x1 layer that none of the kernels above took: as in forward()
         hipError_t e = launch_direct_conv(stream0(streams), dY, W, dX, N, OH, OW, OC, IH, IW, IC, FH, FW, 1, 1, FH - 1 - ph, FW - 1 - pw,
                                           (FH * FW - 1) * IC, -IC, FH * FW * IC, (long)OC * FH * FW * IC, nullptr, ep,

@@ -90,7 +90,10 @@ hipError_t launch_direct_conv(hipStream_t stream, const float *A, const float *B
         // 64-wide ones would - 96 channels are two blocks of 48 (3 per lane: 12 MFMAs a step and tile instead of 16 on one
         // full and one half-empty block) -, where the channel count is a multiple of it
         const int n = (CO + 16 * a.nblocks - 1) / (16 * a.nblocks);
-        if (n < 4 && CO % n == 0) return launch_direct_conv_narrow(stream, a, n);
+        const int nj = (n < 4 && CO % n == 0) ? n : 4;
+        // an odd number of steps per item: the kernels that add an empty step, where a workgroup has whole items at all
+        if (((TH * TW * (AC >> 4)) & 1) && dc_whole_items((a.items + wgs - 1) / wgs) > 0) return launch_direct_conv_odd(stream, a, nj);
+        if (nj < 4) return launch_direct_conv_narrow(stream, a, nj);
     }
     a.base = a.items / wgs;
     a.items_left = a.items - a.base * wgs;

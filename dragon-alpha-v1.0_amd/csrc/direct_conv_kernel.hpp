@@ -137,10 +137,16 @@ static __device__ __forceinline__ floatx4 dc_load(__amdgpu_buffer_rsrc_t rsrc, u
 // NJ: produced channels per lane, 1 to 4 - a block of produced channels is 16 NJ wide and a step costs 4 NJ MFMAs a tile.
 // 4 = the 64-wide blocks; 96 produced channels are two blocks of 48 with NJ = 3 instead of one full and one half-empty
 // block of 64. (NJ < 4 without the lent scratch, whose pieces are 64 wide.)
-template <bool EPI, bool WS = false, int NJ = 4>
+// ODD: for layers with an odd number of steps per item (48 channels under a 3x3 filter: 27; 48 under a 1x1 filter: 3). The
+// loop over whole items multiplies two steps per turn; here an item's steps are followed by one empty step - its loads
+// of A lie beyond the descriptor and return zeros - so that such layers have whole items too. (Without it all their items
+// are shared by the workgroup's eight wavefronts in runs of a single group: 1x1 48 -> 192 on 64x28x28 pixels 0.028 ms
+// where 32 -> 192 takes 0.014.) Without the lent scratch.
+template <bool EPI, bool WS = false, int NJ = 4, bool ODD = false>
 __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArgs p)
 {
     static_assert(NJ == 4 || !WS, "pieces in the lent scratch are 64 channels wide");
+    static_assert(!ODD || !WS, "the form with an empty step takes no lent scratch");
     extern __shared__ __attribute__((aligned(16))) float dc_smem[];
     floatx4 *part = reinterpret_cast<floatx4 *>(dc_smem);   // [8 wavefronts][4 DC_SPLIT_T units][64 lanes]
     const int t = threadIdx.x, lane = t & 63;
@@ -155,9 +161,10 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
     // An odd number of steps per item (48 channels under a 3x3 filter: 27): the loop over whole items multiplies two steps
     // per turn, so such a layer has no whole items - all of them are shared, in runs of a single group, whose parts
     // may be odd.
-    const int f = (((p.AC >> 4) * p.TH * p.TW) & 1) ? 0 : dc_whole_items(g_hi - g_lo);
+    const int f = (!ODD && (((p.AC >> 4) * p.TH * p.TW) & 1)) ? 0 : dc_whole_items(g_hi - g_lo);
     const int i_lo = g_lo + (w & 3) * f + (w >> 2) * (f >> 1), i_hi = i_lo + (f >> 1);
     const int CH = p.AC >> 4, taps = p.TH * p.TW, KS = taps * CH;   // steps per group
+    const int KW = ODD ? KS + 1 : KS;                                // the same with the empty step, for whole items
     const bool pointwise = taps == 1 && p.sh == 1 && p.sw == 1 && p.ph == 0 && p.pw == 0;
 
     const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A), 0, p.a_bytes, 0x00020000);
@@ -207,6 +214,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         // cursor, which restarts from these values at every group, in vector registers)
         const int tap_lo = __builtin_amdgcn_readfirstlane(k_lo / CH), ch_lo = __builtin_amdgcn_readfirstlane(k_lo - tap_lo * CH);
         int c_tile = tile0, c_tap = tap_lo, c_ch = ch_lo, c_left = count * k_n;
+        bool c_empty = false;   // ODD, whole items: the step being requested next is an item's empty one
         int org[T];          // byte offset of (this lane's pixel's window origin, channel 4q); may lie before the tensor
         unsigned rc[T];      // bit th: window row th is inside the image; bit 16 + tw: window column tw is
         unsigned voff[T];    // this tap's load offset, or DC_NEVER in the padding
@@ -262,12 +270,23 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
                     if (c_ch == CH) {
                         c_ch = 0;
                         c_tap++;
-                        if (!SPLIT && c_tap == taps) {
-                            c_tap = 0;
-                            c_tile += stride;
-                            locate();
+                        if (ODD && !SPLIT && c_tap == taps && !c_empty) {
+                            // the empty step: A out of range for every tile, B once more from the last step's place; the
+                            // next turn of the cursor passes the end of the taps again
+                            c_empty = true;
+                            c_tap = taps - 1;
+                            c_ch = CH - 1;
+#pragma unroll
+                            for (int i = 0; i < T; i++) voff[i] = DC_NEVER;
+                        } else {
+                            if (!SPLIT && c_tap == taps) {
+                                c_empty = false;
+                                c_tap = 0;
+                                c_tile += stride;
+                                locate();
+                            }
+                            aim();
                         }
-                        aim();
                     }
                 }
             }
@@ -423,13 +442,13 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
         int n4, n3, n2, n1;
         groups_of(f >> 1, n4, n3, n2, n1);
         int base = t0;
-        run(DcInt<4>{}, DcInt<0>{}, nb_first, base + 4 * w, n4, 0, KS, 32);
+        run(DcInt<4>{}, DcInt<0>{}, nb_first, base + 4 * w, n4, 0, KW, 32);
         base += 32 * n4;
-        run(DcInt<3>{}, DcInt<0>{}, nb_first, base + 3 * w, n3, 0, KS, 24);
+        run(DcInt<3>{}, DcInt<0>{}, nb_first, base + 3 * w, n3, 0, KW, 24);
         base += 24 * n3;
-        run(DcInt<2>{}, DcInt<0>{}, nb_first, base + 2 * w, n2, 0, KS, 16);
+        run(DcInt<2>{}, DcInt<0>{}, nb_first, base + 2 * w, n2, 0, KW, 16);
         base += 16 * n2;
-        run(DcInt<1>{}, DcInt<0>{}, nb_first, base + w, n1, 0, KS, 8);
+        run(DcInt<1>{}, DcInt<0>{}, nb_first, base + w, n1, 0, KW, 8);
     } else {
         int i = i_lo;
         while (i < i_hi) {
@@ -437,10 +456,10 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
             const int cnt = min(i_hi - i, p.tiles - tile0);
             int n4, n3, n2, n1;
             groups_of(cnt, n4, n3, n2, n1);
-            run(DcInt<4>{}, DcInt<0>{}, nb, tile0, n4, 0, KS, 4);
-            run(DcInt<3>{}, DcInt<0>{}, nb, tile0 + 4 * n4, n3, 0, KS, 3);
-            run(DcInt<2>{}, DcInt<0>{}, nb, tile0 + 4 * n4 + 3 * n3, n2, 0, KS, 2);
-            run(DcInt<1>{}, DcInt<0>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1, 0, KS, 1);
+            run(DcInt<4>{}, DcInt<0>{}, nb, tile0, n4, 0, KW, 4);
+            run(DcInt<3>{}, DcInt<0>{}, nb, tile0 + 4 * n4, n3, 0, KW, 3);
+            run(DcInt<2>{}, DcInt<0>{}, nb, tile0 + 4 * n4 + 3 * n3, n2, 0, KW, 2);
+            run(DcInt<1>{}, DcInt<0>{}, nb, tile0 + 4 * n4 + 3 * n3 + 2 * n2, n1, 0, KW, 1);
             i += cnt;
         }
     }
@@ -501,5 +520,7 @@ __global__ __launch_bounds__(512, 1) void direct_conv_kernel(const DirectConvArg
 
 // direct_conv_narrow.hip: the kernels with fewer than four produced channels per lane (no lent scratch)
 hipError_t launch_direct_conv_narrow(hipStream_t stream, const DirectConvArgs &a, int nj);
+// direct_conv_odd.hip: the kernels for an odd number of steps per item, nj = 1 to 4 produced channels per lane (no lent scratch)
+hipError_t launch_direct_conv_odd(hipStream_t stream, const DirectConvArgs &a, int nj);
 
 }  // namespace alpha

@@ -69,6 +69,7 @@ FUSED_SHAPES = [
     (4, 12, 12, 32, 32, 3, 3, 2, 2, 1, 1, "the same, 2 per lane"),
     (4, 12, 12, 32, 16, 5, 5, 1, 1, 2, 2, "the same, 1 per lane"),
     (4, 10, 10, 48, 36, 3, 3, 1, 1, 1, 1, "the same, 36 of a block of 48"),
+    (128, 24, 24, 48, 64, 3, 3, 1, 1, 1, 1, "the same, 27 steps and 18 items per workgroup: whole items with an empty step"),
 ]
 
 
@@ -129,6 +130,7 @@ DX_SHAPES = [
     (4, 12, 12, 32, 64, 5, 2),      # the same, 2 per lane
     (4, 10, 10, 16, 32, 3, 1),      # the same, 1 per lane
     (4, 10, 10, 36, 64, 3, 1),      # the same, 36 of a block of 48
+    (128, 24, 24, 64, 48, 3, 1),    # the same, 27 steps and 18 items per workgroup: whole items with an empty step
 ]
 
 

@@ -458,6 +458,12 @@ DIRECT_CONV_SHAPES = [
     (8, 14, 14, 32, 20, 3, 3, 2, 2, 1, 1),      # 20 of a block of 32
     (8, 14, 14, 32, 12, 1, 1, 1, 1, 0, 0),      # 12 of a block of 16, 1x1
     (8, 14, 14, 32, 40, 3, 3, 1, 1, 1, 1),      # 40 = 3 per lane would split a lane's group at the end: four per lane
+    # an odd number of steps and 16 or more items per workgroup: whole items, each followed by an empty step
+    (128, 28, 28, 48, 192, 1, 1, 1, 1, 0, 0),   # 1x1, 48 channels: 3 steps + 1; 18816 items = 73 or 74 per workgroup
+    (128, 28, 28, 16, 64, 3, 3, 1, 1, 1, 1),    # 9 steps + 1; 6272 items = 24 or 25 per workgroup
+    (192, 24, 24, 16, 64, 1, 1, 1, 1, 0, 0),    # a single step + 1; 27 items per workgroup
+    (96, 30, 30, 48, 48, 3, 3, 2, 2, 1, 1),     # 27 steps + 1, strided, one block of 48 produced channels; 5400 items = 21 or 22 per workgroup
+    (64, 33, 31, 16, 20, 5, 5, 1, 1, 2, 2),     # 25 steps + 1, 20 of a block of 32, ragged last tile; 4092 items
     (50, 14, 14, 48, 256, 3, 3, 1, 1, 1, 1),    # 27 steps, 2452 items: 9 or 10 per workgroup - a group of two tiles per SIMD, steps 14 + 14
 ]
 

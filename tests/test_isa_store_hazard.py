@@ -74,8 +74,8 @@ def _compile(src, tmp):
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not found")
 def test_no_store_is_followed_by_a_write_to_its_data_registers(tmp_path):
     srcs = _sources()
-    assert len(srcs) >= 7, srcs          # the kernels with 128-bit buffer stores, direct_conv.hip and direct_conv_narrow.hip among them
-    assert any(s.endswith("direct_conv.hip") for s in srcs) and any(s.endswith("direct_conv_narrow.hip") for s in srcs)
+    assert len(srcs) >= 8, srcs          # the kernels with 128-bit buffer stores, direct_conv.hip, direct_conv_narrow.hip and direct_conv_odd.hip among them
+    assert all(any(s.endswith(f) for s in srcs) for f in ("direct_conv.hip", "direct_conv_narrow.hip", "direct_conv_odd.hip"))
     assert not [s for s in srcs if "__builtin_amdgcn_raw_buffer_store_b128" in open(s).read()], "a store bypasses the guarded helper"
     with concurrent.futures.ThreadPoolExecutor(max_workers=6) as ex:
         results = list(ex.map(lambda s: _compile(s, str(tmp_path)), srcs))
