@@ -83,6 +83,16 @@ static DwsCut dws_cut(long items, long TG, int G, int GZ, long bytes)
     return {most, false};
 }
 
+// A 1x1 filter at stride 1 without padding reads pixel k of X for pixel k of deltaY: the rows and images are one run of
+// pixels, and the kernel takes it as a single row (or a row per image where that is too long for the 32-bit offsets within
+// a row) - no pixel group is left partly empty at the end of a 7- or 14-pixel row, and no row ever ends.
+static void dws_pointwise_rows(int &N, int &OH, int &OW, int IC, int OC)
+{
+    const long P = (long)OH * OW, C = IC > OC ? IC : OC;
+    if (((long)N * P + 8) * C * 4 < (1L << 28)) { OW = (int)(N * P); OH = 1; N = 1; }
+    else if ((P + 8) * C * 4 < (1L << 28)) { OW = (int)P; OH = 1; }
+}
+
 // Pixel groups as four consecutive pixels of an image (row-major) instead of an output row: where a row's groups are
 // empty to three sixteenths or more (rows of 1, 2, 3, 5, 6, 9 or 13 pixels). Images beyond 512 MB do not fit the 32-bit offsets
 // within an image.
@@ -114,11 +124,13 @@ static DwsCut dws_cut_of_layer(int units, int N, int OH, int OW, int IC, int OC,
     // the stricter of the split-K entries' two thresholds (the stride is not known here)
     if (deltaW_stream_block_fill(IC, OC) < 40) return {0, false};
     const long icb = (IC + 63) / 64, ocb = (OC + 63) / 64;
+    const long bytes = (long)N * OH * OW * ((long)IC + OC) * 4;
+    if (FH == 1 && FW == 1) dws_pointwise_rows(N, OH, OW, IC, OC);   // (taken to be at stride 1 without padding, as nearly all are)
     // (the input's size is not known here: the launcher's other condition for groups by image, an image of X below 512 MB)
     const bool flat = dws_flat_rows(OH, OW, OC);
     const long items = icb * ocb * FH * FW, TG = flat ? (long)N * (((long)OH * OW + 3) / 4) : (long)N * OH * ((OW + 3) / 4);
     if (items >= (1L << 20) || TG >= (1L << 30)) return {0, false};
-    return dws_cut(items, TG, units, GZ, (long)N * OH * OW * ((long)IC + OC) * 4);
+    return dws_cut(items, TG, units, GZ, bytes);
 }
 
 // The least split-K factor <= GZ with which launch_deltaW_stream on a device of `units` compute units cuts the layer
@@ -155,6 +167,11 @@ hipError_t launch_deltaW_stream(hipStream_t stream, const float *X, const float 
     if ((long)(OW + 4) * OC * 4 >= (1L << 28) || ((long)(OW + 4) * sw + FW + pw) * IC * 4 >= (1L << 28)) return hipErrorNotSupported;
     const long GK = (long)N * OH * OW;
     if (GK >= (1L << 31)) return hipErrorNotSupported;
+    if (FH == 1 && FW == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && OH == IH && OW == IW) {
+        dws_pointwise_rows(N, OH, OW, IC, OC);
+        IH = OH;
+        IW = OW;
+    }
     const int cus = device_cu_count();
     if (cus < 1) return hipErrorNotSupported;
     DwStreamFlatArgs a{};
