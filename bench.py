@@ -640,7 +640,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS))
+    ap.add_argument("--layer", default="c3a", choices=sorted(LAYERS) + sorted(OTHER_LAYERS),
+                    help="a layer of BASELINE.json's configs (default c3a, the headline) or one of --sweep's, measured alone (profiles)")
     ap.add_argument("--op", default=None, choices=["fwd", "fwd_bias", "fwd_cached", "fwd_fused", "dx", "dw", "dw_least", "wino", "dx_wino", "dw_wino"],
                     help="wino = forward through Winograd F(2x2,3x3) (3x3 stride-1 layers), reported in direct-conv-equivalent FLOPs")
     ap.add_argument("--layers", action="store_true", help="accepted for compatibility: the layers array is part of the default line")
@@ -704,10 +705,14 @@ def main():
         print(json.dumps({"sweep": "layers outside the five configs", "layers": len(OTHER_LAYERS), "steps": args.steps,
                           "parity_failed": bad, "worst_max_err_ratio": worst}, separators=(",", ":")), flush=True)
         return
+    config_layers = sorted(LAYERS)
+    if args.layer in OTHER_LAYERS:   # a layer outside the configs, alone: its seed as in --sweep, no array of the configs' layers
+        LAYERS[args.layer] = OTHER_LAYERS[args.layer]
+        args.no_layers = True
     op = args.op or LAYERS[args.layer][9][0]
 
     def seed_of(layer):
-        return 1000 + sorted(LAYERS).index(layer)
+        return 1000 + config_layers.index(layer) if layer in config_layers else 5000 + list(OTHER_LAYERS).index(layer)
 
     wl = Workload(pkg, torch, args.layer, seed_of(args.layer))
     head = measure(wl, op, args.steps, args.warmup, with_parity=not args.no_parity)
@@ -748,7 +753,7 @@ def main():
     del wl
     rows = []
     if not args.no_layers:
-        for layer in sorted(LAYERS):
+        for layer in config_layers:
             wl = Workload(pkg, torch, layer, seed_of(layer))
             for o in layer_ops(layer):
                 if o == "bn_bwd":
