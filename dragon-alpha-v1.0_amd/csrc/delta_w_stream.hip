@@ -61,7 +61,7 @@ static DwsCut dws_cut(long items, long TG, int G, int GZ, long bytes)
     // (2) Tensors well beyond the L2s (56 MB: measured between 50 and 65) whose shares of the line start at 32 or more
     // different places of the pixel range (G / gcd(items, G): 27, 72, 200 items on 256 workgroups; with 144 items pairs
     // of shares run over the same pixels, with 576 eight at a time, and the line stays the faster cut): every workgroup
-    // then streams pixels of its own and the L2s serve nobody twice (5x5 96 -> 256 on 64x27x27: 1.8 GB fetched for 65 MB
+    // then streams pixels of its own and the L2s serve nobody twice (5x5 96 -> 256 on 64x27x27: 3.8 GB fetched for 65 MB
     // of tensors). Whole units instead, ceil(P items / G) per workgroup: the workgroups of an XCD go through the same
     // piece of the pixels at the same time, each for an item of its own. P minimises the modelled time, a unit's
     // end (partial sums through LDS, stores, the loads of the next from cold) counted as 64 pixel groups.
