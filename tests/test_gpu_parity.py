@@ -358,6 +358,13 @@ POINTWISE_SHAPES = [
     (64, 28, 30, 32, 200),    # 53760 pixels = 3360 tiles over 2048 wavefronts: shares of 1 and 2 tiles; 200 = 3 blocks + 8 channels
     (32, 56, 56, 64, 32),     # 100352 pixels = 6272 tiles: shares of 3 and 4 tiles (c5 geometry with fewer channels)
     (64, 60, 64, 32, 32),     # 245760 pixels = 15360 tiles: shares of 7 and 8 tiles (4 + 3 and 4 + 4)
+    # what the library chooses by shape for narrow 1x1 layers with 64 pixels or more per compute unit
+    (64, 28, 28, 192, 16),    # forward: 16 produced channels, blocks of 16 in the kernel of direct_conv; backward: 16 reduced channels = one step and an empty one per whole item
+    (64, 28, 28, 192, 32),    # forward: blocks of 32; backward: 32 reduced into 192, the kernel without LDS of the 1x1 family
+    (64, 28, 28, 192, 48),    # forward: a block of 48; backward: 48 reduced channels = 3 steps and an empty one
+    (32, 28, 28, 192, 96),    # backward: 96 reduced into 192
+    (96, 24, 24, 16, 64),     # forward: 16 reduced channels, 13 or 14 items per workgroup (no whole items: the generic kernel by shape)
+    (192, 24, 24, 16, 64),    # the same with 27 items per workgroup: whole items, one step and an empty one
 ]
 
 
