@@ -14,7 +14,8 @@ Before it, every layer and operator of BASELINE.json's five configs is printed a
 is measured (same step count as the headline): its time, its roofline fractions and its parity against the fp64 CPU
 oracle on a subset of the same seeded tensors (images for forward / backward-data, output channels over the full batch
 for backward-filter), with the tolerance it is held to. The same rows are also written to a file, as one array.
---no-layers leaves them out.
+--no-layers leaves them out. `--sweep` measures the layers outside the configs (OTHER_LAYERS) the same way, one JSON line
+each; `--layer <one of them>` measures that layer alone (for profiles).
 The cpu_baseline leg times the CPU oracle's float-accumulate direct loops on a bounded sample on the host cores
 (baseline only, never a target): the headline operator on all cores, backward-data and backward-filter of c5b on all
 cores, and config 1 forward on one core.
