@@ -187,6 +187,28 @@ def test_deltaW_whole_units_for_large_tensors_with_few_items():
     assert E.plan_deltaW(cfg, 32, 32, 32, 32, 3, 3, 64, 128, 256, 1, 1).GridZ == 7
 
 
+def test_deltaW_least_GridZ_is_idempotent_and_never_raises():
+    """Over seeded random layers and each setting of the cut switch: the reduced factor is at most GridZ (and at least 2
+    where GridZ is), and reducing it again changes nothing - a caller that passes it gets the cut it was computed for."""
+    import random
+    rnd = random.Random(20240611)
+    L = pkg.lib()
+    f = L.alpha_dconv3D_deltaW_least_GridZ
+    try:
+        for units in (-1, 0, 1):
+            assert L.alpha_conv_set_deltaW_units(units) == 0
+            for _ in range(400):
+                OH = rnd.choice([1, 2, 4, 7, 8, 13, 14, 16, 27, 28, 32, 56, 112]); OW = rnd.choice([OH, OH, rnd.randint(1, 60)])
+                F = rnd.choice([1, 3, 3, 5, 7]); N = rnd.choice([1, 8, 32, 64, 128, 512])
+                IC = rnd.choice([4, 16, 32, 48, 64, 96, 128, 192, 256, 512, 1024]); OC = rnd.choice([16, 32, 64, 96, 128, 208, 256, 384, 512, 2048])
+                GZ = rnd.choice([1, 2, 3, 5, 8, 14, 28, 64, 128, 392, 1000]); cus = rnd.choice([256, 304, 64])
+                g = f(cus, GZ, OH, OW, F, F, N, IC, OC)
+                assert g <= GZ and (g >= 2 or GZ < 2), (units, cus, GZ, OH, OW, F, N, IC, OC, g)
+                assert f(cus, g, OH, OW, F, F, N, IC, OC) == g, (units, cus, GZ, OH, OW, F, N, IC, OC, g)
+    finally:
+        L.alpha_conv_set_deltaW_units(-1)
+
+
 def test_deltaX_plans():
     cfg = E.default_config(256)
     assert E.plan_deltaX(cfg, 224, 224, 112, 112, 7, 7, 64, 4, 64, 2, 2).entry_name == "dconv3D_deltaX_crossAdd"   # IC <= 8
