@@ -65,17 +65,19 @@ static DwsCut dws_cut(long items, long TG, int G, int GZ, long bytes)
     // of tensors). Whole units instead, ceil(P items / G) per workgroup: the workgroups of an XCD go through the same
     // piece of the pixels at the same time, each for an item of its own. P minimises the modelled time, a unit's
     // end (partial sums through LDS, stores, the loads of the next from cold) counted as 64 pixel groups.
-    const int sw = dws_units_switch();
-    long g = items, h = G;
-    while (h) { const long r = g % h; g = h; h = r; }
-    const long line = (items * TG + G - 1) / G + 128;
-    long best = 0;
+    const int forced = dws_units_switch();
+    long gcd = items;
+    for (long b = G; b != 0;) { const long r = gcd % b; gcd = b; b = r; }
+    constexpr long UNIT_END = 64;   // pixel groups
+    const long line_time = (items * TG + G - 1) / G + 2 * UNIT_END;
+    long best_time = 0;
     int best_P = 0;
     for (int P = 1; P <= GZ && 8L * P <= TG; P++) {
-        const long t = (P * items + G - 1) / G * ((TG + P - 1) / P + 64);
-        if (best_P == 0 || t < best) best = t, best_P = P;
+        const long t = (P * items + G - 1) / G * ((TG + P - 1) / P + UNIT_END);
+        if (best_P == 0 || t < best_time) best_time = t, best_P = P;
     }
-    if (best_P > 0 && (sw == 1 || (sw < 0 && bytes > (56L << 20) && g * 32 <= G && 100 * best <= 108 * line))) return {best_P, true};
+    const bool by_shape = bytes > (56L << 20) && gcd * 32 <= G && 100 * best_time <= 108 * line_time;
+    if (best_P > 0 && (forced == 1 || (forced < 0 && by_shape))) return {best_P, true};
     // (3) the line of items; with fewer buffers than the shares an item would meet (the Java engine passes GridZ = 2 for
     // 4x4 maps at N = 512, where 72 items on 256 workgroups meet up to 5 shares each) whole units all the same, some
     // workgroups idle - still several times faster than the kernels with one workgroup per slice (3x3 96 -> 208 there: 0.463 ms)
