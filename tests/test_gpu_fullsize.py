@@ -345,6 +345,56 @@ def test_kernel_split_shared_groups_full_size(dev, case):
     assert float(err.max()) <= 0.0, "%s: the two distributions differ beyond twice the bar" % (case,)
 
 
+@pytest.mark.parametrize("case", [(64, 27, 27, 96, 256, 5, 2, 14, 5),      # AlexNet's second layer: 200 items, 65 MB: 5 pieces per item, 3 or 4 units per workgroup
+                                  (512, 16, 16, 64, 192, 3, 1, 85, 9),     # 27 items, 134 MB: 9 pieces, one unit per workgroup on 243 of them
+                                  (64, 32, 32, 128, 256, 3, 1, 42, 7)])    # 72 items, 101 MB: 7 pieces, 1 or 2 units per workgroup
+def test_deltaW_whole_units_by_shape_full_size(dev, case):
+    """Large tensors whose line of items would start every share at a different place of the pixel range get the cut into
+    whole (piece, item) units by shape: the buffers beyond the P pieces are zeros, the sums under both cuts agree, and
+    output channels of both are checked against the oracle."""
+    torch = dev.torch
+    L = pkg.lib()
+    DW = pkg.Cuda_dconv3D_deltaW
+    N, IH, IW, IC, OC, F, p, GridZ, P = case
+    OH, OW = out_dim(IH, IW, F, F, 1, 1, p, p)
+    g = torch.Generator(device="cpu").manual_seed(8500 + IH)
+    X = torch.randn((N, IH, IW, IC), generator=g)
+    dY = torch.randn((N, OH, OW, OC), generator=g)
+    x, dy = X.to(dev.dev), dY.to(dev.dev)
+    sizeW = OC * F * F * IC
+
+    def run(units):
+        assert L.alpha_conv_set_deltaW_units(units) == 0
+        dw = torch.full((OC, F, F, IC), float("nan"), device=dev.dev)
+        buf = torch.full((GridZ - 1, sizeW), float("nan"), device=dev.dev)
+        DW.dconv3D_deltaW_GemmSK(dev.streams, 1, GridZ, x.data_ptr(), IH, IW, dy.data_ptr(), OH, OW, dw.data_ptr(), buf.data_ptr(),
+                                 F, F, N, IC, OC, 1, 1, p, p)
+        dev.sync()
+        return dw, buf
+
+    try:
+        line = run(0)
+        by_shape = run(-1)
+        units = run(1)
+    finally:
+        L.alpha_conv_set_deltaW_units(-1)
+    assert torch.equal(by_shape[0].view(torch.int32), units[0].view(torch.int32)) and torch.equal(by_shape[1].view(torch.int32), units[1].view(torch.int32)), \
+        "the choice by shape is not the cut into whole units"
+    if pkg.device_info()[0] == 256:
+        assert not bool(by_shape[1][P - 1:].any()) and bool(by_shape[1][P - 2].any()), "expected %d pieces per item" % P
+    ocs = [0, OC // 2 + 1, OC - 1]
+    want = O.deltaW_f64(X.numpy(), np.ascontiguousarray(dY.numpy()[..., ocs]), F, F, 1, 1, p, p)
+    sums = {}
+    for name, (dw, buf) in (("line", line), ("units", by_shape)):
+        tot = (dw.double() + buf.double().sum(0).view(OC, F, F, IC))
+        sums[name] = tot
+        _check(tot[ocs].cpu().numpy(), want, "deltaW %s %s" % (name, case))
+    ref = sums["line"]
+    floor = 1e-5 * max(1.0, float(ref.pow(2).mean().sqrt()))
+    err = (sums["units"] - ref).abs() - 2 * torch.clamp(1e-4 * ref.abs(), min=floor)
+    assert float(err.max()) <= 0.0, "%s: the two cuts differ beyond twice the bar" % (case,)
+
+
 # Tensors between 2 GB and the 2^31 elements the entries accept: the kernels that address through 2 GB buffer
 # descriptors refuse them (nothing launched) and the layer goes to the kernels that index elements. X and deltaX are
 # 2.2 GB here (44 x 512 x 512 x 48); first and last image against the oracle; backward-filter with deltaY zero outside
